@@ -1,0 +1,298 @@
+/*
+ * C ABI of the MI355X (gfx950) kernel library for the speculative MTP-4
+ * verify step.  This is the layer a provider binds where the reference's
+ * provider calls the free functions of namespace expert::runtime::cuda
+ * (runtime/include/expert/runtime/cuda/transformer_kernels.hpp): raw device
+ * pointers, a stream passed as void*, plain integers, no C++ types.
+ *
+ * Every entry point returns a qllm_status code (0 = ok).  The codes mirror
+ * the reference's ErrorCode enum (runtime/include/expert/runtime/storage.hpp:
+ * 17-29); the text of the last failure on the calling thread is available
+ * from qllm_last_error().  All pointers are device pointers unless a
+ * parameter is documented as host memory.  Work is enqueued on `stream`
+ * (a hipStream_t; NULL = the default stream) and is not synchronised.
+ *
+ * The library is HIP-only: there is no CPU fallback.  A call made on a
+ * machine without a gfx950 device fails with QLLM_INTERNAL.
+ */
+#ifndef QLLM_KERNELS_H
+#define QLLM_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum qllm_status {
+  QLLM_OK = 0,
+  QLLM_CANCELLED = 1,
+  QLLM_DEADLINE_EXCEEDED = 2,
+  QLLM_BACKPRESSURE = 3,
+  QLLM_INVALID_ARGUMENT = 4,
+  QLLM_OPEN_FAILED = 5,
+  QLLM_IO_FAILED = 6,
+  QLLM_SHORT_READ = 7,
+  QLLM_CHECKSUM_MISMATCH = 8,
+  QLLM_UPLOAD_FAILED = 9,
+  QLLM_INTERNAL = 10
+};
+
+/* Text of the most recent non-ok status returned on this thread. */
+const char* qllm_last_error(void);
+
+/* Library build identification: "qllm-hip gfx950 <abi>". */
+const char* qllm_version(void);
+
+/* ---- FP4 weight matrices ------------------------------------------------ */
+
+enum qllm_scale_scheme {
+  /* Reference quant ABI 3: one UE8M0 byte per 32 padded columns
+   * (transformer_kernels.hpp:23-32, struct Fp4Block32Matrix). */
+  QLLM_SCALE_UE8M0_BLOCK32 = 0,
+  /* One IEEE binary16 scale per 16 columns (the block-16 analogue of
+   * struct Nvfp4Block16Matrix, transformer_kernels.hpp:44-54, with an F16
+   * scale and no global factors). */
+  QLLM_SCALE_F16_BLOCK16 = 1
+};
+
+/* Row-major packed E2M1 codes, low nibble = even column; rows keep their
+ * logical column count while storage pads every row to padded_columns
+ * (a multiple of 32).  Mirrors Fp4Block32Matrix plus the scheme tag. */
+typedef struct qllm_fp4_matrix {
+  const uint8_t* weights; /* [rows, padded_columns/2] */
+  const void* scales;     /* u8 [rows, padded/32] or f16 [rows, padded/16] */
+  uint32_t rows;
+  uint32_t columns;
+  uint32_t padded_columns;
+  uint32_t scale_scheme;  /* enum qllm_scale_scheme */
+} qllm_fp4_matrix;
+
+enum qllm_output_kind {
+  QLLM_OUT_F32 = 0,         /* float [batch, rows] */
+  QLLM_OUT_F32_BF16_ROUNDED = 1, /* float storage, values rounded to bf16
+                                    (the reference's bf16_output flag) */
+  QLLM_OUT_BF16 = 2         /* bf16 storage [batch, rows] */
+};
+
+/* replaces quantize_q8_batch / quantize_q8_batch_bf16
+ * (transformer_kernels.hpp:76-83). */
+int32_t qllm_quantize_q8_batch(const float* input, int8_t* output,
+                               float* scales, uint32_t rows,
+                               uint32_t columns, uint32_t padded_columns,
+                               int32_t bf16_input, void* stream);
+
+/* replaces convert_f32_to_bf16_batch (transformer_kernels.hpp:84-87). */
+int32_t qllm_convert_f32_to_bf16_batch(const float* input, void* output,
+                                       size_t output_bytes, uint32_t rows,
+                                       uint32_t columns,
+                                       uint32_t padded_columns, void* stream);
+
+/* FP4 weights x Q8 activations, batch <= 8; out[m*rows+n].
+ * replaces fp4_gemv_q8_batch_weight_reuse (transformer_kernels.hpp:92-97).
+ * Block-32 UE8M0 matrices only. */
+int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
+                               const int8_t* input,
+                               const float* input_scales, float* output,
+                               uint32_t batch, int32_t bf16_output,
+                               void* stream);
+
+/* FP4 weights x BF16 activations [batch, padded_columns], F32 accumulate,
+ * batch <= 8.  replaces fp4_gemm_bf16_block32
+ * (transformer_kernels.hpp:109-112) and extends it to block-16 F16 scales.
+ * `residual` (optional, float [batch, rows]) is added to the result before
+ * it is stored; output may alias residual. */
+int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix, const void* input,
+                           size_t input_bytes, void* output,
+                           uint32_t output_kind, const float* residual,
+                           uint32_t batch, void* stream);
+
+/* Gate and up projections of one SwiGLU block in a single pass over a shared
+ * BF16 input: out[m,n] = bf16(bf16(silu(gate[m,n])) * up[m,n]) stored as
+ * bf16 [batch, rows].  Fuses two qllm_fp4_gemm_bf16 calls with silu_product
+ * (transformer_kernels.hpp:415-418, run_ffn dense_fp4_provider.cpp:8250-8293).
+ * Both matrices must share shape and scale scheme. */
+int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
+                             const qllm_fp4_matrix* up, const void* input,
+                             size_t input_bytes, void* output,
+                             uint32_t batch, void* stream);
+
+/* replaces fp4_embedding_batch (transformer_kernels.hpp:68-70). */
+int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
+                                 const uint32_t* tokens, float* output,
+                                 uint32_t batch, void* stream);
+
+/* ---- normalisation and elementwise ---------------------------------------- */
+
+/* replaces rms_norm_batch / weightless_rms_norm_batch and the zero-centred
+ * variant (transformer_kernels.hpp:303-309).  weight may be NULL.  Exactly
+ * one of output_f32 / output_bf16 may be NULL; bf16 rows are padded with
+ * zeros to bf16_padded_columns. */
+int32_t qllm_rms_norm_batch(const float* input, const float* weight,
+                            float* output_f32, void* output_bf16,
+                            uint32_t bf16_padded_columns, uint32_t rows,
+                            uint32_t elements, float epsilon,
+                            int32_t zero_centered, void* stream);
+
+/* replaces add_in_place (transformer_kernels.hpp:310-312). */
+int32_t qllm_add_in_place(float* destination, const float* source,
+                          uint32_t elements, int32_t bf16_output,
+                          void* stream);
+
+/* replaces silu_product (transformer_kernels.hpp:415-418). */
+int32_t qllm_silu_product(const float* gate, const float* up, float* output,
+                          uint32_t elements, int32_t bf16_activations,
+                          void* stream);
+
+/* ---- attention: Q4H ("q4-f16-per-head") paged cache ----------------------- */
+
+/* Bytes one layer occupies inside a Q4H page:
+ * page_tokens * kv_heads * 2 * (head_dim/2 + 2). */
+size_t qllm_q4h_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                            uint32_t head_dim);
+
+/* Per-head RMSNorm (1+w) [skipped when the weight pointer is NULL], NeoX
+ * rotary on the first rotary_dim dimensions, then Q4H-encode and store the
+ * K/V rows of `rows` consecutive positions into their pages.
+ * replaces gated_gqa_qkv_rope_cache_paged_q4_per_head_batch
+ * (transformer_kernels.hpp:719-729).  query_stride is the distance in floats
+ * between consecutive query heads (2*head_dim for the output-gated layout,
+ * head_dim for plain GQA); query is updated in place. */
+int32_t qllm_qkv_rope_cache_paged_q4h_batch(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream);
+
+/* replaces store_gqa_kv_paged_q4_per_head_batch (the store-only form used
+ * by runtime/tools/dense_fp4_cuda_smoke.cpp:1828-1832). */
+int32_t qllm_store_kv_paged_q4h_batch(const float* key, const float* value,
+                                      const void* const* page_table,
+                                      uint32_t full_attention_layer,
+                                      uint32_t page_tokens,
+                                      uint32_t first_cache_position,
+                                      uint32_t rows, uint32_t kv_heads,
+                                      uint32_t head_dim, void* stream);
+
+/* replaces quantize_gqa_queries_q8 (transformer_kernels.hpp:851-854). */
+int32_t qllm_quantize_gqa_queries_q8(const float* query,
+                                     uint32_t query_stride, int8_t* q8,
+                                     float* query_scales, uint32_t rows,
+                                     uint32_t query_heads, uint32_t head_dim,
+                                     void* stream);
+
+/* Mirrors PagedQ4BfpGatedGqaAttentionLaunch (transformer_kernels.hpp:826-846)
+ * for gated_gqa_attention_microbatch_paged_q4_per_head_tensor_core. */
+typedef struct qllm_q4h_attention_launch {
+  const float* query;           /* [rows, query_heads, query_stride], 16-byte
+                                   aligned; the kernel quantises it itself */
+  const int8_t* q8_queries;     /* accepted for layout parity with the
+                                   reference struct; may be NULL, unused */
+  const float* query_scales;    /* as above */
+  const void* const* page_table;
+  void* output;                 /* [rows, query_heads, head_dim] */
+  float* partial_maxima;        /* [rows, maximum_splits, query_heads] */
+  float* partial_sums;          /* same */
+  float* partial_outputs;       /* [rows, maximum_splits, query_heads, d] */
+  uint32_t first_context_tokens;/* row r attends tokens [0, first + r) */
+  uint32_t rows;
+  uint32_t full_attention_layer;
+  uint32_t page_tokens;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t head_dim;
+  uint32_t split_tokens;
+  uint32_t maximum_splits;
+  uint32_t query_stride;        /* floats between heads in `query` */
+  int32_t output_gated;         /* multiply by sigmoid(query[d + i]) */
+  uint32_t output_kind;         /* QLLM_OUT_F32 or QLLM_OUT_BF16 */
+  void* stream;
+} qllm_q4h_attention_launch;
+
+/* Split phase + split-K combine.  rows * (query_heads/kv_heads) <= 48,
+ * head_dim in {128, 256}, page_tokens % 64 == 0, split_tokens % 64 == 0. */
+int32_t qllm_attention_paged_q4h(const qllm_q4h_attention_launch* launch);
+
+/* ---- attention: exact F16 paged cache ---------------------------------------- */
+
+/* Per-layer page layout: K [page_tokens][kv_heads][head_dim] then
+ * V [page_tokens][kv_heads][head_dim], binary16
+ * (transformer_kernels.cu:6594-6606).
+ * replaces store_gqa_kv_fp16_to_paged. */
+int32_t qllm_store_kv_paged_f16_batch(const float* key, const float* value,
+                                      const void* const* page_table,
+                                      uint32_t full_attention_layer,
+                                      uint32_t page_tokens,
+                                      uint32_t first_cache_position,
+                                      uint32_t rows, uint32_t kv_heads,
+                                      uint32_t head_dim, void* stream);
+
+/* Mirrors DeviceFp16GatedGqaAttentionLaunch (transformer_kernels.hpp:
+ * 1071-1092), paged-device form, for gated_gqa_attention_staged_device_fp16.
+ * Unlike the reference's sequential split loop, splits run in parallel and
+ * are merged by the same combine kernel as the Q4H path. */
+typedef struct qllm_f16_attention_launch {
+  const float* query;
+  const void* const* device_pages;
+  void* output;
+  float* partial_maxima;
+  float* partial_sums;
+  float* partial_outputs;
+  uint32_t first_context_tokens;
+  uint32_t rows;
+  uint32_t device_page_layer;
+  uint32_t device_page_tokens;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t head_dim;
+  uint32_t split_tokens;
+  uint32_t maximum_splits;
+  uint32_t query_stride;
+  int32_t output_gated;
+  uint32_t output_kind;
+  void* stream;
+} qllm_f16_attention_launch;
+
+int32_t qllm_attention_paged_f16(const qllm_f16_attention_launch* launch);
+
+/* ---- token selection ------------------------------------------------------------ */
+
+/* replaces argmax_batch (transformer_kernels.hpp:1266-1269): ties to the
+ * lower index, NaN never wins.  workspace: at least
+ * qllm_argmax_workspace_bytes(count, batch) bytes of device memory. */
+size_t qllm_argmax_workspace_bytes(uint32_t count, uint32_t batch);
+int32_t qllm_argmax_batch(const float* values, uint32_t count,
+                          uint32_t batch, uint32_t* output, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* replaces topk_logits (transformer_kernels.hpp:1271-1290): exact descending
+ * top-k of one row, ties to the lower id, NaN excluded, k <= 1024. */
+size_t qllm_topk_workspace_bytes(uint32_t count, uint32_t top_k);
+int32_t qllm_topk_logits(const float* values, uint32_t count, uint32_t top_k,
+                         float* output_values, uint32_t* output_indices,
+                         void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/* replaces apply_presence_penalty (transformer_kernels.hpp:1292-1294). */
+int32_t qllm_apply_presence_penalty(float* logits, const uint8_t* emitted,
+                                    uint32_t count, float penalty,
+                                    void* stream);
+
+/* ---- synthetic data (benchmarks and tests) ------------------------------------- */
+
+/* Fill device memory from a counter-based generator (splitmix64 of seed and
+ * element index), so a host restatement can rebuild the same bytes.
+ * kind: 0 = uniform bytes, 1 = N(0,1) float, 2 = N(0,1) bf16,
+ *       3 = log-normal(0, 0.5) binary16, 4 = N(0,1) binary16,
+ *       5 = UE8M0 codes uniform in [124, 130]. */
+int32_t qllm_fill_random(void* destination, size_t elements, uint32_t kind,
+                         uint64_t seed, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,857 @@
+// Decode attention over the Q4H ("q4-f16-per-head") paged KV cache for a
+// micro-batch of query rows (1 guaranteed + drafts), plus the K/V store and
+// query quantisation that precede it.
+//
+// Replaces, from runtime/src/cuda/transformer_kernels.cu of the reference:
+//   store_paged_kv_record<q4_per_head>                         :241-288
+//   gated_gqa_qkv_rope_paged_batch_kernel<q4_per_head>         :3550-3643
+//   quantize_gqa_queries_q8_kernel                             :4391-4416
+//   gated_gqa_attention_paged_bfp_microbatch_split_kernel      :4420-4976
+//   gated_gqa_attention_paged_fp4_prefill_combine_kernel       :5741-5798
+//
+// Split kernel, one workgroup (8 waves) per (kv head, context split); each
+// wave walks 64-token tiles of the split with its own online-softmax state:
+//   scores  S[tok][row] = K4 . Q15       v_mfma_i32_16x16x64_i8, exact ints:
+//           K nibbles are widened to int8*16 with two bit operations and the
+//           query is carried as two int8 planes (15 bits), built in-kernel
+//           from the F32 query - a single Q8 plane, as the reference uses,
+//           is ~1e-2 away from exact attention on N(0,1) inputs
+//   softmax in F32 per lane (a lane owns one query row of a 16-row tile)
+//   output  O^T[d][row] += V^T . P^T     v_mfma_f32_16x16x32_f16, V staged
+//           through LDS and read back transposed with ds_read_b64_tr_b4,
+//           the per-token V scale folded into the nibble->f16 conversion.
+// The eight wave states are merged in LDS and one (max, sum, unnormalised
+// output) partial per (row, split, head) is written; the combine kernel
+// merges the splits.  Maxima are kept in the log2 domain.
+#include "common.hpp"
+
+namespace qllm {
+namespace {
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kSplitWaves = 8;
+constexpr float kMaskedMax = -1.0e30f;
+
+struct Q4hPlanes {
+  const uint8_t* key_codes;
+  const uint8_t* key_scales;
+  const uint8_t* value_codes;
+  const uint8_t* value_scales;
+};
+
+__host__ __device__ inline size_t q4h_layer_bytes(uint32_t page_tokens,
+                                                  uint32_t kv_heads,
+                                                  uint32_t head_dim) {
+  return static_cast<size_t>(page_tokens) * kv_heads * 2u *
+         (head_dim / 2u + 2u);
+}
+
+__device__ __forceinline__ Q4hPlanes q4h_planes(const void* page,
+                                                uint32_t layer,
+                                                uint32_t page_tokens,
+                                                uint32_t kv_heads,
+                                                uint32_t head_dim) {
+  const size_t records = static_cast<size_t>(page_tokens) * kv_heads;
+  Q4hPlanes planes;
+  planes.key_codes = static_cast<const uint8_t*>(page) +
+                     layer * q4h_layer_bytes(page_tokens, kv_heads, head_dim);
+  planes.key_scales = planes.key_codes + records * (head_dim / 2u);
+  planes.value_codes = planes.key_scales + records * 2u;
+  planes.value_scales = planes.value_codes + records * (head_dim / 2u);
+  return planes;
+}
+
+// max over the lanes {l, l^16, l^32, l^48}
+__device__ __forceinline__ float quad_row_max(float value) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  value = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float quad_row_sum(float value) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  value = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+struct SplitArgs {
+  const float* query;
+  uint32_t query_stride;
+  const void* const* page_table;
+  float* partial_maxima;
+  float* partial_sums;
+  float* partial_outputs;
+  uint32_t first_context_tokens;
+  uint32_t rows;
+  uint32_t layer;
+  uint32_t page_tokens;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t split_tokens;
+  uint32_t maximum_splits;
+};
+
+// D = head_dim (128 or 256), RT = number of 16-row tiles (rows*group <= 16*RT).
+template <int D, int RT>
+__global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
+    const SplitArgs args) {
+  constexpr int KSTEPS = D / 64;      // int8 MFMA k-steps over head_dim
+  constexpr int DT = D / 16;          // 16-wide tiles of head_dim
+  constexpr int VROW = D / 2 + 16;    // padded LDS row of V codes (bytes)
+  constexpr int STATE = 16 * RT * (D + 2);  // floats per merged wave state
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t col = lane & 15u;   // query row inside a row tile / token / d
+  const uint32_t quad = lane >> 4;   // 0..3
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t split = blockIdx.y;
+  const uint32_t group = args.query_heads / args.kv_heads;
+  const uint32_t matrix_rows = args.rows * group;
+  const uint32_t last_context = args.first_context_tokens + args.rows - 1u;
+  const uint32_t split_begin = split * args.split_tokens;
+  const uint32_t split_end = min(split_begin + args.split_tokens, last_context);
+  const uint32_t tiles =
+      split_end > split_begin ? (split_end - split_begin + 63u) / 64u : 0u;
+
+  uint8_t* v_stage = lds_raw + wave * (64 * VROW);
+
+  // ---- query operands (B side of S = K.Q), built once ------------------------
+  // The F32 query row is quantised here to 15 bits and split into two int8
+  // planes, q = scale * (128*hi + lo) with hi in [-127,127], lo in [-64,63],
+  // so the integer scores carry the query to ~3e-5 relative instead of the
+  // 4e-3 of a single Q8 plane.
+  i32x4 q_high[RT][KSTEPS];
+  i32x4 q_low[RT][KSTEPS];
+  float q_scale[RT];
+  uint32_t row_limit[RT];  // tokens visible to this lane's query row
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const uint32_t matrix_row = 16u * rt + col;
+    const bool valid = matrix_row < matrix_rows;
+    const uint32_t row = valid ? matrix_row / group : 0u;
+    const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
+    const size_t record = static_cast<size_t>(row) * args.query_heads + head;
+    row_limit[rt] = args.first_context_tokens + row;
+    float values[KSTEPS][16];
+    float maximum = 0.0f;
+#pragma unroll
+    for (int h = 0; h < KSTEPS; ++h) {
+      const uint32_t d0 = 128u * (h / 2) + 32u * quad + 16u * (h % 2);
+#pragma unroll
+      for (int piece = 0; piece < 4; ++piece) {
+        float4 loaded = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (valid)
+          loaded = *reinterpret_cast<const float4*>(
+              args.query + record * args.query_stride + d0 + 4u * piece);
+        values[h][4 * piece + 0] = loaded.x;
+        values[h][4 * piece + 1] = loaded.y;
+        values[h][4 * piece + 2] = loaded.z;
+        values[h][4 * piece + 3] = loaded.w;
+        maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(loaded.x), fabsf(loaded.y)),
+                                       fmaxf(fabsf(loaded.z), fabsf(loaded.w))));
+      }
+    }
+    maximum = quad_row_max(maximum);
+    const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
+    const float inverse = 1.0f / scale;
+    q_scale[rt] = valid ? scale : 0.0f;
+#pragma unroll
+    for (int h = 0; h < KSTEPS; ++h) {
+      uint32_t high_bytes[16], low_bytes[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        int quantized = __float2int_rn(values[h][j] * inverse);
+        quantized = max(-16319, min(16319, quantized));
+        const int high = (quantized + 64) >> 7;  // floor((v+64)/128)
+        const int low = quantized - (high << 7);
+        high_bytes[j] = static_cast<uint32_t>(high) & 0xffu;
+        low_bytes[j] = static_cast<uint32_t>(low) & 0xffu;
+      }
+      // byte order inside each 8-element half: even d first, then odd d,
+      // matching the order in which the key nibbles are widened
+      const int order[16] = {0, 2, 4, 6, 1, 3, 5, 7, 8, 10, 12, 14, 9, 11, 13, 15};
+#pragma unroll
+      for (int word = 0; word < 4; ++word) {
+        uint32_t high_word = 0u, low_word = 0u;
+#pragma unroll
+        for (int byte = 0; byte < 4; ++byte) {
+          high_word |= high_bytes[order[4 * word + byte]] << (8 * byte);
+          low_word |= low_bytes[order[4 * word + byte]] << (8 * byte);
+        }
+        q_high[rt][h][word] = static_cast<int>(high_word);
+        q_low[rt][h][word] = static_cast<int>(low_word);
+      }
+    }
+  }
+  // score = int_dot/16 * q_scale * k_scale / sqrt(D), in log2 units
+  const float score_unit =
+      1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D)));
+
+  // ---- running state ---------------------------------------------------------
+  float running_max[RT];
+  float running_sum[RT];
+  f32x4 out[DT][RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    running_max[rt] = kMaskedMax;
+    running_sum[rt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
+  }
+
+  for (uint32_t tile = wave; tile < tiles; tile += kSplitWaves) {
+    const uint32_t tile_begin = split_begin + tile * 64u;
+    const void* page = args.page_table[tile_begin / args.page_tokens];
+    const Q4hPlanes planes = q4h_planes(page, args.layer, args.page_tokens,
+                                        args.kv_heads, D);
+    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
+                           tile_begin % args.page_tokens;
+
+    // K codes: sub-tile st (16 tokens), lane (token=col, quad) reads 16 bytes
+    uint4 key_raw[4][D / 128];
+#pragma unroll
+    for (int st = 0; st < 4; ++st)
+#pragma unroll
+      for (int c = 0; c < D / 128; ++c)
+        key_raw[st][c] = *reinterpret_cast<const uint4*>(
+            planes.key_codes + (record0 + 16u * st + col) * (D / 2) + 64u * c +
+            16u * quad);
+    // scales of tokens 16t + 4*quad + i (i = 0..3), t = 0..3
+    uint2 key_scale_raw[4];
+    uint2 value_scale_raw[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      key_scale_raw[t] = *reinterpret_cast<const uint2*>(
+          planes.key_scales + (record0 + 16u * t + 4u * quad) * 2u);
+      value_scale_raw[t] = *reinterpret_cast<const uint2*>(
+          planes.value_scales + (record0 + 16u * t + 4u * quad) * 2u);
+    }
+    // V codes -> LDS (token-major rows, padded), 16 tokens per pass
+#pragma unroll
+    for (int pass = 0; pass < 4 * (D / 128); ++pass) {
+      const uint32_t piece = pass * 64u + lane;          // 16-byte pieces
+      const uint32_t token = piece / (D / 32);           // D/32 pieces / token
+      const uint32_t part = piece % (D / 32);
+      const uint4 value = *reinterpret_cast<const uint4*>(
+          planes.value_codes + (record0 + token) * (D / 2) + part * 16u);
+      // LDS row of token T = 16*((T/4)%4) + 4*(T/16) + T%4, so the 16 tokens a
+      // lane group reads back transposed sit in 16 consecutive padded rows
+      const uint32_t stage_row =
+          16u * ((token >> 2) & 3u) + 4u * (token >> 4) + (token & 3u);
+      *reinterpret_cast<uint4*>(v_stage + stage_row * VROW + part * 16u) = value;
+    }
+
+    // ---- S = K . Q ------------------------------------------------------------
+    float score[RT][4][4];
+    const bool needs_mask = tile_begin + 64u > args.first_context_tokens;
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      i32x4 key_operand[KSTEPS];
+#pragma unroll
+      for (int c = 0; c < D / 128; ++c) {
+        const uint32_t x[4] = {key_raw[st][c].x, key_raw[st][c].y,
+                               key_raw[st][c].z, key_raw[st][c].w};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          i32x4 operand;
+          operand[0] = static_cast<int>((x[2 * half] << 4) & 0xf0f0f0f0u);
+          operand[1] = static_cast<int>(x[2 * half] & 0xf0f0f0f0u);
+          operand[2] = static_cast<int>((x[2 * half + 1] << 4) & 0xf0f0f0f0u);
+          operand[3] = static_cast<int>(x[2 * half + 1] & 0xf0f0f0f0u);
+          key_operand[2 * c + half] = operand;
+        }
+      }
+      const float k_scale[4] = {
+          f16_bits_to_f32(key_scale_raw[st].x & 0xffffu) * score_unit,
+          f16_bits_to_f32(key_scale_raw[st].x >> 16) * score_unit,
+          f16_bits_to_f32(key_scale_raw[st].y & 0xffffu) * score_unit,
+          f16_bits_to_f32(key_scale_raw[st].y >> 16) * score_unit};
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        i32x4 dot_high = {0, 0, 0, 0};
+        i32x4 dot_low = {0, 0, 0, 0};
+#pragma unroll
+        for (int h = 0; h < KSTEPS; ++h) {
+          dot_high = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+              key_operand[h], q_high[rt][h], dot_high, 0, 0, 0);
+          dot_low = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+              key_operand[h], q_low[rt][h], dot_low, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int dot = (dot_high[i] << 7) + dot_low[i];
+          float value = static_cast<float>(dot) * k_scale[i] * q_scale[rt];
+          if (needs_mask) {
+            const uint32_t token = tile_begin + 16u * st + 4u * quad + i;
+            if (token >= row_limit[rt]) value = -INFINITY;
+          }
+          score[rt][st][i] = value;
+        }
+      }
+    }
+
+    // ---- online softmax (lane owns query row `col` of each row tile) ----------
+    float new_max[RT];
+    bool grew = false;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float tile_max = score[rt][0][0];
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          tile_max = fmaxf(tile_max, score[rt][st][i]);
+      tile_max = quad_row_max(tile_max);
+      new_max[rt] = fmaxf(running_max[rt], tile_max);
+      grew = grew || new_max[rt] > running_max[rt];
+    }
+    if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const float factor = __builtin_amdgcn_exp2f(running_max[rt] - new_max[rt]);
+        running_max[rt] = new_max[rt];
+        running_sum[rt] *= factor;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+      }
+    }
+    // P^T operands: k-step u covers sub-tiles 2u, 2u+1; register c pairs the
+    // tokens (2u, i=c) and (2u+1, i=c)
+    f16x8 p_operand[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float p0 = __builtin_amdgcn_exp2f(score[rt][2 * u][c] - running_max[rt]);
+          const float p1 = __builtin_amdgcn_exp2f(score[rt][2 * u + 1][c] - running_max[rt]);
+          const _Float16 h0 = static_cast<_Float16>(p0);
+          const _Float16 h1 = static_cast<_Float16>(p1);
+          sum += static_cast<float>(h0) + static_cast<float>(h1);
+          p_operand[rt][u][2 * c] = h0;
+          p_operand[rt][u][2 * c + 1] = h1;
+        }
+      running_sum[rt] += sum;
+    }
+
+    // ---- V scales as f16 pairs matching the nibble pairing --------------------
+    // pair (u, c) = (scale[token 16*(2u) + 4*quad + c], scale[16*(2u+1) + ..])
+    f16x2 v_scale[2][4], v_scale16[2][4];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t even[2] = {value_scale_raw[2 * u].x, value_scale_raw[2 * u].y};
+      const uint32_t odd[2] = {value_scale_raw[2 * u + 1].x,
+                               value_scale_raw[2 * u + 1].y};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        uint32_t lo = (even[c / 2] >> (16 * (c % 2))) & 0xffffu;
+        uint32_t hi = (odd[c / 2] >> (16 * (c % 2))) & 0xffffu;
+        if (needs_mask) {
+          // never let uninitialised records (tokens no row can see) reach the
+          // matrix core: a NaN scale times a zero probability is still NaN
+          if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
+          if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context) hi = 0u;
+        }
+        const f16x2 pair = __builtin_bit_cast(f16x2, lo | (hi << 16));
+        v_scale[u][c] = pair;
+        v_scale16[u][c] = pair * static_cast<_Float16>(0.0625f);
+      }
+    }
+
+    // ---- O^T += V^T . P^T -------------------------------------------------------
+    __builtin_amdgcn_wave_barrier();
+    // lane (col, quad) supplies LDS row 16*quad + col, i.e. token
+    // 16*(col/4) + 4*quad + col%4 of the tile
+    const uint32_t stage_row = 16u * quad + col;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const i32x2 transposed = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
+          (__attribute__((address_space(3))) i32x2*)(v_stage +
+                                                     stage_row * VROW + dt * 8));
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint32_t x = static_cast<uint32_t>(transposed[u]) ^ 0x88888888u;
+        const uint32_t y = x >> 8;
+        f16x8 v_operand;
+        // 0x6400 | u is the binary16 number 1024 + u (u = code + 8); the
+        // subtraction is exact, the multiply rounds once.
+        const f16x2 offset0 = {static_cast<_Float16>(-1032.0f),
+                               static_cast<_Float16>(-1032.0f)};
+        const f16x2 offset1 = {static_cast<_Float16>(-1152.0f),
+                               static_cast<_Float16>(-1152.0f)};
+        const f16x2 e0 =
+            (__builtin_bit_cast(f16x2, (x & 0x000f000fu) | 0x64006400u) + offset0) *
+            v_scale[u][0];
+        const f16x2 e1 =
+            (__builtin_bit_cast(f16x2, (x & 0x00f000f0u) | 0x64006400u) + offset1) *
+            v_scale16[u][1];
+        const f16x2 e2 =
+            (__builtin_bit_cast(f16x2, (y & 0x000f000fu) | 0x64006400u) + offset0) *
+            v_scale[u][2];
+        const f16x2 e3 =
+            (__builtin_bit_cast(f16x2, (y & 0x00f000f0u) | 0x64006400u) + offset1) *
+            v_scale16[u][3];
+        v_operand[0] = e0[0]; v_operand[1] = e0[1];
+        v_operand[2] = e1[0]; v_operand[3] = e1[1];
+        v_operand[4] = e2[0]; v_operand[5] = e2[1];
+        v_operand[6] = e3[0]; v_operand[7] = e3[1];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          out[dt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+              v_operand, p_operand[rt][u], out[dt][rt], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // each lane summed only its own tokens
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) running_sum[rt] = quad_row_sum(running_sum[rt]);
+
+  // ---- merge the eight wave states in LDS (tree: 4+4, 2+2, 1+1) --------------
+  // state layout per wave slot: max[16*RT] | sum[16*RT] | out[16*RT][D]
+  float* slots = reinterpret_cast<float*>(lds_raw);
+  __syncthreads();  // V staging no longer needed
+#pragma unroll
+  for (int span = kSplitWaves / 2; span >= 1; span /= 2) {
+    if (wave >= static_cast<uint32_t>(span) &&
+        wave < static_cast<uint32_t>(2 * span)) {
+      float* slot = slots + (wave - span) * STATE;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (quad == 0u) {
+          slot[16 * rt + col] = running_max[rt];
+          slot[16 * RT + 16 * rt + col] = running_sum[rt];
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          *reinterpret_cast<f32x4*>(slot + 32 * RT + (16 * rt + col) * D +
+                                    16 * dt + 4 * quad) = out[dt][rt];
+      }
+    }
+    __syncthreads();
+    if (wave < static_cast<uint32_t>(span)) {
+      const float* slot = slots + wave * STATE;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const float other_max = slot[16 * rt + col];
+        const float other_sum = slot[16 * RT + 16 * rt + col];
+        const float merged = fmaxf(running_max[rt], other_max);
+        const float mine = __builtin_amdgcn_exp2f(running_max[rt] - merged);
+        const float theirs = __builtin_amdgcn_exp2f(other_max - merged);
+        running_max[rt] = merged;
+        running_sum[rt] = running_sum[rt] * mine + other_sum * theirs;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          const f32x4 other = *reinterpret_cast<const f32x4*>(
+              slot + 32 * RT + (16 * rt + col) * D + 16 * dt + 4 * quad);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            out[dt][rt][i] = out[dt][rt][i] * mine + other[i] * theirs;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  if (wave != 0u) return;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const uint32_t matrix_row = 16u * rt + col;
+    if (matrix_row >= matrix_rows) continue;
+    const uint32_t row = matrix_row / group;
+    const uint32_t head = kv_head * group + matrix_row % group;
+    const size_t partial =
+        (static_cast<size_t>(row) * args.maximum_splits + split) *
+            args.query_heads + head;
+    if (quad == 0u) {
+      args.partial_maxima[partial] = running_max[rt];
+      args.partial_sums[partial] = running_sum[rt];
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<f32x4*>(args.partial_outputs + partial * D + 16 * dt +
+                                4 * quad) = out[dt][rt];
+  }
+}
+
+// Split-K merge (maxima in log2 units), optional sigmoid output gate.
+__global__ void attention_combine_kernel(
+    const float* query, uint32_t query_stride, int output_gated,
+    const float* partial_maxima, const float* partial_sums,
+    const float* partial_outputs, void* output, uint32_t output_kind,
+    uint32_t first_context_tokens, uint32_t maximum_splits,
+    uint32_t split_tokens, uint32_t query_heads, uint32_t head_dim) {
+  const uint32_t head = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t dimension = threadIdx.x;
+  const uint32_t active =
+      (first_context_tokens + row + split_tokens - 1u) / split_tokens;
+  float maximum = kMaskedMax;
+  for (uint32_t split = 0; split < active; ++split)
+    maximum = fmaxf(
+        maximum, partial_maxima[(static_cast<size_t>(row) * maximum_splits +
+                                 split) * query_heads + head]);
+  float sum = 0.0f;
+  float result = 0.0f;
+  for (uint32_t split = 0; split < active; ++split) {
+    const size_t partial =
+        (static_cast<size_t>(row) * maximum_splits + split) * query_heads + head;
+    const float weight = __builtin_amdgcn_exp2f(partial_maxima[partial] - maximum);
+    sum += partial_sums[partial] * weight;
+    if (dimension < head_dim)
+      result += partial_outputs[partial * head_dim + dimension] * weight;
+  }
+  if (dimension >= head_dim) return;
+  result /= sum;
+  const size_t record = static_cast<size_t>(row) * query_heads + head;
+  if (output_gated) {
+    const float gate = query[record * query_stride + head_dim + dimension];
+    result *= 1.0f / (1.0f + expf(-gate));
+  }
+  const size_t index = record * head_dim + dimension;
+  if (output_kind == QLLM_OUT_BF16)
+    static_cast<uint16_t*>(output)[index] =
+        static_cast<uint16_t>(f32_to_bf16_bits(result));
+  else
+    static_cast<float*>(output)[index] = result;
+}
+
+// ---- K/V store ----------------------------------------------------------------
+
+// One wave encodes one (token, kv head) K or V vector.
+__device__ __forceinline__ void q4h_encode_record(const float* source,
+                                                  uint32_t head_dim,
+                                                  uint8_t* codes,
+                                                  uint8_t* scale_slot,
+                                                  uint32_t lane) {
+  float maximum = 0.0f;
+  for (uint32_t index = lane; index < head_dim; index += 64u)
+    maximum = fmaxf(maximum, fabsf(source[index]));
+  maximum = wave_max(maximum);
+  const uint32_t scale_bits =
+      f32_to_f16_bits(fmaxf(__fdiv_rn(maximum, 7.0f), 0x1p-24f));
+  const float scale = f16_bits_to_f32(scale_bits);
+  if (lane == 0u)
+    *reinterpret_cast<uint16_t*>(scale_slot) = static_cast<uint16_t>(scale_bits);
+  for (uint32_t pair = lane; pair < head_dim / 2u; pair += 64u) {
+    const int low = max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair], scale))));
+    const int high =
+        max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair + 1u], scale))));
+    codes[pair] = static_cast<uint8_t>((low & 0x0f) | ((high & 0x0f) << 4));
+  }
+}
+
+__global__ __launch_bounds__(64) void q4h_store_kernel(
+    const float* key, const float* value, const void* const* page_table,
+    uint32_t layer, uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t kv_heads, uint32_t head_dim) {
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t lane = threadIdx.x;
+  const uint32_t position = first_cache_position + row;
+  uint8_t* page = static_cast<uint8_t*>(
+      const_cast<void*>(page_table[position / page_tokens]));
+  const Q4hPlanes planes =
+      q4h_planes(page, layer, page_tokens, kv_heads, head_dim);
+  const size_t record =
+      static_cast<size_t>(kv_head) * page_tokens + position % page_tokens;
+  const size_t source = (static_cast<size_t>(row) * kv_heads + kv_head) * head_dim;
+  q4h_encode_record(key + source, head_dim,
+                    const_cast<uint8_t*>(planes.key_codes) + record * (head_dim / 2u),
+                    const_cast<uint8_t*>(planes.key_scales) + record * 2u, lane);
+  q4h_encode_record(value + source, head_dim,
+                    const_cast<uint8_t*>(planes.value_codes) + record * (head_dim / 2u),
+                    const_cast<uint8_t*>(planes.value_scales) + record * 2u, lane);
+}
+
+// Per-head RMSNorm(1+w) and NeoX rotary, in place; one wave per (head, row).
+// Blocks with head < kv_heads also process the K row.
+__device__ __forceinline__ void head_norm_rope(float* x, const float* weight,
+                                               uint32_t head_dim,
+                                               uint32_t rotary_dim,
+                                               uint32_t position, float epsilon,
+                                               float theta, bool bf16_activations,
+                                               float* shared, uint32_t lane) {
+  if (weight) {
+    float square = 0.0f;
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      square = fmaf(x[index], x[index], square);
+    square = wave_sum(square);
+    const float inverse =
+        rsqrtf(square / static_cast<float>(head_dim) + epsilon);
+    for (uint32_t index = lane; index < head_dim; index += 64u) {
+      const float value = x[index] * inverse * (1.0f + weight[index]);
+      shared[index] = bf16_activations ? bf16_round(value) : value;
+    }
+  } else {
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      shared[index] = x[index];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t half = rotary_dim / 2u;
+  for (uint32_t index = lane; index < head_dim; index += 64u) {
+    float result = shared[index];
+    if (index < rotary_dim) {
+      const uint32_t pair = index % half;
+      const float angle =
+          static_cast<float>(position) *
+          powf(theta, -2.0f * static_cast<float>(pair) /
+                          static_cast<float>(rotary_dim));
+      const float other =
+          index < half ? -shared[index + half] : shared[index - half];
+      float cosine = cosf(angle);
+      float sine = sinf(angle);
+      if (bf16_activations) {
+        cosine = bf16_round(cosine);
+        sine = bf16_round(sine);
+      }
+      result = shared[index] * cosine + other * sine;
+    }
+    x[index] = bf16_activations ? bf16_round(result) : result;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+__global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_weight, const float* k_weight,
+    const void* const* page_table, uint32_t layer, uint32_t page_tokens,
+    uint32_t first_cache_position, uint32_t first_rotary_position,
+    uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations) {
+  __shared__ float shared[256];
+  const uint32_t head = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t lane = threadIdx.x;
+  const uint32_t rotary_position = first_rotary_position + row;
+  float* q = query + (static_cast<size_t>(row) * query_heads + head) * query_stride;
+  head_norm_rope(q, q_weight, head_dim, rotary_dim, rotary_position, epsilon,
+                 theta, bf16_activations, shared, lane);
+  if (head >= kv_heads) return;
+  float* k = key + (static_cast<size_t>(row) * kv_heads + head) * head_dim;
+  head_norm_rope(k, k_weight, head_dim, rotary_dim, rotary_position, epsilon,
+                 theta, bf16_activations, shared, lane);
+  __threadfence_block();
+  const uint32_t position = first_cache_position + row;
+  uint8_t* page = static_cast<uint8_t*>(
+      const_cast<void*>(page_table[position / page_tokens]));
+  const Q4hPlanes planes =
+      q4h_planes(page, layer, page_tokens, kv_heads, head_dim);
+  const size_t record =
+      static_cast<size_t>(head) * page_tokens + position % page_tokens;
+  q4h_encode_record(k, head_dim,
+                    const_cast<uint8_t*>(planes.key_codes) + record * (head_dim / 2u),
+                    const_cast<uint8_t*>(planes.key_scales) + record * 2u, lane);
+  q4h_encode_record(value + (static_cast<size_t>(row) * kv_heads + head) * head_dim,
+                    head_dim,
+                    const_cast<uint8_t*>(planes.value_codes) + record * (head_dim / 2u),
+                    const_cast<uint8_t*>(planes.value_scales) + record * 2u, lane);
+}
+
+// transformer_kernels.cu:4391-4416
+__global__ __launch_bounds__(64) void quantize_queries_q8_kernel(
+    const float* query, uint32_t query_stride, int8_t* q8, float* scales,
+    uint32_t query_heads, uint32_t head_dim) {
+  const uint32_t head = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t lane = threadIdx.x;
+  const size_t record = static_cast<size_t>(row) * query_heads + head;
+  const float* source = query + record * query_stride;
+  float maximum = 0.0f;
+  for (uint32_t index = lane; index < head_dim; index += 64u)
+    maximum = fmaxf(maximum, fabsf(source[index]));
+  maximum = wave_max(maximum);
+  const float scale = fmaxf(__fdiv_rn(maximum, 127.0f), 0x1p-24f);
+  if (lane == 0u) scales[record] = scale;
+  for (uint32_t index = lane; index < head_dim; index += 64u) {
+    const int quantized =
+        max(-127, min(127, __float2int_rn(__fdiv_rn(source[index], scale))));
+    q8[record * head_dim + index] = static_cast<int8_t>(quantized);
+  }
+}
+
+template <int D>
+int32_t launch_split(const SplitArgs& args, uint32_t row_tiles, dim3 grid,
+                     hipStream_t stream) {
+  constexpr size_t stage = static_cast<size_t>(kSplitWaves) * 64 * (D / 2 + 16);
+  const size_t merge = static_cast<size_t>(kSplitWaves / 2) * 16 * row_tiles *
+                       (D + 2) * sizeof(float);
+  const size_t lds = stage > merge ? stage : merge;
+  switch (row_tiles) {
+    case 1:
+      q4h_attention_split_kernel<D, 1><<<grid, kSplitWaves * 64, lds, stream>>>(args);
+      break;
+    case 2:
+      q4h_attention_split_kernel<D, 2><<<grid, kSplitWaves * 64, lds, stream>>>(args);
+      break;
+    default:
+      if constexpr (D == 128) {
+        q4h_attention_split_kernel<D, 3>
+            <<<grid, kSplitWaves * 64, lds, stream>>>(args);
+        break;
+      } else {
+        return fail(QLLM_INVALID_ARGUMENT,
+                    "Q4H attention: three row tiles need head_dim 128");
+      }
+  }
+  return launched("Q4H attention split");
+}
+
+}  // namespace
+
+// shared with the exact-F16 path
+int32_t launch_attention_combine(const float* query, uint32_t query_stride,
+                                 int output_gated, const float* partial_maxima,
+                                 const float* partial_sums,
+                                 const float* partial_outputs, void* output,
+                                 uint32_t output_kind,
+                                 uint32_t first_context_tokens,
+                                 uint32_t maximum_splits, uint32_t split_tokens,
+                                 uint32_t rows, uint32_t query_heads,
+                                 uint32_t head_dim, hipStream_t stream) {
+  const dim3 grid(query_heads, rows);
+  attention_combine_kernel<<<grid, head_dim, 0, stream>>>(
+      query, query_stride, output_gated, partial_maxima, partial_sums,
+      partial_outputs, output, output_kind, first_context_tokens,
+      maximum_splits, split_tokens, query_heads, head_dim);
+  return launched("attention split combine");
+}
+
+}  // namespace qllm
+
+using namespace qllm;
+
+extern "C" size_t qllm_q4h_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                                       uint32_t head_dim) {
+  return q4h_layer_bytes(page_tokens, kv_heads, head_dim);
+}
+
+extern "C" int32_t qllm_store_kv_paged_q4h_batch(
+    const float* key, const float* value, const void* const* page_table,
+    uint32_t full_attention_layer, uint32_t page_tokens,
+    uint32_t first_cache_position, uint32_t rows, uint32_t kv_heads,
+    uint32_t head_dim, void* stream) {
+  if (!key || !value || !page_table || !page_tokens || !rows || !kv_heads ||
+      !head_dim || head_dim % 2u || head_dim > 256u ||
+      first_cache_position > 0xffffffffu - (rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H K/V store");
+  q4h_store_kernel<<<dim3(kv_heads, rows), 64, 0, as_stream(stream)>>>(
+      key, value, page_table, full_attention_layer, page_tokens,
+      first_cache_position, kv_heads, head_dim);
+  return launched("Q4H K/V store");
+}
+
+extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream) {
+  if (!query || !key || !value || !page_table || !page_tokens || !rows ||
+      !query_heads || !kv_heads || query_heads < kv_heads ||
+      query_heads % kv_heads || !head_dim || head_dim > 256u || head_dim % 2u ||
+      query_stride < head_dim || !rotary_dim || rotary_dim > head_dim ||
+      rotary_dim % 2u || !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
+      first_cache_position > 0xffffffffu - (rows - 1u) ||
+      first_rotary_position > 0xffffffffu - (rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H QKV rope cache batch");
+  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+      query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
+      full_attention_layer, page_tokens, first_cache_position,
+      first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
+      epsilon, rope_theta, bf16_activations != 0);
+  return launched("Q4H QKV rope cache batch");
+}
+
+extern "C" int32_t qllm_quantize_gqa_queries_q8(
+    const float* query, uint32_t query_stride, int8_t* q8, float* query_scales,
+    uint32_t rows, uint32_t query_heads, uint32_t head_dim, void* stream) {
+  if (!query || !q8 || !query_scales || !rows || !query_heads || !head_dim ||
+      query_stride < head_dim)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid GQA query Q8 quantization");
+  quantize_queries_q8_kernel<<<dim3(query_heads, rows), 64, 0,
+                               as_stream(stream)>>>(
+      query, query_stride, q8, query_scales, query_heads, head_dim);
+  return launched("GQA query Q8 quantization");
+}
+
+extern "C" int32_t qllm_attention_paged_q4h(
+    const qllm_q4h_attention_launch* launch) {
+  if (!launch || !launch->query || !launch->page_table || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u ||
+      !launch->partial_maxima || !launch->partial_sums ||
+      !launch->partial_outputs || !launch->first_context_tokens ||
+      !launch->rows || !launch->page_tokens || launch->page_tokens % 64u ||
+      !launch->query_heads || !launch->kv_heads ||
+      launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      !launch->split_tokens || launch->split_tokens % 64u ||
+      !launch->maximum_splits ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t matrix_rows = launch->rows * group;
+  const uint32_t row_tiles = (matrix_rows + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q4H paged attention: rows * (query_heads/kv_heads) exceeds "
+                "48 (32 at head_dim 256)");
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      (last_context + launch->split_tokens - 1u) / launch->split_tokens;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q4H paged attention: context needs more splits than "
+                "maximum_splits");
+  SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.page_table = launch->page_table;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.layer = launch->full_attention_layer;
+  args.page_tokens = launch->page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  const dim3 grid(launch->kv_heads, splits);
+  const hipStream_t stream = as_stream(launch->stream);
+  int32_t status = launch->head_dim == 128u
+                       ? launch_split<128>(args, row_tiles, grid, stream)
+                       : launch_split<256>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, stream);
+}

@@ -1,0 +1,294 @@
+// Small per-row kernels of the verify step: activation quantisation,
+// embedding gather, RMSNorm, residual add, SiLU product, synthetic fills.
+// Each replaces the reference launcher named beside its entry point.
+#include "common.hpp"
+
+#include <cstdio>
+#include <cstring>
+
+namespace qllm {
+
+namespace {
+thread_local char last_error[256] = "";
+}
+
+int32_t fail(int32_t code, const char* message) {
+  std::snprintf(last_error, sizeof(last_error), "%s", message);
+  return code;
+}
+
+int32_t checked(hipError_t error, const char* what) {
+  if (error == hipSuccess) return QLLM_OK;
+  std::snprintf(last_error, sizeof(last_error), "%s: %s", what,
+                hipGetErrorString(error));
+  return QLLM_INTERNAL;
+}
+
+namespace {
+
+// transformer_kernels.cu:912-946
+__global__ __launch_bounds__(256) void quantize_q8_batch_kernel(
+    const float* input, int8_t* output, float* scales, uint32_t columns,
+    uint32_t padded_columns, bool bf16_input) {
+  __shared__ float scratch[4];
+  const uint32_t row = blockIdx.x;
+  const float* source = input + static_cast<size_t>(row) * columns;
+  int8_t* target = output + static_cast<size_t>(row) * padded_columns;
+  float maximum = 0.0f;
+  for (uint32_t column = threadIdx.x; column < columns; column += blockDim.x) {
+    const float value = bf16_input ? bf16_round(source[column]) : source[column];
+    maximum = fmaxf(maximum, fabsf(value));
+  }
+  maximum = block_max(maximum, scratch);
+  const float scale = maximum > 0.0f ? maximum / 127.0f : 1.0f;
+  if (threadIdx.x == 0) scales[row] = scale;
+  for (uint32_t column = threadIdx.x; column < padded_columns;
+       column += blockDim.x) {
+    int quantized = 0;
+    if (column < columns) {
+      const float value =
+          bf16_input ? bf16_round(source[column]) : source[column];
+      quantized = __float2int_rn(__fdiv_rn(value, scale));
+    }
+    quantized = max(-127, min(127, quantized));
+    target[column] = static_cast<int8_t>(quantized);
+  }
+}
+
+// transformer_kernels.cu:948-959
+__global__ __launch_bounds__(256) void convert_f32_to_bf16_batch_kernel(
+    const float* input, uint16_t* output, uint32_t columns,
+    uint32_t padded_columns) {
+  const uint32_t row = blockIdx.x;
+  const float* source = input + static_cast<size_t>(row) * columns;
+  uint16_t* target = output + static_cast<size_t>(row) * padded_columns;
+  for (uint32_t column = threadIdx.x; column < padded_columns;
+       column += blockDim.x)
+    target[column] = column < columns
+                         ? static_cast<uint16_t>(f32_to_bf16_bits(source[column]))
+                         : 0u;
+}
+
+// transformer_kernels.cu:801-821
+__global__ __launch_bounds__(256) void fp4_embedding_batch_kernel(
+    const uint8_t* weights, const uint8_t* scales, uint32_t scheme,
+    const uint32_t* tokens, float* output, uint32_t columns,
+    uint32_t padded_columns) {
+  const uint32_t request = blockIdx.x;
+  const size_t token = tokens[request];
+  const uint8_t* row_codes = weights + token * (padded_columns / 2u);
+  for (uint32_t column = threadIdx.x; column < columns; column += blockDim.x) {
+    const uint8_t byte = row_codes[column / 2u];
+    const uint32_t code = (column & 1u) ? byte >> 4 : byte & 0x0fu;
+    const uint32_t index = code & 7u;
+    const float twice = index <= 4u ? static_cast<float>(index)
+                        : index == 5u ? 6.0f
+                        : index == 6u ? 8.0f
+                                      : 12.0f;
+    float scale;
+    if (scheme == QLLM_SCALE_F16_BLOCK16)
+      scale = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(
+          scales)[token * (padded_columns / 16u) + column / 16u]);
+    else
+      scale = ue8m0_to_f32(scales[token * (padded_columns / 32u) + column / 32u]);
+    const float value = twice * 0.5f * scale;
+    output[static_cast<size_t>(request) * columns + column] =
+        (code & 8u) ? -value : value;
+  }
+}
+
+// transformer_kernels.cu:2469-2521
+__global__ __launch_bounds__(256) void rms_norm_batch_kernel(
+    const float* input, const float* weight, float* output_f32,
+    uint16_t* output_bf16, uint32_t bf16_padded_columns, uint32_t elements,
+    float epsilon, bool zero_centered) {
+  __shared__ float scratch[4];
+  const uint32_t row = blockIdx.x;
+  const float* x = input + static_cast<size_t>(row) * elements;
+  float square = 0.0f;
+  for (uint32_t index = threadIdx.x; index < elements; index += blockDim.x)
+    square = fmaf(x[index], x[index], square);
+  square = block_sum(square, scratch);
+  const float inverse =
+      rsqrtf(square / static_cast<float>(elements) + epsilon);
+  const uint32_t limit = output_bf16 && bf16_padded_columns > elements
+                             ? bf16_padded_columns
+                             : elements;
+  for (uint32_t index = threadIdx.x; index < limit; index += blockDim.x) {
+    float value = 0.0f;
+    if (index < elements) {
+      float factor = 1.0f;
+      if (weight) factor = zero_centered ? 1.0f + weight[index] : weight[index];
+      value = x[index] * inverse * factor;
+      if (output_f32)
+        output_f32[static_cast<size_t>(row) * elements + index] = value;
+    }
+    if (output_bf16)
+      output_bf16[static_cast<size_t>(row) * bf16_padded_columns + index] =
+          static_cast<uint16_t>(f32_to_bf16_bits(value));
+  }
+}
+
+// transformer_kernels.cu:2522-2528
+__global__ void add_kernel(float* destination, const float* source,
+                           uint32_t count, bool bf16_output) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) {
+    const float value = destination[i] + source[i];
+    destination[i] = bf16_output ? bf16_round(value) : value;
+  }
+}
+
+// transformer_kernels.cu:2774-2783
+__global__ void silu_product_kernel(const float* gate, const float* up,
+                                    float* output, uint32_t count,
+                                    bool bf16_activations) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) {
+    float activated = gate[i] / (1.0f + expf(-gate[i]));
+    if (bf16_activations) activated = bf16_round(activated);
+    const float value = activated * up[i];
+    output[i] = bf16_activations ? bf16_round(value) : value;
+  }
+}
+
+__device__ __forceinline__ float uniform_open(uint64_t bits) {
+  return (static_cast<float>(bits >> 40) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+__device__ __forceinline__ float normal_from(uint64_t seed, uint64_t index) {
+  const float u1 = uniform_open(mix64(seed, 2u * index));
+  const float u2 = uniform_open(mix64(seed, 2u * index + 1u));
+  return sqrtf(-2.0f * logf(u1)) * cosf(6.2831853f * u2);
+}
+
+__global__ void fill_random_kernel(void* destination, size_t elements,
+                                   uint32_t kind, uint64_t seed) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t index = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+       index < elements; index += stride) {
+    switch (kind) {
+      case 0:
+        static_cast<uint8_t*>(destination)[index] =
+            static_cast<uint8_t>(mix64(seed, index) >> 24);
+        break;
+      case 1:
+        static_cast<float*>(destination)[index] = normal_from(seed, index);
+        break;
+      case 2:
+        static_cast<uint16_t*>(destination)[index] =
+            static_cast<uint16_t>(f32_to_bf16_bits(normal_from(seed, index)));
+        break;
+      case 3:
+        static_cast<uint16_t*>(destination)[index] = static_cast<uint16_t>(
+            f32_to_f16_bits(expf(0.5f * normal_from(seed, index))));
+        break;
+      case 4:
+        static_cast<uint16_t*>(destination)[index] =
+            static_cast<uint16_t>(f32_to_f16_bits(normal_from(seed, index)));
+        break;
+      default:
+        static_cast<uint8_t*>(destination)[index] =
+            static_cast<uint8_t>(124u + (mix64(seed, index) >> 32) % 7u);
+        break;
+    }
+  }
+}
+
+}  // namespace
+}  // namespace qllm
+
+using namespace qllm;
+
+extern "C" const char* qllm_last_error(void) { return last_error; }
+
+extern "C" const char* qllm_version(void) { return "qllm-hip gfx950 1"; }
+
+extern "C" int32_t qllm_quantize_q8_batch(const float* input, int8_t* output,
+                                          float* scales, uint32_t rows,
+                                          uint32_t columns,
+                                          uint32_t padded_columns,
+                                          int32_t bf16_input, void* stream) {
+  if (!input || !output || !scales || !rows || !columns ||
+      padded_columns < columns)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 batch quantization");
+  quantize_q8_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
+      input, output, scales, columns, padded_columns, bf16_input != 0);
+  return launched("quantize Q8 batch");
+}
+
+extern "C" int32_t qllm_convert_f32_to_bf16_batch(
+    const float* input, void* output, size_t output_bytes, uint32_t rows,
+    uint32_t columns, uint32_t padded_columns, void* stream) {
+  if (!input || !output || !rows || !columns || padded_columns < columns ||
+      output_bytes < static_cast<size_t>(rows) * padded_columns * 2u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid F32 to BF16 conversion");
+  convert_f32_to_bf16_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
+      input, static_cast<uint16_t*>(output), columns, padded_columns);
+  return launched("convert F32 to BF16");
+}
+
+extern "C" int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
+                                            const uint32_t* tokens,
+                                            float* output, uint32_t batch,
+                                            void* stream) {
+  if (!matrix || !matrix->weights || !matrix->scales || !matrix->rows ||
+      !matrix->columns || matrix->padded_columns < matrix->columns ||
+      matrix->padded_columns % 32u || matrix->scale_scheme > 1u || !tokens ||
+      !output || !batch)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 embedding batch");
+  fp4_embedding_batch_kernel<<<batch, 256, 0, as_stream(stream)>>>(
+      matrix->weights, static_cast<const uint8_t*>(matrix->scales),
+      matrix->scale_scheme, tokens, output, matrix->columns,
+      matrix->padded_columns);
+  return launched("FP4 embedding batch");
+}
+
+extern "C" int32_t qllm_rms_norm_batch(const float* input, const float* weight,
+                                       float* output_f32, void* output_bf16,
+                                       uint32_t bf16_padded_columns,
+                                       uint32_t rows, uint32_t elements,
+                                       float epsilon, int32_t zero_centered,
+                                       void* stream) {
+  if (!input || (!output_f32 && !output_bf16) || !rows || !elements ||
+      !(epsilon > 0.0f) ||
+      (output_bf16 && bf16_padded_columns < elements))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid RMSNorm batch");
+  rms_norm_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
+      input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
+      bf16_padded_columns, elements, epsilon, zero_centered != 0);
+  return launched("RMSNorm batch");
+}
+
+extern "C" int32_t qllm_add_in_place(float* destination, const float* source,
+                                     uint32_t elements, int32_t bf16_output,
+                                     void* stream) {
+  if (!destination || !source || !elements)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid residual add");
+  add_kernel<<<(elements + 255u) / 256u, 256, 0, as_stream(stream)>>>(
+      destination, source, elements, bf16_output != 0);
+  return launched("residual add");
+}
+
+extern "C" int32_t qllm_silu_product(const float* gate, const float* up,
+                                     float* output, uint32_t elements,
+                                     int32_t bf16_activations, void* stream) {
+  if (!gate || !up || !output || !elements)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid SiLU product");
+  silu_product_kernel<<<(elements + 255u) / 256u, 256, 0, as_stream(stream)>>>(
+      gate, up, output, elements, bf16_activations != 0);
+  return launched("SiLU product");
+}
+
+extern "C" int32_t qllm_fill_random(void* destination, size_t elements,
+                                    uint32_t kind, uint64_t seed,
+                                    void* stream) {
+  if (!destination || !elements || kind > 5u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid random fill");
+  const size_t blocks = (elements + 255u) / 256u;
+  const unsigned grid =
+      static_cast<unsigned>(blocks < 65536u ? blocks : 65536u);
+  fill_random_kernel<<<grid, 256, 0, as_stream(stream)>>>(destination, elements,
+                                                          kind, seed);
+  return launched("random fill");
+}

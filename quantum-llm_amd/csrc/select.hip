@@ -1,0 +1,258 @@
+// Token selection over the lm_head logits: batched argmax, exact descending
+// top-k and the presence penalty.  Replaces argmax_batch_kernel,
+// topk_logits_partials_kernel / topk_logits_reduce_kernel and
+// presence_penalty_kernel (runtime/src/cuda/transformer_kernels.cu:7059-7186).
+// Ordering rule everywhere: larger value first, equal values by lower index,
+// NaN never selected.
+#include "common.hpp"
+
+namespace qllm {
+namespace {
+
+constexpr uint32_t kNoIndex = 0xffffffffu;
+constexpr uint32_t kArgmaxChunk = 8192;   // items per stage-1 block
+constexpr uint32_t kTopkChunk = 4096;     // items per stage-1 block
+constexpr uint32_t kTopkThreads = 256;
+constexpr uint32_t kTopkPerThread = kTopkChunk / kTopkThreads;
+
+__device__ __forceinline__ bool better(float value, uint32_t index, float best,
+                                       uint32_t best_index) {
+  return value > best || (value == best && index < best_index);
+}
+
+__device__ __forceinline__ void wave_best(float& value, uint32_t& index) {
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) {
+    const float other = __shfl_xor(value, offset, 64);
+    const uint32_t other_index = __shfl_xor(index, offset, 64);
+    if (better(other, other_index, value, index)) {
+      value = other;
+      index = other_index;
+    }
+  }
+}
+
+// Block-wide best; result valid in every thread.
+__device__ __forceinline__ void block_best(float& value, uint32_t& index,
+                                           float* values, uint32_t* indices) {
+  wave_best(value, index);
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t waves = (blockDim.x + 63u) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63u) == 0u) {
+    values[wave] = value;
+    indices[wave] = index;
+  }
+  __syncthreads();
+  value = values[0];
+  index = indices[0];
+  for (uint32_t other = 1; other < waves; ++other)
+    if (better(values[other], indices[other], value, index)) {
+      value = values[other];
+      index = indices[other];
+    }
+}
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(
+    const float* values, uint32_t count, float* partial_values,
+    uint32_t* partial_indices, uint32_t blocks_per_row) {
+  __shared__ float shared_values[4];
+  __shared__ uint32_t shared_indices[4];
+  const uint32_t request = blockIdx.y;
+  const float* row = values + static_cast<size_t>(request) * count;
+  const uint32_t first = blockIdx.x * kArgmaxChunk;
+  const uint32_t last = min(count, first + kArgmaxChunk);
+  float best = -INFINITY;
+  uint32_t index = kNoIndex;
+  for (uint32_t item = first + threadIdx.x; item < last; item += blockDim.x) {
+    const float value = row[item];
+    if (better(value, item, best, index)) {
+      best = value;
+      index = item;
+    }
+  }
+  block_best(best, index, shared_values, shared_indices);
+  if (threadIdx.x == 0u) {
+    partial_values[request * blocks_per_row + blockIdx.x] = best;
+    partial_indices[request * blocks_per_row + blockIdx.x] = index;
+  }
+}
+
+__global__ __launch_bounds__(256) void argmax_final_kernel(
+    const float* partial_values, const uint32_t* partial_indices,
+    uint32_t blocks_per_row, uint32_t* output) {
+  __shared__ float shared_values[4];
+  __shared__ uint32_t shared_indices[4];
+  const uint32_t request = blockIdx.x;
+  float best = -INFINITY;
+  uint32_t index = kNoIndex;
+  for (uint32_t item = threadIdx.x; item < blocks_per_row; item += blockDim.x) {
+    const float value = partial_values[request * blocks_per_row + item];
+    const uint32_t candidate = partial_indices[request * blocks_per_row + item];
+    if (better(value, candidate, best, index)) {
+      best = value;
+      index = candidate;
+    }
+  }
+  block_best(best, index, shared_values, shared_indices);
+  if (threadIdx.x == 0u) output[request] = index;
+}
+
+// Stage 1: every block extracts the top_k of its chunk, in order, by top_k
+// rounds of "block argmax, winner retires".  Stage 2 (one block) does the
+// same over the stage-1 survivors.  Items live in registers.
+template <uint32_t PER_THREAD>
+__device__ __forceinline__ void select_rounds(float (&value)[PER_THREAD],
+                                              uint32_t (&index)[PER_THREAD],
+                                              uint32_t top_k, float* out_values,
+                                              uint32_t* out_indices,
+                                              float* shared_values,
+                                              uint32_t* shared_indices) {
+  for (uint32_t rank = 0; rank < top_k; ++rank) {
+    float best = -INFINITY;
+    uint32_t best_index = kNoIndex;
+#pragma unroll
+    for (uint32_t slot = 0; slot < PER_THREAD; ++slot)
+      if (index[slot] != kNoIndex &&
+          better(value[slot], index[slot], best, best_index)) {
+        best = value[slot];
+        best_index = index[slot];
+      }
+    block_best(best, best_index, shared_values, shared_indices);
+    if (threadIdx.x == 0u) {
+      out_values[rank] = best;
+      out_indices[rank] = best_index;
+    }
+    if (best_index == kNoIndex) {
+      // fewer than top_k candidates: pad the remaining ranks
+      for (uint32_t rest = rank + 1u + threadIdx.x; rest < top_k;
+           rest += blockDim.x) {
+        out_values[rest] = -INFINITY;
+        out_indices[rest] = kNoIndex;
+      }
+      return;
+    }
+#pragma unroll
+    for (uint32_t slot = 0; slot < PER_THREAD; ++slot)
+      if (index[slot] == best_index) index[slot] = kNoIndex;
+  }
+}
+
+__global__ __launch_bounds__(kTopkThreads) void topk_partial_kernel(
+    const float* values, uint32_t count, uint32_t top_k, float* partial_values,
+    uint32_t* partial_indices) {
+  __shared__ float shared_values[4];
+  __shared__ uint32_t shared_indices[4];
+  const uint32_t first = blockIdx.x * kTopkChunk;
+  float value[kTopkPerThread];
+  uint32_t index[kTopkPerThread];
+#pragma unroll
+  for (uint32_t slot = 0; slot < kTopkPerThread; ++slot) {
+    const uint32_t item = first + slot * kTopkThreads + threadIdx.x;
+    float loaded = item < count ? values[item] : NAN;
+    const bool usable = item < count && !isnan(loaded);
+    value[slot] = usable ? loaded : -INFINITY;
+    index[slot] = usable ? item : kNoIndex;
+  }
+  select_rounds<kTopkPerThread>(value, index, top_k,
+                                partial_values + blockIdx.x * top_k,
+                                partial_indices + blockIdx.x * top_k,
+                                shared_values, shared_indices);
+}
+
+constexpr uint32_t kMergeThreads = 1024;
+constexpr uint32_t kMergePerThread = 40;  // up to 40960 survivors
+
+__global__ __launch_bounds__(kMergeThreads) void topk_merge_kernel(
+    const float* partial_values, const uint32_t* partial_indices,
+    uint32_t survivors, uint32_t top_k, float* output_values,
+    uint32_t* output_indices) {
+  __shared__ float shared_values[16];
+  __shared__ uint32_t shared_indices[16];
+  float value[kMergePerThread];
+  uint32_t index[kMergePerThread];
+#pragma unroll
+  for (uint32_t slot = 0; slot < kMergePerThread; ++slot) {
+    const uint32_t item = slot * kMergeThreads + threadIdx.x;
+    const bool usable = item < survivors && partial_indices[item] != kNoIndex;
+    value[slot] = usable ? partial_values[item] : -INFINITY;
+    index[slot] = usable ? partial_indices[item] : kNoIndex;
+  }
+  select_rounds<kMergePerThread>(value, index, top_k, output_values,
+                                 output_indices, shared_values, shared_indices);
+}
+
+// transformer_kernels.cu:7180-7186
+__global__ void presence_penalty_kernel(float* logits, const uint8_t* emitted,
+                                        uint32_t count, float penalty) {
+  const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
+  if (index < count && emitted[index] != 0u) logits[index] -= penalty;
+}
+
+}  // namespace
+}  // namespace qllm
+
+using namespace qllm;
+
+extern "C" size_t qllm_argmax_workspace_bytes(uint32_t count, uint32_t batch) {
+  const size_t blocks = (static_cast<size_t>(count) + kArgmaxChunk - 1u) / kArgmaxChunk;
+  return blocks * batch * (sizeof(float) + sizeof(uint32_t));
+}
+
+extern "C" int32_t qllm_argmax_batch(const float* values, uint32_t count,
+                                     uint32_t batch, uint32_t* output,
+                                     void* workspace, size_t workspace_bytes,
+                                     void* stream) {
+  if (!values || !count || !batch || !output || !workspace ||
+      workspace_bytes < qllm_argmax_workspace_bytes(count, batch))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid argmax batch");
+  const uint32_t blocks = (count + kArgmaxChunk - 1u) / kArgmaxChunk;
+  float* partial_values = static_cast<float*>(workspace);
+  uint32_t* partial_indices = reinterpret_cast<uint32_t*>(
+      partial_values + static_cast<size_t>(blocks) * batch);
+  argmax_partial_kernel<<<dim3(blocks, batch), 256, 0, as_stream(stream)>>>(
+      values, count, partial_values, partial_indices, blocks);
+  argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
+      partial_values, partial_indices, blocks, output);
+  return launched("argmax batch");
+}
+
+extern "C" size_t qllm_topk_workspace_bytes(uint32_t count, uint32_t top_k) {
+  const size_t blocks = (static_cast<size_t>(count) + kTopkChunk - 1u) / kTopkChunk;
+  return blocks * top_k * (sizeof(float) + sizeof(uint32_t));
+}
+
+extern "C" int32_t qllm_topk_logits(const float* values, uint32_t count,
+                                    uint32_t top_k, float* output_values,
+                                    uint32_t* output_indices, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  if (!values || !count || !top_k || top_k > 1024u || top_k > count ||
+      !output_values || !output_indices || !workspace ||
+      workspace_bytes < qllm_topk_workspace_bytes(count, top_k))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid top-k logits");
+  const uint32_t blocks = (count + kTopkChunk - 1u) / kTopkChunk;
+  const uint64_t survivors = static_cast<uint64_t>(blocks) * top_k;
+  if (survivors > static_cast<uint64_t>(kMergeThreads) * kMergePerThread)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "top-k logits: count * top_k exceeds the merge capacity");
+  float* partial_values = static_cast<float*>(workspace);
+  uint32_t* partial_indices = reinterpret_cast<uint32_t*>(
+      partial_values + static_cast<size_t>(blocks) * top_k);
+  topk_partial_kernel<<<blocks, kTopkThreads, 0, as_stream(stream)>>>(
+      values, count, top_k, partial_values, partial_indices);
+  topk_merge_kernel<<<1, kMergeThreads, 0, as_stream(stream)>>>(
+      partial_values, partial_indices, static_cast<uint32_t>(survivors), top_k,
+      output_values, output_indices);
+  return launched("top-k logits");
+}
+
+extern "C" int32_t qllm_apply_presence_penalty(float* logits,
+                                               const uint8_t* emitted,
+                                               uint32_t count, float penalty,
+                                               void* stream) {
+  if (!logits || !emitted || !count)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid presence penalty");
+  presence_penalty_kernel<<<(count + 255u) / 256u, 256, 0, as_stream(stream)>>>(
+      logits, emitted, count, penalty);
+  return launched("presence penalty");
+}
