@@ -57,17 +57,44 @@ enum qllm_scale_scheme {
   QLLM_SCALE_F16_BLOCK16 = 1
 };
 
-/* Row-major packed E2M1 codes, low nibble = even column; rows keep their
- * logical column count while storage pads every row to padded_columns
- * (a multiple of 32).  Mirrors Fp4Block32Matrix plus the scheme tag. */
+enum qllm_fp4_layout {
+  /* The artifact layout: row-major codes and scales as stored in QPack
+   * records and handed over by the tensor store. */
+  QLLM_LAYOUT_ROW_MAJOR = 0,
+  /* The provider's device layout produced once, at upload, by
+   * qllm_fp4_prepack: rows grouped in tiles of 32, columns in chunks of 64,
+   * the 64 sixteen-byte pieces of one (tile, chunk) contiguous in the order
+   * the GEMM's lanes consume them, so weights stream in 1 KiB bursts. */
+  QLLM_LAYOUT_TILED = 1
+};
+
+/* Packed E2M1 codes, low nibble = even column; rows keep their logical column
+ * count while storage pads every row to padded_columns (a multiple of 32).
+ * Mirrors Fp4Block32Matrix plus the scheme and layout tags. */
 typedef struct qllm_fp4_matrix {
-  const uint8_t* weights; /* [rows, padded_columns/2] */
+  const uint8_t* weights; /* row-major: [rows, padded_columns/2] */
   const void* scales;     /* u8 [rows, padded/32] or f16 [rows, padded/16] */
   uint32_t rows;
   uint32_t columns;
   uint32_t padded_columns;
   uint32_t scale_scheme;  /* enum qllm_scale_scheme */
+  uint32_t layout;        /* enum qllm_fp4_layout */
+  uint32_t reserved;
 } qllm_fp4_matrix;
+
+/* Device bytes needed for the tiled copy of a matrix. */
+size_t qllm_fp4_packed_weight_bytes(uint32_t rows, uint32_t padded_columns);
+size_t qllm_fp4_packed_scale_bytes(uint32_t rows, uint32_t padded_columns,
+                                   uint32_t scale_scheme);
+
+/* Re-lays a row-major matrix (padded_columns % 64 == 0) into the tiled
+ * layout; `packed` (host struct) receives the descriptor of the copy.  This is
+ * the device half of the provider's tensor upload
+ * (runtime/tools/dense_fp4_provider.cpp:3486-3660); it moves bytes and changes
+ * no value. */
+int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source, void* packed_weights,
+                         void* packed_scales, qllm_fp4_matrix* packed,
+                         void* stream);
 
 enum qllm_output_kind {
   QLLM_OUT_F32 = 0,         /* float [batch, rows] */
@@ -91,7 +118,7 @@ int32_t qllm_convert_f32_to_bf16_batch(const float* input, void* output,
 
 /* FP4 weights x Q8 activations, batch <= 8; out[m*rows+n].
  * replaces fp4_gemv_q8_batch_weight_reuse (transformer_kernels.hpp:92-97).
- * Block-32 UE8M0 matrices only. */
+ * Block-32 UE8M0 row-major matrices only. */
 int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
                                const int8_t* input,
                                const float* input_scales, float* output,

@@ -234,7 +234,8 @@ extern "C" int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
                                             void* stream) {
   if (!matrix || !matrix->weights || !matrix->scales || !matrix->rows ||
       !matrix->columns || matrix->padded_columns < matrix->columns ||
-      matrix->padded_columns % 32u || matrix->scale_scheme > 1u || !tokens ||
+      matrix->padded_columns % 32u || matrix->scale_scheme > 1u ||
+      matrix->layout != QLLM_LAYOUT_ROW_MAJOR || !tokens ||
       !output || !batch)
     return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 embedding batch");
   fp4_embedding_batch_kernel<<<batch, 256, 0, as_stream(stream)>>>(

@@ -17,6 +17,8 @@
 //    output row; used for shapes the MFMA kernel does not take.
 #include "common.hpp"
 
+#include <cstdlib>
+
 namespace qllm {
 namespace {
 
@@ -24,7 +26,6 @@ constexpr int kSchemeUe8m0 = QLLM_SCALE_UE8M0_BLOCK32;
 constexpr int kSchemeF16 = QLLM_SCALE_F16_BLOCK16;
 
 constexpr uint32_t kChunk = 64;            // K elements per wave step
-constexpr uint32_t kLdsActivationBytes = 64 * 1024;
 
 __device__ __forceinline__ bf16x8 expand_fp4x8(uint32_t packed, float scale) {
   const bf16x2 p0 = fp4x2_to_bf16<0>(packed, scale);
@@ -66,7 +67,6 @@ struct GemmArgs {
   const float* residual;
   uint32_t rows;
   uint32_t padded_columns;
-  uint32_t phase_columns;       // K handled per LDS staging phase
   uint32_t output_kind;
   uint32_t swiglu;              // tile 1 is the up projection of tile 0
 };
@@ -91,14 +91,31 @@ __device__ __forceinline__ void store_output(void* output, uint32_t kind,
 // i.e. 16-blocks {2g, 2g+1} of the chunk.  One v_permlane32_swap per dword
 // pair regroups that into "half g of block b" - the B-operand layout of the
 // 32x32x16 MFMA - without touching LDS.
-template <int SCHEME, int BATCH, int TILES, int WAVES>
+//
+// Activations travel with the weights: together with the weight pieces of a
+// chunk a wave prefetches the batch x 64 activation values of that chunk
+// (8*batch sixteen-byte pieces, one per lane), drops them into a small
+// wave-private LDS ring in MFMA A-fragment order and reads the four 16-block
+// fragments back.  Nothing is staged per workgroup, so there is no barrier in
+// the K loop and any K that is a multiple of 64 is handled alike.
+//
+// TILED selects the provider's streaming layout (see qllm_fp4_prepack): the
+// 64 sixteen-byte pieces a wave loads for one (tile, chunk) are contiguous,
+// so every wave-level load is one 1 KiB burst.  With the row-major layout the
+// same pieces sit a row stride apart (64 separate 16-byte requests).
+template <int SCHEME, int BATCH, int TILES, int WAVES, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     const GemmArgs args) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
-  uint4* fragments = reinterpret_cast<uint4*>(lds_raw);
+  constexpr int PF = 4;             // chunks in flight per lane
+  constexpr int PIECES = 8 * BATCH; // activation pieces per chunk
+  // ring slot: PIECES pieces of 16 bytes, padded to 64 pieces
+  __shared__ __attribute__((aligned(16))) uint4 ring[WAVES][2][64];
+  __shared__ float reduce[WAVES][TILES][4][64];
 
   const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t wave = threadIdx.x >> 6;
+  // wave index as a scalar, so everything derived from it (chunk counts,
+  // loop bounds) is uniform control flow
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t n = lane & 31u;
   const uint32_t g = lane >> 5;
   const uint32_t K = args.padded_columns;
@@ -107,88 +124,83 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       SCHEME == kSchemeF16 ? K / 8u : K / 32u;
   const uint32_t m_lane = n < BATCH ? n : BATCH - 1u;
 
+  // per-chunk byte strides of the two streams
+  constexpr uint32_t kScaleChunk = SCHEME == kSchemeF16 ? 8u : 2u;
+  const uint32_t weight_step = TILED ? 1024u : 32u;
+  const uint32_t scale_step = TILED ? 32u * kScaleChunk : kScaleChunk;
   const uint8_t* weight_row[TILES];
   const uint8_t* scale_row[TILES];
-  uint32_t out_row[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
-    uint32_t row;
-    if (args.swiglu)
-      row = blockIdx.x * 32u + n;
-    else
-      row = (blockIdx.x * TILES + t) * 32u + n;
-    out_row[t] = row;
-    const uint32_t safe = row < args.rows ? row : args.rows - 1u;
-    weight_row[t] = args.tile[t].weights + static_cast<size_t>(safe) * row_bytes +
-                    g * 16u;
-    scale_row[t] = args.tile[t].scales + static_cast<size_t>(safe) * scale_row_bytes;
+    const uint32_t tile = args.swiglu ? blockIdx.x : blockIdx.x * TILES + t;
+    if (TILED) {
+      const uint32_t tiles = (args.rows + 31u) / 32u;
+      const size_t first_chunk =
+          static_cast<size_t>(tile < tiles ? tile : tiles - 1u) * (K / kChunk);
+      weight_row[t] = args.tile[t].weights + first_chunk * 1024u + lane * 16u;
+      scale_row[t] = args.tile[t].scales +
+                     (first_chunk * 32u + n) * kScaleChunk;
+    } else {
+      const uint32_t row = tile * 32u + n;
+      const uint32_t safe = row < args.rows ? row : args.rows - 1u;
+      weight_row[t] = args.tile[t].weights +
+                      static_cast<size_t>(safe) * row_bytes + g * 16u;
+      scale_row[t] =
+          args.tile[t].scales + static_cast<size_t>(safe) * scale_row_bytes;
+    }
   }
+  // activation piece this lane fetches per chunk: piece p = (block*2+half)*
+  // BATCH + m  ->  act[m][chunk*64 + (block*2+half)*8 .. +8]
+  const uint32_t piece = lane < PIECES ? lane : PIECES - 1u;
+  const uint16_t* activation_piece =
+      args.activations + static_cast<size_t>(piece % BATCH) * K +
+      (piece / BATCH) * 8u;
 
-  // F16 scheme: per-block results are scaled in F32 after the MFMA.
-  // UE8M0 scheme: the power-of-two scale is folded into the nibble->bf16
-  // conversion (exact), so the MFMA accumulates across the whole K range.
   float acc[TILES][4];
-  f32x16 macc[TILES];
 #pragma unroll
-  for (int t = 0; t < TILES; ++t) {
+  for (int t = 0; t < TILES; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[t][i] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) macc[t][i] = 0.0f;
-  }
 
-  constexpr int PF = 4;  // chunks in flight per lane
-  for (uint32_t phase_begin = 0; phase_begin < K;
-       phase_begin += args.phase_columns) {
-    const uint32_t phase_columns =
-        min(args.phase_columns, K - phase_begin);
-    const uint32_t phase_chunks = phase_columns / kChunk;
-    const uint32_t my_chunks =
-        phase_chunks > wave ? (phase_chunks - wave + WAVES - 1u) / WAVES : 0u;
+  const uint32_t chunks = K / kChunk;
+  const uint32_t my_chunks =
+      chunks > wave ? (chunks - wave + WAVES - 1u) / WAVES : 0u;
+  // Prefetch is unconditional: indices past the wave's last chunk are clamped
+  // to it (loaded again and ignored), which keeps the load/wait pattern of the
+  // unrolled ring static.
+  const uint32_t last_index = my_chunks ? my_chunks - 1u : 0u;
 
-    uint4 codes[PF][TILES];
-    uint2 scales[PF][TILES];
-    auto issue = [&](int slot, uint32_t index) {
-      const uint32_t chunk = phase_begin / kChunk + wave + index * WAVES;
+  uint4 codes[PF][TILES];
+  uint2 scales[PF][TILES];
+  uint4 activation[PF];
+  auto issue = [&](int slot, uint32_t index) {
+    const uint32_t chunk = wave + index * WAVES;
 #pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-        codes[slot][t] = load_stream16(weight_row[t] + chunk * 32u);
-        if (SCHEME == kSchemeF16) {
-          scales[slot][t] = load_stream8(scale_row[t] + chunk * 8u);
-        } else {
-          const uint32_t pair = *reinterpret_cast<const uint16_t*>(
-              scale_row[t] + chunk * 2u);
-          scales[slot][t] = make_uint2(pair & 0xffu, pair >> 8);
-        }
-      }
-    };
-#pragma unroll
-    for (int slot = 0; slot < PF; ++slot)
-      if (static_cast<uint32_t>(slot) < my_chunks) issue(slot, slot);
-
-    // Stage this phase's activations into LDS in fragment order:
-    // fragments[(block*2 + half)*BATCH + m] = act[m][block*16 + half*8 .. +8].
-    __syncthreads();  // previous phase's readers are done
-    {
-      const uint32_t pieces_per_row = phase_columns / 8u;
-      const uint32_t pieces = pieces_per_row * BATCH;
-      for (uint32_t piece = threadIdx.x; piece < pieces;
-           piece += WAVES * 64u) {
-        const uint32_t m = piece / pieces_per_row;
-        const uint32_t position = piece - m * pieces_per_row;
-        const uint4 value = *reinterpret_cast<const uint4*>(
-            args.activations + static_cast<size_t>(m) * K + phase_begin +
-            position * 8u);
-        fragments[position * BATCH + m] = value;
+    for (int t = 0; t < TILES; ++t) {
+      codes[slot][t] =
+          load_stream16(weight_row[t] + static_cast<size_t>(chunk) * weight_step);
+      if (SCHEME == kSchemeF16) {
+        scales[slot][t] =
+            load_stream8(scale_row[t] + static_cast<size_t>(chunk) * scale_step);
+      } else {
+        const uint32_t pair = *reinterpret_cast<const uint16_t*>(
+            scale_row[t] + static_cast<size_t>(chunk) * scale_step);
+        scales[slot][t] = make_uint2(pair & 0xffu, pair >> 8);
       }
     }
-    __syncthreads();
+    activation[slot] =
+        *reinterpret_cast<const uint4*>(activation_piece + chunk * kChunk);
+  };
+
+  if (my_chunks) {
+#pragma unroll
+    for (int slot = 0; slot < PF; ++slot)
+      issue(slot, min(static_cast<uint32_t>(slot), last_index));
 
     for (uint32_t base = 0; base < my_chunks; base += PF) {
 #pragma unroll
       for (int slot = 0; slot < PF; ++slot) {
         const uint32_t index = base + slot;
-        if (index >= my_chunks) break;
         uint4 q[TILES];
         uint2 s[TILES];
 #pragma unroll
@@ -196,17 +208,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
           q[t] = codes[slot][t];
           s[t] = scales[slot][t];
         }
-        if (index + PF < my_chunks) issue(slot, index + PF);
+        const uint4 x = activation[slot];
+        issue(slot, min(index + PF, last_index));
+        if (index >= my_chunks) continue;
 
-        const uint32_t local_chunk = wave + index * WAVES;
-        // activation fragments of the four 16-blocks of this chunk
+        // activation pieces -> wave-private ring -> A fragments
+        uint4* stage = ring[wave][slot & 1];
+        stage[lane] = x;
+        __builtin_amdgcn_wave_barrier();
         bf16x8 a[4];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const uint4 raw =
-              fragments[((local_chunk * 4u + b) * 2u + g) * BATCH + m_lane];
-          a[b] = __builtin_bit_cast(bf16x8, raw);
-        }
+        for (int b = 0; b < 4; ++b)
+          a[b] = __builtin_bit_cast(bf16x8,
+                                    stage[(b * 2u + g) * BATCH + m_lane]);
+        __builtin_amdgcn_wave_barrier();
+
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
           const auto s01 = __builtin_amdgcn_permlane32_swap(q[t].x, q[t].y,
@@ -216,53 +232,45 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
           // block order inside the chunk: s01[0]=b0, s23[0]=b1, s01[1]=b2,
           // s23[1]=b3
           const uint32_t packed[4] = {s01[0], s23[0], s01[1], s23[1]};
+          float scale[4];
+          float fold[4];
           if (SCHEME == kSchemeF16) {
-            const float scale[4] = {
-                f16_bits_to_f32(s[t].x & 0xffffu), f16_bits_to_f32(s[t].x >> 16),
-                f16_bits_to_f32(s[t].y & 0xffffu), f16_bits_to_f32(s[t].y >> 16)};
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-              const bf16x8 w = expand_fp4x8(packed[b], 1.0f);
-              f32x16 zero;
-#pragma unroll
-              for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
-              const f32x16 d = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                  a[b], w, zero, 0, 0, 0);
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                acc[t][i] = fmaf(d[i], scale[b], acc[t][i]);
-            }
+            // binary16 scale applied in F32 after the block's MFMA
+            scale[0] = f16_bits_to_f32(s[t].x & 0xffffu);
+            scale[1] = f16_bits_to_f32(s[t].x >> 16);
+            scale[2] = f16_bits_to_f32(s[t].y & 0xffffu);
+            scale[3] = f16_bits_to_f32(s[t].y >> 16);
+            fold[0] = fold[1] = fold[2] = fold[3] = 1.0f;
           } else {
-            const float scale_low = ue8m0_to_f32(s[t].x);
-            const float scale_high = ue8m0_to_f32(s[t].y);
-#pragma unroll
-            for (int b = 0; b < 4; ++b) {
-              const bf16x8 w =
-                  expand_fp4x8(packed[b], b < 2 ? scale_low : scale_high);
-              macc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                  a[b], w, macc[t], 0, 0, 0);
-            }
+            // power-of-two scale folded into the nibble->bf16 conversion
+            fold[0] = fold[1] = ue8m0_to_f32(s[t].x);
+            fold[2] = fold[3] = ue8m0_to_f32(s[t].y);
+            scale[0] = scale[1] = scale[2] = scale[3] = 1.0f;
           }
+          f32x16 d[4];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            const bf16x8 w = expand_fp4x8(packed[b], fold[b]);
+            f32x16 zero;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
+            d[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[b], w, zero, 0, 0, 0);
+          }
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[t][i] = fmaf(d[b][i], scale[b], acc[t][i]);
         }
       }
     }
   }
 
-  if (SCHEME != kSchemeF16) {
-#pragma unroll
-    for (int t = 0; t < TILES; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[t][i] = macc[t][i];
-  }
-
-  // Cross-wave reduction through LDS (reuses the activation staging area).
-  __syncthreads();
-  float* reduce = reinterpret_cast<float*>(lds_raw);
+  // Cross-wave reduction through LDS.
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      reduce[((wave * TILES + t) * 4 + i) * 64 + lane] = acc[t][i];
+    for (int i = 0; i < 4; ++i) reduce[wave][t][i][lane] = acc[t][i];
   __syncthreads();
 
   const uint32_t items = (args.swiglu ? 1u : TILES) * 256u;
@@ -277,14 +285,13 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     if (m >= BATCH || row >= args.rows) continue;
     float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
-      total += reduce[((w * TILES + t) * 4 + i) * 64 + source_lane];
+    for (int w = 0; w < WAVES; ++w) total += reduce[w][t][i][source_lane];
     const size_t index = static_cast<size_t>(m) * args.rows + row;
     if (args.swiglu) {
       float up = 0.0f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w)
-        up += reduce[((w * TILES + (TILES - 1)) * 4 + i) * 64 + source_lane];
+        up += reduce[w][TILES - 1][i][source_lane];
       const float activated = bf16_round(total / (1.0f + __expf(-total)));
       static_cast<uint16_t*>(args.output)[index] =
           static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
@@ -293,7 +300,6 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       store_output(args.output, args.output_kind, index, total);
     }
   }
-  (void)out_row;
 }
 
 // ---- generic fallback: one wave per output row -------------------------------
@@ -383,85 +389,118 @@ bool matrix_ok(const qllm_fp4_matrix* m) {
   return m && m->weights && m->scales && m->rows && m->columns &&
          m->padded_columns >= m->columns && m->padded_columns % 32u == 0u &&
          (m->scale_scheme == QLLM_SCALE_UE8M0_BLOCK32 ||
-          m->scale_scheme == QLLM_SCALE_F16_BLOCK16);
+          m->scale_scheme == QLLM_SCALE_F16_BLOCK16) &&
+         (m->layout == QLLM_LAYOUT_ROW_MAJOR ||
+          (m->layout == QLLM_LAYOUT_TILED && m->padded_columns % kChunk == 0u));
 }
 
-uint32_t phase_columns_for(uint32_t K, uint32_t batch, uint32_t waves) {
-  const uint32_t granule = kChunk * waves;
-  const uint32_t limit = kLdsActivationBytes / (2u * batch) / granule * granule;
-  if (K <= limit) return K;
-  const uint32_t phases = (K + limit - 1u) / limit;
-  return ((K + phases - 1u) / phases + granule - 1u) / granule * granule;
-}
-
-template <int SCHEME, int BATCH, int TILES>
+template <int SCHEME, int BATCH, int TILES, bool TILED>
 int32_t launch_mfma_waves(const GemmArgs& args, uint32_t grid, uint32_t waves,
                           size_t lds_bytes, hipStream_t stream) {
   switch (waves) {
     case 4:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4>
+      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4, TILED>
           <<<grid, 256, lds_bytes, stream>>>(args);
       break;
     case 8:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8>
+      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8, TILED>
           <<<grid, 512, lds_bytes, stream>>>(args);
       break;
     default:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 16>
+      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 16, TILED>
           <<<grid, 1024, lds_bytes, stream>>>(args);
       break;
   }
   return launched("FP4 MFMA GEMM");
 }
 
-template <int SCHEME, int TILES>
+template <int SCHEME, int TILES, bool TILED>
 int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
                           uint32_t waves, size_t lds_bytes,
                           hipStream_t stream) {
   switch (batch) {
-    case 1: return launch_mfma_waves<SCHEME, 1, TILES>(args, grid, waves, lds_bytes, stream);
-    case 2: return launch_mfma_waves<SCHEME, 2, TILES>(args, grid, waves, lds_bytes, stream);
-    case 3: return launch_mfma_waves<SCHEME, 3, TILES>(args, grid, waves, lds_bytes, stream);
-    case 4: return launch_mfma_waves<SCHEME, 4, TILES>(args, grid, waves, lds_bytes, stream);
-    case 5: return launch_mfma_waves<SCHEME, 5, TILES>(args, grid, waves, lds_bytes, stream);
-    case 6: return launch_mfma_waves<SCHEME, 6, TILES>(args, grid, waves, lds_bytes, stream);
-    case 7: return launch_mfma_waves<SCHEME, 7, TILES>(args, grid, waves, lds_bytes, stream);
-    default: return launch_mfma_waves<SCHEME, 8, TILES>(args, grid, waves, lds_bytes, stream);
+    case 1: return launch_mfma_waves<SCHEME, 1, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 2: return launch_mfma_waves<SCHEME, 2, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 3: return launch_mfma_waves<SCHEME, 3, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 4: return launch_mfma_waves<SCHEME, 4, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 5: return launch_mfma_waves<SCHEME, 5, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 6: return launch_mfma_waves<SCHEME, 6, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 7: return launch_mfma_waves<SCHEME, 7, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    default: return launch_mfma_waves<SCHEME, 8, TILES, TILED>(args, grid, waves, lds_bytes, stream);
   }
 }
 
-// Chooses tiles per workgroup and waves per workgroup so that the launch
-// keeps roughly 3-5 thousand waves in flight on 256 CUs (4 SIMDs each).
-int32_t launch_mfma(GemmArgs args, int scheme, uint32_t batch, bool swiglu,
-                    hipStream_t stream) {
+// One tile of 32 rows per workgroup (two for the fused gate/up pair); four
+// waves split K, eight when the matrix has too few tiles to fill 256 CUs.
+// Measured on MI355X: 16-wave groups lose to register pressure, two plain
+// tiles per group never beat one.
+int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
+                    bool swiglu, hipStream_t stream) {
   const uint32_t tiles = (args.rows + 31u) / 32u;
-  uint32_t tiles_per_group = 1u;
-  uint32_t waves = 4u;
-  if (swiglu) {
-    tiles_per_group = 2u;
-    waves = tiles >= 768u ? 4u : (tiles >= 384u ? 8u : 16u);
-  } else if (tiles >= 1024u) {
-    tiles_per_group = 2u;
-  } else if (tiles < 384u) {
-    waves = tiles >= 192u ? 8u : 16u;
-  }
+  uint32_t tiles_per_group = swiglu ? 2u : 1u;
+  uint32_t waves = tiles < 384u ? 8u : 4u;
+  if (const char* forced = getenv("QLLM_GEMM_WAVES")) waves = atoi(forced);
+  if (const char* forced = getenv("QLLM_GEMM_TILES"))
+    if (!swiglu) tiles_per_group = atoi(forced);
   const uint32_t grid =
       swiglu ? tiles : (tiles + tiles_per_group - 1u) / tiles_per_group;
-  args.phase_columns = phase_columns_for(args.padded_columns, batch, waves);
   args.swiglu = swiglu ? 1u : 0u;
-  const size_t stage_bytes =
-      static_cast<size_t>(args.phase_columns) * 2u * batch;
-  const size_t reduce_bytes =
-      static_cast<size_t>(waves) * tiles_per_group * 4u * 64u * sizeof(float);
-  const size_t lds_bytes = stage_bytes > reduce_bytes ? stage_bytes : reduce_bytes;
+  const size_t lds_bytes = 0;
+#define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                 \
+  return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, grid, waves, \
+                                                    lds_bytes, stream)
   if (scheme == kSchemeF16) {
-    if (tiles_per_group == 2u)
-      return launch_mfma_batch<kSchemeF16, 2>(args, batch, grid, waves, lds_bytes, stream);
-    return launch_mfma_batch<kSchemeF16, 1>(args, batch, grid, waves, lds_bytes, stream);
+    if (tiled) {
+      if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeF16, 2, true);
+      QLLM_LAUNCH(kSchemeF16, 1, true);
+    }
+    if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeF16, 2, false);
+    QLLM_LAUNCH(kSchemeF16, 1, false);
   }
-  if (tiles_per_group == 2u)
-    return launch_mfma_batch<kSchemeUe8m0, 2>(args, batch, grid, waves, lds_bytes, stream);
-  return launch_mfma_batch<kSchemeUe8m0, 1>(args, batch, grid, waves, lds_bytes, stream);
+  if (tiled) {
+    if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeUe8m0, 2, true);
+    QLLM_LAUNCH(kSchemeUe8m0, 1, true);
+  }
+  if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeUe8m0, 2, false);
+  QLLM_LAUNCH(kSchemeUe8m0, 1, false);
+#undef QLLM_LAUNCH
+}
+
+// Row-major -> streaming layout.  Output piece p = (tile*chunks + chunk)*64 +
+// lane holds, for lane = half*32 + n, the 16 bytes of row 32*tile + n at byte
+// offset chunk*32 + half*16; rows past the matrix are zero.  Scales follow
+// per (tile, chunk) as 32 consecutive row entries of 4 binary16 / 2 UE8M0.
+__global__ void fp4_prepack_kernel(const uint8_t* weights,
+                                   const uint8_t* scales, uint8_t* out_weights,
+                                   uint8_t* out_scales, uint32_t rows,
+                                   uint32_t padded_columns,
+                                   uint32_t scale_chunk_bytes) {
+  const uint32_t chunks = padded_columns / kChunk;
+  const uint32_t tiles = (rows + 31u) / 32u;
+  const size_t pieces = static_cast<size_t>(tiles) * chunks * 64u;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t piece = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+       piece < pieces; piece += stride) {
+    const uint32_t lane = static_cast<uint32_t>(piece & 63u);
+    const size_t block = piece >> 6;
+    const uint32_t chunk = static_cast<uint32_t>(block % chunks);
+    const uint32_t tile = static_cast<uint32_t>(block / chunks);
+    const uint32_t row = tile * 32u + (lane & 31u);
+    uint4 value = make_uint4(0u, 0u, 0u, 0u);
+    if (row < rows)
+      value = *reinterpret_cast<const uint4*>(
+          weights + static_cast<size_t>(row) * (padded_columns / 2u) +
+          chunk * 32u + (lane >> 5) * 16u);
+    *reinterpret_cast<uint4*>(out_weights + piece * 16u) = value;
+    if (lane < 32u) {
+      uint8_t* target = out_scales + (block * 32u + lane) * scale_chunk_bytes;
+      const uint8_t* source =
+          scales + static_cast<size_t>(row) * (chunks * scale_chunk_bytes) +
+          chunk * scale_chunk_bytes;
+      for (uint32_t byte = 0; byte < scale_chunk_bytes; ++byte)
+        target[byte] = row < rows ? source[byte] : 0u;
+    }
+  }
 }
 
 }  // namespace
@@ -494,10 +533,13 @@ extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
     args.rows = matrix->rows;
     args.padded_columns = matrix->padded_columns;
     args.output_kind = output_kind;
-    return launch_mfma(args, static_cast<int>(matrix->scale_scheme), batch,
-                       false, as_stream(stream));
+    return launch_mfma(args, static_cast<int>(matrix->scale_scheme),
+                       matrix->layout == QLLM_LAYOUT_TILED, batch, false,
+                       as_stream(stream));
   }
   const uint32_t grid = (matrix->rows + 3u) / 4u;
+  if (matrix->layout != QLLM_LAYOUT_ROW_MAJOR)
+    return fail(QLLM_INVALID_ARGUMENT, "tiled FP4 matrix needs K % 64 == 0");
   if (matrix->scale_scheme == QLLM_SCALE_F16_BLOCK16)
     fp4_gemv_generic_kernel<kSchemeF16, false>
         <<<grid, 256, 0, as_stream(stream)>>>(
@@ -520,7 +562,8 @@ extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
                                         void* stream) {
   if (!matrix_ok(gate) || !matrix_ok(up) || gate->rows != up->rows ||
       gate->padded_columns != up->padded_columns ||
-      gate->scale_scheme != up->scale_scheme || !input || !output || !batch ||
+      gate->scale_scheme != up->scale_scheme || gate->layout != up->layout ||
+      !input || !output || !batch ||
       batch > 8u || gate->padded_columns % kChunk != 0u ||
       input_bytes < static_cast<size_t>(batch) * gate->padded_columns * 2u)
     return fail(QLLM_INVALID_ARGUMENT, "invalid fused FP4 SwiGLU GEMM");
@@ -532,7 +575,8 @@ extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
   args.rows = gate->rows;
   args.padded_columns = gate->padded_columns;
   args.output_kind = QLLM_OUT_BF16;
-  return launch_mfma(args, static_cast<int>(gate->scale_scheme), batch, true,
+  return launch_mfma(args, static_cast<int>(gate->scale_scheme),
+                     gate->layout == QLLM_LAYOUT_TILED, batch, true,
                      as_stream(stream));
 }
 
@@ -542,7 +586,8 @@ extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
                                           float* output, uint32_t batch,
                                           int32_t bf16_output, void* stream) {
   if (!matrix_ok(matrix) || matrix->scale_scheme != QLLM_SCALE_UE8M0_BLOCK32 ||
-      !input || !input_scales || !output || !batch || batch > 8u)
+      matrix->layout != QLLM_LAYOUT_ROW_MAJOR || !input || !input_scales ||
+      !output || !batch || batch > 8u)
     return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 Q8 weight-reuse GEMV");
   const uint32_t grid = (matrix->rows + 3u) / 4u;
   fp4_gemv_generic_kernel<kSchemeUe8m0, true>
@@ -551,4 +596,43 @@ extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
           input_scales, output, nullptr, matrix->rows, matrix->padded_columns,
           batch, bf16_output ? QLLM_OUT_F32_BF16_ROUNDED : QLLM_OUT_F32);
   return launched("FP4 Q8 weight-reuse GEMV");
+}
+
+extern "C" size_t qllm_fp4_packed_weight_bytes(uint32_t rows,
+                                               uint32_t padded_columns) {
+  return static_cast<size_t>((rows + 31u) / 32u) * 32u * (padded_columns / 2u);
+}
+
+extern "C" size_t qllm_fp4_packed_scale_bytes(uint32_t rows,
+                                              uint32_t padded_columns,
+                                              uint32_t scale_scheme) {
+  const size_t per_row = scale_scheme == QLLM_SCALE_F16_BLOCK16
+                             ? padded_columns / 8u
+                             : padded_columns / 32u;
+  return static_cast<size_t>((rows + 31u) / 32u) * 32u * per_row;
+}
+
+extern "C" int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source,
+                                    void* packed_weights, void* packed_scales,
+                                    qllm_fp4_matrix* packed, void* stream) {
+  if (!matrix_ok(source) || source->layout != QLLM_LAYOUT_ROW_MAJOR ||
+      source->padded_columns % kChunk != 0u || !packed_weights ||
+      !packed_scales || !packed)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 prepack");
+  const uint32_t scale_chunk_bytes =
+      source->scale_scheme == QLLM_SCALE_F16_BLOCK16 ? 8u : 2u;
+  const size_t pieces = qllm_fp4_packed_weight_bytes(source->rows,
+                                                     source->padded_columns) / 16u;
+  const size_t blocks = (pieces + 255u) / 256u;
+  fp4_prepack_kernel<<<static_cast<unsigned>(blocks < 65536u ? blocks : 65536u),
+                       256, 0, as_stream(stream)>>>(
+      source->weights, static_cast<const uint8_t*>(source->scales),
+      static_cast<uint8_t*>(packed_weights),
+      static_cast<uint8_t*>(packed_scales), source->rows,
+      source->padded_columns, scale_chunk_bytes);
+  *packed = *source;
+  packed->weights = static_cast<const uint8_t*>(packed_weights);
+  packed->scales = packed_scales;
+  packed->layout = QLLM_LAYOUT_TILED;
+  return launched("FP4 prepack");
 }

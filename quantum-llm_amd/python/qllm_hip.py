@@ -13,7 +13,9 @@ from ctypes import (POINTER, Structure, c_char_p, c_float, c_int32, c_size_t,
                     c_uint32, c_uint64, c_void_p)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIBRARY_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libqllm_hip.so")
+LIBRARY_PATH = os.environ.get(
+    "QLLM_HIP_LIBRARY",
+    os.path.join(os.path.dirname(_HERE), "lib", "libqllm_hip.so"))
 
 SCALE_UE8M0_BLOCK32 = 0
 SCALE_F16_BLOCK16 = 1
@@ -31,7 +33,8 @@ class QllmError(RuntimeError):
 class Fp4Matrix(Structure):
     _fields_ = [("weights", c_void_p), ("scales", c_void_p),
                 ("rows", c_uint32), ("columns", c_uint32),
-                ("padded_columns", c_uint32), ("scale_scheme", c_uint32)]
+                ("padded_columns", c_uint32), ("scale_scheme", c_uint32),
+                ("layout", c_uint32), ("reserved", c_uint32)]
 
 
 class Q4hAttentionLaunch(Structure):
@@ -70,6 +73,9 @@ SIGNATURES = {
     "qllm_fp4_gemv_q8_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_fp4_gemm_bf16": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
     "qllm_fp4_swiglu_bf16": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32]),
+    "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
+    "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
     "qllm_fp4_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_uint32, c_void_p]),
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
@@ -127,4 +133,19 @@ def ptr(tensor) -> int:
 
 def fp4_matrix(weights, scales, rows, columns, padded_columns, scheme) -> Fp4Matrix:
     return Fp4Matrix(ptr(weights), ptr(scales), rows, columns, padded_columns,
-                     scheme)
+                     scheme, 0, 0)
+
+
+def prepack(matrix: Fp4Matrix, device):
+    """Tiled device copy of a row-major matrix: (descriptor, keepalive)."""
+    import torch
+    weight_bytes = call("qllm_fp4_packed_weight_bytes", matrix.rows,
+                        matrix.padded_columns)
+    scale_bytes = call("qllm_fp4_packed_scale_bytes", matrix.rows,
+                       matrix.padded_columns, matrix.scale_scheme)
+    weights = torch.empty(weight_bytes, dtype=torch.uint8, device=device)
+    scales = torch.empty(scale_bytes, dtype=torch.uint8, device=device)
+    packed = Fp4Matrix()
+    call("qllm_fp4_prepack", ctypes.byref(matrix), ptr(weights), ptr(scales),
+         ctypes.byref(packed), None)
+    return packed, (weights, scales)
