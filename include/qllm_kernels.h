@@ -195,6 +195,18 @@ int32_t qllm_qkv_rope_cache_paged_q4h_batch(
     uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
     float rope_theta, int32_t bf16_activations, void* stream);
 
+/* The same per-head RMSNorm + rotary without the K/V store, for caches that
+ * store K/V separately.  replaces gated_gqa_qkv_rope_fp16_batch
+ * (runtime/src/cuda/transformer_kernels.cu:3645-3726). */
+int32_t qllm_qkv_rope_batch(float* query, uint32_t query_stride, float* key,
+                            const float* q_norm_weight,
+                            const float* k_norm_weight,
+                            uint32_t first_rotary_position, uint32_t rows,
+                            uint32_t query_heads, uint32_t kv_heads,
+                            uint32_t head_dim, uint32_t rotary_dim,
+                            float epsilon, float rope_theta,
+                            int32_t bf16_activations, void* stream);
+
 /* replaces store_gqa_kv_paged_q4_per_head_batch (the store-only form used
  * by runtime/tools/dense_fp4_cuda_smoke.cpp:1828-1832). */
 int32_t qllm_store_kv_paged_q4h_batch(const float* key, const float* value,

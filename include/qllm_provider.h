@@ -1,0 +1,147 @@
+/*
+ * C ABI over the MI355X dense-FP4 provider (quantum-llm_amd/provider), for
+ * hosts that cannot link the C++ IOperationProvider object directly: test
+ * drivers, benchmarks, foreign-language workers.  Each call forwards to the
+ * provider method named beside it; the provider itself mirrors the reference's
+ * runtime/tools/dense_fp4_provider.cpp.
+ *
+ * Status codes are those of qllm_kernels.h; qllm_provider_last_error() holds
+ * the text of the last failure on the calling thread.  Host pointers are
+ * plain process memory; nothing here takes or returns device pointers except
+ * qllm_provider_logits / qllm_provider_hidden.
+ */
+#ifndef QLLM_PROVIDER_H
+#define QLLM_PROVIDER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct qllm_provider qllm_provider;
+
+/* Geometry an artifact declares for a dense decoder
+ * (validate_dense_fp4_descriptor, dense_fp4_provider.cpp:804-994). */
+typedef struct qllm_dense_geometry {
+  uint32_t hidden;
+  uint32_t intermediate;
+  uint32_t layers;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t head_dim;
+  uint32_t rotary_dim;
+  uint32_t vocabulary;
+  float rope_theta;
+  float norm_epsilon;
+  int32_t output_gated;
+  int32_t qk_norm;
+  int32_t zero_centered_norm;
+  uint32_t scale_scheme;   /* enum qllm_scale_scheme */
+  uint32_t kv_encoding;    /* 0 = "q4-f16-per-head", 1 = "fp16" */
+  uint32_t kv_page_tokens;
+  uint32_t max_context;
+  uint32_t draft_depth;
+} qllm_dense_geometry;
+
+const char* qllm_provider_last_error(void);
+
+/* make_<name>_callable_provider (dense_fp4_provider.cpp:11402-11412). */
+qllm_provider* qllm_provider_create(const qllm_dense_geometry* geometry);
+void qllm_provider_destroy(qllm_provider* provider);
+
+/* Capability table of make_<name>_provider(): writes up to `capacity`
+ * NUL-separated "capability\0" strings, returns the count. */
+uint32_t qllm_provider_capabilities(char* buffer, size_t capacity);
+
+/* Stages one host tensor for the next qllm_provider_prepare call.
+ * encoding "FP4_E2M1": data = packed codes, scales = scale bytes,
+ * quant_abi 3 (UE8M0 / 32) or 16 (binary16 / 16); encoding "F32": data only.
+ * The bytes are copied. */
+int32_t qllm_provider_stage_tensor(qllm_provider* provider, const char* role,
+                                   const char* encoding, uint32_t quant_abi,
+                                   uint32_t rows, uint32_t columns,
+                                   const void* data, size_t data_bytes,
+                                   const void* scales, size_t scale_bytes);
+
+/* IOperationProvider::prepare for one artifact operation with the staged
+ * tensors (then clears the staging area). */
+int32_t qllm_provider_prepare(qllm_provider* provider, const char* capability);
+
+/* IOperationProvider::prepare_exact_decode (ABI 2). */
+int32_t qllm_provider_prepare_exact_decode(qllm_provider* provider,
+                                           const char* capability);
+
+/* Random-init model / KV cache generated on the device. */
+int32_t qllm_provider_load_synthetic_weights(qllm_provider* provider,
+                                             uint64_t seed);
+int32_t qllm_provider_prefill_synthetic_kv(qllm_provider* provider,
+                                           uint32_t tokens, uint64_t seed);
+
+/* create_request_state + request parameters
+ * (moe_vm_runner.cpp:318-347): sampling_temperature_ppm, sampling_top_p_ppm,
+ * sampling_top_k, sampling_min_p_ppm, sampling_seed. */
+int32_t qllm_provider_begin_request(qllm_provider* provider,
+                                    uint32_t temperature_ppm,
+                                    uint32_t top_p_ppm, uint32_t top_k,
+                                    uint32_t min_p_ppm, uint64_t seed);
+
+/* synchronize_exact_decode_batch with one token: the stream stands at
+ * `position` with `token` guaranteed. */
+int32_t qllm_provider_synchronize(qllm_provider* provider, uint32_t token,
+                                  uint32_t position);
+
+/* Drafts for the next verify step.  distribution_counts[i] entries of
+ * (tokens, probabilities) describe draft i's proposal distribution q; a count
+ * of 0 means the one-hot distribution on the draft token (greedy). */
+int32_t qllm_provider_set_drafts(qllm_provider* provider,
+                                 const uint32_t* draft_tokens,
+                                 uint32_t draft_count,
+                                 const uint32_t* distribution_counts,
+                                 const uint32_t* distribution_tokens,
+                                 const double* distribution_probabilities);
+
+/* execute_exact_decode: emitted[0] is the guaranteed token, then the
+ * accepted drafts; returns counts through the out parameters. */
+int32_t qllm_provider_verify(qllm_provider* provider, uint32_t guaranteed_token,
+                             uint32_t position, uint32_t context_limit,
+                             uint32_t* emitted, uint32_t* emitted_count,
+                             uint32_t* next_token,
+                             uint32_t* positions_advanced);
+
+/* run_target alone (no sampling), and its graph-captured replay. */
+int32_t qllm_provider_run_target(qllm_provider* provider,
+                                 const uint32_t* tokens, uint32_t rows,
+                                 uint32_t first_position);
+int32_t qllm_provider_capture_target(qllm_provider* provider,
+                                     const uint32_t* tokens, uint32_t rows,
+                                     uint32_t first_position);
+int32_t qllm_provider_replay_target(qllm_provider* provider);
+int32_t qllm_provider_synchronize_stream(qllm_provider* provider);
+
+/* Synchronise the provider's stream and copy logits [rows, vocabulary] /
+ * hidden state [rows, hidden] of the last target pass to host memory. */
+int32_t qllm_provider_copy_logits(qllm_provider* provider, uint32_t rows,
+                                  float* host_output);
+int32_t qllm_provider_copy_hidden(qllm_provider* provider, uint32_t rows,
+                                  float* host_output);
+
+/* Bytes of one KV page (all layers) and a host copy of page `page_index`
+ * (zero-filled if the page has not been allocated yet). */
+uint64_t qllm_provider_kv_page_bytes(const qllm_provider* provider);
+int32_t qllm_provider_copy_kv_page(qllm_provider* provider, uint32_t page_index,
+                                   void* host_output);
+
+const float* qllm_provider_logits(const qllm_provider* provider);
+const float* qllm_provider_hidden(const qllm_provider* provider);
+void* qllm_provider_stream(const qllm_provider* provider);
+uint64_t qllm_provider_weight_bytes(const qllm_provider* provider);
+/* telemetry(): value of one counter, 0 if unknown. */
+uint64_t qllm_provider_telemetry(const qllm_provider* provider,
+                                 const char* name);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

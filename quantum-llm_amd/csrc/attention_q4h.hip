@@ -648,6 +648,7 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
   float* k = key + (static_cast<size_t>(row) * kv_heads + head) * head_dim;
   head_norm_rope(k, k_weight, head_dim, rotary_dim, rotary_position, epsilon,
                  theta, bf16_activations, shared, lane);
+  if (!page_table) return;  // rotary only; the caller stores K/V itself
   __threadfence_block();
   const uint32_t position = first_cache_position + row;
   uint8_t* page = static_cast<uint8_t*>(
@@ -780,6 +781,26 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
       epsilon, rope_theta, bf16_activations != 0);
   return launched("Q4H QKV rope cache batch");
+}
+
+extern "C" int32_t qllm_qkv_rope_batch(
+    float* query, uint32_t query_stride, float* key,
+    const float* q_norm_weight, const float* k_norm_weight,
+    uint32_t first_rotary_position, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream) {
+  if (!query || !key || !rows || !query_heads || !kv_heads ||
+      query_heads < kv_heads || query_heads % kv_heads || !head_dim ||
+      head_dim > 256u || head_dim % 2u || query_stride < head_dim ||
+      !rotary_dim || rotary_dim > head_dim || rotary_dim % 2u ||
+      !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
+      first_rotary_position > 0xffffffffu - (rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid QKV rope batch");
+  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+      query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
+      0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
+      rotary_dim, epsilon, rope_theta, bf16_activations != 0);
+  return launched("QKV rope batch");
 }
 
 extern "C" int32_t qllm_quantize_gqa_queries_q8(

@@ -1,0 +1,1041 @@
+#include "dense_fp4_provider.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <bit>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+#include <stdexcept>
+
+namespace qllm {
+namespace {
+
+constexpr std::uint32_t kMaximumGpuSamplingTopK = 64U;  // provider.cpp:8359
+
+void hip_check(hipError_t error, const char* what) {
+  if (error != hipSuccess)
+    throw std::runtime_error(std::string(what) + ": " +
+                             hipGetErrorString(error));
+}
+
+void status_check(std::int32_t status) {
+  if (status != QLLM_OK) throw std::runtime_error(qllm_last_error());
+}
+
+std::uint32_t pad32(std::uint32_t value) { return (value + 31U) / 32U * 32U; }
+
+std::uint64_t request_parameter(const er::ProgramRequestContext& request,
+                                std::string_view name) {
+  const auto found = request.parameters.find(name);
+  if (found == request.parameters.end())
+    throw std::runtime_error("request parameter is absent: " +
+                             std::string(name));
+  return found->second;
+}
+
+er::ExactDecodeExecutionHandle completed_exact(
+    er::ExactDecodeExecutionResult result) {
+  auto shared = std::make_shared<std::optional<er::ExactDecodeExecutionResult>>(
+      std::move(result));
+  return er::ExactDecodeExecutionHandle::from_callbacks(
+      [shared]() {
+        auto value = std::move(*shared);
+        shared->reset();
+        return value;
+      },
+      []() {});
+}
+
+const er::ImmutableModelTensor& tensor_for(
+    std::span<const er::PreparedTensorBinding> tensors, std::string_view role) {
+  for (const auto& binding : tensors)
+    if (binding.role == role && binding.tensor) return *binding.tensor;
+  throw std::runtime_error("tensor role is not bound: " + std::string(role));
+}
+
+const er::ImmutableModelTensor* optional_tensor(
+    std::span<const er::PreparedTensorBinding> tensors, std::string_view role) {
+  for (const auto& binding : tensors)
+    if (binding.role == role && binding.tensor) return binding.tensor.get();
+  return nullptr;
+}
+
+class PreparedMarker final : public er::IPreparedOperation {
+ public:
+  explicit PreparedMarker(std::string capability)
+      : capability_(std::move(capability)) {}
+  const std::string& capability() const noexcept { return capability_; }
+
+ private:
+  std::string capability_;
+};
+
+er::Status validate_parameters(
+    const std::map<std::string, std::uint64_t, std::less<>>& parameters) {
+  for (const auto& [name, value] : parameters) {
+    if (name.size() > 9 && name.ends_with("_f32_bits")) {
+      const auto number =
+          std::bit_cast<float>(static_cast<std::uint32_t>(value));
+      if (!std::isfinite(number) || !(number > 0.0F))
+        return {er::ErrorCode::invalid_argument,
+                "float parameter is not finite and positive: " + name};
+    }
+  }
+  return er::Status::success();
+}
+
+}  // namespace
+
+struct Mi355DenseFp4Provider::PreparedOp {};
+
+er::WorkerProviderDefinition make_mi355_dense_fp4_provider() {
+  const auto validator = [](const auto& parameters) {
+    return validate_parameters(parameters);
+  };
+  // The capability strings the dense Qwen-style program requires
+  // (dense_fp4_provider.cpp:996-1052; emitted by
+  // compiler/expert_pack/adapters.py:1682-1697) plus the block-16 variants.
+  return {"mi355-dense-fp4",
+          200U,
+          {{"embedding.lookup.fp4-block32.v1", 1U, 2U, validator},
+           {"dense.activation-input.bfloat16.v1", 1U, 1U, validator},
+           {"block.full-attention.output-gated.v1", 1U, 2U, validator},
+           {"block.full-attention.standard-gqa.v1", 1U, 1U, validator},
+           {"ffn.swiglu.dense.fp4-block32.v1", 1U, 2U, validator},
+           {"head.rmsnorm.token-select.fp4-block32.v1", 1U, 2U, validator},
+           {"decode.mtp.dense-full-attention.fp4-block32.exact.v2", 2U, 2U,
+            validator},
+           {"embedding.lookup.fp4-f16-block16.v1", 1U, 1U, validator},
+           {"ffn.swiglu.dense.fp4-f16-block16.v1", 1U, 1U, validator},
+           {"head.rmsnorm.token-select.fp4-f16-block16.v1", 1U, 1U, validator},
+           {"decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2", 2U, 2U,
+            validator}},
+          nullptr};
+}
+
+Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
+    : g_(geometry) {
+  const bool bad =
+      !g_.hidden || !g_.intermediate || !g_.layers || !g_.query_heads ||
+      !g_.kv_heads || g_.query_heads % g_.kv_heads || !g_.vocabulary ||
+      (g_.head_dim != 128U && g_.head_dim != 256U) || !g_.rotary_dim ||
+      g_.rotary_dim > g_.head_dim || g_.rotary_dim % 2U ||
+      !g_.kv_page_tokens || g_.kv_page_tokens % 64U || !g_.max_context ||
+      g_.draft_depth == 0U || g_.draft_depth > 7U || g_.hidden % 64U ||
+      g_.intermediate % 64U || (g_.query_heads * g_.head_dim) % 64U ||
+      g_.scale_scheme > QLLM_SCALE_F16_BLOCK16 ||
+      !(g_.norm_epsilon > 0.0F) || !(g_.rope_theta > 0.0F);
+  if (bad) throw std::invalid_argument("dense FP4 geometry is not supported");
+  if (g_.kv_encoding == KvEncoding::fp16 &&
+      g_.query_heads / g_.kv_heads > 16U)
+    throw std::invalid_argument("exact F16 KV supports at most 16 grouped heads");
+  hipStream_t stream{};
+  hip_check(hipStreamCreate(&stream), "create provider stream");
+  stream_ = stream;
+  layers_.resize(g_.layers);
+  accepted_depth_calls_.assign(g_.draft_depth + 1U, 0U);
+  max_rows_ = g_.draft_depth + 1U;
+  try {
+    allocate_workspaces();
+  } catch (...) {
+    release();
+    throw;
+  }
+}
+
+Mi355DenseFp4Provider::~Mi355DenseFp4Provider() { release(); }
+
+void Mi355DenseFp4Provider::release() {
+  if (graph_exec_) {
+    (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
+    graph_exec_ = nullptr;
+  }
+  if (stream_) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
+  for (void* pointer : allocations_) (void)hipFree(pointer);
+  allocations_.clear();
+  for (void* page : pages_)
+    if (page) (void)hipFree(page);
+  pages_.clear();
+  if (stream_) {
+    (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
+    stream_ = nullptr;
+  }
+}
+
+std::uint64_t Mi355DenseFp4Provider::kv_bytes_per_token_layer() const noexcept {
+  if (g_.kv_encoding == KvEncoding::fp16)
+    return std::uint64_t{g_.kv_heads} * g_.head_dim * 2U * 2U;
+  return std::uint64_t{g_.kv_heads} * 2U * (g_.head_dim / 2U + 2U);
+}
+
+void Mi355DenseFp4Provider::allocate_workspaces() {
+  const auto device_alloc = [this](std::size_t bytes) {
+    void* pointer{};
+    hip_check(hipMalloc(&pointer, bytes), "allocate provider workspace");
+    allocations_.push_back(pointer);
+    return pointer;
+  };
+  const std::size_t rows = max_rows_;
+  const std::size_t query_width =
+      std::size_t{g_.query_heads} * g_.head_dim * (g_.output_gated ? 2U : 1U);
+  const std::size_t kv_width = std::size_t{g_.kv_heads} * g_.head_dim;
+  const std::size_t widest =
+      std::max<std::size_t>({g_.hidden, g_.intermediate,
+                             std::size_t{g_.query_heads} * g_.head_dim});
+  tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+  hidden_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
+  normalized_ = static_cast<std::uint16_t*>(device_alloc(rows * widest * 2U));
+  query_ = static_cast<float*>(device_alloc(rows * query_width * 4U));
+  key_ = static_cast<float*>(device_alloc(rows * kv_width * 4U));
+  value_ = static_cast<float*>(device_alloc(rows * kv_width * 4U));
+  attention_ = static_cast<std::uint16_t*>(
+      device_alloc(rows * g_.query_heads * g_.head_dim * 2U));
+  activation_ =
+      static_cast<std::uint16_t*>(device_alloc(rows * g_.intermediate * 2U));
+  logits_ = static_cast<float*>(device_alloc(rows * g_.vocabulary * 4U));
+
+  // Context splits: a split is a multiple of 64 tokens sized so that
+  // kv_heads * splits workgroups roughly fill the 256 CUs at full context,
+  // never shorter than 512 tokens (one 64-token tile per wave).
+  const std::uint32_t wanted_splits =
+      std::max(1U, 256U / std::max(1U, g_.kv_heads));
+  std::uint32_t split = (g_.max_context + wanted_splits - 1U) / wanted_splits;
+  split = std::max(512U, (split + 63U) / 64U * 64U);
+  split_tokens_ = split;
+  maximum_splits_ = (g_.max_context + split - 1U) / split;
+  const std::size_t partials = rows * maximum_splits_ * g_.query_heads;
+  partial_maxima_ = static_cast<float*>(device_alloc(partials * 4U));
+  partial_sums_ = static_cast<float*>(device_alloc(partials * 4U));
+  partial_outputs_ =
+      static_cast<float*>(device_alloc(partials * g_.head_dim * 4U));
+
+  select_workspace_bytes_ = std::max(
+      qllm_argmax_workspace_bytes(g_.vocabulary, max_rows_),
+      qllm_topk_workspace_bytes(g_.vocabulary, kMaximumGpuSamplingTopK));
+  select_workspace_ = device_alloc(select_workspace_bytes_);
+  argmax_tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+  top_logits_ = static_cast<float*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
+  top_tokens_ =
+      static_cast<std::uint32_t*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
+
+  // Page geometry: every page holds all layers back to back
+  // (dense_fp4_provider.cpp:2582-2599, 6554-6588).
+  kv_page_bytes_ = kv_bytes_per_token_layer() * g_.kv_page_tokens * g_.layers;
+  const std::size_t page_count =
+      (g_.max_context + g_.kv_page_tokens - 1U) / g_.kv_page_tokens;
+  pages_.assign(page_count, nullptr);
+  device_page_table_ =
+      static_cast<void**>(device_alloc(page_count * sizeof(void*)));
+  hip_check(hipMemset(device_page_table_, 0, page_count * sizeof(void*)),
+            "clear device page table");
+}
+
+void Mi355DenseFp4Provider::ensure_pages(std::uint32_t last_position) {
+  const std::size_t last_page = last_position / g_.kv_page_tokens;
+  if (last_page >= pages_.size())
+    throw std::runtime_error("KV position exceeds the configured context");
+  for (std::size_t page = 0; page <= last_page; ++page) {
+    if (pages_[page]) continue;
+    void* pointer{};
+    hip_check(hipMalloc(&pointer, kv_page_bytes_), "allocate KV page");
+    hip_check(hipMemset(pointer, 0, kv_page_bytes_), "clear KV page");
+    pages_[page] = pointer;
+    hip_check(hipMemcpy(device_page_table_ + page, &pointer, sizeof(pointer),
+                        hipMemcpyHostToDevice),
+              "publish KV page");
+  }
+}
+
+DeviceFp4Matrix Mi355DenseFp4Provider::upload_matrix(
+    const er::ImmutableModelTensor& tensor, bool tiled) {
+  if (tensor.encoding != "FP4_E2M1" || tensor.shape.size() != 2U ||
+      !tensor.value.valid())
+    throw std::runtime_error("FP4 tensor is invalid: " + tensor.name);
+  const std::uint32_t rows = tensor.shape[0];
+  const std::uint32_t columns = tensor.shape[1];
+  const std::uint32_t padded = pad32(columns);
+  const bool block16 = tensor.quant_abi == 16U;
+  if (!block16 && tensor.quant_abi != 3U)
+    throw std::runtime_error("FP4 tensor quant ABI is not supported: " +
+                             tensor.name);
+  const std::uint64_t code_bytes = std::uint64_t{rows} * padded / 2U;
+  const std::uint64_t scale_bytes =
+      block16 ? std::uint64_t{rows} * (padded / 16U) * 2U
+              : std::uint64_t{rows} * (padded / 32U);
+  // geometry check of dense_fp4_provider.cpp:3569-3580
+  if (tensor.data_bytes != code_bytes || tensor.scale_bytes != scale_bytes ||
+      tensor.data_offset + code_bytes > tensor.value.bytes ||
+      tensor.scale_offset + scale_bytes > tensor.value.bytes)
+    throw std::runtime_error("FP4 tensor geometry mismatch: " + tensor.name);
+
+  void* staged_codes{};
+  void* staged_scales{};
+  hip_check(hipMalloc(&staged_codes, code_bytes), "allocate FP4 weights");
+  hip_check(hipMalloc(&staged_scales, scale_bytes), "allocate FP4 scales");
+  hip_check(hipMemcpy(staged_codes, tensor.value.data + tensor.data_offset,
+                      code_bytes, hipMemcpyHostToDevice),
+            "upload FP4 weights");
+  hip_check(hipMemcpy(staged_scales, tensor.value.data + tensor.scale_offset,
+                      scale_bytes, hipMemcpyHostToDevice),
+            "upload FP4 scales");
+  DeviceFp4Matrix matrix;
+  matrix.descriptor = {static_cast<const std::uint8_t*>(staged_codes),
+                       staged_scales,
+                       rows,
+                       columns,
+                       padded,
+                       block16 ? std::uint32_t{QLLM_SCALE_F16_BLOCK16}
+                               : std::uint32_t{QLLM_SCALE_UE8M0_BLOCK32},
+                       QLLM_LAYOUT_ROW_MAJOR,
+                       0U};
+  if (tiled && padded % 64U == 0U) {
+    void* packed_codes{};
+    void* packed_scales{};
+    hip_check(hipMalloc(&packed_codes, qllm_fp4_packed_weight_bytes(rows, padded)),
+              "allocate tiled FP4 weights");
+    hip_check(hipMalloc(&packed_scales,
+                        qllm_fp4_packed_scale_bytes(
+                            rows, padded, matrix.descriptor.scale_scheme)),
+              "allocate tiled FP4 scales");
+    qllm_fp4_matrix packed{};
+    status_check(qllm_fp4_prepack(&matrix.descriptor, packed_codes,
+                                  packed_scales, &packed, stream_));
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "prepack FP4 weights");
+    (void)hipFree(staged_codes);
+    (void)hipFree(staged_scales);
+    matrix.descriptor = packed;
+    staged_codes = packed_codes;
+    staged_scales = packed_scales;
+  }
+  matrix.weights = staged_codes;
+  matrix.scales = staged_scales;
+  allocations_.push_back(staged_codes);
+  allocations_.push_back(staged_scales);
+  weight_bytes_ += code_bytes + scale_bytes;
+  return matrix;
+}
+
+float* Mi355DenseFp4Provider::upload_f32(const er::ImmutableModelTensor& tensor,
+                                         std::uint32_t elements) {
+  if (tensor.encoding != "F32" || !tensor.value.valid() ||
+      tensor.data_bytes != std::uint64_t{elements} * 4U ||
+      tensor.data_offset + tensor.data_bytes > tensor.value.bytes)
+    throw std::runtime_error("F32 tensor is invalid: " + tensor.name);
+  void* pointer{};
+  hip_check(hipMalloc(&pointer, tensor.data_bytes), "allocate F32 tensor");
+  allocations_.push_back(pointer);
+  hip_check(hipMemcpy(pointer, tensor.value.data + tensor.data_offset,
+                      tensor.data_bytes, hipMemcpyHostToDevice),
+            "upload F32 tensor");
+  return static_cast<float*>(pointer);
+}
+
+er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
+    const er::OperationPreparationContext& context) {
+  try {
+    std::lock_guard lock(mutex_);
+    auto status = validate_parameters(context.parameters);
+    if (!status.ok()) return {status, {}};
+    const std::string& capability = context.capability;
+    const auto query_rows =
+        g_.query_heads * g_.head_dim * (g_.output_gated ? 2U : 1U);
+    const auto require_shape = [](const DeviceFp4Matrix& matrix,
+                                  std::uint32_t rows, std::uint32_t columns,
+                                  const char* role) {
+      if (matrix.descriptor.rows != rows || matrix.descriptor.columns != columns)
+        throw std::runtime_error(std::string("tensor shape mismatch: ") + role);
+    };
+    if (capability.starts_with("embedding.lookup.")) {
+      embedding_ = upload_matrix(tensor_for(context.tensors, "token_embedding"),
+                                 false);
+      require_shape(embedding_, g_.vocabulary, g_.hidden, "token_embedding");
+      embedding_ready_ = true;
+    } else if (capability.starts_with("block.full-attention.")) {
+      const bool gated = capability.find("output-gated") != std::string::npos;
+      if (gated != g_.output_gated)
+        throw std::runtime_error(
+            "attention capability does not match the declared geometry");
+      if (attention_ops_ >= g_.layers)
+        throw std::runtime_error("more attention blocks than layers");
+      auto& layer = layers_[attention_ops_];
+      layer.input_norm =
+          upload_f32(tensor_for(context.tensors, "input_norm"), g_.hidden);
+      layer.query = upload_matrix(
+          tensor_for(context.tensors, "query_projection"), true);
+      layer.key =
+          upload_matrix(tensor_for(context.tensors, "key_projection"), true);
+      layer.value =
+          upload_matrix(tensor_for(context.tensors, "value_projection"), true);
+      layer.output = upload_matrix(
+          tensor_for(context.tensors, "output_projection"), true);
+      require_shape(layer.query, query_rows, g_.hidden, "query_projection");
+      require_shape(layer.key, g_.kv_heads * g_.head_dim, g_.hidden,
+                    "key_projection");
+      require_shape(layer.value, g_.kv_heads * g_.head_dim, g_.hidden,
+                    "value_projection");
+      require_shape(layer.output, g_.hidden, g_.query_heads * g_.head_dim,
+                    "output_projection");
+      if (g_.qk_norm) {
+        layer.query_norm =
+            upload_f32(tensor_for(context.tensors, "query_norm"), g_.head_dim);
+        layer.key_norm =
+            upload_f32(tensor_for(context.tensors, "key_norm"), g_.head_dim);
+      }
+      ++attention_ops_;
+    } else if (capability.starts_with("ffn.swiglu.dense.")) {
+      if (ffn_ops_ >= g_.layers)
+        throw std::runtime_error("more FFN blocks than layers");
+      auto& layer = layers_[ffn_ops_];
+      layer.post_attention_norm = upload_f32(
+          tensor_for(context.tensors, "post_attention_norm"), g_.hidden);
+      layer.gate =
+          upload_matrix(tensor_for(context.tensors, "gate_projection"), true);
+      layer.up =
+          upload_matrix(tensor_for(context.tensors, "up_projection"), true);
+      layer.down =
+          upload_matrix(tensor_for(context.tensors, "down_projection"), true);
+      require_shape(layer.gate, g_.intermediate, g_.hidden, "gate_projection");
+      require_shape(layer.up, g_.intermediate, g_.hidden, "up_projection");
+      require_shape(layer.down, g_.hidden, g_.intermediate, "down_projection");
+      ++ffn_ops_;
+    } else if (capability.starts_with("head.rmsnorm.token-select.")) {
+      final_norm_ =
+          upload_f32(tensor_for(context.tensors, "hidden_norm"), g_.hidden);
+      head_ = upload_matrix(tensor_for(context.tensors, "output_head"), true);
+      require_shape(head_, g_.vocabulary, g_.hidden, "output_head");
+      head_ready_ = true;
+    } else {
+      return {{er::ErrorCode::invalid_argument,
+               "capability is not provided: " + capability},
+              {}};
+    }
+    (void)optional_tensor;
+    return {er::Status::success(),
+            std::make_shared<PreparedMarker>(capability)};
+  } catch (const std::exception& error) {
+    return {{er::ErrorCode::internal, error.what()}, {}};
+  }
+}
+
+er::PrepareOperationResult Mi355DenseFp4Provider::prepare_exact_decode(
+    const er::ExactDecodePreparationContext& context) {
+  try {
+    std::lock_guard lock(mutex_);
+    if (!context.capability.starts_with("decode.mtp.dense-full-attention.") ||
+        context.abi != 2U)
+      return {{er::ErrorCode::invalid_argument,
+               "exact decode capability or ABI is not provided"},
+              {}};
+    const auto depth = context.parameters.find("draft_depth");
+    if (depth == context.parameters.end() || depth->second != g_.draft_depth)
+      return {{er::ErrorCode::invalid_argument,
+               "exact decode draft depth does not match the provider"},
+              {}};
+    if (!embedding_ready_ || !head_ready_ || attention_ops_ != g_.layers ||
+        ffn_ops_ != g_.layers)
+      return {{er::ErrorCode::invalid_argument,
+               "target program is not fully prepared"},
+              {}};
+    exact_ = std::make_shared<PreparedMarker>(context.capability);
+    return {er::Status::success(), exact_};
+  } catch (const std::exception& error) {
+    return {{er::ErrorCode::internal, error.what()}, {}};
+  }
+}
+
+er::CreateOperationRequestStateResult
+Mi355DenseFp4Provider::create_request_state(const er::ProgramRequestContext&) {
+  try {
+    return {er::Status::success(), std::make_shared<DenseFp4RequestState>()};
+  } catch (const std::exception& error) {
+    return {{er::ErrorCode::internal, error.what()}, {}};
+  }
+}
+
+// Records where the verified stream stands after prefill / a previous step
+// (dense_fp4_provider.cpp:11011-11130).  Producing the drafts themselves is
+// the proposer's job; they arrive through set_draft_predictions().
+er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
+    const er::IPreparedOperation& operation,
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    const er::ExactDecodeSynchronizationBatch& synchronization) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto state =
+        std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+    if (&operation != exact_.get() || !state ||
+        synchronization.next_tokens.empty())
+      return {er::ErrorCode::invalid_argument,
+              "exact decode synchronization is invalid"};
+    for (const auto token : synchronization.next_tokens)
+      if (token >= g_.vocabulary)
+        return {er::ErrorCode::invalid_argument,
+                "synchronized token is outside the vocabulary"};
+    state->synchronized_token = synchronization.next_tokens.back();
+    state->mtp_length =
+        synchronization.first_target_position +
+        static_cast<std::uint32_t>(synchronization.next_tokens.size()) - 1U;
+    state->draft_valid = false;
+    state->draft_predictions.clear();
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::set_draft_predictions(
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    std::vector<DraftPrediction> drafts) {
+  std::lock_guard lock(mutex_);
+  const auto state =
+      std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+  if (!state || drafts.empty() || drafts.size() > g_.draft_depth)
+    return {er::ErrorCode::invalid_argument, "draft predictions are invalid"};
+  for (const auto& draft : drafts)
+    if (draft.token >= g_.vocabulary)
+      return {er::ErrorCode::invalid_argument,
+              "draft token is outside the vocabulary"};
+  state->draft_predictions = std::move(drafts);
+  state->draft_valid = true;
+  return er::Status::success();
+}
+
+// ---- target pass ------------------------------------------------------------
+
+void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
+                                           std::uint32_t rows,
+                                           std::uint32_t first_position) {
+  void* const stream = stream_;
+  const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+  const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
+  const std::size_t attention_bytes =
+      std::size_t{rows} * g_.query_heads * g_.head_dim * 2U;
+  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
+                                        hidden_, rows, stream));
+  for (std::uint32_t index = 0; index < g_.layers; ++index) {
+    const auto& layer = layers_[index];
+    // full attention block (run_full_attention, :6892)
+    status_check(qllm_rms_norm_batch(hidden_, layer.input_norm, nullptr,
+                                     normalized_, g_.hidden, rows, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm,
+                                     stream));
+    status_check(qllm_fp4_gemm_bf16(&layer.query.descriptor, normalized_,
+                                    hidden_bytes, query_, QLLM_OUT_F32, nullptr,
+                                    rows, stream));
+    status_check(qllm_fp4_gemm_bf16(&layer.key.descriptor, normalized_,
+                                    hidden_bytes, key_, QLLM_OUT_F32, nullptr,
+                                    rows, stream));
+    status_check(qllm_fp4_gemm_bf16(&layer.value.descriptor, normalized_,
+                                    hidden_bytes, value_, QLLM_OUT_F32, nullptr,
+                                    rows, stream));
+    if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
+      status_check(qllm_qkv_rope_cache_paged_q4h_batch(
+          query_, query_stride, key_, value_, layer.query_norm, layer.key_norm,
+          const_cast<const void* const*>(device_page_table_), index,
+          g_.kv_page_tokens, first_position, first_position, rows,
+          g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
+          g_.norm_epsilon, g_.rope_theta, 0, stream));
+      qllm_q4h_attention_launch launch{};
+      launch.query = query_;
+      launch.page_table = const_cast<const void* const*>(device_page_table_);
+      launch.output = attention_;
+      launch.partial_maxima = partial_maxima_;
+      launch.partial_sums = partial_sums_;
+      launch.partial_outputs = partial_outputs_;
+      launch.first_context_tokens = first_position + 1U;  // :7915
+      launch.rows = rows;
+      launch.full_attention_layer = index;
+      launch.page_tokens = g_.kv_page_tokens;
+      launch.query_heads = g_.query_heads;
+      launch.kv_heads = g_.kv_heads;
+      launch.head_dim = g_.head_dim;
+      launch.split_tokens = split_tokens_;
+      launch.maximum_splits = maximum_splits_;
+      launch.query_stride = query_stride;
+      launch.output_gated = g_.output_gated;
+      launch.output_kind = QLLM_OUT_BF16;
+      launch.stream = stream;
+      status_check(qllm_attention_paged_q4h(&launch));
+    } else {
+      status_check(qllm_qkv_rope_batch(
+          query_, query_stride, key_, layer.query_norm, layer.key_norm,
+          first_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
+          g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+      status_check(qllm_store_kv_paged_f16_batch(
+          key_, value_, const_cast<const void* const*>(device_page_table_),
+          index, g_.kv_page_tokens, first_position, rows, g_.kv_heads,
+          g_.head_dim, stream));
+      qllm_f16_attention_launch launch{};
+      launch.query = query_;
+      launch.device_pages = const_cast<const void* const*>(device_page_table_);
+      launch.output = attention_;
+      launch.partial_maxima = partial_maxima_;
+      launch.partial_sums = partial_sums_;
+      launch.partial_outputs = partial_outputs_;
+      launch.first_context_tokens = first_position + 1U;
+      launch.rows = rows;
+      launch.device_page_layer = index;
+      launch.device_page_tokens = g_.kv_page_tokens;
+      launch.query_heads = g_.query_heads;
+      launch.kv_heads = g_.kv_heads;
+      launch.head_dim = g_.head_dim;
+      launch.split_tokens = split_tokens_;
+      launch.maximum_splits = maximum_splits_;
+      launch.query_stride = query_stride;
+      launch.output_gated = g_.output_gated;
+      launch.output_kind = QLLM_OUT_BF16;
+      launch.stream = stream;
+      status_check(qllm_attention_paged_f16(&launch));
+    }
+    status_check(qllm_fp4_gemm_bf16(&layer.output.descriptor, attention_,
+                                    attention_bytes, hidden_, QLLM_OUT_F32,
+                                    hidden_, rows, stream));
+    // dense SwiGLU block (run_ffn, :8250-8293)
+    status_check(qllm_rms_norm_batch(hidden_, layer.post_attention_norm,
+                                     nullptr, normalized_, g_.hidden, rows,
+                                     g_.hidden, g_.norm_epsilon,
+                                     g_.zero_centered_norm, stream));
+    status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
+                                      &layer.up.descriptor, normalized_,
+                                      hidden_bytes, activation_, rows, stream));
+    status_check(qllm_fp4_gemm_bf16(
+        &layer.down.descriptor, activation_,
+        std::size_t{rows} * g_.intermediate * 2U, hidden_, QLLM_OUT_F32,
+        hidden_, rows, stream));
+  }
+  // head (run_head, :8393-8527)
+  status_check(qllm_rms_norm_batch(hidden_, final_norm_, nullptr, normalized_,
+                                   g_.hidden, rows, g_.hidden, g_.norm_epsilon,
+                                   g_.zero_centered_norm, stream));
+  status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_, hidden_bytes,
+                                  logits_, QLLM_OUT_F32, nullptr, rows, stream));
+  status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
+                                 select_workspace_, select_workspace_bytes_,
+                                 stream));
+}
+
+er::Status Mi355DenseFp4Provider::run_target(const std::uint32_t* tokens,
+                                             std::uint32_t rows,
+                                             std::uint32_t first_position) {
+  try {
+    if (!tokens || !rows || rows > max_rows_ ||
+        first_position > g_.max_context - rows)
+      return {er::ErrorCode::invalid_argument, "target rows are invalid"};
+    if (!embedding_ready_ || !head_ready_)
+      return {er::ErrorCode::invalid_argument, "target program is not prepared"};
+    ensure_pages(first_position + rows - 1U);
+    hip_check(hipMemcpyAsync(tokens_, tokens, rows * sizeof(std::uint32_t),
+                             hipMemcpyHostToDevice,
+                             static_cast<hipStream_t>(stream_)),
+              "upload target tokens");
+    enqueue_target(tokens_, rows, first_position);
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::capture_target_graph(
+    const std::uint32_t* tokens, std::uint32_t rows,
+    std::uint32_t first_position) {
+  try {
+    if (!tokens || !rows || rows > max_rows_ ||
+        first_position > g_.max_context - rows)
+      return {er::ErrorCode::invalid_argument, "target rows are invalid"};
+    ensure_pages(first_position + rows - 1U);
+    const auto stream = static_cast<hipStream_t>(stream_);
+    hip_check(hipMemcpy(tokens_, tokens, rows * sizeof(std::uint32_t),
+                        hipMemcpyHostToDevice),
+              "upload target tokens");
+    if (graph_exec_) {
+      hip_check(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_)),
+                "destroy previous graph");
+      graph_exec_ = nullptr;
+    }
+    hipGraph_t graph{};
+    hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal),
+              "begin target capture");
+    try {
+      enqueue_target(tokens_, rows, first_position);
+    } catch (...) {
+      (void)hipStreamEndCapture(stream, &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      throw;
+    }
+    hip_check(hipStreamEndCapture(stream, &graph), "end target capture");
+    hipGraphExec_t exec{};
+    const auto status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    hip_check(status, "instantiate target graph");
+    graph_exec_ = exec;
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::replay_target_graph() {
+  if (!graph_exec_)
+    return {er::ErrorCode::invalid_argument, "no target graph was captured"};
+  const auto status = hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_),
+                                     static_cast<hipStream_t>(stream_));
+  if (status != hipSuccess)
+    return {er::ErrorCode::internal, hipGetErrorString(status)};
+  return er::Status::success();
+}
+
+er::Status Mi355DenseFp4Provider::synchronize() {
+  const auto status = hipStreamSynchronize(static_cast<hipStream_t>(stream_));
+  if (status != hipSuccess)
+    return {er::ErrorCode::internal, hipGetErrorString(status)};
+  return er::Status::success();
+}
+
+// ---- sampling ---------------------------------------------------------------
+
+// distribution_from_logits, dense_fp4_provider.cpp:8331-8391.  top_k == 0
+// selects the whole-vocabulary path of the scalar sampler (sample_token,
+// :773-799): the row is copied to the host and ordered there.
+er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
+    std::uint32_t row, const er::ProgramRequestContext& request) {
+  const auto stream = static_cast<hipStream_t>(stream_);
+  float* row_logits = logits_ + std::size_t{row} * g_.vocabulary;
+  const auto temperature = request_parameter(request, "sampling_temperature_ppm");
+  if (temperature == 0U) {
+    std::uint32_t token{};
+    hip_check(hipMemcpyAsync(&token, argmax_tokens_ + row, sizeof(token),
+                             hipMemcpyDeviceToHost, stream),
+              "copy exact greedy token");
+    hip_check(hipStreamSynchronize(stream), "copy exact greedy token");
+    return {{{token, 1.0}}};
+  }
+  const auto top_p = static_cast<std::uint32_t>(
+      request_parameter(request, "sampling_top_p_ppm"));
+  const auto min_p = static_cast<std::uint32_t>(
+      request_parameter(request, "sampling_min_p_ppm"));
+  const auto top_k = request_parameter(request, "sampling_top_k");
+  if (top_k > kMaximumGpuSamplingTopK || top_k > g_.vocabulary)
+    throw std::runtime_error(
+        "sampled exact decode requires top-k of at most 64 (0 = whole row)");
+  std::vector<float> host_logits;
+  std::vector<std::uint32_t> host_tokens;
+  if (top_k == 0U) {
+    std::vector<float> full(g_.vocabulary);
+    hip_check(hipMemcpyAsync(full.data(), row_logits, full.size() * 4U,
+                             hipMemcpyDeviceToHost, stream),
+              "copy logit row");
+    hip_check(hipStreamSynchronize(stream), "copy logit row");
+    host_tokens.resize(g_.vocabulary);
+    std::iota(host_tokens.begin(), host_tokens.end(), 0U);
+    std::sort(host_tokens.begin(), host_tokens.end(),
+              [&](std::uint32_t left, std::uint32_t right) {
+                const float a = full[left];
+                const float b = full[right];
+                if (std::isnan(a)) return false;
+                if (std::isnan(b)) return true;
+                return a == b ? left < right : a > b;
+              });
+    host_logits.reserve(g_.vocabulary);
+    for (const auto token : host_tokens) host_logits.push_back(full[token]);
+    sampling_logit_transfer_bytes_ += full.size() * 4U;
+  } else {
+    status_check(qllm_topk_logits(row_logits, g_.vocabulary,
+                                  static_cast<std::uint32_t>(top_k), top_logits_,
+                                  top_tokens_, select_workspace_,
+                                  select_workspace_bytes_, stream_));
+    host_logits.resize(top_k);
+    host_tokens.resize(top_k);
+    hip_check(hipMemcpyAsync(host_logits.data(), top_logits_, top_k * 4U,
+                             hipMemcpyDeviceToHost, stream),
+              "copy speculative top-k logits");
+    hip_check(hipMemcpyAsync(host_tokens.data(), top_tokens_, top_k * 4U,
+                             hipMemcpyDeviceToHost, stream),
+              "copy speculative top-k tokens");
+    hip_check(hipStreamSynchronize(stream), "copy speculative top-k");
+    ++sampling_gpu_calls_;
+    sampling_logit_transfer_bytes_ += top_k * 8U;
+  }
+  return er::make_sampling_distribution(
+      host_logits, host_tokens, static_cast<std::uint32_t>(temperature), top_p,
+      min_p);
+}
+
+// ---- the verify step (execute_exact_decode ABI 2, :11156-11318) -------------
+
+er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
+    const er::IPreparedOperation& operation,
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    const er::ExactDecodeInvocation& invocation) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto state =
+        std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+    if (&operation != exact_.get() || !state || !state->draft_valid ||
+        invocation.guaranteed_token != state->synchronized_token ||
+        invocation.position != state->mtp_length ||
+        invocation.position + 1U >= invocation.context_limit ||
+        invocation.context_limit > g_.max_context)
+      throw std::runtime_error("exact MTP invocation stream is invalid");
+    const auto proposal_count = state->draft_predictions.size();
+    if (proposal_count == 0U || proposal_count > g_.draft_depth ||
+        invocation.position + proposal_count >= invocation.context_limit)
+      throw std::runtime_error("multi-draft MTP state is invalid");
+
+    std::vector<std::uint32_t> target_tokens{invocation.guaranteed_token};
+    for (const auto& proposal : state->draft_predictions) {
+      if (!(proposal.distribution.probability(proposal.token) > 0.0))
+        throw std::runtime_error("MTP proposal has zero draft mass");
+      target_tokens.push_back(proposal.token);
+    }
+    const auto rows = static_cast<std::uint32_t>(target_tokens.size());
+    auto status = run_target(target_tokens.data(), rows, invocation.position);
+    if (!status.ok()) throw std::runtime_error(std::string(status.message()));
+
+    std::vector<er::SamplingDistribution> target_distributions;
+    target_distributions.reserve(rows);
+    for (std::uint32_t row = 0; row < rows; ++row)
+      target_distributions.push_back(
+          distribution_from_logits(row, invocation.request));
+
+    const auto seed = request_parameter(invocation.request, "sampling_seed");
+    std::size_t accepted{};
+    std::uint32_t next_token{};
+    bool rejected{};
+    for (; accepted < proposal_count; ++accepted) {
+      const auto& proposal = state->draft_predictions[accepted];
+      const auto depth = static_cast<std::uint32_t>(accepted);
+      const auto decision = er::rejection_sample(
+          proposal.token, target_distributions[accepted], proposal.distribution,
+          er::counter_uniform(seed, invocation.position + depth, 100U, depth),
+          er::counter_uniform(seed, invocation.position + depth, 200U, depth));
+      if (!decision.accepted) {
+        next_token = decision.token;
+        rejected = true;
+        break;
+      }
+    }
+    if (!rejected)
+      next_token = er::sample_distribution(
+          target_distributions.back(),
+          er::counter_uniform(
+              seed, invocation.position + static_cast<std::uint32_t>(accepted),
+              300U));
+
+    const auto positions_advanced = static_cast<std::uint32_t>(accepted + 1U);
+    state->mtp_length = invocation.position + positions_advanced;
+    state->synchronized_token = next_token;
+    state->draft_valid = false;
+    state->draft_predictions.clear();
+
+    er::ExactDecodeExecutionResult result;
+    result.status = er::Status::success();
+    result.emitted_tokens.push_back(invocation.guaranteed_token);
+    for (std::size_t index = 0; index < accepted; ++index)
+      result.emitted_tokens.push_back(target_tokens[index + 1U]);
+    result.next_token = next_token;
+    result.positions_advanced = positions_advanced;
+    ++exact_calls_;
+    accepted_drafts_ += accepted;
+    ++accepted_depth_calls_.at(accepted);
+    program_steps_ += positions_advanced;
+    return completed_exact(std::move(result));
+  } catch (const std::exception& error) {
+    er::ExactDecodeExecutionResult failure;
+    failure.status = {er::ErrorCode::internal, error.what()};
+    return completed_exact(std::move(failure));
+  }
+}
+
+// ---- synthetic model / cache ---------------------------------------------------
+
+DeviceFp4Matrix Mi355DenseFp4Provider::synthetic_matrix(std::uint32_t rows,
+                                                        std::uint32_t columns,
+                                                        std::uint64_t seed,
+                                                        bool tiled) {
+  const std::uint32_t padded = pad32(columns);
+  const bool block16 = g_.scale_scheme == QLLM_SCALE_F16_BLOCK16;
+  // the row-major and the tiled layout hold the same multiset of bytes per
+  // matrix; a random-init model may be generated in either directly
+  const std::size_t padded_rows = tiled ? (rows + 31U) / 32U * 32U : rows;
+  const std::size_t code_bytes = padded_rows * padded / 2U;
+  const std::size_t scale_count = padded_rows * (padded / (block16 ? 16U : 32U));
+  const std::size_t scale_bytes = scale_count * (block16 ? 2U : 1U);
+  void* codes{};
+  void* scales{};
+  hip_check(hipMalloc(&codes, code_bytes), "allocate synthetic weights");
+  hip_check(hipMalloc(&scales, scale_bytes), "allocate synthetic scales");
+  allocations_.push_back(codes);
+  allocations_.push_back(scales);
+  status_check(qllm_fill_random(codes, code_bytes, 0U, seed, stream_));
+  status_check(qllm_fill_random(scales, scale_count, block16 ? 3U : 5U,
+                                seed ^ 0x5ca1eULL, stream_));
+  DeviceFp4Matrix matrix;
+  matrix.weights = codes;
+  matrix.scales = scales;
+  matrix.descriptor = {static_cast<const std::uint8_t*>(codes),
+                       scales,
+                       rows,
+                       columns,
+                       padded,
+                       g_.scale_scheme,
+                       tiled && padded % 64U == 0U
+                           ? std::uint32_t{QLLM_LAYOUT_TILED}
+                           : std::uint32_t{QLLM_LAYOUT_ROW_MAJOR},
+                       0U};
+  weight_bytes_ += std::uint64_t{rows} * padded / 2U +
+                   std::uint64_t{rows} * (padded / (block16 ? 16U : 32U)) *
+                       (block16 ? 2U : 1U);
+  return matrix;
+}
+
+er::Status Mi355DenseFp4Provider::load_synthetic_weights(std::uint64_t seed) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto ones = [this](std::uint32_t elements, float value) {
+      std::vector<float> host(elements, value);
+      void* pointer{};
+      hip_check(hipMalloc(&pointer, elements * 4U), "allocate norm weight");
+      allocations_.push_back(pointer);
+      hip_check(hipMemcpy(pointer, host.data(), elements * 4U,
+                          hipMemcpyHostToDevice),
+                "upload norm weight");
+      return static_cast<float*>(pointer);
+    };
+    const float unit = g_.zero_centered_norm ? 0.0F : 1.0F;
+    const auto query_rows =
+        g_.query_heads * g_.head_dim * (g_.output_gated ? 2U : 1U);
+    std::uint64_t stream_seed = seed;
+    const auto next_seed = [&stream_seed]() {
+      stream_seed += 0x9e3779b97f4a7c15ULL;
+      return stream_seed;
+    };
+    embedding_ = synthetic_matrix(g_.vocabulary, g_.hidden, next_seed(), false);
+    for (auto& layer : layers_) {
+      layer.input_norm = ones(g_.hidden, unit);
+      layer.post_attention_norm = ones(g_.hidden, unit);
+      if (g_.qk_norm) {
+        layer.query_norm = ones(g_.head_dim, 0.0F);
+        layer.key_norm = ones(g_.head_dim, 0.0F);
+      }
+      layer.query = synthetic_matrix(query_rows, g_.hidden, next_seed(), true);
+      layer.key = synthetic_matrix(g_.kv_heads * g_.head_dim, g_.hidden,
+                                   next_seed(), true);
+      layer.value = synthetic_matrix(g_.kv_heads * g_.head_dim, g_.hidden,
+                                     next_seed(), true);
+      layer.output = synthetic_matrix(g_.hidden, g_.query_heads * g_.head_dim,
+                                      next_seed(), true);
+      layer.gate = synthetic_matrix(g_.intermediate, g_.hidden, next_seed(), true);
+      layer.up = synthetic_matrix(g_.intermediate, g_.hidden, next_seed(), true);
+      layer.down = synthetic_matrix(g_.hidden, g_.intermediate, next_seed(), true);
+    }
+    final_norm_ = ones(g_.hidden, unit);
+    head_ = synthetic_matrix(g_.vocabulary, g_.hidden, next_seed(), true);
+    attention_ops_ = ffn_ops_ = g_.layers;
+    embedding_ready_ = head_ready_ = true;
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "generate synthetic weights");
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::prefill_synthetic_kv(std::uint32_t tokens,
+                                                       std::uint64_t seed) {
+  try {
+    std::lock_guard lock(mutex_);
+    if (!tokens || tokens > g_.max_context)
+      return {er::ErrorCode::invalid_argument, "prefill length is invalid"};
+    ensure_pages(tokens - 1U);
+    const std::uint32_t chunk = 4096U;
+    const std::size_t width = std::size_t{g_.kv_heads} * g_.head_dim;
+    float* keys{};
+    float* values{};
+    hip_check(hipMalloc(&keys, chunk * width * 4U), "allocate prefill keys");
+    hip_check(hipMalloc(&values, chunk * width * 4U), "allocate prefill values");
+    for (std::uint32_t layer = 0; layer < g_.layers; ++layer) {
+      for (std::uint32_t first = 0; first < tokens; first += chunk) {
+        const std::uint32_t count = std::min(chunk, tokens - first);
+        const std::uint64_t salt =
+            seed + (std::uint64_t{layer} << 32U) + first;
+        status_check(qllm_fill_random(keys, count * width, 1U, salt, stream_));
+        status_check(qllm_fill_random(values, count * width, 1U,
+                                      salt ^ 0xabcdef12345ULL, stream_));
+        if (g_.kv_encoding == KvEncoding::q4_f16_per_head)
+          status_check(qllm_store_kv_paged_q4h_batch(
+              keys, values, const_cast<const void* const*>(device_page_table_),
+              layer, g_.kv_page_tokens, first, count, g_.kv_heads, g_.head_dim,
+              stream_));
+        else
+          status_check(qllm_store_kv_paged_f16_batch(
+              keys, values, const_cast<const void* const*>(device_page_table_),
+              layer, g_.kv_page_tokens, first, count, g_.kv_heads, g_.head_dim,
+              stream_));
+      }
+    }
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "prefill synthetic KV");
+    (void)hipFree(keys);
+    (void)hipFree(values);
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::copy_kv_page(std::uint32_t page_index,
+                                               void* host_output) {
+  std::lock_guard lock(mutex_);
+  if (!host_output || page_index >= pages_.size())
+    return {er::ErrorCode::invalid_argument, "KV page index is invalid"};
+  auto status = hipStreamSynchronize(static_cast<hipStream_t>(stream_));
+  if (status == hipSuccess) {
+    if (pages_[page_index])
+      status = hipMemcpy(host_output, pages_[page_index], kv_page_bytes_,
+                         hipMemcpyDeviceToHost);
+    else
+      std::memset(host_output, 0, kv_page_bytes_);
+  }
+  if (status != hipSuccess)
+    return {er::ErrorCode::internal, hipGetErrorString(status)};
+  return er::Status::success();
+}
+
+std::map<std::string, std::uint64_t, std::less<>>
+Mi355DenseFp4Provider::telemetry() const {
+  std::lock_guard lock(mutex_);
+  std::map<std::string, std::uint64_t, std::less<>> values;
+  values["provider_exact_calls"] = exact_calls_;
+  values["provider_accepted_drafts"] = accepted_drafts_;
+  values["provider_program_steps"] = program_steps_;
+  values["provider_sampling_gpu_calls"] = sampling_gpu_calls_;
+  values["provider_sampling_logit_transfer_bytes"] =
+      sampling_logit_transfer_bytes_;
+  for (std::size_t depth = 0; depth < accepted_depth_calls_.size(); ++depth)
+    values["provider_accepted_depth_" + std::to_string(depth)] =
+        accepted_depth_calls_[depth];
+  values["provider_weight_bytes"] = weight_bytes_;
+  values["provider_kv_page_bytes"] = kv_page_bytes_;
+  return values;
+}
+
+er::ServiceContract Mi355DenseFp4Provider::service_contract() const {
+  er::ServiceContract contract;
+  contract.kv_dtype = g_.kv_encoding == KvEncoding::fp16 ? "fp16"
+                                                          : "q4-f16-per-head";
+  contract.kv_allocation = "on-demand-pages";
+  contract.kv_page_tokens = g_.kv_page_tokens;
+  contract.kv_page_bytes = kv_page_bytes_;
+  contract.kv_page_capacity = pages_.size();
+  contract.placement_mode = "resident";
+  contract.mtp_resource_available = true;
+  contract.mtp_runtime_ready = static_cast<bool>(exact_);
+  contract.mtp_enabled = static_cast<bool>(exact_);
+  contract.sampling_supported = true;
+  return contract;
+}
+
+}  // namespace qllm

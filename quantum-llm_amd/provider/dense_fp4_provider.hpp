@@ -1,0 +1,218 @@
+// MI355X provider for the dense FP4 decoder's speculative verify step.
+//
+// Plays the role of the reference's "sm86-dense-fp4" provider
+// (runtime/tools/dense_fp4_provider.cpp): it implements IOperationProvider,
+// advertises the same capability strings, owns the device copies of the
+// weights, the paged KV cache and the step workspaces, and runs
+// execute_exact_decode (:11139-11318) - target pass over 1+drafts rows, target
+// distributions, accept-longest-prefix, residual/bonus token - by enqueueing
+// the gfx950 kernels of include/qllm_kernels.h on one HIP stream.
+#pragma once
+
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "qllm_kernels.h"
+#include "runtime_interface.hpp"
+#include "speculative_sampling.hpp"
+
+namespace qllm {
+
+namespace er = expert::runtime;
+
+enum class KvEncoding : std::uint32_t { q4_f16_per_head = 0, fp16 = 1 };
+
+// Geometry the artifact declares for the dense decoder
+// (validate_dense_fp4_descriptor, dense_fp4_provider.cpp:804-994).
+struct DenseGeometry final {
+  std::uint32_t hidden{};
+  std::uint32_t intermediate{};
+  std::uint32_t layers{};
+  std::uint32_t query_heads{};
+  std::uint32_t kv_heads{};
+  std::uint32_t head_dim{};
+  std::uint32_t rotary_dim{};
+  std::uint32_t vocabulary{};
+  float rope_theta{1.0e6F};
+  float norm_epsilon{1.0e-6F};
+  bool output_gated{};        // q projection emits [query, gate] per head
+  bool qk_norm{};             // per-head RMSNorm(1+w) on q and k
+  bool zero_centered_norm{};  // block norms use (1 + w)
+  std::uint32_t scale_scheme{QLLM_SCALE_F16_BLOCK16};
+  KvEncoding kv_encoding{KvEncoding::q4_f16_per_head};
+  std::uint32_t kv_page_tokens{256};
+  std::uint32_t max_context{};
+  std::uint32_t draft_depth{4};
+};
+
+struct DraftPrediction final {
+  std::uint32_t token{};
+  er::SamplingDistribution distribution;
+};
+
+class DenseFp4RequestState final : public er::IOperationProviderRequestState {
+ public:
+  std::uint32_t synchronized_token{};
+  std::uint32_t mtp_length{};   // position of the guaranteed token
+  bool draft_valid{};
+  std::vector<DraftPrediction> draft_predictions;
+};
+
+struct DeviceFp4Matrix final {
+  qllm_fp4_matrix descriptor{};
+  void* weights{};
+  void* scales{};
+};
+
+struct LayerWeights final {
+  float* input_norm{};
+  float* post_attention_norm{};
+  float* query_norm{};
+  float* key_norm{};
+  DeviceFp4Matrix query, key, value, output, gate, up, down;
+};
+
+class Mi355DenseFp4Provider final : public er::IOperationProvider {
+ public:
+  explicit Mi355DenseFp4Provider(const DenseGeometry& geometry);
+  ~Mi355DenseFp4Provider() override;
+  Mi355DenseFp4Provider(const Mi355DenseFp4Provider&) = delete;
+  Mi355DenseFp4Provider& operator=(const Mi355DenseFp4Provider&) = delete;
+
+  // IOperationProvider
+  [[nodiscard]] er::PrepareOperationResult prepare(
+      const er::OperationPreparationContext& context) override;
+  [[nodiscard]] er::CreateOperationRequestStateResult create_request_state(
+      const er::ProgramRequestContext& request) override;
+  [[nodiscard]] er::PrepareOperationResult prepare_exact_decode(
+      const er::ExactDecodePreparationContext& context) override;
+  [[nodiscard]] er::Status synchronize_exact_decode_batch(
+      const er::IPreparedOperation& operation,
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      const er::ExactDecodeSynchronizationBatch& synchronization) override;
+  [[nodiscard]] er::ExactDecodeExecutionHandle execute_exact_decode(
+      const er::IPreparedOperation& operation,
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      const er::ExactDecodeInvocation& invocation) override;
+
+  // The proposer (run_mtp) is outside this provider's scope; whoever owns it
+  // hands the drafts for the next verify step over here.
+  [[nodiscard]] er::Status set_draft_predictions(
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      std::vector<DraftPrediction> drafts);
+
+  // Random-init weights generated on the device (benchmarks, large tests).
+  [[nodiscard]] er::Status load_synthetic_weights(std::uint64_t seed);
+  // Fill the KV cache of positions [0, tokens) with encoded N(0,1) rows.
+  [[nodiscard]] er::Status prefill_synthetic_kv(std::uint32_t tokens,
+                                                std::uint64_t seed);
+
+  // One target pass over `tokens` at consecutive `first_position`.. rows,
+  // leaving logits [rows, vocabulary] in logits() (run_target, :8529-8635).
+  [[nodiscard]] er::Status run_target(const std::uint32_t* tokens,
+                                      std::uint32_t rows,
+                                      std::uint32_t first_position);
+  // Replays the captured graph of the last run_target shape (same rows and
+  // position); used by the benchmark's timed loop.
+  [[nodiscard]] er::Status capture_target_graph(const std::uint32_t* tokens,
+                                                std::uint32_t rows,
+                                                std::uint32_t first_position);
+  [[nodiscard]] er::Status replay_target_graph();
+  [[nodiscard]] er::Status synchronize();
+
+  [[nodiscard]] const float* logits() const noexcept { return logits_; }
+  [[nodiscard]] const float* hidden() const noexcept { return hidden_; }
+  [[nodiscard]] void* stream() const noexcept { return stream_; }
+  [[nodiscard]] const DenseGeometry& geometry() const noexcept { return g_; }
+  [[nodiscard]] std::map<std::string, std::uint64_t, std::less<>> telemetry()
+      const;
+  [[nodiscard]] er::ServiceContract service_contract() const;
+  [[nodiscard]] std::uint64_t weight_bytes() const noexcept {
+    return weight_bytes_;
+  }
+  [[nodiscard]] std::uint64_t kv_bytes_per_token_layer() const noexcept;
+  [[nodiscard]] std::uint64_t kv_page_bytes() const noexcept {
+    return kv_page_bytes_;
+  }
+  [[nodiscard]] er::Status copy_kv_page(std::uint32_t page_index,
+                                        void* host_output);
+
+ private:
+  struct PreparedOp;
+  void allocate_workspaces();
+  void ensure_pages(std::uint32_t last_position);
+  DeviceFp4Matrix upload_matrix(const er::ImmutableModelTensor& tensor,
+                                bool tiled);
+  float* upload_f32(const er::ImmutableModelTensor& tensor,
+                    std::uint32_t elements);
+  DeviceFp4Matrix synthetic_matrix(std::uint32_t rows, std::uint32_t columns,
+                                   std::uint64_t seed, bool tiled);
+  void enqueue_target(const std::uint32_t* device_tokens, std::uint32_t rows,
+                      std::uint32_t first_position);
+  er::SamplingDistribution distribution_from_logits(
+      std::uint32_t row, const er::ProgramRequestContext& request);
+  void release();
+
+  DenseGeometry g_;
+  mutable std::mutex mutex_;
+  void* stream_{};
+  std::vector<void*> allocations_;
+  std::uint64_t weight_bytes_{};
+
+  DeviceFp4Matrix embedding_{};
+  DeviceFp4Matrix head_{};
+  float* final_norm_{};
+  std::vector<LayerWeights> layers_;
+  std::uint32_t attention_ops_{};
+  std::uint32_t ffn_ops_{};
+  bool embedding_ready_{};
+  bool head_ready_{};
+  std::shared_ptr<const er::IPreparedOperation> exact_;
+
+  // KV cache
+  std::vector<void*> pages_;
+  void** device_page_table_{};
+  std::uint64_t kv_page_bytes_{};
+  std::uint32_t split_tokens_{};
+  std::uint32_t maximum_splits_{};
+
+  // workspaces (device)
+  std::uint32_t max_rows_{};
+  std::uint32_t* tokens_{};
+  float* hidden_{};
+  std::uint16_t* normalized_{};
+  float* query_{};
+  float* key_{};
+  float* value_{};
+  std::uint16_t* attention_{};
+  std::uint16_t* activation_{};
+  float* logits_{};
+  float* partial_maxima_{};
+  float* partial_sums_{};
+  float* partial_outputs_{};
+  void* select_workspace_{};
+  std::size_t select_workspace_bytes_{};
+  std::uint32_t* argmax_tokens_{};
+  float* top_logits_{};
+  std::uint32_t* top_tokens_{};
+
+  void* graph_exec_{};
+
+  // telemetry (dense_fp4_provider.cpp:3109-3257)
+  std::uint64_t exact_calls_{};
+  std::uint64_t accepted_drafts_{};
+  std::vector<std::uint64_t> accepted_depth_calls_;
+  std::uint64_t program_steps_{};
+  std::uint64_t sampling_gpu_calls_{};
+  std::uint64_t sampling_logit_transfer_bytes_{};
+};
+
+// Metadata factory, the analogue of make_sm86_dense_fp4_provider()
+// (dense_fp4_provider.cpp:11398-11400).
+[[nodiscard]] er::WorkerProviderDefinition make_mi355_dense_fp4_provider();
+
+}  // namespace qllm

@@ -1,0 +1,360 @@
+// extern "C" surface of the provider (include/qllm_provider.h).
+#include "qllm_provider.h"
+
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "dense_fp4_provider.hpp"
+
+namespace er = expert::runtime;
+
+struct qllm_provider {
+  std::unique_ptr<qllm::Mi355DenseFp4Provider> provider;
+  std::vector<er::PreparedTensorBinding> staged;
+  std::vector<std::shared_ptr<const er::IPreparedOperation>> operations;
+  std::shared_ptr<const er::IPreparedOperation> exact;
+  std::shared_ptr<er::IOperationProviderRequestState> state;
+  er::ProgramRequestContext request;
+};
+
+namespace {
+
+thread_local char last_error[512] = "";
+
+int32_t fail(int32_t code, const std::string& message) {
+  std::snprintf(last_error, sizeof(last_error), "%s", message.c_str());
+  return code;
+}
+
+int32_t from_status(const er::Status& status) {
+  if (status.ok()) return QLLM_OK;
+  return fail(static_cast<int32_t>(status.code()), std::string(status.message()));
+}
+
+}  // namespace
+
+extern "C" const char* qllm_provider_last_error(void) { return last_error; }
+
+extern "C" qllm_provider* qllm_provider_create(
+    const qllm_dense_geometry* geometry) {
+  if (!geometry) {
+    fail(QLLM_INVALID_ARGUMENT, "geometry is null");
+    return nullptr;
+  }
+  try {
+    qllm::DenseGeometry g;
+    g.hidden = geometry->hidden;
+    g.intermediate = geometry->intermediate;
+    g.layers = geometry->layers;
+    g.query_heads = geometry->query_heads;
+    g.kv_heads = geometry->kv_heads;
+    g.head_dim = geometry->head_dim;
+    g.rotary_dim = geometry->rotary_dim;
+    g.vocabulary = geometry->vocabulary;
+    g.rope_theta = geometry->rope_theta;
+    g.norm_epsilon = geometry->norm_epsilon;
+    g.output_gated = geometry->output_gated != 0;
+    g.qk_norm = geometry->qk_norm != 0;
+    g.zero_centered_norm = geometry->zero_centered_norm != 0;
+    g.scale_scheme = geometry->scale_scheme;
+    g.kv_encoding = geometry->kv_encoding == 1U
+                        ? qllm::KvEncoding::fp16
+                        : qllm::KvEncoding::q4_f16_per_head;
+    g.kv_page_tokens = geometry->kv_page_tokens;
+    g.max_context = geometry->max_context;
+    g.draft_depth = geometry->draft_depth;
+    auto handle = std::make_unique<qllm_provider>();
+    handle->provider = std::make_unique<qllm::Mi355DenseFp4Provider>(g);
+    return handle.release();
+  } catch (const std::exception& error) {
+    fail(QLLM_INTERNAL, error.what());
+    return nullptr;
+  }
+}
+
+extern "C" void qllm_provider_destroy(qllm_provider* provider) {
+  delete provider;
+}
+
+extern "C" uint32_t qllm_provider_capabilities(char* buffer, size_t capacity) {
+  const auto definition = qllm::make_mi355_dense_fp4_provider();
+  size_t used = 0;
+  uint32_t count = 0;
+  for (const auto& capability : definition.capabilities) {
+    const auto bytes = capability.capability.size() + 1U;
+    if (buffer && used + bytes <= capacity) {
+      std::memcpy(buffer + used, capability.capability.c_str(), bytes);
+      used += bytes;
+    }
+    ++count;
+  }
+  return count;
+}
+
+extern "C" int32_t qllm_provider_stage_tensor(
+    qllm_provider* provider, const char* role, const char* encoding,
+    uint32_t quant_abi, uint32_t rows, uint32_t columns, const void* data,
+    size_t data_bytes, const void* scales, size_t scale_bytes) {
+  if (!provider || !role || !encoding || !data || !data_bytes)
+    return fail(QLLM_INVALID_ARGUMENT, "staged tensor is invalid");
+  try {
+    auto blob = std::make_shared<std::vector<std::byte>>(data_bytes + scale_bytes);
+    std::memcpy(blob->data(), data, data_bytes);
+    if (scale_bytes) std::memcpy(blob->data() + data_bytes, scales, scale_bytes);
+    auto tensor = std::make_shared<er::ImmutableModelTensor>();
+    tensor->name = role;
+    tensor->encoding = encoding;
+    tensor->quant_abi = quant_abi;
+    tensor->shape = columns ? std::vector<uint32_t>{rows, columns}
+                            : std::vector<uint32_t>{rows};
+    tensor->data_offset = 0;
+    tensor->data_bytes = data_bytes;
+    tensor->scale_offset = data_bytes;
+    tensor->scale_bytes = scale_bytes;
+    tensor->value.abi = "artifact.dense-record.v1";
+    tensor->value.memory_domain = "host.mmap.readonly";
+    tensor->value.owner = blob;
+    tensor->value.data = blob->data();
+    tensor->value.bytes = blob->size();
+    provider->staged.push_back({role, tensor});
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+extern "C" int32_t qllm_provider_prepare(qllm_provider* provider,
+                                         const char* capability) {
+  if (!provider || !capability)
+    return fail(QLLM_INVALID_ARGUMENT, "prepare arguments are invalid");
+  er::OperationPreparationContext context;
+  context.capability = capability;
+  context.abi = 1U;
+  context.tensors = provider->staged;
+  auto result = provider->provider->prepare(context);
+  provider->staged.clear();
+  if (!result.status.ok()) return from_status(result.status);
+  provider->operations.push_back(result.operation);
+  return QLLM_OK;
+}
+
+extern "C" int32_t qllm_provider_prepare_exact_decode(qllm_provider* provider,
+                                                      const char* capability) {
+  if (!provider || !capability)
+    return fail(QLLM_INVALID_ARGUMENT, "prepare arguments are invalid");
+  er::ExactDecodePreparationContext context;
+  context.capability = capability;
+  context.abi = 2U;
+  context.parameters["draft_depth"] = provider->provider->geometry().draft_depth;
+  context.parameters["source_mtp_layers"] = 1U;
+  auto result = provider->provider->prepare_exact_decode(context);
+  if (!result.status.ok()) return from_status(result.status);
+  provider->exact = result.operation;
+  return QLLM_OK;
+}
+
+extern "C" int32_t qllm_provider_load_synthetic_weights(qllm_provider* provider,
+                                                        uint64_t seed) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->load_synthetic_weights(seed));
+}
+
+extern "C" int32_t qllm_provider_prefill_synthetic_kv(qllm_provider* provider,
+                                                      uint32_t tokens,
+                                                      uint64_t seed) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->prefill_synthetic_kv(tokens, seed));
+}
+
+extern "C" int32_t qllm_provider_begin_request(qllm_provider* provider,
+                                               uint32_t temperature_ppm,
+                                               uint32_t top_p_ppm,
+                                               uint32_t top_k,
+                                               uint32_t min_p_ppm,
+                                               uint64_t seed) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  provider->request = {};
+  provider->request.parameters["sampling_temperature_ppm"] = temperature_ppm;
+  provider->request.parameters["sampling_top_p_ppm"] = top_p_ppm;
+  provider->request.parameters["sampling_top_k"] = top_k;
+  provider->request.parameters["sampling_min_p_ppm"] = min_p_ppm;
+  provider->request.parameters["sampling_seed"] = seed;
+  provider->request.parameters["sampling_presence_penalty_biased_ppm"] =
+      2'000'000U;
+  provider->request.parameters["exact_decode_enabled"] = 1U;
+  auto result = provider->provider->create_request_state(provider->request);
+  if (!result.status.ok()) return from_status(result.status);
+  provider->state = result.state;
+  return QLLM_OK;
+}
+
+extern "C" int32_t qllm_provider_synchronize(qllm_provider* provider,
+                                             uint32_t token,
+                                             uint32_t position) {
+  if (!provider || !provider->exact || !provider->state)
+    return fail(QLLM_INVALID_ARGUMENT, "exact decode is not prepared");
+  const uint32_t tokens[1] = {token};
+  er::ExactDecodeSynchronizationBatch batch{provider->request, tokens, position,
+                                            true};
+  return from_status(provider->provider->synchronize_exact_decode_batch(
+      *provider->exact, provider->state, batch));
+}
+
+extern "C" int32_t qllm_provider_set_drafts(
+    qllm_provider* provider, const uint32_t* draft_tokens, uint32_t draft_count,
+    const uint32_t* distribution_counts, const uint32_t* distribution_tokens,
+    const double* distribution_probabilities) {
+  if (!provider || !provider->state || !draft_tokens || !draft_count)
+    return fail(QLLM_INVALID_ARGUMENT, "draft arguments are invalid");
+  try {
+    std::vector<qllm::DraftPrediction> drafts(draft_count);
+    size_t offset = 0;
+    for (uint32_t index = 0; index < draft_count; ++index) {
+      drafts[index].token = draft_tokens[index];
+      const uint32_t count = distribution_counts ? distribution_counts[index] : 0U;
+      if (count == 0U) {
+        drafts[index].distribution.entries = {{draft_tokens[index], 1.0}};
+      } else {
+        if (!distribution_tokens || !distribution_probabilities)
+          return fail(QLLM_INVALID_ARGUMENT, "draft distribution is missing");
+        drafts[index].distribution.entries.reserve(count);
+        for (uint32_t entry = 0; entry < count; ++entry)
+          drafts[index].distribution.entries.push_back(
+              {distribution_tokens[offset + entry],
+               distribution_probabilities[offset + entry]});
+        offset += count;
+      }
+    }
+    return from_status(provider->provider->set_draft_predictions(
+        provider->state, std::move(drafts)));
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+extern "C" int32_t qllm_provider_verify(qllm_provider* provider,
+                                        uint32_t guaranteed_token,
+                                        uint32_t position,
+                                        uint32_t context_limit,
+                                        uint32_t* emitted,
+                                        uint32_t* emitted_count,
+                                        uint32_t* next_token,
+                                        uint32_t* positions_advanced) {
+  if (!provider || !provider->exact || !provider->state || !emitted ||
+      !emitted_count || !next_token || !positions_advanced)
+    return fail(QLLM_INVALID_ARGUMENT, "verify arguments are invalid");
+  er::ExactDecodeInvocation invocation{provider->request, guaranteed_token,
+                                       position, context_limit};
+  auto handle = provider->provider->execute_exact_decode(
+      *provider->exact, provider->state, invocation);
+  if (!handle.valid())
+    return fail(QLLM_INVALID_ARGUMENT, "exact decode invocation was rejected");
+  auto result = handle.poll();
+  if (!result) return fail(QLLM_INTERNAL, "exact decode did not complete");
+  if (!result->status.ok()) return from_status(result->status);
+  *emitted_count = static_cast<uint32_t>(result->emitted_tokens.size());
+  for (size_t index = 0; index < result->emitted_tokens.size(); ++index)
+    emitted[index] = result->emitted_tokens[index];
+  *next_token = result->next_token;
+  *positions_advanced = result->positions_advanced;
+  return QLLM_OK;
+}
+
+extern "C" int32_t qllm_provider_run_target(qllm_provider* provider,
+                                            const uint32_t* tokens,
+                                            uint32_t rows,
+                                            uint32_t first_position) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->run_target(tokens, rows, first_position));
+}
+
+extern "C" int32_t qllm_provider_capture_target(qllm_provider* provider,
+                                                const uint32_t* tokens,
+                                                uint32_t rows,
+                                                uint32_t first_position) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(
+      provider->provider->capture_target_graph(tokens, rows, first_position));
+}
+
+extern "C" int32_t qllm_provider_replay_target(qllm_provider* provider) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->replay_target_graph());
+}
+
+extern "C" int32_t qllm_provider_synchronize_stream(qllm_provider* provider) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->synchronize());
+}
+
+namespace {
+int32_t copy_rows(qllm_provider* provider, const float* source, size_t count,
+                  float* host_output) {
+  if (!provider || !source || !host_output || !count)
+    return fail(QLLM_INVALID_ARGUMENT, "copy arguments are invalid");
+  auto status = provider->provider->synchronize();
+  if (!status.ok()) return from_status(status);
+  const auto error = hipMemcpy(host_output, source, count * sizeof(float),
+                               hipMemcpyDeviceToHost);
+  if (error != hipSuccess) return fail(QLLM_INTERNAL, hipGetErrorString(error));
+  return QLLM_OK;
+}
+}  // namespace
+
+extern "C" int32_t qllm_provider_copy_logits(qllm_provider* provider,
+                                             uint32_t rows,
+                                             float* host_output) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return copy_rows(provider, provider->provider->logits(),
+                   size_t{rows} * provider->provider->geometry().vocabulary,
+                   host_output);
+}
+
+extern "C" int32_t qllm_provider_copy_hidden(qllm_provider* provider,
+                                             uint32_t rows,
+                                             float* host_output) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return copy_rows(provider, provider->provider->hidden(),
+                   size_t{rows} * provider->provider->geometry().hidden,
+                   host_output);
+}
+
+extern "C" uint64_t qllm_provider_kv_page_bytes(const qllm_provider* provider) {
+  return provider ? provider->provider->kv_page_bytes() : 0U;
+}
+
+extern "C" int32_t qllm_provider_copy_kv_page(qllm_provider* provider,
+                                              uint32_t page_index,
+                                              void* host_output) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->copy_kv_page(page_index, host_output));
+}
+
+extern "C" const float* qllm_provider_logits(const qllm_provider* provider) {
+  return provider ? provider->provider->logits() : nullptr;
+}
+
+extern "C" const float* qllm_provider_hidden(const qllm_provider* provider) {
+  return provider ? provider->provider->hidden() : nullptr;
+}
+
+extern "C" void* qllm_provider_stream(const qllm_provider* provider) {
+  return provider ? provider->provider->stream() : nullptr;
+}
+
+extern "C" uint64_t qllm_provider_weight_bytes(const qllm_provider* provider) {
+  return provider ? provider->provider->weight_bytes() : 0U;
+}
+
+extern "C" uint64_t qllm_provider_telemetry(const qllm_provider* provider,
+                                            const char* name) {
+  if (!provider || !name) return 0U;
+  const auto values = provider->provider->telemetry();
+  const auto found = values.find(name);
+  return found == values.end() ? 0U : found->second;
+}

@@ -1,0 +1,182 @@
+"""CPU statement of one target pass + acceptance for a small dense decoder,
+composed from the oracle's per-op functions in the order of the reference's
+run_target (runtime/tools/dense_fp4_provider.cpp:8529-8635), run_full_attention
+(:6892), run_ffn (:8250-8293) and run_head (:8393-8432).  Test infrastructure."""
+from __future__ import annotations
+
+import numpy as np
+
+import oracle_lib as ol
+import synth
+
+
+class TinyModel:
+    """Random-init dense decoder held as host tensors (row-major FP4)."""
+
+    def __init__(self, rng, hidden, intermediate, layers, query_heads, kv_heads,
+                 head_dim, vocabulary, scheme, output_gated=False, qk_norm=False,
+                 zero_centered=False, rotary_dim=None, rope_theta=1.0e6,
+                 eps=1.0e-6, weight_scale=0.05):
+        self.hidden, self.intermediate, self.layers = hidden, intermediate, layers
+        self.query_heads, self.kv_heads, self.head_dim = query_heads, kv_heads, head_dim
+        self.vocabulary, self.scheme = vocabulary, scheme
+        self.output_gated, self.qk_norm, self.zero_centered = output_gated, qk_norm, zero_centered
+        self.rotary_dim = rotary_dim or head_dim
+        self.rope_theta, self.eps = rope_theta, eps
+        q_rows = query_heads * head_dim * (2 if output_gated else 1)
+
+        def matrix(rows, columns, gain=1.0):
+            # weights ~ gain / sqrt(columns) in RMS, so every block's output is
+            # comparable to the residual stream (a well-conditioned decoder)
+            codes = rng.integers(0, 256, size=(rows, columns // 2), dtype=np.uint8)
+            target = gain / (2.93 * np.sqrt(columns))
+            if scheme == ol.SCALE_F16_BLOCK16:
+                scales = (target * np.exp(0.5 * rng.standard_normal(
+                    (rows, columns // 16)))).astype(np.float16).view(np.uint16)
+            else:
+                base = int(np.round(np.log2(target)))
+                scales = (127 + base + rng.integers(
+                    -1, 2, size=(rows, columns // 32))).astype(np.uint8)
+            return codes, scales
+
+        def norm(n):
+            base = 0.0 if zero_centered else 1.0
+            return (base + 0.1 * rng.standard_normal(n)).astype(np.float32)
+
+        self.embedding = matrix(vocabulary, hidden, gain=np.sqrt(hidden))
+        self.blocks = []
+        for _ in range(layers):
+            block = dict(
+                input_norm=norm(hidden), post_attention_norm=norm(hidden),
+                query=matrix(q_rows, hidden), key=matrix(kv_heads * head_dim, hidden),
+                value=matrix(kv_heads * head_dim, hidden),
+                output=matrix(hidden, query_heads * head_dim),
+                gate=matrix(intermediate, hidden), up=matrix(intermediate, hidden),
+                down=matrix(hidden, intermediate))
+            if qk_norm:
+                block["query_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
+                block["key_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
+            self.blocks.append(block)
+        self.final_norm = norm(hidden)
+        self.head = matrix(vocabulary, hidden)
+
+    def linear(self, m, x_bf16, rows):
+        codes, scales = m
+        return ol.fp4_linear_f64(codes, scales, self.scheme, rows, codes.shape[1] * 2,
+                                 x_bf16)
+
+
+def _record_slices(model, layer, page_tokens, position, kv_head):
+    """Byte ranges (K codes, K scale, V codes, V scale) of one Q4H record."""
+    d, KV = model.head_dim, model.kv_heads
+    records = page_tokens * KV
+    base = layer * ol.q4h_layer_bytes(page_tokens, KV, d)
+    record = kv_head * page_tokens + position % page_tokens
+    key_codes = base + record * (d // 2)
+    key_scale = base + records * (d // 2) + record * 2
+    value_codes = base + records * (d // 2) + records * 2 + record * (d // 2)
+    value_scale = base + 2 * records * (d // 2) + records * 2 + record * 2
+    return [slice(key_codes, key_codes + d // 2), slice(key_scale, key_scale + 2),
+            slice(value_codes, value_codes + d // 2),
+            slice(value_scale, value_scale + 2)]
+
+
+def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
+               observed_pages=None, report=None):
+    """Returns (logits [rows, V], hidden [rows, H]); writes K/V of the rows into
+    kv_pages (list of uint8 arrays, Q4H, all layers per page).
+
+    Q4H encoding is a discontinuous function of K/V: a last-bit difference in
+    a projection can move a value across a rounding boundary and change a
+    4-bit code.  When `observed_pages` (the pages of the implementation under
+    test) is given, every record this pass writes is compared with the
+    observed one - differing bytes are counted in report["record_byte_diffs"]
+    - and the observed record is then adopted, so that the comparison of the
+    downstream values is not dominated by such flips."""
+    m = model
+    rows = len(tokens)
+    d, Q, KV = m.head_dim, m.query_heads, m.kv_heads
+    stride = d * (2 if m.output_gated else 1)
+    codes, scales = m.embedding
+    hidden = ol.fp4_embedding(codes, scales, m.scheme, m.hidden, m.hidden, tokens)
+    for layer, block in enumerate(m.blocks):
+        x = ol.rms_norm_rows(hidden, block["input_norm"], m.eps, m.zero_centered, True)
+        q = m.linear(block["query"], x, Q * stride).reshape(rows, Q, stride)
+        k = m.linear(block["key"], x, KV * d).reshape(rows, KV, d)
+        v = m.linear(block["value"], x, KV * d).reshape(rows, KV, d)
+        for r in range(rows):
+            position = first_position + r
+            for h in range(Q):
+                q[r, h, :d] = ol.head_norm_rope(
+                    q[r, h, :d], block.get("query_norm"), m.rotary_dim, position,
+                    m.eps, m.rope_theta)
+            for h in range(KV):
+                k[r, h] = ol.head_norm_rope(
+                    k[r, h], block.get("key_norm"), m.rotary_dim, position,
+                    m.eps, m.rope_theta)
+                page = kv_pages[position // page_tokens]
+                ol.q4h_store(page, layer, page_tokens, position, h, KV, d,
+                             k[r, h], v[r, h])
+                if observed_pages is not None:
+                    observed = observed_pages[position // page_tokens]
+                    for part in _record_slices(m, layer, page_tokens, position, h):
+                        if report is not None:
+                            report["record_bytes"] = report.get("record_bytes", 0) + (part.stop - part.start)
+                            report["record_byte_diffs"] = report.get("record_byte_diffs", 0) + int((page[part] != observed[part]).sum())
+                        page[part] = observed[part]
+        shape = ol.AttentionShape(rows, Q, KV, d, first_position + 1, page_tokens,
+                                  layer, int(m.output_gated))
+        attention = ol.attention_q4h(shape, q, kv_pages, "f64")
+        attention = ol.bf16_round(attention.reshape(rows, Q * d))
+        hidden = hidden + m.linear(block["output"], attention, m.hidden)
+        x = ol.rms_norm_rows(hidden, block["post_attention_norm"], m.eps,
+                             m.zero_centered, True)
+        gate = m.linear(block["gate"], x, m.intermediate)
+        up = m.linear(block["up"], x, m.intermediate)
+        activation = ol.silu_product(gate, up, True)
+        hidden = hidden + m.linear(block["down"], activation, m.hidden)
+    x = ol.rms_norm_rows(hidden, m.final_norm, m.eps, m.zero_centered, True)
+    logits = m.linear(m.head, x, m.vocabulary)
+    return logits, hidden
+
+
+def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
+                   kv_encoding=0):
+    """Hands the host tensors to the provider operation by operation, the way
+    the common VM calls prepare() in artifact order."""
+    m = model
+    provider = qp.Provider(
+        hidden=m.hidden, intermediate=m.intermediate, layers=m.layers,
+        query_heads=m.query_heads, kv_heads=m.kv_heads, head_dim=m.head_dim,
+        rotary_dim=m.rotary_dim, vocabulary=m.vocabulary, rope_theta=m.rope_theta,
+        norm_epsilon=m.eps, output_gated=int(m.output_gated), qk_norm=int(m.qk_norm),
+        zero_centered_norm=int(m.zero_centered), scale_scheme=m.scheme,
+        kv_encoding=kv_encoding, kv_page_tokens=page_tokens, max_context=max_context,
+        draft_depth=4)
+    abi = 16 if m.scheme == ol.SCALE_F16_BLOCK16 else 3
+    tag = "fp4-f16-block16" if m.scheme == ol.SCALE_F16_BLOCK16 else "fp4-block32"
+    d, Q, KV, H, I, V = m.head_dim, m.query_heads, m.kv_heads, m.hidden, m.intermediate, m.vocabulary
+    provider.stage_fp4("token_embedding", *m.embedding, V, H, abi)
+    provider.prepare(f"embedding.lookup.{tag}.v1")
+    for block in m.blocks:
+        provider.stage_f32("input_norm", block["input_norm"])
+        provider.stage_fp4("query_projection", *block["query"],
+                           Q * d * (2 if m.output_gated else 1), H, abi)
+        provider.stage_fp4("key_projection", *block["key"], KV * d, H, abi)
+        provider.stage_fp4("value_projection", *block["value"], KV * d, H, abi)
+        provider.stage_fp4("output_projection", *block["output"], H, Q * d, abi)
+        if m.qk_norm:
+            provider.stage_f32("query_norm", block["query_norm"])
+            provider.stage_f32("key_norm", block["key_norm"])
+        provider.prepare("block.full-attention.output-gated.v1" if m.output_gated
+                         else "block.full-attention.standard-gqa.v1")
+        provider.stage_f32("post_attention_norm", block["post_attention_norm"])
+        provider.stage_fp4("gate_projection", *block["gate"], I, H, abi)
+        provider.stage_fp4("up_projection", *block["up"], I, H, abi)
+        provider.stage_fp4("down_projection", *block["down"], H, I, abi)
+        provider.prepare(f"ffn.swiglu.dense.{tag}.v1")
+    provider.stage_f32("hidden_norm", m.final_norm)
+    provider.stage_fp4("output_head", *m.head, V, H, abi)
+    provider.prepare(f"head.rmsnorm.token-select.{tag}.v1")
+    provider.prepare_exact_decode(f"decode.mtp.dense-full-attention.{tag}.exact.v2")
+    return provider

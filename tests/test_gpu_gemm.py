@@ -1,0 +1,146 @@
+"""FP4 GEMM parity on the GPU, through the C ABI, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as gu
+import oracle_lib as ol
+import qllm_hip as qh
+import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_F16_BLOCK16, ol.SCALE_UE8M0_BLOCK32])
+@pytest.mark.parametrize("rows,padded,batch", [
+    (64, 256, 5), (100, 320, 5), (67, 96, 3), (33, 64, 1), (1024, 5120, 5),
+    (512, 8192, 5), (256, 17408, 5), (333, 5120, 8), (4096, 1024, 2)])
+def test_gemm_matches_oracle(device, scheme, rows, padded, batch):
+    rng = np.random.default_rng(rows * 31 + padded + batch + scheme)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
+    row_major = gu.gemm(device, codes, scales, scheme, rows, padded, act, tiled=False)
+    gu.assert_close(row_major, want, what="row-major")
+    if padded % 64 == 0:
+        tiled = gu.gemm(device, codes, scales, scheme, rows, padded, act, tiled=True)
+        # the tiled copy moves bytes only: same arithmetic, same bits
+        assert np.array_equal(tiled, row_major)
+
+
+def test_gemm_config1_shape_and_output_kinds(device):
+    """BASELINE config 1: [17408, 5120], M=5, binary16 scale per 16, bf16 out."""
+    rng = np.random.default_rng(1)
+    rows, padded, batch, scheme = 17408, 5120, 5, ol.SCALE_F16_BLOCK16
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
+    got = gu.gemm(device, codes, scales, scheme, rows, padded, act)
+    gu.assert_close(got, want, what="f32 out")
+    got_bf16 = gu.gemm(device, codes, scales, scheme, rows, padded, act,
+                       out_kind=qh.OUT_BF16)
+    assert np.array_equal(got_bf16, ol.bf16_round(got))
+    rounded = gu.gemm(device, codes, scales, scheme, rows, padded, act,
+                      out_kind=qh.OUT_F32_BF16_ROUNDED)
+    assert np.array_equal(rounded, got_bf16)
+    residual = rng.standard_normal((batch, rows)).astype(np.float32)
+    with_residual = gu.gemm(device, codes, scales, scheme, rows, padded, act,
+                            residual=residual)
+    gu.assert_close(with_residual, want + residual, what="residual")
+
+
+def test_gemm_is_linear_in_the_activations(device):
+    """Size-independent property at the lm_head shape: W(a+b) = Wa + Wb when the
+    sum is exactly representable (powers of two)."""
+    rng = np.random.default_rng(2)
+    rows, padded, scheme = 151936, 5120, ol.SCALE_F16_BLOCK16
+    codes = torch.empty((rows, padded // 2), dtype=torch.uint8, device=device)
+    scales = torch.empty((rows, padded // 16), dtype=torch.float16, device=device)
+    qh.call("qllm_fill_random", qh.ptr(codes), codes.numel(), 0, 11, None)
+    qh.call("qllm_fill_random", qh.ptr(scales), scales.numel(), 3, 12, None)
+    matrix, keep = qh.prepack(qh.fp4_matrix(codes, scales, rows, padded, padded, scheme),
+                              device)
+    a = (2.0 ** rng.integers(-2, 3, (2, padded))).astype(np.float32)
+    a[1] *= rng.choice([-1.0, 1.0], padded).astype(np.float32)
+    stacked = np.stack([a[0], a[1], np.zeros(padded, np.float32)])
+    d_act = gu.device_tensor(ol.bf16_bits(stacked), device)
+    out = torch.zeros((3, rows), device=device)
+    qh.call("qllm_fp4_gemm_bf16", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(out), qh.OUT_F32, None, 3, None)
+    torch.cuda.synchronize()
+    host = out.cpu().numpy()
+    assert not host[2].any()                      # zero activations -> zero
+    # spot-check 64 rows against the oracle (rows fetched back from the device)
+    pick = rng.choice(rows, 64, replace=False)
+    sub_codes = codes.cpu().numpy()[pick]
+    sub_scales = scales.view(torch.uint16).cpu().numpy()[pick]
+    want = ol.fp4_linear_f64(sub_codes, sub_scales, scheme, 64, padded, stacked)
+    gu.assert_close(host[:, pick], want, what="lm_head rows")
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_F16_BLOCK16, ol.SCALE_UE8M0_BLOCK32])
+def test_fused_swiglu_matches_oracle(device, scheme):
+    rng = np.random.default_rng(3 + scheme)
+    rows, padded, batch = 1024, 5120, 5
+    gate = synth.fp4_matrix(rng, rows, padded, scheme)
+    up = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(0.02 * rng.standard_normal((batch, padded)).astype(np.float32))
+    g = ol.fp4_linear_f64(*gate, scheme, rows, padded, act)
+    u = ol.fp4_linear_f64(*up, scheme, rows, padded, act)
+    want = ol.silu_product(g, u, True)
+    tensors = [gu.device_tensor(x, device) for x in (*gate, *up)]
+    gate_m, keep_g = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded,
+                                              padded, scheme), device)
+    up_m, keep_u = qh.prepack(qh.fp4_matrix(tensors[2], tensors[3], rows, padded,
+                                            padded, scheme), device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    out = torch.zeros((batch, rows), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_fp4_swiglu_bf16", gate_m, up_m, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(out), batch, None)
+    torch.cuda.synchronize()
+    # one bf16 step of slack on top of the F32 tolerance
+    gu.assert_close(out.float().cpu().numpy(), want, rtol=1e-2, atol=1e-3,
+                    what="swiglu")
+
+
+def test_q8_gemv_matches_reference_integer_statement(device):
+    """Reference arithmetic (ABI 3 weights x Q8 activations), fixture of
+    runtime/tools/dense_fp4_cuda_smoke.cpp:139-216, threshold 2e-4 (:4911)."""
+    rows, columns, padded, batch = 67, 100, 128, 5
+    r = np.arange(rows)[:, None]
+    scales = (124 + (r + np.arange(padded // 32)[None, :]) % 7).astype(np.uint8)
+    pair = np.arange(padded // 2)[None, :]
+    codes = (((r + 3 * pair) % 16) | (((5 * r + pair + 1) % 16) << 4)).astype(np.uint8)
+    x = (np.sin(np.arange(batch * columns, dtype=np.float32) * np.float32(0.071)) *
+         np.float32(0.7)).astype(np.float32).reshape(batch, columns)
+    want_q8, want_scales = ol.quantize_q8_rows(x, padded)
+    d_x = gu.device_tensor(x, device)
+    d_q8 = torch.zeros((batch, padded), dtype=torch.int8, device=device)
+    d_s = torch.zeros(batch, device=device)
+    qh.call("qllm_quantize_q8_batch", qh.ptr(d_x), qh.ptr(d_q8), qh.ptr(d_s), batch,
+            columns, padded, 0, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_q8.cpu().numpy(), want_q8)          # byte-exact
+    assert np.array_equal(d_s.cpu().numpy(), want_scales)
+    want = ol.fp4_linear_block32_q8(codes, scales, rows, padded, want_q8, want_scales)
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    out = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemv_q8_batch",
+            qh.fp4_matrix(d_codes, d_scales, rows, columns, padded, 0), qh.ptr(d_q8),
+            qh.ptr(d_s), qh.ptr(out), batch, 0, None)
+    torch.cuda.synchronize()
+    assert np.abs(out.cpu().numpy() - want).max() < 2e-4
+
+
+def test_invalid_arguments_are_rejected(device):
+    with pytest.raises(qh.QllmError) as error:
+        qh.call("qllm_fp4_gemm_bf16", qh.fp4_matrix(None, None, 4, 4, 32, 0), None, 0,
+                None, 0, None, 5, None)
+    assert error.value.code == 4
+    codes = torch.zeros(64 * 32, dtype=torch.uint8, device=device)
+    scales = torch.zeros(64 * 4, dtype=torch.uint8, device=device)
+    act = torch.zeros((9, 64), dtype=torch.bfloat16, device=device)
+    out = torch.zeros((9, 64), device=device)
+    with pytest.raises(qh.QllmError):   # batch > 8
+        qh.call("qllm_fp4_gemm_bf16", qh.fp4_matrix(codes, scales, 64, 64, 64, 0),
+                qh.ptr(act), act.numel() * 2, qh.ptr(out), 0, None, 9, None)

@@ -1,0 +1,152 @@
+"""Small per-row kernels and token selection on the GPU against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as gu
+import oracle_lib as ol
+import qllm_hip as qh
+import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("scheme", [0, 1])
+def test_embedding_is_exact(device, scheme):
+    rng = np.random.default_rng(scheme)
+    V, H = 300, 256
+    codes, scales = synth.fp4_matrix(rng, V, H, scheme)
+    tokens = np.array([0, 5, 299, 17, 5], dtype=np.uint32)
+    want = ol.fp4_embedding(codes, scales, scheme, H, H, tokens)
+    tensors = [gu.device_tensor(x, device) for x in (codes, scales, tokens)]
+    out = torch.zeros((5, H), device=device)
+    qh.call("qllm_fp4_embedding_batch",
+            qh.fp4_matrix(tensors[0], tensors[1], V, H, H, scheme), qh.ptr(tensors[2]),
+            qh.ptr(out), 5, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("zero_centered", [0, 1])
+def test_rms_norm(device, zero_centered):
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((5, 5120)) * 3).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(5120)).astype(np.float32)
+    d_x, d_w = gu.device_tensor(x, device), gu.device_tensor(w, device)
+    out_f32 = torch.zeros((5, 5120), device=device)
+    out_bf16 = torch.zeros((5, 5120), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_batch", qh.ptr(d_x), qh.ptr(d_w), qh.ptr(out_f32),
+            qh.ptr(out_bf16), 5120, 5, 5120, 1e-6, zero_centered, None)
+    torch.cuda.synchronize()
+    want = ol.rms_norm_rows(x, w, 1e-6, bool(zero_centered))
+    assert np.abs(out_f32.cpu().numpy() - want).max() < 2e-5   # reference: 2e-5
+    assert np.array_equal(out_bf16.float().cpu().numpy(),
+                          ol.bf16_round(out_f32.cpu().numpy()))
+
+
+def test_add_silu_and_bf16_convert(device):
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal(3000).astype(np.float32) * 3
+    b = rng.standard_normal(3000).astype(np.float32)
+    d_a, d_b = gu.device_tensor(a, device), gu.device_tensor(b, device)
+    out = torch.zeros(3000, device=device)
+    for bf16 in (0, 1):
+        qh.call("qllm_silu_product", qh.ptr(d_a), qh.ptr(d_b), qh.ptr(out), 3000, bf16,
+                None)
+        torch.cuda.synchronize()
+        want = ol.silu_product(a, b, bool(bf16))
+        gu.assert_close(out.cpu().numpy(), want, rtol=1e-5 if not bf16 else 8e-3,
+                        atol=1e-6, what="silu")
+    # bf16 mode rounding points of the reference (dense_fp4_cuda_smoke.cpp:4424+)
+    qh.call("qllm_add_in_place", qh.ptr(d_a), qh.ptr(d_b), 3000, 1, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_a.cpu().numpy(), ol.bf16_round(a + b))
+    x = rng.standard_normal((2, 100)).astype(np.float32)
+    d_x = gu.device_tensor(x, device)
+    converted = torch.ones((2, 128), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_convert_f32_to_bf16_batch", qh.ptr(d_x), qh.ptr(converted),
+            converted.numel() * 2, 2, 100, 128, None)
+    torch.cuda.synchronize()
+    host = converted.float().cpu().numpy()
+    assert np.array_equal(host[:, :100], ol.bf16_round(x)) and not host[:, 100:].any()
+
+
+def test_argmax_ties_nan_and_large_vocabulary(device):
+    nan = float("nan")
+    rng = np.random.default_rng(4)
+    V = 151936
+    logits = rng.standard_normal((5, V)).astype(np.float32)
+    logits[0, 77] = logits[0, 140000] = 9.0          # tie -> lower index
+    logits[1, :] = nan
+    logits[1, 5000] = -3.0                           # NaN never wins
+    logits[2, :] = -np.inf                           # all -inf -> index 0
+    logits[3, V - 1] = 12.0
+    d_logits = gu.device_tensor(logits, device)
+    out = torch.zeros(5, dtype=torch.int32, device=device)
+    size = qh.call("qllm_argmax_workspace_bytes", V, 5)
+    workspace = torch.zeros(size, dtype=torch.uint8, device=device)
+    qh.call("qllm_argmax_batch", qh.ptr(d_logits), V, 5, qh.ptr(out), qh.ptr(workspace),
+            size, None)
+    torch.cuda.synchronize()
+    want = [ol.argmax(logits[r]) for r in range(5)]
+    assert out.cpu().numpy().astype(np.uint32).tolist() == want
+    assert want[:4] == [77, 5000, 0, V - 1]
+
+
+def test_topk_known_answers(device):
+    nan = float("nan")
+
+    def run(values, k):
+        d_values = gu.device_tensor(values, device)
+        out_v = torch.zeros(k, device=device)
+        out_i = torch.zeros(k, dtype=torch.int32, device=device)
+        size = qh.call("qllm_topk_workspace_bytes", len(values), k)
+        workspace = torch.zeros(size, dtype=torch.uint8, device=device)
+        qh.call("qllm_topk_logits", qh.ptr(d_values), len(values), k, qh.ptr(out_v),
+                qh.ptr(out_i), qh.ptr(workspace), size, None)
+        torch.cuda.synchronize()
+        return out_v.cpu().numpy(), out_i.cpu().numpy().astype(np.uint32)
+
+    # runtime/tools/dense_fp4_cuda_smoke.cpp:4313-4335
+    values, indices = run(np.array([1.0, 7.0, nan, 7.0, -2.0, 4.5, 4.5, 9.0, 0.0],
+                                   np.float32), 5)
+    assert indices.tolist() == [7, 1, 3, 5, 6]
+    assert values.tolist() == [9.0, 7.0, 7.0, 4.5, 4.5]
+    # :4337-4359
+    v = 248320
+    i = np.arange(v, dtype=np.float32)
+    big = (np.sin(i * np.float32(0.0137)) + np.float32(0.37) * np.cos(i * np.float32(0.0071))
+           ).astype(np.float32)
+    big[19] = big[127] = 7.0
+    big[1021] = nan
+    values, indices = run(big, 20)
+    want_v, want_i = ol.topk(big, 20)
+    assert indices.tolist() == want_i.tolist() and np.array_equal(values, want_v)
+    rng = np.random.default_rng(5)
+    random_logits = rng.standard_normal(151936).astype(np.float32)
+    values, indices = run(random_logits, 64)
+    want_v, want_i = ol.topk(random_logits, 64)
+    assert indices.tolist() == want_i.tolist() and np.array_equal(values, want_v)
+
+
+def test_presence_penalty_known_answer(device):
+    logits = gu.device_tensor(np.array([3.0, 2.0, 1.0, -1.0], np.float32), device)
+    emitted = gu.device_tensor(np.array([0, 1, 1, 0], np.uint8), device)
+    qh.call("qllm_apply_presence_penalty", qh.ptr(logits), qh.ptr(emitted), 4, 1.5, None)
+    torch.cuda.synchronize()
+    assert logits.cpu().numpy().tolist() == [3.0, 0.5, -0.5, -1.0]
+
+
+def test_query_q8_quantisation_is_byte_exact(device):
+    rng = np.random.default_rng(6)
+    rows, Q, d = 5, 24, 256
+    q = rng.standard_normal((rows, Q, 2 * d)).astype(np.float32)
+    want_q8, want_scales = ol.quantize_queries_q8(q, rows, Q, d, 2 * d)
+    d_q = gu.device_tensor(q, device)
+    q8 = torch.zeros((rows, Q, d), dtype=torch.int8, device=device)
+    scales = torch.zeros((rows, Q), device=device)
+    qh.call("qllm_quantize_gqa_queries_q8", qh.ptr(d_q), 2 * d, qh.ptr(q8),
+            qh.ptr(scales), rows, Q, d, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(q8.cpu().numpy(), want_q8)
+    assert np.array_equal(scales.cpu().numpy(), want_scales)
