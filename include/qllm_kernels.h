@@ -195,6 +195,18 @@ int32_t qllm_qkv_rope_cache_paged_q4h_batch(
     uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
     float rope_theta, int32_t bf16_activations, void* stream);
 
+/* The same operation with the positions read on the device when the kernel
+ * runs: device_positions[0] = first cache position, [1] = first rotary
+ * position.  Lets a captured HIP graph be replayed at advancing positions. */
+int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, const uint32_t* device_positions, uint32_t rows,
+    uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, void* stream);
+
 /* The same per-head RMSNorm + rotary without the K/V store, for caches that
  * store K/V separately.  replaces gated_gqa_qkv_rope_fp16_batch
  * (runtime/src/cuda/transformer_kernels.cu:3645-3726). */
@@ -250,6 +262,11 @@ typedef struct qllm_q4h_attention_launch {
   int32_t output_gated;         /* multiply by sigmoid(query[d + i]) */
   uint32_t output_kind;         /* QLLM_OUT_F32 or QLLM_OUT_BF16 */
   void* stream;
+  /* Optional (NULL = unused).  When set, first_context_tokens is read from
+   * device_positions[2] when the kernels run and the launch covers all
+   * maximum_splits, so a captured graph can be replayed as the context
+   * grows.  No counterpart in the reference struct. */
+  const uint32_t* device_positions;
 } qllm_q4h_attention_launch;
 
 /* Split phase + split-K combine.  rows * (query_heads/kv_heads) <= 48,

@@ -127,6 +127,13 @@ int32_t qllm_provider_copy_logits(qllm_provider* provider, uint32_t rows,
 int32_t qllm_provider_copy_hidden(qllm_provider* provider, uint32_t rows,
                                   float* host_output);
 
+/* Average launch duration (microseconds) of one hot kernel, measured with HIP
+ * events on the provider's stream over rounds x layers launches on distinct
+ * per-layer data.  which: "ffn_gate_up", "ffn_down", "attention", "lm_head". */
+int32_t qllm_provider_time_kernel(qllm_provider* provider, const char* which,
+                                  uint32_t rounds, uint32_t context_tokens,
+                                  double* microseconds, uint64_t* launches);
+
 /* Bytes of one KV page (all layers) and a host copy of page `page_index`
  * (zero-filled if the page has not been allocated yet). */
 uint64_t qllm_provider_kv_page_bytes(const qllm_provider* provider);

@@ -97,6 +97,7 @@ struct SplitArgs {
   uint32_t kv_heads;
   uint32_t split_tokens;
   uint32_t maximum_splits;
+  const uint32_t* device_positions;  // optional: [2] = first_context_tokens
 };
 
 // D = head_dim (128 or 256), RT = number of 16-row tiles (rows*group <= 16*RT).
@@ -117,7 +118,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   const uint32_t split = blockIdx.y;
   const uint32_t group = args.query_heads / args.kv_heads;
   const uint32_t matrix_rows = args.rows * group;
-  const uint32_t last_context = args.first_context_tokens + args.rows - 1u;
+  const uint32_t first_context_tokens =
+      args.device_positions ? args.device_positions[2]
+                            : args.first_context_tokens;
+  const uint32_t last_context = first_context_tokens + args.rows - 1u;
   const uint32_t split_begin = split * args.split_tokens;
   const uint32_t split_end = min(split_begin + args.split_tokens, last_context);
   const uint32_t tiles =
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     const uint32_t row = valid ? matrix_row / group : 0u;
     const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
     const size_t record = static_cast<size_t>(row) * args.query_heads + head;
-    row_limit[rt] = args.first_context_tokens + row;
+    row_limit[rt] = first_context_tokens + row;
     float values[KSTEPS][16];
     float maximum = 0.0f;
 #pragma unroll
@@ -255,7 +259,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
     // ---- S = K . Q ------------------------------------------------------------
     float score[RT][4][4];
-    const bool needs_mask = tile_begin + 64u > args.first_context_tokens;
+    const bool needs_mask = tile_begin + 64u > first_context_tokens;
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
       i32x4 key_operand[KSTEPS];
@@ -497,7 +501,9 @@ __global__ void attention_combine_kernel(
     const float* partial_maxima, const float* partial_sums,
     const float* partial_outputs, void* output, uint32_t output_kind,
     uint32_t first_context_tokens, uint32_t maximum_splits,
-    uint32_t split_tokens, uint32_t query_heads, uint32_t head_dim) {
+    uint32_t split_tokens, uint32_t query_heads, uint32_t head_dim,
+    const uint32_t* device_positions) {
+  if (device_positions) first_context_tokens = device_positions[2];
   const uint32_t head = blockIdx.x;
   const uint32_t row = blockIdx.y;
   const uint32_t dimension = threadIdx.x;
@@ -635,8 +641,13 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     const void* const* page_table, uint32_t layer, uint32_t page_tokens,
     uint32_t first_cache_position, uint32_t first_rotary_position,
     uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
-    uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations) {
+    uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations,
+    const uint32_t* device_positions) {
   __shared__ float shared[256];
+  if (device_positions) {
+    first_cache_position = device_positions[0];
+    first_rotary_position = device_positions[1];
+  }
   const uint32_t head = blockIdx.x;
   const uint32_t row = blockIdx.y;
   const uint32_t lane = threadIdx.x;
@@ -726,12 +737,14 @@ int32_t launch_attention_combine(const float* query, uint32_t query_stride,
                                  uint32_t first_context_tokens,
                                  uint32_t maximum_splits, uint32_t split_tokens,
                                  uint32_t rows, uint32_t query_heads,
-                                 uint32_t head_dim, hipStream_t stream) {
+                                 uint32_t head_dim,
+                                 const uint32_t* device_positions,
+                                 hipStream_t stream) {
   const dim3 grid(query_heads, rows);
   attention_combine_kernel<<<grid, head_dim, 0, stream>>>(
       query, query_stride, output_gated, partial_maxima, partial_sums,
       partial_outputs, output, output_kind, first_context_tokens,
-      maximum_splits, split_tokens, query_heads, head_dim);
+      maximum_splits, split_tokens, query_heads, head_dim, device_positions);
   return launched("attention split combine");
 }
 
@@ -779,8 +792,32 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
-      epsilon, rope_theta, bf16_activations != 0);
+      epsilon, rope_theta, bf16_activations != 0, nullptr);
   return launched("Q4H QKV rope cache batch");
+}
+
+extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, const uint32_t* device_positions, uint32_t rows,
+    uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, void* stream) {
+  if (!query || !key || !value || !page_table || !page_tokens ||
+      !device_positions || !rows || !query_heads || !kv_heads ||
+      query_heads < kv_heads || query_heads % kv_heads || !head_dim ||
+      head_dim > 256u || head_dim % 2u || query_stride < head_dim ||
+      !rotary_dim || rotary_dim > head_dim || rotary_dim % 2u ||
+      !(epsilon > 0.0f) || !(rope_theta > 0.0f))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "invalid deferred Q4H QKV rope cache batch");
+  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+      query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
+      full_attention_layer, page_tokens, 0u, 0u, query_heads, kv_heads,
+      head_dim, rotary_dim, epsilon, rope_theta, bf16_activations != 0,
+      device_positions);
+  return launched("deferred Q4H QKV rope cache batch");
 }
 
 extern "C" int32_t qllm_qkv_rope_batch(
@@ -799,7 +836,7 @@ extern "C" int32_t qllm_qkv_rope_batch(
   qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
-      rotary_dim, epsilon, rope_theta, bf16_activations != 0);
+      rotary_dim, epsilon, rope_theta, bf16_activations != 0, nullptr);
   return launched("QKV rope batch");
 }
 
@@ -842,8 +879,12 @@ extern "C" int32_t qllm_attention_paged_q4h(
                 "Q4H paged attention: rows * (query_heads/kv_heads) exceeds "
                 "48 (32 at head_dim 256)");
   const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  // with device-side positions the context is not known here: cover every
+  // split (workgroups past the context write neutral partials)
   const uint32_t splits =
-      (last_context + launch->split_tokens - 1u) / launch->split_tokens;
+      launch->device_positions
+          ? launch->maximum_splits
+          : (last_context + launch->split_tokens - 1u) / launch->split_tokens;
   if (splits > launch->maximum_splits)
     return fail(QLLM_INVALID_ARGUMENT,
                 "Q4H paged attention: context needs more splits than "
@@ -863,6 +904,7 @@ extern "C" int32_t qllm_attention_paged_q4h(
   args.kv_heads = launch->kv_heads;
   args.split_tokens = launch->split_tokens;
   args.maximum_splits = launch->maximum_splits;
+  args.device_positions = launch->device_positions;
   const dim3 grid(launch->kv_heads, splits);
   const hipStream_t stream = as_stream(launch->stream);
   int32_t status = launch->head_dim == 128u
@@ -874,5 +916,5 @@ extern "C" int32_t qllm_attention_paged_q4h(
       launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
       launch->output, launch->output_kind, launch->first_context_tokens,
       launch->maximum_splits, launch->split_tokens, launch->rows,
-      launch->query_heads, launch->head_dim, stream);
+      launch->query_heads, launch->head_dim, launch->device_positions, stream);
 }

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <bit>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 #include <stdexcept>
@@ -148,10 +149,9 @@ Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
 Mi355DenseFp4Provider::~Mi355DenseFp4Provider() { release(); }
 
 void Mi355DenseFp4Provider::release() {
-  if (graph_exec_) {
-    (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
-    graph_exec_ = nullptr;
-  }
+  for (void* graph : graphs_)
+    if (graph) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph));
+  graphs_.clear();
   if (stream_) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
   for (void* pointer : allocations_) (void)hipFree(pointer);
   allocations_.clear();
@@ -185,6 +185,10 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
       std::max<std::size_t>({g_.hidden, g_.intermediate,
                              std::size_t{g_.query_heads} * g_.head_dim});
   tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+  positions_ = static_cast<std::uint32_t*>(device_alloc(4U * 4U));
+  graphs_.assign(max_rows_ + 1U, nullptr);
+  if (const char* eager = std::getenv("QLLM_PROVIDER_EAGER"))
+    use_graphs_ = eager[0] == '0';
   hidden_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
   normalized_ = static_cast<std::uint16_t*>(device_alloc(rows * widest * 2U));
   query_ = static_cast<float*>(device_alloc(rows * query_width * 4U));
@@ -507,7 +511,8 @@ er::Status Mi355DenseFp4Provider::set_draft_predictions(
 
 void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                            std::uint32_t rows,
-                                           std::uint32_t first_position) {
+                                           std::uint32_t first_position,
+                                           bool deferred_positions) {
   void* const stream = stream_;
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
@@ -532,12 +537,20 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                     hidden_bytes, value_, QLLM_OUT_F32, nullptr,
                                     rows, stream));
     if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-      status_check(qllm_qkv_rope_cache_paged_q4h_batch(
-          query_, query_stride, key_, value_, layer.query_norm, layer.key_norm,
-          const_cast<const void* const*>(device_page_table_), index,
-          g_.kv_page_tokens, first_position, first_position, rows,
-          g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
-          g_.norm_epsilon, g_.rope_theta, 0, stream));
+      if (deferred_positions)
+        status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
+            query_, query_stride, key_, value_, layer.query_norm,
+            layer.key_norm, const_cast<const void* const*>(device_page_table_),
+            index, g_.kv_page_tokens, positions_, rows, g_.query_heads,
+            g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
+            g_.rope_theta, 0, stream));
+      else
+        status_check(qllm_qkv_rope_cache_paged_q4h_batch(
+            query_, query_stride, key_, value_, layer.query_norm,
+            layer.key_norm, const_cast<const void* const*>(device_page_table_),
+            index, g_.kv_page_tokens, first_position, first_position, rows,
+            g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
+            g_.norm_epsilon, g_.rope_theta, 0, stream));
       qllm_q4h_attention_launch launch{};
       launch.query = query_;
       launch.page_table = const_cast<const void* const*>(device_page_table_);
@@ -558,6 +571,7 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
       launch.output_gated = g_.output_gated;
       launch.output_kind = QLLM_OUT_BF16;
       launch.stream = stream;
+      launch.device_positions = deferred_positions ? positions_ : nullptr;
       status_check(qllm_attention_paged_q4h(&launch));
     } else {
       status_check(qllm_qkv_rope_batch(
@@ -631,7 +645,56 @@ er::Status Mi355DenseFp4Provider::run_target(const std::uint32_t* tokens,
                              hipMemcpyHostToDevice,
                              static_cast<hipStream_t>(stream_)),
               "upload target tokens");
-    enqueue_target(tokens_, rows, first_position);
+    enqueue_target(tokens_, rows, first_position, false);
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+er::Status Mi355DenseFp4Provider::run_target_graph(const std::uint32_t* tokens,
+                                                   std::uint32_t rows,
+                                                   std::uint32_t first_position) {
+  if (g_.kv_encoding != KvEncoding::q4_f16_per_head)
+    return run_target(tokens, rows, first_position);
+  try {
+    if (!tokens || !rows || rows > max_rows_ ||
+        first_position > g_.max_context - rows)
+      return {er::ErrorCode::invalid_argument, "target rows are invalid"};
+    if (!embedding_ready_ || !head_ready_)
+      return {er::ErrorCode::invalid_argument, "target program is not prepared"};
+    ensure_pages(first_position + rows - 1U);
+    const auto stream = static_cast<hipStream_t>(stream_);
+    const std::uint32_t positions[4] = {first_position, first_position,
+                                        first_position + 1U, rows};
+    hip_check(hipMemcpyAsync(tokens_, tokens, rows * sizeof(std::uint32_t),
+                             hipMemcpyHostToDevice, stream),
+              "upload target tokens");
+    hip_check(hipMemcpyAsync(positions_, positions, sizeof(positions),
+                             hipMemcpyHostToDevice, stream),
+              "upload target positions");
+    if (!graphs_[rows]) {
+      hip_check(hipStreamSynchronize(stream), "drain stream before capture");
+      hipGraph_t graph{};
+      hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal),
+                "begin target capture");
+      try {
+        enqueue_target(tokens_, rows, first_position, true);
+      } catch (...) {
+        (void)hipStreamEndCapture(stream, &graph);
+        if (graph) (void)hipGraphDestroy(graph);
+        throw;
+      }
+      hip_check(hipStreamEndCapture(stream, &graph), "end target capture");
+      hipGraphExec_t exec{};
+      const auto status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+      (void)hipGraphDestroy(graph);
+      hip_check(status, "instantiate target graph");
+      graphs_[rows] = exec;
+    }
+    hip_check(hipGraphLaunch(static_cast<hipGraphExec_t>(graphs_[rows]), stream),
+              "launch target graph");
+    last_graph_rows_ = rows;
     return er::Status::success();
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};
@@ -641,50 +704,101 @@ er::Status Mi355DenseFp4Provider::run_target(const std::uint32_t* tokens,
 er::Status Mi355DenseFp4Provider::capture_target_graph(
     const std::uint32_t* tokens, std::uint32_t rows,
     std::uint32_t first_position) {
+  return run_target_graph(tokens, rows, first_position);
+}
+
+er::Status Mi355DenseFp4Provider::replay_target_graph() {
+  if (!last_graph_rows_ || !graphs_[last_graph_rows_])
+    return {er::ErrorCode::invalid_argument, "no target graph was captured"};
+  const auto status =
+      hipGraphLaunch(static_cast<hipGraphExec_t>(graphs_[last_graph_rows_]),
+                     static_cast<hipStream_t>(stream_));
+  if (status != hipSuccess)
+    return {er::ErrorCode::internal, hipGetErrorString(status)};
+  return er::Status::success();
+}
+
+er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
+                                              std::uint32_t rounds,
+                                              std::uint32_t context_tokens,
+                                              double* microseconds,
+                                              std::uint64_t* launches) {
   try {
-    if (!tokens || !rows || rows > max_rows_ ||
-        first_position > g_.max_context - rows)
-      return {er::ErrorCode::invalid_argument, "target rows are invalid"};
-    ensure_pages(first_position + rows - 1U);
+    std::lock_guard lock(mutex_);
+    if (!microseconds || !launches || !rounds || !head_ready_)
+      return {er::ErrorCode::invalid_argument, "kernel timing request is invalid"};
     const auto stream = static_cast<hipStream_t>(stream_);
-    hip_check(hipMemcpy(tokens_, tokens, rows * sizeof(std::uint32_t),
-                        hipMemcpyHostToDevice),
-              "upload target tokens");
-    if (graph_exec_) {
-      hip_check(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_)),
-                "destroy previous graph");
-      graph_exec_ = nullptr;
+    const std::uint32_t rows = max_rows_;
+    const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
+    const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+    if (which == "attention") {
+      if (!context_tokens || context_tokens + rows > g_.max_context)
+        return {er::ErrorCode::invalid_argument, "timing context is invalid"};
+      ensure_pages(context_tokens + rows - 1U);
     }
-    hipGraph_t graph{};
-    hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal),
-              "begin target capture");
-    try {
-      enqueue_target(tokens_, rows, first_position);
-    } catch (...) {
-      (void)hipStreamEndCapture(stream, &graph);
-      if (graph) (void)hipGraphDestroy(graph);
-      throw;
-    }
-    hip_check(hipStreamEndCapture(stream, &graph), "end target capture");
-    hipGraphExec_t exec{};
-    const auto status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    (void)hipGraphDestroy(graph);
-    hip_check(status, "instantiate target graph");
-    graph_exec_ = exec;
+    const auto launch_one = [&](std::uint32_t index) {
+      const auto& layer = layers_[index % g_.layers];
+      if (which == "ffn_gate_up") {
+        status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
+                                          &layer.up.descriptor, normalized_,
+                                          hidden_bytes, activation_, rows,
+                                          stream_));
+      } else if (which == "ffn_down") {
+        status_check(qllm_fp4_gemm_bf16(
+            &layer.down.descriptor, activation_,
+            std::size_t{rows} * g_.intermediate * 2U, query_, QLLM_OUT_F32,
+            nullptr, rows, stream_));
+      } else if (which == "lm_head") {
+        status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
+                                        hidden_bytes, logits_, QLLM_OUT_F32,
+                                        nullptr, rows, stream_));
+      } else if (which == "attention") {
+        qllm_q4h_attention_launch launch{};
+        launch.query = query_;
+        launch.page_table = const_cast<const void* const*>(device_page_table_);
+        launch.output = attention_;
+        launch.partial_maxima = partial_maxima_;
+        launch.partial_sums = partial_sums_;
+        launch.partial_outputs = partial_outputs_;
+        launch.first_context_tokens = context_tokens + 1U;
+        launch.rows = rows;
+        launch.full_attention_layer = index % g_.layers;
+        launch.page_tokens = g_.kv_page_tokens;
+        launch.query_heads = g_.query_heads;
+        launch.kv_heads = g_.kv_heads;
+        launch.head_dim = g_.head_dim;
+        launch.split_tokens = split_tokens_;
+        launch.maximum_splits = maximum_splits_;
+        launch.query_stride = query_stride;
+        launch.output_gated = g_.output_gated;
+        launch.output_kind = QLLM_OUT_BF16;
+        launch.stream = stream_;
+        status_check(qllm_attention_paged_q4h(&launch));
+      } else {
+        throw std::runtime_error("unknown kernel name: " + which);
+      }
+    };
+    const std::uint32_t per_round = which == "lm_head" ? 1U : g_.layers;
+    for (std::uint32_t index = 0; index < per_round; ++index) launch_one(index);
+    hipEvent_t begin{};
+    hipEvent_t end{};
+    hip_check(hipEventCreate(&begin), "create timing event");
+    hip_check(hipEventCreate(&end), "create timing event");
+    hip_check(hipEventRecord(begin, stream), "record timing event");
+    for (std::uint32_t round = 0; round < rounds; ++round)
+      for (std::uint32_t index = 0; index < per_round; ++index) launch_one(index);
+    hip_check(hipEventRecord(end, stream), "record timing event");
+    hip_check(hipEventSynchronize(end), "wait for timing event");
+    float milliseconds{};
+    hip_check(hipEventElapsedTime(&milliseconds, begin, end), "read timing");
+    (void)hipEventDestroy(begin);
+    (void)hipEventDestroy(end);
+    *launches = std::uint64_t{rounds} * per_round;
+    *microseconds = 1000.0 * milliseconds / static_cast<double>(*launches);
     return er::Status::success();
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};
   }
-}
-
-er::Status Mi355DenseFp4Provider::replay_target_graph() {
-  if (!graph_exec_)
-    return {er::ErrorCode::invalid_argument, "no target graph was captured"};
-  const auto status = hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_),
-                                     static_cast<hipStream_t>(stream_));
-  if (status != hipSuccess)
-    return {er::ErrorCode::internal, hipGetErrorString(status)};
-  return er::Status::success();
 }
 
 er::Status Mi355DenseFp4Provider::synchronize() {
@@ -791,7 +905,10 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       target_tokens.push_back(proposal.token);
     }
     const auto rows = static_cast<std::uint32_t>(target_tokens.size());
-    auto status = run_target(target_tokens.data(), rows, invocation.position);
+    auto status = use_graphs_ ? run_target_graph(target_tokens.data(), rows,
+                                                 invocation.position)
+                              : run_target(target_tokens.data(), rows,
+                                           invocation.position);
     if (!status.ok()) throw std::runtime_error(std::string(status.message()));
 
     std::vector<er::SamplingDistribution> target_distributions;

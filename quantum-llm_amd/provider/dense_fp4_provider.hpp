@@ -116,13 +116,28 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   [[nodiscard]] er::Status run_target(const std::uint32_t* tokens,
                                       std::uint32_t rows,
                                       std::uint32_t first_position);
-  // Replays the captured graph of the last run_target shape (same rows and
-  // position); used by the benchmark's timed loop.
+  // The same pass launched as one HIP graph (captured once per row count;
+  // tokens and positions live in device memory, so the graph is replayed
+  // unchanged as the stream advances).  execute_exact_decode uses this form.
+  [[nodiscard]] er::Status run_target_graph(const std::uint32_t* tokens,
+                                            std::uint32_t rows,
+                                            std::uint32_t first_position);
+  // capture = run_target_graph; replay relaunches the last graph on the same
+  // tokens and positions (benchmark loops).
   [[nodiscard]] er::Status capture_target_graph(const std::uint32_t* tokens,
                                                 std::uint32_t rows,
                                                 std::uint32_t first_position);
   [[nodiscard]] er::Status replay_target_graph();
   [[nodiscard]] er::Status synchronize();
+  // Average duration, in microseconds, of one launch of a hot kernel measured
+  // with HIP events on the provider's stream: the kernel is launched once per
+  // layer (distinct weights / KV each time) for `rounds` passes over the
+  // layers.  which: "ffn_gate_up", "ffn_down", "attention", "lm_head".
+  [[nodiscard]] er::Status time_kernel(const std::string& which,
+                                       std::uint32_t rounds,
+                                       std::uint32_t context_tokens,
+                                       double* microseconds,
+                                       std::uint64_t* launches);
 
   [[nodiscard]] const float* logits() const noexcept { return logits_; }
   [[nodiscard]] const float* hidden() const noexcept { return hidden_; }
@@ -152,7 +167,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   DeviceFp4Matrix synthetic_matrix(std::uint32_t rows, std::uint32_t columns,
                                    std::uint64_t seed, bool tiled);
   void enqueue_target(const std::uint32_t* device_tokens, std::uint32_t rows,
-                      std::uint32_t first_position);
+                      std::uint32_t first_position, bool deferred_positions);
   er::SamplingDistribution distribution_from_logits(
       std::uint32_t row, const er::ProgramRequestContext& request);
   void release();
@@ -200,7 +215,10 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* top_logits_{};
   std::uint32_t* top_tokens_{};
 
-  void* graph_exec_{};
+  std::uint32_t* positions_{};   // device: cache, rotary, first-context
+  std::vector<void*> graphs_;    // hipGraphExec_t per row count
+  std::uint32_t last_graph_rows_{};
+  bool use_graphs_{true};
 
   // telemetry (dense_fp4_provider.cpp:3109-3257)
   std::uint64_t exact_calls_{};

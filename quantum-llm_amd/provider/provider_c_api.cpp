@@ -324,6 +324,16 @@ extern "C" int32_t qllm_provider_copy_hidden(qllm_provider* provider,
                    host_output);
 }
 
+extern "C" int32_t qllm_provider_time_kernel(qllm_provider* provider,
+                                             const char* which, uint32_t rounds,
+                                             uint32_t context_tokens,
+                                             double* microseconds,
+                                             uint64_t* launches) {
+  if (!provider || !which) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->time_kernel(
+      which, rounds, context_tokens, microseconds, launches));
+}
+
 extern "C" uint64_t qllm_provider_kv_page_bytes(const qllm_provider* provider) {
   return provider ? provider->provider->kv_page_bytes() : 0U;
 }

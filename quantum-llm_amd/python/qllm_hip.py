@@ -48,7 +48,7 @@ class Q4hAttentionLaunch(Structure):
                 ("head_dim", c_uint32), ("split_tokens", c_uint32),
                 ("maximum_splits", c_uint32), ("query_stride", c_uint32),
                 ("output_gated", c_int32), ("output_kind", c_uint32),
-                ("stream", c_void_p)]
+                ("stream", c_void_p), ("device_positions", c_void_p)]
 
 
 class F16AttentionLaunch(Structure):
@@ -82,6 +82,7 @@ SIGNATURES = {
     "qllm_silu_product": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_q4h_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_qkv_rope_cache_paged_q4h_batch": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
+    "qllm_qkv_rope_cache_paged_q4h_batch_deferred": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
     "qllm_qkv_rope_batch": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
     "qllm_store_kv_paged_q4h_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_quantize_gqa_queries_q8": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),

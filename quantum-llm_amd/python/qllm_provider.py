@@ -50,6 +50,7 @@ SIGNATURES = {
     "qllm_provider_synchronize_stream": (c_int32, [c_void_p]),
     "qllm_provider_copy_logits": (c_int32, [c_void_p, c_uint32, c_void_p]),
     "qllm_provider_copy_hidden": (c_int32, [c_void_p, c_uint32, c_void_p]),
+    "qllm_provider_time_kernel": (c_int32, [c_void_p, c_char_p, c_uint32, c_uint32, POINTER(c_double), POINTER(c_uint64)]),
     "qllm_provider_kv_page_bytes": (c_uint64, [c_void_p]),
     "qllm_provider_copy_kv_page": (c_int32, [c_void_p, c_uint32, c_void_p]),
     "qllm_provider_logits": (c_void_p, [c_void_p]),
@@ -195,6 +196,15 @@ class Provider:
         _check(self.lib.qllm_provider_copy_hidden(self.handle, rows,
                                                   out.ctypes.data))
         return out
+
+    def time_kernel(self, which, rounds, context_tokens=0):
+        """(average microseconds per launch, launches) from HIP events."""
+        microseconds = c_double(0.0)
+        launches = c_uint64(0)
+        _check(self.lib.qllm_provider_time_kernel(
+            self.handle, which.encode(), rounds, context_tokens,
+            ctypes.byref(microseconds), ctypes.byref(launches)))
+        return microseconds.value, launches.value
 
     def kv_page(self, page_index):
         import numpy as np

@@ -176,3 +176,21 @@ def test_graph_replay_reproduces_the_eager_pass(device):
         provider.replay_target()
         assert np.array_equal(provider.logits(5), eager)
     provider.close()
+
+
+def test_one_graph_follows_advancing_positions(device):
+    """The graph captured at the first position is replayed with new tokens and
+    positions in device memory; it must match eager launches step by step."""
+    rng, model, graphed = make("baseline", 9)
+    _, _, eager = make("baseline", 9)            # same seed -> same model
+    position = 0
+    for step in range(6):
+        tokens = rng.integers(0, model.vocabulary, 5).astype(np.uint32)
+        graphed.capture_target(tokens, position)    # run_target_graph
+        eager.run_target(tokens, position)
+        assert np.array_equal(graphed.logits(5), eager.logits(5)), step
+        for page in range(2):
+            assert np.array_equal(graphed.kv_page(page), eager.kv_page(page))
+        position += int(rng.integers(1, 6))
+    graphed.close()
+    eager.close()
