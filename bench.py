@@ -1,0 +1,240 @@
+#!/usr/bin/env python3
+"""MTP-4 verify-step benchmark on one MI355X.
+
+A "step" is one speculative verify call of the provider (execute_exact_decode):
+target pass over 1 guaranteed + 4 draft rows of a random-init 27B-class dense
+FP4 decoder (64 layers, hidden 5120, 64 Q / 8 KV heads, head_dim 128, SwiGLU
+17408, vocabulary 151936, binary16 scale per 16 weights) with a Q4H KV cache
+prefilled to 32768 tokens, greedy target distributions and accept-longest-
+prefix.  Weights and KV contents are generated on the device before the timed
+region; every step starts with all inputs resident in HBM.
+
+Prints one JSON line: tok/s over the timed steps (emitted tokens / wall time),
+the HBM roofline of the dominant kernel (fused gate/up FP4 GEMM) measured with
+HIP events in this process, and a CPU baseline (the oracle's port of the same
+arithmetic on the host cores, bounded sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+sys.path.insert(0, os.path.join(ROOT, "quantum-llm_amd", "python"))
+
+HBM_PEAK_GBS = 8000.0
+
+MODEL = dict(hidden=5120, intermediate=17408, layers=64, query_heads=64, kv_heads=8,
+             head_dim=128, rotary_dim=128, vocabulary=151936, rope_theta=1.0e6,
+             norm_epsilon=1.0e-6, output_gated=0, qk_norm=0, zero_centered_norm=0,
+             scale_scheme=1, kv_encoding=0, kv_page_tokens=256, draft_depth=4)
+CONTEXT = 32768
+
+
+def fp4_bytes(rows, columns):
+    """codes + binary16 scale per 16 columns."""
+    return rows * columns // 2 + rows * (columns // 16) * 2
+
+
+def cpu_baseline(rows):
+    """Times the oracle (a CPU port of the step's arithmetic: double-precision
+    FP4 linears and Q4H attention, OpenMP over the host cores) on a bounded
+    sample and scales it to one full step."""
+    import numpy as np
+
+    import oracle_lib as ol
+    import synth
+
+    rng = np.random.default_rng(0)
+    H, I, Q, KV, d = (MODEL["hidden"], MODEL["intermediate"], MODEL["query_heads"],
+                      MODEL["kv_heads"], MODEL["head_dim"])
+    shapes = [(Q * d, H), (KV * d, H), (KV * d, H), (H, Q * d), (I, H), (I, H), (H, I)]
+    matrices = []
+    for n, k in shapes:
+        codes = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+        scales = np.exp(0.5 * rng.standard_normal((n, k // 16))).astype(
+            np.float16).view(np.uint16)
+        act = ol.bf16_round(rng.standard_normal((rows, k)).astype(np.float32))
+        matrices.append((codes, scales, n, k, act))
+    keys = rng.standard_normal((CONTEXT + rows - 1, KV, d)).astype(np.float32)
+    values = rng.standard_normal((CONTEXT + rows - 1, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, MODEL["kv_page_tokens"])
+    query = rng.standard_normal((rows, Q, d)).astype(np.float32)
+    shape = ol.AttentionShape(rows, Q, KV, d, CONTEXT, MODEL["kv_page_tokens"], 0, 0)
+    sample_layers = 6
+    begin = time.perf_counter()
+    for _ in range(sample_layers):
+        for codes, scales, n, k, act in matrices:
+            ol.fp4_linear_f64(codes, scales, 1, n, k, act)
+        ol.attention_q4h(shape, query, pages, "f64")
+    layer_seconds = (time.perf_counter() - begin) / sample_layers
+    # lm_head: one eighth of the vocabulary rows, scaled
+    head_rows = MODEL["vocabulary"] // 8
+    codes = rng.integers(0, 256, (head_rows, H // 2), dtype=np.uint8)
+    scales = np.exp(0.5 * rng.standard_normal((head_rows, H // 16))).astype(
+        np.float16).view(np.uint16)
+    act = ol.bf16_round(rng.standard_normal((rows, H)).astype(np.float32))
+    begin = time.perf_counter()
+    ol.fp4_linear_f64(codes, scales, 1, head_rows, H, act)
+    head_seconds = (time.perf_counter() - begin) * 8
+    step_seconds = MODEL["layers"] * layer_seconds + head_seconds
+    return {
+        "value": 1.0 / step_seconds,
+        "unit": "tok/s",
+        "cores": int(ol.oracle().qo_num_threads()),
+        "kind": "port",
+        "sample": (f"{sample_layers} of {MODEL['layers']} layers (seven FP4 linears at "
+                   f"M={rows} + Q4H attention at {CONTEXT} tokens each) and 1/8 of the "
+                   "lm_head rows, scaled to one step emitting 1 token; CPU oracle in "
+                   "double precision, OpenMP"),
+        "seconds_per_step": step_seconds,
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=40)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--layers", type=int, default=MODEL["layers"],
+                        help="for quick experiments only; the reported config is 64")
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    arguments = parser.parse_args()
+    if arguments.gpus != 1:
+        print("bench.py: this build runs the verify step on ONE GPU only "
+              f"(--gpus {arguments.gpus} is not supported; there are no collectives "
+              "on this path)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import qllm_provider as qp
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    rows = MODEL["draft_depth"] + 1
+    steps, warmup = arguments.steps, arguments.warmup
+    geometry = dict(MODEL)
+    geometry["layers"] = arguments.layers
+    # room for every step to advance by up to 5 positions
+    needed = CONTEXT + (steps + warmup + 2) * rows + 8
+    geometry["max_context"] = (needed + 255) // 256 * 256
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(20241125)
+    provider.prefill_synthetic_kv(CONTEXT, 7)
+    tag = "fp4-f16-block16"
+    provider.prepare_exact_decode(f"decode.mtp.dense-full-attention.{tag}.exact.v2")
+    provider.begin_request(temperature_ppm=0)
+
+    rng = np.random.default_rng(1)
+    vocabulary = MODEL["vocabulary"]
+    position = CONTEXT
+    token = int(rng.integers(0, vocabulary))
+    provider.synchronize(token, position)
+
+    def step():
+        nonlocal token, position
+        drafts = rng.integers(0, vocabulary, MODEL["draft_depth"]).astype(np.uint32)
+        provider.set_drafts(drafts)
+        emitted, next_token, advanced = provider.verify(
+            token, position, geometry["max_context"])
+        token, position = next_token, position + advanced
+        return len(emitted)
+
+    for _ in range(warmup):
+        step()
+    provider.synchronize_stream()
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    emitted_tokens = 0
+    for _ in range(steps):
+        emitted_tokens += step()
+    provider.synchronize_stream()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    ms_per_step = 1000.0 * elapsed / steps
+    tokens_per_second = emitted_tokens / elapsed
+
+    # dominant kernel: fused gate/up FP4 GEMM of the SwiGLU block
+    H, I = MODEL["hidden"], MODEL["intermediate"]
+    kernel_us, launches = provider.time_kernel("ffn_gate_up", 4)
+    kernel_bytes = 2 * fp4_bytes(I, H) + rows * H * 2 + rows * I * 2
+    achieved = kernel_bytes / kernel_us / 1e3   # GB/s
+    roofline = {
+        "bound": "hbm",
+        "kernel": "fp4_gemm_mfma_kernel (fused gate/up, [2x17408, 5120], M=5)",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "algorithmic_bytes_per_launch": kernel_bytes,
+        "avg_launch_us": round(kernel_us, 3),
+        "launches_timed": launches,
+    }
+    other_kernels = {}
+    for name, bytes_per_launch in (
+            ("ffn_down", fp4_bytes(H, I) + rows * I * 2 + rows * H * 4),
+            ("lm_head", fp4_bytes(vocabulary, H) + rows * H * 2 + rows * vocabulary * 4),
+            ("attention", CONTEXT * MODEL["kv_heads"] * 2 * (MODEL["head_dim"] // 2 + 2)
+             + 2 * rows * MODEL["query_heads"] * MODEL["head_dim"] * 2)):
+        us, _ = provider.time_kernel(name, 4, CONTEXT)
+        other_kernels[name] = {"avg_launch_us": round(us, 3),
+                               "achieved_GBps": round(bytes_per_launch / us / 1e3, 1),
+                               "frac": round(bytes_per_launch / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    weight_bytes = provider.weight_bytes()
+    layers = geometry["layers"]
+    step_bytes = (layers * (fp4_bytes(MODEL["query_heads"] * 128, H) +
+                            2 * fp4_bytes(MODEL["kv_heads"] * 128, H) +
+                            fp4_bytes(H, MODEL["query_heads"] * 128) +
+                            2 * fp4_bytes(I, H) + fp4_bytes(H, I) +
+                            CONTEXT * MODEL["kv_heads"] * 2 * 66) +
+                  fp4_bytes(vocabulary, H))
+    result = {
+        "metric": "MTP-4 decode tok/s at 32K ctx (verify step)",
+        "value": round(tokens_per_second, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp4 weights x bf16 activations, f32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": ("full MTP-4 verify step, 27B-class dense FP4 decoder, "
+                         f"{layers} layers, hidden 5120, 64Q/8KV heads, head_dim 128, "
+                         "FFN 17408, vocab 151936, Q4H KV prefilled to 32768 tokens, "
+                         "greedy acceptance, 5 rows (1 guaranteed + 4 random drafts)"),
+            "context_tokens": CONTEXT,
+            "rows": rows,
+            "emitted_tokens": emitted_tokens,
+            "accepted_drafts": int(provider.telemetry("provider_accepted_drafts")),
+            "weight_bytes": int(weight_bytes),
+            "algorithmic_bytes_per_step": int(step_bytes),
+            "step_hbm_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "step_roofline_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 /
+                                        HBM_PEAK_GBS, 4),
+            "reference_published_tok_s_rtx3090": 54.54,
+            "projected_tok_s_at_reference_acceptance_2.6667": round(
+                2.6667 * 1000.0 / ms_per_step, 1),
+        },
+        "roofline": roofline,
+        "kernels": other_kernels,
+    }
+    provider.close()
+    if not arguments.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(rows)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
