@@ -256,8 +256,12 @@ typedef struct qllm_q4h_attention_launch {
   uint32_t query_heads;
   uint32_t kv_heads;
   uint32_t head_dim;
-  uint32_t split_tokens;
-  uint32_t maximum_splits;
+  uint32_t split_tokens;        /* tokens per context split, a multiple of 64;
+                                   0 = balanced: the context's 64-token tiles
+                                   are dealt evenly over maximum_splits
+                                   workgroups, whatever the context length
+                                   (no counterpart in the reference) */
+  uint32_t maximum_splits;      /* <= 2048 */
   uint32_t query_stride;        /* floats between heads in `query` */
   int32_t output_gated;         /* multiply by sigmoid(query[d + i]) */
   uint32_t output_kind;         /* QLLM_OUT_F32 or QLLM_OUT_BF16 */
@@ -270,7 +274,8 @@ typedef struct qllm_q4h_attention_launch {
 } qllm_q4h_attention_launch;
 
 /* Split phase + split-K combine.  rows * (query_heads/kv_heads) <= 48,
- * head_dim in {128, 256}, page_tokens % 64 == 0, split_tokens % 64 == 0. */
+ * head_dim in {128, 256}, page_tokens % 64 == 0, split_tokens % 64 == 0.
+ * The pages must hold every 64-token tile that overlaps the context. */
 int32_t qllm_attention_paged_q4h(const qllm_q4h_attention_launch* launch);
 
 /* ---- attention: exact F16 paged cache ---------------------------------------- */

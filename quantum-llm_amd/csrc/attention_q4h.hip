@@ -25,6 +25,8 @@
 // merges the splits.  Maxima are kept in the log2 domain.
 #include "common.hpp"
 
+#include <utility>
+
 namespace qllm {
 namespace {
 
@@ -100,18 +102,146 @@ struct SplitArgs {
   const uint32_t* device_positions;  // optional: [2] = first_context_tokens
 };
 
+
+
+
+// Page table entry at a wave-uniform index, fetched with a scalar load (the
+// table is never written while attention kernels run), so everything derived
+// from the page address stays in scalar registers.
+__device__ __forceinline__ const void* uniform_page(
+    const void* const* page_table, uint32_t index) {
+  typedef const void* __attribute__((address_space(4))) const* constant_table;
+  return ((constant_table)page_table)[index];
+}
+
+// Direct global -> LDS loads (no VGPRs): lane l of the wave fetches 16 (4)
+// bytes at base + offset[l] and they land at lds + 16*l (4*l).  `base` and
+// `lds` are wave-uniform.  Written as assembly so that the address stays in
+// the scalar-base + 32-bit-lane-offset form (one VGPR for all loads of a tile)
+// and so that the compiler, which would otherwise wait for every outstanding
+// load before any later LDS access, leaves the waiting to this kernel.
+__device__ __forceinline__ void copy16_to_lds(const uint8_t* base,
+                                              uint32_t lane_offset,
+                                              uint32_t lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :: "v"(lane_offset), "s"(base), "s"(lds) : "memory", "m0");
+}
+__device__ __forceinline__ void copy4_to_lds(const uint8_t* base,
+                                             uint32_t lane_offset,
+                                             uint32_t lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %0, %1"
+      :: "v"(lane_offset), "s"(base), "s"(lds) : "memory", "m0");
+}
+
+// LDS reads of staged tiles.  They are written as inline assembly on purpose:
+// the compiler then does not know that they touch memory a direct-to-LDS load
+// may still be filling, so it inserts no blanket "wait for every outstanding
+// load" in front of them, and the kernel places its own, exact waits
+// (vmem loads complete in issue order).  The values are not valid until
+// lds_wait() has been given them.
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+template <int OFFSET>
+__device__ __forceinline__ u32x4 lds_read16(uint32_t address) {
+  u32x4 result;
+  asm volatile("ds_read_b128 %0, %1 offset:%2"
+               : "=v"(result) : "v"(address), "n"(OFFSET));
+  return result;
+}
+template <int OFFSET>
+__device__ __forceinline__ u32x2 lds_read8(uint32_t address) {
+  u32x2 result;
+  asm volatile("ds_read_b64 %0, %1 offset:%2"
+               : "=v"(result) : "v"(address), "n"(OFFSET));
+  return result;
+}
+// 16x16 transpose of 4-bit elements across each group of 16 lanes
+template <int OFFSET>
+__device__ __forceinline__ u32x2 lds_read8_transposed4(uint32_t address) {
+  u32x2 result;
+  asm volatile("ds_read_b64_tr_b4 %0, %1 offset:%2"
+               : "=v"(result) : "v"(address), "n"(OFFSET));
+  return result;
+}
+// waits for the LDS reads above and ties the values to the wait
+template <int N, typename T>
+__device__ __forceinline__ void lds_wait(T (&values)[N]) {
+  static_assert(N == 4 || N == 8 || N == 16, "unsupported operand count");
+  if constexpr (N == 4)
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(values[0]), "+v"(values[1]), "+v"(values[2]),
+                   "+v"(values[3]) :: "memory");
+  else if constexpr (N == 8)
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(values[0]), "+v"(values[1]), "+v"(values[2]),
+                   "+v"(values[3]), "+v"(values[4]), "+v"(values[5]),
+                   "+v"(values[6]), "+v"(values[7]) :: "memory");
+  else
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(values[0]), "+v"(values[1]), "+v"(values[2]),
+                   "+v"(values[3]), "+v"(values[4]), "+v"(values[5]),
+                   "+v"(values[6]), "+v"(values[7]), "+v"(values[8]),
+                   "+v"(values[9]), "+v"(values[10]), "+v"(values[11]),
+                   "+v"(values[12]), "+v"(values[13]), "+v"(values[14]),
+                   "+v"(values[15]) :: "memory");
+}
+// at most COUNT vmem loads (direct-to-LDS loads included) still in flight
+template <int COUNT>
+__device__ __forceinline__ void vmem_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(COUNT) : "memory");
+}
+// Lane index recomputed where it is needed (two instructions) instead of
+// being kept in a register across the tile loop.
+__device__ __forceinline__ uint32_t fresh_lane_index() {
+  uint32_t lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0"
+               : "=v"(lane));
+  return lane;
+}
+__device__ __forceinline__ uint32_t lds_address(const void* pointer) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) const void*)pointer));
+}
+
 // D = head_dim (128 or 256), RT = number of 16-row tiles (rows*group <= 16*RT).
+//
+// Each wave owns a contiguous run of 64-token tiles.  A tile's K codes, V
+// codes and scales travel global -> LDS with direct loads into a wave-private
+// staging area [K codes + scales | V codes]; each half is refilled with the
+// next tile as soon as the current tile has been read out of it, so the
+// loads fly while the matrix cores and the softmax work on registers.
 template <int D, int RT>
 __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     const SplitArgs args) {
   constexpr int KSTEPS = D / 64;      // int8 MFMA k-steps over head_dim
   constexpr int DT = D / 16;          // 16-wide tiles of head_dim
-  constexpr int VROW = D / 2 + 16;    // padded LDS row of V codes (bytes)
-  constexpr int STATE = 16 * RT * (D + 2);  // floats per merged wave state
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
+  constexpr int ROW = D / 2;          // bytes of codes per token
+  constexpr int CODES = 64 * ROW;     // bytes of K (or V) codes per tile
+  // staging area of a wave: K codes | K scales | V codes | V scales
+  constexpr int STAGE = 2 * CODES + 512;
+  constexpr int STATE = 16 * RT * (D + 2);   // floats per merged wave state
+  constexpr int PASSES = ROW / 16;    // direct loads per code plane and tile
+  constexpr int KS_LOADS = PASSES + 1;       // K codes + K scales
+  constexpr int V_LOADS = PASSES + 1;        // V codes + V scales
+  // merge slots that fit into the staging memory once the tiles are done
+  constexpr int SLOTS =
+      kSplitWaves * STAGE >= 4 * STATE * 4 ? 4 : 2;
+  static_assert(kSplitWaves * STAGE >= SLOTS * STATE * 4, "merge does not fit");
+  __shared__ __attribute__((aligned(16))) uint8_t stage[kSplitWaves * STAGE];
+  // query operands in MFMA order, then per matrix row its scale and the number
+  // of tokens it may attend
+  __shared__ __attribute__((aligned(16)))
+  uint8_t exchange[RT * KSTEPS * 2 * 1024 + 2 * RT * 64];
 
   const uint32_t lane = threadIdx.x & 63u;
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t col = lane & 15u;   // query row inside a row tile / token / d
   const uint32_t quad = lane >> 4;   // 0..3
   const uint32_t kv_head = blockIdx.x;
@@ -122,30 +252,105 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       args.device_positions ? args.device_positions[2]
                             : args.first_context_tokens;
   const uint32_t last_context = first_context_tokens + args.rows - 1u;
-  const uint32_t split_begin = split * args.split_tokens;
-  const uint32_t split_end = min(split_begin + args.split_tokens, last_context);
-  const uint32_t tiles =
-      split_end > split_begin ? (split_end - split_begin + 63u) / 64u : 0u;
+  const uint32_t context_tiles = (last_context + 63u) / 64u;
 
-  uint8_t* v_stage = lds_raw + wave * (64 * VROW);
+  // tiles [tile_first, tile_last) of this wave
+  uint32_t tile_first, tile_last;
+  if (args.split_tokens == 0u) {
+    // balanced: the context's tiles are dealt evenly over every wave of the
+    // grid row, whatever the context length
+    const uint32_t slots = gridDim.y * kSplitWaves;
+    const uint32_t slot = split * kSplitWaves + wave;
+    tile_first = static_cast<uint32_t>(
+        static_cast<uint64_t>(slot) * context_tiles / slots);
+    tile_last = static_cast<uint32_t>(
+        static_cast<uint64_t>(slot + 1u) * context_tiles / slots);
+  } else {
+    const uint32_t split_tiles = args.split_tokens / 64u;
+    const uint32_t begin = min(split * split_tiles, context_tiles);
+    const uint32_t count = min(begin + split_tiles, context_tiles) - begin;
+    tile_first = begin + wave * count / kSplitWaves;
+    tile_last = begin + (wave + 1u) * count / kSplitWaves;
+  }
 
-  // ---- query operands (B side of S = K.Q), built once ------------------------
+  uint8_t* stage_k = stage + wave * STAGE;
+  const uint32_t stage_k_lds =
+      __builtin_amdgcn_readfirstlane(lds_address(stage_k));
+  const uint32_t stage_s_lds = stage_k_lds + CODES;
+  const uint32_t stage_v_lds = stage_s_lds + 256;
+  const uint32_t stage_vs_lds = stage_v_lds + CODES;
+  float* exchange_scale =
+      reinterpret_cast<float*>(exchange + RT * KSTEPS * 2 * 1024);
+  uint32_t* exchange_limit =
+      reinterpret_cast<uint32_t*>(exchange + RT * KSTEPS * 2 * 1024 + RT * 64);
+
+  constexpr uint32_t kParts = ROW / 16;        // 16-byte pieces per token
+  constexpr uint32_t kPassRows = 64 / kParts;  // LDS rows per pass
+  // V scales sit one V code plane + one K scale plane past the K scales
+  const uint32_t value_scale_distance =
+      args.page_tokens * args.kv_heads * (ROW + 2u);
+
+  // KS_LOADS direct loads: K codes and K scales of a tile.  Pass `pass` covers
+  // the 1 KiB at pass*1024 of the tile's K rows; lanes 0..31 then fetch the
+  // scales of tokens 2l, 2l+1 (lanes 32..63 repeat them).
+  auto stage_keys = [&](uint32_t tile) {
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t tile_begin = tile * 64u;
+    const void* page = uniform_page(args.page_table, tile_begin / args.page_tokens);
+    const Q4hPlanes planes =
+        q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
+    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
+                           tile_begin % args.page_tokens;
+    const uint8_t* key_rows = planes.key_codes + record0 * ROW;  // uniform
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass)
+      copy16_to_lds(key_rows + pass * 1024, lane_now * 16u,
+                    stage_k_lds + pass * 1024);
+    copy4_to_lds(planes.key_scales + record0 * 2u, 4u * (lane_now & 31u),
+                 stage_s_lds);
+  };
+  // V_LOADS direct loads: V codes and V scales of a tile.  V row R holds token
+  // 16*((R/4)%4) + 4*(R/16) + R%4, so the 16 tokens a lane group reads back
+  // transposed sit in 16 consecutive rows; the lane's share of that map is
+  // separable from the pass's share.
+  auto stage_values = [&](uint32_t tile) {
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t lane_row = lane_now / kParts;  // row inside a pass
+    const uint32_t value_lane_offset =
+        (16u * ((lane_row >> 2) & 3u) + 4u * (lane_row >> 4) + (lane_row & 3u)) *
+            ROW + (lane_now % kParts) * 16u;
+    const uint32_t tile_begin = tile * 64u;
+    const void* page = uniform_page(args.page_table, tile_begin / args.page_tokens);
+    const Q4hPlanes planes =
+        q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
+    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
+                           tile_begin % args.page_tokens;
+    const uint8_t* value_rows = planes.value_codes + record0 * ROW;  // uniform
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const uint32_t first_row = pass * kPassRows;
+      const uint32_t pass_token = 16u * ((first_row >> 2) & 3u) +
+                                  4u * (first_row >> 4) + (first_row & 3u);
+      copy16_to_lds(value_rows + pass_token * ROW, value_lane_offset,
+                    stage_v_lds + pass * 1024);
+    }
+    copy4_to_lds(planes.key_scales + record0 * 2u + value_scale_distance,
+                 4u * (lane_now & 31u), stage_vs_lds);
+  };
+
+  // ---- query operands (B side of S = K.Q), built once per workgroup ---------
   // The F32 query row is quantised here to 15 bits and split into two int8
   // planes, q = scale * (128*hi + lo) with hi in [-127,127], lo in [-64,63],
   // so the integer scores carry the query to ~3e-5 relative instead of the
-  // 4e-3 of a single Q8 plane.
-  i32x4 q_high[RT][KSTEPS];
-  i32x4 q_low[RT][KSTEPS];
-  float q_scale[RT];
-  uint32_t row_limit[RT];  // tokens visible to this lane's query row
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
+  // 4e-3 of a single Q8 plane.  Wave rt builds row tile rt and publishes it in
+  // MFMA operand order.
+  if (wave < static_cast<uint32_t>(RT)) {
+    const uint32_t rt = wave;
     const uint32_t matrix_row = 16u * rt + col;
     const bool valid = matrix_row < matrix_rows;
     const uint32_t row = valid ? matrix_row / group : 0u;
     const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
     const size_t record = static_cast<size_t>(row) * args.query_heads + head;
-    row_limit[rt] = first_context_tokens + row;
     float values[KSTEPS][16];
     float maximum = 0.0f;
 #pragma unroll
@@ -165,10 +370,17 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
                                        fmaxf(fabsf(loaded.z), fabsf(loaded.w))));
       }
     }
+    if (tile_first < tile_last) {
+      stage_keys(tile_first);
+      stage_values(tile_first);
+    }
     maximum = quad_row_max(maximum);
     const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
     const float inverse = 1.0f / scale;
-    q_scale[rt] = valid ? scale : 0.0f;
+    if (quad == 0u) {
+      exchange_scale[16 * rt + col] = scale;
+      exchange_limit[16 * rt + col] = first_context_tokens + row;
+    }
 #pragma unroll
     for (int h = 0; h < KSTEPS; ++h) {
       uint32_t high_bytes[16], low_bytes[16];
@@ -184,6 +396,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       // byte order inside each 8-element half: even d first, then odd d,
       // matching the order in which the key nibbles are widened
       const int order[16] = {0, 2, 4, 6, 1, 3, 5, 7, 8, 10, 12, 14, 9, 11, 13, 15};
+      i32x4 high_operand, low_operand;
 #pragma unroll
       for (int word = 0; word < 4; ++word) {
         uint32_t high_word = 0u, low_word = 0u;
@@ -192,17 +405,43 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
           high_word |= high_bytes[order[4 * word + byte]] << (8 * byte);
           low_word |= low_bytes[order[4 * word + byte]] << (8 * byte);
         }
-        q_high[rt][h][word] = static_cast<int>(high_word);
-        q_low[rt][h][word] = static_cast<int>(low_word);
+        high_operand[word] = static_cast<int>(high_word);
+        low_operand[word] = static_cast<int>(low_word);
       }
+      *reinterpret_cast<i32x4*>(exchange + ((rt * KSTEPS + h) * 2 + 0) * 1024 +
+                                lane * 16u) = high_operand;
+      *reinterpret_cast<i32x4*>(exchange + ((rt * KSTEPS + h) * 2 + 1) * 1024 +
+                                lane * 16u) = low_operand;
     }
+  } else if (tile_first < tile_last) {
+    stage_keys(tile_first);
+    stage_values(tile_first);
   }
-  // score = int_dot/16 * q_scale * k_scale / sqrt(D), in log2 units
+  __syncthreads();
+
+  // The operands stay in LDS and are re-read for every 16-token sub-tile, and
+  // so are the per-row scale (> 0 also for rows past the batch) and token
+  // limit: holding them next to the output accumulators would push the kernel
+  // into scratch memory.
+  const uint8_t* q_operands = exchange + lane * 16u;
+  // Scores are kept as t = int_dot * k_scale * unit; the true score in log2
+  // units is t * q_scale (q_scale is constant per query row, so maxima can be
+  // taken over t).
   const float score_unit =
       1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D)));
 
+  // per-lane LDS addresses of the staged tile
+  // K: lane (token = col, quad) takes 16 bytes of each sub-tile's K row
+  const uint32_t key_address = stage_k_lds + col * ROW + 16u * quad;
+  // scales of tokens 16*st + 4*quad + i (i = 0..3)
+  const uint32_t scale_address = stage_s_lds + 8u * quad;
+  const uint32_t value_scale_address = stage_vs_lds + 8u * quad;
+  // V: lane (col, quad) supplies LDS row 16*quad + col, i.e. token
+  // 16*(col/4) + 4*quad + col%4 of the tile
+  const uint32_t value_address = stage_v_lds + (16u * quad + col) * ROW;
+
   // ---- running state ---------------------------------------------------------
-  float running_max[RT];
+  float running_max[RT];   // in t units
   float running_sum[RT];
   f32x4 out[DT][RT];
 #pragma unroll
@@ -215,58 +454,40 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
   }
 
-  for (uint32_t tile = wave; tile < tiles; tile += kSplitWaves) {
-    const uint32_t tile_begin = split_begin + tile * 64u;
-    const void* page = args.page_table[tile_begin / args.page_tokens];
-    const Q4hPlanes planes = q4h_planes(page, args.layer, args.page_tokens,
-                                        args.kv_heads, D);
-    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
-                           tile_begin % args.page_tokens;
+  // Loads in flight at the top of an iteration, oldest first: this tile's
+  // K+scales, this tile's V.
+  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+    const uint32_t tile_begin = tile * 64u;
+    const bool needs_mask = tile_begin + 64u > first_context_tokens;
+    const bool has_next = tile + 1u < tile_last;
 
-    // K codes: sub-tile st (16 tokens), lane (token=col, quad) reads 16 bytes
-    uint4 key_raw[4][D / 128];
-#pragma unroll
-    for (int st = 0; st < 4; ++st)
-#pragma unroll
-      for (int c = 0; c < D / 128; ++c)
-        key_raw[st][c] = *reinterpret_cast<const uint4*>(
-            planes.key_codes + (record0 + 16u * st + col) * (D / 2) + 64u * c +
-            16u * quad);
-    // scales of tokens 16t + 4*quad + i (i = 0..3), t = 0..3
-    uint2 key_scale_raw[4];
-    uint2 value_scale_raw[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      key_scale_raw[t] = *reinterpret_cast<const uint2*>(
-          planes.key_scales + (record0 + 16u * t + 4u * quad) * 2u);
-      value_scale_raw[t] = *reinterpret_cast<const uint2*>(
-          planes.value_scales + (record0 + 16u * t + 4u * quad) * 2u);
-    }
-    // V codes -> LDS (token-major rows, padded), 16 tokens per pass
-#pragma unroll
-    for (int pass = 0; pass < 4 * (D / 128); ++pass) {
-      const uint32_t piece = pass * 64u + lane;          // 16-byte pieces
-      const uint32_t token = piece / (D / 32);           // D/32 pieces / token
-      const uint32_t part = piece % (D / 32);
-      const uint4 value = *reinterpret_cast<const uint4*>(
-          planes.value_codes + (record0 + token) * (D / 2) + part * 16u);
-      // LDS row of token T = 16*((T/4)%4) + 4*(T/16) + T%4, so the 16 tokens a
-      // lane group reads back transposed sit in 16 consecutive padded rows
-      const uint32_t stage_row =
-          16u * ((token >> 2) & 3u) + 4u * (token >> 4) + (token & 3u);
-      *reinterpret_cast<uint4*>(v_stage + stage_row * VROW + part * 16u) = value;
-    }
+    // ---- K codes and scales out of LDS ----------------------------------------
+    vmem_wait<V_LOADS>();
+    u32x4 key_raw[4 * (D / 128)];
+    u32x2 scale_raw[4];  // K scales of sub-tile st
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+      ((key_raw[I] = lds_read16<(I / (D / 128)) * 16 * ROW + (I % (D / 128)) * 64>(
+            key_address)), ...);
+    }(std::make_integer_sequence<int, 4 * (D / 128)>{});
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+      ((scale_raw[I] = lds_read8<I * 32>(scale_address)), ...);
+    }(std::make_integer_sequence<int, 4>{});
+    lds_wait(key_raw);
+    lds_wait(scale_raw);
+    // that half of the staging area is free: fetch the next tile's K
+    if (has_next) stage_keys(tile + 1u);
 
     // ---- S = K . Q ------------------------------------------------------------
     float score[RT][4][4];
-    const bool needs_mask = tile_begin + 64u > first_context_tokens;
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
+      // keeps the compiler from merging the query operand reads of the four
+      // sub-tiles into registers that live across the whole tile
+      asm volatile("" ::: "memory");
       i32x4 key_operand[KSTEPS];
 #pragma unroll
       for (int c = 0; c < D / 128; ++c) {
-        const uint32_t x[4] = {key_raw[st][c].x, key_raw[st][c].y,
-                               key_raw[st][c].z, key_raw[st][c].w};
+        const u32x4 x = key_raw[st * (D / 128) + c];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
           i32x4 operand;
@@ -278,35 +499,74 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         }
       }
       const float k_scale[4] = {
-          f16_bits_to_f32(key_scale_raw[st].x & 0xffffu) * score_unit,
-          f16_bits_to_f32(key_scale_raw[st].x >> 16) * score_unit,
-          f16_bits_to_f32(key_scale_raw[st].y & 0xffffu) * score_unit,
-          f16_bits_to_f32(key_scale_raw[st].y >> 16) * score_unit};
+          f16_bits_to_f32(scale_raw[st][0] & 0xffffu) * score_unit,
+          f16_bits_to_f32(scale_raw[st][0] >> 16) * score_unit,
+          f16_bits_to_f32(scale_raw[st][1] & 0xffffu) * score_unit,
+          f16_bits_to_f32(scale_raw[st][1] >> 16) * score_unit};
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         i32x4 dot_high = {0, 0, 0, 0};
         i32x4 dot_low = {0, 0, 0, 0};
 #pragma unroll
         for (int h = 0; h < KSTEPS; ++h) {
+          const i32x4 q_high = *reinterpret_cast<const i32x4*>(
+              q_operands + ((rt * KSTEPS + h) * 2 + 0) * 1024);
+          const i32x4 q_low = *reinterpret_cast<const i32x4*>(
+              q_operands + ((rt * KSTEPS + h) * 2 + 1) * 1024);
           dot_high = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-              key_operand[h], q_high[rt][h], dot_high, 0, 0, 0);
+              key_operand[h], q_high, dot_high, 0, 0, 0);
           dot_low = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-              key_operand[h], q_low[rt][h], dot_low, 0, 0, 0);
+              key_operand[h], q_low, dot_low, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int dot = (dot_high[i] << 7) + dot_low[i];
-          float value = static_cast<float>(dot) * k_scale[i] * q_scale[rt];
+          float value = static_cast<float>(dot) * k_scale[i];
           if (needs_mask) {
             const uint32_t token = tile_begin + 16u * st + 4u * quad + i;
-            if (token >= row_limit[rt]) value = -INFINITY;
+            if (token >= exchange_limit[16 * rt + col]) value = -INFINITY;
           }
           score[rt][st][i] = value;
         }
       }
     }
 
+    // ---- V scales out of LDS ---------------------------------------------------
+    // in flight, oldest first: this tile's V, the next tile's K
+    if (has_next)
+      vmem_wait<KS_LOADS>();
+    else
+      vmem_wait<0>();
+    u32x2 value_scale_raw[4];
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+      ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
+    }(std::make_integer_sequence<int, 4>{});
+    lds_wait(value_scale_raw);
+    // folded into the probabilities: pair (u, c) =
+    // (scale[token 16*(2u) + 4*quad + c], scale[token 16*(2u+1) + 4*quad + c])
+    f16x2 v_scale[2][4];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        uint32_t lo = (value_scale_raw[2 * u][c / 2] >> (16 * (c % 2))) & 0xffffu;
+        uint32_t hi =
+            (value_scale_raw[2 * u + 1][c / 2] >> (16 * (c % 2))) & 0xffffu;
+        if (needs_mask) {
+          // records no row can see may be uninitialised: keep their scale
+          // (any bit pattern) away from the matrix core
+          if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
+          if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context)
+            hi = 0u;
+        }
+        v_scale[u][c] = __builtin_bit_cast(f16x2, lo | (hi << 16));
+      }
+    }
+
     // ---- online softmax (lane owns query row `col` of each row tile) ----------
+    float q_scale[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) q_scale[rt] = exchange_scale[16 * rt + col];
     float new_max[RT];
     bool grew = false;
 #pragma unroll
@@ -324,7 +584,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
-        const float factor = __builtin_amdgcn_exp2f(running_max[rt] - new_max[rt]);
+        const float factor = __builtin_amdgcn_exp2f(
+            (running_max[rt] - new_max[rt]) * q_scale[rt]);
         running_max[rt] = new_max[rt];
         running_sum[rt] *= factor;
 #pragma unroll
@@ -333,84 +594,58 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
           for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
       }
     }
-    // P^T operands: k-step u covers sub-tiles 2u, 2u+1; register c pairs the
-    // tokens (2u, i=c) and (2u+1, i=c)
+    // P^T operands (probability times the token's V scale): k-step u covers
+    // sub-tiles 2u, 2u+1; register c pairs the tokens (2u, i=c), (2u+1, i=c)
     f16x8 p_operand[RT][2];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+      const float offset = -running_max[rt] * q_scale[rt];
       float sum = 0.0f;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          const float p0 = __builtin_amdgcn_exp2f(score[rt][2 * u][c] - running_max[rt]);
-          const float p1 = __builtin_amdgcn_exp2f(score[rt][2 * u + 1][c] - running_max[rt]);
-          const _Float16 h0 = static_cast<_Float16>(p0);
-          const _Float16 h1 = static_cast<_Float16>(p1);
-          sum += static_cast<float>(h0) + static_cast<float>(h1);
-          p_operand[rt][u][2 * c] = h0;
-          p_operand[rt][u][2 * c + 1] = h1;
+          const float p0 = __builtin_amdgcn_exp2f(
+              fmaf(score[rt][2 * u][c], q_scale[rt], offset));
+          const float p1 = __builtin_amdgcn_exp2f(
+              fmaf(score[rt][2 * u + 1][c], q_scale[rt], offset));
+          sum += p0 + p1;
+          f16x2 pair = {static_cast<_Float16>(p0), static_cast<_Float16>(p1)};
+          pair *= v_scale[u][c];
+          p_operand[rt][u][2 * c] = pair[0];
+          p_operand[rt][u][2 * c + 1] = pair[1];
         }
       running_sum[rt] += sum;
     }
 
-    // ---- V scales as f16 pairs matching the nibble pairing --------------------
-    // pair (u, c) = (scale[token 16*(2u) + 4*quad + c], scale[16*(2u+1) + ..])
-    f16x2 v_scale[2][4], v_scale16[2][4];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const uint32_t even[2] = {value_scale_raw[2 * u].x, value_scale_raw[2 * u].y};
-      const uint32_t odd[2] = {value_scale_raw[2 * u + 1].x,
-                               value_scale_raw[2 * u + 1].y};
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        uint32_t lo = (even[c / 2] >> (16 * (c % 2))) & 0xffffu;
-        uint32_t hi = (odd[c / 2] >> (16 * (c % 2))) & 0xffffu;
-        if (needs_mask) {
-          // never let uninitialised records (tokens no row can see) reach the
-          // matrix core: a NaN scale times a zero probability is still NaN
-          if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
-          if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context) hi = 0u;
-        }
-        const f16x2 pair = __builtin_bit_cast(f16x2, lo | (hi << 16));
-        v_scale[u][c] = pair;
-        v_scale16[u][c] = pair * static_cast<_Float16>(0.0625f);
-      }
-    }
+    // ---- V codes out of LDS, transposed to d-major ----------------------------
+    u32x2 transposed[DT];
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+      ((transposed[I] = lds_read8_transposed4<I * 8>(value_address)), ...);
+    }(std::make_integer_sequence<int, DT>{});
+    lds_wait(transposed);
+    if (has_next) stage_values(tile + 1u);
 
     // ---- O^T += V^T . P^T -------------------------------------------------------
-    __builtin_amdgcn_wave_barrier();
-    // lane (col, quad) supplies LDS row 16*quad + col, i.e. token
-    // 16*(col/4) + 4*quad + col%4 of the tile
-    const uint32_t stage_row = 16u * quad + col;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      const i32x2 transposed = __builtin_amdgcn_ds_read_tr4_b64_v2i32(
-          (__attribute__((address_space(3))) i32x2*)(v_stage +
-                                                     stage_row * VROW + dt * 8));
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const uint32_t x = static_cast<uint32_t>(transposed[u]) ^ 0x88888888u;
-        const uint32_t y = x >> 8;
+        // two's complement nibble -> code + 8, dropped into mantissa bits 6..9
+        // of the binary16 number 16.0: the bit pattern is 16 + (code + 8)
+        // exactly, and subtracting 24 leaves the signed code.
+        const uint32_t x = transposed[dt][u] ^ 0x88888888u;
+        const f16x2 bias = {static_cast<_Float16>(-24.0f),
+                            static_cast<_Float16>(-24.0f)};
+        const f16x2 e0 = __builtin_bit_cast(
+            f16x2, ((x << 6) & 0x03c003c0u) | 0x4c004c00u) + bias;
+        const f16x2 e1 = __builtin_bit_cast(
+            f16x2, ((x << 2) & 0x03c003c0u) | 0x4c004c00u) + bias;
+        const f16x2 e2 = __builtin_bit_cast(
+            f16x2, ((x >> 2) & 0x03c003c0u) | 0x4c004c00u) + bias;
+        const f16x2 e3 = __builtin_bit_cast(
+            f16x2, ((x >> 6) & 0x03c003c0u) | 0x4c004c00u) + bias;
         f16x8 v_operand;
-        // 0x6400 | u is the binary16 number 1024 + u (u = code + 8); the
-        // subtraction is exact, the multiply rounds once.
-        const f16x2 offset0 = {static_cast<_Float16>(-1032.0f),
-                               static_cast<_Float16>(-1032.0f)};
-        const f16x2 offset1 = {static_cast<_Float16>(-1152.0f),
-                               static_cast<_Float16>(-1152.0f)};
-        const f16x2 e0 =
-            (__builtin_bit_cast(f16x2, (x & 0x000f000fu) | 0x64006400u) + offset0) *
-            v_scale[u][0];
-        const f16x2 e1 =
-            (__builtin_bit_cast(f16x2, (x & 0x00f000f0u) | 0x64006400u) + offset1) *
-            v_scale16[u][1];
-        const f16x2 e2 =
-            (__builtin_bit_cast(f16x2, (y & 0x000f000fu) | 0x64006400u) + offset0) *
-            v_scale[u][2];
-        const f16x2 e3 =
-            (__builtin_bit_cast(f16x2, (y & 0x00f000f0u) | 0x64006400u) + offset1) *
-            v_scale16[u][3];
         v_operand[0] = e0[0]; v_operand[1] = e0[1];
         v_operand[2] = e1[0]; v_operand[3] = e1[1];
         v_operand[4] = e2[0]; v_operand[5] = e2[1];
@@ -421,57 +656,67 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
               v_operand, p_operand[rt][u], out[dt][rt], 0, 0, 0);
       }
     }
-    __builtin_amdgcn_wave_barrier();
   }
 
-  // each lane summed only its own tokens
+  // each lane summed only its own tokens; maxima go to true log2 units
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) running_sum[rt] = quad_row_sum(running_sum[rt]);
+  for (int rt = 0; rt < RT; ++rt) {
+    running_sum[rt] = quad_row_sum(running_sum[rt]);
+    running_max[rt] = running_max[rt] > 0.5f * kMaskedMax
+                          ? running_max[rt] * exchange_scale[16 * rt + col]
+                          : kMaskedMax;
+  }
 
   // ---- merge the eight wave states in LDS (tree: 4+4, 2+2, 1+1) --------------
-  // state layout per wave slot: max[16*RT] | sum[16*RT] | out[16*RT][D]
-  float* slots = reinterpret_cast<float*>(lds_raw);
-  __syncthreads();  // V staging no longer needed
+  // SLOTS states fit into the staging memory at a time; a level with more
+  // senders than that runs in batches.
+  // state layout per slot: max[16*RT] | sum[16*RT] | out[16*RT][D]
+  float* slots = reinterpret_cast<float*>(stage);
+  __syncthreads();  // staging no longer needed
 #pragma unroll
   for (int span = kSplitWaves / 2; span >= 1; span /= 2) {
-    if (wave >= static_cast<uint32_t>(span) &&
-        wave < static_cast<uint32_t>(2 * span)) {
-      float* slot = slots + (wave - span) * STATE;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (quad == 0u) {
-          slot[16 * rt + col] = running_max[rt];
-          slot[16 * RT + 16 * rt + col] = running_sum[rt];
-        }
+    for (int batch = 0; batch < span; batch += SLOTS) {
+      const uint32_t first_sender = span + batch;
+      const uint32_t senders = min(SLOTS, span - batch);
+      if (wave >= first_sender && wave < first_sender + senders) {
+        float* slot = slots + (wave - first_sender) * STATE;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          *reinterpret_cast<f32x4*>(slot + 32 * RT + (16 * rt + col) * D +
-                                    16 * dt + 4 * quad) = out[dt][rt];
-      }
-    }
-    __syncthreads();
-    if (wave < static_cast<uint32_t>(span)) {
-      const float* slot = slots + wave * STATE;
+        for (int rt = 0; rt < RT; ++rt) {
+          if (quad == 0u) {
+            slot[16 * rt + col] = running_max[rt];
+            slot[16 * RT + 16 * rt + col] = running_sum[rt];
+          }
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const float other_max = slot[16 * rt + col];
-        const float other_sum = slot[16 * RT + 16 * rt + col];
-        const float merged = fmaxf(running_max[rt], other_max);
-        const float mine = __builtin_amdgcn_exp2f(running_max[rt] - merged);
-        const float theirs = __builtin_amdgcn_exp2f(other_max - merged);
-        running_max[rt] = merged;
-        running_sum[rt] = running_sum[rt] * mine + other_sum * theirs;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          const f32x4 other = *reinterpret_cast<const f32x4*>(
-              slot + 32 * RT + (16 * rt + col) * D + 16 * dt + 4 * quad);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            out[dt][rt][i] = out[dt][rt][i] * mine + other[i] * theirs;
+          for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<f32x4*>(slot + 32 * RT + (16 * rt + col) * D +
+                                      16 * dt + 4 * quad) = out[dt][rt];
         }
       }
+      __syncthreads();
+      if (wave >= static_cast<uint32_t>(batch) && wave < batch + senders) {
+        const float* slot = slots + (wave - batch) * STATE;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const float other_max = slot[16 * rt + col];
+          const float other_sum = slot[16 * RT + 16 * rt + col];
+          const float merged = fmaxf(running_max[rt], other_max);
+          const float mine = __builtin_amdgcn_exp2f(running_max[rt] - merged);
+          const float theirs = __builtin_amdgcn_exp2f(other_max - merged);
+          running_max[rt] = merged;
+          running_sum[rt] = running_sum[rt] * mine + other_sum * theirs;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const f32x4 other = *reinterpret_cast<const f32x4*>(
+                slot + 32 * RT + (16 * rt + col) * D + 16 * dt + 4 * quad);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              out[dt][rt][i] = out[dt][rt][i] * mine + other[i] * theirs;
+          }
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 
   if (wave != 0u) return;
@@ -496,6 +741,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 }
 
 // Split-K merge (maxima in log2 units), optional sigmoid output gate.
+// One workgroup per (query head, row), one thread per output dimension.  The
+// per-split weights exp2(m_s - M) are computed once, cooperatively, into LDS;
+// the accumulation over splits then has independent loads that pipeline.
+constexpr uint32_t kCombineSplitCapacity = 2048;
+
 __global__ void attention_combine_kernel(
     const float* query, uint32_t query_stride, int output_gated,
     const float* partial_maxima, const float* partial_sums,
@@ -503,28 +753,47 @@ __global__ void attention_combine_kernel(
     uint32_t first_context_tokens, uint32_t maximum_splits,
     uint32_t split_tokens, uint32_t query_heads, uint32_t head_dim,
     const uint32_t* device_positions) {
+  __shared__ float weights[kCombineSplitCapacity];
+  __shared__ float scratch[4];
   if (device_positions) first_context_tokens = device_positions[2];
   const uint32_t head = blockIdx.x;
   const uint32_t row = blockIdx.y;
   const uint32_t dimension = threadIdx.x;
+  // balanced launches (split_tokens == 0) use every split
   const uint32_t active =
-      (first_context_tokens + row + split_tokens - 1u) / split_tokens;
-  float maximum = kMaskedMax;
-  for (uint32_t split = 0; split < active; ++split)
-    maximum = fmaxf(
-        maximum, partial_maxima[(static_cast<size_t>(row) * maximum_splits +
-                                 split) * query_heads + head]);
-  float sum = 0.0f;
-  float result = 0.0f;
-  for (uint32_t split = 0; split < active; ++split) {
-    const size_t partial =
-        (static_cast<size_t>(row) * maximum_splits + split) * query_heads + head;
-    const float weight = __builtin_amdgcn_exp2f(partial_maxima[partial] - maximum);
-    sum += partial_sums[partial] * weight;
-    if (dimension < head_dim)
-      result += partial_outputs[partial * head_dim + dimension] * weight;
+      split_tokens ? (first_context_tokens + row + split_tokens - 1u) / split_tokens
+                   : maximum_splits;
+  const size_t first_partial =
+      static_cast<size_t>(row) * maximum_splits * query_heads + head;
+  float local_max = kMaskedMax;
+  for (uint32_t split = threadIdx.x; split < active; split += blockDim.x)
+    local_max = fmaxf(local_max,
+                      partial_maxima[first_partial +
+                                     static_cast<size_t>(split) * query_heads]);
+  const float maximum = block_max(local_max, scratch);
+  float local_sum = 0.0f;
+  for (uint32_t split = threadIdx.x; split < active; split += blockDim.x) {
+    const size_t partial = first_partial + static_cast<size_t>(split) * query_heads;
+    const float weight =
+        __builtin_amdgcn_exp2f(partial_maxima[partial] - maximum);
+    weights[split] = weight;
+    local_sum += partial_sums[partial] * weight;
   }
-  if (dimension >= head_dim) return;
+  const float sum = block_sum(local_sum, scratch);  // also publishes weights[]
+  float result = 0.0f;
+  const float* source = partial_outputs + first_partial * head_dim + dimension;
+  const size_t stride = static_cast<size_t>(query_heads) * head_dim;
+  uint32_t split = 0;
+  for (; split + 4u <= active; split += 4u) {
+    const float a = source[(split + 0u) * stride];
+    const float b = source[(split + 1u) * stride];
+    const float c = source[(split + 2u) * stride];
+    const float d = source[(split + 3u) * stride];
+    result += a * weights[split] + b * weights[split + 1u] +
+              c * weights[split + 2u] + d * weights[split + 3u];
+  }
+  for (; split < active; ++split)
+    result += source[split * stride] * weights[split];
   result /= sum;
   const size_t record = static_cast<size_t>(row) * query_heads + head;
   if (output_gated) {
@@ -702,10 +971,7 @@ __global__ __launch_bounds__(64) void quantize_queries_q8_kernel(
 template <int D>
 int32_t launch_split(const SplitArgs& args, uint32_t row_tiles, dim3 grid,
                      hipStream_t stream) {
-  constexpr size_t stage = static_cast<size_t>(kSplitWaves) * 64 * (D / 2 + 16);
-  const size_t merge = static_cast<size_t>(kSplitWaves / 2) * 16 * row_tiles *
-                       (D + 2) * sizeof(float);
-  const size_t lds = stage > merge ? stage : merge;
+  const size_t lds = 0;  // all LDS of the split kernel is static
   switch (row_tiles) {
     case 1:
       q4h_attention_split_kernel<D, 1><<<grid, kSplitWaves * 64, lds, stream>>>(args);
@@ -863,8 +1129,8 @@ extern "C" int32_t qllm_attention_paged_q4h(
       !launch->query_heads || !launch->kv_heads ||
       launch->query_heads % launch->kv_heads ||
       (launch->head_dim != 128u && launch->head_dim != 256u) ||
-      !launch->split_tokens || launch->split_tokens % 64u ||
-      !launch->maximum_splits ||
+      launch->split_tokens % 64u || !launch->maximum_splits ||
+      launch->maximum_splits > kCombineSplitCapacity ||
       launch->query_stride <
           (launch->output_gated ? 2u : 1u) * launch->head_dim ||
       (launch->output_kind != QLLM_OUT_F32 &&
@@ -882,7 +1148,7 @@ extern "C" int32_t qllm_attention_paged_q4h(
   // with device-side positions the context is not known here: cover every
   // split (workgroups past the context write neutral partials)
   const uint32_t splits =
-      launch->device_positions
+      launch->device_positions || !launch->split_tokens
           ? launch->maximum_splits
           : (last_context + launch->split_tokens - 1u) / launch->split_tokens;
   if (splits > launch->maximum_splits)

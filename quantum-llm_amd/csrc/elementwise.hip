@@ -129,6 +129,65 @@ __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
   }
 }
 
+// Same operation for rows of up to 16384 elements (a multiple of 4): 1024
+// threads per row, the row is read once with 16-byte loads and kept in
+// registers between the reduction and the scaling.
+__global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
+    const float* input, const float* weight, float* output_f32,
+    uint16_t* output_bf16, uint32_t bf16_padded_columns, uint32_t elements,
+    float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const uint32_t row = blockIdx.x;
+  const float4* x =
+      reinterpret_cast<const float4*>(input + static_cast<size_t>(row) * elements);
+  const uint32_t vectors = elements / 4u;
+  float4 values[4];
+  float square = 0.0f;
+#pragma unroll
+  for (int slot = 0; slot < 4; ++slot) {
+    const uint32_t index = slot * 1024u + threadIdx.x;
+    values[slot] = index < vectors ? x[index] : make_float4(0.f, 0.f, 0.f, 0.f);
+    square = fmaf(values[slot].x, values[slot].x, square);
+    square = fmaf(values[slot].y, values[slot].y, square);
+    square = fmaf(values[slot].z, values[slot].z, square);
+    square = fmaf(values[slot].w, values[slot].w, square);
+  }
+  square = block_sum(square, scratch);
+  const float inverse =
+      rsqrtf(square / static_cast<float>(elements) + epsilon);
+#pragma unroll
+  for (int slot = 0; slot < 4; ++slot) {
+    const uint32_t index = slot * 1024u + threadIdx.x;
+    if (index >= vectors) continue;
+    float4 factor = make_float4(1.f, 1.f, 1.f, 1.f);
+    if (weight) {
+      factor = reinterpret_cast<const float4*>(weight)[index];
+      if (zero_centered) {
+        factor.x += 1.0f; factor.y += 1.0f; factor.z += 1.0f; factor.w += 1.0f;
+      }
+    }
+    float4 result;
+    result.x = values[slot].x * inverse * factor.x;
+    result.y = values[slot].y * inverse * factor.y;
+    result.z = values[slot].z * inverse * factor.z;
+    result.w = values[slot].w * inverse * factor.w;
+    if (output_f32)
+      reinterpret_cast<float4*>(output_f32 +
+                                static_cast<size_t>(row) * elements)[index] = result;
+    if (output_bf16) {
+      uint2 packed;
+      packed.x = f32_to_bf16_bits(result.x) | (f32_to_bf16_bits(result.y) << 16);
+      packed.y = f32_to_bf16_bits(result.z) | (f32_to_bf16_bits(result.w) << 16);
+      reinterpret_cast<uint2*>(output_bf16 + static_cast<size_t>(row) *
+                                                 bf16_padded_columns)[index] = packed;
+    }
+  }
+  if (output_bf16)
+    for (uint32_t index = elements + threadIdx.x; index < bf16_padded_columns;
+         index += 1024u)
+      output_bf16[static_cast<size_t>(row) * bf16_padded_columns + index] = 0u;
+}
+
 // transformer_kernels.cu:2522-2528
 __global__ void add_kernel(float* destination, const float* source,
                            uint32_t count, bool bf16_output) {
@@ -255,9 +314,20 @@ extern "C" int32_t qllm_rms_norm_batch(const float* input, const float* weight,
       !(epsilon > 0.0f) ||
       (output_bf16 && bf16_padded_columns < elements))
     return fail(QLLM_INVALID_ARGUMENT, "invalid RMSNorm batch");
-  rms_norm_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
-      input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
-      bf16_padded_columns, elements, epsilon, zero_centered != 0);
+  const bool aligned =
+      ((reinterpret_cast<uintptr_t>(input) |
+        reinterpret_cast<uintptr_t>(weight) |
+        reinterpret_cast<uintptr_t>(output_f32)) & 15u) == 0u &&
+      (reinterpret_cast<uintptr_t>(output_bf16) & 7u) == 0u;
+  if (elements % 4u == 0u && elements <= 16384u && aligned &&
+      bf16_padded_columns % 4u == 0u)
+    rms_norm_batch_wide_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+        input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
+        bf16_padded_columns, elements, epsilon, zero_centered != 0);
+  else
+    rms_norm_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
+        input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
+        bf16_padded_columns, elements, epsilon, zero_centered != 0);
   return launched("RMSNorm batch");
 }
 

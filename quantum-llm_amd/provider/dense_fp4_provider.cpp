@@ -209,6 +209,13 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   split = std::max(512U, (split + 63U) / 64U * 64U);
   split_tokens_ = split;
   maximum_splits_ = (g_.max_context + split - 1U) / split;
+  if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
+    // the Q4H kernel deals the context's 64-token tiles evenly over the grid
+    // itself (split_tokens 0), whatever the context length
+    split_tokens_ = 0U;
+    maximum_splits_ =
+        std::min(wanted_splits, std::max(1U, (g_.max_context + 511U) / 512U));
+  }
   const std::size_t partials = rows * maximum_splits_ * g_.query_heads;
   partial_maxima_ = static_cast<float*>(device_alloc(partials * 4U));
   partial_sums_ = static_cast<float*>(device_alloc(partials * 4U));

@@ -48,14 +48,17 @@ def gemm(device, codes, scales, scheme, rows, padded, act_bf16_values, *,
 
 def q4h_attention(device, pages, query, rows, query_heads, kv_heads, head_dim,
                   first_context, page_tokens, split_tokens, gated, layer=0,
-                  out_kind=qh.OUT_F32):
+                  out_kind=qh.OUT_F32, balanced_splits=32):
+    """split_tokens 0 selects the balanced partition over `balanced_splits`
+    workgroups per KV head."""
     stride = head_dim * (2 if gated else 1)
     d_pages = [device_tensor(page, device) for page in pages]
     table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
                          device=device)
     d_query = device_tensor(query, device)
     context = first_context + rows - 1
-    splits = (context + split_tokens - 1) // split_tokens
+    splits = ((context + split_tokens - 1) // split_tokens if split_tokens
+              else balanced_splits)
     maxima = torch.zeros((rows, splits, query_heads), device=device)
     sums = torch.zeros_like(maxima)
     outputs = torch.zeros((rows, splits, query_heads, head_dim), device=device)

@@ -36,7 +36,13 @@ def run_case(device, rng, tokens, rows, Q, KV, d, page_tokens, split_tokens, gat
     (700, 5, 24, 4, 256, 256, 512, True),     # reference geometry, gated
     (3000, 1, 64, 8, 128, 256, 1024, False),  # single-row decode
     (257, 3, 16, 8, 128, 64, 128, True),
-    (4100, 5, 64, 8, 128, 256, 512, False)])
+    (4100, 5, 64, 8, 128, 256, 512, False),
+    # split 0: tiles dealt evenly over 32 workgroups per KV head
+    (5, 5, 8, 2, 128, 64, 0, False),          # most waves have no tile at all
+    (100, 5, 64, 8, 128, 256, 0, False),
+    (4100, 5, 64, 8, 128, 256, 0, False),
+    (20000, 5, 64, 8, 128, 256, 0, False),    # 2-3 tiles per wave
+    (1500, 4, 24, 4, 256, 256, 0, True)])
 def test_attention_matches_oracle(device, tokens, rows, Q, KV, d, page, split, gated):
     rng = np.random.default_rng(tokens + 7 * rows + Q)
     got, want, _ = run_case(device, rng, tokens, rows, Q, KV, d, page, split, gated)
@@ -73,7 +79,7 @@ def test_attention_is_split_invariant_at_32k(device):
     query = ol.bf16_round(rng.standard_normal((rows, Q, d)).astype(np.float32))
     first = tokens - 4
     results = [gu.q4h_attention(device, pages, query, rows, Q, KV, d, first, page,
-                                split, False) for split in (1024, 4096, 32768)]
+                                split, False) for split in (1024, 4096, 32768, 0)]
     for other in results[1:]:
         assert np.abs(other - results[0]).max() < 2e-5
     # oracle on two KV heads' worth of query heads (full double precision)
