@@ -114,6 +114,17 @@ __device__ __forceinline__ const void* uniform_page(
   return ((constant_table)page_table)[index];
 }
 
+// Tells the compiler that a pointer every lane computes alike is wave-uniform,
+// so that it can live in scalar registers.
+__device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* pointer) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(pointer);
+  const uint32_t low =
+      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t high =
+      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(high) << 32) | low);
+}
+
 // Direct global -> LDS loads (no VGPRs): lane l of the wave fetches 16 (4)
 // bytes at base + offset[l] and they land at lds + 16*l (4*l).  `base` and
 // `lds` are wave-uniform.  Written as assembly so that the address stays in
@@ -205,6 +216,13 @@ __device__ __forceinline__ uint32_t fresh_lane_index() {
                : "=v"(lane));
   return lane;
 }
+// (value & mask) | (base & ~mask) in one instruction
+__device__ __forceinline__ uint32_t insert_bits(uint32_t mask, uint32_t value,
+                                                uint32_t base) {
+  uint32_t result;
+  asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(result) : "s"(mask), "v"(value), "v"(base));
+  return result;
+}
 __device__ __forceinline__ uint32_t lds_address(const void* pointer) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (__attribute__((address_space(3))) const void*)pointer));
@@ -226,14 +244,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   constexpr int CODES = 64 * ROW;     // bytes of K (or V) codes per tile
   // staging area of a wave: K codes | K scales | V codes | V scales
   constexpr int STAGE = 2 * CODES + 512;
-  constexpr int STATE = 16 * RT * (D + 2);   // floats per merged wave state
   constexpr int PASSES = ROW / 16;    // direct loads per code plane and tile
   constexpr int KS_LOADS = PASSES + 1;       // K codes + K scales
   constexpr int V_LOADS = PASSES + 1;        // V codes + V scales
-  // merge slots that fit into the staging memory once the tiles are done
-  constexpr int SLOTS =
-      kSplitWaves * STAGE >= 4 * STATE * 4 ? 4 : 2;
-  static_assert(kSplitWaves * STAGE >= SLOTS * STATE * 4, "merge does not fit");
   __shared__ __attribute__((aligned(16))) uint8_t stage[kSplitWaves * STAGE];
   // query operands in MFMA order, then per matrix row its scale and the number
   // of tokens it may attend
@@ -301,13 +314,13 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
     const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
                            tile_begin % args.page_tokens;
-    const uint8_t* key_rows = planes.key_codes + record0 * ROW;  // uniform
+    const uint8_t* key_rows = uniform_pointer(planes.key_codes + record0 * ROW);
+    const uint8_t* key_scales = uniform_pointer(planes.key_scales + record0 * 2u);
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass)
       copy16_to_lds(key_rows + pass * 1024, lane_now * 16u,
                     stage_k_lds + pass * 1024);
-    copy4_to_lds(planes.key_scales + record0 * 2u, 4u * (lane_now & 31u),
-                 stage_s_lds);
+    copy4_to_lds(key_scales, 4u * (lane_now & 31u), stage_s_lds);
   };
   // V_LOADS direct loads: V codes and V scales of a tile.  V row R holds token
   // 16*((R/4)%4) + 4*(R/16) + R%4, so the 16 tokens a lane group reads back
@@ -325,7 +338,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
     const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
                            tile_begin % args.page_tokens;
-    const uint8_t* value_rows = planes.value_codes + record0 * ROW;  // uniform
+    const uint8_t* value_rows =
+        uniform_pointer(planes.value_codes + record0 * ROW);
+    const uint8_t* value_scales = uniform_pointer(
+        planes.key_scales + record0 * 2u + value_scale_distance);
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
       const uint32_t first_row = pass * kPassRows;
@@ -334,24 +350,26 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       copy16_to_lds(value_rows + pass_token * ROW, value_lane_offset,
                     stage_v_lds + pass * 1024);
     }
-    copy4_to_lds(planes.key_scales + record0 * 2u + value_scale_distance,
-                 4u * (lane_now & 31u), stage_vs_lds);
+    copy4_to_lds(value_scales, 4u * (lane_now & 31u), stage_vs_lds);
   };
 
   // ---- query operands (B side of S = K.Q), built once per workgroup ---------
   // The F32 query row is quantised here to 15 bits and split into two int8
   // planes, q = scale * (128*hi + lo) with hi in [-127,127], lo in [-64,63],
   // so the integer scores carry the query to ~3e-5 relative instead of the
-  // 4e-3 of a single Q8 plane.  Wave rt builds row tile rt and publishes it in
-  // MFMA operand order.
-  if (wave < static_cast<uint32_t>(RT)) {
-    const uint32_t rt = wave;
+  // 4e-3 of a single Q8 plane.  The operands are published in MFMA order.
+  static_assert(RT * KSTEPS <= kSplitWaves, "one wave per operand pair");
+  if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
+    // wave u builds k-step u % KSTEPS of row tile u / KSTEPS (the row's scale
+    // needs the whole row, so every such wave reads all of it)
+    const uint32_t rt = wave / KSTEPS;
+    const uint32_t step = wave % KSTEPS;
     const uint32_t matrix_row = 16u * rt + col;
     const bool valid = matrix_row < matrix_rows;
     const uint32_t row = valid ? matrix_row / group : 0u;
     const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
     const size_t record = static_cast<size_t>(row) * args.query_heads + head;
-    float values[KSTEPS][16];
+    float values[16];
     float maximum = 0.0f;
 #pragma unroll
     for (int h = 0; h < KSTEPS; ++h) {
@@ -362,10 +380,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         if (valid)
           loaded = *reinterpret_cast<const float4*>(
               args.query + record * args.query_stride + d0 + 4u * piece);
-        values[h][4 * piece + 0] = loaded.x;
-        values[h][4 * piece + 1] = loaded.y;
-        values[h][4 * piece + 2] = loaded.z;
-        values[h][4 * piece + 3] = loaded.w;
+        if (static_cast<uint32_t>(h) == step) {
+          values[4 * piece + 0] = loaded.x;
+          values[4 * piece + 1] = loaded.y;
+          values[4 * piece + 2] = loaded.z;
+          values[4 * piece + 3] = loaded.w;
+        }
         maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(loaded.x), fabsf(loaded.y)),
                                        fmaxf(fabsf(loaded.z), fabsf(loaded.w))));
       }
@@ -377,42 +397,40 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     maximum = quad_row_max(maximum);
     const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
     const float inverse = 1.0f / scale;
-    if (quad == 0u) {
-      exchange_scale[16 * rt + col] = scale;
+    if (quad == 0u && step == 0u) {
+      exchange_scale[16 * rt + col] =
+          scale * (1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D))));
       exchange_limit[16 * rt + col] = first_context_tokens + row;
     }
+    uint32_t high_bytes[16], low_bytes[16];
 #pragma unroll
-    for (int h = 0; h < KSTEPS; ++h) {
-      uint32_t high_bytes[16], low_bytes[16];
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        int quantized = __float2int_rn(values[h][j] * inverse);
-        quantized = max(-16319, min(16319, quantized));
-        const int high = (quantized + 64) >> 7;  // floor((v+64)/128)
-        const int low = quantized - (high << 7);
-        high_bytes[j] = static_cast<uint32_t>(high) & 0xffu;
-        low_bytes[j] = static_cast<uint32_t>(low) & 0xffu;
-      }
-      // byte order inside each 8-element half: even d first, then odd d,
-      // matching the order in which the key nibbles are widened
-      const int order[16] = {0, 2, 4, 6, 1, 3, 5, 7, 8, 10, 12, 14, 9, 11, 13, 15};
-      i32x4 high_operand, low_operand;
-#pragma unroll
-      for (int word = 0; word < 4; ++word) {
-        uint32_t high_word = 0u, low_word = 0u;
-#pragma unroll
-        for (int byte = 0; byte < 4; ++byte) {
-          high_word |= high_bytes[order[4 * word + byte]] << (8 * byte);
-          low_word |= low_bytes[order[4 * word + byte]] << (8 * byte);
-        }
-        high_operand[word] = static_cast<int>(high_word);
-        low_operand[word] = static_cast<int>(low_word);
-      }
-      *reinterpret_cast<i32x4*>(exchange + ((rt * KSTEPS + h) * 2 + 0) * 1024 +
-                                lane * 16u) = high_operand;
-      *reinterpret_cast<i32x4*>(exchange + ((rt * KSTEPS + h) * 2 + 1) * 1024 +
-                                lane * 16u) = low_operand;
+    for (int j = 0; j < 16; ++j) {
+      int quantized = __float2int_rn(values[j] * inverse);
+      quantized = max(-16319, min(16319, quantized));
+      const int high = (quantized + 64) >> 7;  // floor((v+64)/128)
+      const int low = quantized - (high << 7);
+      high_bytes[j] = static_cast<uint32_t>(high) & 0xffu;
+      low_bytes[j] = static_cast<uint32_t>(low) & 0xffu;
     }
+    // byte order inside each 8-element half: even d first, then odd d,
+    // matching the order in which the key nibbles are widened
+    const int order[16] = {0, 2, 4, 6, 1, 3, 5, 7, 8, 10, 12, 14, 9, 11, 13, 15};
+    i32x4 high_operand, low_operand;
+#pragma unroll
+    for (int word = 0; word < 4; ++word) {
+      uint32_t high_word = 0u, low_word = 0u;
+#pragma unroll
+      for (int byte = 0; byte < 4; ++byte) {
+        high_word |= high_bytes[order[4 * word + byte]] << (8 * byte);
+        low_word |= low_bytes[order[4 * word + byte]] << (8 * byte);
+      }
+      high_operand[word] = static_cast<int>(high_word);
+      low_operand[word] = static_cast<int>(low_word);
+    }
+    *reinterpret_cast<i32x4*>(exchange + (wave * 2u + 0u) * 1024u + lane * 16u) =
+        high_operand;
+    *reinterpret_cast<i32x4*>(exchange + (wave * 2u + 1u) * 1024u + lane * 16u) =
+        low_operand;
   } else if (tile_first < tile_last) {
     stage_keys(tile_first);
     stage_values(tile_first);
@@ -424,11 +442,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // limit: holding them next to the output accumulators would push the kernel
   // into scratch memory.
   const uint8_t* q_operands = exchange + lane * 16u;
-  // Scores are kept as t = int_dot * k_scale * unit; the true score in log2
-  // units is t * q_scale (q_scale is constant per query row, so maxima can be
-  // taken over t).
-  const float score_unit =
-      1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D)));
+  // Scores are kept as t = int_dot * k_scale; the true score in log2 units is
+  // t * q_scale, where q_scale (constant per query row, so maxima can be taken
+  // over t) carries the query's quantisation step, 1/16 for the widened key
+  // nibbles, 1/sqrt(D) and log2(e).
 
   // per-lane LDS addresses of the staged tile
   // K: lane (token = col, quad) takes 16 bytes of each sub-tile's K row
@@ -477,14 +494,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     // that half of the staging area is free: fetch the next tile's K
     if (has_next) stage_keys(tile + 1u);
 
-    // ---- S = K . Q ------------------------------------------------------------
-    float score[RT][4][4];
+    // K nibbles widened to int8 * 16 (sub-tile st, k-step h), scales of tokens
+    // 16*st + 4*quad + i
+    i32x4 key_operand[4][KSTEPS];
+    float k_scale[4][4];
 #pragma unroll
     for (int st = 0; st < 4; ++st) {
-      // keeps the compiler from merging the query operand reads of the four
-      // sub-tiles into registers that live across the whole tile
-      asm volatile("" ::: "memory");
-      i32x4 key_operand[KSTEPS];
 #pragma unroll
       for (int c = 0; c < D / 128; ++c) {
         const u32x4 x = key_raw[st * (D / 128) + c];
@@ -495,120 +510,136 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
           operand[1] = static_cast<int>(x[2 * half] & 0xf0f0f0f0u);
           operand[2] = static_cast<int>((x[2 * half + 1] << 4) & 0xf0f0f0f0u);
           operand[3] = static_cast<int>(x[2 * half + 1] & 0xf0f0f0f0u);
-          key_operand[2 * c + half] = operand;
+          key_operand[st][2 * c + half] = operand;
         }
       }
-      const float k_scale[4] = {
-          f16_bits_to_f32(scale_raw[st][0] & 0xffffu) * score_unit,
-          f16_bits_to_f32(scale_raw[st][0] >> 16) * score_unit,
-          f16_bits_to_f32(scale_raw[st][1] & 0xffffu) * score_unit,
-          f16_bits_to_f32(scale_raw[st][1] >> 16) * score_unit};
+      k_scale[st][0] = f16_bits_to_f32(scale_raw[st][0] & 0xffffu);
+      k_scale[st][1] = f16_bits_to_f32(scale_raw[st][0] >> 16);
+      k_scale[st][2] = f16_bits_to_f32(scale_raw[st][1] & 0xffffu);
+      k_scale[st][3] = f16_bits_to_f32(scale_raw[st][1] >> 16);
+    }
+
+    // V scales, folded into the probabilities: pair (u, c) =
+    // (scale[token 16*(2u) + 4*quad + c], scale[token 16*(2u+1) + 4*quad + c])
+    f16x2 v_scale[2][4];
+    // P^T operands (probability times the token's V scale): k-step u covers
+    // sub-tiles 2u, 2u+1; register c pairs the tokens (2u, i=c), (2u+1, i=c)
+    f16x8 p_operand[RT][2];
+
+    // One row tile at a time: scores, online softmax, probabilities.  A lane
+    // owns query row `col` of the row tile and 16 of the 64 tokens.
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
+      // keeps the compiler from fetching the query operands of all row tiles
+      // ahead of time (they would live across the whole tile)
+      asm volatile("" ::: "memory");
+      i32x4 q_high[KSTEPS], q_low[KSTEPS];
+#pragma unroll
+      for (int h = 0; h < KSTEPS; ++h) {
+        q_high[h] = *reinterpret_cast<const i32x4*>(
+            q_operands + ((rt * KSTEPS + h) * 2 + 0) * 1024);
+        q_low[h] = *reinterpret_cast<const i32x4*>(
+            q_operands + ((rt * KSTEPS + h) * 2 + 1) * 1024);
+      }
+      const float q_scale = exchange_scale[16 * rt + col];
+
+      // ---- S = K . Q ----------------------------------------------------------
+      float score[4][4];
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
         i32x4 dot_high = {0, 0, 0, 0};
         i32x4 dot_low = {0, 0, 0, 0};
 #pragma unroll
         for (int h = 0; h < KSTEPS; ++h) {
-          const i32x4 q_high = *reinterpret_cast<const i32x4*>(
-              q_operands + ((rt * KSTEPS + h) * 2 + 0) * 1024);
-          const i32x4 q_low = *reinterpret_cast<const i32x4*>(
-              q_operands + ((rt * KSTEPS + h) * 2 + 1) * 1024);
           dot_high = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-              key_operand[h], q_high, dot_high, 0, 0, 0);
+              key_operand[st][h], q_high[h], dot_high, 0, 0, 0);
           dot_low = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-              key_operand[h], q_low, dot_low, 0, 0, 0);
+              key_operand[st][h], q_low[h], dot_low, 0, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int dot = (dot_high[i] << 7) + dot_low[i];
-          float value = static_cast<float>(dot) * k_scale[i];
-          if (needs_mask) {
-            const uint32_t token = tile_begin + 16u * st + 4u * quad + i;
-            if (token >= exchange_limit[16 * rt + col]) value = -INFINITY;
+          score[st][i] = static_cast<float>(dot) * k_scale[st][i];
+        }
+      }
+      if (needs_mask) {
+        // only the tiles that reach past the first row's context get here
+        const uint32_t first_token = tile_begin + 4u * quad;
+        const uint32_t limit = exchange_limit[16 * rt + col];
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (first_token + 16u * st + i >= limit) score[st][i] = -INFINITY;
+      }
+
+      if (rt == 0) {
+        // ---- V scales out of LDS ----------------------------------------------
+        // in flight, oldest first: this tile's V, the next tile's K
+        if (has_next)
+          vmem_wait<KS_LOADS>();
+        else
+          vmem_wait<0>();
+        u32x2 value_scale_raw[4];
+        [&]<int... I>(std::integer_sequence<int, I...>) {
+          ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
+        }(std::make_integer_sequence<int, 4>{});
+        lds_wait(value_scale_raw);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            uint32_t lo =
+                (value_scale_raw[2 * u][c / 2] >> (16 * (c % 2))) & 0xffffu;
+            uint32_t hi =
+                (value_scale_raw[2 * u + 1][c / 2] >> (16 * (c % 2))) & 0xffffu;
+            if (needs_mask) {
+              // records no row can see may be uninitialised: keep their scale
+              // (any bit pattern) away from the matrix core
+              if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
+              if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context)
+                hi = 0u;
+            }
+            v_scale[u][c] = __builtin_bit_cast(f16x2, lo | (hi << 16));
           }
-          score[rt][st][i] = value;
         }
       }
-    }
 
-    // ---- V scales out of LDS ---------------------------------------------------
-    // in flight, oldest first: this tile's V, the next tile's K
-    if (has_next)
-      vmem_wait<KS_LOADS>();
-    else
-      vmem_wait<0>();
-    u32x2 value_scale_raw[4];
-    [&]<int... I>(std::integer_sequence<int, I...>) {
-      ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
-    }(std::make_integer_sequence<int, 4>{});
-    lds_wait(value_scale_raw);
-    // folded into the probabilities: pair (u, c) =
-    // (scale[token 16*(2u) + 4*quad + c], scale[token 16*(2u+1) + 4*quad + c])
-    f16x2 v_scale[2][4];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        uint32_t lo = (value_scale_raw[2 * u][c / 2] >> (16 * (c % 2))) & 0xffffu;
-        uint32_t hi =
-            (value_scale_raw[2 * u + 1][c / 2] >> (16 * (c % 2))) & 0xffffu;
-        if (needs_mask) {
-          // records no row can see may be uninitialised: keep their scale
-          // (any bit pattern) away from the matrix core
-          if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
-          if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context)
-            hi = 0u;
-        }
-        v_scale[u][c] = __builtin_bit_cast(f16x2, lo | (hi << 16));
-      }
-    }
-
-    // ---- online softmax (lane owns query row `col` of each row tile) ----------
-    float q_scale[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) q_scale[rt] = exchange_scale[16 * rt + col];
-    float new_max[RT];
-    bool grew = false;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      float tile_max = score[rt][0][0];
+      // ---- online softmax -----------------------------------------------------
+      // The running maximum only follows the tile maximum when that is more
+      // than 8 (log2 units) ahead - probabilities then stay below 2^8, harmless
+      // in F32 sums and binary16 operands - so the accumulators are rarely
+      // rescaled; on a wave's first tile there is nothing to rescale yet.
+      float tile_max = score[0][0];
 #pragma unroll
       for (int st = 0; st < 4; ++st)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          tile_max = fmaxf(tile_max, score[rt][st][i]);
+        for (int i = 0; i < 4; ++i) tile_max = fmaxf(tile_max, score[st][i]);
       tile_max = quad_row_max(tile_max);
-      new_max[rt] = fmaxf(running_max[rt], tile_max);
-      grew = grew || new_max[rt] > running_max[rt];
-    }
-    if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+      const bool grew = (tile_max - running_max[rt]) * q_scale > 8.0f;
+      if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+        const float new_max = fmaxf(running_max[rt], tile_max);
+        if (tile != tile_first) {
+          const float factor =
+              __builtin_amdgcn_exp2f((running_max[rt] - new_max) * q_scale);
+          running_sum[rt] *= factor;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const float factor = __builtin_amdgcn_exp2f(
-            (running_max[rt] - new_max[rt]) * q_scale[rt]);
-        running_max[rt] = new_max[rt];
-        running_sum[rt] *= factor;
+          for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+            for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+        }
+        running_max[rt] = new_max;
       }
-    }
-    // P^T operands (probability times the token's V scale): k-step u covers
-    // sub-tiles 2u, 2u+1; register c pairs the tokens (2u, i=c), (2u+1, i=c)
-    f16x8 p_operand[RT][2];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const float offset = -running_max[rt] * q_scale[rt];
+      const float offset = -running_max[rt] * q_scale;
       float sum = 0.0f;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-          const float p0 = __builtin_amdgcn_exp2f(
-              fmaf(score[rt][2 * u][c], q_scale[rt], offset));
-          const float p1 = __builtin_amdgcn_exp2f(
-              fmaf(score[rt][2 * u + 1][c], q_scale[rt], offset));
+          const float p0 =
+              __builtin_amdgcn_exp2f(fmaf(score[2 * u][c], q_scale, offset));
+          const float p1 =
+              __builtin_amdgcn_exp2f(fmaf(score[2 * u + 1][c], q_scale, offset));
           sum += p0 + p1;
           f16x2 pair = {static_cast<_Float16>(p0), static_cast<_Float16>(p1)};
           pair *= v_scale[u][c];
@@ -631,20 +662,25 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        // two's complement nibble -> code + 8, dropped into mantissa bits 6..9
-        // of the binary16 number 16.0: the bit pattern is 16 + (code + 8)
-        // exactly, and subtracting 24 leaves the signed code.
+        // two's complement nibble -> u = code + 8 (one XOR per 8 nibbles),
+        // inserted into the mantissa of a binary16 constant so that the bit
+        // pattern is a small integer plus u exactly: 1024 + u for a nibble in
+        // bits 0..3 (0x6400, ulp 1), 64 + u for one in bits 4..7 (0x5400, ulp
+        // 1/16).  Subtracting the constant plus 8 leaves the signed code.
         const uint32_t x = transposed[dt][u] ^ 0x88888888u;
-        const f16x2 bias = {static_cast<_Float16>(-24.0f),
-                            static_cast<_Float16>(-24.0f)};
+        const uint32_t y = x >> 8;
+        const f16x2 bias_low = {static_cast<_Float16>(-1032.0f),
+                                static_cast<_Float16>(-1032.0f)};
+        const f16x2 bias_high = {static_cast<_Float16>(-72.0f),
+                                 static_cast<_Float16>(-72.0f)};
         const f16x2 e0 = __builtin_bit_cast(
-            f16x2, ((x << 6) & 0x03c003c0u) | 0x4c004c00u) + bias;
+            f16x2, insert_bits(0x000f000fu, x, 0x64006400u)) + bias_low;
         const f16x2 e1 = __builtin_bit_cast(
-            f16x2, ((x << 2) & 0x03c003c0u) | 0x4c004c00u) + bias;
+            f16x2, insert_bits(0x00f000f0u, x, 0x54005400u)) + bias_high;
         const f16x2 e2 = __builtin_bit_cast(
-            f16x2, ((x >> 2) & 0x03c003c0u) | 0x4c004c00u) + bias;
+            f16x2, insert_bits(0x000f000fu, y, 0x64006400u)) + bias_low;
         const f16x2 e3 = __builtin_bit_cast(
-            f16x2, ((x >> 6) & 0x03c003c0u) | 0x4c004c00u) + bias;
+            f16x2, insert_bits(0x00f000f0u, y, 0x54005400u)) + bias_high;
         f16x8 v_operand;
         v_operand[0] = e0[0]; v_operand[1] = e0[1];
         v_operand[2] = e1[0]; v_operand[3] = e1[1];
@@ -667,59 +703,86 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
                           : kMaskedMax;
   }
 
-  // ---- merge the eight wave states in LDS (tree: 4+4, 2+2, 1+1) --------------
-  // SLOTS states fit into the staging memory at a time; a level with more
-  // senders than that runs in batches.
-  // state layout per slot: max[16*RT] | sum[16*RT] | out[16*RT][D]
-  float* slots = reinterpret_cast<float*>(stage);
-  __syncthreads();  // staging no longer needed
+  // ---- merge the eight wave states -------------------------------------------
+  // 1. every wave publishes its (max, sum) per row; all waves derive the
+  //    merged maximum and bring their own accumulators to it.
+  // 2. the accumulators are summed reduce-scatter style, eight 1 KiB register
+  //    vectors (one per receiving wave) at a time: each wave drops the eight
+  //    vectors of the group into LDS, lane-linear (no bank conflicts), and
+  //    wave v adds up vector v of all eight waves in a fixed order.  Wave v
+  //    ends up owning vectors v, v+8, ... of the result and writes them out.
+  constexpr int VECTORS = DT * RT;   // f32x4 accumulator vectors per wave
+  static_assert(VECTORS % kSplitWaves == 0, "vectors are dealt to 8 waves");
+  static_assert(kSplitWaves * kSplitWaves * 1024 <= kSplitWaves * STAGE,
+                "merge pool does not fit the staging memory");
+  static_assert(kSplitWaves * RT * 64 * 8 <= sizeof(exchange),
+                "row summaries do not fit the exchange area");
+  float2* summary = reinterpret_cast<float2*>(exchange);  // [wave][rt][lane]
+  float* pool = reinterpret_cast<float*>(stage);          // [wave][slot][lane] x 4
+  __syncthreads();  // tiles done: staging and the operand exchange are free
 #pragma unroll
-  for (int span = kSplitWaves / 2; span >= 1; span /= 2) {
+  for (int rt = 0; rt < RT; ++rt)
+    summary[(wave * RT + rt) * 64 + lane] =
+        make_float2(running_max[rt], running_sum[rt]);
+  __syncthreads();
+  float merged_max[RT], merged_sum[RT];
 #pragma unroll
-    for (int batch = 0; batch < span; batch += SLOTS) {
-      const uint32_t first_sender = span + batch;
-      const uint32_t senders = min(SLOTS, span - batch);
-      if (wave >= first_sender && wave < first_sender + senders) {
-        float* slot = slots + (wave - first_sender) * STATE;
+  for (int rt = 0; rt < RT; ++rt) {
+    float2 part[kSplitWaves];
+    float maximum = kMaskedMax;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          if (quad == 0u) {
-            slot[16 * rt + col] = running_max[rt];
-            slot[16 * RT + 16 * rt + col] = running_sum[rt];
-          }
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt)
-            *reinterpret_cast<f32x4*>(slot + 32 * RT + (16 * rt + col) * D +
-                                      16 * dt + 4 * quad) = out[dt][rt];
-        }
-      }
-      __syncthreads();
-      if (wave >= static_cast<uint32_t>(batch) && wave < batch + senders) {
-        const float* slot = slots + (wave - batch) * STATE;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          const float other_max = slot[16 * rt + col];
-          const float other_sum = slot[16 * RT + 16 * rt + col];
-          const float merged = fmaxf(running_max[rt], other_max);
-          const float mine = __builtin_amdgcn_exp2f(running_max[rt] - merged);
-          const float theirs = __builtin_amdgcn_exp2f(other_max - merged);
-          running_max[rt] = merged;
-          running_sum[rt] = running_sum[rt] * mine + other_sum * theirs;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) {
-            const f32x4 other = *reinterpret_cast<const f32x4*>(
-                slot + 32 * RT + (16 * rt + col) * D + 16 * dt + 4 * quad);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              out[dt][rt][i] = out[dt][rt][i] * mine + other[i] * theirs;
-          }
-        }
-      }
-      __syncthreads();
+    for (int w = 0; w < kSplitWaves; ++w) {
+      part[w] = summary[(w * RT + rt) * 64 + lane];
+      maximum = fmaxf(maximum, part[w].x);
     }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w)
+      sum = fmaf(part[w].y, __builtin_amdgcn_exp2f(part[w].x - maximum), sum);
+    const float factor = __builtin_amdgcn_exp2f(running_max[rt] - maximum);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+    merged_max[rt] = maximum;
+    merged_sum[rt] = sum;
+  }
+  f32x4 merged[VECTORS / kSplitWaves];
+#pragma unroll
+  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
+#pragma unroll
+    for (int v = 0; v < kSplitWaves; ++v) {
+      const int k = group_index * kSplitWaves + v;
+      *reinterpret_cast<f32x4*>(pool + ((wave * kSplitWaves + v) * 64 + lane) * 4u) =
+          out[k / RT][k % RT];
+    }
+    __syncthreads();
+    f32x4 total = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w)
+      total += *reinterpret_cast<const f32x4*>(
+          pool + ((w * kSplitWaves + wave) * 64 + lane) * 4u);
+    merged[group_index] = total;
+    __syncthreads();
   }
 
-  if (wave != 0u) return;
+  // ---- partials: wave v writes the vectors it owns, wave 0 also max and sum ----
+#pragma unroll
+  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
+    const uint32_t k = group_index * kSplitWaves + wave;
+    const uint32_t dt = k / RT;
+    const uint32_t rt = k % RT;
+    const uint32_t matrix_row = 16u * rt + col;
+    if (matrix_row >= matrix_rows) continue;
+    const uint32_t row = matrix_row / group;
+    const uint32_t head = kv_head * group + matrix_row % group;
+    const size_t partial =
+        (static_cast<size_t>(row) * args.maximum_splits + split) *
+            args.query_heads + head;
+    *reinterpret_cast<f32x4*>(args.partial_outputs + partial * D + 16u * dt +
+                              4u * quad) = merged[group_index];
+  }
+  if (wave != 0u || quad != 0u) return;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const uint32_t matrix_row = 16u * rt + col;
@@ -729,14 +792,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     const size_t partial =
         (static_cast<size_t>(row) * args.maximum_splits + split) *
             args.query_heads + head;
-    if (quad == 0u) {
-      args.partial_maxima[partial] = running_max[rt];
-      args.partial_sums[partial] = running_sum[rt];
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      *reinterpret_cast<f32x4*>(args.partial_outputs + partial * D + 16 * dt +
-                                4 * quad) = out[dt][rt];
+    args.partial_maxima[partial] = merged_max[rt];
+    args.partial_sums[partial] = merged_sum[rt];
   }
 }
 
