@@ -62,9 +62,10 @@ enum qllm_fp4_layout {
    * records and handed over by the tensor store. */
   QLLM_LAYOUT_ROW_MAJOR = 0,
   /* The provider's device layout produced once, at upload, by
-   * qllm_fp4_prepack: rows grouped in tiles of 32, columns in chunks of 64,
-   * the 64 sixteen-byte pieces of one (tile, chunk) contiguous in the order
-   * the GEMM's lanes consume them, so weights stream in 1 KiB bursts. */
+   * qllm_fp4_prepack: rows grouped in tiles of tile_rows (at most 32), columns
+   * in chunks of 64, the sixteen-byte pieces of one (tile, chunk) contiguous
+   * in the order the GEMM's lanes consume them, so weights stream in bursts of
+   * up to 1 KiB. */
   QLLM_LAYOUT_TILED = 1
 };
 
@@ -79,22 +80,25 @@ typedef struct qllm_fp4_matrix {
   uint32_t padded_columns;
   uint32_t scale_scheme;  /* enum qllm_scale_scheme */
   uint32_t layout;        /* enum qllm_fp4_layout */
-  uint32_t reserved;
+  uint32_t tile_rows;     /* tiled layout: rows per tile, 8..32 (0 = 32) */
 } qllm_fp4_matrix;
 
-/* Device bytes needed for the tiled copy of a matrix. */
-size_t qllm_fp4_packed_weight_bytes(uint32_t rows, uint32_t padded_columns);
+/* Device bytes needed for the tiled copy of a matrix; tile_rows in 8..32,
+ * 0 = 32. */
+size_t qllm_fp4_packed_weight_bytes(uint32_t rows, uint32_t padded_columns,
+                                    uint32_t tile_rows);
 size_t qllm_fp4_packed_scale_bytes(uint32_t rows, uint32_t padded_columns,
-                                   uint32_t scale_scheme);
+                                   uint32_t scale_scheme, uint32_t tile_rows);
 
 /* Re-lays a row-major matrix (padded_columns % 64 == 0) into the tiled
- * layout; `packed` (host struct) receives the descriptor of the copy.  This is
- * the device half of the provider's tensor upload
+ * layout with tiles of tile_rows rows (8..32, 0 = 32); `packed`
+ * (host struct) receives the descriptor of the copy.  This is the device half
+ * of the provider's tensor upload
  * (runtime/tools/dense_fp4_provider.cpp:3486-3660); it moves bytes and changes
  * no value. */
-int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source, void* packed_weights,
-                         void* packed_scales, qllm_fp4_matrix* packed,
-                         void* stream);
+int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source, uint32_t tile_rows,
+                         void* packed_weights, void* packed_scales,
+                         qllm_fp4_matrix* packed, void* stream);
 
 enum qllm_output_kind {
   QLLM_OUT_F32 = 0,         /* float [batch, rows] */
@@ -134,6 +138,24 @@ int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix, const void* input,
                            size_t input_bytes, void* output,
                            uint32_t output_kind, const float* residual,
                            uint32_t batch, void* stream);
+
+/* One launch for projections that share their input and were stored as one
+ * matrix, rows concatenated: segment s receives the next `rows` output rows
+ * as its own [batch, rows] array.  The provider uses it for the q, k and v
+ * projections of an attention block, three fp4_gemm_bf16_block32 calls in the
+ * reference (run_full_attention, dense_fp4_provider.cpp:7004-7011); every
+ * output value equals what the separate calls give.  K % 64 == 0, at most
+ * three segments. */
+typedef struct qllm_gemm_segment {
+  void* output;         /* [batch, rows] */
+  uint32_t rows;
+  uint32_t output_kind; /* enum qllm_output_kind */
+} qllm_gemm_segment;
+int32_t qllm_fp4_gemm_bf16_split(const qllm_fp4_matrix* matrix,
+                                 const void* input, size_t input_bytes,
+                                 const qllm_gemm_segment* segments,
+                                 uint32_t segment_count, uint32_t batch,
+                                 void* stream);
 
 /* Gate and up projections of one SwiGLU block in a single pass over a shared
  * BF16 input: out[m,n] = bf16(bf16(silu(gate[m,n])) * up[m,n]) stored as

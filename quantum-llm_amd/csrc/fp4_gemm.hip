@@ -69,6 +69,14 @@ struct GemmArgs {
   uint32_t padded_columns;
   uint32_t output_kind;
   uint32_t swiglu;              // tile 1 is the up projection of tile 0
+  uint32_t tile_rows;           // weight rows per tile, 8..32
+  // Optional split of the output rows over up to three buffers (the q, k and
+  // v projections stored as one matrix): segment s takes the next
+  // segment_rows[s] rows.  segments == 0: everything goes to `output`.
+  uint32_t segments;
+  uint32_t segment_rows[3];
+  uint32_t segment_kind[3];
+  void* segment_output[3];
 };
 
 // Epilogue store of one value.
@@ -83,14 +91,19 @@ __device__ __forceinline__ void store_output(void* output, uint32_t kind,
     static_cast<float*>(output)[index] = value;
 }
 
-// Workgroup = WAVES waves.  The workgroup owns TILES tiles of 32 weight rows;
+// Workgroup = WAVES waves.  The workgroup owns TILES tiles of h = tile_rows
+// (at most 32) weight rows - lanes n >= h repeat row h-1 and are ignored;
 // its waves interleave over 64-column chunks of K (wave w takes chunks
-// w, w+WAVES, ...), so together they stream whole 128-byte lines of each row.
-// Lane (n = lane%32, g = lane/32) loads the 16 bytes at
-//   row n, byte offset chunk*32 + g*16
-// i.e. 16-blocks {2g, 2g+1} of the chunk.  One v_permlane32_swap per dword
-// pair regroups that into "half g of block b" - the B-operand layout of the
-// 32x32x16 MFMA - without touching LDS.
+// w, w+WAVES, ...).  Lane (n = lane%32, g = lane/32) supplies, for each of the
+// chunk's four 16-blocks b, the half g (8 weights = 4 bytes) of row n - the
+// B-operand layout of the 32x32x16 MFMA.
+//
+// TILED selects the provider's streaming layout (see qllm_fp4_prepack): the
+// 64 sixteen-byte pieces a wave loads for one (tile, chunk) are contiguous
+// (one 1 KiB burst) and already hold the lane's four half-blocks.  With the
+// row-major layout lane (n, g) loads the 16 bytes at row n, byte offset
+// chunk*32 + g*16 (64 separate requests) and one v_permlane32_swap per dword
+// pair regroups them.
 //
 // Activations travel with the weights: together with the weight pieces of a
 // chunk a wave prefetches the batch x 64 activation values of that chunk
@@ -99,22 +112,27 @@ __device__ __forceinline__ void store_output(void* output, uint32_t kind,
 // fragments back.  Nothing is staged per workgroup, so there is no barrier in
 // the K loop and any K that is a multiple of 64 is handled alike.
 //
-// TILED selects the provider's streaming layout (see qllm_fp4_prepack): the
-// 64 sixteen-byte pieces a wave loads for one (tile, chunk) are contiguous,
-// so every wave-level load is one 1 KiB burst.  With the row-major layout the
-// same pieces sit a row stride apart (64 separate 16-byte requests).
+// Every block's MFMA starts from zero and its result is scaled in F32 by the
+// block's binary16 scale, so only the accumulator registers that hold batch
+// rows cost an FMA.  Batches of up to 6 rows sit in MFMA rows {0,1,2,4,5,6}:
+// those are registers 0..2 of both lane halves, one FMA fewer than rows 0..5.
 template <int SCHEME, int BATCH, int TILES, int WAVES, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     const GemmArgs args) {
-  constexpr int PF = 4;             // chunks in flight per lane
+  // chunks in flight per lane; three with two tiles per group, which keeps
+  // the kernel at three workgroups per CU so that the 544 groups of the fused
+  // gate/up launch are all resident at once
+  constexpr int PF = TILES == 2 ? 3 : 4;
   constexpr int PIECES = 8 * BATCH; // activation pieces per chunk
+  constexpr bool COMPACT = BATCH <= 6;
+  constexpr int REGS = COMPACT ? 3 : 4;  // accumulator registers in use
   // ring slot: PIECES pieces of 16 bytes, padded to 64 pieces
   __shared__ __attribute__((aligned(16))) uint4 ring[WAVES][2][64];
-  __shared__ float reduce[WAVES][TILES][4][64];
+  __shared__ float reduce[WAVES][TILES][REGS][64];
 
   const uint32_t lane = threadIdx.x & 63u;
   // wave index as a scalar, so everything derived from it (chunk counts,
-  // loop bounds) is uniform control flow
+  // loop bounds, addresses) is uniform
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t n = lane & 31u;
   const uint32_t g = lane >> 5;
@@ -122,45 +140,57 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint32_t row_bytes = K / 2u;
   const uint32_t scale_row_bytes =
       SCHEME == kSchemeF16 ? K / 8u : K / 32u;
-  const uint32_t m_lane = n < BATCH ? n : BATCH - 1u;
+  // batch row carried by MFMA row n on the A side (rows past the batch are
+  // don't-care and repeat the last one)
+  uint32_t batch_row = COMPACT ? (n >> 2) * 3u + (n & 3u) : n;
+  if (batch_row >= BATCH) batch_row = BATCH - 1u;
 
-  // per-chunk byte strides of the two streams
+  // Weight and scale streams: wave-uniform start of the tile's stream plus a
+  // 32-bit lane offset; consecutive chunks are weight_step / scale_step apart.
   constexpr uint32_t kScaleChunk = SCHEME == kSchemeF16 ? 8u : 2u;
-  const uint32_t weight_step = TILED ? 1024u : 32u;
-  const uint32_t scale_step = TILED ? 32u * kScaleChunk : kScaleChunk;
-  const uint8_t* weight_row[TILES];
-  const uint8_t* scale_row[TILES];
+  const uint32_t h = args.tile_rows;
+  const uint32_t tile_lane = n < h ? n : h - 1u;
+  const uint32_t weight_step = TILED ? 32u * h : 32u;
+  const uint32_t scale_step = TILED ? h * kScaleChunk : kScaleChunk;
+  const uint8_t* weight_base[TILES];
+  const uint8_t* scale_base[TILES];
+  uint32_t weight_lane[TILES];
+  uint32_t scale_lane[TILES];
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
     const uint32_t tile = args.swiglu ? blockIdx.x : blockIdx.x * TILES + t;
+    const uint32_t tiles = (args.rows + h - 1u) / h;
+    const uint32_t safe_tile = tile < tiles ? tile : tiles - 1u;
     if (TILED) {
-      const uint32_t tiles = (args.rows + 31u) / 32u;
-      const size_t first_chunk =
-          static_cast<size_t>(tile < tiles ? tile : tiles - 1u) * (K / kChunk);
-      weight_row[t] = args.tile[t].weights + first_chunk * 1024u + lane * 16u;
-      scale_row[t] = args.tile[t].scales +
-                     (first_chunk * 32u + n) * kScaleChunk;
+      const size_t first_chunk = static_cast<size_t>(safe_tile) * (K / kChunk);
+      weight_base[t] = args.tile[t].weights + first_chunk * weight_step;
+      scale_base[t] = args.tile[t].scales + first_chunk * scale_step;
+      weight_lane[t] = (g * h + tile_lane) * 16u;
+      scale_lane[t] = tile_lane * kScaleChunk;
     } else {
-      const uint32_t row = tile * 32u + n;
-      const uint32_t safe = row < args.rows ? row : args.rows - 1u;
-      weight_row[t] = args.tile[t].weights +
-                      static_cast<size_t>(safe) * row_bytes + g * 16u;
-      scale_row[t] =
-          args.tile[t].scales + static_cast<size_t>(safe) * scale_row_bytes;
+      const uint32_t first_row = safe_tile * h;
+      const uint32_t row = min(first_row + tile_lane, args.rows - 1u) - first_row;
+      weight_base[t] =
+          args.tile[t].weights + static_cast<size_t>(first_row) * row_bytes;
+      scale_base[t] =
+          args.tile[t].scales + static_cast<size_t>(first_row) * scale_row_bytes;
+      weight_lane[t] = row * row_bytes + g * 16u;
+      scale_lane[t] = row * scale_row_bytes;
     }
   }
   // activation piece this lane fetches per chunk: piece p = (block*2+half)*
   // BATCH + m  ->  act[m][chunk*64 + (block*2+half)*8 .. +8]
   const uint32_t piece = lane < PIECES ? lane : PIECES - 1u;
-  const uint16_t* activation_piece =
-      args.activations + static_cast<size_t>(piece % BATCH) * K +
-      (piece / BATCH) * 8u;
+  const uint32_t activation_lane =
+      ((piece % BATCH) * K + (piece / BATCH) * 8u) * 2u;
+  const uint8_t* activation_base =
+      reinterpret_cast<const uint8_t*>(args.activations);
 
-  float acc[TILES][4];
+  float acc[TILES][REGS];
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[t][i] = 0.0f;
+    for (int i = 0; i < REGS; ++i) acc[t][i] = 0.0f;
 
   const uint32_t chunks = K / kChunk;
   const uint32_t my_chunks =
@@ -174,22 +204,23 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   uint2 scales[PF][TILES];
   uint4 activation[PF];
   auto issue = [&](int slot, uint32_t index) {
-    const uint32_t chunk = wave + index * WAVES;
+    const uint32_t chunk = wave + index * WAVES;   // uniform
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      codes[slot][t] =
-          load_stream16(weight_row[t] + static_cast<size_t>(chunk) * weight_step);
+      codes[slot][t] = load_stream16(
+          weight_base[t] + static_cast<size_t>(chunk) * weight_step +
+          weight_lane[t]);
+      const uint8_t* scale_address =
+          scale_base[t] + static_cast<size_t>(chunk) * scale_step + scale_lane[t];
       if (SCHEME == kSchemeF16) {
-        scales[slot][t] =
-            load_stream8(scale_row[t] + static_cast<size_t>(chunk) * scale_step);
+        scales[slot][t] = load_stream8(scale_address);
       } else {
-        const uint32_t pair = *reinterpret_cast<const uint16_t*>(
-            scale_row[t] + static_cast<size_t>(chunk) * scale_step);
+        const uint32_t pair = *reinterpret_cast<const uint16_t*>(scale_address);
         scales[slot][t] = make_uint2(pair & 0xffu, pair >> 8);
       }
     }
-    activation[slot] =
-        *reinterpret_cast<const uint4*>(activation_piece + chunk * kChunk);
+    activation[slot] = *reinterpret_cast<const uint4*>(
+        activation_base + chunk * (kChunk * 2u) + activation_lane);
   };
 
   if (my_chunks) {
@@ -220,18 +251,23 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
         for (int b = 0; b < 4; ++b)
           a[b] = __builtin_bit_cast(bf16x8,
-                                    stage[(b * 2u + g) * BATCH + m_lane]);
+                                    stage[(b * 2u + g) * BATCH + batch_row]);
         __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
-          const auto s01 = __builtin_amdgcn_permlane32_swap(q[t].x, q[t].y,
-                                                            false, false);
-          const auto s23 = __builtin_amdgcn_permlane32_swap(q[t].z, q[t].w,
-                                                            false, false);
-          // block order inside the chunk: s01[0]=b0, s23[0]=b1, s01[1]=b2,
-          // s23[1]=b3
-          const uint32_t packed[4] = {s01[0], s23[0], s01[1], s23[1]};
+          uint32_t packed[4];  // half g of blocks 0..3 of row n
+          if (TILED) {
+            packed[0] = q[t].x; packed[1] = q[t].y;
+            packed[2] = q[t].z; packed[3] = q[t].w;
+          } else {
+            const auto s01 = __builtin_amdgcn_permlane32_swap(q[t].x, q[t].y,
+                                                              false, false);
+            const auto s23 = __builtin_amdgcn_permlane32_swap(q[t].z, q[t].w,
+                                                              false, false);
+            packed[0] = s01[0]; packed[1] = s23[0];
+            packed[2] = s01[1]; packed[3] = s23[1];
+          }
           float scale[4];
           float fold[4];
           if (SCHEME == kSchemeF16) {
@@ -259,7 +295,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
           for (int b = 0; b < 4; ++b)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < REGS; ++i)
               acc[t][i] = fmaf(d[b][i], scale[b], acc[t][i]);
         }
       }
@@ -270,19 +306,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) reduce[wave][t][i][lane] = acc[t][i];
+    for (int i = 0; i < REGS; ++i) reduce[wave][t][i][lane] = acc[t][i];
   __syncthreads();
 
-  const uint32_t items = (args.swiglu ? 1u : TILES) * 256u;
+  // item = (tile, register i, lane): lane (n, g) register i holds MFMA row
+  // 4*g + i, i.e. batch row (COMPACT ? 3 : 4)*g + i
+  const uint32_t items = (args.swiglu ? 1u : TILES) * REGS * 64u;
   for (uint32_t item = threadIdx.x; item < items; item += WAVES * 64u) {
-    const uint32_t t = item >> 8;
-    const uint32_t i = (item >> 6) & 3u;
+    const uint32_t t = item / (REGS * 64u);
+    const uint32_t i = (item / 64u) % REGS;
     const uint32_t source_lane = item & 63u;
-    const uint32_t m = 4u * (source_lane >> 5) + i;
+    const uint32_t m = (COMPACT ? 3u : 4u) * (source_lane >> 5) + i;
+    const uint32_t tile_row = source_lane & 31u;
     const uint32_t row =
-        args.swiglu ? blockIdx.x * 32u + (source_lane & 31u)
-                    : (blockIdx.x * TILES + t) * 32u + (source_lane & 31u);
-    if (m >= BATCH || row >= args.rows) continue;
+        (args.swiglu ? blockIdx.x : blockIdx.x * TILES + t) * h + tile_row;
+    if (m >= BATCH || tile_row >= h || row >= args.rows) continue;
     float total = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) total += reduce[w][t][i][source_lane];
@@ -295,6 +333,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       const float activated = bf16_round(total / (1.0f + __expf(-total)));
       static_cast<uint16_t*>(args.output)[index] =
           static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
+    } else if (args.segments) {
+      uint32_t local = row;
+      uint32_t segment = 0;
+      while (segment + 1u < args.segments && local >= args.segment_rows[segment]) {
+        local -= args.segment_rows[segment];
+        ++segment;
+      }
+      store_output(args.segment_output[segment], args.segment_kind[segment],
+                   static_cast<size_t>(m) * args.segment_rows[segment] + local,
+                   total);
     } else {
       if (args.residual) total += args.residual[index];
       store_output(args.output, args.output_kind, index, total);
@@ -391,109 +439,105 @@ bool matrix_ok(const qllm_fp4_matrix* m) {
          (m->scale_scheme == QLLM_SCALE_UE8M0_BLOCK32 ||
           m->scale_scheme == QLLM_SCALE_F16_BLOCK16) &&
          (m->layout == QLLM_LAYOUT_ROW_MAJOR ||
-          (m->layout == QLLM_LAYOUT_TILED && m->padded_columns % kChunk == 0u));
+          (m->layout == QLLM_LAYOUT_TILED && m->padded_columns % kChunk == 0u &&
+           (m->tile_rows == 0u || (m->tile_rows >= 8u && m->tile_rows <= 32u))));
 }
 
 template <int SCHEME, int BATCH, int TILES, bool TILED>
 int32_t launch_mfma_waves(const GemmArgs& args, uint32_t grid, uint32_t waves,
-                          size_t lds_bytes, hipStream_t stream) {
-  switch (waves) {
-    case 4:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4, TILED>
-          <<<grid, 256, lds_bytes, stream>>>(args);
-      break;
-    case 8:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8, TILED>
-          <<<grid, 512, lds_bytes, stream>>>(args);
-      break;
-    default:
-      fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 16, TILED>
-          <<<grid, 1024, lds_bytes, stream>>>(args);
-      break;
-  }
+                          hipStream_t stream) {
+  if (waves == 4u)
+    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4, TILED>
+        <<<grid, 256, 0, stream>>>(args);
+  else
+    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8, TILED>
+        <<<grid, 512, 0, stream>>>(args);
   return launched("FP4 MFMA GEMM");
 }
 
 template <int SCHEME, int TILES, bool TILED>
 int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
-                          uint32_t waves, size_t lds_bytes,
-                          hipStream_t stream) {
+                          uint32_t waves, hipStream_t stream) {
   switch (batch) {
-    case 1: return launch_mfma_waves<SCHEME, 1, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 2: return launch_mfma_waves<SCHEME, 2, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 3: return launch_mfma_waves<SCHEME, 3, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 4: return launch_mfma_waves<SCHEME, 4, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 5: return launch_mfma_waves<SCHEME, 5, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 6: return launch_mfma_waves<SCHEME, 6, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    case 7: return launch_mfma_waves<SCHEME, 7, TILES, TILED>(args, grid, waves, lds_bytes, stream);
-    default: return launch_mfma_waves<SCHEME, 8, TILES, TILED>(args, grid, waves, lds_bytes, stream);
+    case 1: return launch_mfma_waves<SCHEME, 1, TILES, TILED>(args, grid, waves, stream);
+    case 2: return launch_mfma_waves<SCHEME, 2, TILES, TILED>(args, grid, waves, stream);
+    case 3: return launch_mfma_waves<SCHEME, 3, TILES, TILED>(args, grid, waves, stream);
+    case 4: return launch_mfma_waves<SCHEME, 4, TILES, TILED>(args, grid, waves, stream);
+    case 5: return launch_mfma_waves<SCHEME, 5, TILES, TILED>(args, grid, waves, stream);
+    case 6: return launch_mfma_waves<SCHEME, 6, TILES, TILED>(args, grid, waves, stream);
+    case 7: return launch_mfma_waves<SCHEME, 7, TILES, TILED>(args, grid, waves, stream);
+    default: return launch_mfma_waves<SCHEME, 8, TILES, TILED>(args, grid, waves, stream);
   }
 }
 
-// One tile of 32 rows per workgroup (two for the fused gate/up pair); four
-// waves split K, eight when the matrix has too few tiles to fill 256 CUs.
-// Measured on MI355X: 16-wave groups lose to register pressure, two plain
-// tiles per group never beat one.
+// One tile per workgroup (a gate tile and its up tile for the fused SwiGLU
+// pair); four waves split K, eight when the matrix has few tiles.
 int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
                     bool swiglu, hipStream_t stream) {
-  const uint32_t tiles = (args.rows + 31u) / 32u;
-  uint32_t tiles_per_group = swiglu ? 2u : 1u;
-  uint32_t waves = tiles < 384u ? 8u : 4u;
-  if (const char* forced = getenv("QLLM_GEMM_WAVES")) waves = atoi(forced);
-  if (const char* forced = getenv("QLLM_GEMM_TILES"))
-    if (!swiglu) tiles_per_group = atoi(forced);
-  const uint32_t grid =
-      swiglu ? tiles : (tiles + tiles_per_group - 1u) / tiles_per_group;
+  const uint32_t tiles = (args.rows + args.tile_rows - 1u) / args.tile_rows;
+  const uint32_t waves = tiles <= 384u && !swiglu ? 8u : 4u;
   args.swiglu = swiglu ? 1u : 0u;
-  const size_t lds_bytes = 0;
-#define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                 \
-  return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, grid, waves, \
-                                                    lds_bytes, stream)
+#define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
+  return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
+                                                    stream)
   if (scheme == kSchemeF16) {
     if (tiled) {
-      if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeF16, 2, true);
+      if (swiglu) QLLM_LAUNCH(kSchemeF16, 2, true);
       QLLM_LAUNCH(kSchemeF16, 1, true);
     }
-    if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeF16, 2, false);
+    if (swiglu) QLLM_LAUNCH(kSchemeF16, 2, false);
     QLLM_LAUNCH(kSchemeF16, 1, false);
   }
   if (tiled) {
-    if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeUe8m0, 2, true);
+    if (swiglu) QLLM_LAUNCH(kSchemeUe8m0, 2, true);
     QLLM_LAUNCH(kSchemeUe8m0, 1, true);
   }
-  if (tiles_per_group == 2u) QLLM_LAUNCH(kSchemeUe8m0, 2, false);
+  if (swiglu) QLLM_LAUNCH(kSchemeUe8m0, 2, false);
   QLLM_LAUNCH(kSchemeUe8m0, 1, false);
 #undef QLLM_LAUNCH
 }
 
-// Row-major -> streaming layout.  Output piece p = (tile*chunks + chunk)*64 +
-// lane holds, for lane = half*32 + n, the 16 bytes of row 32*tile + n at byte
-// offset chunk*32 + half*16; rows past the matrix are zero.  Scales follow
-// per (tile, chunk) as 32 consecutive row entries of 4 binary16 / 2 UE8M0.
+uint32_t matrix_tile_rows(const qllm_fp4_matrix* matrix) {
+  if (matrix->layout == QLLM_LAYOUT_TILED)
+    return matrix->tile_rows ? matrix->tile_rows : 32u;
+  return 32u;  // row-major: any height works; full MFMA tiles are cheapest
+}
+
+// Row-major -> streaming layout with tiles of h rows.  The block of (tile,
+// chunk) holds 2*h pieces of 16 bytes, piece half*h + n = the four 4-byte
+// half-blocks of row h*tile + n at byte offsets chunk*32 + b*8 + half*4
+// (b = 0..3): exactly what lane (n, half) feeds to the four block MFMAs, and
+// one contiguous burst per wave-level load.  Rows past the matrix are zero.
+// Scales follow per (tile, chunk) as h consecutive row entries of 4 binary16 /
+// 2 UE8M0.
 __global__ void fp4_prepack_kernel(const uint8_t* weights,
                                    const uint8_t* scales, uint8_t* out_weights,
                                    uint8_t* out_scales, uint32_t rows,
                                    uint32_t padded_columns,
-                                   uint32_t scale_chunk_bytes) {
+                                   uint32_t scale_chunk_bytes, uint32_t h) {
   const uint32_t chunks = padded_columns / kChunk;
-  const uint32_t tiles = (rows + 31u) / 32u;
-  const size_t pieces = static_cast<size_t>(tiles) * chunks * 64u;
+  const uint32_t tiles = (rows + h - 1u) / h;
+  const size_t pieces = static_cast<size_t>(tiles) * chunks * 2u * h;
   const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
   for (size_t piece = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
        piece < pieces; piece += stride) {
-    const uint32_t lane = static_cast<uint32_t>(piece & 63u);
-    const size_t block = piece >> 6;
+    const uint32_t within = static_cast<uint32_t>(piece % (2u * h));
+    const size_t block = piece / (2u * h);
+    const uint32_t half = within / h;
+    const uint32_t n = within % h;
     const uint32_t chunk = static_cast<uint32_t>(block % chunks);
     const uint32_t tile = static_cast<uint32_t>(block / chunks);
-    const uint32_t row = tile * 32u + (lane & 31u);
+    const uint32_t row = tile * h + n;
     uint4 value = make_uint4(0u, 0u, 0u, 0u);
-    if (row < rows)
-      value = *reinterpret_cast<const uint4*>(
+    if (row < rows) {
+      const uint32_t* source = reinterpret_cast<const uint32_t*>(
           weights + static_cast<size_t>(row) * (padded_columns / 2u) +
-          chunk * 32u + (lane >> 5) * 16u);
+          chunk * 32u + half * 4u);
+      value = make_uint4(source[0], source[2], source[4], source[6]);
+    }
     *reinterpret_cast<uint4*>(out_weights + piece * 16u) = value;
-    if (lane < 32u) {
-      uint8_t* target = out_scales + (block * 32u + lane) * scale_chunk_bytes;
+    if (half == 0u) {
+      uint8_t* target = out_scales + (block * h + n) * scale_chunk_bytes;
       const uint8_t* source =
           scales + static_cast<size_t>(row) * (chunks * scale_chunk_bytes) +
           chunk * scale_chunk_bytes;
@@ -533,6 +577,7 @@ extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
     args.rows = matrix->rows;
     args.padded_columns = matrix->padded_columns;
     args.output_kind = output_kind;
+    args.tile_rows = matrix_tile_rows(matrix);
     return launch_mfma(args, static_cast<int>(matrix->scale_scheme),
                        matrix->layout == QLLM_LAYOUT_TILED, batch, false,
                        as_stream(stream));
@@ -555,6 +600,70 @@ extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
   return launched("FP4 BF16 GEMV");
 }
 
+extern "C" int32_t qllm_fp4_gemm_bf16_split(
+    const qllm_fp4_matrix* matrix, const void* input, size_t input_bytes,
+    const qllm_gemm_segment* segments, uint32_t segment_count, uint32_t batch,
+    void* stream) {
+  if (!matrix_ok(matrix) || !input || !segments || !segment_count ||
+      segment_count > 3u || !batch || batch > 8u ||
+      input_bytes < static_cast<size_t>(batch) * matrix->padded_columns * 2u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid split FP4 BF16 GEMM");
+  if (matrix->padded_columns % kChunk != 0u) {
+    // shapes the MFMA kernel does not take (row-major only): one plain call
+    // per segment on that segment's rows
+    const size_t row_bytes = matrix->padded_columns / 2u;
+    const size_t scale_row_bytes =
+        matrix->scale_scheme == QLLM_SCALE_F16_BLOCK16
+            ? matrix->padded_columns / 8u
+            : matrix->padded_columns / 32u;
+    uint64_t first_row = 0;
+    for (uint32_t s = 0; s < segment_count; ++s) {
+      if (!segments[s].rows || first_row + segments[s].rows > matrix->rows)
+        return fail(QLLM_INVALID_ARGUMENT, "invalid split FP4 BF16 GEMM segment");
+      qllm_fp4_matrix part = *matrix;
+      part.weights = matrix->weights + first_row * row_bytes;
+      part.scales =
+          static_cast<const uint8_t*>(matrix->scales) + first_row * scale_row_bytes;
+      part.rows = segments[s].rows;
+      const int32_t status =
+          qllm_fp4_gemm_bf16(&part, input, input_bytes, segments[s].output,
+                             segments[s].output_kind, nullptr, batch, stream);
+      if (status != QLLM_OK) return status;
+      first_row += segments[s].rows;
+    }
+    if (first_row != matrix->rows)
+      return fail(QLLM_INVALID_ARGUMENT,
+                  "split FP4 BF16 GEMM: segment rows do not add up to the matrix");
+    return QLLM_OK;
+  }
+  GemmArgs args{};
+  uint64_t total_rows = 0;
+  for (uint32_t s = 0; s < segment_count; ++s) {
+    if (!segments[s].output || !segments[s].rows ||
+        segments[s].output_kind > QLLM_OUT_BF16)
+      return fail(QLLM_INVALID_ARGUMENT, "invalid split FP4 BF16 GEMM segment");
+    args.segment_rows[s] = segments[s].rows;
+    args.segment_kind[s] = segments[s].output_kind;
+    args.segment_output[s] = segments[s].output;
+    total_rows += segments[s].rows;
+  }
+  if (total_rows != matrix->rows)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "split FP4 BF16 GEMM: segment rows do not add up to the matrix");
+  args.segments = segment_count;
+  args.tile[0] = {matrix->weights, static_cast<const uint8_t*>(matrix->scales)};
+  args.tile[1] = args.tile[0];
+  args.activations = static_cast<const uint16_t*>(input);
+  args.output = segments[0].output;
+  args.rows = matrix->rows;
+  args.padded_columns = matrix->padded_columns;
+  args.output_kind = segments[0].output_kind;
+  args.tile_rows = matrix_tile_rows(matrix);
+  return launch_mfma(args, static_cast<int>(matrix->scale_scheme),
+                     matrix->layout == QLLM_LAYOUT_TILED, batch, false,
+                     as_stream(stream));
+}
+
 extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
                                         const qllm_fp4_matrix* up,
                                         const void* input, size_t input_bytes,
@@ -563,6 +672,7 @@ extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
   if (!matrix_ok(gate) || !matrix_ok(up) || gate->rows != up->rows ||
       gate->padded_columns != up->padded_columns ||
       gate->scale_scheme != up->scale_scheme || gate->layout != up->layout ||
+      matrix_tile_rows(gate) != matrix_tile_rows(up) ||
       !input || !output || !batch ||
       batch > 8u || gate->padded_columns % kChunk != 0u ||
       input_bytes < static_cast<size_t>(batch) * gate->padded_columns * 2u)
@@ -575,6 +685,7 @@ extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
   args.rows = gate->rows;
   args.padded_columns = gate->padded_columns;
   args.output_kind = QLLM_OUT_BF16;
+  args.tile_rows = matrix_tile_rows(gate);
   return launch_mfma(args, static_cast<int>(gate->scale_scheme),
                      gate->layout == QLLM_LAYOUT_TILED, batch, true,
                      as_stream(stream));
@@ -598,41 +709,58 @@ extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
   return launched("FP4 Q8 weight-reuse GEMV");
 }
 
+// A tile costs the same matrix-core and conversion time whatever its height,
+// so full 32-row tiles are the default; shorter ones only pay off when a
+// matrix has too few rows to give every CU a tile.
+static uint32_t resolve_tile_rows(uint32_t, uint32_t tile_rows) {
+  return tile_rows ? tile_rows : 32u;
+}
+
 extern "C" size_t qllm_fp4_packed_weight_bytes(uint32_t rows,
-                                               uint32_t padded_columns) {
-  return static_cast<size_t>((rows + 31u) / 32u) * 32u * (padded_columns / 2u);
+                                               uint32_t padded_columns,
+                                               uint32_t tile_rows) {
+  if (!rows || tile_rows > 32u || (tile_rows && tile_rows < 8u)) return 0;
+  const uint32_t h = resolve_tile_rows(rows, tile_rows);
+  return static_cast<size_t>((rows + h - 1u) / h) * h * (padded_columns / 2u);
 }
 
 extern "C" size_t qllm_fp4_packed_scale_bytes(uint32_t rows,
                                               uint32_t padded_columns,
-                                              uint32_t scale_scheme) {
-  const size_t per_row = scale_scheme == QLLM_SCALE_F16_BLOCK16
-                             ? padded_columns / 8u
-                             : padded_columns / 32u;
-  return static_cast<size_t>((rows + 31u) / 32u) * 32u * per_row;
+                                              uint32_t scale_scheme,
+                                              uint32_t tile_rows) {
+  if (!rows || tile_rows > 32u || (tile_rows && tile_rows < 8u)) return 0;
+  const uint32_t h = resolve_tile_rows(rows, tile_rows);
+  const size_t padded_rows = static_cast<size_t>((rows + h - 1u) / h) * h;
+  return scale_scheme == QLLM_SCALE_F16_BLOCK16
+             ? padded_rows * (padded_columns / 16u) * 2u
+             : padded_rows * (padded_columns / 32u);
 }
 
 extern "C" int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source,
-                                    void* packed_weights, void* packed_scales,
+                                    uint32_t tile_rows, void* packed_weights,
+                                    void* packed_scales,
                                     qllm_fp4_matrix* packed, void* stream) {
   if (!matrix_ok(source) || source->layout != QLLM_LAYOUT_ROW_MAJOR ||
       source->padded_columns % kChunk != 0u || !packed_weights ||
-      !packed_scales || !packed)
+      !packed_scales || !packed || tile_rows > 32u ||
+      (tile_rows && tile_rows < 8u))
     return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 prepack");
-  const uint32_t scale_chunk_bytes =
+  const uint32_t h = resolve_tile_rows(source->rows, tile_rows);
+  const uint32_t scale_chunk =
       source->scale_scheme == QLLM_SCALE_F16_BLOCK16 ? 8u : 2u;
-  const size_t pieces = qllm_fp4_packed_weight_bytes(source->rows,
-                                                     source->padded_columns) / 16u;
-  const size_t blocks = (pieces + 255u) / 256u;
-  fp4_prepack_kernel<<<static_cast<unsigned>(blocks < 65536u ? blocks : 65536u),
-                       256, 0, as_stream(stream)>>>(
+  const size_t pieces =
+      qllm_fp4_packed_weight_bytes(source->rows, source->padded_columns, h) / 16u;
+  const uint32_t grid =
+      static_cast<uint32_t>(pieces / 256u < 16384u ? pieces / 256u + 1u : 16384u);
+  fp4_prepack_kernel<<<grid, 256, 0, as_stream(stream)>>>(
       source->weights, static_cast<const uint8_t*>(source->scales),
       static_cast<uint8_t*>(packed_weights),
       static_cast<uint8_t*>(packed_scales), source->rows,
-      source->padded_columns, scale_chunk_bytes);
+      source->padded_columns, scale_chunk, h);
   *packed = *source;
   packed->weights = static_cast<const uint8_t*>(packed_weights);
   packed->scales = packed_scales;
   packed->layout = QLLM_LAYOUT_TILED;
+  packed->tile_rows = h;
   return launched("FP4 prepack");
 }

@@ -304,14 +304,16 @@ DeviceFp4Matrix Mi355DenseFp4Provider::upload_matrix(
   if (tiled && padded % 64U == 0U) {
     void* packed_codes{};
     void* packed_scales{};
-    hip_check(hipMalloc(&packed_codes, qllm_fp4_packed_weight_bytes(rows, padded)),
+    // tile height 0: full 32-row tiles
+    hip_check(hipMalloc(&packed_codes,
+                        qllm_fp4_packed_weight_bytes(rows, padded, 0U)),
               "allocate tiled FP4 weights");
     hip_check(hipMalloc(&packed_scales,
                         qllm_fp4_packed_scale_bytes(
-                            rows, padded, matrix.descriptor.scale_scheme)),
+                            rows, padded, matrix.descriptor.scale_scheme, 0U)),
               "allocate tiled FP4 scales");
     qllm_fp4_matrix packed{};
-    status_check(qllm_fp4_prepack(&matrix.descriptor, packed_codes,
+    status_check(qllm_fp4_prepack(&matrix.descriptor, 0U, packed_codes,
                                   packed_scales, &packed, stream_));
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
               "prepack FP4 weights");
@@ -327,6 +329,78 @@ DeviceFp4Matrix Mi355DenseFp4Provider::upload_matrix(
   allocations_.push_back(staged_scales);
   weight_bytes_ += code_bytes + scale_bytes;
   return matrix;
+}
+
+DeviceFp4Matrix Mi355DenseFp4Provider::concatenate_rows(
+    std::vector<DeviceFp4Matrix> parts) {
+  const qllm_fp4_matrix& first = parts.front().descriptor;
+  std::uint32_t rows = 0;
+  for (const auto& part : parts) {
+    const qllm_fp4_matrix& d = part.descriptor;
+    if (d.layout != QLLM_LAYOUT_ROW_MAJOR || d.columns != first.columns ||
+        d.padded_columns != first.padded_columns ||
+        d.scale_scheme != first.scale_scheme)
+      throw std::runtime_error("projections cannot be stored as one matrix");
+    rows += d.rows;
+  }
+  const std::uint32_t padded = first.padded_columns;
+  const bool block16 = first.scale_scheme == QLLM_SCALE_F16_BLOCK16;
+  const std::size_t row_code_bytes = padded / 2U;
+  const std::size_t row_scale_bytes =
+      block16 ? std::size_t{padded / 16U} * 2U : padded / 32U;
+  void* codes{};
+  void* scales{};
+  hip_check(hipMalloc(&codes, rows * row_code_bytes), "allocate joined weights");
+  hip_check(hipMalloc(&scales, rows * row_scale_bytes), "allocate joined scales");
+  std::size_t row = 0;
+  for (const auto& part : parts) {
+    const std::uint32_t part_rows = part.descriptor.rows;
+    hip_check(hipMemcpy(static_cast<std::uint8_t*>(codes) + row * row_code_bytes,
+                        part.weights, part_rows * row_code_bytes,
+                        hipMemcpyDeviceToDevice),
+              "join weights");
+    hip_check(hipMemcpy(static_cast<std::uint8_t*>(scales) + row * row_scale_bytes,
+                        part.scales, part_rows * row_scale_bytes,
+                        hipMemcpyDeviceToDevice),
+              "join scales");
+    row += part_rows;
+    for (void* pointer : {part.weights, part.scales}) {
+      allocations_.erase(
+          std::find(allocations_.begin(), allocations_.end(), pointer));
+      (void)hipFree(pointer);
+    }
+  }
+  DeviceFp4Matrix joined;
+  joined.descriptor = first;
+  joined.descriptor.weights = static_cast<const std::uint8_t*>(codes);
+  joined.descriptor.scales = scales;
+  joined.descriptor.rows = rows;
+  if (padded % 64U == 0U) {
+    void* packed_codes{};
+    void* packed_scales{};
+    hip_check(hipMalloc(&packed_codes,
+                        qllm_fp4_packed_weight_bytes(rows, padded, 0U)),
+              "allocate tiled FP4 weights");
+    hip_check(hipMalloc(&packed_scales,
+                        qllm_fp4_packed_scale_bytes(rows, padded,
+                                                    first.scale_scheme, 0U)),
+              "allocate tiled FP4 scales");
+    qllm_fp4_matrix packed{};
+    status_check(qllm_fp4_prepack(&joined.descriptor, 0U, packed_codes,
+                                  packed_scales, &packed, stream_));
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "prepack joined FP4 weights");
+    (void)hipFree(codes);
+    (void)hipFree(scales);
+    joined.descriptor = packed;
+    codes = packed_codes;
+    scales = packed_scales;
+  }
+  joined.weights = codes;
+  joined.scales = scales;
+  allocations_.push_back(codes);
+  allocations_.push_back(scales);
+  return joined;
 }
 
 float* Mi355DenseFp4Provider::upload_f32(const er::ImmutableModelTensor& tensor,
@@ -374,19 +448,20 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
       auto& layer = layers_[attention_ops_];
       layer.input_norm =
           upload_f32(tensor_for(context.tensors, "input_norm"), g_.hidden);
-      layer.query = upload_matrix(
-          tensor_for(context.tensors, "query_projection"), true);
-      layer.key =
-          upload_matrix(tensor_for(context.tensors, "key_projection"), true);
-      layer.value =
-          upload_matrix(tensor_for(context.tensors, "value_projection"), true);
+      DeviceFp4Matrix query = upload_matrix(
+          tensor_for(context.tensors, "query_projection"), false);
+      DeviceFp4Matrix key =
+          upload_matrix(tensor_for(context.tensors, "key_projection"), false);
+      DeviceFp4Matrix value =
+          upload_matrix(tensor_for(context.tensors, "value_projection"), false);
       layer.output = upload_matrix(
           tensor_for(context.tensors, "output_projection"), true);
-      require_shape(layer.query, query_rows, g_.hidden, "query_projection");
-      require_shape(layer.key, g_.kv_heads * g_.head_dim, g_.hidden,
+      require_shape(query, query_rows, g_.hidden, "query_projection");
+      require_shape(key, g_.kv_heads * g_.head_dim, g_.hidden,
                     "key_projection");
-      require_shape(layer.value, g_.kv_heads * g_.head_dim, g_.hidden,
+      require_shape(value, g_.kv_heads * g_.head_dim, g_.hidden,
                     "value_projection");
+      layer.qkv = concatenate_rows({query, key, value});
       require_shape(layer.output, g_.hidden, g_.query_heads * g_.head_dim,
                     "output_projection");
       if (g_.qk_norm) {
@@ -534,15 +609,15 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                      normalized_, g_.hidden, rows, g_.hidden,
                                      g_.norm_epsilon, g_.zero_centered_norm,
                                      stream));
-    status_check(qllm_fp4_gemm_bf16(&layer.query.descriptor, normalized_,
-                                    hidden_bytes, query_, QLLM_OUT_F32, nullptr,
-                                    rows, stream));
-    status_check(qllm_fp4_gemm_bf16(&layer.key.descriptor, normalized_,
-                                    hidden_bytes, key_, QLLM_OUT_F32, nullptr,
-                                    rows, stream));
-    status_check(qllm_fp4_gemm_bf16(&layer.value.descriptor, normalized_,
-                                    hidden_bytes, value_, QLLM_OUT_F32, nullptr,
-                                    rows, stream));
+    // query, key and value projections (:7004-7011) in one launch
+    const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+    const qllm_gemm_segment projections[3] = {
+        {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+        {key_, kv_rows, QLLM_OUT_F32},
+        {value_, kv_rows, QLLM_OUT_F32}};
+    status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
+                                          hidden_bytes, projections, 3U, rows,
+                                          stream));
     if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
       if (deferred_positions)
         status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
@@ -983,7 +1058,11 @@ DeviceFp4Matrix Mi355DenseFp4Provider::synthetic_matrix(std::uint32_t rows,
   const bool block16 = g_.scale_scheme == QLLM_SCALE_F16_BLOCK16;
   // the row-major and the tiled layout hold the same multiset of bytes per
   // matrix; a random-init model may be generated in either directly
-  const std::size_t padded_rows = tiled ? (rows + 31U) / 32U * 32U : rows;
+  const bool use_tiles = tiled && padded % 64U == 0U;
+  const std::uint32_t tile_rows = use_tiles ? 32U : 0U;
+  const std::size_t padded_rows =
+      use_tiles ? std::size_t{(rows + tile_rows - 1U) / tile_rows} * tile_rows
+                : rows;
   const std::size_t code_bytes = padded_rows * padded / 2U;
   const std::size_t scale_count = padded_rows * (padded / (block16 ? 16U : 32U));
   const std::size_t scale_bytes = scale_count * (block16 ? 2U : 1U);
@@ -1005,10 +1084,9 @@ DeviceFp4Matrix Mi355DenseFp4Provider::synthetic_matrix(std::uint32_t rows,
                        columns,
                        padded,
                        g_.scale_scheme,
-                       tiled && padded % 64U == 0U
-                           ? std::uint32_t{QLLM_LAYOUT_TILED}
-                           : std::uint32_t{QLLM_LAYOUT_ROW_MAJOR},
-                       0U};
+                       use_tiles ? std::uint32_t{QLLM_LAYOUT_TILED}
+                                 : std::uint32_t{QLLM_LAYOUT_ROW_MAJOR},
+                       tile_rows};
   weight_bytes_ += std::uint64_t{rows} * padded / 2U +
                    std::uint64_t{rows} * (padded / (block16 ? 16U : 32U)) *
                        (block16 ? 2U : 1U);
@@ -1044,11 +1122,9 @@ er::Status Mi355DenseFp4Provider::load_synthetic_weights(std::uint64_t seed) {
         layer.query_norm = ones(g_.head_dim, 0.0F);
         layer.key_norm = ones(g_.head_dim, 0.0F);
       }
-      layer.query = synthetic_matrix(query_rows, g_.hidden, next_seed(), true);
-      layer.key = synthetic_matrix(g_.kv_heads * g_.head_dim, g_.hidden,
-                                   next_seed(), true);
-      layer.value = synthetic_matrix(g_.kv_heads * g_.head_dim, g_.hidden,
-                                     next_seed(), true);
+      layer.qkv =
+          synthetic_matrix(query_rows + 2U * g_.kv_heads * g_.head_dim,
+                           g_.hidden, next_seed(), true);
       layer.output = synthetic_matrix(g_.hidden, g_.query_heads * g_.head_dim,
                                       next_seed(), true);
       layer.gate = synthetic_matrix(g_.intermediate, g_.hidden, next_seed(), true);

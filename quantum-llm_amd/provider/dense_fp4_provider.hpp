@@ -73,7 +73,9 @@ struct LayerWeights final {
   float* post_attention_norm{};
   float* query_norm{};
   float* key_norm{};
-  DeviceFp4Matrix query, key, value, output, gate, up, down;
+  // query, key and value rows concatenated: one streaming matrix, one launch
+  DeviceFp4Matrix qkv;
+  DeviceFp4Matrix output, gate, up, down;
 };
 
 class Mi355DenseFp4Provider final : public er::IOperationProvider {
@@ -162,6 +164,9 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void ensure_pages(std::uint32_t last_position);
   DeviceFp4Matrix upload_matrix(const er::ImmutableModelTensor& tensor,
                                 bool tiled);
+  // One tiled matrix holding the rows of the given row-major matrices in
+  // order (same columns and scale scheme); the parts are released.
+  DeviceFp4Matrix concatenate_rows(std::vector<DeviceFp4Matrix> parts);
   float* upload_f32(const er::ImmutableModelTensor& tensor,
                     std::uint32_t elements);
   DeviceFp4Matrix synthetic_matrix(std::uint32_t rows, std::uint32_t columns,

@@ -34,7 +34,7 @@ class Fp4Matrix(Structure):
     _fields_ = [("weights", c_void_p), ("scales", c_void_p),
                 ("rows", c_uint32), ("columns", c_uint32),
                 ("padded_columns", c_uint32), ("scale_scheme", c_uint32),
-                ("layout", c_uint32), ("reserved", c_uint32)]
+                ("layout", c_uint32), ("tile_rows", c_uint32)]
 
 
 class Q4hAttentionLaunch(Structure):
@@ -72,10 +72,11 @@ SIGNATURES = {
     "qllm_convert_f32_to_bf16_batch": (c_int32, [c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_gemv_q8_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_fp4_gemm_bf16": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_bf16_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_swiglu_bf16": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
-    "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32]),
-    "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
-    "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
+    "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
+    "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32, c_uint32]),
+    "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
     "qllm_fp4_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_uint32, c_void_p]),
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
@@ -96,6 +97,11 @@ SIGNATURES = {
     "qllm_apply_presence_penalty": (c_int32, [c_void_p, c_void_p, c_uint32, c_float, c_void_p]),
     "qllm_fill_random": (c_int32, [c_void_p, c_size_t, c_uint32, c_uint64, c_void_p]),
 }
+
+class GemmSegment(ctypes.Structure):
+    """Mirror of qllm_gemm_segment."""
+    _fields_ = [("output", c_void_p), ("rows", c_uint32), ("output_kind", c_uint32)]
+
 
 _STATUS_FUNCTIONS = {name for name, (restype, _) in SIGNATURES.items()
                      if restype is c_int32}
@@ -138,16 +144,17 @@ def fp4_matrix(weights, scales, rows, columns, padded_columns, scheme) -> Fp4Mat
                      scheme, 0, 0)
 
 
-def prepack(matrix: Fp4Matrix, device):
-    """Tiled device copy of a row-major matrix: (descriptor, keepalive)."""
+def prepack(matrix: Fp4Matrix, device, tile_rows=0):
+    """Tiled device copy of a row-major matrix: (descriptor, keepalive).
+    tile_rows 0 = full 32-row tiles."""
     import torch
     weight_bytes = call("qllm_fp4_packed_weight_bytes", matrix.rows,
-                        matrix.padded_columns)
+                        matrix.padded_columns, tile_rows)
     scale_bytes = call("qllm_fp4_packed_scale_bytes", matrix.rows,
-                       matrix.padded_columns, matrix.scale_scheme)
+                       matrix.padded_columns, matrix.scale_scheme, tile_rows)
     weights = torch.empty(weight_bytes, dtype=torch.uint8, device=device)
     scales = torch.empty(scale_bytes, dtype=torch.uint8, device=device)
     packed = Fp4Matrix()
-    call("qllm_fp4_prepack", ctypes.byref(matrix), ptr(weights), ptr(scales),
+    call("qllm_fp4_prepack", ctypes.byref(matrix), tile_rows, ptr(weights), ptr(scales),
          ctypes.byref(packed), None)
     return packed, (weights, scales)

@@ -26,8 +26,9 @@ def assert_close(got, want, rtol=RTOL, atol=ATOL, what=""):
 
 
 def gemm(device, codes, scales, scheme, rows, padded, act_bf16_values, *,
-         tiled=True, out_kind=qh.OUT_F32, residual=None):
-    """qllm_fp4_gemm_bf16 on host numpy inputs; returns a numpy array."""
+         tiled=True, out_kind=qh.OUT_F32, residual=None, tile_rows=0):
+    """qllm_fp4_gemm_bf16 on host numpy inputs; returns a numpy array.
+    tile_rows 0 = full 32-row tiles."""
     batch = act_bf16_values.shape[0]
     d_codes = device_tensor(codes, device)
     d_scales = device_tensor(scales, device)
@@ -35,7 +36,7 @@ def gemm(device, codes, scales, scheme, rows, padded, act_bf16_values, *,
     matrix = qh.fp4_matrix(d_codes, d_scales, rows, padded, padded, scheme)
     keep = None
     if tiled:
-        matrix, keep = qh.prepack(matrix, device)
+        matrix, keep = qh.prepack(matrix, device, tile_rows)
     dtype = torch.bfloat16 if out_kind == qh.OUT_BF16 else torch.float32
     out = torch.zeros((batch, rows), dtype=dtype, device=device)
     d_residual = None if residual is None else device_tensor(residual, device)

@@ -28,6 +28,63 @@ def test_gemm_matches_oracle(device, scheme, rows, padded, batch):
         assert np.array_equal(tiled, row_major)
 
 
+@pytest.mark.parametrize("tile_rows", [8, 20, 23, 32])
+@pytest.mark.parametrize("rows,padded,batch", [(333, 5120, 5), (2000, 1024, 6),
+                                               (40, 128, 7)])
+def test_gemm_tile_heights(device, tile_rows, rows, padded, batch):
+    """Every tile height of the streaming layout (partial last tile included)
+    computes the same rows; only the summation order over K may differ."""
+    rng = np.random.default_rng(rows + tile_rows)
+    scheme = ol.SCALE_F16_BLOCK16
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
+    got = gu.gemm(device, codes, scales, scheme, rows, padded, act,
+                  tile_rows=tile_rows)
+    gu.assert_close(got, want, what=f"tile height {tile_rows}")
+
+
+@pytest.mark.parametrize("padded,tiled", [(5120, True), (5120, False), (96, False)])
+def test_split_gemm_equals_separate_calls(device, padded, tiled):
+    """q, k and v stored as one matrix: each output segment carries exactly the
+    bits of a separate call on that projection."""
+    import ctypes
+    rng = np.random.default_rng(padded + tiled)
+    scheme, batch, parts = ol.SCALE_F16_BLOCK16, 5, (256, 64, 72)
+    rows = sum(parts)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    matrix = qh.fp4_matrix(d_codes, d_scales, rows, padded, padded, scheme)
+    if tiled:
+        matrix, keep = qh.prepack(matrix, device)
+    outputs = [torch.zeros((batch, part), device=device) for part in parts]
+    segments = (qh.GemmSegment * 3)(*[
+        qh.GemmSegment(qh.ptr(out), part, qh.OUT_F32)
+        for out, part in zip(outputs, parts)])
+    qh.call("qllm_fp4_gemm_bf16_split", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            ctypes.cast(segments, ctypes.c_void_p), 3, batch, None)
+    torch.cuda.synchronize()
+    first = 0
+    for out, part in zip(outputs, parts):
+        separate = gu.gemm(device, codes[first:first + part], scales[first:first + part],
+                           scheme, part, padded, act, tiled=tiled and padded % 64 == 0)
+        got = out.cpu().numpy()
+        want = ol.fp4_linear_f64(codes[first:first + part], scales[first:first + part],
+                                 scheme, part, padded, act)
+        gu.assert_close(got, want, what="split segment")
+        if padded % 64:
+            assert np.array_equal(got, separate)
+        else:   # K is split over four or eight waves depending on the tile count
+            assert np.abs(got - separate).max() <= 2e-5 * np.abs(want).max()
+        first += part
+    with pytest.raises(qh.QllmError):
+        segments[2].rows += 1
+        qh.call("qllm_fp4_gemm_bf16_split", matrix, qh.ptr(d_act), d_act.numel() * 2,
+                ctypes.cast(segments, ctypes.c_void_p), 3, batch, None)
+
+
 def test_gemm_config1_shape_and_output_kinds(device):
     """BASELINE config 1: [17408, 5120], M=5, binary16 scale per 16, bf16 out."""
     rng = np.random.default_rng(1)
