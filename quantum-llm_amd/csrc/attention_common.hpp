@@ -1,0 +1,186 @@
+// Pieces shared by the paged decode-attention split kernels (Q4H and exact
+// F16 caches): lane-group reductions, the scalar page-table fetch, and the
+// merge of a workgroup's eight wave states into one split partial.
+#pragma once
+
+#include "common.hpp"
+
+namespace qllm {
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kSplitWaves = 8;
+constexpr float kMaskedMax = -1.0e30f;
+
+// max over the lanes {l, l^16, l^32, l^48}
+__device__ __forceinline__ float quad_row_max(float value) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  value = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+__device__ __forceinline__ float quad_row_sum(float value) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  value = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
+                                            __float_as_uint(value), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// Page table entry at a wave-uniform index, fetched with a scalar load (the
+// table is never written while attention kernels run), so everything derived
+// from the page address stays in scalar registers.
+__device__ __forceinline__ const void* uniform_page(
+    const void* const* page_table, uint32_t index) {
+  typedef const void* __attribute__((address_space(4))) const* constant_table;
+  return ((constant_table)page_table)[index];
+}
+
+// Tiles [first, last) of the context that wave `wave` of split `split` walks.
+// split_tokens == 0: balanced - the context's tiles are dealt evenly over
+// every wave of the grid row, whatever the context length.  Otherwise split
+// s covers tokens [s*split_tokens, (s+1)*split_tokens) and its tiles are dealt
+// evenly over the workgroup's waves.
+__device__ __forceinline__ void wave_tile_range(uint32_t context_tiles,
+                                                uint32_t tile_tokens,
+                                                uint32_t split_tokens,
+                                                uint32_t split, uint32_t splits,
+                                                uint32_t wave,
+                                                uint32_t& tile_first,
+                                                uint32_t& tile_last) {
+  if (split_tokens == 0u) {
+    const uint32_t slots = splits * kSplitWaves;
+    const uint32_t slot = split * kSplitWaves + wave;
+    tile_first = static_cast<uint32_t>(
+        static_cast<uint64_t>(slot) * context_tiles / slots);
+    tile_last = static_cast<uint32_t>(
+        static_cast<uint64_t>(slot + 1u) * context_tiles / slots);
+  } else {
+    const uint32_t split_tiles = split_tokens / tile_tokens;
+    const uint32_t begin = min(split * split_tiles, context_tiles);
+    const uint32_t count = min(begin + split_tiles, context_tiles) - begin;
+    tile_first = begin + wave * count / kSplitWaves;
+    tile_last = begin + (wave + 1u) * count / kSplitWaves;
+  }
+}
+
+struct PartialTarget {
+  float* partial_maxima;   // [rows, maximum_splits, query_heads]
+  float* partial_sums;     // same
+  float* partial_outputs;  // [rows, maximum_splits, query_heads, D]
+  uint32_t maximum_splits;
+  uint32_t query_heads;
+  uint32_t kv_head;
+  uint32_t split;
+  uint32_t group;          // query heads per KV head
+  uint32_t matrix_rows;    // rows * group
+};
+
+// Merges the eight wave states of a workgroup and writes the split partial.
+// A wave's state: per row tile rt (16 matrix rows; lane (col = lane%16, quad =
+// lane/16) owns matrix row 16*rt + col) the running maximum (log2 units) and
+// sum, and out[dt][rt] = O^T elements d = 16*dt + 4*quad .. +3 of that row.
+//  1. every wave publishes its (max, sum) per row; all waves derive the
+//     merged maximum and bring their own accumulators to it.
+//  2. the accumulators are summed reduce-scatter style, eight 1 KiB register
+//     vectors (one per receiving wave) at a time: each wave drops the eight
+//     vectors of the group into LDS, lane-linear (no bank conflicts), and
+//     wave v adds up vector v of all eight waves in a fixed order.  Wave v
+//     ends up owning vectors v, v+8, ... of the result and writes them out.
+// `pool` needs 64 KiB of LDS, `summary` 512*RT bytes per wave; both may
+// overlap whatever the tile loop used (the function starts with a barrier).
+template <int D, int RT>
+__device__ __forceinline__ void merge_wave_states(
+    float (&running_max)[RT], float (&running_sum)[RT],
+    f32x4 (&out)[D / 16][RT], float* pool, float2* summary, uint32_t wave,
+    uint32_t lane, const PartialTarget& target) {
+  constexpr int DT = D / 16;
+  constexpr int VECTORS = DT * RT;   // f32x4 accumulator vectors per wave
+  static_assert(VECTORS % kSplitWaves == 0, "vectors are dealt to 8 waves");
+  const uint32_t col = lane & 15u;
+  const uint32_t quad = lane >> 4;
+  __syncthreads();  // tiles done: the LDS they used is free
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+    summary[(wave * RT + rt) * 64 + lane] =
+        make_float2(running_max[rt], running_sum[rt]);
+  __syncthreads();
+  float merged_max[RT], merged_sum[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float2 part[kSplitWaves];
+    float maximum = kMaskedMax;
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w) {
+      part[w] = summary[(w * RT + rt) * 64 + lane];
+      maximum = fmaxf(maximum, part[w].x);
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w)
+      sum = fmaf(part[w].y, __builtin_amdgcn_exp2f(part[w].x - maximum), sum);
+    const float factor = __builtin_amdgcn_exp2f(running_max[rt] - maximum);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+    merged_max[rt] = maximum;
+    merged_sum[rt] = sum;
+  }
+  f32x4 merged[VECTORS / kSplitWaves];
+#pragma unroll
+  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
+#pragma unroll
+    for (int v = 0; v < kSplitWaves; ++v) {
+      const int k = group_index * kSplitWaves + v;
+      *reinterpret_cast<f32x4*>(pool + ((wave * kSplitWaves + v) * 64 + lane) * 4u) =
+          out[k / RT][k % RT];
+    }
+    __syncthreads();
+    f32x4 total = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int w = 0; w < kSplitWaves; ++w)
+      total += *reinterpret_cast<const f32x4*>(
+          pool + ((w * kSplitWaves + wave) * 64 + lane) * 4u);
+    merged[group_index] = total;
+    __syncthreads();
+  }
+
+  // partials: wave v writes the vectors it owns, wave 0 also max and sum
+#pragma unroll
+  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
+    const uint32_t k = group_index * kSplitWaves + wave;
+    const uint32_t dt = k / RT;
+    const uint32_t rt = k % RT;
+    const uint32_t matrix_row = 16u * rt + col;
+    if (matrix_row >= target.matrix_rows) continue;
+    const uint32_t row = matrix_row / target.group;
+    const uint32_t head = target.kv_head * target.group + matrix_row % target.group;
+    const size_t partial =
+        (static_cast<size_t>(row) * target.maximum_splits + target.split) *
+            target.query_heads + head;
+    *reinterpret_cast<f32x4*>(target.partial_outputs + partial * D + 16u * dt +
+                              4u * quad) = merged[group_index];
+  }
+  if (wave != 0u || quad != 0u) return;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const uint32_t matrix_row = 16u * rt + col;
+    if (matrix_row >= target.matrix_rows) continue;
+    const uint32_t row = matrix_row / target.group;
+    const uint32_t head = target.kv_head * target.group + matrix_row % target.group;
+    const size_t partial =
+        (static_cast<size_t>(row) * target.maximum_splits + target.split) *
+            target.query_heads + head;
+    target.partial_maxima[partial] = merged_max[rt];
+    target.partial_sums[partial] = merged_sum[rt];
+  }
+}
+
+}  // namespace qllm

@@ -1,6 +1,17 @@
 // Exact-F16 paged KV cache: K/V store and decode attention.
-// (attention kernel follows; this first part is the page store)
-#include "common.hpp"
+//
+// Replaces, from runtime/src/cuda/transformer_kernels.cu of the reference:
+//   store_gqa_kv_fp16_to_paged                                  :4208
+//   gated_gqa_attention_staged_fp16_impl and its kernels        :10214-10476,
+//                                                               :6517-6665, :7023-7057
+// The reference walks its context splits one after the other and keeps one
+// running softmax state; here the splits run in parallel, each workgroup
+// leaves an (max, sum, unnormalised output) partial and the split combine
+// shared with the Q4H path merges them.  Arithmetic follows the reference:
+// the query is rounded to binary16, scores are F32 sums of binary16
+// products, probabilities are rounded to binary16 before they weigh V and
+// before they enter the denominator.
+#include "attention_common.hpp"
 
 namespace qllm {
 namespace {
@@ -30,7 +41,300 @@ __global__ void f16_store_kernel(const float* key, const float* value,
       static_cast<uint16_t>(f32_to_f16_bits(value[source]));
 }
 
+
+struct F16SplitArgs {
+  const float* query;
+  uint32_t query_stride;
+  const void* const* pages;
+  float* partial_maxima;
+  float* partial_sums;
+  float* partial_outputs;
+  uint32_t first_context_tokens;
+  uint32_t rows;
+  uint32_t layer;
+  uint32_t page_tokens;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t split_tokens;
+  uint32_t maximum_splits;
+};
+
+constexpr uint32_t kF16Tile = 32;  // tokens per wave step
+
+// One workgroup (8 waves) per (kv head, context split); a wave walks 32-token
+// tiles with its own online-softmax state:
+//   scores  S[tok][row] = K . Q     v_mfma_f32_16x16x32_f16; K rows come
+//           straight from the page as A operands (16 bytes per lane), the
+//           binary16 query sits in LDS in B-operand order
+//   output  O^T[d][row] += V^T . P^T   v_mfma_f32_16x16x16_f16; the V tile is
+//           staged in LDS, rows swizzled so that the transposing read
+//           (ds_read_b64_tr_b16: 4 tokens x 16 dims per lane group) is free
+//           of bank conflicts, and the score registers of a 16-token sub-tile
+//           are already the B operand.
+// D = head_dim (128 or 256), RT = 16-row tiles of rows*group query rows.
+template <int D, int RT>
+__global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
+    const F16SplitArgs args) {
+  constexpr int KSTEPS = D / 32;  // k-steps of the score MFMA over head_dim
+  constexpr int DT = D / 16;      // 16-wide tiles of head_dim
+  constexpr int GR = D / 8;       // 16-byte granules per V row
+  constexpr int STAGE = kF16Tile * D * 2;  // V tile of a wave (bytes)
+  constexpr int UNITS = RT * KSTEPS;       // query operands of 1 KiB
+  constexpr int POOL = kSplitWaves * kSplitWaves * 1024;  // merge needs 64 KiB
+  constexpr int EXCHANGE_Q = UNITS * 1024 + RT * 64;
+  constexpr int EXCHANGE_MERGE = kSplitWaves * RT * 512;
+  __shared__ __attribute__((aligned(16)))
+  uint8_t stage[kSplitWaves * STAGE > POOL ? kSplitWaves * STAGE : POOL];
+  __shared__ __attribute__((aligned(16)))
+  uint8_t exchange[EXCHANGE_Q > EXCHANGE_MERGE ? EXCHANGE_Q : EXCHANGE_MERGE];
+
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t col = lane & 15u;
+  const uint32_t quad = lane >> 4;
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t split = blockIdx.y;
+  const uint32_t group = args.query_heads / args.kv_heads;
+  const uint32_t matrix_rows = args.rows * group;
+  const uint32_t first_context_tokens = args.first_context_tokens;
+  const uint32_t last_context = first_context_tokens + args.rows - 1u;
+  const uint32_t context_tiles = (last_context + kF16Tile - 1u) / kF16Tile;
+  uint32_t tile_first, tile_last;
+  wave_tile_range(context_tiles, kF16Tile, args.split_tokens, split, gridDim.y,
+                  wave, tile_first, tile_last);
+
+  // ---- query operands (B side of S = K.Q) in binary16, built once -------------
+  uint32_t* exchange_limit = reinterpret_cast<uint32_t*>(exchange + UNITS * 1024);
+  for (uint32_t unit = wave; unit < static_cast<uint32_t>(UNITS);
+       unit += kSplitWaves) {
+    const uint32_t rt = unit / KSTEPS;
+    const uint32_t step = unit % KSTEPS;
+    const uint32_t matrix_row = 16u * rt + col;
+    const bool valid = matrix_row < matrix_rows;
+    const uint32_t row = valid ? matrix_row / group : 0u;
+    const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
+    const float* source =
+        args.query +
+        (static_cast<size_t>(row) * args.query_heads + head) * args.query_stride +
+        32u * step + 8u * quad;
+    f16x8 operand;
+#pragma unroll
+    for (int piece = 0; piece < 2; ++piece) {
+      float4 loaded = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (valid) loaded = *reinterpret_cast<const float4*>(source + 4 * piece);
+      operand[4 * piece + 0] = static_cast<_Float16>(loaded.x);
+      operand[4 * piece + 1] = static_cast<_Float16>(loaded.y);
+      operand[4 * piece + 2] = static_cast<_Float16>(loaded.z);
+      operand[4 * piece + 3] = static_cast<_Float16>(loaded.w);
+    }
+    *reinterpret_cast<f16x8*>(exchange + unit * 1024u + lane * 16u) = operand;
+    if (step == 0u && quad == 0u)
+      exchange_limit[16u * rt + col] = first_context_tokens + row;
+  }
+  __syncthreads();
+  const uint8_t* q_operands = exchange + lane * 16u;
+  const float score_unit =
+      1.4426950408889634f / sqrtf(static_cast<float>(D));  // log2 units
+
+  // ---- page geometry ------------------------------------------------------------
+  const size_t page_values =
+      static_cast<size_t>(args.page_tokens) * args.kv_heads * D;
+  const size_t layer_offset = static_cast<size_t>(args.layer) * 2u * page_values;
+  const uint32_t row_stride = args.kv_heads * D;  // halves between tokens
+  uint8_t* stage_v = stage + wave * STAGE;
+  // transposing read: lane (quad, col = 4*r + j) supplies the 8 bytes of token
+  // 4*quad + r (of the 16-token sub-tile), halves 16*dt + 4*j .. +3.  Granule
+  // (16 bytes) p of token t lives at granule p ^ (2 * (t & 7)) of its row.
+  const uint32_t read_token = 4u * quad + (col >> 2);
+  const uint32_t read_swizzle = read_token & 7u;
+  const uint32_t read_base =
+      read_token * (GR * 16u) + ((col >> 1) & 1u) * 16u + (col & 1u) * 8u;
+
+  float running_max[RT];
+  float running_sum[RT];
+  f32x4 out[DT][RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    running_max[rt] = kMaskedMax;
+    running_sum[rt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
+  }
+
+  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+    const uint32_t tile_begin = tile * kF16Tile;
+    const bool needs_mask = tile_begin + kF16Tile > first_context_tokens;
+    const uint16_t* page = static_cast<const uint16_t*>(
+        uniform_page(args.pages, tile_begin / args.page_tokens));
+    const uint16_t* keys =
+        page + layer_offset +
+        static_cast<size_t>(tile_begin % args.page_tokens) * row_stride +
+        kv_head * D;
+    const uint16_t* values = keys + page_values;
+
+    // ---- V tile -> LDS (swizzled rows) ----------------------------------------
+#pragma unroll
+    for (int pass = 0; pass < kF16Tile * GR / 64; ++pass) {
+      const uint32_t piece = pass * 64u + lane;
+      const uint32_t token = piece / GR;
+      const uint32_t part = piece % GR;
+      uint4 value = *reinterpret_cast<const uint4*>(
+          values + static_cast<size_t>(token) * row_stride + part * 8u);
+      // records no row can see may be uninitialised: a NaN there would
+      // survive its zero probability
+      if (needs_mask && tile_begin + token >= last_context)
+        value = make_uint4(0u, 0u, 0u, 0u);
+      *reinterpret_cast<uint4*>(stage_v + (token * GR + (part ^ (2u * (token & 7u)))) *
+                                              16u) = value;
+    }
+
+    // ---- S = K . Q, online softmax, probabilities per row tile ------------------
+    f16x4 p_operand[RT][2];
+    f16x8 key_operand[2][KSTEPS];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        key_operand[st][ks] = *reinterpret_cast<const f16x8*>(
+            keys + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
+            8u * quad);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      asm volatile("" ::: "memory");  // one row tile's query operands at a time
+      float score[2][4];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        f32x4 dot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const f16x8 q = *reinterpret_cast<const f16x8*>(
+              q_operands + (rt * KSTEPS + ks) * 1024);
+          dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand[st][ks], q,
+                                                       dot, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) score[st][i] = dot[i] * score_unit;
+      }
+      if (needs_mask) {
+        const uint32_t first_token = tile_begin + 4u * quad;
+        const uint32_t limit = exchange_limit[16 * rt + col];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (first_token + 16u * st + i >= limit) score[st][i] = -INFINITY;
+      }
+      // the running maximum follows the tile maximum only when that is more
+      // than 8 (log2 units) ahead: probabilities stay below 2^8
+      float tile_max = score[0][0];
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tile_max = fmaxf(tile_max, score[st][i]);
+      tile_max = quad_row_max(tile_max);
+      const bool grew = tile_max - running_max[rt] > 8.0f;
+      if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+        const float new_max = fmaxf(running_max[rt], tile_max);
+        if (tile != tile_first) {
+          const float factor = __builtin_amdgcn_exp2f(running_max[rt] - new_max);
+          running_sum[rt] *= factor;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+        }
+        running_max[rt] = new_max;
+      }
+      float sum = 0.0f;
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const _Float16 p = static_cast<_Float16>(
+              __builtin_amdgcn_exp2f(score[st][i] - running_max[rt]));
+          p_operand[rt][st][i] = p;
+          sum += static_cast<float>(p);
+        }
+      running_sum[rt] += sum;
+    }
+
+    // ---- O^T += V^T . P^T -------------------------------------------------------
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        // granule 2*dt + (j >> 1) of the row, swizzled; (j >> 1) and the byte
+        // offset of (j & 1) are already in read_base
+        const uint32_t address = st * 16u * (GR * 16u) + read_base +
+                                 ((2u * dt) ^ (2u * read_swizzle)) * 16u;
+        typedef short i16x4 __attribute__((ext_vector_type(4)));
+        const f16x4 v = __builtin_bit_cast(
+            f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                       (__attribute__((address_space(3))) i16x4*)(stage_v +
+                                                                  address)));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          out[dt][rt] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+              v, p_operand[rt][st], out[dt][rt], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) running_sum[rt] = quad_row_sum(running_sum[rt]);
+
+  static_assert(kSplitWaves * RT * 512 <= sizeof(exchange), "summaries fit");
+  const PartialTarget target{args.partial_maxima, args.partial_sums,
+                             args.partial_outputs, args.maximum_splits,
+                             args.query_heads, kv_head, split, group,
+                             matrix_rows};
+  merge_wave_states<D, RT>(running_max, running_sum, out,
+                           reinterpret_cast<float*>(stage),
+                           reinterpret_cast<float2*>(exchange), wave, lane,
+                           target);
+}
+
+template <int D>
+int32_t launch_f16_split(const F16SplitArgs& args, uint32_t row_tiles, dim3 grid,
+                         hipStream_t stream) {
+  switch (row_tiles) {
+    case 1:
+      f16_attention_split_kernel<D, 1><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      break;
+    case 2:
+      f16_attention_split_kernel<D, 2><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      break;
+    default:
+      if constexpr (D == 128) {
+        f16_attention_split_kernel<D, 3>
+            <<<grid, kSplitWaves * 64, 0, stream>>>(args);
+        break;
+      } else {
+        return fail(QLLM_INVALID_ARGUMENT,
+                    "F16 attention: three row tiles need head_dim 128");
+      }
+  }
+  return launched("F16 attention split");
+}
+
 }  // namespace
+
+// defined with the Q4H kernels
+int32_t launch_attention_combine(const float* query, uint32_t query_stride,
+                                 int output_gated, const float* partial_maxima,
+                                 const float* partial_sums,
+                                 const float* partial_outputs, void* output,
+                                 uint32_t output_kind,
+                                 uint32_t first_context_tokens,
+                                 uint32_t maximum_splits, uint32_t split_tokens,
+                                 uint32_t rows, uint32_t query_heads,
+                                 uint32_t head_dim,
+                                 const uint32_t* device_positions,
+                                 hipStream_t stream);
 }  // namespace qllm
 
 using namespace qllm;
@@ -54,6 +358,63 @@ extern "C" int32_t qllm_store_kv_paged_f16_batch(
 
 extern "C" int32_t qllm_attention_paged_f16(
     const qllm_f16_attention_launch* launch) {
-  (void)launch;
-  return fail(QLLM_INTERNAL, "exact-F16 attention kernel is not built yet");
+  if (!launch || !launch->query || !launch->device_pages || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      !launch->first_context_tokens || !launch->rows ||
+      !launch->device_page_tokens || launch->device_page_tokens % kF16Tile ||
+      !launch->query_heads || !launch->kv_heads ||
+      launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      launch->split_tokens % kF16Tile || !launch->maximum_splits ||
+      launch->maximum_splits > 2048u ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid F16 paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t row_tiles = (launch->rows * group + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "F16 paged attention: rows * (query_heads/kv_heads) exceeds "
+                "48 (32 at head_dim 256)");
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      launch->split_tokens
+          ? (last_context + launch->split_tokens - 1u) / launch->split_tokens
+          : launch->maximum_splits;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "F16 paged attention: context needs more splits than "
+                "maximum_splits");
+  F16SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.pages = launch->device_pages;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.layer = launch->device_page_layer;
+  args.page_tokens = launch->device_page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  const dim3 grid(launch->kv_heads, splits);
+  const hipStream_t stream = as_stream(launch->stream);
+  const int32_t status =
+      launch->head_dim == 128u ? launch_f16_split<128>(args, row_tiles, grid, stream)
+                               : launch_f16_split<256>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, nullptr, stream);
 }

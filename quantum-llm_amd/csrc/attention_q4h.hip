@@ -23,18 +23,13 @@
 // The eight wave states are merged in LDS and one (max, sum, unnormalised
 // output) partial per (row, split, head) is written; the combine kernel
 // merges the splits.  Maxima are kept in the log2 domain.
-#include "common.hpp"
+#include "attention_common.hpp"
 
 #include <utility>
 
 namespace qllm {
 namespace {
 
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-
-constexpr int kSplitWaves = 8;
-constexpr float kMaskedMax = -1.0e30f;
 
 struct Q4hPlanes {
   const uint8_t* key_codes;
@@ -65,25 +60,6 @@ __device__ __forceinline__ Q4hPlanes q4h_planes(const void* page,
   return planes;
 }
 
-// max over the lanes {l, l^16, l^32, l^48}
-__device__ __forceinline__ float quad_row_max(float value) {
-  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
-                                            __float_as_uint(value), false, false);
-  value = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
-                                            __float_as_uint(value), false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-
-__device__ __forceinline__ float quad_row_sum(float value) {
-  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(value),
-                                            __float_as_uint(value), false, false);
-  value = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
-                                            __float_as_uint(value), false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
 struct SplitArgs {
   const float* query;
   uint32_t query_stride;
@@ -104,15 +80,6 @@ struct SplitArgs {
 
 
 
-
-// Page table entry at a wave-uniform index, fetched with a scalar load (the
-// table is never written while attention kernels run), so everything derived
-// from the page address stays in scalar registers.
-__device__ __forceinline__ const void* uniform_page(
-    const void* const* page_table, uint32_t index) {
-  typedef const void* __attribute__((address_space(4))) const* constant_table;
-  return ((constant_table)page_table)[index];
-}
 
 // Tells the compiler that a pointer every lane computes alike is wave-uniform,
 // so that it can live in scalar registers.
@@ -269,22 +236,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
   // tiles [tile_first, tile_last) of this wave
   uint32_t tile_first, tile_last;
-  if (args.split_tokens == 0u) {
-    // balanced: the context's tiles are dealt evenly over every wave of the
-    // grid row, whatever the context length
-    const uint32_t slots = gridDim.y * kSplitWaves;
-    const uint32_t slot = split * kSplitWaves + wave;
-    tile_first = static_cast<uint32_t>(
-        static_cast<uint64_t>(slot) * context_tiles / slots);
-    tile_last = static_cast<uint32_t>(
-        static_cast<uint64_t>(slot + 1u) * context_tiles / slots);
-  } else {
-    const uint32_t split_tiles = args.split_tokens / 64u;
-    const uint32_t begin = min(split * split_tiles, context_tiles);
-    const uint32_t count = min(begin + split_tiles, context_tiles) - begin;
-    tile_first = begin + wave * count / kSplitWaves;
-    tile_last = begin + (wave + 1u) * count / kSplitWaves;
-  }
+  wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y, wave,
+                  tile_first, tile_last);
 
   uint8_t* stage_k = stage + wave * STAGE;
   const uint32_t stage_k_lds =
@@ -703,98 +656,19 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
                           : kMaskedMax;
   }
 
-  // ---- merge the eight wave states -------------------------------------------
-  // 1. every wave publishes its (max, sum) per row; all waves derive the
-  //    merged maximum and bring their own accumulators to it.
-  // 2. the accumulators are summed reduce-scatter style, eight 1 KiB register
-  //    vectors (one per receiving wave) at a time: each wave drops the eight
-  //    vectors of the group into LDS, lane-linear (no bank conflicts), and
-  //    wave v adds up vector v of all eight waves in a fixed order.  Wave v
-  //    ends up owning vectors v, v+8, ... of the result and writes them out.
-  constexpr int VECTORS = DT * RT;   // f32x4 accumulator vectors per wave
-  static_assert(VECTORS % kSplitWaves == 0, "vectors are dealt to 8 waves");
+  // ---- merge the eight wave states, write the split partial ------------------
   static_assert(kSplitWaves * kSplitWaves * 1024 <= kSplitWaves * STAGE,
                 "merge pool does not fit the staging memory");
   static_assert(kSplitWaves * RT * 64 * 8 <= sizeof(exchange),
                 "row summaries do not fit the exchange area");
-  float2* summary = reinterpret_cast<float2*>(exchange);  // [wave][rt][lane]
-  float* pool = reinterpret_cast<float*>(stage);          // [wave][slot][lane] x 4
-  __syncthreads();  // tiles done: staging and the operand exchange are free
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
-    summary[(wave * RT + rt) * 64 + lane] =
-        make_float2(running_max[rt], running_sum[rt]);
-  __syncthreads();
-  float merged_max[RT], merged_sum[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    float2 part[kSplitWaves];
-    float maximum = kMaskedMax;
-#pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w) {
-      part[w] = summary[(w * RT + rt) * 64 + lane];
-      maximum = fmaxf(maximum, part[w].x);
-    }
-    float sum = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w)
-      sum = fmaf(part[w].y, __builtin_amdgcn_exp2f(part[w].x - maximum), sum);
-    const float factor = __builtin_amdgcn_exp2f(running_max[rt] - maximum);
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
-    merged_max[rt] = maximum;
-    merged_sum[rt] = sum;
-  }
-  f32x4 merged[VECTORS / kSplitWaves];
-#pragma unroll
-  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
-#pragma unroll
-    for (int v = 0; v < kSplitWaves; ++v) {
-      const int k = group_index * kSplitWaves + v;
-      *reinterpret_cast<f32x4*>(pool + ((wave * kSplitWaves + v) * 64 + lane) * 4u) =
-          out[k / RT][k % RT];
-    }
-    __syncthreads();
-    f32x4 total = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w)
-      total += *reinterpret_cast<const f32x4*>(
-          pool + ((w * kSplitWaves + wave) * 64 + lane) * 4u);
-    merged[group_index] = total;
-    __syncthreads();
-  }
-
-  // ---- partials: wave v writes the vectors it owns, wave 0 also max and sum ----
-#pragma unroll
-  for (int group_index = 0; group_index < VECTORS / kSplitWaves; ++group_index) {
-    const uint32_t k = group_index * kSplitWaves + wave;
-    const uint32_t dt = k / RT;
-    const uint32_t rt = k % RT;
-    const uint32_t matrix_row = 16u * rt + col;
-    if (matrix_row >= matrix_rows) continue;
-    const uint32_t row = matrix_row / group;
-    const uint32_t head = kv_head * group + matrix_row % group;
-    const size_t partial =
-        (static_cast<size_t>(row) * args.maximum_splits + split) *
-            args.query_heads + head;
-    *reinterpret_cast<f32x4*>(args.partial_outputs + partial * D + 16u * dt +
-                              4u * quad) = merged[group_index];
-  }
-  if (wave != 0u || quad != 0u) return;
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const uint32_t matrix_row = 16u * rt + col;
-    if (matrix_row >= matrix_rows) continue;
-    const uint32_t row = matrix_row / group;
-    const uint32_t head = kv_head * group + matrix_row % group;
-    const size_t partial =
-        (static_cast<size_t>(row) * args.maximum_splits + split) *
-            args.query_heads + head;
-    args.partial_maxima[partial] = merged_max[rt];
-    args.partial_sums[partial] = merged_sum[rt];
-  }
+  const PartialTarget target{args.partial_maxima, args.partial_sums,
+                             args.partial_outputs, args.maximum_splits,
+                             args.query_heads, kv_head, split, group,
+                             matrix_rows};
+  merge_wave_states<D, RT>(running_max, running_sum, out,
+                           reinterpret_cast<float*>(stage),
+                           reinterpret_cast<float2*>(exchange), wave, lane,
+                           target);
 }
 
 // Split-K merge (maxima in log2 units), optional sigmoid output gate.

@@ -200,22 +200,14 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
       static_cast<std::uint16_t*>(device_alloc(rows * g_.intermediate * 2U));
   logits_ = static_cast<float*>(device_alloc(rows * g_.vocabulary * 4U));
 
-  // Context splits: a split is a multiple of 64 tokens sized so that
-  // kv_heads * splits workgroups roughly fill the 256 CUs at full context,
-  // never shorter than 512 tokens (one 64-token tile per wave).
+  // Context splits: kv_heads * splits workgroups fill the 256 CUs; the
+  // attention kernels deal the context's tiles evenly over them themselves
+  // (split_tokens 0), whatever the context length.
   const std::uint32_t wanted_splits =
       std::max(1U, 256U / std::max(1U, g_.kv_heads));
-  std::uint32_t split = (g_.max_context + wanted_splits - 1U) / wanted_splits;
-  split = std::max(512U, (split + 63U) / 64U * 64U);
-  split_tokens_ = split;
-  maximum_splits_ = (g_.max_context + split - 1U) / split;
-  if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-    // the Q4H kernel deals the context's 64-token tiles evenly over the grid
-    // itself (split_tokens 0), whatever the context length
-    split_tokens_ = 0U;
-    maximum_splits_ =
-        std::min(wanted_splits, std::max(1U, (g_.max_context + 511U) / 512U));
-  }
+  split_tokens_ = 0U;
+  maximum_splits_ =
+      std::min(wanted_splits, std::max(1U, (g_.max_context + 511U) / 512U));
   const std::size_t partials = rows * maximum_splits_ * g_.query_heads;
   partial_maxima_ = static_cast<float*>(device_alloc(partials * 4U));
   partial_sums_ = static_cast<float*>(device_alloc(partials * 4U));

@@ -73,3 +73,29 @@ def q4h_attention(device, pages, query, rows, query_heads, kv_heads, head_dim,
     qh.call("qllm_attention_paged_q4h", launch)
     torch.cuda.synchronize()
     return out.float().cpu().numpy()
+
+
+def f16_attention(device, pages, query, rows, query_heads, kv_heads, head_dim,
+                  first_context, page_tokens, split_tokens, gated, layer=0,
+                  out_kind=qh.OUT_F32, balanced_splits=32):
+    """qllm_attention_paged_f16 on host pages (list of uint8 arrays)."""
+    stride = head_dim * (2 if gated else 1)
+    d_pages = [device_tensor(page, device) for page in pages]
+    table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
+                         device=device)
+    d_query = device_tensor(query, device)
+    context = first_context + rows - 1
+    splits = ((context + split_tokens - 1) // split_tokens if split_tokens
+              else balanced_splits)
+    maxima = torch.zeros((rows, splits, query_heads), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((rows, splits, query_heads, head_dim), device=device)
+    dtype = torch.bfloat16 if out_kind == qh.OUT_BF16 else torch.float32
+    out = torch.zeros((rows, query_heads, head_dim), dtype=dtype, device=device)
+    launch = qh.F16AttentionLaunch(
+        qh.ptr(d_query), qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), first_context, rows, layer, page_tokens, query_heads,
+        kv_heads, head_dim, split_tokens, splits, stride, int(gated), out_kind, None)
+    qh.call("qllm_attention_paged_f16", launch)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()

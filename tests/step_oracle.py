@@ -81,10 +81,20 @@ def _record_slices(model, layer, page_tokens, position, kv_head):
             slice(value_scale, value_scale + 2)]
 
 
+def _f16_store(page, layer, page_tokens, position, kv_head, kv_heads, d, key, value):
+    """Exact-F16 page: per layer K [page_tokens][kv][d] then V, binary16."""
+    halves = page.view(np.float16)
+    page_values = page_tokens * kv_heads * d
+    base = layer * 2 * page_values + ((position % page_tokens) * kv_heads + kv_head) * d
+    halves[base: base + d] = key.astype(np.float16)
+    halves[base + page_values: base + page_values + d] = value.astype(np.float16)
+
+
 def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
-               observed_pages=None, report=None):
+               observed_pages=None, report=None, kv_encoding=0):
     """Returns (logits [rows, V], hidden [rows, H]); writes K/V of the rows into
-    kv_pages (list of uint8 arrays, Q4H, all layers per page).
+    kv_pages (list of uint8 arrays, all layers per page; Q4H records, or
+    binary16 K/V planes when kv_encoding is 1).
 
     Q4H encoding is a discontinuous function of K/V: a last-bit difference in
     a projection can move a value across a rounding boundary and change a
@@ -115,6 +125,10 @@ def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
                     k[r, h], block.get("key_norm"), m.rotary_dim, position,
                     m.eps, m.rope_theta)
                 page = kv_pages[position // page_tokens]
+                if kv_encoding == 1:
+                    _f16_store(page, layer, page_tokens, position, h, KV, d,
+                               k[r, h], v[r, h])
+                    continue
                 ol.q4h_store(page, layer, page_tokens, position, h, KV, d,
                              k[r, h], v[r, h])
                 if observed_pages is not None:
@@ -126,7 +140,10 @@ def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
                         page[part] = observed[part]
         shape = ol.AttentionShape(rows, Q, KV, d, first_position + 1, page_tokens,
                                   layer, int(m.output_gated))
-        attention = ol.attention_q4h(shape, q, kv_pages, "f64")
+        if kv_encoding == 1:
+            attention = ol.attention_f16(shape, q, kv_pages, True)
+        else:
+            attention = ol.attention_q4h(shape, q, kv_pages, "f64")
         attention = ol.bf16_round(attention.reshape(rows, Q * d))
         hidden = hidden + m.linear(block["output"], attention, m.hidden)
         x = ol.rms_norm_rows(hidden, block["post_attention_norm"], m.eps,

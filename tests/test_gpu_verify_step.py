@@ -63,6 +63,35 @@ def test_target_pass_matches_composed_oracle(device, name):
 
 
 @pytest.mark.parametrize("name", list(CONFIGS))
+def test_target_pass_with_exact_f16_cache(device, name):
+    """The same pass over the exact-F16 KV cache (kv-cache-dtype fp16)."""
+    rng = np.random.default_rng(11)
+    c = CONFIGS[name]
+    model = step_oracle.TinyModel(
+        rng, 256, 512, 2, 8, 2, c["head_dim"], 1024, c["scheme"],
+        output_gated=c["output_gated"], qk_norm=c["qk_norm"],
+        zero_centered=c["zero_centered"], rotary_dim=c["rotary_dim"])
+    provider = step_oracle.build_provider(model, qp, kv_encoding=1)
+    page_tokens = 64
+    page_bytes = model.layers * 2 * page_tokens * model.kv_heads * model.head_dim * 2
+    pages = [np.zeros(page_bytes, dtype=np.uint8) for _ in range(4)]
+    position = 0
+    for step in range(3):
+        tokens = rng.integers(0, model.vocabulary, 5).astype(np.uint32)
+        provider.run_target(tokens, position)
+        logits, hidden = provider.logits(5), provider.hidden(5)
+        want_logits, want_hidden = step_oracle.run_target(
+            model, tokens, position, pages, page_tokens, kv_encoding=1)
+        relative = (np.linalg.norm(logits - want_logits) /
+                    np.linalg.norm(want_logits))
+        assert relative < 2e-2, relative
+        assert np.abs(hidden - want_hidden).max() < 0.05 * np.abs(want_hidden).max()
+        assert np.array_equal(logits.argmax(1), want_logits.argmax(1))
+        position += 5
+    provider.close()
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
 def test_acceptance_is_bit_exact_on_the_same_logits(device, name):
     rng, model, provider = make(name, 11)
     V = model.vocabulary
