@@ -101,20 +101,26 @@ __device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* pointer
 __device__ __forceinline__ void copy16_to_lds(const uint8_t* base,
                                               uint32_t lane_offset,
                                               uint32_t lds) {
+  uint32_t saved_m0;  // M0 carries the LDS address; it is put back afterwards
   asm volatile(
-      "s_mov_b32 m0, %2\n\t"
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %0, %1"
-      :: "v"(lane_offset), "s"(base), "s"(lds) : "memory", "m0");
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0) : "v"(lane_offset), "s"(base), "s"(lds) : "memory");
 }
 __device__ __forceinline__ void copy4_to_lds(const uint8_t* base,
                                              uint32_t lane_offset,
                                              uint32_t lds) {
+  uint32_t saved_m0;  // M0 carries the LDS address; it is put back afterwards
   asm volatile(
-      "s_mov_b32 m0, %2\n\t"
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dword %0, %1"
-      :: "v"(lane_offset), "s"(base), "s"(lds) : "memory", "m0");
+      "global_load_lds_dword %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0) : "v"(lane_offset), "s"(base), "s"(lds) : "memory");
 }
 
 // LDS reads of staged tiles.  They are written as inline assembly on purpose:
