@@ -25,6 +25,10 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 sys.path.insert(0, os.path.join(ROOT, "quantum-llm_amd", "python"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the fused gate/up kernel moves, from the FETCH_SIZE and
+# WRITE_SIZE hardware counters scaled by a 256 MiB copy (summary and commands
+# in profiles/hot_kernels_hbm_traffic.md); 1.04x the algorithmic bytes.
+GATE_UP_TRAFFIC_BYTES = 115941396
 
 MODEL = dict(hidden=5120, intermediate=17408, layers=64, query_heads=64, kv_heads=8,
              head_dim=128, rotary_dim=128, vocabulary=151936, rope_theta=1.0e6,
@@ -101,6 +105,9 @@ def main():
     parser.add_argument("--layers", type=int, default=MODEL["layers"],
                         help="for quick experiments only; the reported config is 64")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--calibration-copy", action="store_true",
+                        help="also run one 256 MiB device copy (a kernel of known "
+                             "traffic to scale hardware counters by)")
     arguments = parser.parse_args()
     if arguments.gpus != 1:
         print("bench.py: this build runs the verify step on ONE GPU only "
@@ -171,7 +178,7 @@ def main():
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": GATE_UP_TRAFFIC_BYTES if geometry["layers"] == MODEL["layers"] else None,
         "algorithmic_bytes_per_launch": kernel_bytes,
         "avg_launch_us": round(kernel_us, 3),
         "launches_timed": launches,
@@ -230,6 +237,11 @@ def main():
         "kernels": other_kernels,
     }
     provider.close()
+    if arguments.calibration_copy:
+        source = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
+        target = torch.empty_like(source)
+        target.copy_(source)
+        torch.cuda.synchronize()
     if not arguments.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(rows)
     print(json.dumps(result))
