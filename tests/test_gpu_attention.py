@@ -31,7 +31,7 @@ def run_case(device, rng, tokens, rows, Q, KV, d, page_tokens, split_tokens, gat
 @pytest.mark.parametrize("tokens,rows,Q,KV,d,page,split,gated", [
     (5, 5, 8, 2, 128, 64, 512, False),        # context of the rows alone
     (12, 5, 8, 1, 128, 64, 64, False),
-    (100, 5, 64, 8, 128, 256, 64, False),     # several splits, BASELINE heads
+    (100, 5, 64, 8, 128, 256, 64, False),     # several splits, 64Q/8KV heads
     (1000, 5, 64, 8, 128, 256, 256, False),
     (700, 5, 24, 4, 256, 256, 512, True),     # reference geometry, gated
     (3000, 1, 64, 8, 128, 256, 1024, False),  # single-row decode
@@ -69,7 +69,7 @@ def test_reference_arithmetic_is_within_its_own_error(device):
 
 
 def test_attention_is_split_invariant_at_32k(device):
-    """BASELINE config 2 shape (5 rows, 64Q/8KV, d=128, L=32768): the result
+    """Benchmark attention shape (5 rows, 64Q/8KV, d=128, L=32768): the result
     must not depend on the split size, and the causal rows must differ."""
     rng = np.random.default_rng(7)
     tokens, rows, Q, KV, d, page = 32768, 5, 64, 8, 128, 256

@@ -29,7 +29,7 @@ def run_case(device, rng, tokens, rows, Q, KV, d, page_tokens, split_tokens, gat
 @pytest.mark.parametrize("tokens,rows,Q,KV,d,page,split,gated", [
     (5, 5, 8, 2, 128, 32, 512, False),        # context of the rows alone
     (12, 5, 8, 1, 128, 64, 32, False),
-    (100, 5, 64, 8, 128, 256, 64, False),     # several splits, BASELINE heads
+    (100, 5, 64, 8, 128, 256, 64, False),     # several splits, 64Q/8KV heads
     (1000, 5, 64, 8, 128, 256, 256, False),
     (700, 5, 24, 4, 256, 256, 512, True),     # reference geometry, gated
     (3000, 1, 64, 8, 128, 256, 1024, False),  # single-row decode
@@ -39,7 +39,7 @@ def run_case(device, rng, tokens, rows, Q, KV, d, page_tokens, split_tokens, gat
     (1500, 4, 24, 4, 256, 256, 0, True)])
 def test_f16_attention_matches_oracle(device, tokens, rows, Q, KV, d, page, split,
                                       gated):
-    """Tolerance of the north star (rtol 1e-2, atol 1e-3) against the
+    """rtol 1e-2, atol 1e-3 (F32 accumulate) against the
     reference's arithmetic (binary16 query and probabilities) and against
     exact attention on the same binary16 cache."""
     rng = np.random.default_rng(tokens + 7 * rows + Q)

@@ -86,7 +86,7 @@ def test_split_gemm_equals_separate_calls(device, padded, tiled):
 
 
 def test_gemm_config1_shape_and_output_kinds(device):
-    """BASELINE config 1: [17408, 5120], M=5, binary16 scale per 16, bf16 out."""
+    """Benchmark shape of one linear: [17408, 5120], M=5, binary16 scale per 16, bf16 out."""
     rng = np.random.default_rng(1)
     rows, padded, batch, scheme = 17408, 5120, 5, ol.SCALE_F16_BLOCK16
     codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)

@@ -12,7 +12,7 @@ import step_oracle
 pytestmark = pytest.mark.gpu
 
 CONFIGS = {
-    # BASELINE-style: plain GQA, full rotary, binary16 scale per 16
+    # benchmark model style: plain GQA, full rotary, binary16 scale per 16
     "baseline": dict(scheme=ol.SCALE_F16_BLOCK16, output_gated=False, qk_norm=False,
                      zero_centered=False, head_dim=128, rotary_dim=None),
     # reference-style: ABI 3 weights, output gate, q/k norm, partial rotary, d=256
