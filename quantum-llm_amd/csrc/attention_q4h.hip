@@ -794,13 +794,15 @@ __global__ __launch_bounds__(64) void q4h_store_kernel(
 }
 
 // Per-head RMSNorm(1+w) and NeoX rotary, in place; one wave per (head, row).
-// Blocks with head < kv_heads also process the K row.
+// The rotated row is also left in `rotated` (LDS) for a caller that goes on to
+// encode it.
 __device__ __forceinline__ void head_norm_rope(float* x, const float* weight,
                                                uint32_t head_dim,
                                                uint32_t rotary_dim,
                                                uint32_t position, float epsilon,
                                                float theta, bool bf16_activations,
-                                               float* shared, uint32_t lane) {
+                                               float* shared, float* rotated,
+                                               uint32_t lane) {
   if (weight) {
     float square = 0.0f;
     for (uint32_t index = lane; index < head_dim; index += 64u)
@@ -828,19 +830,23 @@ __device__ __forceinline__ void head_norm_rope(float* x, const float* weight,
                           static_cast<float>(rotary_dim));
       const float other =
           index < half ? -shared[index + half] : shared[index - half];
-      float cosine = cosf(angle);
-      float sine = sinf(angle);
+      float sine, cosine;
+      sincosf(angle, &sine, &cosine);
       if (bf16_activations) {
         cosine = bf16_round(cosine);
         sine = bf16_round(sine);
       }
       result = shared[index] * cosine + other * sine;
     }
-    x[index] = bf16_activations ? bf16_round(result) : result;
+    result = bf16_activations ? bf16_round(result) : result;
+    x[index] = result;
+    rotated[index] = result;
   }
   __builtin_amdgcn_wave_barrier();
 }
 
+// grid (query_heads + kv_heads, rows): blocks [0, query_heads) rotate a query
+// head, the others rotate a key head and encode that K/V record.
 __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     float* query, uint32_t query_stride, float* key, const float* value,
     const float* q_weight, const float* k_weight,
@@ -850,23 +856,27 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations,
     const uint32_t* device_positions) {
   __shared__ float shared[256];
+  __shared__ float rotated[256];
   if (device_positions) {
     first_cache_position = device_positions[0];
     first_rotary_position = device_positions[1];
   }
-  const uint32_t head = blockIdx.x;
   const uint32_t row = blockIdx.y;
   const uint32_t lane = threadIdx.x;
   const uint32_t rotary_position = first_rotary_position + row;
-  float* q = query + (static_cast<size_t>(row) * query_heads + head) * query_stride;
-  head_norm_rope(q, q_weight, head_dim, rotary_dim, rotary_position, epsilon,
-                 theta, bf16_activations, shared, lane);
-  if (head >= kv_heads) return;
+  if (blockIdx.x < query_heads) {
+    const uint32_t head = blockIdx.x;
+    float* q =
+        query + (static_cast<size_t>(row) * query_heads + head) * query_stride;
+    head_norm_rope(q, q_weight, head_dim, rotary_dim, rotary_position, epsilon,
+                   theta, bf16_activations, shared, rotated, lane);
+    return;
+  }
+  const uint32_t head = blockIdx.x - query_heads;
   float* k = key + (static_cast<size_t>(row) * kv_heads + head) * head_dim;
   head_norm_rope(k, k_weight, head_dim, rotary_dim, rotary_position, epsilon,
-                 theta, bf16_activations, shared, lane);
+                 theta, bf16_activations, shared, rotated, lane);
   if (!page_table) return;  // rotary only; the caller stores K/V itself
-  __threadfence_block();
   const uint32_t position = first_cache_position + row;
   uint8_t* page = static_cast<uint8_t*>(
       const_cast<void*>(page_table[position / page_tokens]));
@@ -874,7 +884,7 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
       q4h_planes(page, layer, page_tokens, kv_heads, head_dim);
   const size_t record =
       static_cast<size_t>(head) * page_tokens + position % page_tokens;
-  q4h_encode_record(k, head_dim,
+  q4h_encode_record(rotated, head_dim,
                     const_cast<uint8_t*>(planes.key_codes) + record * (head_dim / 2u),
                     const_cast<uint8_t*>(planes.key_scales) + record * 2u, lane);
   q4h_encode_record(value + (static_cast<size_t>(row) * kv_heads + head) * head_dim,
@@ -991,7 +1001,8 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       first_cache_position > 0xffffffffu - (rows - 1u) ||
       first_rotary_position > 0xffffffffu - (rows - 1u))
     return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H QKV rope cache batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
@@ -1015,7 +1026,8 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
       !(epsilon > 0.0f) || !(rope_theta > 0.0f))
     return fail(QLLM_INVALID_ARGUMENT,
                 "invalid deferred Q4H QKV rope cache batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, 0u, 0u, query_heads, kv_heads,
       head_dim, rotary_dim, epsilon, rope_theta, bf16_activations != 0,
@@ -1036,7 +1048,8 @@ extern "C" int32_t qllm_qkv_rope_batch(
       !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
       first_rotary_position > 0xffffffffu - (rows - 1u))
     return fail(QLLM_INVALID_ARGUMENT, "invalid QKV rope batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads, rows), 64, 0, as_stream(stream)>>>(
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
       rotary_dim, epsilon, rope_theta, bf16_activations != 0, nullptr);
