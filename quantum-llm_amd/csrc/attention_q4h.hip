@@ -702,6 +702,15 @@ __global__ void attention_combine_kernel(
                    : maximum_splits;
   const size_t first_partial =
       static_cast<size_t>(row) * maximum_splits * query_heads + head;
+  // The first kCombinePrefetch partial outputs are fetched before anything
+  // depends on them, so that they travel together with the maxima and sums.
+  constexpr uint32_t kCombinePrefetch = 32;
+  const float* source = partial_outputs + first_partial * head_dim + dimension;
+  const size_t stride = static_cast<size_t>(query_heads) * head_dim;
+  float fetched[kCombinePrefetch];
+#pragma unroll
+  for (uint32_t split = 0; split < kCombinePrefetch; ++split)
+    fetched[split] = split < active ? source[split * stride] : 0.0f;
   float local_max = kMaskedMax;
   for (uint32_t split = threadIdx.x; split < active; split += blockDim.x)
     local_max = fmaxf(local_max,
@@ -718,19 +727,11 @@ __global__ void attention_combine_kernel(
   }
   const float sum = block_sum(local_sum, scratch);  // also publishes weights[]
   float result = 0.0f;
-  const float* source = partial_outputs + first_partial * head_dim + dimension;
-  const size_t stride = static_cast<size_t>(query_heads) * head_dim;
-  uint32_t split = 0;
-  for (; split + 4u <= active; split += 4u) {
-    const float a = source[(split + 0u) * stride];
-    const float b = source[(split + 1u) * stride];
-    const float c = source[(split + 2u) * stride];
-    const float d = source[(split + 3u) * stride];
-    result += a * weights[split] + b * weights[split + 1u] +
-              c * weights[split + 2u] + d * weights[split + 3u];
-  }
-  for (; split < active; ++split)
-    result += source[split * stride] * weights[split];
+#pragma unroll
+  for (uint32_t split = 0; split < kCombinePrefetch; ++split)
+    if (split < active) result = fmaf(fetched[split], weights[split], result);
+  for (uint32_t split = kCombinePrefetch; split < active; ++split)
+    result = fmaf(source[split * stride], weights[split], result);
   result /= sum;
   const size_t record = static_cast<size_t>(row) * query_heads + head;
   if (output_gated) {

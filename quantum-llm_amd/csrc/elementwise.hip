@@ -141,12 +141,20 @@ __global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
   const float4* x =
       reinterpret_cast<const float4*>(input + static_cast<size_t>(row) * elements);
   const uint32_t vectors = elements / 4u;
+  // the row and its weights are fetched together, before the reduction
   float4 values[4];
+  float4 factors[4];
   float square = 0.0f;
 #pragma unroll
   for (int slot = 0; slot < 4; ++slot) {
     const uint32_t index = slot * 1024u + threadIdx.x;
     values[slot] = index < vectors ? x[index] : make_float4(0.f, 0.f, 0.f, 0.f);
+    factors[slot] = make_float4(1.f, 1.f, 1.f, 1.f);
+    if (weight && index < vectors)
+      factors[slot] = reinterpret_cast<const float4*>(weight)[index];
+  }
+#pragma unroll
+  for (int slot = 0; slot < 4; ++slot) {
     square = fmaf(values[slot].x, values[slot].x, square);
     square = fmaf(values[slot].y, values[slot].y, square);
     square = fmaf(values[slot].z, values[slot].z, square);
@@ -159,12 +167,9 @@ __global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
   for (int slot = 0; slot < 4; ++slot) {
     const uint32_t index = slot * 1024u + threadIdx.x;
     if (index >= vectors) continue;
-    float4 factor = make_float4(1.f, 1.f, 1.f, 1.f);
-    if (weight) {
-      factor = reinterpret_cast<const float4*>(weight)[index];
-      if (zero_centered) {
-        factor.x += 1.0f; factor.y += 1.0f; factor.z += 1.0f; factor.w += 1.0f;
-      }
+    float4 factor = factors[slot];
+    if (weight && zero_centered) {
+      factor.x += 1.0f; factor.y += 1.0f; factor.z += 1.0f; factor.w += 1.0f;
     }
     float4 result;
     result.x = values[slot].x * inverse * factor.x;

@@ -186,6 +186,19 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint8_t* activation_base =
       reinterpret_cast<const uint8_t*>(args.activations);
 
+  // The residual of this thread's output item (see the epilogue) is fetched
+  // now, so that the value is there when the K loop ends.
+  float residual_value = 0.0f;
+  if constexpr (TILES == 1) {
+    if (args.residual && !args.segments) {
+      const uint32_t reg = (threadIdx.x / 64u) % REGS;
+      const uint32_t batch = (COMPACT ? 3u : 4u) * (lane >> 5) + reg;
+      const uint32_t row = blockIdx.x * h + n;
+      if (threadIdx.x < REGS * 64u && batch < BATCH && n < h && row < args.rows)
+        residual_value = args.residual[static_cast<size_t>(batch) * args.rows + row];
+    }
+  }
+
   float acc[TILES][REGS];
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
@@ -309,44 +322,46 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     for (int i = 0; i < REGS; ++i) reduce[wave][t][i][lane] = acc[t][i];
   __syncthreads();
 
-  // item = (tile, register i, lane): lane (n, g) register i holds MFMA row
-  // 4*g + i, i.e. batch row (COMPACT ? 3 : 4)*g + i
+  // Output item of this thread: item = (tile, register i, lane); lane (n, g)
+  // register i holds MFMA row 4*g + i, i.e. batch row (COMPACT ? 3 : 4)*g + i.
+  // (two tiles per workgroup are the gate/up pair: one output per row pair)
+  static_assert(TILES <= 2 && REGS * 64 <= WAVES * 64,
+                "one output item per thread");
   const uint32_t items = (args.swiglu ? 1u : TILES) * REGS * 64u;
-  for (uint32_t item = threadIdx.x; item < items; item += WAVES * 64u) {
-    const uint32_t t = item / (REGS * 64u);
-    const uint32_t i = (item / 64u) % REGS;
-    const uint32_t source_lane = item & 63u;
-    const uint32_t m = (COMPACT ? 3u : 4u) * (source_lane >> 5) + i;
-    const uint32_t tile_row = source_lane & 31u;
-    const uint32_t row =
-        (args.swiglu ? blockIdx.x : blockIdx.x * TILES + t) * h + tile_row;
-    if (m >= BATCH || tile_row >= h || row >= args.rows) continue;
-    float total = 0.0f;
+  const uint32_t item_tile = threadIdx.x / (REGS * 64u);
+  const uint32_t item_reg = (threadIdx.x / 64u) % REGS;
+  const uint32_t item_lane = threadIdx.x & 63u;
+  const uint32_t item_batch = (COMPACT ? 3u : 4u) * (item_lane >> 5) + item_reg;
+  const uint32_t item_tile_row = item_lane & 31u;
+  const uint32_t item_row =
+      (args.swiglu ? blockIdx.x : blockIdx.x * TILES + item_tile) * h + item_tile_row;
+  const bool item_valid = threadIdx.x < items && item_batch < BATCH &&
+                          item_tile_row < h && item_row < args.rows;
+  const size_t item_index = static_cast<size_t>(item_batch) * args.rows + item_row;
+  if (!item_valid) return;
+  float total = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) total += reduce[w][t][i][source_lane];
-    const size_t index = static_cast<size_t>(m) * args.rows + row;
-    if (args.swiglu) {
-      float up = 0.0f;
+  for (int w = 0; w < WAVES; ++w) total += reduce[w][item_tile][item_reg][item_lane];
+  if (args.swiglu) {
+    float up = 0.0f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w)
-        up += reduce[w][TILES - 1][i][source_lane];
-      const float activated = bf16_round(total / (1.0f + __expf(-total)));
-      static_cast<uint16_t*>(args.output)[index] =
-          static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
-    } else if (args.segments) {
-      uint32_t local = row;
-      uint32_t segment = 0;
-      while (segment + 1u < args.segments && local >= args.segment_rows[segment]) {
-        local -= args.segment_rows[segment];
-        ++segment;
-      }
-      store_output(args.segment_output[segment], args.segment_kind[segment],
-                   static_cast<size_t>(m) * args.segment_rows[segment] + local,
-                   total);
-    } else {
-      if (args.residual) total += args.residual[index];
-      store_output(args.output, args.output_kind, index, total);
+    for (int w = 0; w < WAVES; ++w)
+      up += reduce[w][TILES - 1][item_reg][item_lane];
+    const float activated = bf16_round(total / (1.0f + __expf(-total)));
+    static_cast<uint16_t*>(args.output)[item_index] =
+        static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
+  } else if (args.segments) {
+    uint32_t local = item_row;
+    uint32_t segment = 0;
+    while (segment + 1u < args.segments && local >= args.segment_rows[segment]) {
+      local -= args.segment_rows[segment];
+      ++segment;
     }
+    store_output(args.segment_output[segment], args.segment_kind[segment],
+                 static_cast<size_t>(item_batch) * args.segment_rows[segment] + local,
+                 total);
+  } else {
+    store_output(args.output, args.output_kind, item_index, total + residual_value);
   }
 }
 
