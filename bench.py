@@ -43,9 +43,16 @@ def fp4_bytes(rows, columns):
 
 
 def cpu_baseline(rows):
-    """Times the oracle (a CPU port of the step's arithmetic: double-precision
-    FP4 linears and Q4H attention, OpenMP over the host cores) on a bounded
-    sample and scales it to one full step."""
+    """CPU time of one verify step on the host cores, bounded sample.
+
+    Linears: the reference's own all-core CPU executor
+    (runtime/src/cpu/fp4_host_executor.cpp, FP4 ABI-3 weights x Q8 activations,
+    AVX2), compiled from its source into oracle/_ref, timed on one layer's
+    SwiGLU block (gate, up, down at the benchmark shape) and scaled by weight
+    bytes to the seven linears of 64 layers plus lm_head.  Attention has no CPU
+    path in the reference; its share is the oracle port (double precision,
+    OpenMP) timed on one layer at 32768 tokens.  When oracle/_ref is absent the
+    linears fall back to the oracle port as well (kind "port")."""
     import numpy as np
 
     import oracle_lib as ol
@@ -54,47 +61,125 @@ def cpu_baseline(rows):
     rng = np.random.default_rng(0)
     H, I, Q, KV, d = (MODEL["hidden"], MODEL["intermediate"], MODEL["query_heads"],
                       MODEL["kv_heads"], MODEL["head_dim"])
-    shapes = [(Q * d, H), (KV * d, H), (KV * d, H), (H, Q * d), (I, H), (I, H), (H, I)]
-    matrices = []
-    for n, k in shapes:
-        codes = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
-        scales = np.exp(0.5 * rng.standard_normal((n, k // 16))).astype(
+    cores = min(64, os.cpu_count() or 1)
+    if os.environ.get("OMP_NUM_THREADS"):
+        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    layer_parameters = (Q * d * H + 2 * KV * d * H + H * Q * d + 3 * I * H)
+    ffn_parameters = 3 * I * H
+    head_parameters = MODEL["vocabulary"] * H
+
+    def abi3(n, k):
+        return (rng.integers(0, 256, (n, k // 2), dtype=np.uint8),
+                rng.integers(124, 131, (n, k // 32), dtype=np.uint8))
+
+    reference = ol.ref() is not None and hasattr(ol.ref(), "qref_fp4_swiglu")
+    x = rng.standard_normal((rows, H)).astype(np.float32)
+    if reference:
+        gate, up, down = abi3(I, H), abi3(I, H), abi3(H, I)
+        _, ffn_seconds = ol.reference_fp4_swiglu(gate, up, down, H, I, x, threads=cores,
+                                                 bf16_intermediate=True, repeats=8)
+        linear_note = ("FP4 linears: reference CPU executor (fp4_host_executor.cpp, ABI-3 "
+                       "weights x Q8, AVX2) on one layer's SwiGLU block, best of 8, scaled "
+                       "by weight bytes to 7 linears x 64 layers + lm_head")
+    else:
+        codes = rng.integers(0, 256, (I // 8, H // 2), dtype=np.uint8)
+        scales = np.exp(0.5 * rng.standard_normal((I // 8, H // 16))).astype(
             np.float16).view(np.uint16)
-        act = ol.bf16_round(rng.standard_normal((rows, k)).astype(np.float32))
-        matrices.append((codes, scales, n, k, act))
+        act = ol.bf16_round(x)
+        begin = time.perf_counter()
+        ol.fp4_linear_f64(codes, scales, 1, I // 8, H, act)
+        ffn_seconds = (time.perf_counter() - begin) * 8 * 3
+        linear_note = ("FP4 linears: oracle port (double precision) on 1/8 of one "
+                       "[17408, 5120] matrix, scaled by weight bytes")
+    linear_seconds = ffn_seconds * (MODEL["layers"] * layer_parameters +
+                                    head_parameters) / ffn_parameters
     keys = rng.standard_normal((CONTEXT + rows - 1, KV, d)).astype(np.float32)
     values = rng.standard_normal((CONTEXT + rows - 1, KV, d)).astype(np.float32)
     pages = synth.q4h_pages(keys, values, MODEL["kv_page_tokens"])
     query = rng.standard_normal((rows, Q, d)).astype(np.float32)
     shape = ol.AttentionShape(rows, Q, KV, d, CONTEXT, MODEL["kv_page_tokens"], 0, 0)
-    sample_layers = 6
     begin = time.perf_counter()
-    for _ in range(sample_layers):
-        for codes, scales, n, k, act in matrices:
-            ol.fp4_linear_f64(codes, scales, 1, n, k, act)
-        ol.attention_q4h(shape, query, pages, "f64")
-    layer_seconds = (time.perf_counter() - begin) / sample_layers
-    # lm_head: one eighth of the vocabulary rows, scaled
-    head_rows = MODEL["vocabulary"] // 8
-    codes = rng.integers(0, 256, (head_rows, H // 2), dtype=np.uint8)
-    scales = np.exp(0.5 * rng.standard_normal((head_rows, H // 16))).astype(
-        np.float16).view(np.uint16)
-    act = ol.bf16_round(rng.standard_normal((rows, H)).astype(np.float32))
-    begin = time.perf_counter()
-    ol.fp4_linear_f64(codes, scales, 1, head_rows, H, act)
-    head_seconds = (time.perf_counter() - begin) * 8
-    step_seconds = MODEL["layers"] * layer_seconds + head_seconds
+    ol.attention_q4h(shape, query, pages, "f64")
+    attention_seconds = (time.perf_counter() - begin) * MODEL["layers"]
+    step_seconds = linear_seconds + attention_seconds
     return {
         "value": 1.0 / step_seconds,
         "unit": "tok/s",
-        "cores": int(ol.oracle().qo_num_threads()),
-        "kind": "port",
-        "sample": (f"{sample_layers} of {MODEL['layers']} layers (seven FP4 linears at "
-                   f"M={rows} + Q4H attention at {CONTEXT} tokens each) and 1/8 of the "
-                   "lm_head rows, scaled to one step emitting 1 token; CPU oracle in "
-                   "double precision, OpenMP"),
+        "cores": cores,
+        "kind": "reference" if reference else "port",
+        "sample": (linear_note + f"; Q4H attention at {CONTEXT} tokens: the reference has "
+                   "no CPU attention, so the oracle port (double precision, OpenMP) on "
+                   "one layer, x 64; one step emitting 1 token"),
         "seconds_per_step": step_seconds,
+        "linears_seconds_per_step": linear_seconds,
+        "attention_seconds_per_step": attention_seconds,
+        "linears_only_tok_s": 1.0 / linear_seconds,
     }
+
+
+def measure_long_contexts(qp, np, rows):
+    """tok/s of the same 64-layer verify step with the Q4H cache prefilled to
+    131072 tokens, and the exact-F16 attention kernel over 262144 tokens
+    (1.07 GB of K/V per layer; 4 layers of cache, so consecutive launches read
+    different memory)."""
+    report = {}
+    context = 131072
+    steps, warmup = 10, 2
+    geometry = dict(MODEL)
+    geometry["max_context"] = context + (steps + warmup + 2) * rows + 256
+    geometry["max_context"] = (geometry["max_context"] + 255) // 256 * 256
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(20241125)
+    provider.prefill_synthetic_kv(context, 7)
+    provider.prepare_exact_decode("decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2")
+    provider.begin_request(temperature_ppm=0)
+    rng = np.random.default_rng(2)
+    token, position = 1, context
+    provider.synchronize(token, position)
+    emitted = 0
+    begin = None
+    for index in range(steps + warmup):
+        if index == warmup:
+            provider.synchronize_stream()
+            begin = time.perf_counter()
+        provider.set_drafts(rng.integers(0, MODEL["vocabulary"],
+                                         MODEL["draft_depth"]).astype(np.uint32))
+        tokens, token, advanced = provider.verify(token, position, geometry["max_context"])
+        position += advanced
+        if index >= warmup:
+            emitted += len(tokens)
+    provider.synchronize_stream()
+    elapsed = time.perf_counter() - begin
+    attention_us, _ = provider.time_kernel("attention", 2, context)
+    attention_bytes = context * MODEL["kv_heads"] * 2 * (MODEL["head_dim"] // 2 + 2)
+    report["q4h_131072"] = {
+        "tok_s": round(emitted / elapsed, 2),
+        "ms_per_step": round(1000.0 * elapsed / steps, 4),
+        "projected_tok_s_at_reference_acceptance_2.6667": round(
+            2.6667 * steps / elapsed, 1),
+        "attention_avg_launch_us": round(attention_us, 2),
+        "attention_GBps": round(attention_bytes / attention_us / 1e3, 1),
+        "attention_frac": round(attention_bytes / attention_us / 1e3 / HBM_PEAK_GBS, 4),
+    }
+    provider.close()
+
+    context = 262144
+    geometry = dict(MODEL)
+    geometry.update(layers=4, kv_encoding=1, max_context=context + 512)
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(3)
+    provider.prefill_synthetic_kv(context, 9)
+    attention_us, launches = provider.time_kernel("attention", 3, context)
+    attention_bytes = context * MODEL["kv_heads"] * MODEL["head_dim"] * 2 * 2
+    report["f16_attention_262144"] = {
+        "avg_launch_us": round(attention_us, 2),
+        "launches_timed": launches,
+        "algorithmic_bytes_per_launch": attention_bytes,
+        "achieved_GBps": round(attention_bytes / attention_us / 1e3, 1),
+        "frac": round(attention_bytes / attention_us / 1e3 / HBM_PEAK_GBS, 4),
+    }
+    provider.close()
+    return report
 
 
 def main():
@@ -105,6 +190,9 @@ def main():
     parser.add_argument("--layers", type=int, default=MODEL["layers"],
                         help="for quick experiments only; the reported config is 64")
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--skip-long-contexts", action="store_true",
+                        help="skip the 131072-token step and the 262144-token F16 "
+                             "attention measurements")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one 256 MiB device copy (a kernel of known "
                              "traffic to scale hardware counters by)")
@@ -194,7 +282,15 @@ def main():
                                "achieved_GBps": round(bytes_per_launch / us / 1e3, 1),
                                "frac": round(bytes_per_launch / us / 1e3 / HBM_PEAK_GBS, 4)}
 
+    # the other contexts of the metric: the same step at 131072 tokens (Q4H) and
+    # the exact-F16 attention kernel at 262144 tokens, on providers of their own
     weight_bytes = provider.weight_bytes()
+    accepted_drafts = int(provider.telemetry("provider_accepted_drafts"))
+    long_context = {}
+    if arguments.layers == MODEL["layers"] and not arguments.skip_long_contexts:
+        provider.close()
+        provider = None
+        long_context = measure_long_contexts(qp, np, rows)
     layers = geometry["layers"]
     step_bytes = (layers * (fp4_bytes(MODEL["query_heads"] * 128, H) +
                             2 * fp4_bytes(MODEL["kv_heads"] * 128, H) +
@@ -223,7 +319,7 @@ def main():
             "context_tokens": CONTEXT,
             "rows": rows,
             "emitted_tokens": emitted_tokens,
-            "accepted_drafts": int(provider.telemetry("provider_accepted_drafts")),
+            "accepted_drafts": accepted_drafts,
             "weight_bytes": int(weight_bytes),
             "algorithmic_bytes_per_step": int(step_bytes),
             "step_hbm_GBps": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
@@ -236,7 +332,10 @@ def main():
         "roofline": roofline,
         "kernels": other_kernels,
     }
-    provider.close()
+    if provider is not None:
+        provider.close()
+    if long_context:
+        result["long_context"] = long_context
     if arguments.calibration_copy:
         source = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
         target = torch.empty_like(source)

@@ -826,6 +826,28 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
         status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
                                         hidden_bytes, logits_, QLLM_OUT_F32,
                                         nullptr, rows, stream_));
+      } else if (which == "attention" && g_.kv_encoding == KvEncoding::fp16) {
+        qllm_f16_attention_launch launch{};
+        launch.query = query_;
+        launch.device_pages = const_cast<const void* const*>(device_page_table_);
+        launch.output = attention_;
+        launch.partial_maxima = partial_maxima_;
+        launch.partial_sums = partial_sums_;
+        launch.partial_outputs = partial_outputs_;
+        launch.first_context_tokens = context_tokens + 1U;
+        launch.rows = rows;
+        launch.device_page_layer = index % g_.layers;
+        launch.device_page_tokens = g_.kv_page_tokens;
+        launch.query_heads = g_.query_heads;
+        launch.kv_heads = g_.kv_heads;
+        launch.head_dim = g_.head_dim;
+        launch.split_tokens = split_tokens_;
+        launch.maximum_splits = maximum_splits_;
+        launch.query_stride = query_stride;
+        launch.output_gated = g_.output_gated;
+        launch.output_kind = QLLM_OUT_BF16;
+        launch.stream = stream_;
+        status_check(qllm_attention_paged_f16(&launch));
       } else if (which == "attention") {
         qllm_q4h_attention_launch launch{};
         launch.query = query_;

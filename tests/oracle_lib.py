@@ -109,6 +109,42 @@ def _p(array: np.ndarray):
     return array.ctypes.data_as(c_void_p)
 
 
+def reference_fp4_swiglu(gate, up, down, hidden, intermediate, inputs, threads=1,
+                         bf16_intermediate=False, repeats=1):
+    """down(silu(gate x) * up x) by the reference's own CPU executor
+    (runtime/src/cpu/fp4_host_executor.cpp) compiled into oracle/_ref.
+    gate/up/down = (codes, scales) of ABI-3 matrices; returns (out, seconds of
+    the best call).  Raises if the reference library was not built."""
+    library = ref()
+    if library is None or not hasattr(library, "qref_fp4_swiglu"):
+        raise RuntimeError("oracle/_ref/libqllm_ref.so is not built")
+    sections = [np.ascontiguousarray(part).view(np.uint8).ravel()
+                for matrix in (gate, up, down) for part in matrix]
+    offsets, cursor = [], 0
+    for section in sections:
+        offsets.append(cursor)
+        cursor += (section.size + 63) // 64 * 64
+    record = np.zeros(cursor, dtype=np.uint8)
+    for offset, section in zip(offsets, sections):
+        record[offset: offset + section.size] = section
+    offsets = np.array(offsets, dtype=np.uint64)
+    inputs = np.ascontiguousarray(inputs, dtype=np.float32)
+    rows = inputs.shape[0]
+    out = np.zeros((rows, hidden), dtype=np.float32)
+    seconds = c_double(0.0)
+    library.qref_fp4_swiglu.restype = c_int
+    library.qref_fp4_swiglu.argtypes = [
+        c_void_p, c_uint64, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32,
+        c_void_p, c_uint32, c_int, c_uint32, ctypes.POINTER(c_double)]
+    status = library.qref_fp4_swiglu(_p(record), record.size, _p(offsets), hidden,
+                                     intermediate, _p(inputs), rows, _p(out), threads,
+                                     int(bf16_intermediate), repeats,
+                                     ctypes.byref(seconds))
+    if status != 0:
+        raise RuntimeError(f"reference FP4 executor failed ({status})")
+    return out, seconds.value
+
+
 # ---- numpy-facing wrappers ------------------------------------------------
 
 def bf16_round(x: np.ndarray) -> np.ndarray:

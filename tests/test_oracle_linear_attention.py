@@ -3,6 +3,7 @@ numpy float64 restatements built from library routines (table lookup + matmul,
 scipy softmax), against the reference's closed-form smoke fixtures, and through
 identities a wrong index or a dropped term would break."""
 import numpy as np
+import pytest
 from scipy.special import softmax
 
 import oracle_lib as ol
@@ -280,3 +281,32 @@ def test_silu_product_and_embedding():
         got = ol.fp4_embedding(codes, scales, scheme, 64, 64, tokens)
         want = synth.dequantize(codes, scales, scheme)[tokens]
         assert np.array_equal(got, want.astype(np.float32))
+
+
+@pytest.mark.skipif(ol.ref() is None or not hasattr(ol.ref(), "qref_fp4_swiglu"),
+                    reason="oracle/_ref (built from the reference tree) is absent")
+@pytest.mark.parametrize("bf16_intermediate", [False, True])
+def test_q8_linear_matches_the_reference_cpu_executor(bf16_intermediate):
+    """The reference's own all-core FP4 x Q8 SwiGLU executor
+    (runtime/src/cpu/fp4_host_executor.cpp), compiled from its source, against
+    the oracle's statement of the same three linears: Q8 rows -> gate/up ->
+    silu(g)*u -> Q8 -> down."""
+    rng = np.random.default_rng(21 + bf16_intermediate)
+    hidden, intermediate, rows = 256, 448, 5
+    scheme = ol.SCALE_UE8M0_BLOCK32
+    gate = synth.fp4_matrix(rng, intermediate, hidden, scheme)
+    up = synth.fp4_matrix(rng, intermediate, hidden, scheme)
+    down = synth.fp4_matrix(rng, hidden, intermediate, scheme)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    got, _ = ol.reference_fp4_swiglu(gate, up, down, hidden, intermediate, x,
+                                     threads=3, bf16_intermediate=bf16_intermediate)
+    q, s = ol.quantize_q8_rows(x, hidden)
+    g = ol.fp4_linear_block32_q8(*gate, intermediate, hidden, q, s)
+    u = ol.fp4_linear_block32_q8(*up, intermediate, hidden, q, s)
+    act = (g / (1.0 + np.exp(-g.astype(np.float64)))).astype(np.float32) * u
+    if bf16_intermediate:
+        act = ol.bf16_round(act)
+    q2, s2 = ol.quantize_q8_rows(act, intermediate)
+    want = ol.fp4_linear_block32_q8(*down, hidden, intermediate, q2, s2)
+    # identical integer block sums; F32 accumulation order and expf differ
+    assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max()
