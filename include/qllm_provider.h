@@ -148,6 +148,49 @@ uint64_t qllm_provider_weight_bytes(const qllm_provider* provider);
 uint64_t qllm_provider_telemetry(const qllm_provider* provider,
                                  const char* name);
 
+/* ---- host sampling mathematics of the verify step -------------------------
+ * The four functions of runtime/include/expert/runtime/speculative_sampling.hpp
+ * (make_sampling_distribution :23-27, sample_distribution :29-30,
+ * rejection_sample :42-45, counter_uniform :49-52) as the provider links them.
+ * They run on the host and need no device.  Distributions cross the boundary
+ * as parallel arrays (token ids, double probabilities).  A std::invalid_argument
+ * of the reference becomes QLLM_INVALID_ARGUMENT, a std::runtime_error
+ * QLLM_INTERNAL; the text is left in qllm_provider_last_error(). */
+
+/* Candidates sorted by descending logit (ties: ascending id).  Writes the
+ * retained entries to tokens_out / probabilities_out (capacity >= count) and
+ * their number to count_out. */
+int32_t qllm_sampling_make_distribution(const float* sorted_logits,
+                                        const uint32_t* sorted_tokens,
+                                        uint32_t count,
+                                        uint32_t temperature_ppm,
+                                        uint32_t top_p_ppm, uint32_t min_p_ppm,
+                                        uint32_t* tokens_out,
+                                        double* probabilities_out,
+                                        uint32_t* count_out);
+/* Inverse-CDF draw in entry order with uniform in [0, 1). */
+int32_t qllm_sampling_sample(const uint32_t* tokens,
+                             const double* probabilities, uint32_t count,
+                             double uniform, uint32_t* token_out);
+/* Leviathan rejection step: accept `proposal` with min(1, p/q), else draw from
+ * the normalised residual max(p - q, 0). */
+int32_t qllm_sampling_rejection(uint32_t proposal,
+                                const uint32_t* target_tokens,
+                                const double* target_probabilities,
+                                uint32_t target_count,
+                                const uint32_t* draft_tokens,
+                                const double* draft_probabilities,
+                                uint32_t draft_count,
+                                double acceptance_uniform,
+                                double correction_uniform, int32_t* accepted_out,
+                                uint32_t* token_out,
+                                double* target_probability_out,
+                                double* draft_probability_out);
+/* Counter-based uniform in [0, 1): splitmix64 over (seed, position, stream,
+ * index), top 53 bits. */
+double qllm_sampling_counter_uniform(uint64_t seed, uint32_t position,
+                                     uint32_t stream, uint32_t index);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -367,4 +368,96 @@ extern "C" uint64_t qllm_provider_telemetry(const qllm_provider* provider,
   const auto values = provider->provider->telemetry();
   const auto found = values.find(name);
   return found == values.end() ? 0U : found->second;
+}
+
+// ---- host sampling mathematics ----------------------------------------------
+
+namespace {
+
+er::SamplingDistribution distribution_from(const uint32_t* tokens,
+                                           const double* probabilities,
+                                           uint32_t count) {
+  er::SamplingDistribution distribution;
+  distribution.entries.reserve(count);
+  for (uint32_t i = 0; i < count; ++i)
+    distribution.entries.push_back({tokens[i], probabilities[i]});
+  return distribution;
+}
+
+template <typename Body>
+int32_t guarded(Body&& body) {
+  try {
+    body();
+    return QLLM_OK;
+  } catch (const std::invalid_argument& error) {
+    return fail(QLLM_INVALID_ARGUMENT, error.what());
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+}  // namespace
+
+extern "C" int32_t qllm_sampling_make_distribution(
+    const float* sorted_logits, const uint32_t* sorted_tokens, uint32_t count,
+    uint32_t temperature_ppm, uint32_t top_p_ppm, uint32_t min_p_ppm,
+    uint32_t* tokens_out, double* probabilities_out, uint32_t* count_out) {
+  if ((count && (!sorted_logits || !sorted_tokens || !tokens_out ||
+                 !probabilities_out)) || !count_out)
+    return fail(QLLM_INVALID_ARGUMENT, "null sampling buffer");
+  return guarded([&] {
+    const auto distribution = er::make_sampling_distribution(
+        {sorted_logits, count}, {sorted_tokens, count}, temperature_ppm,
+        top_p_ppm, min_p_ppm);
+    *count_out = static_cast<uint32_t>(distribution.entries.size());
+    for (std::size_t i = 0; i < distribution.entries.size(); ++i) {
+      tokens_out[i] = distribution.entries[i].token;
+      probabilities_out[i] = distribution.entries[i].probability;
+    }
+  });
+}
+
+extern "C" int32_t qllm_sampling_sample(const uint32_t* tokens,
+                                        const double* probabilities,
+                                        uint32_t count, double uniform,
+                                        uint32_t* token_out) {
+  if ((count && (!tokens || !probabilities)) || !token_out)
+    return fail(QLLM_INVALID_ARGUMENT, "null sampling buffer");
+  return guarded([&] {
+    *token_out = er::sample_distribution(
+        distribution_from(tokens, probabilities, count), uniform);
+  });
+}
+
+extern "C" int32_t qllm_sampling_rejection(
+    uint32_t proposal, const uint32_t* target_tokens,
+    const double* target_probabilities, uint32_t target_count,
+    const uint32_t* draft_tokens, const double* draft_probabilities,
+    uint32_t draft_count, double acceptance_uniform, double correction_uniform,
+    int32_t* accepted_out, uint32_t* token_out, double* target_probability_out,
+    double* draft_probability_out) {
+  if ((target_count && (!target_tokens || !target_probabilities)) ||
+      (draft_count && (!draft_tokens || !draft_probabilities)) ||
+      !accepted_out || !token_out)
+    return fail(QLLM_INVALID_ARGUMENT, "null sampling buffer");
+  return guarded([&] {
+    const auto result = er::rejection_sample(
+        proposal,
+        distribution_from(target_tokens, target_probabilities, target_count),
+        distribution_from(draft_tokens, draft_probabilities, draft_count),
+        acceptance_uniform, correction_uniform);
+    *accepted_out = result.accepted ? 1 : 0;
+    *token_out = result.token;
+    if (target_probability_out)
+      *target_probability_out = result.target_probability;
+    if (draft_probability_out)
+      *draft_probability_out = result.draft_probability;
+  });
+}
+
+extern "C" double qllm_sampling_counter_uniform(uint64_t seed,
+                                                uint32_t position,
+                                                uint32_t stream,
+                                                uint32_t index) {
+  return er::counter_uniform(seed, position, stream, index);
 }

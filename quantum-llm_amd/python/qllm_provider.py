@@ -58,6 +58,10 @@ SIGNATURES = {
     "qllm_provider_stream": (c_void_p, [c_void_p]),
     "qllm_provider_weight_bytes": (c_uint64, [c_void_p]),
     "qllm_provider_telemetry": (c_uint64, [c_void_p, c_char_p]),
+    "qllm_sampling_make_distribution": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, POINTER(c_uint32)]),
+    "qllm_sampling_sample": (c_int32, [c_void_p, c_void_p, c_uint32, c_double, POINTER(c_uint32)]),
+    "qllm_sampling_rejection": (c_int32, [c_uint32, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_double, c_double, POINTER(c_int32), POINTER(c_uint32), POINTER(c_double), POINTER(c_double)]),
+    "qllm_sampling_counter_uniform": (c_double, [c_uint64, c_uint32, c_uint32, c_uint32]),
 }
 
 _library = None
@@ -231,3 +235,57 @@ def capabilities():
     raw = buffer.raw
     names = [part.decode() for part in raw.split(b"\0") if part][:count]
     return names
+
+
+# ---- host sampling mathematics (no device needed) ----------------------------
+
+def _arrays(tokens, probabilities):
+    import numpy as np
+    t = np.ascontiguousarray(tokens, dtype=np.uint32)
+    p = np.ascontiguousarray(probabilities, dtype=np.float64)
+    return t, p
+
+
+def make_sampling_distribution(sorted_logits, sorted_tokens, temperature_ppm,
+                               top_p_ppm, min_p_ppm):
+    """Returns (tokens, probabilities); raises ProviderError on invalid input."""
+    import numpy as np
+    logits = np.ascontiguousarray(sorted_logits, dtype=np.float32)
+    tokens = np.ascontiguousarray(sorted_tokens, dtype=np.uint32)
+    out_tokens = np.zeros(max(len(tokens), 1), dtype=np.uint32)
+    out_probabilities = np.zeros(max(len(tokens), 1), dtype=np.float64)
+    count = c_uint32(0)
+    _check(load().qllm_sampling_make_distribution(
+        logits.ctypes.data, tokens.ctypes.data, len(tokens), temperature_ppm,
+        top_p_ppm, min_p_ppm, out_tokens.ctypes.data,
+        out_probabilities.ctypes.data, ctypes.byref(count)))
+    return (out_tokens[:count.value].tolist(),
+            out_probabilities[:count.value].tolist())
+
+
+def sample_distribution(tokens, probabilities, uniform):
+    t, p = _arrays(tokens, probabilities)
+    token = c_uint32(0)
+    _check(load().qllm_sampling_sample(t.ctypes.data, p.ctypes.data, len(t),
+                                       uniform, ctypes.byref(token)))
+    return token.value
+
+
+def rejection_sample(proposal, target, draft, acceptance_uniform,
+                     correction_uniform):
+    """target / draft: (tokens, probabilities).  Returns (accepted, token,
+    target probability, draft probability) of the proposal."""
+    tt, tp = _arrays(*target)
+    dt, dp = _arrays(*draft)
+    accepted, token = c_int32(0), c_uint32(0)
+    p, q = c_double(0.0), c_double(0.0)
+    _check(load().qllm_sampling_rejection(
+        proposal, tt.ctypes.data, tp.ctypes.data, len(tt), dt.ctypes.data,
+        dp.ctypes.data, len(dt), acceptance_uniform, correction_uniform,
+        ctypes.byref(accepted), ctypes.byref(token), ctypes.byref(p),
+        ctypes.byref(q)))
+    return bool(accepted.value), token.value, p.value, q.value
+
+
+def counter_uniform(seed, position, stream, index=0):
+    return load().qllm_sampling_counter_uniform(seed, position, stream, index)
