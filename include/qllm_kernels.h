@@ -80,18 +80,18 @@ typedef struct qllm_fp4_matrix {
   uint32_t padded_columns;
   uint32_t scale_scheme;  /* enum qllm_scale_scheme */
   uint32_t layout;        /* enum qllm_fp4_layout */
-  uint32_t tile_rows;     /* tiled layout: rows per tile, 8..32 (0 = 32) */
+  uint32_t tile_rows;     /* tiled layout: rows per tile, even, 8..32 (0 = 32) */
 } qllm_fp4_matrix;
 
-/* Device bytes needed for the tiled copy of a matrix; tile_rows in 8..32,
- * 0 = 32. */
+/* Device bytes needed for the tiled copy of a matrix; tile_rows even in
+ * 8..32, 0 = 32; other heights return 0. */
 size_t qllm_fp4_packed_weight_bytes(uint32_t rows, uint32_t padded_columns,
                                     uint32_t tile_rows);
 size_t qllm_fp4_packed_scale_bytes(uint32_t rows, uint32_t padded_columns,
                                    uint32_t scale_scheme, uint32_t tile_rows);
 
 /* Re-lays a row-major matrix (padded_columns % 64 == 0) into the tiled
- * layout with tiles of tile_rows rows (8..32, 0 = 32); `packed`
+ * layout with tiles of tile_rows rows (even, 8..32, 0 = 32); `packed`
  * (host struct) receives the descriptor of the copy.  This is the device half
  * of the provider's tensor upload
  * (runtime/tools/dense_fp4_provider.cpp:3486-3660); it moves bytes and changes

@@ -68,8 +68,7 @@ struct GemmArgs {
   uint32_t rows;
   uint32_t padded_columns;
   uint32_t output_kind;
-  uint32_t swiglu;              // tile 1 is the up projection of tile 0
-  uint32_t tile_rows;           // weight rows per tile, 8..32
+  uint32_t tile_rows;           // weight rows per tile: even, 8..32
   // Optional split of the output rows over up to three buffers (the q, k and
   // v projections stored as one matrix): segment s takes the next
   // segment_rows[s] rows.  segments == 0: everything goes to `output`.
@@ -91,119 +90,160 @@ __device__ __forceinline__ void store_output(void* output, uint32_t kind,
     static_cast<float*>(output)[index] = value;
 }
 
-// Workgroup = WAVES waves.  The workgroup owns TILES tiles of h = tile_rows
-// (at most 32) weight rows - lanes n >= h repeat row h-1 and are ignored;
-// its waves interleave over 64-column chunks of K (wave w takes chunks
-// w, w+WAVES, ...).  Lane (n = lane%32, g = lane/32) supplies, for each of the
-// chunk's four 16-blocks b, the half g (8 weights = 4 bytes) of row n - the
-// B-operand layout of the 32x32x16 MFMA.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// 4x4 transpose of dwords across the four 16-lane rows of a wave: on return
+// register d of row c holds what register c of row d held.
+__device__ __forceinline__ void transpose_rows4(uint32_t (&v)[4]) {
+  const auto a = __builtin_amdgcn_permlane32_swap(v[0], v[2], false, false);
+  const auto b = __builtin_amdgcn_permlane32_swap(v[1], v[3], false, false);
+  const auto c = __builtin_amdgcn_permlane16_swap(a[0], b[0], false, false);
+  const auto d = __builtin_amdgcn_permlane16_swap(a[1], b[1], false, false);
+  v[0] = c[0]; v[1] = c[1]; v[2] = d[0]; v[3] = d[1];
+}
+
+// Workgroup = WAVES waves, one tile of h = tile_rows weight rows (for the fused
+// SwiGLU pair: the gate tile and the up tile of the same rows).  Its waves
+// interleave over 64-column chunks of K (wave w takes chunks w, w+WAVES, ...).
 //
-// TILED selects the provider's streaming layout (see qllm_fp4_prepack): the
-// 64 sixteen-byte pieces a wave loads for one (tile, chunk) are contiguous
-// (one 1 KiB burst) and already hold the lane's four half-blocks.  With the
-// row-major layout lane (n, g) loads the 16 bytes at row n, byte offset
-// chunk*32 + g*16 (64 separate requests) and one v_permlane32_swap per dword
-// pair regroups them.
+// The contraction runs on v_mfma_f32_16x16x32_bf16.  One instruction takes 16
+// weight rows (N side) and 32 columns of K, i.e. two 16-blocks that carry
+// different binary16 scales.  The M side has 16 rows and the batch at most 8,
+// so the two blocks are kept apart there: MFMA rows 0..7 see the activations
+// of the first block and zeros for the second, rows 8..15 the opposite.  The
+// result then holds the two per-block partial sums in different lanes (row
+// groups 0,1 / 2,3), each is scaled in F32 by its own block scale, and the two
+// halves are added once after the K loop.  A chunk of one tile is four such
+// instructions (j = first / second half of the tile's rows, s = columns 0..31 /
+// 32..63); a half has h/2 <= 16 rows, lanes n >= h/2 repeat the last row and
+// are ignored.
+//
+// Lane (n = lane%16, g = lane/16) supplies to instruction (j, s) the 8 weights
+// (4 bytes) of row j*h/2 + n, columns 32s+8g..+8, and needs the scale of block
+// 2s + g/2 of that row.  TILED selects the provider's streaming layout (see
+// qllm_fp4_prepack): the 64 sixteen-byte pieces a wave loads for one (tile,
+// chunk) are contiguous (one 1 KiB burst) and hold the lane's four dwords in
+// (j, s) order, scales likewise.  With the row-major layout lane (n, g) loads
+// the 16 bytes of row 16(g/2)+n at byte chunk*32 + (g%2)*16 and a 4x4 dword
+// transpose across the four lane rows regroups them (h is 32 there).
 //
 // Activations travel with the weights: together with the weight pieces of a
 // chunk a wave prefetches the batch x 64 activation values of that chunk
 // (8*batch sixteen-byte pieces, one per lane), drops them into a small
-// wave-private LDS ring in MFMA A-fragment order and reads the four 16-block
-// fragments back.  Nothing is staged per workgroup, so there is no barrier in
-// the K loop and any K that is a multiple of 64 is handled alike.
+// wave-private LDS ring and reads the two A fragments back; lanes whose MFMA
+// row belongs to the other block (or to no batch row) read a zero piece kept
+// in the same ring slot.  Nothing is staged per workgroup, so there is no
+// barrier in the K loop and any K that is a multiple of 64 is handled alike.
 //
-// Every block's MFMA starts from zero and its result is scaled in F32 by the
-// block's binary16 scale, so only the accumulator registers that hold batch
-// rows cost an FMA.  Batches of up to 6 rows sit in MFMA rows {0,1,2,4,5,6}:
-// those are registers 0..2 of both lane halves, one FMA fewer than rows 0..5.
+// Batches of up to 6 rows sit in MFMA rows {0,1,2,4,5,6} of each half: those
+// are accumulator registers 0..2 of both row groups, one FMA fewer than rows
+// 0..5 would cost.
 template <int SCHEME, int BATCH, int TILES, int WAVES, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     const GemmArgs args) {
-  // chunks in flight per lane; three with two tiles per group, which keeps
-  // the kernel at three workgroups per CU so that the 544 groups of the fused
-  // gate/up launch are all resident at once
-  constexpr int PF = TILES == 2 ? 3 : 4;
-  constexpr int PIECES = 8 * BATCH; // activation pieces per chunk
+  constexpr int PF = 4;                // chunks in flight per lane
+  constexpr int PIECES = 8 * BATCH;    // activation pieces per chunk
   constexpr bool COMPACT = BATCH <= 6;
   constexpr int REGS = COMPACT ? 3 : 4;  // accumulator registers in use
-  // ring slot: PIECES pieces of 16 bytes, padded to 64 pieces
-  __shared__ __attribute__((aligned(16))) uint4 ring[WAVES][2][64];
-  __shared__ float reduce[WAVES][TILES][REGS][64];
+  constexpr int kZeroPiece = 64;
+  constexpr bool F16 = SCHEME == kSchemeF16;
+  // scale registers per (slot, tile): tiled = the lane's four scales;
+  // row-major = the chunk's scales of rows n and 16+n
+  constexpr int SCALE_WORDS = TILED ? (F16 ? 2 : 1) : (F16 ? 4 : 2);
+  __shared__ __attribute__((aligned(16))) uint4 ring[WAVES][2][kZeroPiece + 1];
+  __shared__ float reduce[WAVES][TILES][2][REGS][32];
 
   const uint32_t lane = threadIdx.x & 63u;
   // wave index as a scalar, so everything derived from it (chunk counts,
   // loop bounds, addresses) is uniform
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t n = lane & 31u;
-  const uint32_t g = lane >> 5;
+  const uint32_t n = lane & 15u;
+  const uint32_t g = lane >> 4;
   const uint32_t K = args.padded_columns;
   const uint32_t row_bytes = K / 2u;
-  const uint32_t scale_row_bytes =
-      SCHEME == kSchemeF16 ? K / 8u : K / 32u;
-  // batch row carried by MFMA row n on the A side (rows past the batch are
-  // don't-care and repeat the last one)
-  uint32_t batch_row = COMPACT ? (n >> 2) * 3u + (n & 3u) : n;
-  if (batch_row >= BATCH) batch_row = BATCH - 1u;
+  const uint32_t scale_row_bytes = F16 ? K / 8u : K / 32u;
+  constexpr uint32_t kScaleChunk = F16 ? 8u : 2u;   // scale bytes per row, chunk
+  const uint32_t h = args.tile_rows;
+  const uint32_t half_rows = h / 2u;
+  const uint32_t tile_lane = n < half_rows ? n : half_rows - 1u;
+  const uint32_t first_row = blockIdx.x * h;
 
   // Weight and scale streams: wave-uniform start of the tile's stream plus a
   // 32-bit lane offset; consecutive chunks are weight_step / scale_step apart.
-  constexpr uint32_t kScaleChunk = SCHEME == kSchemeF16 ? 8u : 2u;
-  const uint32_t h = args.tile_rows;
-  const uint32_t tile_lane = n < h ? n : h - 1u;
   const uint32_t weight_step = TILED ? 32u * h : 32u;
   const uint32_t scale_step = TILED ? h * kScaleChunk : kScaleChunk;
   const uint8_t* weight_base[TILES];
   const uint8_t* scale_base[TILES];
-  uint32_t weight_lane[TILES];
-  uint32_t scale_lane[TILES];
+  uint32_t weight_lane, scale_lane[2];
+  if (TILED) {
+    weight_lane = (g * half_rows + tile_lane) * 16u;
+    scale_lane[0] = F16 ? ((g >> 1) * half_rows + tile_lane) * 8u : tile_lane * 4u;
+    scale_lane[1] = scale_lane[0];
+  } else {
+    const uint32_t last = args.rows - 1u - first_row;   // rows past the end repeat it
+    weight_lane = min((g >> 1) * 16u + n, last) * row_bytes + (g & 1u) * 16u;
+    scale_lane[0] = min(n, last) * scale_row_bytes;
+    scale_lane[1] = min(16u + n, last) * scale_row_bytes;
+  }
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
-    const uint32_t tile = args.swiglu ? blockIdx.x : blockIdx.x * TILES + t;
-    const uint32_t tiles = (args.rows + h - 1u) / h;
-    const uint32_t safe_tile = tile < tiles ? tile : tiles - 1u;
     if (TILED) {
-      const size_t first_chunk = static_cast<size_t>(safe_tile) * (K / kChunk);
+      const size_t first_chunk = static_cast<size_t>(blockIdx.x) * (K / kChunk);
       weight_base[t] = args.tile[t].weights + first_chunk * weight_step;
       scale_base[t] = args.tile[t].scales + first_chunk * scale_step;
-      weight_lane[t] = (g * h + tile_lane) * 16u;
-      scale_lane[t] = tile_lane * kScaleChunk;
     } else {
-      const uint32_t first_row = safe_tile * h;
-      const uint32_t row = min(first_row + tile_lane, args.rows - 1u) - first_row;
       weight_base[t] =
           args.tile[t].weights + static_cast<size_t>(first_row) * row_bytes;
       scale_base[t] =
           args.tile[t].scales + static_cast<size_t>(first_row) * scale_row_bytes;
-      weight_lane[t] = row * row_bytes + g * 16u;
-      scale_lane[t] = row * scale_row_bytes;
     }
   }
-  // activation piece this lane fetches per chunk: piece p = (block*2+half)*
-  // BATCH + m  ->  act[m][chunk*64 + (block*2+half)*8 .. +8]
+  // activation piece this lane fetches per chunk: piece p = octet*BATCH + m
+  //   ->  act[m][chunk*64 + octet*8 .. +8]
   const uint32_t piece = lane < PIECES ? lane : PIECES - 1u;
   const uint32_t activation_lane =
       ((piece % BATCH) * K + (piece / BATCH) * 8u) * 2u;
   const uint8_t* activation_base =
       reinterpret_cast<const uint8_t*>(args.activations);
+  // A fragment of span s: MFMA row n carries batch row m of block n/8; lane
+  // (n, g) holds columns 8g..8g+7 of the span, i.e. octet 4s+g, which belongs
+  // to block g/2.
+  uint32_t fragment_piece[2];
+  {
+    const uint32_t r = n & 7u;
+    const uint32_t m = COMPACT ? (r >> 2) * 3u + (r & 3u) : r;
+    const bool live =
+        m < BATCH && (!COMPACT || (r & 3u) < 3u) && (g >> 1) == (n >> 3);
+    fragment_piece[0] = live ? g * BATCH + m : kZeroPiece;
+    fragment_piece[1] = live ? (4u + g) * BATCH + m : kZeroPiece;
+  }
+  if (lane < 2u) ring[wave][lane][kZeroPiece] = make_uint4(0u, 0u, 0u, 0u);
 
-  // The residual of this thread's output item (see the epilogue) is fetched
+  // Output item of this thread (see the epilogue); its residual is fetched
   // now, so that the value is there when the K loop ends.
+  constexpr uint32_t kItems = 2u * REGS * 32u;
+  static_assert(kItems <= WAVES * 64u, "one output item per thread");
+  const uint32_t item_lane = threadIdx.x & 31u;
+  const uint32_t item_reg = (threadIdx.x >> 5) % REGS;
+  const uint32_t item_half = (threadIdx.x >> 5) / REGS;         // j
+  const uint32_t item_batch = (COMPACT ? 3u : 4u) * (item_lane >> 4) + item_reg;
+  const uint32_t item_row = first_row + item_half * half_rows + (item_lane & 15u);
+  const bool item_valid = threadIdx.x < kItems && item_batch < BATCH &&
+                          (item_lane & 15u) < half_rows && item_row < args.rows;
+  const size_t item_index = static_cast<size_t>(item_batch) * args.rows + item_row;
   float residual_value = 0.0f;
   if constexpr (TILES == 1) {
-    if (args.residual && !args.segments) {
-      const uint32_t reg = (threadIdx.x / 64u) % REGS;
-      const uint32_t batch = (COMPACT ? 3u : 4u) * (lane >> 5) + reg;
-      const uint32_t row = blockIdx.x * h + n;
-      if (threadIdx.x < REGS * 64u && batch < BATCH && n < h && row < args.rows)
-        residual_value = args.residual[static_cast<size_t>(batch) * args.rows + row];
-    }
+    if (args.residual && !args.segments && item_valid)
+      residual_value = args.residual[item_index];
   }
 
-  float acc[TILES][REGS];
+  float acc[TILES][2][REGS];
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < REGS; ++i) acc[t][i] = 0.0f;
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < REGS; ++i) acc[t][j][i] = 0.0f;
 
   const uint32_t chunks = K / kChunk;
   const uint32_t my_chunks =
@@ -214,22 +254,35 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint32_t last_index = my_chunks ? my_chunks - 1u : 0u;
 
   uint4 codes[PF][TILES];
-  uint2 scales[PF][TILES];
+  uint32_t scales[PF][TILES][SCALE_WORDS];
   uint4 activation[PF];
   auto issue = [&](int slot, uint32_t index) {
     const uint32_t chunk = wave + index * WAVES;   // uniform
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       codes[slot][t] = load_stream16(
-          weight_base[t] + static_cast<size_t>(chunk) * weight_step +
-          weight_lane[t]);
-      const uint8_t* scale_address =
-          scale_base[t] + static_cast<size_t>(chunk) * scale_step + scale_lane[t];
-      if (SCHEME == kSchemeF16) {
-        scales[slot][t] = load_stream8(scale_address);
+          weight_base[t] + static_cast<size_t>(chunk) * weight_step + weight_lane);
+      const uint8_t* scale_chunk =
+          scale_base[t] + static_cast<size_t>(chunk) * scale_step;
+      if (TILED && F16) {
+        const uint2 v = load_stream8(scale_chunk + scale_lane[0]);
+        scales[slot][t][0] = v.x;
+        scales[slot][t][1] = v.y;
+      } else if (TILED) {
+        scales[slot][t][0] =
+            *reinterpret_cast<const uint32_t*>(scale_chunk + scale_lane[0]);
+      } else if (F16) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const uint2 v = load_stream8(scale_chunk + scale_lane[j]);
+          scales[slot][t][2 * j] = v.x;
+          scales[slot][t][2 * j + 1] = v.y;
+        }
       } else {
-        const uint32_t pair = *reinterpret_cast<const uint16_t*>(scale_address);
-        scales[slot][t] = make_uint2(pair & 0xffu, pair >> 8);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          scales[slot][t][j] =
+              *reinterpret_cast<const uint16_t*>(scale_chunk + scale_lane[j]);
       }
     }
     activation[slot] = *reinterpret_cast<const uint4*>(
@@ -246,11 +299,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       for (int slot = 0; slot < PF; ++slot) {
         const uint32_t index = base + slot;
         uint4 q[TILES];
-        uint2 s[TILES];
+        uint32_t s[TILES][SCALE_WORDS];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
           q[t] = codes[slot][t];
-          s[t] = scales[slot][t];
+#pragma unroll
+          for (int w = 0; w < SCALE_WORDS; ++w) s[t][w] = scales[slot][t][w];
         }
         const uint4 x = activation[slot];
         issue(slot, min(index + PF, last_index));
@@ -260,93 +314,94 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
         uint4* stage = ring[wave][slot & 1];
         stage[lane] = x;
         __builtin_amdgcn_wave_barrier();
-        bf16x8 a[4];
+        bf16x8 a[2];
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
-          a[b] = __builtin_bit_cast(bf16x8,
-                                    stage[(b * 2u + g) * BATCH + batch_row]);
+        for (int span = 0; span < 2; ++span)
+          a[span] = __builtin_bit_cast(bf16x8, stage[fragment_piece[span]]);
         __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
-          uint32_t packed[4];  // half g of blocks 0..3 of row n
-          if (TILED) {
-            packed[0] = q[t].x; packed[1] = q[t].y;
-            packed[2] = q[t].z; packed[3] = q[t].w;
-          } else {
-            const auto s01 = __builtin_amdgcn_permlane32_swap(q[t].x, q[t].y,
-                                                              false, false);
-            const auto s23 = __builtin_amdgcn_permlane32_swap(q[t].z, q[t].w,
-                                                              false, false);
-            packed[0] = s01[0]; packed[1] = s23[0];
-            packed[2] = s01[1]; packed[3] = s23[1];
-          }
+          // packed[2j+s] = the lane's 8 weights for instruction (j, s);
+          // scale / fold [2j+s] likewise
+          uint32_t packed[4] = {q[t].x, q[t].y, q[t].z, q[t].w};
+          if (!TILED) transpose_rows4(packed);
           float scale[4];
           float fold[4];
-          if (SCHEME == kSchemeF16) {
+          if (F16) {
             // binary16 scale applied in F32 after the block's MFMA
-            scale[0] = f16_bits_to_f32(s[t].x & 0xffffu);
-            scale[1] = f16_bits_to_f32(s[t].x >> 16);
-            scale[2] = f16_bits_to_f32(s[t].y & 0xffffu);
-            scale[3] = f16_bits_to_f32(s[t].y >> 16);
+            uint32_t pair[2];   // scales of (j, 0), (j, 1) as two halves
+            if (TILED) {
+              pair[0] = s[t][0];
+              pair[1] = s[t][1];
+            } else {
+              // row j holds blocks 0..3 in two words; this lane wants blocks
+              // g/2 and 2 + g/2
+#pragma unroll
+              for (int j = 0; j < 2; ++j)
+                pair[j] = (g >> 1) ? (s[t][2 * j] >> 16) | (s[t][2 * j + 1] & 0xffff0000u)
+                                   : (s[t][2 * j] & 0xffffu) | (s[t][2 * j + 1] << 16);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              scale[2 * j] = f16_bits_to_f32(pair[j] & 0xffffu);
+              scale[2 * j + 1] = f16_bits_to_f32(pair[j] >> 16);
+            }
             fold[0] = fold[1] = fold[2] = fold[3] = 1.0f;
           } else {
             // power-of-two scale folded into the nibble->bf16 conversion
-            fold[0] = fold[1] = ue8m0_to_f32(s[t].x);
-            fold[2] = fold[3] = ue8m0_to_f32(s[t].y);
-            scale[0] = scale[1] = scale[2] = scale[3] = 1.0f;
-          }
-          f32x16 d[4];
+            const uint32_t bytes = TILED ? s[t][0] : s[t][0] | (s[t][1] << 16);
 #pragma unroll
-          for (int b = 0; b < 4; ++b) {
-            const bf16x8 w = expand_fp4x8(packed[b], fold[b]);
-            f32x16 zero;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) zero[i] = 0.0f;
-            d[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[b], w, zero, 0, 0, 0);
+            for (int k = 0; k < 4; ++k) {
+              fold[k] = ue8m0_to_f32((bytes >> (8 * k)) & 0xffu);
+              scale[k] = 1.0f;
+            }
           }
 #pragma unroll
-          for (int b = 0; b < 4; ++b)
+          for (int j = 0; j < 2; ++j) {
+            f32x4 d[2];
 #pragma unroll
-            for (int i = 0; i < REGS; ++i)
-              acc[t][i] = fmaf(d[b][i], scale[b], acc[t][i]);
+            for (int span = 0; span < 2; ++span) {
+              const bf16x8 w = expand_fp4x8(packed[2 * j + span], fold[2 * j + span]);
+              const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+              d[span] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[span], w, zero,
+                                                                0, 0, 0);
+            }
+#pragma unroll
+            for (int span = 0; span < 2; ++span)
+#pragma unroll
+              for (int i = 0; i < REGS; ++i)
+                acc[t][j][i] = fmaf(d[span][i], scale[2 * j + span], acc[t][j][i]);
+          }
         }
       }
     }
   }
 
-  // Cross-wave reduction through LDS.
+  // The two blocks of a span sit in lanes 32 apart: add them, then reduce
+  // across waves through LDS.  Lane (n, g < 2) register i now holds batch row
+  // (COMPACT ? 3 : 4) * g + i of weight row j*h/2 + n.
 #pragma unroll
   for (int t = 0; t < TILES; ++t)
 #pragma unroll
-    for (int i = 0; i < REGS; ++i) reduce[wave][t][i][lane] = acc[t][i];
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < REGS; ++i) {
+        const float total = acc[t][j][i] + __shfl_xor(acc[t][j][i], 32, kWave);
+        if (lane < 32u) reduce[wave][t][j][i][lane] = total;
+      }
   __syncthreads();
 
-  // Output item of this thread: item = (tile, register i, lane); lane (n, g)
-  // register i holds MFMA row 4*g + i, i.e. batch row (COMPACT ? 3 : 4)*g + i.
-  // (two tiles per workgroup are the gate/up pair: one output per row pair)
-  static_assert(TILES <= 2 && REGS * 64 <= WAVES * 64,
-                "one output item per thread");
-  const uint32_t items = (args.swiglu ? 1u : TILES) * REGS * 64u;
-  const uint32_t item_tile = threadIdx.x / (REGS * 64u);
-  const uint32_t item_reg = (threadIdx.x / 64u) % REGS;
-  const uint32_t item_lane = threadIdx.x & 63u;
-  const uint32_t item_batch = (COMPACT ? 3u : 4u) * (item_lane >> 5) + item_reg;
-  const uint32_t item_tile_row = item_lane & 31u;
-  const uint32_t item_row =
-      (args.swiglu ? blockIdx.x : blockIdx.x * TILES + item_tile) * h + item_tile_row;
-  const bool item_valid = threadIdx.x < items && item_batch < BATCH &&
-                          item_tile_row < h && item_row < args.rows;
-  const size_t item_index = static_cast<size_t>(item_batch) * args.rows + item_row;
   if (!item_valid) return;
   float total = 0.0f;
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) total += reduce[w][item_tile][item_reg][item_lane];
-  if (args.swiglu) {
+  for (int w = 0; w < WAVES; ++w) total += reduce[w][0][item_half][item_reg][item_lane];
+  if (TILES == 2) {
+    // tile 1 is the up projection of the same rows
     float up = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w)
-      up += reduce[w][TILES - 1][item_reg][item_lane];
+      up += reduce[w][TILES - 1][item_half][item_reg][item_lane];
     const float activated = bf16_round(total / (1.0f + __expf(-total)));
     static_cast<uint16_t*>(args.output)[item_index] =
         static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
@@ -448,6 +503,18 @@ __global__ __launch_bounds__(256) void fp4_gemv_generic_kernel(
   }
 }
 
+// Tile heights of the streaming layout: even, 8..32; 0 stands for 32.
+bool tile_rows_ok(uint32_t tile_rows) {
+  return tile_rows == 0u ||
+         (tile_rows >= 8u && tile_rows <= 32u && tile_rows % 2u == 0u);
+}
+
+uint32_t matrix_tile_rows(const qllm_fp4_matrix* matrix) {
+  return matrix->layout == QLLM_LAYOUT_TILED && matrix->tile_rows
+             ? matrix->tile_rows
+             : 32u;
+}
+
 bool matrix_ok(const qllm_fp4_matrix* m) {
   return m && m->weights && m->scales && m->rows && m->columns &&
          m->padded_columns >= m->columns && m->padded_columns % 32u == 0u &&
@@ -455,7 +522,7 @@ bool matrix_ok(const qllm_fp4_matrix* m) {
           m->scale_scheme == QLLM_SCALE_F16_BLOCK16) &&
          (m->layout == QLLM_LAYOUT_ROW_MAJOR ||
           (m->layout == QLLM_LAYOUT_TILED && m->padded_columns % kChunk == 0u &&
-           (m->tile_rows == 0u || (m->tile_rows >= 8u && m->tile_rows <= 32u))));
+           tile_rows_ok(m->tile_rows)));
 }
 
 template <int SCHEME, int BATCH, int TILES, bool TILED>
@@ -491,7 +558,6 @@ int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
                     bool swiglu, hipStream_t stream) {
   const uint32_t tiles = (args.rows + args.tile_rows - 1u) / args.tile_rows;
   const uint32_t waves = tiles <= 384u && !swiglu ? 8u : 4u;
-  args.swiglu = swiglu ? 1u : 0u;
 #define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
   return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
                                                     stream)
@@ -512,53 +578,66 @@ int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
 #undef QLLM_LAUNCH
 }
 
-uint32_t matrix_tile_rows(const qllm_fp4_matrix* matrix) {
-  if (matrix->layout == QLLM_LAYOUT_TILED)
-    return matrix->tile_rows ? matrix->tile_rows : 32u;
-  return 32u;  // row-major: any height works; full MFMA tiles are cheapest
-}
-
-// Row-major -> streaming layout with tiles of h rows.  The block of (tile,
-// chunk) holds 2*h pieces of 16 bytes, piece half*h + n = the four 4-byte
-// half-blocks of row h*tile + n at byte offsets chunk*32 + b*8 + half*4
-// (b = 0..3): exactly what lane (n, half) feeds to the four block MFMAs, and
-// one contiguous burst per wave-level load.  Rows past the matrix are zero.
-// Scales follow per (tile, chunk) as h consecutive row entries of 4 binary16 /
-// 2 UE8M0.
+// Row-major -> streaming layout with tiles of h rows (even).  The block of
+// (tile, chunk) holds 2h pieces of 16 bytes, piece g*h/2 + n = four dwords in
+// (j, s) order, dword 2j+s = the 8 weights of row h*tile + j*h/2 + n, columns
+// 64*chunk + 32s + 8g..+8: exactly what lane 16g + n feeds to the four
+// instructions of the chunk, and one contiguous burst per wave-level load.
+// Rows past the matrix are zero.  Scales follow per (tile, chunk): binary16 as
+// h entries of 8 bytes, entry p*h/2 + n = the scales of blocks 2s + p of rows
+// j*h/2 + n in (j, s) order; UE8M0 as h/2 entries of 4 bytes, entry n = the
+// scales of 32-blocks s of rows j*h/2 + n in (j, s) order.
 __global__ void fp4_prepack_kernel(const uint8_t* weights,
                                    const uint8_t* scales, uint8_t* out_weights,
                                    uint8_t* out_scales, uint32_t rows,
-                                   uint32_t padded_columns,
-                                   uint32_t scale_chunk_bytes, uint32_t h) {
+                                   uint32_t padded_columns, uint32_t f16_scales,
+                                   uint32_t h) {
   const uint32_t chunks = padded_columns / kChunk;
   const uint32_t tiles = (rows + h - 1u) / h;
+  const uint32_t half_rows = h / 2u;
   const size_t pieces = static_cast<size_t>(tiles) * chunks * 2u * h;
   const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const uint32_t scale_chunk_bytes = f16_scales ? 8u : 2u;
+  const uint32_t scale_entries = f16_scales ? h : half_rows;
   for (size_t piece = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
        piece < pieces; piece += stride) {
     const uint32_t within = static_cast<uint32_t>(piece % (2u * h));
     const size_t block = piece / (2u * h);
-    const uint32_t half = within / h;
-    const uint32_t n = within % h;
+    const uint32_t g = within / half_rows;
+    const uint32_t n = within % half_rows;
     const uint32_t chunk = static_cast<uint32_t>(block % chunks);
     const uint32_t tile = static_cast<uint32_t>(block / chunks);
-    const uint32_t row = tile * h + n;
-    uint4 value = make_uint4(0u, 0u, 0u, 0u);
-    if (row < rows) {
-      const uint32_t* source = reinterpret_cast<const uint32_t*>(
-          weights + static_cast<size_t>(row) * (padded_columns / 2u) +
-          chunk * 32u + half * 4u);
-      value = make_uint4(source[0], source[2], source[4], source[6]);
-    }
-    *reinterpret_cast<uint4*>(out_weights + piece * 16u) = value;
-    if (half == 0u) {
-      uint8_t* target = out_scales + (block * h + n) * scale_chunk_bytes;
-      const uint8_t* source =
-          scales + static_cast<size_t>(row) * (chunks * scale_chunk_bytes) +
-          chunk * scale_chunk_bytes;
-      for (uint32_t byte = 0; byte < scale_chunk_bytes; ++byte)
-        target[byte] = row < rows ? source[byte] : 0u;
-    }
+    uint32_t value[4];
+    for (uint32_t j = 0; j < 2u; ++j)
+      for (uint32_t s = 0; s < 2u; ++s) {
+        const uint32_t row = tile * h + j * half_rows + n;
+        value[2u * j + s] =
+            row < rows ? *reinterpret_cast<const uint32_t*>(
+                             weights + static_cast<size_t>(row) * (padded_columns / 2u) +
+                             chunk * 32u + s * 16u + g * 4u)
+                       : 0u;
+      }
+    *reinterpret_cast<uint4*>(out_weights + piece * 16u) =
+        make_uint4(value[0], value[1], value[2], value[3]);
+    // the first pieces of a (tile, chunk) also write its scale entries
+    if (within >= scale_entries) continue;
+    const uint32_t p = within / half_rows;   // block parity (binary16 only)
+    for (uint32_t j = 0; j < 2u; ++j)
+      for (uint32_t s = 0; s < 2u; ++s) {
+        const uint32_t row = tile * h + j * half_rows + n;
+        const uint8_t* source =
+            scales + static_cast<size_t>(row) * (chunks * scale_chunk_bytes) +
+            chunk * scale_chunk_bytes;
+        if (f16_scales) {
+          uint16_t* target = reinterpret_cast<uint16_t*>(
+              out_scales + (block * h + within) * 8u);
+          target[2u * j + s] =
+              row < rows ? reinterpret_cast<const uint16_t*>(source)[2u * s + p] : 0u;
+        } else {
+          uint8_t* target = out_scales + (block * half_rows + within) * 4u;
+          target[2u * j + s] = row < rows ? source[s] : 0u;
+        }
+      }
   }
 }
 
@@ -724,18 +803,11 @@ extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
   return launched("FP4 Q8 weight-reuse GEMV");
 }
 
-// A tile costs the same matrix-core and conversion time whatever its height,
-// so full 32-row tiles are the default; shorter ones only pay off when a
-// matrix has too few rows to give every CU a tile.
-static uint32_t resolve_tile_rows(uint32_t, uint32_t tile_rows) {
-  return tile_rows ? tile_rows : 32u;
-}
-
 extern "C" size_t qllm_fp4_packed_weight_bytes(uint32_t rows,
                                                uint32_t padded_columns,
                                                uint32_t tile_rows) {
-  if (!rows || tile_rows > 32u || (tile_rows && tile_rows < 8u)) return 0;
-  const uint32_t h = resolve_tile_rows(rows, tile_rows);
+  if (!rows || !tile_rows_ok(tile_rows)) return 0;
+  const uint32_t h = tile_rows ? tile_rows : 32u;
   return static_cast<size_t>((rows + h - 1u) / h) * h * (padded_columns / 2u);
 }
 
@@ -743,8 +815,8 @@ extern "C" size_t qllm_fp4_packed_scale_bytes(uint32_t rows,
                                               uint32_t padded_columns,
                                               uint32_t scale_scheme,
                                               uint32_t tile_rows) {
-  if (!rows || tile_rows > 32u || (tile_rows && tile_rows < 8u)) return 0;
-  const uint32_t h = resolve_tile_rows(rows, tile_rows);
+  if (!rows || !tile_rows_ok(tile_rows)) return 0;
+  const uint32_t h = tile_rows ? tile_rows : 32u;
   const size_t padded_rows = static_cast<size_t>((rows + h - 1u) / h) * h;
   return scale_scheme == QLLM_SCALE_F16_BLOCK16
              ? padded_rows * (padded_columns / 16u) * 2u
@@ -757,12 +829,9 @@ extern "C" int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source,
                                     qllm_fp4_matrix* packed, void* stream) {
   if (!matrix_ok(source) || source->layout != QLLM_LAYOUT_ROW_MAJOR ||
       source->padded_columns % kChunk != 0u || !packed_weights ||
-      !packed_scales || !packed || tile_rows > 32u ||
-      (tile_rows && tile_rows < 8u))
+      !packed_scales || !packed || !tile_rows_ok(tile_rows))
     return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 prepack");
-  const uint32_t h = resolve_tile_rows(source->rows, tile_rows);
-  const uint32_t scale_chunk =
-      source->scale_scheme == QLLM_SCALE_F16_BLOCK16 ? 8u : 2u;
+  const uint32_t h = tile_rows ? tile_rows : 32u;
   const size_t pieces =
       qllm_fp4_packed_weight_bytes(source->rows, source->padded_columns, h) / 16u;
   const uint32_t grid =
@@ -771,7 +840,8 @@ extern "C" int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source,
       source->weights, static_cast<const uint8_t*>(source->scales),
       static_cast<uint8_t*>(packed_weights),
       static_cast<uint8_t*>(packed_scales), source->rows,
-      source->padded_columns, scale_chunk, h);
+      source->padded_columns,
+      source->scale_scheme == QLLM_SCALE_F16_BLOCK16 ? 1u : 0u, h);
   *packed = *source;
   packed->weights = static_cast<const uint8_t*>(packed_weights);
   packed->scales = packed_scales;

@@ -28,14 +28,14 @@ def test_gemm_matches_oracle(device, scheme, rows, padded, batch):
         assert np.array_equal(tiled, row_major)
 
 
-@pytest.mark.parametrize("tile_rows", [8, 20, 23, 32])
+@pytest.mark.parametrize("tile_rows", [8, 20, 24, 32])
 @pytest.mark.parametrize("rows,padded,batch", [(333, 5120, 5), (2000, 1024, 6),
-                                               (40, 128, 7)])
-def test_gemm_tile_heights(device, tile_rows, rows, padded, batch):
+                                               (40, 128, 7), (17, 64, 8)])
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_gemm_tile_heights(device, scheme, tile_rows, rows, padded, batch):
     """Every tile height of the streaming layout (partial last tile included)
     computes the same rows; only the summation order over K may differ."""
     rng = np.random.default_rng(rows + tile_rows)
-    scheme = ol.SCALE_F16_BLOCK16
     codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
     act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
     want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
