@@ -264,14 +264,14 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
           weight_base[t] + static_cast<size_t>(chunk) * weight_step + weight_lane);
       const uint8_t* scale_chunk =
           scale_base[t] + static_cast<size_t>(chunk) * scale_step;
-      if (TILED && F16) {
+      if constexpr (TILED && F16) {
         const uint2 v = load_stream8(scale_chunk + scale_lane[0]);
         scales[slot][t][0] = v.x;
         scales[slot][t][1] = v.y;
-      } else if (TILED) {
+      } else if constexpr (TILED) {
         scales[slot][t][0] =
             *reinterpret_cast<const uint32_t*>(scale_chunk + scale_lane[0]);
-      } else if (F16) {
+      } else if constexpr (F16) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const uint2 v = load_stream8(scale_chunk + scale_lane[j]);
@@ -328,10 +328,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
           if (!TILED) transpose_rows4(packed);
           float scale[4];
           float fold[4];
-          if (F16) {
+          if constexpr (F16) {
             // binary16 scale applied in F32 after the block's MFMA
             uint32_t pair[2];   // scales of (j, 0), (j, 1) as two halves
-            if (TILED) {
+            if constexpr (TILED) {
               pair[0] = s[t][0];
               pair[1] = s[t][1];
             } else {
@@ -350,7 +350,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
             fold[0] = fold[1] = fold[2] = fold[3] = 1.0f;
           } else {
             // power-of-two scale folded into the nibble->bf16 conversion
-            const uint32_t bytes = TILED ? s[t][0] : s[t][0] | (s[t][1] << 16);
+            uint32_t bytes = s[t][0];
+            if constexpr (!TILED) bytes |= s[t][1] << 16;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
               fold[k] = ue8m0_to_f32((bytes >> (8 * k)) & 0xffu);
@@ -553,11 +554,12 @@ int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
 }
 
 // One tile per workgroup (a gate tile and its up tile for the fused SwiGLU
-// pair); four waves split K, eight when the matrix has few tiles.
+// pair); four waves split K, eight when the matrix has too few tiles to give
+// every CU one.
 int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
                     bool swiglu, hipStream_t stream) {
   const uint32_t tiles = (args.rows + args.tile_rows - 1u) / args.tile_rows;
-  const uint32_t waves = tiles <= 384u && !swiglu ? 8u : 4u;
+  const uint32_t waves = tiles <= 256u && !swiglu ? 8u : 4u;
 #define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
   return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
                                                     stream)
