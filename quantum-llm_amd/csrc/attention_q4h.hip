@@ -318,6 +318,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // so the integer scores carry the query to ~3e-5 relative instead of the
   // 4e-3 of a single Q8 plane.  The operands are published in MFMA order.
   static_assert(RT * KSTEPS <= kSplitWaves, "one wave per operand pair");
+  // the wave's first tile sets out before anything else: its flight time covers
+  // the query work below
+  if (tile_first < tile_last) {
+    stage_keys(tile_first);
+    stage_values(tile_first);
+  }
   if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
     // wave u builds k-step u % KSTEPS of row tile u / KSTEPS (the row's scale
     // needs the whole row, so every such wave reads all of it)
@@ -348,10 +354,6 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(loaded.x), fabsf(loaded.y)),
                                        fmaxf(fabsf(loaded.z), fabsf(loaded.w))));
       }
-    }
-    if (tile_first < tile_last) {
-      stage_keys(tile_first);
-      stage_values(tile_first);
     }
     maximum = quad_row_max(maximum);
     const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
@@ -390,9 +392,6 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         high_operand;
     *reinterpret_cast<i32x4*>(exchange + (wave * 2u + 1u) * 1024u + lane * 16u) =
         low_operand;
-  } else if (tile_first < tile_last) {
-    stage_keys(tile_first);
-    stage_values(tile_first);
   }
   __syncthreads();
 
