@@ -594,6 +594,113 @@ void qo_attention_q4h_int8(const struct qo_attention_shape* shape,
   free(q8);
 }
 
+size_t qo_q8_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                         uint32_t head_dim) {
+  return (size_t)2u * page_tokens * kv_heads * (head_dim + 2u);
+}
+
+static void q8_encode(uint8_t* record, const float* x, uint32_t d) {
+  float maximum = 0.0f;
+  for (uint32_t index = 0; index < d; ++index) {
+    const float magnitude = fabsf(x[index]);
+    if (magnitude > maximum) maximum = magnitude;
+  }
+  const uint16_t scale_bits = qo_f16_bits(fmaxf(maximum / 127.0f, 0x1p-24f));
+  const float scale = qo_f16_value(scale_bits);
+  for (uint32_t index = 0; index < d; ++index) {
+    int code = (int)nearbyintf(x[index] / scale);
+    if (code > 127) code = 127;
+    if (code < -127) code = -127;
+    record[index] = (uint8_t)(int8_t)code;
+  }
+  memcpy(record + d, &scale_bits, sizeof(scale_bits));
+}
+
+static void q8_decode(const uint8_t* record, uint32_t d, float* x) {
+  uint16_t scale_bits;
+  memcpy(&scale_bits, record + d, sizeof(scale_bits));
+  const float scale = qo_f16_value(scale_bits);
+  for (uint32_t index = 0; index < d; ++index)
+    x[index] = (float)(int8_t)record[index] * scale;
+}
+
+void qo_q8_store(uint8_t* page, size_t layer_offset, uint32_t page_tokens,
+                 uint32_t position, uint32_t kv_head, uint32_t kv_heads,
+                 uint32_t head_dim, const float* key, const float* value) {
+  const size_t record_bytes = head_dim + 2u;
+  const size_t records = (size_t)page_tokens * kv_heads;
+  const size_t record = (size_t)(position % page_tokens) * kv_heads + kv_head;
+  uint8_t* keys = page + layer_offset;
+  q8_encode(keys + record * record_bytes, key, head_dim);
+  q8_encode(keys + (records + record) * record_bytes, value, head_dim);
+}
+
+void qo_q8_load(const uint8_t* page, size_t layer_offset, uint32_t page_tokens,
+                uint32_t position, uint32_t kv_head, uint32_t kv_heads,
+                uint32_t head_dim, float* key, float* value) {
+  const size_t record_bytes = head_dim + 2u;
+  const size_t records = (size_t)page_tokens * kv_heads;
+  const size_t record = (size_t)(position % page_tokens) * kv_heads + kv_head;
+  const uint8_t* keys = page + layer_offset;
+  q8_decode(keys + record * record_bytes, head_dim, key);
+  q8_decode(keys + (records + record) * record_bytes, head_dim, value);
+}
+
+void qo_attention_q8_f64(const struct qo_attention_shape* shape,
+                         size_t layer_offset, const float* queries,
+                         const uint8_t* const* page_table, float* out) {
+  const uint32_t d = shape->head_dim;
+  const uint32_t group = shape->query_heads / shape->kv_heads;
+  const uint32_t stride = query_stride_of(shape);
+  const uint32_t last_context = shape->first_context_tokens + shape->rows - 1u;
+#pragma omp parallel for schedule(dynamic, 1)
+  for (long kv_index = 0; kv_index < (long)shape->kv_heads; ++kv_index) {
+    const uint32_t kv_head = (uint32_t)kv_index;
+    float* keys = (float*)malloc(sizeof(float) * (size_t)last_context * d);
+    float* values = (float*)malloc(sizeof(float) * (size_t)last_context * d);
+    double* scores = (double*)malloc(sizeof(double) * last_context);
+    double* accumulator = (double*)malloc(sizeof(double) * d);
+    for (uint32_t token = 0; token < last_context; ++token)
+      qo_q8_load(page_table[token / shape->page_tokens], layer_offset,
+                 shape->page_tokens, token, kv_head, shape->kv_heads, d,
+                 keys + (size_t)token * d, values + (size_t)token * d);
+    for (uint32_t member = 0; member < group; ++member) {
+      const uint32_t head = kv_head * group + member;
+      for (uint32_t row = 0; row < shape->rows; ++row) {
+        const uint32_t context = shape->first_context_tokens + row;
+        const size_t record = (size_t)row * shape->query_heads + head;
+        const float* q = queries + record * stride;
+        double maximum = -INFINITY;
+        for (uint32_t token = 0; token < context; ++token) {
+          double dot = 0.0;
+          for (uint32_t index = 0; index < d; ++index)
+            dot += (double)q[index] * (double)keys[(size_t)token * d + index];
+          scores[token] = dot / sqrt((double)d);
+          if (scores[token] > maximum) maximum = scores[token];
+        }
+        double denominator = 0.0;
+        for (uint32_t index = 0; index < d; ++index) accumulator[index] = 0.0;
+        for (uint32_t token = 0; token < context; ++token) {
+          const double p = exp(scores[token] - maximum);
+          denominator += p;
+          for (uint32_t index = 0; index < d; ++index)
+            accumulator[index] += p * (double)values[(size_t)token * d + index];
+        }
+        for (uint32_t index = 0; index < d; ++index) {
+          double result = accumulator[index] / denominator;
+          if (shape->output_gated)
+            result /= 1.0 + exp(-(double)q[d + index]);
+          out[record * d + index] = (float)result;
+        }
+      }
+    }
+    free(keys);
+    free(values);
+    free(scores);
+    free(accumulator);
+  }
+}
+
 void qo_attention_f16_f64(const struct qo_attention_shape* shape,
                           const float* queries,
                           const uint8_t* const* page_table,

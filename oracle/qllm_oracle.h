@@ -194,6 +194,32 @@ void qo_attention_q4h_int8(const struct qo_attention_shape* shape,
                            const float* queries,
                            const uint8_t* const* page_table, float* out);
 
+/* Q8 KV records (the proposer's cache): per layer, page_tokens*kv_heads key
+ * records, then as many value records; record (token % page_tokens)*kv_heads
+ * + kv_head holds head_dim int8 codes followed by one binary16 scale:
+ *   scale = f16(max(absmax/127, 2^-24)), code = clamp(rn(x/scale), -127, 127).
+ * `layer_offset` is the byte offset of the layer inside the page.
+ * runtime/src/cuda/transformer_kernels.cu:601-625 (encoder), :5093-5101
+ * (record addressing), record size :70-76; independent encoder of the
+ * fixture runtime/tools/dense_fp4_cuda_smoke.cpp:1061-1088. */
+size_t qo_q8_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                         uint32_t head_dim);
+void qo_q8_store(uint8_t* page, size_t layer_offset, uint32_t page_tokens,
+                 uint32_t position, uint32_t kv_head, uint32_t kv_heads,
+                 uint32_t head_dim, const float* key, const float* value);
+void qo_q8_load(const uint8_t* page, size_t layer_offset, uint32_t page_tokens,
+                uint32_t position, uint32_t kv_head, uint32_t kv_heads,
+                uint32_t head_dim, float* key, float* value);
+
+/* Textbook softmax(q.k/sqrt(d)) v over the dequantised Q8 cache, all in
+ * double (shape->layer is ignored, the layer sits at layer_offset).  The
+ * reference's float statement of the same attention rounds q, k, v and the
+ * probabilities to bf16 (runtime/tools/dense_fp4_cuda_smoke.cpp:986-1024,
+ * :1138-1167) and accepts 2e-3 between the two (:4921-4926). */
+void qo_attention_q8_f64(const struct qo_attention_shape* shape,
+                         size_t layer_offset, const float* queries,
+                         const uint8_t* const* page_table, float* out);
+
 /* Exact-F16 KV pages: per layer  K [page_tokens][kv][d] then
  * V [page_tokens][kv][d], binary16.
  * runtime/src/cuda/transformer_kernels.cu:6594-6606.

@@ -260,6 +260,40 @@ def q4h_load(page: np.ndarray, layer, page_tokens, position, kv_head, kv_heads,
     return key, value
 
 
+def q8_layer_bytes(page_tokens, kv_heads, head_dim):
+    return 2 * page_tokens * kv_heads * (head_dim + 2)
+
+
+def q8_store(page: np.ndarray, layer_offset, page_tokens, position, kv_head,
+             kv_heads, head_dim, key, value):
+    key = np.ascontiguousarray(key, dtype=np.float32)
+    value = np.ascontiguousarray(value, dtype=np.float32)
+    oracle().qo_q8_store(_p(page), c_size_t(layer_offset), c_uint32(page_tokens),
+                         c_uint32(position), c_uint32(kv_head),
+                         c_uint32(kv_heads), c_uint32(head_dim), _p(key),
+                         _p(value))
+
+
+def q8_load(page: np.ndarray, layer_offset, page_tokens, position, kv_head,
+            kv_heads, head_dim):
+    key = np.empty(head_dim, dtype=np.float32)
+    value = np.empty(head_dim, dtype=np.float32)
+    oracle().qo_q8_load(_p(page), c_size_t(layer_offset), c_uint32(page_tokens),
+                        c_uint32(position), c_uint32(kv_head),
+                        c_uint32(kv_heads), c_uint32(head_dim), _p(key),
+                        _p(value))
+    return key, value
+
+
+def attention_q8(shape: AttentionShape, queries, pages, layer_offset=0):
+    queries = np.ascontiguousarray(queries, dtype=np.float32)
+    out = np.empty((shape.rows, shape.query_heads, shape.head_dim), np.float32)
+    table = _page_table(pages)
+    oracle().qo_attention_q8_f64(ctypes.byref(shape), c_size_t(layer_offset),
+                                 _p(queries), table, _p(out))
+    return out
+
+
 def quantize_queries_q8(queries, rows, query_heads, head_dim, stride):
     queries = np.ascontiguousarray(queries, dtype=np.float32)
     q8 = np.empty((rows, query_heads, head_dim), dtype=np.int8)
