@@ -342,6 +342,61 @@ typedef struct qllm_f16_attention_launch {
 
 int32_t qllm_attention_paged_f16(const qllm_f16_attention_launch* launch);
 
+/* ---- attention: Q8 paged cache (the proposer's) ------------------------------- */
+
+/* Symmetric int8 codes with one binary16 scale per K or V head record,
+ *   scale = f16(max(absmax/127, 2^-24)), code = clamp(rn(x/scale), -127, 127)
+ * (transformer_kernels.cu:601-625).  The reference interleaves codes and scale
+ * in records of head_dim + 2 bytes; this library keeps the same values in
+ * planes, `page_offset_bytes` (a multiple of 16) into the page:
+ *   K codes [page_tokens][kv_heads][head_dim] int8, V codes likewise,
+ *   K scales [kv_heads][page_tokens] binary16, V scales likewise
+ * - qllm_q8_layer_bytes() per layer, the reference's size.  The pages are
+ * private to the provider, so the placement is not an interface.
+ * replaces store_gqa_kv_paged_q8_batch (transformer_kernels.hpp:403-409). */
+size_t qllm_q8_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                           uint32_t head_dim);
+int32_t qllm_store_kv_paged_q8_batch(const float* key, const float* value,
+                                     const void* const* page_table,
+                                     size_t page_offset_bytes,
+                                     uint32_t page_tokens,
+                                     uint32_t first_cache_position,
+                                     uint32_t rows, uint32_t kv_heads,
+                                     uint32_t head_dim, void* stream);
+
+/* replaces gated_gqa_attention_microbatch_paged_q8_tensor_core and
+ * gated_gqa_attention_decode_paged_q8_tensor_core (transformer_kernels.hpp:
+ * 873, 944; launch struct PagedQ8GatedGqaPrefillLaunch): row r attends tokens
+ * [0, first_context_tokens + r).  Codes enter the matrix cores as exact
+ * binary16 integers, the query as binary16 (the reference rounds q, k, v and
+ * the probabilities to bf16), splits run in parallel and share the combine
+ * kernel of the other caches.  page_tokens % 32 == 0, head_dim 128 or 256,
+ * rows * (query_heads/kv_heads) <= 48 (32 at head_dim 256), split_tokens % 32
+ * == 0 (0 = context dealt evenly over maximum_splits workgroups per KV head). */
+typedef struct qllm_q8_attention_launch {
+  const float* query;
+  const void* const* device_pages;
+  void* output;
+  float* partial_maxima;
+  float* partial_sums;
+  float* partial_outputs;
+  size_t page_offset_bytes;
+  uint32_t first_context_tokens;
+  uint32_t rows;
+  uint32_t page_tokens;
+  uint32_t query_heads;
+  uint32_t kv_heads;
+  uint32_t head_dim;
+  uint32_t split_tokens;
+  uint32_t maximum_splits;
+  uint32_t query_stride;
+  int32_t output_gated;
+  uint32_t output_kind;
+  void* stream;
+} qllm_q8_attention_launch;
+
+int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launch);
+
 /* ---- token selection ------------------------------------------------------------ */
 
 /* replaces argmax_batch (transformer_kernels.hpp:1266-1269): ties to the

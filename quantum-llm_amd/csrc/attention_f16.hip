@@ -1,4 +1,4 @@
-// Exact-F16 paged KV cache: K/V store and decode attention.
+// Exact-F16 and Q8 paged KV caches: K/V store and decode attention.
 //
 // Replaces, from runtime/src/cuda/transformer_kernels.cu of the reference:
 //   store_gqa_kv_fp16_to_paged                                  :4208
@@ -11,6 +11,12 @@
 // the query is rounded to binary16, scores are F32 sums of binary16
 // products, probabilities are rounded to binary16 before they weigh V and
 // before they enter the denominator.
+//
+// The same kernel, instantiated for the proposer's Q8 cache (int8 codes, one
+// binary16 scale per record; reference encoder :601-625, attention
+// gated_gqa_attention_microbatch_paged_q8_tensor_core :9732): codes become
+// exact binary16 integers on the way into the matrix cores, the K scale
+// multiplies the score and the V scale the probability.
 #include "attention_common.hpp"
 
 namespace qllm {
@@ -42,6 +48,72 @@ __global__ void f16_store_kernel(const float* key, const float* value,
 }
 
 
+// Q8 layout inside a page, `page_offset` bytes in:  K codes
+// [page_tokens][kv_heads][head_dim] int8, V codes likewise, K scales
+// [kv_heads][page_tokens] binary16, V scales likewise - the reference's
+// records (codes followed by their scale, :5093-5101) with codes and scales in
+// separate planes, which keeps every row 16-byte aligned; the bytes per layer
+// are the same, page_tokens * kv_heads * 2 * (head_dim + 2).
+// One wave per (token, kv head); scale = f16(max(absmax/127, 2^-24)),
+// code = clamp(rn(x / scale), -127, 127)  (:601-625).
+__global__ __launch_bounds__(64) void q8_store_kernel(
+    const float* key, const float* value, const void* const* page_table,
+    size_t page_offset, uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t kv_heads, uint32_t head_dim) {
+  const uint32_t lane = threadIdx.x;
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t row = blockIdx.y;
+  const uint32_t position = first_cache_position + row;
+  uint8_t* page = static_cast<uint8_t*>(const_cast<void*>(
+                      page_table[position / page_tokens])) + page_offset;
+  const uint32_t slot = position % page_tokens;
+  const size_t codes_bytes = static_cast<size_t>(page_tokens) * kv_heads * head_dim;
+  const size_t record = static_cast<size_t>(slot) * kv_heads + kv_head;
+#pragma unroll
+  for (int kind = 0; kind < 2; ++kind) {
+    const float* source = (kind ? value : key) +
+                          (static_cast<size_t>(row) * kv_heads + kv_head) * head_dim;
+    float maximum = 0.0f;
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      maximum = fmaxf(maximum, fabsf(source[index]));
+    maximum = wave_max(maximum);
+    const uint32_t scale_bits = f32_to_f16_bits(fmaxf(maximum / 127.0f, 0x1p-24f));
+    const float scale = f16_bits_to_f32(scale_bits);
+    int8_t* codes = reinterpret_cast<int8_t*>(page + kind * codes_bytes) +
+                    record * head_dim;
+    for (uint32_t index = lane; index < head_dim; index += 64u) {
+      const int code = max(-127, min(127, __float2int_rn(source[index] / scale)));
+      codes[index] = static_cast<int8_t>(code);
+    }
+    if (lane == 0u) {
+      uint16_t* scales = reinterpret_cast<uint16_t*>(page + 2u * codes_bytes) +
+                         static_cast<size_t>(kind) * kv_heads * page_tokens;
+      scales[static_cast<size_t>(kv_head) * page_tokens + slot] =
+          static_cast<uint16_t>(scale_bits);
+    }
+  }
+}
+
+// 8 int8 codes -> 8 exact binary16 values: code + 128 becomes the low mantissa
+// byte of 1024.0 (bit pattern 0x6400 + u = 1024 + u exactly), minus 1152.
+__device__ __forceinline__ f16x8 int8x8_to_f16(uint2 codes) {
+  const uint32_t low = codes.x ^ 0x80808080u;
+  const uint32_t high = codes.y ^ 0x80808080u;
+  const f16x2 bias = {static_cast<_Float16>(-1152.0f), static_cast<_Float16>(-1152.0f)};
+  const f16x2 e0 = __builtin_bit_cast(
+      f16x2, __builtin_amdgcn_perm(0x64646464u, low, 0x04010400u)) + bias;
+  const f16x2 e1 = __builtin_bit_cast(
+      f16x2, __builtin_amdgcn_perm(0x64646464u, low, 0x04030402u)) + bias;
+  const f16x2 e2 = __builtin_bit_cast(
+      f16x2, __builtin_amdgcn_perm(0x64646464u, high, 0x04010400u)) + bias;
+  const f16x2 e3 = __builtin_bit_cast(
+      f16x2, __builtin_amdgcn_perm(0x64646464u, high, 0x04030402u)) + bias;
+  f16x8 result;
+  result[0] = e0[0]; result[1] = e0[1]; result[2] = e1[0]; result[3] = e1[1];
+  result[4] = e2[0]; result[5] = e2[1]; result[6] = e3[0]; result[7] = e3[1];
+  return result;
+}
+
 struct F16SplitArgs {
   const float* query;
   uint32_t query_stride;
@@ -57,6 +129,7 @@ struct F16SplitArgs {
   uint32_t kv_heads;
   uint32_t split_tokens;
   uint32_t maximum_splits;
+  size_t page_offset;   // Q8: byte offset of the layer inside a page
 };
 
 constexpr uint32_t kF16Tile = 32;  // tokens per wave step
@@ -71,8 +144,9 @@ constexpr uint32_t kF16Tile = 32;  // tokens per wave step
 //           (ds_read_b64_tr_b16: 4 tokens x 16 dims per lane group) is free
 //           of bank conflicts, and the score registers of a 16-token sub-tile
 //           are already the B operand.
-// D = head_dim (128 or 256), RT = 16-row tiles of rows*group query rows.
-template <int D, int RT>
+// D = head_dim (128 or 256), RT = 16-row tiles of rows*group query rows,
+// Q8 = the cache holds int8 codes and per-record scales instead of binary16.
+template <int D, int RT, bool Q8>
 __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
     const F16SplitArgs args) {
   constexpr int KSTEPS = D / 32;  // k-steps of the score MFMA over head_dim
@@ -140,7 +214,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
   const size_t page_values =
       static_cast<size_t>(args.page_tokens) * args.kv_heads * D;
   const size_t layer_offset = static_cast<size_t>(args.layer) * 2u * page_values;
-  const uint32_t row_stride = args.kv_heads * D;  // halves between tokens
+  const uint32_t row_stride = args.kv_heads * D;  // elements between tokens
   uint8_t* stage_v = stage + wave * STAGE;
   // transposing read: lane (quad, col = 4*r + j) supplies the 8 bytes of token
   // 4*quad + r (of the 16-token sub-tile), halves 16*dt + 4*j .. +3.  Granule
@@ -166,13 +240,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
   for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
     const uint32_t tile_begin = tile * kF16Tile;
     const bool needs_mask = tile_begin + kF16Tile > first_context_tokens;
-    const uint16_t* page = static_cast<const uint16_t*>(
-        uniform_page(args.pages, tile_begin / args.page_tokens));
-    const uint16_t* keys =
-        page + layer_offset +
-        static_cast<size_t>(tile_begin % args.page_tokens) * row_stride +
-        kv_head * D;
+    const void* page_base = uniform_page(args.pages, tile_begin / args.page_tokens);
+    const uint32_t tile_slot = tile_begin % args.page_tokens;
+    // binary16 cache
+    const uint16_t* keys = static_cast<const uint16_t*>(page_base) + layer_offset +
+                           static_cast<size_t>(tile_slot) * row_stride + kv_head * D;
     const uint16_t* values = keys + page_values;
+    // Q8 cache: code planes, then scale planes [kv_heads][page_tokens]
+    const uint8_t* keys8 = static_cast<const uint8_t*>(page_base) + args.page_offset +
+                           static_cast<size_t>(tile_slot) * row_stride + kv_head * D;
+    const uint8_t* values8 = keys8 + page_values;
+    const uint16_t* key_scales =
+        reinterpret_cast<const uint16_t*>(static_cast<const uint8_t*>(page_base) +
+                                          args.page_offset + 2u * page_values) +
+        static_cast<size_t>(kv_head) * args.page_tokens + tile_slot;
+    const uint16_t* value_scales =
+        key_scales + static_cast<size_t>(args.kv_heads) * args.page_tokens;
 
     // ---- V tile -> LDS (swizzled rows) ----------------------------------------
 #pragma unroll
@@ -180,8 +263,14 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
       const uint32_t piece = pass * 64u + lane;
       const uint32_t token = piece / GR;
       const uint32_t part = piece % GR;
-      uint4 value = *reinterpret_cast<const uint4*>(
-          values + static_cast<size_t>(token) * row_stride + part * 8u);
+      uint4 value;
+      if constexpr (Q8)
+        value = __builtin_bit_cast(
+            uint4, int8x8_to_f16(*reinterpret_cast<const uint2*>(
+                       values8 + static_cast<size_t>(token) * row_stride + part * 8u)));
+      else
+        value = *reinterpret_cast<const uint4*>(
+            values + static_cast<size_t>(token) * row_stride + part * 8u);
       // records no row can see may be uninitialised: a NaN there would
       // survive its zero probability
       if (needs_mask && tile_begin + token >= last_context)
@@ -196,10 +285,40 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
 #pragma unroll
     for (int st = 0; st < 2; ++st)
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-        key_operand[st][ks] = *reinterpret_cast<const f16x8*>(
-            keys + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
-            8u * quad);
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        if constexpr (Q8)
+          key_operand[st][ks] = int8x8_to_f16(*reinterpret_cast<const uint2*>(
+              keys8 + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
+              8u * quad));
+        else
+          key_operand[st][ks] = *reinterpret_cast<const f16x8*>(
+              keys + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
+              8u * quad);
+      }
+    // Q8: scales of the lane's tokens 16*st + 4*quad + i; the K scale goes into
+    // the score, the V scale into the probability.  Records no row can see
+    // may be uninitialised: their V scale (any bit pattern) is replaced by 0.
+    float key_scale[2][4];
+    f16x4 value_scale[2];
+    if constexpr (Q8) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const uint2 k = *reinterpret_cast<const uint2*>(key_scales + 16u * st + 4u * quad);
+        uint2 v = *reinterpret_cast<const uint2*>(value_scales + 16u * st + 4u * quad);
+        key_scale[st][0] = f16_bits_to_f32(k.x & 0xffffu) * score_unit;
+        key_scale[st][1] = f16_bits_to_f32(k.x >> 16) * score_unit;
+        key_scale[st][2] = f16_bits_to_f32(k.y & 0xffffu) * score_unit;
+        key_scale[st][3] = f16_bits_to_f32(k.y >> 16) * score_unit;
+        if (needs_mask) {
+          const uint32_t first_token = tile_begin + 16u * st + 4u * quad;
+          if (first_token + 0u >= last_context) v.x &= 0xffff0000u;
+          if (first_token + 1u >= last_context) v.x &= 0x0000ffffu;
+          if (first_token + 2u >= last_context) v.y &= 0xffff0000u;
+          if (first_token + 3u >= last_context) v.y &= 0x0000ffffu;
+        }
+        value_scale[st] = __builtin_bit_cast(f16x4, v);
+      }
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       asm volatile("" ::: "memory");  // one row tile's query operands at a time
@@ -215,7 +334,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
                                                        dot, 0, 0, 0);
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) score[st][i] = dot[i] * score_unit;
+        for (int i = 0; i < 4; ++i)
+          score[st][i] = dot[i] * (Q8 ? key_scale[st][i] : score_unit);
       }
       if (needs_mask) {
         const uint32_t first_token = tile_begin + 4u * quad;
@@ -257,6 +377,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
           p_operand[rt][st][i] = p;
           sum += static_cast<float>(p);
         }
+      if constexpr (Q8) {
+#pragma unroll
+        for (int st = 0; st < 2; ++st) p_operand[rt][st] *= value_scale[st];
+      }
       running_sum[rt] += sum;
     }
 
@@ -298,19 +422,21 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
                            target);
 }
 
-template <int D>
+template <int D, bool Q8 = false>
 int32_t launch_f16_split(const F16SplitArgs& args, uint32_t row_tiles, dim3 grid,
                          hipStream_t stream) {
   switch (row_tiles) {
     case 1:
-      f16_attention_split_kernel<D, 1><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      f16_attention_split_kernel<D, 1, Q8>
+          <<<grid, kSplitWaves * 64, 0, stream>>>(args);
       break;
     case 2:
-      f16_attention_split_kernel<D, 2><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      f16_attention_split_kernel<D, 2, Q8>
+          <<<grid, kSplitWaves * 64, 0, stream>>>(args);
       break;
     default:
       if constexpr (D == 128) {
-        f16_attention_split_kernel<D, 3>
+        f16_attention_split_kernel<D, 3, Q8>
             <<<grid, kSplitWaves * 64, 0, stream>>>(args);
         break;
       } else {
@@ -410,6 +536,89 @@ extern "C" int32_t qllm_attention_paged_f16(
   const int32_t status =
       launch->head_dim == 128u ? launch_f16_split<128>(args, row_tiles, grid, stream)
                                : launch_f16_split<256>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, nullptr, stream);
+}
+
+extern "C" size_t qllm_q8_layer_bytes(uint32_t page_tokens, uint32_t kv_heads,
+                                      uint32_t head_dim) {
+  return static_cast<size_t>(page_tokens) * kv_heads * 2u * (head_dim + 2u);
+}
+
+extern "C" int32_t qllm_store_kv_paged_q8_batch(
+    const float* key, const float* value, const void* const* page_table,
+    size_t page_offset_bytes, uint32_t page_tokens,
+    uint32_t first_cache_position, uint32_t rows, uint32_t kv_heads,
+    uint32_t head_dim, void* stream) {
+  if (!key || !value || !page_table || !page_tokens || !rows || !kv_heads ||
+      !head_dim || page_offset_bytes % 16u ||
+      first_cache_position > 0xffffffffu - (rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 K/V store");
+  q8_store_kernel<<<dim3(kv_heads, rows), 64, 0, as_stream(stream)>>>(
+      key, value, page_table, page_offset_bytes, page_tokens,
+      first_cache_position, kv_heads, head_dim);
+  return launched("Q8 K/V store");
+}
+
+extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launch) {
+  if (!launch || !launch->query || !launch->device_pages || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      !launch->first_context_tokens || !launch->rows ||
+      !launch->page_tokens || launch->page_tokens % kF16Tile ||
+      launch->page_offset_bytes % 16u || !launch->query_heads ||
+      !launch->kv_heads || launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      launch->split_tokens % kF16Tile || !launch->maximum_splits ||
+      launch->maximum_splits > 2048u ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t row_tiles = (launch->rows * group + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q8 paged attention: rows * (query_heads/kv_heads) exceeds "
+                "48 (32 at head_dim 256)");
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      launch->split_tokens
+          ? (last_context + launch->split_tokens - 1u) / launch->split_tokens
+          : launch->maximum_splits;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q8 paged attention: context needs more splits than "
+                "maximum_splits");
+  F16SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.pages = launch->device_pages;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.page_tokens = launch->page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  args.page_offset = launch->page_offset_bytes;
+  const dim3 grid(launch->kv_heads, splits);
+  const hipStream_t stream = as_stream(launch->stream);
+  const int32_t status =
+      launch->head_dim == 128u
+          ? launch_f16_split<128, true>(args, row_tiles, grid, stream)
+          : launch_f16_split<256, true>(args, row_tiles, grid, stream);
   if (status != QLLM_OK) return status;
   return launch_attention_combine(
       launch->query, launch->query_stride, launch->output_gated,

@@ -64,6 +64,19 @@ class F16AttentionLaunch(Structure):
                 ("output_kind", c_uint32), ("stream", c_void_p)]
 
 
+class Q8AttentionLaunch(Structure):
+    _fields_ = [("query", c_void_p), ("device_pages", c_void_p),
+                ("output", c_void_p), ("partial_maxima", c_void_p),
+                ("partial_sums", c_void_p), ("partial_outputs", c_void_p),
+                ("page_offset_bytes", c_size_t),
+                ("first_context_tokens", c_uint32), ("rows", c_uint32),
+                ("page_tokens", c_uint32), ("query_heads", c_uint32),
+                ("kv_heads", c_uint32), ("head_dim", c_uint32),
+                ("split_tokens", c_uint32), ("maximum_splits", c_uint32),
+                ("query_stride", c_uint32), ("output_gated", c_int32),
+                ("output_kind", c_uint32), ("stream", c_void_p)]
+
+
 # name -> (restype, argtypes); every symbol include/qllm_kernels.h declares.
 SIGNATURES = {
     "qllm_last_error": (c_char_p, []),
@@ -90,6 +103,9 @@ SIGNATURES = {
     "qllm_attention_paged_q4h": (c_int32, [POINTER(Q4hAttentionLaunch)]),
     "qllm_store_kv_paged_f16_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),
+    "qllm_q8_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
+    "qllm_store_kv_paged_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
+    "qllm_attention_paged_q8": (c_int32, [POINTER(Q8AttentionLaunch)]),
     "qllm_argmax_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "qllm_argmax_batch": (c_int32, [c_void_p, c_uint32, c_uint32, c_void_p, c_void_p, c_size_t, c_void_p]),
     "qllm_topk_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),

@@ -99,3 +99,52 @@ def f16_attention(device, pages, query, rows, query_heads, kv_heads, head_dim,
     qh.call("qllm_attention_paged_f16", launch)
     torch.cuda.synchronize()
     return out.float().cpu().numpy()
+
+
+def q8_planes_to_records(page, offset, page_tokens, kv_heads, head_dim):
+    """Re-lays one layer of a device Q8 page (code planes, then scale planes) as
+    the reference's records: [K records | V records], record (slot*kv + head) =
+    head_dim codes followed by the binary16 scale."""
+    d = head_dim
+    records = page_tokens * kv_heads
+    codes = records * d
+    layer = page[offset: offset + 2 * records * (d + 2)]
+    out = np.zeros((2, records, d + 2), dtype=np.uint8)
+    for kind in range(2):
+        out[kind, :, :d] = layer[kind * codes:(kind + 1) * codes].reshape(records, d)
+        scales = layer[2 * codes + kind * records * 2:
+                       2 * codes + (kind + 1) * records * 2].view(np.uint16)
+        scales = scales.reshape(kv_heads, page_tokens).T.reshape(records)   # -> [slot][head]
+        out[kind, :, d:] = np.ascontiguousarray(scales).view(np.uint8).reshape(records, 2)
+    return out.reshape(-1)
+
+
+def q8_store(device, d_pages, table, offset, page_tokens, first_position, keys, values):
+    """qllm_store_kv_paged_q8_batch for rows keys/values [rows, kv_heads, d]."""
+    rows, kv_heads, d = keys.shape
+    d_keys, d_values = device_tensor(keys, device), device_tensor(values, device)
+    qh.call("qllm_store_kv_paged_q8_batch", qh.ptr(d_keys), qh.ptr(d_values),
+            qh.ptr(table), offset, page_tokens, first_position, rows, kv_heads, d, None)
+    torch.cuda.synchronize()
+
+
+def q8_attention(device, d_pages, table, offset, query, rows, query_heads, kv_heads,
+                 head_dim, first_context, page_tokens, split_tokens, gated,
+                 out_kind=qh.OUT_F32, balanced_splits=32):
+    stride = head_dim * (2 if gated else 1)
+    d_query = device_tensor(query, device)
+    context = first_context + rows - 1
+    splits = ((context + split_tokens - 1) // split_tokens if split_tokens
+              else balanced_splits)
+    maxima = torch.zeros((rows, splits, query_heads), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((rows, splits, query_heads, head_dim), device=device)
+    dtype = torch.bfloat16 if out_kind == qh.OUT_BF16 else torch.float32
+    out = torch.zeros((rows, query_heads, head_dim), dtype=dtype, device=device)
+    launch = qh.Q8AttentionLaunch(
+        qh.ptr(d_query), qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), offset, first_context, rows, page_tokens, query_heads,
+        kv_heads, head_dim, split_tokens, splits, stride, int(gated), out_kind, None)
+    qh.call("qllm_attention_paged_q8", launch)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
