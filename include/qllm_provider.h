@@ -43,6 +43,16 @@ typedef struct qllm_dense_geometry {
   uint32_t kv_page_tokens;
   uint32_t max_context;
   uint32_t draft_depth;
+  /* The proposer (run_mtp, dense_fp4_provider.cpp:8681-8852): 1 = the provider
+   * runs one MTP layer with its own Q8 KV cache and produces the drafts itself
+   * (its tensors are staged before qllm_provider_prepare_exact_decode, roles
+   * as in validate_exact :4730-4787: embedding_norm, hidden_norm, draft_norm,
+   * fusion_projection, layer.0.*), 0 = drafts arrive through
+   * qllm_provider_set_drafts. */
+  uint32_t mtp_layers;
+  /* Head rows the proposer scores (project_prefix :6280-6308); 0 =
+   * min(vocabulary, 65536). */
+  uint32_t draft_vocabulary;
 } qllm_dense_geometry;
 
 const char* qllm_provider_last_error(void);
@@ -88,7 +98,11 @@ int32_t qllm_provider_begin_request(qllm_provider* provider,
                                     uint32_t min_p_ppm, uint64_t seed);
 
 /* synchronize_exact_decode_batch with one token: the stream stands at
- * `position` with `token` guaranteed. */
+ * `position` with `token` guaranteed (the batch starts at position - 1, the
+ * target position the token was chosen from).  With an MTP layer this feeds
+ * the proposer that pair - using the hidden state of row 0 of the last target
+ * pass - and rolls the drafts for the next verify out; position 0 only marks
+ * the start of a stream. */
 int32_t qllm_provider_synchronize(qllm_provider* provider, uint32_t token,
                                   uint32_t position);
 
@@ -139,6 +153,16 @@ int32_t qllm_provider_time_kernel(qllm_provider* provider, const char* which,
 uint64_t qllm_provider_kv_page_bytes(const qllm_provider* provider);
 int32_t qllm_provider_copy_kv_page(qllm_provider* provider, uint32_t page_index,
                                    void* host_output);
+
+/* The proposer's state after its last pass: hidden state of the last row
+ * [hidden] and draft logits [draft_vocabulary] (either may be NULL), and the
+ * draft tokens waiting for the next verify step (returns their number). */
+int32_t qllm_provider_copy_mtp_state(qllm_provider* provider,
+                                     float* host_last_hidden,
+                                     float* host_draft_logits);
+uint32_t qllm_provider_drafts(const qllm_provider* provider, uint32_t* tokens,
+                              uint32_t capacity);
+uint32_t qllm_provider_draft_vocabulary(const qllm_provider* provider);
 
 const float* qllm_provider_logits(const qllm_provider* provider);
 const float* qllm_provider_hidden(const qllm_provider* provider);

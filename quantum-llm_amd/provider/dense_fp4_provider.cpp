@@ -127,8 +127,15 @@ Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
       g_.draft_depth == 0U || g_.draft_depth > 7U || g_.hidden % 64U ||
       g_.intermediate % 64U || (g_.query_heads * g_.head_dim) % 64U ||
       g_.scale_scheme > QLLM_SCALE_F16_BLOCK16 ||
-      !(g_.norm_epsilon > 0.0F) || !(g_.rope_theta > 0.0F);
+      !(g_.norm_epsilon > 0.0F) || !(g_.rope_theta > 0.0F) ||
+      g_.mtp_layers > 1U;
   if (bad) throw std::invalid_argument("dense FP4 geometry is not supported");
+  if (g_.draft_vocabulary == 0U)
+    g_.draft_vocabulary = std::min<std::uint32_t>(g_.vocabulary, 65536U);
+  if (g_.mtp_layers &&
+      (g_.draft_vocabulary > g_.vocabulary || g_.draft_vocabulary % 32U))
+    throw std::invalid_argument(
+        "draft vocabulary must be a multiple of 32 within the vocabulary");
   if (g_.kv_encoding == KvEncoding::fp16 &&
       g_.query_heads / g_.kv_heads > 16U)
     throw std::invalid_argument("exact F16 KV supports at most 16 grouped heads");
@@ -223,9 +230,27 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   top_tokens_ =
       static_cast<std::uint32_t*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
 
-  // Page geometry: every page holds all layers back to back
-  // (dense_fp4_provider.cpp:2582-2599, 6554-6588).
+  if (g_.mtp_layers) {
+    mtp_tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+    mtp_embedding_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
+    mtp_fusion_input_ =
+        static_cast<std::uint16_t*>(device_alloc(rows * 2U * g_.hidden * 2U));
+    mtp_hidden_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
+    mtp_last_hidden_ = static_cast<float*>(device_alloc(g_.hidden * 4U));
+    hip_check(hipMemset(mtp_last_hidden_, 0, g_.hidden * 4U),
+              "clear proposer hidden state");
+    mtp_logits_ = static_cast<float*>(device_alloc(g_.draft_vocabulary * 4U));
+    mtp_argmax_ = static_cast<std::uint32_t*>(device_alloc(4U));
+  }
+
+  // Page geometry: every page holds all target layers back to back, then the
+  // proposer's Q8 layer (dense_fp4_provider.cpp:2582-2599, 2690-2759,
+  // 6554-6588).
   kv_page_bytes_ = kv_bytes_per_token_layer() * g_.kv_page_tokens * g_.layers;
+  mtp_page_offset_ = (kv_page_bytes_ + 15U) & ~std::uint64_t{15U};
+  if (g_.mtp_layers)
+    kv_page_bytes_ = mtp_page_offset_ +
+                     qllm_q8_layer_bytes(g_.kv_page_tokens, g_.kv_heads, g_.head_dim);
   const std::size_t page_count =
       (g_.max_context + g_.kv_page_tokens - 1U) / g_.kv_page_tokens;
   pages_.assign(page_count, nullptr);
@@ -517,11 +542,76 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare_exact_decode(
       return {{er::ErrorCode::invalid_argument,
                "target program is not fully prepared"},
               {}};
+    if (g_.mtp_layers && !context.tensors.empty()) prepare_mtp(context.tensors);
+    if (g_.mtp_layers && !mtp_.ready)
+      return {{er::ErrorCode::invalid_argument,
+               "exact decode with an MTP layer needs the proposer's tensors"},
+              {}};
     exact_ = std::make_shared<PreparedMarker>(context.capability);
     return {er::Status::success(), exact_};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
   }
+}
+
+// Tensors of the exact-decode operation (validate_exact, :4730-4787).
+void Mi355DenseFp4Provider::prepare_mtp(
+    std::span<const er::PreparedTensorBinding> tensors) {
+  const auto require_shape = [](const DeviceFp4Matrix& matrix, std::uint32_t rows,
+                                std::uint32_t columns, const char* role) {
+    if (matrix.descriptor.rows != rows || matrix.descriptor.columns != columns)
+      throw std::runtime_error(std::string("tensor shape mismatch: ") + role);
+  };
+  const auto query_rows =
+      g_.query_heads * g_.head_dim * (g_.output_gated ? 2U : 1U);
+  mtp_.embedding_norm = upload_f32(tensor_for(tensors, "embedding_norm"), g_.hidden);
+  mtp_.hidden_norm = upload_f32(tensor_for(tensors, "hidden_norm"), g_.hidden);
+  mtp_.draft_norm = upload_f32(tensor_for(tensors, "draft_norm"), g_.hidden);
+  mtp_.fusion = upload_matrix(tensor_for(tensors, "fusion_projection"), true);
+  require_shape(mtp_.fusion, g_.hidden, 2U * g_.hidden, "fusion_projection");
+  auto& layer = mtp_.layer;
+  layer.input_norm =
+      upload_f32(tensor_for(tensors, "layer.0.input_norm"), g_.hidden);
+  DeviceFp4Matrix query =
+      upload_matrix(tensor_for(tensors, "layer.0.query_projection"), false);
+  DeviceFp4Matrix key =
+      upload_matrix(tensor_for(tensors, "layer.0.key_projection"), false);
+  DeviceFp4Matrix value =
+      upload_matrix(tensor_for(tensors, "layer.0.value_projection"), false);
+  require_shape(query, query_rows, g_.hidden, "layer.0.query_projection");
+  require_shape(key, g_.kv_heads * g_.head_dim, g_.hidden, "layer.0.key_projection");
+  require_shape(value, g_.kv_heads * g_.head_dim, g_.hidden,
+                "layer.0.value_projection");
+  layer.qkv = concatenate_rows({query, key, value});
+  layer.output =
+      upload_matrix(tensor_for(tensors, "layer.0.output_projection"), true);
+  require_shape(layer.output, g_.hidden, g_.query_heads * g_.head_dim,
+                "layer.0.output_projection");
+  if (g_.qk_norm) {
+    layer.query_norm =
+        upload_f32(tensor_for(tensors, "layer.0.query_norm"), g_.head_dim);
+    layer.key_norm =
+        upload_f32(tensor_for(tensors, "layer.0.key_norm"), g_.head_dim);
+  }
+  layer.post_attention_norm =
+      upload_f32(tensor_for(tensors, "layer.0.post_attention_norm"), g_.hidden);
+  layer.gate = upload_matrix(tensor_for(tensors, "layer.0.gate_projection"), true);
+  layer.up = upload_matrix(tensor_for(tensors, "layer.0.up_projection"), true);
+  layer.down = upload_matrix(tensor_for(tensors, "layer.0.down_projection"), true);
+  require_shape(layer.gate, g_.intermediate, g_.hidden, "layer.0.gate_projection");
+  require_shape(layer.up, g_.intermediate, g_.hidden, "layer.0.up_projection");
+  require_shape(layer.down, g_.hidden, g_.intermediate, "layer.0.down_projection");
+  finish_mtp_weights();
+}
+
+// project_prefix (:6280-6308): the proposer scores the first draft_vocabulary
+// rows of the output head; in either layout those are a leading byte range.
+void Mi355DenseFp4Provider::finish_mtp_weights() {
+  if (!head_ready_ && !head_.weights)
+    throw std::runtime_error("the output head must be prepared before the proposer");
+  mtp_.head_prefix = head_.descriptor;
+  mtp_.head_prefix.rows = g_.draft_vocabulary;
+  mtp_.ready = true;
 }
 
 er::CreateOperationRequestStateResult
@@ -552,16 +642,62 @@ er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
       if (token >= g_.vocabulary)
         return {er::ErrorCode::invalid_argument,
                 "synchronized token is outside the vocabulary"};
+    const auto rows =
+        static_cast<std::uint32_t>(synchronization.next_tokens.size());
+    if (rows > max_rows_ ||
+        synchronization.first_target_position > g_.max_context - rows)
+      return {er::ErrorCode::invalid_argument,
+              "exact decode synchronization is invalid"};
     state->synchronized_token = synchronization.next_tokens.back();
-    state->mtp_length =
-        synchronization.first_target_position +
-        static_cast<std::uint32_t>(synchronization.next_tokens.size()) - 1U;
     state->draft_valid = false;
     state->draft_predictions.clear();
+    // next_tokens[r] sits at position first_target_position + r + 1 and was
+    // chosen from the target's hidden state at first_target_position + r; the
+    // proposer is fed exactly these pairs (its cache lags the target's by one
+    // token), after which the guaranteed token stands at mtp_length.
+    state->mtp_length = synchronization.first_target_position;
+    if (mtp_.ready) {
+      const auto sample_position = synchronization.first_target_position + rows;
+      auto draft = run_mtp(*state, synchronization.next_tokens, hidden_,
+                           synchronization.produce_final_draft,
+                           synchronization.produce_final_draft
+                               ? &synchronization.request
+                               : nullptr,
+                           sample_position, 1U);
+      if (synchronization.produce_final_draft) {
+        if (!draft)
+          throw std::runtime_error("MTP synchronization produced no draft");
+        const auto reserved = synchronization.request.parameters.find(
+            "reserved_context_tokens");
+        const auto context_limit =
+            reserved == synchronization.request.parameters.end()
+                ? g_.max_context
+                : static_cast<std::uint32_t>(reserved->second);
+        extend_mtp_rollout(*state, synchronization.request, std::move(*draft),
+                           context_limit);
+      }
+    } else {
+      state->mtp_length += rows;
+    }
     return er::Status::success();
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};
   }
+}
+
+er::Status Mi355DenseFp4Provider::begin_stream(
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    std::uint32_t token) {
+  std::lock_guard lock(mutex_);
+  const auto state =
+      std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+  if (!state || token >= g_.vocabulary)
+    return {er::ErrorCode::invalid_argument, "stream start is invalid"};
+  state->synchronized_token = token;
+  state->mtp_length = 0U;
+  state->draft_valid = false;
+  state->draft_predictions.clear();
+  return er::Status::success();
 }
 
 er::Status Mi355DenseFp4Provider::set_draft_predictions(
@@ -910,13 +1046,14 @@ er::Status Mi355DenseFp4Provider::synchronize() {
 // selects the whole-vocabulary path of the scalar sampler (sample_token,
 // :773-799): the row is copied to the host and ordered there.
 er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
-    std::uint32_t row, const er::ProgramRequestContext& request) {
+    const float* row_logits, std::uint32_t vocabulary,
+    const std::uint32_t* device_argmax,
+    const er::ProgramRequestContext& request) {
   const auto stream = static_cast<hipStream_t>(stream_);
-  float* row_logits = logits_ + std::size_t{row} * g_.vocabulary;
   const auto temperature = request_parameter(request, "sampling_temperature_ppm");
   if (temperature == 0U) {
     std::uint32_t token{};
-    hip_check(hipMemcpyAsync(&token, argmax_tokens_ + row, sizeof(token),
+    hip_check(hipMemcpyAsync(&token, device_argmax, sizeof(token),
                              hipMemcpyDeviceToHost, stream),
               "copy exact greedy token");
     hip_check(hipStreamSynchronize(stream), "copy exact greedy token");
@@ -927,18 +1064,18 @@ er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
   const auto min_p = static_cast<std::uint32_t>(
       request_parameter(request, "sampling_min_p_ppm"));
   const auto top_k = request_parameter(request, "sampling_top_k");
-  if (top_k > kMaximumGpuSamplingTopK || top_k > g_.vocabulary)
+  if (top_k > kMaximumGpuSamplingTopK || top_k > vocabulary)
     throw std::runtime_error(
         "sampled exact decode requires top-k of at most 64 (0 = whole row)");
   std::vector<float> host_logits;
   std::vector<std::uint32_t> host_tokens;
   if (top_k == 0U) {
-    std::vector<float> full(g_.vocabulary);
+    std::vector<float> full(vocabulary);
     hip_check(hipMemcpyAsync(full.data(), row_logits, full.size() * 4U,
                              hipMemcpyDeviceToHost, stream),
               "copy logit row");
     hip_check(hipStreamSynchronize(stream), "copy logit row");
-    host_tokens.resize(g_.vocabulary);
+    host_tokens.resize(vocabulary);
     std::iota(host_tokens.begin(), host_tokens.end(), 0U);
     std::sort(host_tokens.begin(), host_tokens.end(),
               [&](std::uint32_t left, std::uint32_t right) {
@@ -948,11 +1085,11 @@ er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
                 if (std::isnan(b)) return true;
                 return a == b ? left < right : a > b;
               });
-    host_logits.reserve(g_.vocabulary);
+    host_logits.reserve(vocabulary);
     for (const auto token : host_tokens) host_logits.push_back(full[token]);
     sampling_logit_transfer_bytes_ += full.size() * 4U;
   } else {
-    status_check(qllm_topk_logits(row_logits, g_.vocabulary,
+    status_check(qllm_topk_logits(row_logits, vocabulary,
                                   static_cast<std::uint32_t>(top_k), top_logits_,
                                   top_tokens_, select_workspace_,
                                   select_workspace_bytes_, stream_));
@@ -971,6 +1108,176 @@ er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
   return er::make_sampling_distribution(
       host_logits, host_tokens, static_cast<std::uint32_t>(temperature), top_p,
       min_p);
+}
+
+// ---- the proposer (run_mtp / extend_mtp_rollout, :8681-8852) -----------------
+
+std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
+    DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
+    const float* previous_hidden, bool produce_logits,
+    const er::ProgramRequestContext* request, std::uint32_t sample_position,
+    std::uint32_t random_stream) {
+  if (!mtp_.ready || tokens.empty() || tokens.size() > max_rows_ ||
+      !previous_hidden || state.mtp_length + tokens.size() > g_.max_context)
+    throw std::runtime_error("invalid MTP microbatch");
+  const auto rows = static_cast<std::uint32_t>(tokens.size());
+  for (const auto token : tokens)
+    if (token >= g_.vocabulary)
+      throw std::runtime_error("MTP token is outside the vocabulary");
+  void* const stream = stream_;
+  const auto hip_stream = static_cast<hipStream_t>(stream_);
+  const std::uint32_t cache_position = state.mtp_length;       // row 0
+  const std::uint32_t rotary_position = state.mtp_length + 1U;  // row 0
+  ensure_pages(cache_position + rows - 1U);
+  hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
+                           hipMemcpyHostToDevice, hip_stream),
+            "upload MTP token batch");
+  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, mtp_tokens_,
+                                        mtp_embedding_, rows, stream));
+  // [RMSNorm(embedding) | RMSNorm(previous target hidden)] -> fusion projection
+  const std::size_t half_bytes = std::size_t{g_.hidden} * 2U;
+  status_check(qllm_rms_norm_batch(mtp_embedding_, mtp_.embedding_norm, nullptr,
+                                   normalized_, g_.hidden, rows, g_.hidden,
+                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
+  hip_check(hipMemcpy2DAsync(mtp_fusion_input_, 2U * half_bytes, normalized_,
+                             half_bytes, half_bytes, rows,
+                             hipMemcpyDeviceToDevice, hip_stream),
+            "assemble MTP normalized embedding batch");
+  status_check(qllm_rms_norm_batch(previous_hidden, mtp_.hidden_norm, nullptr,
+                                   normalized_, g_.hidden, rows, g_.hidden,
+                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
+  hip_check(hipMemcpy2DAsync(mtp_fusion_input_ + g_.hidden, 2U * half_bytes,
+                             normalized_, half_bytes, half_bytes, rows,
+                             hipMemcpyDeviceToDevice, hip_stream),
+            "assemble MTP target hidden batch");
+  status_check(qllm_fp4_gemm_bf16(&mtp_.fusion.descriptor, mtp_fusion_input_,
+                                  std::size_t{rows} * 2U * half_bytes,
+                                  mtp_hidden_, QLLM_OUT_F32, nullptr, rows,
+                                  stream));
+
+  // one transformer block over its own Q8 cache (run_full_attention + run_ffn)
+  const auto& layer = mtp_.layer;
+  const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+  const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
+  const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+  status_check(qllm_rms_norm_batch(mtp_hidden_, layer.input_norm, nullptr,
+                                   normalized_, g_.hidden, rows, g_.hidden,
+                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
+  const qllm_gemm_segment projections[3] = {
+      {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+      {key_, kv_rows, QLLM_OUT_F32},
+      {value_, kv_rows, QLLM_OUT_F32}};
+  status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
+                                        hidden_bytes, projections, 3U, rows,
+                                        stream));
+  status_check(qllm_qkv_rope_batch(
+      query_, query_stride, key_, layer.query_norm, layer.key_norm,
+      rotary_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
+      g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+  status_check(qllm_store_kv_paged_q8_batch(
+      key_, value_, const_cast<const void* const*>(device_page_table_),
+      mtp_page_offset_, g_.kv_page_tokens, cache_position, rows, g_.kv_heads,
+      g_.head_dim, stream));
+  qllm_q8_attention_launch launch{};
+  launch.query = query_;
+  launch.device_pages = const_cast<const void* const*>(device_page_table_);
+  launch.output = attention_;
+  launch.partial_maxima = partial_maxima_;
+  launch.partial_sums = partial_sums_;
+  launch.partial_outputs = partial_outputs_;
+  launch.page_offset_bytes = mtp_page_offset_;
+  launch.first_context_tokens = cache_position + 1U;
+  launch.rows = rows;
+  launch.page_tokens = g_.kv_page_tokens;
+  launch.query_heads = g_.query_heads;
+  launch.kv_heads = g_.kv_heads;
+  launch.head_dim = g_.head_dim;
+  launch.split_tokens = split_tokens_;
+  launch.maximum_splits = maximum_splits_;
+  launch.query_stride = query_stride;
+  launch.output_gated = g_.output_gated;
+  launch.output_kind = QLLM_OUT_BF16;
+  launch.stream = stream;
+  status_check(qllm_attention_paged_q8(&launch));
+  status_check(qllm_fp4_gemm_bf16(
+      &layer.output.descriptor, attention_,
+      std::size_t{rows} * g_.query_heads * g_.head_dim * 2U, mtp_hidden_,
+      QLLM_OUT_F32, mtp_hidden_, rows, stream));
+  status_check(qllm_rms_norm_batch(mtp_hidden_, layer.post_attention_norm,
+                                   nullptr, normalized_, g_.hidden, rows,
+                                   g_.hidden, g_.norm_epsilon,
+                                   g_.zero_centered_norm, stream));
+  status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor, &layer.up.descriptor,
+                                    normalized_, hidden_bytes, activation_, rows,
+                                    stream));
+  status_check(qllm_fp4_gemm_bf16(
+      &layer.down.descriptor, activation_,
+      std::size_t{rows} * g_.intermediate * 2U, mtp_hidden_, QLLM_OUT_F32,
+      mtp_hidden_, rows, stream));
+  state.mtp_length += rows;
+  ++mtp_passes_;
+  mtp_rows_ += rows;
+  if (!produce_logits) return std::nullopt;
+
+  // draft head: the last row, draft norm, the head's first draft_vocabulary rows
+  const float* final_hidden = mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden;
+  hip_check(hipMemcpyAsync(mtp_last_hidden_, final_hidden, g_.hidden * 4U,
+                           hipMemcpyDeviceToDevice, hip_stream),
+            "retain final MTP hidden state");
+  status_check(qllm_rms_norm_batch(final_hidden, mtp_.draft_norm, nullptr,
+                                   normalized_, g_.hidden, 1U, g_.hidden,
+                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
+  status_check(qllm_fp4_gemm_bf16(&mtp_.head_prefix, normalized_,
+                                  std::size_t{g_.hidden} * 2U, mtp_logits_,
+                                  QLLM_OUT_F32, nullptr, 1U, stream));
+  status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U,
+                                 mtp_argmax_, select_workspace_,
+                                 select_workspace_bytes_, stream));
+  DraftPrediction result;
+  if (request) {
+    result.distribution = distribution_from_logits(
+        mtp_logits_, g_.draft_vocabulary, mtp_argmax_, *request);
+    result.token = er::sample_distribution(
+        result.distribution,
+        er::counter_uniform(request_parameter(*request, "sampling_seed"),
+                            sample_position, random_stream));
+  } else {
+    hip_check(hipMemcpyAsync(&result.token, mtp_argmax_, sizeof(result.token),
+                             hipMemcpyDeviceToHost, hip_stream),
+              "copy final MTP draft token");
+    hip_check(hipStreamSynchronize(hip_stream), "copy final MTP draft token");
+    result.distribution.entries.push_back({result.token, 1.0});
+  }
+  return result;
+}
+
+void Mi355DenseFp4Provider::extend_mtp_rollout(
+    DenseFp4RequestState& state, const er::ProgramRequestContext& request,
+    DraftPrediction first, std::uint32_t context_limit) {
+  if (context_limit > g_.max_context || state.mtp_length >= context_limit ||
+      !(first.distribution.probability(first.token) > 0.0))
+    throw std::runtime_error("invalid MTP rollout root");
+  state.draft_predictions.clear();
+  state.draft_predictions.reserve(g_.draft_depth);
+  const auto committed_length = state.mtp_length;
+  if (committed_length + 1U >= context_limit)
+    throw std::runtime_error("MTP rollout root exceeds context");
+  state.draft_predictions.push_back(std::move(first));
+  while (state.draft_predictions.size() < g_.draft_depth &&
+         state.mtp_length + 2U < context_limit) {
+    // the next pass reads the proposer's own last hidden state before it
+    // replaces it (both on the provider's stream, in order)
+    const auto sample_position = state.mtp_length;
+    const std::uint32_t token[1] = {state.draft_predictions.back().token};
+    auto prediction = run_mtp(
+        state, token, mtp_last_hidden_, true, &request, sample_position,
+        1U + static_cast<std::uint32_t>(state.draft_predictions.size()));
+    if (!prediction) throw std::runtime_error("MTP rollout produced no proposal");
+    state.draft_predictions.push_back(std::move(*prediction));
+  }
+  state.draft_valid = !state.draft_predictions.empty();
+  // speculative rows of the proposer's cache are overwritten by the next pass
+  state.mtp_length = committed_length;
 }
 
 // ---- the verify step (execute_exact_decode ABI 2, :11156-11318) -------------
@@ -1010,8 +1317,9 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
     std::vector<er::SamplingDistribution> target_distributions;
     target_distributions.reserve(rows);
     for (std::uint32_t row = 0; row < rows; ++row)
-      target_distributions.push_back(
-          distribution_from_logits(row, invocation.request));
+      target_distributions.push_back(distribution_from_logits(
+          logits_ + std::size_t{row} * g_.vocabulary, g_.vocabulary,
+          argmax_tokens_ + row, invocation.request));
 
     const auto seed = request_parameter(invocation.request, "sampling_seed");
     std::size_t accepted{};
@@ -1038,10 +1346,33 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
               300U));
 
     const auto positions_advanced = static_cast<std::uint32_t>(accepted + 1U);
-    state->mtp_length = invocation.position + positions_advanced;
+    if (mtp_.ready) {
+      // advance the proposer over the accepted drafts and the next token (row r
+      // pairs the token at position + r + 1 with the target's hidden state at
+      // position + r), then roll the next drafts out (:11262-11288)
+      std::vector<std::uint32_t> mtp_tokens;
+      for (std::size_t index = 0; index < accepted; ++index)
+        mtp_tokens.push_back(state->draft_predictions[index].token);
+      mtp_tokens.push_back(next_token);
+      const bool future_exact = invocation.position + positions_advanced + 1U <
+                                invocation.context_limit;
+      state->mtp_length = invocation.position;
+      state->draft_valid = false;
+      state->draft_predictions.clear();
+      auto first = run_mtp(*state, mtp_tokens, hidden_, future_exact,
+                           future_exact ? &invocation.request : nullptr,
+                           invocation.position + positions_advanced, 1U);
+      if (future_exact) {
+        if (!first) throw std::runtime_error("next MTP rollout produced no root");
+        extend_mtp_rollout(*state, invocation.request, std::move(*first),
+                           invocation.context_limit);
+      }
+    } else {
+      state->mtp_length = invocation.position + positions_advanced;
+      state->draft_valid = false;
+      state->draft_predictions.clear();
+    }
     state->synchronized_token = next_token;
-    state->draft_valid = false;
-    state->draft_predictions.clear();
 
     er::ExactDecodeExecutionResult result;
     result.status = er::Status::success();
@@ -1147,6 +1478,27 @@ er::Status Mi355DenseFp4Provider::load_synthetic_weights(std::uint64_t seed) {
     }
     final_norm_ = ones(g_.hidden, unit);
     head_ = synthetic_matrix(g_.vocabulary, g_.hidden, next_seed(), true);
+    if (g_.mtp_layers) {
+      mtp_.embedding_norm = ones(g_.hidden, unit);
+      mtp_.hidden_norm = ones(g_.hidden, unit);
+      mtp_.draft_norm = ones(g_.hidden, unit);
+      mtp_.fusion = synthetic_matrix(g_.hidden, 2U * g_.hidden, next_seed(), true);
+      auto& layer = mtp_.layer;
+      layer.input_norm = ones(g_.hidden, unit);
+      layer.post_attention_norm = ones(g_.hidden, unit);
+      if (g_.qk_norm) {
+        layer.query_norm = ones(g_.head_dim, 0.0F);
+        layer.key_norm = ones(g_.head_dim, 0.0F);
+      }
+      layer.qkv = synthetic_matrix(query_rows + 2U * g_.kv_heads * g_.head_dim,
+                                   g_.hidden, next_seed(), true);
+      layer.output = synthetic_matrix(g_.hidden, g_.query_heads * g_.head_dim,
+                                      next_seed(), true);
+      layer.gate = synthetic_matrix(g_.intermediate, g_.hidden, next_seed(), true);
+      layer.up = synthetic_matrix(g_.intermediate, g_.hidden, next_seed(), true);
+      layer.down = synthetic_matrix(g_.hidden, g_.intermediate, next_seed(), true);
+      finish_mtp_weights();
+    }
     attention_ops_ = ffn_ops_ = g_.layers;
     embedding_ready_ = head_ready_ = true;
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
@@ -1190,6 +1542,19 @@ er::Status Mi355DenseFp4Provider::prefill_synthetic_kv(std::uint32_t tokens,
               stream_));
       }
     }
+    if (g_.mtp_layers) {
+      for (std::uint32_t first = 0; first < tokens; first += chunk) {
+        const std::uint32_t count = std::min(chunk, tokens - first);
+        const std::uint64_t salt = seed + (std::uint64_t{0xffffU} << 32U) + first;
+        status_check(qllm_fill_random(keys, count * width, 1U, salt, stream_));
+        status_check(qllm_fill_random(values, count * width, 1U,
+                                      salt ^ 0xabcdef12345ULL, stream_));
+        status_check(qllm_store_kv_paged_q8_batch(
+            keys, values, const_cast<const void* const*>(device_page_table_),
+            mtp_page_offset_, g_.kv_page_tokens, first, count, g_.kv_heads,
+            g_.head_dim, stream_));
+      }
+    }
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
               "prefill synthetic KV");
     (void)hipFree(keys);
@@ -1198,6 +1563,23 @@ er::Status Mi355DenseFp4Provider::prefill_synthetic_kv(std::uint32_t tokens,
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};
   }
+}
+
+er::Status Mi355DenseFp4Provider::copy_mtp_state(float* host_last_hidden,
+                                                 float* host_draft_logits) {
+  std::lock_guard lock(mutex_);
+  if (!mtp_.ready)
+    return {er::ErrorCode::invalid_argument, "the provider has no MTP layer"};
+  auto status = hipStreamSynchronize(static_cast<hipStream_t>(stream_));
+  if (status == hipSuccess && host_last_hidden)
+    status = hipMemcpy(host_last_hidden, mtp_last_hidden_, g_.hidden * 4U,
+                       hipMemcpyDeviceToHost);
+  if (status == hipSuccess && host_draft_logits)
+    status = hipMemcpy(host_draft_logits, mtp_logits_, g_.draft_vocabulary * 4U,
+                       hipMemcpyDeviceToHost);
+  if (status != hipSuccess)
+    return {er::ErrorCode::internal, hipGetErrorString(status)};
+  return er::Status::success();
 }
 
 er::Status Mi355DenseFp4Provider::copy_kv_page(std::uint32_t page_index,
@@ -1231,6 +1613,9 @@ Mi355DenseFp4Provider::telemetry() const {
   for (std::size_t depth = 0; depth < accepted_depth_calls_.size(); ++depth)
     values["provider_accepted_depth_" + std::to_string(depth)] =
         accepted_depth_calls_[depth];
+  values["provider_mtp_passes"] = mtp_passes_;
+  values["provider_mtp_rows"] = mtp_rows_;
+  values["provider_mtp_kv_page_offset"] = mtp_page_offset_;
   values["provider_weight_bytes"] = weight_bytes_;
   values["provider_kv_page_bytes"] = kv_page_bytes_;
   return values;

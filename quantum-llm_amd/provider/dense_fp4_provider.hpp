@@ -13,6 +13,8 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <optional>
+#include <span>
 #include <string>
 #include <vector>
 
@@ -47,6 +49,12 @@ struct DenseGeometry final {
   std::uint32_t kv_page_tokens{256};
   std::uint32_t max_context{};
   std::uint32_t draft_depth{4};
+  // The proposer (one MTP layer with its own Q8 KV cache): 0 = drafts come
+  // from outside through set_draft_predictions(), 1 = this provider runs it.
+  std::uint32_t mtp_layers{0};
+  // Rows of the output head the proposer scores (project_prefix); 0 stands
+  // for min(vocabulary, 65536).  A multiple of 32.
+  std::uint32_t draft_vocabulary{0};
 };
 
 struct DraftPrediction final {
@@ -78,6 +86,20 @@ struct LayerWeights final {
   DeviceFp4Matrix output, gate, up, down;
 };
 
+// Tensors of the exact-decode operation (validate_exact,
+// dense_fp4_provider.cpp:4730-4787): two input norms, the fusion projection
+// [hidden, 2*hidden], one transformer block, the draft norm.  Token embedding
+// and output head are the target's.
+struct MtpWeights final {
+  bool ready{};
+  float* embedding_norm{};
+  float* hidden_norm{};
+  float* draft_norm{};
+  DeviceFp4Matrix fusion;
+  LayerWeights layer;
+  qllm_fp4_matrix head_prefix{};   // the first draft_vocabulary rows of the head
+};
+
 class Mi355DenseFp4Provider final : public er::IOperationProvider {
  public:
   explicit Mi355DenseFp4Provider(const DenseGeometry& geometry);
@@ -101,7 +123,12 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       const std::shared_ptr<er::IOperationProviderRequestState>& state,
       const er::ExactDecodeInvocation& invocation) override;
 
-  // The proposer (run_mtp) is outside this provider's scope; whoever owns it
+  // A stream that starts at position 0 with `token` guaranteed: there is no
+  // earlier target position to synchronise from, so no draft is produced.
+  [[nodiscard]] er::Status begin_stream(
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      std::uint32_t token);
+  // Without an MTP layer (geometry.mtp_layers == 0) whoever owns the proposer
   // hands the drafts for the next verify step over here.
   [[nodiscard]] er::Status set_draft_predictions(
       const std::shared_ptr<er::IOperationProviderRequestState>& state,
@@ -141,6 +168,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                        double* microseconds,
                                        std::uint64_t* launches);
 
+  [[nodiscard]] er::Status copy_mtp_state(float* host_last_hidden,
+                                          float* host_draft_logits);
   [[nodiscard]] const float* logits() const noexcept { return logits_; }
   [[nodiscard]] const float* hidden() const noexcept { return hidden_; }
   [[nodiscard]] void* stream() const noexcept { return stream_; }
@@ -174,7 +203,24 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void enqueue_target(const std::uint32_t* device_tokens, std::uint32_t rows,
                       std::uint32_t first_position, bool deferred_positions);
   er::SamplingDistribution distribution_from_logits(
-      std::uint32_t row, const er::ProgramRequestContext& request);
+      const float* row_logits, std::uint32_t vocabulary,
+      const std::uint32_t* device_argmax,
+      const er::ProgramRequestContext& request);
+  // One proposer pass over `tokens` (run_mtp, dense_fp4_provider.cpp:8681-
+  // 8792): row r embeds tokens[r], takes previous_hidden row r (device, F32),
+  // is cached at position mtp_length + r and rotated at mtp_length + r + 1.
+  // With produce_logits the last row's draft (token + distribution) comes back.
+  std::optional<DraftPrediction> run_mtp(
+      DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
+      const float* previous_hidden, bool produce_logits,
+      const er::ProgramRequestContext* request, std::uint32_t sample_position,
+      std::uint32_t random_stream);
+  // extend_mtp_rollout, dense_fp4_provider.cpp:8794-8852
+  void extend_mtp_rollout(DenseFp4RequestState& state,
+                          const er::ProgramRequestContext& request,
+                          DraftPrediction first, std::uint32_t context_limit);
+  void prepare_mtp(std::span<const er::PreparedTensorBinding> tensors);
+  void finish_mtp_weights();
   void release();
 
   DenseGeometry g_;
@@ -192,11 +238,13 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   bool embedding_ready_{};
   bool head_ready_{};
   std::shared_ptr<const er::IPreparedOperation> exact_;
+  MtpWeights mtp_;
 
   // KV cache
   std::vector<void*> pages_;
   void** device_page_table_{};
   std::uint64_t kv_page_bytes_{};
+  std::uint64_t mtp_page_offset_{};   // the proposer's Q8 layer inside a page
   std::uint32_t split_tokens_{};
   std::uint32_t maximum_splits_{};
 
@@ -220,6 +268,15 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* top_logits_{};
   std::uint32_t* top_tokens_{};
 
+  // proposer workspaces
+  std::uint32_t* mtp_tokens_{};
+  float* mtp_embedding_{};
+  std::uint16_t* mtp_fusion_input_{};   // bf16 [rows, 2*hidden]
+  float* mtp_hidden_{};
+  float* mtp_last_hidden_{};
+  float* mtp_logits_{};
+  std::uint32_t* mtp_argmax_{};
+
   std::uint32_t* positions_{};   // device: cache, rotary, first-context
   std::vector<void*> graphs_;    // hipGraphExec_t per row count
   std::uint32_t last_graph_rows_{};
@@ -232,6 +289,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   std::uint64_t program_steps_{};
   std::uint64_t sampling_gpu_calls_{};
   std::uint64_t sampling_logit_transfer_bytes_{};
+  std::uint64_t mtp_passes_{};
+  std::uint64_t mtp_rows_{};
 };
 
 // Metadata factory, the analogue of make_sm86_dense_fp4_provider()

@@ -69,6 +69,8 @@ extern "C" qllm_provider* qllm_provider_create(
     g.kv_page_tokens = geometry->kv_page_tokens;
     g.max_context = geometry->max_context;
     g.draft_depth = geometry->draft_depth;
+    g.mtp_layers = geometry->mtp_layers;
+    g.draft_vocabulary = geometry->draft_vocabulary;
     auto handle = std::make_unique<qllm_provider>();
     handle->provider = std::make_unique<qllm::Mi355DenseFp4Provider>(g);
     return handle.release();
@@ -153,7 +155,9 @@ extern "C" int32_t qllm_provider_prepare_exact_decode(qllm_provider* provider,
   context.abi = 2U;
   context.parameters["draft_depth"] = provider->provider->geometry().draft_depth;
   context.parameters["source_mtp_layers"] = 1U;
+  context.tensors = provider->staged;
   auto result = provider->provider->prepare_exact_decode(context);
+  provider->staged.clear();
   if (!result.status.ok()) return from_status(result.status);
   provider->exact = result.operation;
   return QLLM_OK;
@@ -199,9 +203,14 @@ extern "C" int32_t qllm_provider_synchronize(qllm_provider* provider,
                                              uint32_t position) {
   if (!provider || !provider->exact || !provider->state)
     return fail(QLLM_INVALID_ARGUMENT, "exact decode is not prepared");
+  // `token` stands at `position`; it was chosen from the target's hidden state
+  // one position earlier, which is where the synchronisation batch starts
+  if (position == 0U)
+    return from_status(
+        provider->provider->begin_stream(provider->state, token));
   const uint32_t tokens[1] = {token};
-  er::ExactDecodeSynchronizationBatch batch{provider->request, tokens, position,
-                                            true};
+  er::ExactDecodeSynchronizationBatch batch{provider->request, tokens,
+                                            position - 1U, true};
   return from_status(provider->provider->synchronize_exact_decode_batch(
       *provider->exact, provider->state, batch));
 }
@@ -344,6 +353,30 @@ extern "C" int32_t qllm_provider_copy_kv_page(qllm_provider* provider,
                                               void* host_output) {
   if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
   return from_status(provider->provider->copy_kv_page(page_index, host_output));
+}
+
+extern "C" int32_t qllm_provider_copy_mtp_state(qllm_provider* provider,
+                                                float* host_last_hidden,
+                                                float* host_draft_logits) {
+  if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(
+      provider->provider->copy_mtp_state(host_last_hidden, host_draft_logits));
+}
+
+extern "C" uint32_t qllm_provider_drafts(const qllm_provider* provider,
+                                         uint32_t* tokens, uint32_t capacity) {
+  if (!provider || !provider->state) return 0U;
+  const auto state =
+      std::dynamic_pointer_cast<qllm::DenseFp4RequestState>(provider->state);
+  if (!state || !state->draft_valid) return 0U;
+  const auto count = static_cast<uint32_t>(state->draft_predictions.size());
+  for (uint32_t index = 0; tokens && index < count && index < capacity; ++index)
+    tokens[index] = state->draft_predictions[index].token;
+  return count;
+}
+
+extern "C" uint32_t qllm_provider_draft_vocabulary(const qllm_provider* provider) {
+  return provider ? provider->provider->geometry().draft_vocabulary : 0U;
 }
 
 extern "C" const float* qllm_provider_logits(const qllm_provider* provider) {

@@ -27,7 +27,8 @@ class DenseGeometry(Structure):
                 ("output_gated", c_int32), ("qk_norm", c_int32),
                 ("zero_centered_norm", c_int32), ("scale_scheme", c_uint32),
                 ("kv_encoding", c_uint32), ("kv_page_tokens", c_uint32),
-                ("max_context", c_uint32), ("draft_depth", c_uint32)]
+                ("max_context", c_uint32), ("draft_depth", c_uint32),
+                ("mtp_layers", c_uint32), ("draft_vocabulary", c_uint32)]
 
 
 SIGNATURES = {
@@ -53,6 +54,9 @@ SIGNATURES = {
     "qllm_provider_time_kernel": (c_int32, [c_void_p, c_char_p, c_uint32, c_uint32, POINTER(c_double), POINTER(c_uint64)]),
     "qllm_provider_kv_page_bytes": (c_uint64, [c_void_p]),
     "qllm_provider_copy_kv_page": (c_int32, [c_void_p, c_uint32, c_void_p]),
+    "qllm_provider_copy_mtp_state": (c_int32, [c_void_p, c_void_p, c_void_p]),
+    "qllm_provider_drafts": (c_uint32, [c_void_p, c_void_p, c_uint32]),
+    "qllm_provider_draft_vocabulary": (c_uint32, [c_void_p]),
     "qllm_provider_logits": (c_void_p, [c_void_p]),
     "qllm_provider_hidden": (c_void_p, [c_void_p]),
     "qllm_provider_stream": (c_void_p, [c_void_p]),
@@ -217,6 +221,22 @@ class Provider:
         _check(self.lib.qllm_provider_copy_kv_page(self.handle, page_index,
                                                    out.ctypes.data))
         return out
+
+    def mtp_state(self):
+        """(last hidden [hidden], draft logits [draft_vocabulary]) of the proposer."""
+        import numpy as np
+        hidden = np.empty(self.geometry.hidden, dtype=np.float32)
+        logits = np.empty(self.lib.qllm_provider_draft_vocabulary(self.handle),
+                          dtype=np.float32)
+        _check(self.lib.qllm_provider_copy_mtp_state(
+            self.handle, hidden.ctypes.data, logits.ctypes.data))
+        return hidden, logits
+
+    def drafts(self):
+        import numpy as np
+        tokens = np.zeros(16, dtype=np.uint32)
+        count = self.lib.qllm_provider_drafts(self.handle, tokens.ctypes.data, 16)
+        return tokens[:count].tolist()
 
     def weight_bytes(self):
         return self.lib.qllm_provider_weight_bytes(self.handle)

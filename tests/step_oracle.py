@@ -59,6 +59,20 @@ class TinyModel:
             self.blocks.append(block)
         self.final_norm = norm(hidden)
         self.head = matrix(vocabulary, hidden)
+        # the proposer: two input norms, fusion projection, one block, draft norm
+        # (validate_exact, dense_fp4_provider.cpp:4730-4787)
+        self.mtp = dict(
+            embedding_norm=norm(hidden), hidden_norm=norm(hidden), draft_norm=norm(hidden),
+            fusion=matrix(hidden, 2 * hidden),
+            input_norm=norm(hidden), post_attention_norm=norm(hidden),
+            query=matrix(q_rows, hidden), key=matrix(kv_heads * head_dim, hidden),
+            value=matrix(kv_heads * head_dim, hidden),
+            output=matrix(hidden, query_heads * head_dim),
+            gate=matrix(intermediate, hidden), up=matrix(intermediate, hidden),
+            down=matrix(hidden, intermediate))
+        if qk_norm:
+            self.mtp["query_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
+            self.mtp["key_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
 
     def linear(self, m, x_bf16, rows):
         codes, scales = m
@@ -157,8 +171,81 @@ def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
     return logits, hidden
 
 
+def run_mtp(model: TinyModel, tokens, previous_hidden, mtp_length, q8_pages,
+            page_tokens, draft_vocabulary, observed_pages=None, page_offset=0,
+            report=None):
+    """One proposer pass (run_mtp, dense_fp4_provider.cpp:8681-8792).  Row r
+    embeds tokens[r], takes previous_hidden[r], is cached at mtp_length + r and
+    rotated at mtp_length + r + 1.  q8_pages: list of uint8 arrays holding the
+    proposer's layer as reference records (oracle layout).  Returns (draft
+    logits [draft_vocabulary] of the last row, final hidden [rows, H]).
+    `observed_pages` (reference-record view of the implementation's pages) are
+    adopted record by record after counting differing bytes, as in run_target."""
+    m, w = model, model.mtp
+    rows = len(tokens)
+    d, Q, KV = m.head_dim, m.query_heads, m.kv_heads
+    stride = d * (2 if m.output_gated else 1)
+    codes, scales = m.embedding
+    embedding = ol.fp4_embedding(codes, scales, m.scheme, m.hidden, m.hidden, tokens)
+    fused = np.concatenate([
+        ol.rms_norm_rows(embedding, w["embedding_norm"], m.eps, m.zero_centered, True),
+        ol.rms_norm_rows(previous_hidden, w["hidden_norm"], m.eps, m.zero_centered, True)],
+        axis=1)
+    hidden = m.linear(w["fusion"], fused, m.hidden)
+    x = ol.rms_norm_rows(hidden, w["input_norm"], m.eps, m.zero_centered, True)
+    q = m.linear(w["query"], x, Q * stride).reshape(rows, Q, stride)
+    k = m.linear(w["key"], x, KV * d).reshape(rows, KV, d)
+    v = m.linear(w["value"], x, KV * d).reshape(rows, KV, d)
+    record_bytes = d + 2
+    for r in range(rows):
+        cache_position, rotary_position = mtp_length + r, mtp_length + r + 1
+        for h in range(Q):
+            q[r, h, :d] = ol.head_norm_rope(q[r, h, :d], w.get("query_norm"),
+                                            m.rotary_dim, rotary_position, m.eps,
+                                            m.rope_theta)
+        for h in range(KV):
+            k[r, h] = ol.head_norm_rope(k[r, h], w.get("key_norm"), m.rotary_dim,
+                                        rotary_position, m.eps, m.rope_theta)
+            page = q8_pages[cache_position // page_tokens]
+            ol.q8_store(page, page_offset, page_tokens, cache_position, h, KV, d,
+                        k[r, h], v[r, h])
+            if observed_pages is not None:
+                observed = observed_pages[cache_position // page_tokens]
+                record = (cache_position % page_tokens) * KV + h
+                for kind in range(2):
+                    first = page_offset + (kind * page_tokens * KV + record) * record_bytes
+                    part = slice(first, first + record_bytes)
+                    if report is not None:
+                        report["record_bytes"] = report.get("record_bytes", 0) + record_bytes
+                        report["record_byte_diffs"] = report.get("record_byte_diffs", 0) + int((page[part] != observed[part]).sum())
+                        # the same comparison on the dequantised values, relative
+                        # to the record's largest magnitude
+                        def decode(record):
+                            scale = float(record[d:].view(np.float16)[0])
+                            return record[:d].view(np.int8).astype(np.float64) * scale
+                        mine, theirs = decode(page[part].copy()), decode(observed[part].copy())
+                        report["value_error"] = max(
+                            report.get("value_error", 0.0),
+                            float(np.abs(mine - theirs).max() / max(np.abs(mine).max(), 1e-30)))
+                    page[part] = observed[part]
+    shape = ol.AttentionShape(rows, Q, KV, d, mtp_length + 1, page_tokens, 0,
+                              int(m.output_gated))
+    attention = ol.attention_q8(shape, q, q8_pages, page_offset)
+    attention = ol.bf16_round(attention.reshape(rows, Q * d))
+    hidden = hidden + m.linear(w["output"], attention, m.hidden)
+    x = ol.rms_norm_rows(hidden, w["post_attention_norm"], m.eps, m.zero_centered, True)
+    activation = ol.silu_product(m.linear(w["gate"], x, m.intermediate),
+                                 m.linear(w["up"], x, m.intermediate), True)
+    hidden = hidden + m.linear(w["down"], activation, m.hidden)
+    x = ol.rms_norm_rows(hidden[-1:], w["draft_norm"], m.eps, m.zero_centered, True)
+    head_codes, head_scales = m.head
+    logits = ol.fp4_linear_f64(head_codes[:draft_vocabulary], head_scales[:draft_vocabulary],
+                               m.scheme, draft_vocabulary, m.hidden, x)[0]
+    return logits, hidden
+
+
 def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
-                   kv_encoding=0):
+                   kv_encoding=0, mtp=False, draft_vocabulary=0):
     """Hands the host tensors to the provider operation by operation, the way
     the common VM calls prepare() in artifact order."""
     m = model
@@ -169,7 +256,7 @@ def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
         norm_epsilon=m.eps, output_gated=int(m.output_gated), qk_norm=int(m.qk_norm),
         zero_centered_norm=int(m.zero_centered), scale_scheme=m.scheme,
         kv_encoding=kv_encoding, kv_page_tokens=page_tokens, max_context=max_context,
-        draft_depth=4)
+        draft_depth=4, mtp_layers=int(mtp), draft_vocabulary=draft_vocabulary)
     abi = 16 if m.scheme == ol.SCALE_F16_BLOCK16 else 3
     tag = "fp4-f16-block16" if m.scheme == ol.SCALE_F16_BLOCK16 else "fp4-block32"
     d, Q, KV, H, I, V = m.head_dim, m.query_heads, m.kv_heads, m.hidden, m.intermediate, m.vocabulary
@@ -195,5 +282,23 @@ def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
     provider.stage_f32("hidden_norm", m.final_norm)
     provider.stage_fp4("output_head", *m.head, V, H, abi)
     provider.prepare(f"head.rmsnorm.token-select.{tag}.v1")
+    if mtp:
+        w = m.mtp
+        for role in ("embedding_norm", "hidden_norm", "draft_norm"):
+            provider.stage_f32(role, w[role])
+        provider.stage_fp4("fusion_projection", *w["fusion"], H, 2 * H, abi)
+        provider.stage_f32("layer.0.input_norm", w["input_norm"])
+        provider.stage_fp4("layer.0.query_projection", *w["query"],
+                           Q * d * (2 if m.output_gated else 1), H, abi)
+        provider.stage_fp4("layer.0.key_projection", *w["key"], KV * d, H, abi)
+        provider.stage_fp4("layer.0.value_projection", *w["value"], KV * d, H, abi)
+        provider.stage_fp4("layer.0.output_projection", *w["output"], H, Q * d, abi)
+        if m.qk_norm:
+            provider.stage_f32("layer.0.query_norm", w["query_norm"])
+            provider.stage_f32("layer.0.key_norm", w["key_norm"])
+        provider.stage_f32("layer.0.post_attention_norm", w["post_attention_norm"])
+        provider.stage_fp4("layer.0.gate_projection", *w["gate"], I, H, abi)
+        provider.stage_fp4("layer.0.up_projection", *w["up"], I, H, abi)
+        provider.stage_fp4("layer.0.down_projection", *w["down"], H, I, abi)
     provider.prepare_exact_decode(f"decode.mtp.dense-full-attention.{tag}.exact.v2")
     return provider
