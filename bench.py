@@ -117,6 +117,52 @@ def cpu_baseline(rows):
     }
 
 
+def measure_decode_cycle(qp, np, rows, steps, warmup):
+    """The whole decode cycle of the same model with the proposer inside the
+    provider: verify step, proposer advance over the emitted tokens, rollout of
+    the next four drafts (1 + 3 proposer passes over its Q8 cache, each ending
+    in the 65536-row draft head).  Random-init weights accept almost nothing,
+    so a cycle emits one token; the time per cycle is what real weights would
+    see as well."""
+    geometry = dict(MODEL)
+    geometry["mtp_layers"] = 1
+    needed = CONTEXT + (steps + warmup + 2) * rows + 8
+    geometry["max_context"] = (needed + 255) // 256 * 256
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(20241125)
+    provider.prefill_synthetic_kv(CONTEXT, 7)
+    provider.prepare_exact_decode("decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2")
+    provider.begin_request(temperature_ppm=0)
+    token, position = 1, CONTEXT
+    provider.synchronize(token, position)
+    emitted = 0
+    begin = passes = None
+    for index in range(steps + warmup):
+        if index == warmup:
+            provider.synchronize_stream()
+            begin = time.perf_counter()
+            passes = provider.telemetry("provider_mtp_passes")
+        tokens, token, advanced = provider.verify(token, position, geometry["max_context"])
+        position += advanced
+        if index >= warmup:
+            emitted += len(tokens)
+    provider.synchronize_stream()
+    elapsed = time.perf_counter() - begin
+    report = {
+        "tok_s": round(emitted / elapsed, 2),
+        "ms_per_cycle": round(1000.0 * elapsed / steps, 4),
+        "cycles": steps,
+        "emitted_tokens": emitted,
+        "proposer_passes_per_cycle": round(
+            (provider.telemetry("provider_mtp_passes") - passes) / steps, 2),
+        "accepted_drafts": int(provider.telemetry("provider_accepted_drafts")),
+        "projected_tok_s_at_reference_acceptance_2.6667": round(
+            2.6667 * steps / elapsed, 1),
+    }
+    provider.close()
+    return report
+
+
 def measure_long_contexts(qp, np, rows):
     """tok/s of the same 64-layer verify step with the Q4H cache prefilled to
     131072 tokens, and the exact-F16 attention kernel over 262144 tokens
@@ -193,6 +239,9 @@ def main():
     parser.add_argument("--skip-long-contexts", action="store_true",
                         help="skip the 131072-token step and the 262144-token F16 "
                              "attention measurements")
+    parser.add_argument("--skip-decode-cycle", action="store_true",
+                        help="leave out the decode cycle with the proposer (a second "
+                             "provider with the MTP layer)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one 256 MiB device copy (a kernel of known "
                              "traffic to scale hardware counters by)")
@@ -287,8 +336,14 @@ def main():
     weight_bytes = provider.weight_bytes()
     accepted_drafts = int(provider.telemetry("provider_accepted_drafts"))
     long_context = {}
-    if arguments.layers == MODEL["layers"] and not arguments.skip_long_contexts:
+    decode_cycle = {}
+    if arguments.layers == MODEL["layers"] and not arguments.skip_decode_cycle:
         provider.close()
+        provider = None
+        decode_cycle = measure_decode_cycle(qp, np, rows, min(steps, 20), min(warmup, 3))
+    if arguments.layers == MODEL["layers"] and not arguments.skip_long_contexts:
+        if provider is not None:
+            provider.close()
         provider = None
         long_context = measure_long_contexts(qp, np, rows)
     layers = geometry["layers"]
@@ -334,6 +389,8 @@ def main():
     }
     if provider is not None:
         provider.close()
+    if decode_cycle:
+        result["decode_cycle_with_proposer"] = decode_cycle
     if long_context:
         result["long_context"] = long_context
     if arguments.calibration_copy:

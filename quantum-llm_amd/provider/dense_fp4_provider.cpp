@@ -197,6 +197,8 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   if (const char* eager = std::getenv("QLLM_PROVIDER_EAGER"))
     use_graphs_ = eager[0] == '0';
   hidden_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
+  // read by the proposer when a stream is synchronised before any target pass
+  hip_check(hipMemset(hidden_, 0, rows * g_.hidden * 4U), "clear hidden state");
   normalized_ = static_cast<std::uint16_t*>(device_alloc(rows * widest * 2U));
   query_ = static_cast<float*>(device_alloc(rows * query_width * 4U));
   key_ = static_cast<float*>(device_alloc(rows * kv_width * 4U));
