@@ -184,6 +184,21 @@ int32_t qllm_rms_norm_batch(const float* input, const float* weight,
                             uint32_t elements, float epsilon,
                             int32_t zero_centered, void* stream);
 
+/* Two normalisations into one bf16 batch: output row r, of 2 * elements
+ * columns, is [RMSNorm(first[r]) | RMSNorm(second[r])], each half with its own
+ * weight (either may be NULL) and the values of qllm_rms_norm_batch.  The
+ * proposer's fusion input; replaces two normalize_rows calls and the two
+ * cudaMemcpy2D that interleave them (runtime/tools/dense_fp4_provider.cpp:
+ * 8710-8723).  elements % 4 == 0, at most 16384; inputs and weights 16-byte
+ * aligned. */
+int32_t qllm_rms_norm_concat_batch(const float* first,
+                                   const float* first_weight,
+                                   const float* second,
+                                   const float* second_weight,
+                                   void* output_bf16, uint32_t rows,
+                                   uint32_t elements, float epsilon,
+                                   int32_t zero_centered, void* stream);
+
 /* replaces add_in_place (transformer_kernels.hpp:310-312). */
 int32_t qllm_add_in_place(float* destination, const float* source,
                           uint32_t elements, int32_t bf16_output,
@@ -240,6 +255,18 @@ int32_t qllm_qkv_rope_batch(float* query, uint32_t query_stride, float* key,
                             uint32_t head_dim, uint32_t rotary_dim,
                             float epsilon, float rope_theta,
                             int32_t bf16_activations, void* stream);
+
+/* qllm_qkv_rope_batch with the position read on the device when the kernel
+ * runs: device_positions[1] = first rotary position. */
+int32_t qllm_qkv_rope_batch_deferred(float* query, uint32_t query_stride,
+                                     float* key, const float* q_norm_weight,
+                                     const float* k_norm_weight,
+                                     const uint32_t* device_positions,
+                                     uint32_t rows, uint32_t query_heads,
+                                     uint32_t kv_heads, uint32_t head_dim,
+                                     uint32_t rotary_dim, float epsilon,
+                                     float rope_theta,
+                                     int32_t bf16_activations, void* stream);
 
 /* replaces store_gqa_kv_paged_q4_per_head_batch (the store-only form used
  * by runtime/tools/dense_fp4_cuda_smoke.cpp:1828-1832). */
@@ -364,6 +391,14 @@ int32_t qllm_store_kv_paged_q8_batch(const float* key, const float* value,
                                      uint32_t rows, uint32_t kv_heads,
                                      uint32_t head_dim, void* stream);
 
+/* The same store with the position read on the device when the kernel runs:
+ * device_positions[0] = first cache position. */
+int32_t qllm_store_kv_paged_q8_batch_deferred(
+    const float* key, const float* value, const void* const* page_table,
+    size_t page_offset_bytes, uint32_t page_tokens,
+    const uint32_t* device_positions, uint32_t rows, uint32_t kv_heads,
+    uint32_t head_dim, void* stream);
+
 /* replaces gated_gqa_attention_microbatch_paged_q8_tensor_core and
  * gated_gqa_attention_decode_paged_q8_tensor_core (transformer_kernels.hpp:
  * 873, 944; launch struct PagedQ8GatedGqaPrefillLaunch): row r attends tokens
@@ -393,11 +428,25 @@ typedef struct qllm_q8_attention_launch {
   int32_t output_gated;
   uint32_t output_kind;
   void* stream;
+  /* optional: when set, first_context_tokens is read from
+   * device_positions[2] when the kernels run and every split is launched */
+  const uint32_t* device_positions;
 } qllm_q8_attention_launch;
 
 int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launch);
 
 /* ---- token selection ------------------------------------------------------------ */
+
+/* Chains greedy proposer passes on the device (no counterpart in the
+ * reference, whose rollout, dense_fp4_provider.cpp:8794-8852, returns to the
+ * host after every pass): selected[0] becomes next_token[0] and
+ * draft_tokens[device_positions[3]] (when that slot is below `capacity`);
+ * device_positions[0..2] - cache position, rotary position, context tokens -
+ * advance by `rows`, the pass's row count, and the draft slot [3] by one. */
+int32_t qllm_rollout_advance(const uint32_t* selected, uint32_t* next_token,
+                             uint32_t* draft_tokens, uint32_t capacity,
+                             uint32_t rows, uint32_t* device_positions,
+                             void* stream);
 
 /* replaces argmax_batch (transformer_kernels.hpp:1266-1269): ties to the
  * lower index, NaN never wins.  workspace: at least

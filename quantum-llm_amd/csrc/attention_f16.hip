@@ -59,10 +59,11 @@ __global__ void f16_store_kernel(const float* key, const float* value,
 __global__ __launch_bounds__(64) void q8_store_kernel(
     const float* key, const float* value, const void* const* page_table,
     size_t page_offset, uint32_t page_tokens, uint32_t first_cache_position,
-    uint32_t kv_heads, uint32_t head_dim) {
+    uint32_t kv_heads, uint32_t head_dim, const uint32_t* device_positions) {
   const uint32_t lane = threadIdx.x;
   const uint32_t kv_head = blockIdx.x;
   const uint32_t row = blockIdx.y;
+  if (device_positions) first_cache_position = device_positions[0];
   const uint32_t position = first_cache_position + row;
   uint8_t* page = static_cast<uint8_t*>(const_cast<void*>(
                       page_table[position / page_tokens])) + page_offset;
@@ -130,6 +131,7 @@ struct F16SplitArgs {
   uint32_t split_tokens;
   uint32_t maximum_splits;
   size_t page_offset;   // Q8: byte offset of the layer inside a page
+  const uint32_t* device_positions;  // optional: [2] = first_context_tokens
 };
 
 constexpr uint32_t kF16Tile = 32;  // tokens per wave step
@@ -170,7 +172,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
   const uint32_t split = blockIdx.y;
   const uint32_t group = args.query_heads / args.kv_heads;
   const uint32_t matrix_rows = args.rows * group;
-  const uint32_t first_context_tokens = args.first_context_tokens;
+  const uint32_t first_context_tokens =
+      args.device_positions ? args.device_positions[2]
+                            : args.first_context_tokens;
   const uint32_t last_context = first_context_tokens + args.rows - 1u;
   const uint32_t context_tiles = (last_context + kF16Tile - 1u) / kF16Tile;
   uint32_t tile_first, tile_last;
@@ -561,8 +565,22 @@ extern "C" int32_t qllm_store_kv_paged_q8_batch(
     return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 K/V store");
   q8_store_kernel<<<dim3(kv_heads, rows), 64, 0, as_stream(stream)>>>(
       key, value, page_table, page_offset_bytes, page_tokens,
-      first_cache_position, kv_heads, head_dim);
+      first_cache_position, kv_heads, head_dim, nullptr);
   return launched("Q8 K/V store");
+}
+
+extern "C" int32_t qllm_store_kv_paged_q8_batch_deferred(
+    const float* key, const float* value, const void* const* page_table,
+    size_t page_offset_bytes, uint32_t page_tokens,
+    const uint32_t* device_positions, uint32_t rows, uint32_t kv_heads,
+    uint32_t head_dim, void* stream) {
+  if (!key || !value || !page_table || !page_tokens || !device_positions ||
+      !rows || !kv_heads || !head_dim || page_offset_bytes % 16u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid deferred Q8 K/V store");
+  q8_store_kernel<<<dim3(kv_heads, rows), 64, 0, as_stream(stream)>>>(
+      key, value, page_table, page_offset_bytes, page_tokens, 0u, kv_heads,
+      head_dim, device_positions);
+  return launched("deferred Q8 K/V store");
 }
 
 extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launch) {
@@ -570,7 +588,8 @@ extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launc
       (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
       launch->query_stride % 4u || !launch->partial_maxima ||
       !launch->partial_sums || !launch->partial_outputs ||
-      !launch->first_context_tokens || !launch->rows ||
+      (!launch->device_positions && !launch->first_context_tokens) ||
+      !launch->rows ||
       !launch->page_tokens || launch->page_tokens % kF16Tile ||
       launch->page_offset_bytes % 16u || !launch->query_heads ||
       !launch->kv_heads || launch->query_heads % launch->kv_heads ||
@@ -590,10 +609,12 @@ extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launc
                 "Q8 paged attention: rows * (query_heads/kv_heads) exceeds "
                 "48 (32 at head_dim 256)");
   const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  // with device-side positions the context is not known here: cover every
+  // split (workgroups past the context write neutral partials)
   const uint32_t splits =
-      launch->split_tokens
-          ? (last_context + launch->split_tokens - 1u) / launch->split_tokens
-          : launch->maximum_splits;
+      launch->device_positions || !launch->split_tokens
+          ? launch->maximum_splits
+          : (last_context + launch->split_tokens - 1u) / launch->split_tokens;
   if (splits > launch->maximum_splits)
     return fail(QLLM_INVALID_ARGUMENT,
                 "Q8 paged attention: context needs more splits than "
@@ -613,6 +634,7 @@ extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launc
   args.split_tokens = launch->split_tokens;
   args.maximum_splits = launch->maximum_splits;
   args.page_offset = launch->page_offset_bytes;
+  args.device_positions = launch->device_positions;
   const dim3 grid(launch->kv_heads, splits);
   const hipStream_t stream = as_stream(launch->stream);
   const int32_t status =
@@ -625,5 +647,5 @@ extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launc
       launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
       launch->output, launch->output_kind, launch->first_context_tokens,
       launch->maximum_splits, launch->split_tokens, launch->rows,
-      launch->query_heads, launch->head_dim, nullptr, stream);
+      launch->query_heads, launch->head_dim, launch->device_positions, stream);
 }

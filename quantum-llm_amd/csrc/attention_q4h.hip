@@ -1056,6 +1056,26 @@ extern "C" int32_t qllm_qkv_rope_batch(
   return launched("QKV rope batch");
 }
 
+extern "C" int32_t qllm_qkv_rope_batch_deferred(
+    float* query, uint32_t query_stride, float* key,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const uint32_t* device_positions, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream) {
+  if (!query || !key || !device_positions || !rows || !query_heads ||
+      !kv_heads || query_heads < kv_heads || query_heads % kv_heads ||
+      !head_dim || head_dim > 256u || head_dim % 2u ||
+      query_stride < head_dim || !rotary_dim || rotary_dim > head_dim ||
+      rotary_dim % 2u || !(epsilon > 0.0f) || !(rope_theta > 0.0f))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid deferred QKV rope batch");
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
+      query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
+      0u, 1u, 0u, 0u, query_heads, kv_heads, head_dim, rotary_dim, epsilon,
+      rope_theta, bf16_activations != 0, device_positions);
+  return launched("deferred QKV rope batch");
+}
+
 extern "C" int32_t qllm_quantize_gqa_queries_q8(
     const float* query, uint32_t query_stride, int8_t* q8, float* query_scales,
     uint32_t rows, uint32_t query_heads, uint32_t head_dim, void* stream) {

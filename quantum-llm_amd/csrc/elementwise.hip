@@ -97,6 +97,43 @@ __global__ __launch_bounds__(256) void fp4_embedding_batch_kernel(
   }
 }
 
+// Same values as fp4_embedding_batch_kernel, eight columns (one dword of
+// codes, half a scale block) per thread and the row spread over blockIdx.y,
+// so that a one-token lookup is not a single workgroup's serial loop.
+__global__ __launch_bounds__(256) void fp4_embedding_batch_wide_kernel(
+    const uint8_t* weights, const uint8_t* scales, uint32_t scheme,
+    const uint32_t* tokens, float* output, uint32_t columns,
+    uint32_t padded_columns) {
+  const uint32_t request = blockIdx.x;
+  const uint32_t column = (blockIdx.y * blockDim.x + threadIdx.x) * 8u;
+  if (column >= columns) return;
+  const size_t token = tokens[request];
+  const uint32_t codes = *reinterpret_cast<const uint32_t*>(
+      weights + token * (padded_columns / 2u) + column / 2u);
+  float scale;
+  if (scheme == QLLM_SCALE_F16_BLOCK16)
+    scale = f16_bits_to_f32(reinterpret_cast<const uint16_t*>(
+        scales)[token * (padded_columns / 16u) + column / 16u]);
+  else
+    scale = ue8m0_to_f32(scales[token * (padded_columns / 32u) + column / 32u]);
+  float values[8];
+#pragma unroll
+  for (uint32_t i = 0; i < 8u; ++i) {
+    const uint32_t code = (codes >> (4u * i)) & 0x0fu;
+    const uint32_t index = code & 7u;
+    const float twice = index <= 4u ? static_cast<float>(index)
+                        : index == 5u ? 6.0f
+                        : index == 6u ? 8.0f
+                                      : 12.0f;
+    const float value = twice * 0.5f * scale;
+    values[i] = (code & 8u) ? -value : value;
+  }
+  float4* destination = reinterpret_cast<float4*>(
+      output + static_cast<size_t>(request) * columns + column);
+  destination[0] = make_float4(values[0], values[1], values[2], values[3]);
+  destination[1] = make_float4(values[4], values[5], values[6], values[7]);
+}
+
 // transformer_kernels.cu:2469-2521
 __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
     const float* input, const float* weight, float* output_f32,
@@ -132,14 +169,14 @@ __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
 // Same operation for rows of up to 16384 elements (a multiple of 4): 1024
 // threads per row, the row is read once with 16-byte loads and kept in
 // registers between the reduction and the scaling.
-__global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
-    const float* input, const float* weight, float* output_f32,
-    uint16_t* output_bf16, uint32_t bf16_padded_columns, uint32_t elements,
-    float epsilon, bool zero_centered) {
-  __shared__ float scratch[16];
-  const uint32_t row = blockIdx.x;
-  const float4* x =
-      reinterpret_cast<const float4*>(input + static_cast<size_t>(row) * elements);
+// One row of up to 16384 elements (a multiple of four) on 1024 threads:
+// `out_f32` / `out_bf16` point at the row's outputs (either may be null) and
+// bf16 columns [elements, bf16_columns) are zeroed.
+__device__ __forceinline__ void rms_norm_row_wide(
+    const float* input_row, const float* weight, float* out_f32,
+    uint16_t* out_bf16, uint32_t bf16_columns, uint32_t elements,
+    float epsilon, bool zero_centered, float* scratch) {
+  const float4* x = reinterpret_cast<const float4*>(input_row);
   const uint32_t vectors = elements / 4u;
   // the row and its weights are fetched together, before the reduction
   float4 values[4];
@@ -176,21 +213,47 @@ __global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
     result.y = values[slot].y * inverse * factor.y;
     result.z = values[slot].z * inverse * factor.z;
     result.w = values[slot].w * inverse * factor.w;
-    if (output_f32)
-      reinterpret_cast<float4*>(output_f32 +
-                                static_cast<size_t>(row) * elements)[index] = result;
-    if (output_bf16) {
+    if (out_f32) reinterpret_cast<float4*>(out_f32)[index] = result;
+    if (out_bf16) {
       uint2 packed;
       packed.x = f32_to_bf16_bits(result.x) | (f32_to_bf16_bits(result.y) << 16);
       packed.y = f32_to_bf16_bits(result.z) | (f32_to_bf16_bits(result.w) << 16);
-      reinterpret_cast<uint2*>(output_bf16 + static_cast<size_t>(row) *
-                                                 bf16_padded_columns)[index] = packed;
+      reinterpret_cast<uint2*>(out_bf16)[index] = packed;
     }
   }
-  if (output_bf16)
-    for (uint32_t index = elements + threadIdx.x; index < bf16_padded_columns;
+  if (out_bf16)
+    for (uint32_t index = elements + threadIdx.x; index < bf16_columns;
          index += 1024u)
-      output_bf16[static_cast<size_t>(row) * bf16_padded_columns + index] = 0u;
+      out_bf16[index] = 0u;
+}
+
+__global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
+    const float* input, const float* weight, float* output_f32,
+    uint16_t* output_bf16, uint32_t bf16_padded_columns, uint32_t elements,
+    float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  rms_norm_row_wide(
+      input + row * elements, weight,
+      output_f32 ? output_f32 + row * elements : nullptr,
+      output_bf16 ? output_bf16 + row * bf16_padded_columns : nullptr,
+      bf16_padded_columns, elements, epsilon, zero_centered, scratch);
+}
+
+// Row r of the output is [RMSNorm(first[r]) | RMSNorm(second[r])] in bf16:
+// blockIdx.y picks the half.
+__global__ __launch_bounds__(1024) void rms_norm_concat_kernel(
+    const float* first, const float* first_weight, const float* second,
+    const float* second_weight, uint16_t* output_bf16, uint32_t elements,
+    float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  const bool second_half = blockIdx.y != 0u;
+  rms_norm_row_wide(
+      (second_half ? second : first) + row * elements,
+      second_half ? second_weight : first_weight, nullptr,
+      output_bf16 + row * 2u * elements + (second_half ? elements : 0u),
+      elements, elements, epsilon, zero_centered, scratch);
 }
 
 // transformer_kernels.cu:2522-2528
@@ -302,10 +365,21 @@ extern "C" int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
       matrix->layout != QLLM_LAYOUT_ROW_MAJOR || !tokens ||
       !output || !batch)
     return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 embedding batch");
-  fp4_embedding_batch_kernel<<<batch, 256, 0, as_stream(stream)>>>(
-      matrix->weights, static_cast<const uint8_t*>(matrix->scales),
-      matrix->scale_scheme, tokens, output, matrix->columns,
-      matrix->padded_columns);
+  const bool wide =
+      matrix->columns % 8u == 0u && matrix->padded_columns % 8u == 0u &&
+      ((reinterpret_cast<uintptr_t>(matrix->weights) & 3u) |
+       (reinterpret_cast<uintptr_t>(output) & 15u)) == 0u;
+  if (wide)
+    fp4_embedding_batch_wide_kernel<<<dim3(batch, (matrix->columns / 8u + 255u) / 256u),
+                                      256, 0, as_stream(stream)>>>(
+        matrix->weights, static_cast<const uint8_t*>(matrix->scales),
+        matrix->scale_scheme, tokens, output, matrix->columns,
+        matrix->padded_columns);
+  else
+    fp4_embedding_batch_kernel<<<batch, 256, 0, as_stream(stream)>>>(
+        matrix->weights, static_cast<const uint8_t*>(matrix->scales),
+        matrix->scale_scheme, tokens, output, matrix->columns,
+        matrix->padded_columns);
   return launched("FP4 embedding batch");
 }
 
@@ -334,6 +408,25 @@ extern "C" int32_t qllm_rms_norm_batch(const float* input, const float* weight,
         input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
         bf16_padded_columns, elements, epsilon, zero_centered != 0);
   return launched("RMSNorm batch");
+}
+
+extern "C" int32_t qllm_rms_norm_concat_batch(
+    const float* first, const float* first_weight, const float* second,
+    const float* second_weight, void* output_bf16, uint32_t rows,
+    uint32_t elements, float epsilon, int32_t zero_centered, void* stream) {
+  if (!first || !second || !output_bf16 || !rows || !elements ||
+      elements % 4u || elements > 16384u || !(epsilon > 0.0f) ||
+      ((reinterpret_cast<uintptr_t>(first) |
+        reinterpret_cast<uintptr_t>(first_weight) |
+        reinterpret_cast<uintptr_t>(second) |
+        reinterpret_cast<uintptr_t>(second_weight)) & 15u) ||
+      (reinterpret_cast<uintptr_t>(output_bf16) & 7u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid RMSNorm concat batch");
+  rms_norm_concat_kernel<<<dim3(rows, 2u), 1024, 0, as_stream(stream)>>>(
+      first, first_weight, second, second_weight,
+      static_cast<uint16_t*>(output_bf16), elements, epsilon,
+      zero_centered != 0);
+  return launched("RMSNorm concat batch");
 }
 
 extern "C" int32_t qllm_add_in_place(float* destination, const float* source,

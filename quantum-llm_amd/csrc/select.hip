@@ -10,7 +10,7 @@ namespace qllm {
 namespace {
 
 constexpr uint32_t kNoIndex = 0xffffffffu;
-constexpr uint32_t kArgmaxChunk = 8192;   // items per stage-1 block
+constexpr uint32_t kArgmaxChunk = 2048;   // items per stage-1 block
 constexpr uint32_t kTopkChunk = 4096;     // items per stage-1 block
 constexpr uint32_t kTopkThreads = 256;
 constexpr uint32_t kTopkPerThread = kTopkChunk / kTopkThreads;
@@ -64,11 +64,34 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(
   const uint32_t last = min(count, first + kArgmaxChunk);
   float best = -INFINITY;
   uint32_t index = kNoIndex;
-  for (uint32_t item = first + threadIdx.x; item < last; item += blockDim.x) {
-    const float value = row[item];
-    if (better(value, item, best, index)) {
-      best = value;
-      index = item;
+  if (last - first == kArgmaxChunk &&
+      (reinterpret_cast<uintptr_t>(row + first) & 15u) == 0u) {
+    // a whole, aligned chunk: both 16-byte loads of a thread are in flight
+    // before the first comparison
+    float4 loaded[kArgmaxChunk / 1024u];
+#pragma unroll
+    for (uint32_t part = 0; part < kArgmaxChunk / 1024u; ++part)
+      loaded[part] = *reinterpret_cast<const float4*>(
+          row + first + part * 1024u + threadIdx.x * 4u);
+#pragma unroll
+    for (uint32_t part = 0; part < kArgmaxChunk / 1024u; ++part) {
+      const uint32_t item = first + part * 1024u + threadIdx.x * 4u;
+      const float four[4] = {loaded[part].x, loaded[part].y, loaded[part].z,
+                             loaded[part].w};
+#pragma unroll
+      for (uint32_t lane = 0; lane < 4u; ++lane)
+        if (better(four[lane], item + lane, best, index)) {
+          best = four[lane];
+          index = item + lane;
+        }
+    }
+  } else {
+    for (uint32_t item = first + threadIdx.x; item < last; item += blockDim.x) {
+      const float value = row[item];
+      if (better(value, item, best, index)) {
+        best = value;
+        index = item;
+      }
     }
   }
   block_best(best, index, shared_values, shared_indices);
@@ -96,6 +119,20 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(
   }
   block_best(best, index, shared_values, shared_indices);
   if (threadIdx.x == 0u) output[request] = index;
+}
+
+__global__ __launch_bounds__(64) void rollout_advance_kernel(
+    const uint32_t* selected, uint32_t* next_token, uint32_t* draft_tokens,
+    uint32_t capacity, uint32_t rows, uint32_t* positions) {
+  if (threadIdx.x != 0u) return;
+  const uint32_t token = selected[0];
+  const uint32_t slot = positions[3];
+  next_token[0] = token;
+  if (slot < capacity) draft_tokens[slot] = token;
+  positions[0] += rows;
+  positions[1] += rows;
+  positions[2] += rows;
+  positions[3] = slot + 1u;
 }
 
 // Stage 1: every block extracts the top_k of its chunk, in order, by top_k
@@ -215,6 +252,19 @@ extern "C" int32_t qllm_argmax_batch(const float* values, uint32_t count,
   argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
       partial_values, partial_indices, blocks, output);
   return launched("argmax batch");
+}
+
+extern "C" int32_t qllm_rollout_advance(const uint32_t* selected,
+                                        uint32_t* next_token,
+                                        uint32_t* draft_tokens,
+                                        uint32_t capacity, uint32_t rows,
+                                        uint32_t* device_positions,
+                                        void* stream) {
+  if (!selected || !next_token || !draft_tokens || !rows || !device_positions)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid rollout advance");
+  rollout_advance_kernel<<<1, 64, 0, as_stream(stream)>>>(
+      selected, next_token, draft_tokens, capacity, rows, device_positions);
+  return launched("rollout advance");
 }
 
 extern "C" size_t qllm_topk_workspace_bytes(uint32_t count, uint32_t top_k) {

@@ -14,6 +14,7 @@ namespace qllm {
 namespace {
 
 constexpr std::uint32_t kMaximumGpuSamplingTopK = 64U;  // provider.cpp:8359
+constexpr std::uint32_t kMaximumDraftDepth = 7U;
 
 void hip_check(hipError_t error, const char* what) {
   if (error != hipSuccess)
@@ -124,7 +125,7 @@ Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
       (g_.head_dim != 128U && g_.head_dim != 256U) || !g_.rotary_dim ||
       g_.rotary_dim > g_.head_dim || g_.rotary_dim % 2U ||
       !g_.kv_page_tokens || g_.kv_page_tokens % 64U || !g_.max_context ||
-      g_.draft_depth == 0U || g_.draft_depth > 7U || g_.hidden % 64U ||
+      g_.draft_depth == 0U || g_.draft_depth > kMaximumDraftDepth || g_.hidden % 64U ||
       g_.intermediate % 64U || (g_.query_heads * g_.head_dim) % 64U ||
       g_.scale_scheme > QLLM_SCALE_F16_BLOCK16 ||
       !(g_.norm_epsilon > 0.0F) || !(g_.rope_theta > 0.0F) ||
@@ -159,6 +160,9 @@ void Mi355DenseFp4Provider::release() {
   for (void* graph : graphs_)
     if (graph) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph));
   graphs_.clear();
+  for (void* graph : mtp_graphs_)
+    if (graph) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph));
+  mtp_graphs_.clear();
   if (stream_) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
   for (void* pointer : allocations_) (void)hipFree(pointer);
   allocations_.clear();
@@ -243,6 +247,10 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
               "clear proposer hidden state");
     mtp_logits_ = static_cast<float*>(device_alloc(g_.draft_vocabulary * 4U));
     mtp_argmax_ = static_cast<std::uint32_t*>(device_alloc(4U));
+    mtp_positions_ = static_cast<std::uint32_t*>(device_alloc(4U * 4U));
+    mtp_draft_tokens_ =
+        static_cast<std::uint32_t*>(device_alloc(kMaximumDraftDepth * 4U));
+    mtp_graphs_.assign(2U * (max_rows_ + 1U), nullptr);
   }
 
   // Page geometry: every page holds all target layers back to back, then the
@@ -1114,44 +1122,44 @@ er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
 
 // ---- the proposer (run_mtp / extend_mtp_rollout, :8681-8852) -----------------
 
-std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
-    DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
-    const float* previous_hidden, bool produce_logits,
-    const er::ProgramRequestContext* request, std::uint32_t sample_position,
-    std::uint32_t random_stream) {
-  if (!mtp_.ready || tokens.empty() || tokens.size() > max_rows_ ||
-      !previous_hidden || state.mtp_length + tokens.size() > g_.max_context)
-    throw std::runtime_error("invalid MTP microbatch");
-  const auto rows = static_cast<std::uint32_t>(tokens.size());
-  for (const auto token : tokens)
-    if (token >= g_.vocabulary)
-      throw std::runtime_error("MTP token is outside the vocabulary");
+// The kernels of one proposer pass over the tokens in mtp_tokens_, through the
+// draft head's argmax when `produce_logits`.  With `deferred_positions` the
+// positions come from mtp_positions_ when the kernels run and the pass ends by
+// advancing them (qllm_rollout_advance), so that a captured pass can be
+// replayed, and greedy passes chained, without the host in between.
+void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
+                                        const float* previous_hidden,
+                                        bool produce_logits,
+                                        std::uint32_t cache_position,
+                                        bool deferred_positions) {
   void* const stream = stream_;
   const auto hip_stream = static_cast<hipStream_t>(stream_);
-  const std::uint32_t cache_position = state.mtp_length;       // row 0
-  const std::uint32_t rotary_position = state.mtp_length + 1U;  // row 0
-  ensure_pages(cache_position + rows - 1U);
-  hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
-                           hipMemcpyHostToDevice, hip_stream),
-            "upload MTP token batch");
+  const std::uint32_t rotary_position = cache_position + 1U;  // row 0
   status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, mtp_tokens_,
                                         mtp_embedding_, rows, stream));
   // [RMSNorm(embedding) | RMSNorm(previous target hidden)] -> fusion projection
   const std::size_t half_bytes = std::size_t{g_.hidden} * 2U;
-  status_check(qllm_rms_norm_batch(mtp_embedding_, mtp_.embedding_norm, nullptr,
-                                   normalized_, g_.hidden, rows, g_.hidden,
-                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
-  hip_check(hipMemcpy2DAsync(mtp_fusion_input_, 2U * half_bytes, normalized_,
-                             half_bytes, half_bytes, rows,
-                             hipMemcpyDeviceToDevice, hip_stream),
-            "assemble MTP normalized embedding batch");
-  status_check(qllm_rms_norm_batch(previous_hidden, mtp_.hidden_norm, nullptr,
-                                   normalized_, g_.hidden, rows, g_.hidden,
-                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
-  hip_check(hipMemcpy2DAsync(mtp_fusion_input_ + g_.hidden, 2U * half_bytes,
-                             normalized_, half_bytes, half_bytes, rows,
-                             hipMemcpyDeviceToDevice, hip_stream),
-            "assemble MTP target hidden batch");
+  if (g_.hidden <= 16384U) {
+    status_check(qllm_rms_norm_concat_batch(
+        mtp_embedding_, mtp_.embedding_norm, previous_hidden, mtp_.hidden_norm,
+        mtp_fusion_input_, rows, g_.hidden, g_.norm_epsilon,
+        g_.zero_centered_norm, stream));
+  } else {
+    status_check(qllm_rms_norm_batch(mtp_embedding_, mtp_.embedding_norm, nullptr,
+                                     normalized_, g_.hidden, rows, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm, stream));
+    hip_check(hipMemcpy2DAsync(mtp_fusion_input_, 2U * half_bytes, normalized_,
+                               half_bytes, half_bytes, rows,
+                               hipMemcpyDeviceToDevice, hip_stream),
+              "assemble MTP normalized embedding batch");
+    status_check(qllm_rms_norm_batch(previous_hidden, mtp_.hidden_norm, nullptr,
+                                     normalized_, g_.hidden, rows, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm, stream));
+    hip_check(hipMemcpy2DAsync(mtp_fusion_input_ + g_.hidden, 2U * half_bytes,
+                               normalized_, half_bytes, half_bytes, rows,
+                               hipMemcpyDeviceToDevice, hip_stream),
+              "assemble MTP target hidden batch");
+  }
   status_check(qllm_fp4_gemm_bf16(&mtp_.fusion.descriptor, mtp_fusion_input_,
                                   std::size_t{rows} * 2U * half_bytes,
                                   mtp_hidden_, QLLM_OUT_F32, nullptr, rows,
@@ -1172,17 +1180,27 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
   status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
                                         hidden_bytes, projections, 3U, rows,
                                         stream));
-  status_check(qllm_qkv_rope_batch(
-      query_, query_stride, key_, layer.query_norm, layer.key_norm,
-      rotary_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
-      g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
-  status_check(qllm_store_kv_paged_q8_batch(
-      key_, value_, const_cast<const void* const*>(device_page_table_),
-      mtp_page_offset_, g_.kv_page_tokens, cache_position, rows, g_.kv_heads,
-      g_.head_dim, stream));
+  const auto pages = const_cast<const void* const*>(device_page_table_);
+  if (deferred_positions) {
+    status_check(qllm_qkv_rope_batch_deferred(
+        query_, query_stride, key_, layer.query_norm, layer.key_norm,
+        mtp_positions_, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
+        g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+    status_check(qllm_store_kv_paged_q8_batch_deferred(
+        key_, value_, pages, mtp_page_offset_, g_.kv_page_tokens,
+        mtp_positions_, rows, g_.kv_heads, g_.head_dim, stream));
+  } else {
+    status_check(qllm_qkv_rope_batch(
+        query_, query_stride, key_, layer.query_norm, layer.key_norm,
+        rotary_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
+        g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+    status_check(qllm_store_kv_paged_q8_batch(
+        key_, value_, pages, mtp_page_offset_, g_.kv_page_tokens,
+        cache_position, rows, g_.kv_heads, g_.head_dim, stream));
+  }
   qllm_q8_attention_launch launch{};
   launch.query = query_;
-  launch.device_pages = const_cast<const void* const*>(device_page_table_);
+  launch.device_pages = pages;
   launch.output = attention_;
   launch.partial_maxima = partial_maxima_;
   launch.partial_sums = partial_sums_;
@@ -1200,6 +1218,7 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
   launch.output_gated = g_.output_gated;
   launch.output_kind = QLLM_OUT_BF16;
   launch.stream = stream;
+  launch.device_positions = deferred_positions ? mtp_positions_ : nullptr;
   status_check(qllm_attention_paged_q8(&launch));
   status_check(qllm_fp4_gemm_bf16(
       &layer.output.descriptor, attention_,
@@ -1212,29 +1231,93 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
   status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor, &layer.up.descriptor,
                                     normalized_, hidden_bytes, activation_, rows,
                                     stream));
+  // a single-row pass leaves its hidden state where the next pass reads it
+  const bool retain_in_place = rows == 1U && produce_logits;
   status_check(qllm_fp4_gemm_bf16(
       &layer.down.descriptor, activation_,
-      std::size_t{rows} * g_.intermediate * 2U, mtp_hidden_, QLLM_OUT_F32,
+      std::size_t{rows} * g_.intermediate * 2U,
+      retain_in_place ? mtp_last_hidden_ : mtp_hidden_, QLLM_OUT_F32,
       mtp_hidden_, rows, stream));
+  if (produce_logits) {
+    // draft head: the last row, draft norm, the head's first draft_vocabulary
+    // rows
+    if (!retain_in_place)
+      hip_check(hipMemcpyAsync(
+                    mtp_last_hidden_,
+                    mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
+                    g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
+                "retain final MTP hidden state");
+    const float* final_hidden = mtp_last_hidden_;
+    status_check(qllm_rms_norm_batch(final_hidden, mtp_.draft_norm, nullptr,
+                                     normalized_, g_.hidden, 1U, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm,
+                                     stream));
+    status_check(qllm_fp4_gemm_bf16(&mtp_.head_prefix, normalized_,
+                                    std::size_t{g_.hidden} * 2U, mtp_logits_,
+                                    QLLM_OUT_F32, nullptr, 1U, stream));
+    status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U,
+                                   mtp_argmax_, select_workspace_,
+                                   select_workspace_bytes_, stream));
+  }
+  if (deferred_positions)
+    status_check(qllm_rollout_advance(mtp_argmax_, mtp_tokens_,
+                                      mtp_draft_tokens_, g_.draft_depth, rows,
+                                      mtp_positions_, stream));
+}
+
+// Replays the proposer pass captured for (rows, source of the previous hidden
+// state); the first use captures it.  `chained` passes read the proposer's own
+// last hidden state, the others the target's.
+void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained) {
+  const auto stream = static_cast<hipStream_t>(stream_);
+  void*& slot = mtp_graphs_.at(2U * rows + (chained ? 1U : 0U));
+  if (!slot) {
+    hip_check(hipStreamSynchronize(stream), "drain stream before capture");
+    hipGraph_t graph{};
+    hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal),
+              "begin proposer capture");
+    try {
+      enqueue_mtp(rows, chained ? mtp_last_hidden_ : hidden_, true, 0U, true);
+    } catch (...) {
+      (void)hipStreamEndCapture(stream, &graph);
+      if (graph) (void)hipGraphDestroy(graph);
+      throw;
+    }
+    hip_check(hipStreamEndCapture(stream, &graph), "end proposer capture");
+    hipGraphExec_t exec{};
+    const auto status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    hip_check(status, "instantiate proposer graph");
+    slot = exec;
+  }
+  hip_check(hipGraphLaunch(static_cast<hipGraphExec_t>(slot), stream),
+            "launch proposer graph");
+}
+
+std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
+    DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
+    const float* previous_hidden, bool produce_logits,
+    const er::ProgramRequestContext* request, std::uint32_t sample_position,
+    std::uint32_t random_stream) {
+  if (!mtp_.ready || tokens.empty() || tokens.size() > max_rows_ ||
+      !previous_hidden || state.mtp_length + tokens.size() > g_.max_context)
+    throw std::runtime_error("invalid MTP microbatch");
+  const auto rows = static_cast<std::uint32_t>(tokens.size());
+  for (const auto token : tokens)
+    if (token >= g_.vocabulary)
+      throw std::runtime_error("MTP token is outside the vocabulary");
+  const auto hip_stream = static_cast<hipStream_t>(stream_);
+  const std::uint32_t cache_position = state.mtp_length;  // row 0
+  ensure_pages(cache_position + rows - 1U);
+  hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
+                           hipMemcpyHostToDevice, hip_stream),
+            "upload MTP token batch");
+  enqueue_mtp(rows, previous_hidden, produce_logits, cache_position, false);
   state.mtp_length += rows;
   ++mtp_passes_;
   mtp_rows_ += rows;
   if (!produce_logits) return std::nullopt;
 
-  // draft head: the last row, draft norm, the head's first draft_vocabulary rows
-  const float* final_hidden = mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden;
-  hip_check(hipMemcpyAsync(mtp_last_hidden_, final_hidden, g_.hidden * 4U,
-                           hipMemcpyDeviceToDevice, hip_stream),
-            "retain final MTP hidden state");
-  status_check(qllm_rms_norm_batch(final_hidden, mtp_.draft_norm, nullptr,
-                                   normalized_, g_.hidden, 1U, g_.hidden,
-                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
-  status_check(qllm_fp4_gemm_bf16(&mtp_.head_prefix, normalized_,
-                                  std::size_t{g_.hidden} * 2U, mtp_logits_,
-                                  QLLM_OUT_F32, nullptr, 1U, stream));
-  status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U,
-                                 mtp_argmax_, select_workspace_,
-                                 select_workspace_bytes_, stream));
   DraftPrediction result;
   if (request) {
     result.distribution = distribution_from_logits(
@@ -1251,6 +1334,92 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
     result.distribution.entries.push_back({result.token, 1.0});
   }
   return result;
+}
+
+// run_mtp over the accepted tokens followed by extend_mtp_rollout, as captured
+// graphs: the first pass pairs `tokens` with the target's hidden rows, every
+// further pass feeds the proposer its own draft and hidden state.  A greedy
+// request runs all passes back to back and reads the drafts once; a sampled
+// one returns to the host after each pass for its distribution.  Positions,
+// sampling positions and streams are those of the two functions it replaces.
+void Mi355DenseFp4Provider::propose_with_graphs(
+    DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
+    const er::ProgramRequestContext& request, std::uint32_t context_limit) {
+  if (!mtp_.ready || tokens.empty() || tokens.size() > max_rows_ ||
+      context_limit > g_.max_context ||
+      state.mtp_length + tokens.size() + 1U >= context_limit)
+    throw std::runtime_error("invalid MTP proposal");
+  for (const auto token : tokens)
+    if (token >= g_.vocabulary)
+      throw std::runtime_error("MTP token is outside the vocabulary");
+  const auto rows = static_cast<std::uint32_t>(tokens.size());
+  const auto stream = static_cast<hipStream_t>(stream_);
+  const std::uint32_t first_position = state.mtp_length;
+  const std::uint32_t committed_length = first_position + rows;
+  // drafts: the root, then as many as depth and context allow
+  // (extend_mtp_rollout's loop, :8794-8852)
+  std::uint32_t drafts = 1U;
+  while (drafts < g_.draft_depth &&
+         committed_length + (drafts - 1U) + 2U < context_limit)
+    ++drafts;
+  // rollout pass i writes the proposer's cache at committed_length + i - 1
+  ensure_pages(committed_length + drafts - 2U);
+  const std::uint32_t positions[4] = {first_position, first_position + 1U,
+                                      first_position + 1U, 0U};
+  hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
+                           hipMemcpyHostToDevice, stream),
+            "upload MTP token batch");
+  hip_check(hipMemcpyAsync(mtp_positions_, positions, sizeof(positions),
+                           hipMemcpyHostToDevice, stream),
+            "upload MTP positions");
+  state.draft_predictions.clear();
+  state.draft_predictions.reserve(drafts);
+  const bool greedy =
+      request_parameter(request, "sampling_temperature_ppm") == 0U;
+  if (greedy) {
+    launch_mtp_graph(rows, false);
+    for (std::uint32_t pass = 1; pass < drafts; ++pass)
+      launch_mtp_graph(1U, true);
+    std::uint32_t chosen[kMaximumDraftDepth]{};
+    hip_check(hipMemcpyAsync(chosen, mtp_draft_tokens_, drafts * 4U,
+                             hipMemcpyDeviceToHost, stream),
+              "copy MTP draft tokens");
+    hip_check(hipStreamSynchronize(stream), "copy MTP draft tokens");
+    for (std::uint32_t depth = 0; depth < drafts; ++depth) {
+      DraftPrediction prediction;
+      prediction.token = chosen[depth];
+      prediction.distribution.entries.push_back({chosen[depth], 1.0});
+      state.draft_predictions.push_back(std::move(prediction));
+    }
+  } else {
+    const auto seed = request_parameter(request, "sampling_seed");
+    for (std::uint32_t depth = 0; depth < drafts; ++depth) {
+      if (depth) {
+        // the device chained its own argmax; the sampled draft replaces it
+        const std::uint32_t token = state.draft_predictions.back().token;
+        hip_check(hipMemcpyAsync(mtp_tokens_, &token, sizeof(token),
+                                 hipMemcpyHostToDevice, stream),
+                  "upload sampled MTP draft");
+        hip_check(hipStreamSynchronize(stream), "upload sampled MTP draft");
+      }
+      launch_mtp_graph(depth ? 1U : rows, depth != 0U);
+      DraftPrediction prediction;
+      prediction.distribution = distribution_from_logits(
+          mtp_logits_, g_.draft_vocabulary, mtp_argmax_, request);
+      prediction.token = er::sample_distribution(
+          prediction.distribution,
+          er::counter_uniform(seed, committed_length + (depth ? depth - 1U : 0U),
+                              1U + depth));
+      if (!(prediction.distribution.probability(prediction.token) > 0.0))
+        throw std::runtime_error("invalid MTP rollout root");
+      state.draft_predictions.push_back(std::move(prediction));
+    }
+  }
+  mtp_passes_ += drafts;
+  mtp_rows_ += rows + drafts - 1U;
+  state.draft_valid = true;
+  // speculative rows of the proposer's cache are overwritten by the next pass
+  state.mtp_length = committed_length;
 }
 
 void Mi355DenseFp4Provider::extend_mtp_rollout(
@@ -1361,13 +1530,19 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       state->mtp_length = invocation.position;
       state->draft_valid = false;
       state->draft_predictions.clear();
-      auto first = run_mtp(*state, mtp_tokens, hidden_, future_exact,
-                           future_exact ? &invocation.request : nullptr,
-                           invocation.position + positions_advanced, 1U);
-      if (future_exact) {
-        if (!first) throw std::runtime_error("next MTP rollout produced no root");
-        extend_mtp_rollout(*state, invocation.request, std::move(*first),
-                           invocation.context_limit);
+      if (future_exact && use_graphs_) {
+        propose_with_graphs(*state, mtp_tokens, invocation.request,
+                            invocation.context_limit);
+      } else {
+        auto first = run_mtp(*state, mtp_tokens, hidden_, future_exact,
+                             future_exact ? &invocation.request : nullptr,
+                             invocation.position + positions_advanced, 1U);
+        if (future_exact) {
+          if (!first)
+            throw std::runtime_error("next MTP rollout produced no root");
+          extend_mtp_rollout(*state, invocation.request, std::move(*first),
+                             invocation.context_limit);
+        }
       }
     } else {
       state->mtp_length = invocation.position + positions_advanced;

@@ -215,6 +215,15 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       const float* previous_hidden, bool produce_logits,
       const er::ProgramRequestContext* request, std::uint32_t sample_position,
       std::uint32_t random_stream);
+  void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
+                   bool produce_logits, std::uint32_t cache_position,
+                   bool deferred_positions);
+  void launch_mtp_graph(std::uint32_t rows, bool chained);
+  // run_mtp + extend_mtp_rollout replayed from captured graphs
+  void propose_with_graphs(DenseFp4RequestState& state,
+                           std::span<const std::uint32_t> tokens,
+                           const er::ProgramRequestContext& request,
+                           std::uint32_t context_limit);
   // extend_mtp_rollout, dense_fp4_provider.cpp:8794-8852
   void extend_mtp_rollout(DenseFp4RequestState& state,
                           const er::ProgramRequestContext& request,
@@ -276,6 +285,9 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* mtp_last_hidden_{};
   float* mtp_logits_{};
   std::uint32_t* mtp_argmax_{};
+  std::uint32_t* mtp_positions_{};      // cache, rotary, context, draft slot
+  std::uint32_t* mtp_draft_tokens_{};
+  std::vector<void*> mtp_graphs_;       // hipGraphExec_t at 2*rows + chained
 
   std::uint32_t* positions_{};   // device: cache, rotary, first-context
   std::vector<void*> graphs_;    // hipGraphExec_t per row count

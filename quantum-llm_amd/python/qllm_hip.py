@@ -74,7 +74,8 @@ class Q8AttentionLaunch(Structure):
                 ("kv_heads", c_uint32), ("head_dim", c_uint32),
                 ("split_tokens", c_uint32), ("maximum_splits", c_uint32),
                 ("query_stride", c_uint32), ("output_gated", c_int32),
-                ("output_kind", c_uint32), ("stream", c_void_p)]
+                ("output_kind", c_uint32), ("stream", c_void_p),
+                ("device_positions", c_void_p)]
 
 
 # name -> (restype, argtypes); every symbol include/qllm_kernels.h declares.
@@ -92,12 +93,14 @@ SIGNATURES = {
     "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
     "qllm_fp4_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_uint32, c_void_p]),
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_silu_product": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_q4h_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_qkv_rope_cache_paged_q4h_batch": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
     "qllm_qkv_rope_cache_paged_q4h_batch_deferred": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
     "qllm_qkv_rope_batch": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
+    "qllm_qkv_rope_batch_deferred": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
     "qllm_store_kv_paged_q4h_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_quantize_gqa_queries_q8": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_q4h": (c_int32, [POINTER(Q4hAttentionLaunch)]),
@@ -105,6 +108,8 @@ SIGNATURES = {
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),
     "qllm_q8_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_store_kv_paged_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
+    "qllm_store_kv_paged_q8_batch_deferred": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
+    "qllm_rollout_advance": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "qllm_attention_paged_q8": (c_int32, [POINTER(Q8AttentionLaunch)]),
     "qllm_argmax_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "qllm_argmax_batch": (c_int32, [c_void_p, c_uint32, c_uint32, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -155,6 +155,39 @@ def test_decode_cycle_runs_on_its_own_drafts(device, temperature, top_k):
     assert streams[0] == streams[1]
 
 
+@pytest.mark.parametrize("temperature,top_k", [(0, 0), (800000, 20)])
+def test_captured_proposer_passes_equal_the_eager_ones(device, monkeypatch,
+                                                       temperature, top_k):
+    """The proposer replayed from captured graphs (positions read on the device,
+    greedy passes chained without the host) against the same passes launched
+    one kernel at a time: tokens, drafts, hidden state and logits are equal."""
+    runs = []
+    for eager in ("1", "0"):
+        monkeypatch.setenv("QLLM_PROVIDER_EAGER", eager)
+        rng, model, provider = make("reference", 41, max_context=256)
+        V = model.vocabulary
+        provider.run_target(rng.integers(0, V, 5).astype(np.uint32), 0)
+        position, token, limit = 5, 11, 40
+        provider.begin_request(temperature_ppm=temperature, top_p_ppm=950000,
+                               top_k=top_k, seed=5)
+        provider.synchronize(token, position)
+        record = []
+        while provider.drafts():
+            drafts = provider.drafts()
+            emitted, token, advanced = provider.verify(token, position, limit)
+            position += advanced
+            hidden, logits = provider.mtp_state()
+            record.append((drafts, emitted, token, hidden.copy(), logits.copy()))
+        assert position >= limit - 2
+        runs.append(record)
+        provider.close()
+    assert len(runs[0]) == len(runs[1]) >= 7
+    for eager_step, graph_step in zip(*runs):
+        assert eager_step[:3] == graph_step[:3]
+        assert np.array_equal(eager_step[3], graph_step[3])
+        assert np.array_equal(eager_step[4], graph_step[4])
+
+
 def test_rollout_stops_at_the_context_limit(device):
     rng, model, provider = make("baseline", 37, max_context=64)
     V = model.vocabulary

@@ -11,18 +11,21 @@ import synth
 pytestmark = pytest.mark.gpu
 
 
+@pytest.mark.parametrize("columns", [256, 252, 5120])
 @pytest.mark.parametrize("scheme", [0, 1])
-def test_embedding_is_exact(device, scheme):
+def test_embedding_is_exact(device, scheme, columns):
+    # 252 columns in 256 padded ones takes the one-column-per-thread kernel,
+    # the multiples of eight the eight-columns-per-thread one.
     rng = np.random.default_rng(scheme)
-    V, H = 300, 256
+    V, H = 300, (columns + 31) // 32 * 32
     codes, scales = synth.fp4_matrix(rng, V, H, scheme)
     tokens = np.array([0, 5, 299, 17, 5], dtype=np.uint32)
-    want = ol.fp4_embedding(codes, scales, scheme, H, H, tokens)
+    want = ol.fp4_embedding(codes, scales, scheme, columns, H, tokens)
     tensors = [gu.device_tensor(x, device) for x in (codes, scales, tokens)]
-    out = torch.zeros((5, H), device=device)
+    out = torch.zeros((5, columns), device=device)
     qh.call("qllm_fp4_embedding_batch",
-            qh.fp4_matrix(tensors[0], tensors[1], V, H, H, scheme), qh.ptr(tensors[2]),
-            qh.ptr(out), 5, None)
+            qh.fp4_matrix(tensors[0], tensors[1], V, columns, H, scheme),
+            qh.ptr(tensors[2]), qh.ptr(out), 5, None)
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy(), want)
 
@@ -42,6 +45,37 @@ def test_rms_norm(device, zero_centered):
     assert np.abs(out_f32.cpu().numpy() - want).max() < 2e-5   # reference: 2e-5
     assert np.array_equal(out_bf16.float().cpu().numpy(),
                           ol.bf16_round(out_f32.cpu().numpy()))
+
+
+@pytest.mark.parametrize("elements", [5120, 256])
+def test_rms_norm_concat_is_two_norms_side_by_side(device, elements):
+    """[RMSNorm(a) | RMSNorm(b)] in one launch: each half within the reference's
+    2e-5 of the oracle before the bf16 rounding, and bit-equal to the two-call
+    form it stands in for."""
+    rng = np.random.default_rng(7)
+    a = (rng.standard_normal((5, elements)) * 2).astype(np.float32)
+    b = rng.standard_normal((5, elements)).astype(np.float32)
+    wa = (1 + 0.1 * rng.standard_normal(elements)).astype(np.float32)
+    wb = (0.1 * rng.standard_normal(elements)).astype(np.float32)
+    d = [gu.device_tensor(x, device) for x in (a, wa, b, wb)]
+    out = torch.zeros((5, 2 * elements), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_concat_batch", qh.ptr(d[0]), qh.ptr(d[1]), qh.ptr(d[2]),
+            qh.ptr(d[3]), qh.ptr(out), 5, elements, 1e-6, 1, None)
+    halves = []
+    for x, w in ((d[0], d[1]), (d[2], d[3])):
+        single = torch.zeros((5, elements), dtype=torch.bfloat16, device=device)
+        qh.call("qllm_rms_norm_batch", qh.ptr(x), qh.ptr(w), None, qh.ptr(single),
+                elements, 5, elements, 1e-6, 1, None)
+        halves.append(single)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.array_equal(got[:, :elements], halves[0].float().cpu().numpy())
+    assert np.array_equal(got[:, elements:], halves[1].float().cpu().numpy())
+    for half, (x, w) in enumerate(((a, wa), (b, wb))):
+        want = ol.rms_norm_rows(x, w, 1e-6, True)
+        piece = got[:, half * elements:(half + 1) * elements]
+        # bf16 keeps 8 significant bits: half an ulp is 2^-9 of the value
+        assert (np.abs(piece - want) <= np.abs(want) * 2.0 ** -8 + 2e-5).all()
 
 
 def test_add_silu_and_bf16_convert(device):
@@ -71,12 +105,14 @@ def test_add_silu_and_bf16_convert(device):
     assert np.array_equal(host[:, :100], ol.bf16_round(x)) and not host[:, 100:].any()
 
 
-def test_argmax_ties_nan_and_large_vocabulary(device):
+@pytest.mark.parametrize("V", [151936, 151937, 65536])
+def test_argmax_ties_nan_and_large_vocabulary(device, V):
+    # an odd row length leaves every second row off the 16-byte alignment the
+    # vector loads need, so both load paths and the ragged last chunk are hit
     nan = float("nan")
     rng = np.random.default_rng(4)
-    V = 151936
     logits = rng.standard_normal((5, V)).astype(np.float32)
-    logits[0, 77] = logits[0, 140000] = 9.0          # tie -> lower index
+    logits[0, 77] = logits[0, V - 1000] = 9.0        # tie -> lower index
     logits[1, :] = nan
     logits[1, 5000] = -3.0                           # NaN never wins
     logits[2, :] = -np.inf                           # all -inf -> index 0
