@@ -57,8 +57,23 @@ typedef struct qllm_dense_geometry {
 
 const char* qllm_provider_last_error(void);
 
-/* make_<name>_callable_provider (dense_fp4_provider.cpp:11402-11412). */
+/* The provider for a geometry given by the host; tensors follow through
+ * qllm_provider_stage_tensor / qllm_provider_prepare. */
 qllm_provider* qllm_provider_create(const qllm_dense_geometry* geometry);
+/* make_<name>_callable_provider(artifact_root, max_context, ..., kv_page_tokens,
+ * kv_cache_dtype, ..., mtp_draft_depth) (dense_fp4_provider.cpp:11402-11470)
+ * followed by the executor's start-up binding (program_executor.cpp:1725-1826):
+ * loads and authenticates the Expert Pack v1 directory, takes the geometry
+ * from its model program, uploads every tensor the program's operations name
+ * and prepares them, the exact-decode program included.  max_context 0 = the
+ * artifact's; kv_page_tokens 0 = 256; kv_cache_dtype NULL or "artifact" =
+ * "q4-f16-per-head", or "fp16"; mtp_draft_depth 0 = the artifact's.  NULL on
+ * failure, with the reason in qllm_provider_last_error(). */
+qllm_provider* qllm_provider_create_from_artifact(const char* artifact_root,
+                                                  uint32_t max_context,
+                                                  uint32_t kv_page_tokens,
+                                                  const char* kv_cache_dtype,
+                                                  uint32_t mtp_draft_depth);
 void qllm_provider_destroy(qllm_provider* provider);
 
 /* Capability table of make_<name>_provider(): writes up to `capacity`
@@ -214,6 +229,52 @@ int32_t qllm_sampling_rejection(uint32_t proposal,
  * index), top 53 bits. */
 double qllm_sampling_counter_uniform(uint64_t seed, uint32_t position,
                                      uint32_t stream, uint32_t index);
+
+/* ---- artifact reader ----------------------------------------------------------
+ * Host only; none of these calls touches a device.  Text results are written
+ * NUL-terminated into `dump` (truncated to `capacity`), their full length
+ * into `*dump_bytes`; on failure the status is the reference's ErrorCode and
+ * the message is in qllm_provider_last_error(). */
+
+/* sha256() of runtime/include/expert/runtime/sha256.hpp:26. */
+int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest32);
+
+/* parse_model_descriptor_artifact (runtime/include/expert/runtime/
+ * model_descriptor.hpp:276-281; runtime/src/model_descriptor.cpp:527-723):
+ * parses and validates the text of runtime-model.tsv.  The result is the
+ * descriptor in a canonical line form: the program's own records with maps in
+ * key order, component namespaces resolved against namespace_base, and the
+ * content hash. */
+int32_t qllm_model_descriptor_parse(const char* text, size_t text_bytes,
+                                    const uint8_t* content_sha256,
+                                    uint64_t namespace_base, char* dump,
+                                    size_t capacity, size_t* dump_bytes);
+/* load_model_descriptor_artifact (model_descriptor.hpp:282-285): the file
+ * must have expected_bytes bytes and the expected SHA-256. */
+int32_t qllm_model_descriptor_load(const char* path, uint64_t expected_bytes,
+                                   const uint8_t* expected_sha256,
+                                   const uint8_t* content_sha256,
+                                   uint64_t namespace_base, char* dump,
+                                   size_t capacity, size_t* dump_bytes);
+
+/* ModelArtifact::load (+ configure_mtp_draft_depth when mtp_draft_depth != 0)
+ * and, with map_tensors, MappedModelTensorStore::create
+ * (runtime/include/expert/runtime/model_artifact.hpp:46-92,
+ * model_tensor_store.hpp:15-34). */
+typedef struct qllm_artifact qllm_artifact;
+int32_t qllm_artifact_open(const char* root, uint32_t mtp_draft_depth,
+                           int32_t map_tensors, qllm_artifact** artifact);
+void qllm_artifact_close(qllm_artifact* artifact);
+/* "pack" and "tensor" lines of the index, then the model descriptor. */
+int32_t qllm_artifact_dump(const qllm_artifact* artifact, char* dump,
+                           size_t capacity, size_t* dump_bytes);
+/* IModelTensorStore::resolve (program_executor.hpp:57-62): the mapped record
+ * of a dense tensor; with check_header the record's 256-byte header is
+ * checked against the index entry first (compiler/expert_pack/validate.py:
+ * 148-325). */
+int32_t qllm_artifact_tensor(qllm_artifact* artifact, const char* name,
+                             int32_t check_header, const void** record,
+                             uint64_t* record_bytes);
 
 #ifdef __cplusplus
 }

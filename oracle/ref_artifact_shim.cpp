@@ -1,0 +1,121 @@
+// C-callable shim over the reference's own artifact reader.  TEST
+// INFRASTRUCTURE ONLY.  Compiled together with the reference sources
+// runtime/src/{model_descriptor,model_artifact,model_tensor_store,sha256,
+// expert_catalog,expert_record}.cpp and core/src/json.cpp, read where they lie
+// in the reference tree, into oracle/_ref/libqllm_ref_artifact.so.  The shim
+// adds no logic: it calls the reference's functions and prints their results
+// with the same writer (descriptor_dump.hpp) the product uses on its own types.
+#include "expert/runtime/model_artifact.hpp"
+#include "expert/runtime/model_descriptor.hpp"
+#include "expert/runtime/model_tensor_store.hpp"
+#include "expert/runtime/sha256.hpp"
+
+#include "descriptor_dump.hpp"
+
+#include <algorithm>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <string>
+
+namespace er = expert::runtime;
+
+namespace {
+
+void copy_text(const std::string& text, char* buffer, std::size_t capacity,
+               std::size_t* bytes) {
+  if (bytes) *bytes = text.size();
+  if (buffer && capacity) {
+    const std::size_t count = std::min(text.size(), capacity - 1U);
+    std::memcpy(buffer, text.data(), count);
+    buffer[count] = '\0';
+  }
+}
+
+// status code; the message goes where the dump would have gone
+int report(const er::Status& status, char* buffer, std::size_t capacity,
+           std::size_t* bytes) {
+  copy_text(std::string(status.message()), buffer, capacity, bytes);
+  return static_cast<int>(status.code());
+}
+
+er::Sha256Digest digest_of(const std::uint8_t* bytes) {
+  er::Sha256Digest digest{};
+  if (bytes) std::memcpy(digest.data(), bytes, digest.size());
+  return digest;
+}
+
+struct Artifact {
+  er::ModelArtifact artifact;
+  er::MappedModelTensorStore store;
+};
+
+}  // namespace
+
+extern "C" {
+
+void qref_sha256(const void* data, std::size_t bytes, std::uint8_t* digest) {
+  const auto result = er::sha256({static_cast<const std::byte*>(data), bytes});
+  std::memcpy(digest, result.data(), result.size());
+}
+
+int qref_model_descriptor_parse(const char* text, std::size_t text_bytes,
+                                const std::uint8_t* content_sha256,
+                                std::uint64_t namespace_base, char* dump,
+                                std::size_t capacity, std::size_t* dump_bytes) {
+  const auto parsed = er::parse_model_descriptor_artifact(
+      {text, text_bytes}, digest_of(content_sha256), namespace_base);
+  if (!parsed.status.ok()) return report(parsed.status, dump, capacity, dump_bytes);
+  copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
+            dump_bytes);
+  return 0;
+}
+
+int qref_model_descriptor_load(const char* path, std::uint64_t expected_bytes,
+                               const std::uint8_t* expected_sha256,
+                               const std::uint8_t* content_sha256,
+                               std::uint64_t namespace_base, char* dump,
+                               std::size_t capacity, std::size_t* dump_bytes) {
+  const auto parsed = er::load_model_descriptor_artifact(
+      path, expected_bytes, digest_of(expected_sha256), digest_of(content_sha256),
+      namespace_base);
+  if (!parsed.status.ok()) return report(parsed.status, dump, capacity, dump_bytes);
+  copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
+            dump_bytes);
+  return 0;
+}
+
+int qref_artifact_open(const char* root, std::uint32_t mtp_draft_depth,
+                       int map_tensors, void** out, char* message,
+                       std::size_t capacity) {
+  *out = nullptr;
+  auto handle = std::make_unique<Artifact>();
+  auto status = er::ModelArtifact::load(root, handle->artifact);
+  if (status.ok() && mtp_draft_depth)
+    status = handle->artifact.configure_mtp_draft_depth(mtp_draft_depth);
+  if (status.ok() && map_tensors)
+    status = er::MappedModelTensorStore::create(handle->artifact, handle->store);
+  if (!status.ok()) return report(status, message, capacity, nullptr);
+  *out = handle.release();
+  return 0;
+}
+
+void qref_artifact_close(void* artifact) { delete static_cast<Artifact*>(artifact); }
+
+void qref_artifact_dump(const void* artifact, char* dump, std::size_t capacity,
+                        std::size_t* dump_bytes) {
+  copy_text(qllm::dump::model_artifact(static_cast<const Artifact*>(artifact)->artifact),
+            dump, capacity, dump_bytes);
+}
+
+int qref_artifact_tensor(void* artifact, const char* name, const void** record,
+                         std::uint64_t* record_bytes, char* message,
+                         std::size_t capacity) {
+  const auto resolved = static_cast<Artifact*>(artifact)->store.resolve(name);
+  if (!resolved.status.ok()) return report(resolved.status, message, capacity, nullptr);
+  *record = resolved.tensor->value.data;
+  *record_bytes = resolved.tensor->value.bytes;
+  return 0;
+}
+
+}  // extern "C"

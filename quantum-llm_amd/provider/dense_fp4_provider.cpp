@@ -64,6 +64,17 @@ const er::ImmutableModelTensor* optional_tensor(
   return nullptr;
 }
 
+// The role the artifact compiler binds (compiler/expert_pack/adapters.py:
+// 1422-1602: "weight", "input_norm", "norm"), or the longer name that hosts
+// without an artifact use for the same tensor.
+const er::ImmutableModelTensor& tensor_for_either(
+    std::span<const er::PreparedTensorBinding> tensors, std::string_view role,
+    std::string_view other_role) {
+  if (const auto* tensor = optional_tensor(tensors, role)) return *tensor;
+  if (const auto* tensor = optional_tensor(tensors, other_role)) return *tensor;
+  throw std::runtime_error("tensor role is not bound: " + std::string(role));
+}
+
 class PreparedMarker final : public er::IPreparedOperation {
  public:
   explicit PreparedMarker(std::string capability)
@@ -93,8 +104,8 @@ er::Status validate_parameters(
 struct Mi355DenseFp4Provider::PreparedOp {};
 
 er::WorkerProviderDefinition make_mi355_dense_fp4_provider() {
-  const auto validator = [](const auto& parameters) {
-    return validate_parameters(parameters);
+  const auto validator = [](const er::ModelDescriptor& model) {
+    return validate_dense_fp4_descriptor(model);
   };
   // The capability strings the dense Qwen-style program requires
   // (dense_fp4_provider.cpp:996-1052; emitted by
@@ -461,8 +472,8 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
         throw std::runtime_error(std::string("tensor shape mismatch: ") + role);
     };
     if (capability.starts_with("embedding.lookup.")) {
-      embedding_ = upload_matrix(tensor_for(context.tensors, "token_embedding"),
-                                 false);
+      embedding_ = upload_matrix(
+          tensor_for_either(context.tensors, "weight", "token_embedding"), false);
       require_shape(embedding_, g_.vocabulary, g_.hidden, "token_embedding");
       embedding_ready_ = true;
     } else if (capability.starts_with("block.full-attention.")) {
@@ -503,7 +514,8 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
         throw std::runtime_error("more FFN blocks than layers");
       auto& layer = layers_[ffn_ops_];
       layer.post_attention_norm = upload_f32(
-          tensor_for(context.tensors, "post_attention_norm"), g_.hidden);
+          tensor_for_either(context.tensors, "input_norm", "post_attention_norm"),
+          g_.hidden);
       layer.gate =
           upload_matrix(tensor_for(context.tensors, "gate_projection"), true);
       layer.up =
@@ -515,9 +527,10 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
       require_shape(layer.down, g_.hidden, g_.intermediate, "down_projection");
       ++ffn_ops_;
     } else if (capability.starts_with("head.rmsnorm.token-select.")) {
-      final_norm_ =
-          upload_f32(tensor_for(context.tensors, "hidden_norm"), g_.hidden);
-      head_ = upload_matrix(tensor_for(context.tensors, "output_head"), true);
+      final_norm_ = upload_f32(
+          tensor_for_either(context.tensors, "norm", "hidden_norm"), g_.hidden);
+      head_ = upload_matrix(
+          tensor_for_either(context.tensors, "weight", "output_head"), true);
       require_shape(head_, g_.vocabulary, g_.hidden, "output_head");
       head_ready_ = true;
     } else {
@@ -525,7 +538,6 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
                "capability is not provided: " + capability},
               {}};
     }
-    (void)optional_tensor;
     return {er::Status::success(),
             std::make_shared<PreparedMarker>(capability)};
   } catch (const std::exception& error) {

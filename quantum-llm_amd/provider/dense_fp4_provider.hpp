@@ -57,6 +57,11 @@ struct DenseGeometry final {
   std::uint32_t draft_vocabulary{0};
 };
 
+// Defined with the artifact factory: the descriptor check behind every
+// capability (validate_dense_fp4_descriptor, dense_fp4_provider.cpp:804-994).
+[[nodiscard]] er::Status validate_dense_fp4_descriptor(
+    const er::ModelDescriptor& model);
+
 struct DraftPrediction final {
   std::uint32_t token{};
   er::SamplingDistribution distribution;

@@ -1,6 +1,7 @@
 // extern "C" surface of the provider (include/qllm_provider.h).
 #include "qllm_provider.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstring>
 #include <memory>
@@ -10,12 +11,17 @@
 
 #include <hip/hip_runtime.h>
 
+#include "artifact_provider.hpp"
 #include "dense_fp4_provider.hpp"
+#include "descriptor_dump.hpp"
 
 namespace er = expert::runtime;
 
 struct qllm_provider {
-  std::unique_ptr<qllm::Mi355DenseFp4Provider> provider;
+  std::shared_ptr<qllm::Mi355DenseFp4Provider> provider;
+  // set when the provider was created from an artifact directory
+  std::shared_ptr<er::ModelArtifact> artifact;
+  std::shared_ptr<er::IModelTensorStore> tensor_store;
   std::vector<er::PreparedTensorBinding> staged;
   std::vector<std::shared_ptr<const er::IPreparedOperation>> operations;
   std::shared_ptr<const er::IPreparedOperation> exact;
@@ -72,7 +78,39 @@ extern "C" qllm_provider* qllm_provider_create(
     g.mtp_layers = geometry->mtp_layers;
     g.draft_vocabulary = geometry->draft_vocabulary;
     auto handle = std::make_unique<qllm_provider>();
-    handle->provider = std::make_unique<qllm::Mi355DenseFp4Provider>(g);
+    handle->provider = std::make_shared<qllm::Mi355DenseFp4Provider>(g);
+    return handle.release();
+  } catch (const std::exception& error) {
+    fail(QLLM_INTERNAL, error.what());
+    return nullptr;
+  }
+}
+
+extern "C" qllm_provider* qllm_provider_create_from_artifact(
+    const char* artifact_root, uint32_t max_context, uint32_t kv_page_tokens,
+    const char* kv_cache_dtype, uint32_t mtp_draft_depth) {
+  if (!artifact_root) {
+    fail(QLLM_INVALID_ARGUMENT, "artifact root is null");
+    return nullptr;
+  }
+  try {
+    qllm::ArtifactProviderOptions options;
+    options.max_context = max_context;
+    if (kv_page_tokens) options.kv_page_tokens = kv_page_tokens;
+    if (kv_cache_dtype) options.kv_cache_dtype = kv_cache_dtype;
+    options.mtp_draft_depth = mtp_draft_depth;
+    auto created =
+        qllm::make_mi355_dense_fp4_callable_provider(artifact_root, options);
+    if (!created.status.ok()) {
+      from_status(created.status);
+      return nullptr;
+    }
+    auto handle = std::make_unique<qllm_provider>();
+    handle->provider = std::move(created.module.implementation);
+    handle->artifact = std::move(created.module.artifact);
+    handle->tensor_store = std::move(created.module.tensor_store);
+    handle->operations = std::move(created.module.operations);
+    handle->exact = std::move(created.module.exact_decode);
     return handle.release();
   } catch (const std::exception& error) {
     fail(QLLM_INTERNAL, error.what());
@@ -493,4 +531,128 @@ extern "C" double qllm_sampling_counter_uniform(uint64_t seed,
                                                 uint32_t stream,
                                                 uint32_t index) {
   return er::counter_uniform(seed, position, stream, index);
+}
+
+
+// ---- artifact reader ----------------------------------------------------------
+
+struct qllm_artifact {
+  er::ModelArtifact artifact;
+  er::MappedModelTensorStore store;
+};
+
+namespace {
+
+int32_t copy_text(const std::string& text, char* buffer, size_t capacity,
+                  size_t* bytes) {
+  if (bytes) *bytes = text.size();
+  if (buffer && capacity) {
+    const size_t count = std::min(text.size(), capacity - 1U);
+    std::memcpy(buffer, text.data(), count);
+    buffer[count] = '\0';
+  }
+  return QLLM_OK;
+}
+
+er::Sha256Digest digest_of(const uint8_t* bytes) {
+  er::Sha256Digest digest{};
+  if (bytes) std::memcpy(digest.data(), bytes, digest.size());
+  return digest;
+}
+
+}  // namespace
+
+extern "C" int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest) {
+  if ((!data && bytes) || !digest)
+    return fail(QLLM_INVALID_ARGUMENT, "SHA-256 arguments are invalid");
+  const auto result =
+      er::sha256({static_cast<const std::byte*>(data), bytes});
+  std::memcpy(digest, result.data(), result.size());
+  return QLLM_OK;
+}
+
+extern "C" int32_t qllm_model_descriptor_parse(
+    const char* text, size_t text_bytes, const uint8_t* content_sha256,
+    uint64_t namespace_base, char* dump, size_t capacity, size_t* dump_bytes) {
+  if (!text && text_bytes)
+    return fail(QLLM_INVALID_ARGUMENT, "model program text is null");
+  const auto parsed = er::parse_model_descriptor_artifact(
+      {text, text_bytes}, digest_of(content_sha256), namespace_base);
+  if (!parsed.status.ok()) return from_status(parsed.status);
+  return copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
+                   dump_bytes);
+}
+
+extern "C" int32_t qllm_model_descriptor_load(
+    const char* path, uint64_t expected_bytes, const uint8_t* expected_sha256,
+    const uint8_t* content_sha256, uint64_t namespace_base, char* dump,
+    size_t capacity, size_t* dump_bytes) {
+  if (!path) return fail(QLLM_INVALID_ARGUMENT, "model program path is null");
+  const auto parsed = er::load_model_descriptor_artifact(
+      path, expected_bytes, digest_of(expected_sha256), digest_of(content_sha256),
+      namespace_base);
+  if (!parsed.status.ok()) return from_status(parsed.status);
+  return copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
+                   dump_bytes);
+}
+
+extern "C" int32_t qllm_artifact_open(const char* root, uint32_t mtp_draft_depth,
+                                      int32_t map_tensors, qllm_artifact** out) {
+  if (!root || !out) return fail(QLLM_INVALID_ARGUMENT, "artifact root is null");
+  *out = nullptr;
+  try {
+    auto handle = std::make_unique<qllm_artifact>();
+    if (auto status = er::ModelArtifact::load(root, handle->artifact); !status.ok())
+      return from_status(status);
+    if (mtp_draft_depth)
+      if (auto status = handle->artifact.configure_mtp_draft_depth(mtp_draft_depth);
+          !status.ok())
+        return from_status(status);
+    if (map_tensors)
+      if (auto status =
+              er::MappedModelTensorStore::create(handle->artifact, handle->store);
+          !status.ok())
+        return from_status(status);
+    *out = handle.release();
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+extern "C" void qllm_artifact_close(qllm_artifact* artifact) { delete artifact; }
+
+extern "C" int32_t qllm_artifact_dump(const qllm_artifact* artifact, char* dump,
+                                      size_t capacity, size_t* dump_bytes) {
+  if (!artifact) return fail(QLLM_INVALID_ARGUMENT, "artifact is null");
+  try {
+    return copy_text(qllm::dump::model_artifact(artifact->artifact), dump, capacity,
+                     dump_bytes);
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+extern "C" int32_t qllm_artifact_tensor(qllm_artifact* artifact, const char* name,
+                                        int32_t check_header, const void** record,
+                                        uint64_t* record_bytes) {
+  if (!artifact || !name || !record || !record_bytes)
+    return fail(QLLM_INVALID_ARGUMENT, "artifact tensor query is invalid");
+  const auto resolved = artifact->store.resolve(name);
+  if (!resolved.status.ok()) return from_status(resolved.status);
+  if (check_header) {
+    const auto& entries = artifact->artifact.dense_tensors();
+    const auto entry = std::find_if(
+        entries.begin(), entries.end(),
+        [name](const er::ArtifactDenseTensor& item) { return item.name == name; });
+    if (entry == entries.end())
+      return fail(QLLM_INVALID_ARGUMENT, "tensor is absent from the dense index");
+    if (auto status = er::validate_dense_record(*entry, resolved.tensor->value.data,
+                                                resolved.tensor->value.bytes);
+        !status.ok())
+      return from_status(status);
+  }
+  *record = resolved.tensor->value.data;
+  *record_bytes = resolved.tensor->value.bytes;
+  return QLLM_OK;
 }

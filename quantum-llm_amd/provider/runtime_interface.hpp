@@ -8,9 +8,13 @@
 // header declares the slice of that boundary the verify path crosses, with
 // the same type names, member names and meanings, so that the provider source
 // compiles against the reference's own headers by swapping this include.
-// Types the verify path never touches (ModelDescriptor, the SSA program
-// descriptors, parking/snapshot results) are reduced to what prepare() needs.
+// Types the verify path never touches (the compiled SSA program, parking and
+// snapshot results) are reduced to what prepare() needs; the model descriptor
+// itself is in model_descriptor.hpp.
 #pragma once
+
+#include "model_descriptor.hpp"
+#include "status.hpp"
 
 #include <chrono>
 #include <cstddef>
@@ -26,36 +30,6 @@
 #include <vector>
 
 namespace expert::runtime {
-
-// storage.hpp:17-45
-enum class ErrorCode : std::uint8_t {
-  ok,
-  cancelled,
-  deadline_exceeded,
-  backpressure,
-  invalid_argument,
-  open_failed,
-  io_failed,
-  short_read,
-  checksum_mismatch,
-  upload_failed,
-  internal,
-};
-
-class Status final {
- public:
-  Status() = default;
-  Status(ErrorCode code, std::string message)
-      : code_(code), message_(std::move(message)) {}
-  [[nodiscard]] static Status success() { return {}; }
-  [[nodiscard]] bool ok() const noexcept { return code_ == ErrorCode::ok; }
-  [[nodiscard]] ErrorCode code() const noexcept { return code_; }
-  [[nodiscard]] std::string_view message() const noexcept { return message_; }
-
- private:
-  ErrorCode code_{ErrorCode::ok};
-  std::string message_;
-};
 
 // program_executor.hpp:24-50
 struct ExecutionValue final {
@@ -80,6 +54,19 @@ struct ImmutableModelTensor final {
   std::uint64_t scale_offset{};
   std::uint64_t scale_bytes{};
   ExecutionValue value;
+};
+
+// program_executor.hpp:52-62
+struct ResolveModelTensorResult final {
+  Status status;
+  std::shared_ptr<const ImmutableModelTensor> tensor;
+};
+
+class IModelTensorStore {
+ public:
+  virtual ~IModelTensorStore() = default;
+  [[nodiscard]] virtual ResolveModelTensorResult resolve(
+      std::string_view name) = 0;
 };
 
 struct PreparedTensorBinding final {
@@ -206,17 +193,7 @@ class IOperationProvider {
   }
 };
 
-// model_descriptor.hpp:60-80 / worker_provider.hpp:16-21.  The validator of
-// the reference takes the ModelDescriptor; here it takes the operation's
-// parameter map, which is what the dense descriptor check reads.
-struct KernelCapability final {
-  std::string capability;
-  std::uint32_t minimum_abi{};
-  std::uint32_t maximum_abi{};
-  std::function<Status(const std::map<std::string, std::uint64_t, std::less<>>&)>
-      validate;
-};
-
+// worker_provider.hpp:16-21 (KernelCapability is in model_descriptor.hpp)
 struct WorkerProviderDefinition final {
   std::string name;
   std::uint32_t priority{};

@@ -1,0 +1,135 @@
+#include "sha256.hpp"
+
+#include <algorithm>
+#include <bit>
+#include <cstring>
+
+namespace expert::runtime {
+namespace {
+
+// First 32 bits of the fractional parts of the cube roots of the first 64
+// primes (FIPS 180-4, 4.2.2).
+constexpr std::uint32_t kRound[64] = {
+    0x428a2f98U, 0x71374491U, 0xb5c0fbcfU, 0xe9b5dba5U, 0x3956c25bU, 0x59f111f1U,
+    0x923f82a4U, 0xab1c5ed5U, 0xd807aa98U, 0x12835b01U, 0x243185beU, 0x550c7dc3U,
+    0x72be5d74U, 0x80deb1feU, 0x9bdc06a7U, 0xc19bf174U, 0xe49b69c1U, 0xefbe4786U,
+    0x0fc19dc6U, 0x240ca1ccU, 0x2de92c6fU, 0x4a7484aaU, 0x5cb0a9dcU, 0x76f988daU,
+    0x983e5152U, 0xa831c66dU, 0xb00327c8U, 0xbf597fc7U, 0xc6e00bf3U, 0xd5a79147U,
+    0x06ca6351U, 0x14292967U, 0x27b70a85U, 0x2e1b2138U, 0x4d2c6dfcU, 0x53380d13U,
+    0x650a7354U, 0x766a0abbU, 0x81c2c92eU, 0x92722c85U, 0xa2bfe8a1U, 0xa81a664bU,
+    0xc24b8b70U, 0xc76c51a3U, 0xd192e819U, 0xd6990624U, 0xf40e3585U, 0x106aa070U,
+    0x19a4c116U, 0x1e376c08U, 0x2748774cU, 0x34b0bcb5U, 0x391c0cb3U, 0x4ed8aa4aU,
+    0x5b9cca4fU, 0x682e6ff3U, 0x748f82eeU, 0x78a5636fU, 0x84c87814U, 0x8cc70208U,
+    0x90befffaU, 0xa4506cebU, 0xbef9a3f7U, 0xc67178f2U};
+
+constexpr std::uint32_t kInitial[8] = {0x6a09e667U, 0xbb67ae85U, 0x3c6ef372U,
+                                       0xa54ff53aU, 0x510e527fU, 0x9b05688cU,
+                                       0x1f83d9abU, 0x5be0cd19U};
+
+}  // namespace
+
+Sha256::Sha256() noexcept {
+  std::copy(std::begin(kInitial), std::end(kInitial), state_.begin());
+}
+
+void Sha256::compress(const std::byte* block) noexcept {
+  std::uint32_t schedule[64];
+  for (int word = 0; word < 16; ++word) {
+    const auto* bytes = reinterpret_cast<const unsigned char*>(block) + 4 * word;
+    schedule[word] = (std::uint32_t{bytes[0]} << 24) |
+                     (std::uint32_t{bytes[1]} << 16) |
+                     (std::uint32_t{bytes[2]} << 8) | std::uint32_t{bytes[3]};
+  }
+  for (int word = 16; word < 64; ++word) {
+    const std::uint32_t x = schedule[word - 15];
+    const std::uint32_t y = schedule[word - 2];
+    const std::uint32_t small0 = std::rotr(x, 7) ^ std::rotr(x, 18) ^ (x >> 3);
+    const std::uint32_t small1 = std::rotr(y, 17) ^ std::rotr(y, 19) ^ (y >> 10);
+    schedule[word] = schedule[word - 16] + small0 + schedule[word - 7] + small1;
+  }
+  std::uint32_t a = state_[0], b = state_[1], c = state_[2], d = state_[3];
+  std::uint32_t e = state_[4], f = state_[5], g = state_[6], h = state_[7];
+  for (int round = 0; round < 64; ++round) {
+    const std::uint32_t big1 = std::rotr(e, 6) ^ std::rotr(e, 11) ^ std::rotr(e, 25);
+    const std::uint32_t choose = (e & f) ^ (~e & g);
+    const std::uint32_t first = h + big1 + choose + kRound[round] + schedule[round];
+    const std::uint32_t big0 = std::rotr(a, 2) ^ std::rotr(a, 13) ^ std::rotr(a, 22);
+    const std::uint32_t majority = (a & b) ^ (a & c) ^ (b & c);
+    const std::uint32_t second = big0 + majority;
+    h = g;
+    g = f;
+    f = e;
+    e = d + first;
+    d = c;
+    c = b;
+    b = a;
+    a = first + second;
+  }
+  state_[0] += a;
+  state_[1] += b;
+  state_[2] += c;
+  state_[3] += d;
+  state_[4] += e;
+  state_[5] += f;
+  state_[6] += g;
+  state_[7] += h;
+}
+
+void Sha256::update(std::span<const std::byte> input) noexcept {
+  if (finalized_) return;
+  message_bytes_ += input.size();
+  const std::byte* cursor = input.data();
+  std::size_t left = input.size();
+  if (pending_bytes_) {
+    const std::size_t take = std::min(left, pending_.size() - pending_bytes_);
+    std::memcpy(pending_.data() + pending_bytes_, cursor, take);
+    pending_bytes_ += take;
+    cursor += take;
+    left -= take;
+    if (pending_bytes_ < pending_.size()) return;
+    compress(pending_.data());
+    pending_bytes_ = 0;
+  }
+  for (; left >= 64; cursor += 64, left -= 64) compress(cursor);
+  if (left) std::memcpy(pending_.data(), cursor, left);
+  pending_bytes_ = left;
+}
+
+Sha256Digest Sha256::finalize() noexcept {
+  if (finalized_) return digest_;
+  const std::uint64_t message_bits = message_bytes_ * 8U;
+  // 0x80, zeros up to 56 mod 64, then the bit length, big endian
+  pending_[pending_bytes_++] = std::byte{0x80};
+  if (pending_bytes_ > 56) {
+    std::memset(pending_.data() + pending_bytes_, 0, 64 - pending_bytes_);
+    compress(pending_.data());
+    pending_bytes_ = 0;
+  }
+  std::memset(pending_.data() + pending_bytes_, 0, 56 - pending_bytes_);
+  for (int index = 0; index < 8; ++index)
+    pending_[56 + index] =
+        static_cast<std::byte>((message_bits >> (8 * (7 - index))) & 0xffU);
+  compress(pending_.data());
+  for (int word = 0; word < 8; ++word)
+    for (int index = 0; index < 4; ++index)
+      digest_[4 * word + index] =
+          static_cast<std::byte>((state_[word] >> (8 * (3 - index))) & 0xffU);
+  finalized_ = true;
+  return digest_;
+}
+
+Sha256Digest sha256(std::span<const std::byte> input) noexcept {
+  Sha256 hash;
+  hash.update(input);
+  return hash.finalize();
+}
+
+bool constant_time_equal(const Sha256Digest& left,
+                         const Sha256Digest& right) noexcept {
+  unsigned difference = 0;
+  for (std::size_t index = 0; index < left.size(); ++index)
+    difference |= std::to_integer<unsigned>(left[index] ^ right[index]);
+  return difference == 0;
+}
+
+}  // namespace expert::runtime

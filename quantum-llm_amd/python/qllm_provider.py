@@ -66,6 +66,14 @@ SIGNATURES = {
     "qllm_sampling_sample": (c_int32, [c_void_p, c_void_p, c_uint32, c_double, POINTER(c_uint32)]),
     "qllm_sampling_rejection": (c_int32, [c_uint32, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_double, c_double, POINTER(c_int32), POINTER(c_uint32), POINTER(c_double), POINTER(c_double)]),
     "qllm_sampling_counter_uniform": (c_double, [c_uint64, c_uint32, c_uint32, c_uint32]),
+    "qllm_provider_create_from_artifact": (c_void_p, [c_char_p, c_uint32, c_uint32, c_char_p, c_uint32]),
+    "qllm_sha256": (c_int32, [c_void_p, c_size_t, c_void_p]),
+    "qllm_model_descriptor_parse": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
+    "qllm_model_descriptor_load": (c_int32, [c_char_p, c_uint64, c_char_p, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
+    "qllm_artifact_open": (c_int32, [c_char_p, c_uint32, c_int32, POINTER(c_void_p)]),
+    "qllm_artifact_close": (None, [c_void_p]),
+    "qllm_artifact_dump": (c_int32, [c_void_p, c_char_p, c_size_t, POINTER(c_size_t)]),
+    "qllm_artifact_tensor": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_void_p), POINTER(c_uint64)]),
 }
 
 _library = None
@@ -101,6 +109,21 @@ class Provider:
         self.handle = self.lib.qllm_provider_create(ctypes.byref(self.geometry))
         if not self.handle:
             raise ProviderError(10, self.lib.qllm_provider_last_error().decode())
+
+    @classmethod
+    def from_artifact(cls, root, geometry, max_context=0, kv_page_tokens=0,
+                      kv_cache_dtype=None, mtp_draft_depth=0):
+        """A provider loaded and prepared from an Expert Pack v1 directory;
+        `geometry` (keyword dictionary) only describes it to this wrapper."""
+        self = cls.__new__(cls)
+        self.geometry = DenseGeometry(**geometry)
+        self.lib = load()
+        self.handle = self.lib.qllm_provider_create_from_artifact(
+            os.fsencode(root), max_context, kv_page_tokens,
+            kv_cache_dtype.encode() if kv_cache_dtype else None, mtp_draft_depth)
+        if not self.handle:
+            raise ProviderError(10, self.lib.qllm_provider_last_error().decode())
+        return self
 
     def close(self):
         if self.handle:
