@@ -28,14 +28,14 @@ constexpr std::uint32_t kInitial[8] = {0x6a09e667U, 0xbb67ae85U, 0x3c6ef372U,
 
 }  // namespace
 
-Sha256::Sha256() noexcept {
-  std::copy(std::begin(kInitial), std::end(kInitial), state_.begin());
+Sha256Stream::Sha256Stream() noexcept {
+  std::copy(std::begin(kInitial), std::end(kInitial), h_);
 }
 
-void Sha256::compress(const std::byte* block) noexcept {
+void Sha256Stream::block(const std::byte* sixty_four_bytes) noexcept {
   std::uint32_t schedule[64];
   for (int word = 0; word < 16; ++word) {
-    const auto* bytes = reinterpret_cast<const unsigned char*>(block) + 4 * word;
+    const auto* bytes = reinterpret_cast<const unsigned char*>(sixty_four_bytes) + 4 * word;
     schedule[word] = (std::uint32_t{bytes[0]} << 24) |
                      (std::uint32_t{bytes[1]} << 16) |
                      (std::uint32_t{bytes[2]} << 8) | std::uint32_t{bytes[3]};
@@ -47,8 +47,8 @@ void Sha256::compress(const std::byte* block) noexcept {
     const std::uint32_t small1 = std::rotr(y, 17) ^ std::rotr(y, 19) ^ (y >> 10);
     schedule[word] = schedule[word - 16] + small0 + schedule[word - 7] + small1;
   }
-  std::uint32_t a = state_[0], b = state_[1], c = state_[2], d = state_[3];
-  std::uint32_t e = state_[4], f = state_[5], g = state_[6], h = state_[7];
+  std::uint32_t a = h_[0], b = h_[1], c = h_[2], d = h_[3];
+  std::uint32_t e = h_[4], f = h_[5], g = h_[6], h = h_[7];
   for (int round = 0; round < 64; ++round) {
     const std::uint32_t big1 = std::rotr(e, 6) ^ std::rotr(e, 11) ^ std::rotr(e, 25);
     const std::uint32_t choose = (e & f) ^ (~e & g);
@@ -65,63 +65,61 @@ void Sha256::compress(const std::byte* block) noexcept {
     b = a;
     a = first + second;
   }
-  state_[0] += a;
-  state_[1] += b;
-  state_[2] += c;
-  state_[3] += d;
-  state_[4] += e;
-  state_[5] += f;
-  state_[6] += g;
-  state_[7] += h;
+  h_[0] += a;
+  h_[1] += b;
+  h_[2] += c;
+  h_[3] += d;
+  h_[4] += e;
+  h_[5] += f;
+  h_[6] += g;
+  h_[7] += h;
 }
 
-void Sha256::update(std::span<const std::byte> input) noexcept {
-  if (finalized_) return;
-  message_bytes_ += input.size();
-  const std::byte* cursor = input.data();
-  std::size_t left = input.size();
-  if (pending_bytes_) {
-    const std::size_t take = std::min(left, pending_.size() - pending_bytes_);
-    std::memcpy(pending_.data() + pending_bytes_, cursor, take);
-    pending_bytes_ += take;
+void Sha256Stream::feed(std::span<const std::byte> bytes) noexcept {
+  total_size_ += bytes.size();
+  const std::byte* cursor = bytes.data();
+  std::size_t left = bytes.size();
+  if (partial_size_) {
+    const std::size_t take = std::min(left, sizeof(partial_) - partial_size_);
+    std::memcpy(partial_ + partial_size_, cursor, take);
+    partial_size_ += take;
     cursor += take;
     left -= take;
-    if (pending_bytes_ < pending_.size()) return;
-    compress(pending_.data());
-    pending_bytes_ = 0;
+    if (partial_size_ < sizeof(partial_)) return;
+    block(partial_);
+    partial_size_ = 0;
   }
-  for (; left >= 64; cursor += 64, left -= 64) compress(cursor);
-  if (left) std::memcpy(pending_.data(), cursor, left);
-  pending_bytes_ = left;
+  for (; left >= 64; cursor += 64, left -= 64) block(cursor);
+  if (left) std::memcpy(partial_, cursor, left);
+  partial_size_ = left;
 }
 
-Sha256Digest Sha256::finalize() noexcept {
-  if (finalized_) return digest_;
-  const std::uint64_t message_bits = message_bytes_ * 8U;
+Sha256Digest Sha256Stream::digest() noexcept {
+  const std::uint64_t message_bits = total_size_ * 8U;
   // 0x80, zeros up to 56 mod 64, then the bit length, big endian
-  pending_[pending_bytes_++] = std::byte{0x80};
-  if (pending_bytes_ > 56) {
-    std::memset(pending_.data() + pending_bytes_, 0, 64 - pending_bytes_);
-    compress(pending_.data());
-    pending_bytes_ = 0;
+  partial_[partial_size_++] = std::byte{0x80};
+  if (partial_size_ > 56) {
+    std::memset(partial_ + partial_size_, 0, 64 - partial_size_);
+    block(partial_);
+    partial_size_ = 0;
   }
-  std::memset(pending_.data() + pending_bytes_, 0, 56 - pending_bytes_);
+  std::memset(partial_ + partial_size_, 0, 56 - partial_size_);
   for (int index = 0; index < 8; ++index)
-    pending_[56 + index] =
+    partial_[56 + index] =
         static_cast<std::byte>((message_bits >> (8 * (7 - index))) & 0xffU);
-  compress(pending_.data());
+  block(partial_);
+  Sha256Digest result;
   for (int word = 0; word < 8; ++word)
     for (int index = 0; index < 4; ++index)
-      digest_[4 * word + index] =
-          static_cast<std::byte>((state_[word] >> (8 * (3 - index))) & 0xffU);
-  finalized_ = true;
-  return digest_;
+      result[4 * word + index] =
+          static_cast<std::byte>((h_[word] >> (8 * (3 - index))) & 0xffU);
+  return result;
 }
 
 Sha256Digest sha256(std::span<const std::byte> input) noexcept {
-  Sha256 hash;
-  hash.update(input);
-  return hash.finalize();
+  Sha256Stream stream;
+  stream.feed(input);
+  return stream.digest();
 }
 
 bool constant_time_equal(const Sha256Digest& left,

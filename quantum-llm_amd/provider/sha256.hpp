@@ -1,7 +1,8 @@
 // SHA-256 (FIPS 180-4) for authenticating artifact files: the program file
-// against the manifest, packs against their index entries, record payloads
-// against their headers.  Same interface as the reference's
-// runtime/include/expert/runtime/sha256.hpp:11-29.
+// against the manifest, packs against their index entries, record names
+// against their headers.  sha256() and constant_time_equal() stand for the
+// functions of the same names in the reference
+// (runtime/include/expert/runtime/sha256.hpp:26-28).
 #pragma once
 
 #include <array>
@@ -14,24 +15,23 @@ namespace expert::runtime {
 // storage.hpp:47
 using Sha256Digest = std::array<std::byte, 32>;
 
-class Sha256 final {
+// Incremental form: feed() any number of times, then digest().
+class Sha256Stream final {
  public:
-  Sha256() noexcept;
-  void update(std::span<const std::byte> input) noexcept;
-  // The digest of everything fed so far; further updates are ignored.
-  [[nodiscard]] Sha256Digest finalize() noexcept;
+  Sha256Stream() noexcept;
+  void feed(std::span<const std::byte> bytes) noexcept;
+  [[nodiscard]] Sha256Digest digest() noexcept;
 
  private:
-  void compress(const std::byte* block) noexcept;
-  std::array<std::uint32_t, 8> state_{};
-  std::array<std::byte, 64> pending_{};
-  std::size_t pending_bytes_{};
-  std::uint64_t message_bytes_{};
-  Sha256Digest digest_{};
-  bool finalized_{};
+  void block(const std::byte* sixty_four_bytes) noexcept;
+  std::uint32_t h_[8];
+  std::byte partial_[64];
+  std::size_t partial_size_{0};
+  std::uint64_t total_size_{0};
 };
 
 [[nodiscard]] Sha256Digest sha256(std::span<const std::byte> input) noexcept;
+// Compares all 32 bytes whatever the first difference is.
 [[nodiscard]] bool constant_time_equal(const Sha256Digest& left,
                                        const Sha256Digest& right) noexcept;
 
