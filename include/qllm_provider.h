@@ -238,6 +238,9 @@ double qllm_sampling_counter_uniform(uint64_t seed, uint32_t position,
 
 /* sha256() of runtime/include/expert/runtime/sha256.hpp:26. */
 int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest32);
+/* The same digest computed without the CPU's SHA instructions, which
+ * qllm_sha256 uses where the host has them. */
+int32_t qllm_sha256_portable(const void* data, size_t bytes, uint8_t* digest32);
 
 /* parse_model_descriptor_artifact (runtime/include/expert/runtime/
  * model_descriptor.hpp:276-281; runtime/src/model_descriptor.cpp:527-723):

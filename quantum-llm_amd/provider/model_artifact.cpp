@@ -7,6 +7,7 @@
 #include "json_reader.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cerrno>
 #include <cstring>
 #include <fstream>
@@ -14,6 +15,7 @@
 #include <map>
 #include <sstream>
 #include <stdexcept>
+#include <thread>
 
 #include <fcntl.h>
 #include <sys/mman.h>
@@ -383,11 +385,36 @@ Status MappedModelTensorStore::create(const ModelArtifact& artifact,
       return {ErrorCode::invalid_argument,
               "mapped tensor store destination is already initialized"};
     auto core = std::make_shared<Core>();
-    for (const auto& pack : artifact.packs()) {
-      if (pack.kind != "dense") continue;
-      std::shared_ptr<MappedPack> mapped;
-      if (auto status = MappedPack::open(pack, mapped); !status.ok()) return status;
-      if (!core->packs.emplace(pack.name, std::move(mapped)).second)
+    // Packs are mapped and hashed side by side (a checksum is sequential
+    // within a file, not across files); the first failure in index order is
+    // the one reported.
+    std::vector<const ArtifactPack*> dense;
+    for (const auto& pack : artifact.packs())
+      if (pack.kind == "dense") dense.push_back(&pack);
+    std::vector<std::shared_ptr<MappedPack>> mapped(dense.size());
+    std::vector<Status> opened(dense.size());
+    {
+      constexpr std::size_t kMaximumThreads = 8;
+      std::atomic<std::size_t> next{0};
+      const auto work = [&]() {
+        for (std::size_t index = next++; index < dense.size(); index = next++) {
+          try {
+            opened[index] = MappedPack::open(*dense[index], mapped[index]);
+          } catch (const std::exception& error) {
+            opened[index] = {ErrorCode::internal, error.what()};
+          }
+        }
+      };
+      std::vector<std::thread> threads;
+      for (std::size_t index = 1;
+           index < std::min(dense.size(), kMaximumThreads); ++index)
+        threads.emplace_back(work);
+      work();
+      for (auto& thread : threads) thread.join();
+    }
+    for (std::size_t index = 0; index < dense.size(); ++index) {
+      if (!opened[index].ok()) return opened[index];
+      if (!core->packs.emplace(dense[index]->name, std::move(mapped[index])).second)
         return {ErrorCode::invalid_argument,
                 "dense artifact pack name is duplicated"};
     }

@@ -571,6 +571,16 @@ extern "C" int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest) 
   return QLLM_OK;
 }
 
+extern "C" int32_t qllm_sha256_portable(const void* data, size_t bytes,
+                                        uint8_t* digest) {
+  if ((!data && bytes) || !digest)
+    return fail(QLLM_INVALID_ARGUMENT, "SHA-256 arguments are invalid");
+  const auto result =
+      er::sha256_portable({static_cast<const std::byte*>(data), bytes});
+  std::memcpy(digest, result.data(), result.size());
+  return QLLM_OK;
+}
+
 extern "C" int32_t qllm_model_descriptor_parse(
     const char* text, size_t text_bytes, const uint8_t* content_sha256,
     uint64_t namespace_base, char* dump, size_t capacity, size_t* dump_bytes) {

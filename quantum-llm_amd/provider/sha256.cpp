@@ -4,6 +4,10 @@
 #include <bit>
 #include <cstring>
 
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
+
 namespace expert::runtime {
 namespace {
 
@@ -26,13 +30,81 @@ constexpr std::uint32_t kInitial[8] = {0x6a09e667U, 0xbb67ae85U, 0x3c6ef372U,
                                        0xa54ff53aU, 0x510e527fU, 0x9b05688cU,
                                        0x1f83d9abU, 0x5be0cd19U};
 
+#if defined(__x86_64__)
+// One or more 64-byte blocks with the x86 SHA extensions: the state lives in
+// two registers as (A,B,E,F) and (C,D,G,H), each sha256rnds2 does two rounds,
+// sha256msg1/msg2 extend the message schedule four words at a time.
+__attribute__((target("sha,sse4.1,ssse3"))) void blocks_sha_ni(
+    std::uint32_t state[8], const std::byte* data, std::size_t blocks) noexcept {
+  const __m128i byte_swap =
+      _mm_set_epi64x(0x0c0d0e0f08090a0bLL, 0x0405060700010203LL);
+  __m128i low = _mm_loadu_si128(reinterpret_cast<const __m128i*>(state));       // DCBA
+  __m128i high = _mm_loadu_si128(reinterpret_cast<const __m128i*>(state + 4));  // HGFE
+  low = _mm_shuffle_epi32(low, 0xb1);                 // CDAB
+  high = _mm_shuffle_epi32(high, 0x1b);               // EFGH
+  __m128i abef = _mm_alignr_epi8(low, high, 8);       // ABEF
+  __m128i cdgh = _mm_blend_epi16(high, low, 0xf0);    // CDGH
+  const auto* constants = reinterpret_cast<const __m128i*>(kRound);
+  for (; blocks; --blocks, data += 64) {
+    const __m128i saved_abef = abef;
+    const __m128i saved_cdgh = cdgh;
+    __m128i words[4];
+    for (int index = 0; index < 4; ++index)
+      words[index] = _mm_shuffle_epi8(
+          _mm_loadu_si128(reinterpret_cast<const __m128i*>(data) + index),
+          byte_swap);
+    for (int quad = 0; quad < 16; ++quad) {
+      __m128i& current = words[quad & 3];
+      if (quad >= 4) {
+        // W[t..t+3] from W[t-16..], W[t-15..] (msg1), W[t-7..] and W[t-2..] (msg2)
+        __m128i extended = _mm_sha256msg1_epu32(current, words[(quad + 1) & 3]);
+        extended = _mm_add_epi32(
+            extended,
+            _mm_alignr_epi8(words[(quad + 3) & 3], words[(quad + 2) & 3], 4));
+        current = _mm_sha256msg2_epu32(extended, words[(quad + 3) & 3]);
+      }
+      __m128i rounds = _mm_add_epi32(current, _mm_loadu_si128(constants + quad));
+      cdgh = _mm_sha256rnds2_epu32(cdgh, abef, rounds);
+      rounds = _mm_shuffle_epi32(rounds, 0x0e);
+      abef = _mm_sha256rnds2_epu32(abef, cdgh, rounds);
+    }
+    abef = _mm_add_epi32(abef, saved_abef);
+    cdgh = _mm_add_epi32(cdgh, saved_cdgh);
+  }
+  low = _mm_shuffle_epi32(abef, 0x1b);                // FEBA
+  high = _mm_shuffle_epi32(cdgh, 0xb1);               // DCHG
+  _mm_storeu_si128(reinterpret_cast<__m128i*>(state),
+                   _mm_blend_epi16(low, high, 0xf0));          // DCBA
+  _mm_storeu_si128(reinterpret_cast<__m128i*>(state + 4),
+                   _mm_alignr_epi8(high, low, 8));             // HGFE
+}
+
+bool has_sha_extensions() noexcept {
+  static const bool available = __builtin_cpu_supports("sha") &&
+                                __builtin_cpu_supports("sse4.1") &&
+                                __builtin_cpu_supports("ssse3");
+  return available;
+}
+#endif
+
 }  // namespace
 
-Sha256Stream::Sha256Stream() noexcept {
+Sha256Stream::Sha256Stream(bool portable) noexcept {
   std::copy(std::begin(kInitial), std::end(kInitial), h_);
+#if defined(__x86_64__)
+  accelerated_ = !portable && has_sha_extensions();
+#else
+  (void)portable;
+#endif
 }
 
 void Sha256Stream::block(const std::byte* sixty_four_bytes) noexcept {
+#if defined(__x86_64__)
+  if (accelerated_) {
+    blocks_sha_ni(h_, sixty_four_bytes, 1);
+    return;
+  }
+#endif
   std::uint32_t schedule[64];
   for (int word = 0; word < 16; ++word) {
     const auto* bytes = reinterpret_cast<const unsigned char*>(sixty_four_bytes) + 4 * word;
@@ -89,6 +161,14 @@ void Sha256Stream::feed(std::span<const std::byte> bytes) noexcept {
     block(partial_);
     partial_size_ = 0;
   }
+#if defined(__x86_64__)
+  if (accelerated_ && left >= 64) {
+    const std::size_t whole = left / 64;
+    blocks_sha_ni(h_, cursor, whole);
+    cursor += whole * 64;
+    left -= whole * 64;
+  }
+#endif
   for (; left >= 64; cursor += 64, left -= 64) block(cursor);
   if (left) std::memcpy(partial_, cursor, left);
   partial_size_ = left;
@@ -118,6 +198,12 @@ Sha256Digest Sha256Stream::digest() noexcept {
 
 Sha256Digest sha256(std::span<const std::byte> input) noexcept {
   Sha256Stream stream;
+  stream.feed(input);
+  return stream.digest();
+}
+
+Sha256Digest sha256_portable(std::span<const std::byte> input) noexcept {
+  Sha256Stream stream(true);
   stream.feed(input);
   return stream.digest();
 }

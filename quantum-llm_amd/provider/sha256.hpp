@@ -18,7 +18,9 @@ using Sha256Digest = std::array<std::byte, 32>;
 // Incremental form: feed() any number of times, then digest().
 class Sha256Stream final {
  public:
-  Sha256Stream() noexcept;
+  // `portable` keeps to plain integer code even where the CPU has SHA
+  // instructions (both give the same digests; the flag exists for testing).
+  explicit Sha256Stream(bool portable = false) noexcept;
   void feed(std::span<const std::byte> bytes) noexcept;
   [[nodiscard]] Sha256Digest digest() noexcept;
 
@@ -28,9 +30,11 @@ class Sha256Stream final {
   std::byte partial_[64];
   std::size_t partial_size_{0};
   std::uint64_t total_size_{0};
+  bool accelerated_{false};
 };
 
 [[nodiscard]] Sha256Digest sha256(std::span<const std::byte> input) noexcept;
+[[nodiscard]] Sha256Digest sha256_portable(std::span<const std::byte> input) noexcept;
 // Compares all 32 bytes whatever the first difference is.
 [[nodiscard]] bool constant_time_equal(const Sha256Digest& left,
                                        const Sha256Digest& right) noexcept;

@@ -68,6 +68,7 @@ SIGNATURES = {
     "qllm_sampling_counter_uniform": (c_double, [c_uint64, c_uint32, c_uint32, c_uint32]),
     "qllm_provider_create_from_artifact": (c_void_p, [c_char_p, c_uint32, c_uint32, c_char_p, c_uint32]),
     "qllm_sha256": (c_int32, [c_void_p, c_size_t, c_void_p]),
+    "qllm_sha256_portable": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_model_descriptor_parse": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_model_descriptor_load": (c_int32, [c_char_p, c_uint64, c_char_p, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_artifact_open": (c_int32, [c_char_p, c_uint32, c_int32, POINTER(c_void_p)]),

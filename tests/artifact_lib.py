@@ -57,6 +57,12 @@ class Product:
         return out.raw
 
     @staticmethod
+    def sha256_portable(data: bytes) -> bytes:
+        out = create_string_buffer(32)
+        assert product().qllm_sha256_portable(data, len(data), out) == 0
+        return out.raw
+
+    @staticmethod
     def parse(text: bytes, content_hash: bytes, namespace_base: int):
         lib = product()
         buffer, length = create_string_buffer(CAPACITY), c_size_t()

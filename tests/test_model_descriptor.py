@@ -56,13 +56,17 @@ def test_sha256_known_answers():
     }
     for message, want in known.items():
         assert al.Product.sha256(message).hex() == want
+        assert al.Product.sha256_portable(message).hex() == want
 
 
 def test_sha256_matches_hashlib_across_block_boundaries():
     rng = np.random.default_rng(1)
     for size in [*range(0, 200), 1000, 4095, 4096, 4097, 1 << 20]:
         data = rng.integers(0, 256, size, dtype=np.uint8).tobytes()
-        assert al.Product.sha256(data) == hashlib.sha256(data).digest(), size
+        want = hashlib.sha256(data).digest()
+        # with the CPU's SHA instructions where present, and without
+        assert al.Product.sha256(data) == want, size
+        assert al.Product.sha256_portable(data) == want, size
 
 
 # ---- the reference's own fixtures --------------------------------------------
