@@ -163,6 +163,38 @@ def measure_decode_cycle(qp, np, rows, steps, warmup):
     return report
 
 
+def measure_prefill(qp, np, prompt_tokens):
+    """Prompt prefill of the same model: `prompt_tokens` synthetic tokens from
+    position 0 - the linears on the tall-batch GEMM (1024 rows at a time),
+    attention and the Q4H store in row batches of five - timed from the call
+    to the prediction of the token after the prompt (time to first token)."""
+    geometry = dict(MODEL)
+    geometry["max_context"] = (prompt_tokens + 16 + 255) // 256 * 256
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(20241125)
+    provider.prepare_exact_decode("decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2")
+    rng = np.random.default_rng(11)
+    tokens = rng.integers(0, MODEL["vocabulary"], prompt_tokens).astype(np.uint32)
+    provider.prefill(tokens[:min(prompt_tokens, 1024)], 0)      # warm-up, allocates
+    provider.synchronize_stream()
+    begin = time.perf_counter()
+    provider.prefill(tokens, 0)
+    elapsed = time.perf_counter() - begin
+    H, I, Q, KV, d = (MODEL["hidden"], MODEL["intermediate"], MODEL["query_heads"],
+                      MODEL["kv_heads"], MODEL["head_dim"])
+    linear_flops = 2.0 * prompt_tokens * MODEL["layers"] * (
+        (Q + 2 * KV) * d * H + H * Q * d + 3 * I * H)
+    report = {
+        "prompt_tokens": prompt_tokens,
+        "seconds_to_first_token": round(elapsed, 3),
+        "tok_s": round(prompt_tokens / elapsed, 1),
+        "linear_tflops_if_all_time_were_linears": round(linear_flops / elapsed / 1e12, 1),
+        "reference_published_ttft_s_32k_rtx3090": 39.6,
+    }
+    provider.close()
+    return report
+
+
 def measure_long_contexts(qp, np, rows):
     """tok/s of the same 64-layer verify step with the Q4H cache prefilled to
     131072 tokens, and the exact-F16 attention kernel over 262144 tokens
@@ -242,6 +274,9 @@ def main():
     parser.add_argument("--skip-decode-cycle", action="store_true",
                         help="leave out the decode cycle with the proposer (a second "
                              "provider with the MTP layer)")
+    parser.add_argument("--prefill-tokens", type=int, default=2048,
+                        help="prompt length of the prefill leg (0 skips it; 32768 "
+                             "is the context of the headline metric)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one 256 MiB device copy (a kernel of known "
                              "traffic to scale hardware counters by)")
@@ -346,6 +381,12 @@ def main():
             provider.close()
         provider = None
         long_context = measure_long_contexts(qp, np, rows)
+    prefill = {}
+    if arguments.layers == MODEL["layers"] and arguments.prefill_tokens > 0:
+        if provider is not None:
+            provider.close()
+        provider = None
+        prefill = measure_prefill(qp, np, arguments.prefill_tokens)
     layers = geometry["layers"]
     step_bytes = (layers * (fp4_bytes(MODEL["query_heads"] * 128, H) +
                             2 * fp4_bytes(MODEL["kv_heads"] * 128, H) +
@@ -393,6 +434,8 @@ def main():
         result["decode_cycle_with_proposer"] = decode_cycle
     if long_context:
         result["long_context"] = long_context
+    if prefill:
+        result["prompt_prefill"] = prefill
     if arguments.calibration_copy:
         source = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
         target = torch.empty_like(source)

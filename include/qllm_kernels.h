@@ -167,6 +167,28 @@ int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
                              size_t input_bytes, void* output,
                              uint32_t batch, void* stream);
 
+/* The GEMM for tall batches (prompt prefill): any batch, a matrix in the tiled
+ * layout with 32-row tiles, input bf16 [batch, padded_columns] (16-byte
+ * aligned), output [batch, rows] in `output_kind`, optional F32 residual of
+ * the same shape.  Workgroups of 128 batch rows x 256 weight rows on the
+ * matrix cores.  With UE8M0 scales the arithmetic is the reference's (exact
+ * bf16 operands, F32 accumulation); with binary16 scales the scaled weights
+ * and the activations enter as binary16 (see the kernel's header).
+ * replaces fp4_gemm_bf16_block32 at batch > 8 (transformer_kernels.cu:
+ * 1284-1430, launched from :7400-7593). */
+int32_t qllm_fp4_gemm_bf16_tall(const qllm_fp4_matrix* matrix, const void* input,
+                                size_t input_bytes, void* output,
+                                uint32_t output_kind, const float* residual,
+                                uint32_t batch, void* stream);
+/* The same with the output columns split over up to three buffers, each a
+ * multiple of 32 weight rows (the q, k and v projections stored as one
+ * matrix). */
+int32_t qllm_fp4_gemm_bf16_tall_split(const qllm_fp4_matrix* matrix,
+                                      const void* input, size_t input_bytes,
+                                      const qllm_gemm_segment* segments,
+                                      uint32_t segment_count, uint32_t batch,
+                                      void* stream);
+
 /* replaces fp4_embedding_batch (transformer_kernels.hpp:68-70). */
 int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
                                  const uint32_t* tokens, float* output,

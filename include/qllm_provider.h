@@ -121,6 +121,19 @@ int32_t qllm_provider_begin_request(qllm_provider* provider,
 int32_t qllm_provider_synchronize(qllm_provider* provider, uint32_t token,
                                   uint32_t position);
 
+/* Prompt prefill: `count` tokens at positions first_position .. through the
+ * target (linears on the tall-batch GEMM, K/V written to the paged cache),
+ * `*predicted` = the greedy token for the position after the prompt, whose
+ * logits are row 0 of qllm_provider_copy_logits.  After
+ * qllm_provider_begin_request the proposer is fed the prompt too and the
+ * first drafts are rolled out, so that qllm_provider_verify can follow with
+ * (*predicted, first_position + count).  This is the worker's feed
+ * (runtime/tools/moe_vm_runner.cpp:682-745: program-sequence prefill, then
+ * synchronize_exact_decode_batch over the prompt in chunks). */
+int32_t qllm_provider_prefill(qllm_provider* provider, const uint32_t* tokens,
+                              uint32_t count, uint32_t first_position,
+                              uint32_t* predicted);
+
 /* Drafts for the next verify step.  distribution_counts[i] entries of
  * (tokens, probabilities) describe draft i's proposal distribution q; a count
  * of 0 means the one-hot distribution on the draft token (greedy). */

@@ -741,6 +741,87 @@ er::Status Mi355DenseFp4Provider::set_draft_predictions(
 
 // ---- target pass ------------------------------------------------------------
 
+// Rotary + per-head norm of the new rows' q and k, their K/V records into the
+// layer's cache and the rows' attention over everything cached so far
+// (run_full_attention, :6892-7960).  `query`, `key`, `value` hold `rows` rows
+// starting at `first_position`; the result goes to `attention_out` in bf16.
+void Mi355DenseFp4Provider::enqueue_attention(
+    std::uint32_t index, std::uint32_t rows, std::uint32_t first_position,
+    bool deferred_positions, float* query, float* key, const float* value,
+    std::uint16_t* attention_out) {
+  void* const stream = stream_;
+  const auto& layer = layers_[index];
+  const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+  if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
+    if (deferred_positions)
+      status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
+          query, query_stride, key, value, layer.query_norm,
+          layer.key_norm, const_cast<const void* const*>(device_page_table_),
+          index, g_.kv_page_tokens, positions_, rows, g_.query_heads,
+          g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
+          g_.rope_theta, 0, stream));
+    else
+      status_check(qllm_qkv_rope_cache_paged_q4h_batch(
+          query, query_stride, key, value, layer.query_norm,
+          layer.key_norm, const_cast<const void* const*>(device_page_table_),
+          index, g_.kv_page_tokens, first_position, first_position, rows,
+          g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
+          g_.norm_epsilon, g_.rope_theta, 0, stream));
+    qllm_q4h_attention_launch launch{};
+    launch.query = query;
+    launch.page_table = const_cast<const void* const*>(device_page_table_);
+    launch.output = attention_out;
+    launch.partial_maxima = partial_maxima_;
+    launch.partial_sums = partial_sums_;
+    launch.partial_outputs = partial_outputs_;
+    launch.first_context_tokens = first_position + 1U;  // :7915
+    launch.rows = rows;
+    launch.full_attention_layer = index;
+    launch.page_tokens = g_.kv_page_tokens;
+    launch.query_heads = g_.query_heads;
+    launch.kv_heads = g_.kv_heads;
+    launch.head_dim = g_.head_dim;
+    launch.split_tokens = split_tokens_;
+    launch.maximum_splits = maximum_splits_;
+    launch.query_stride = query_stride;
+    launch.output_gated = g_.output_gated;
+    launch.output_kind = QLLM_OUT_BF16;
+    launch.stream = stream;
+    launch.device_positions = deferred_positions ? positions_ : nullptr;
+    status_check(qllm_attention_paged_q4h(&launch));
+  } else {
+    status_check(qllm_qkv_rope_batch(
+        query, query_stride, key, layer.query_norm, layer.key_norm,
+        first_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
+        g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+    status_check(qllm_store_kv_paged_f16_batch(
+        key, value, const_cast<const void* const*>(device_page_table_),
+        index, g_.kv_page_tokens, first_position, rows, g_.kv_heads,
+        g_.head_dim, stream));
+    qllm_f16_attention_launch launch{};
+    launch.query = query;
+    launch.device_pages = const_cast<const void* const*>(device_page_table_);
+    launch.output = attention_out;
+    launch.partial_maxima = partial_maxima_;
+    launch.partial_sums = partial_sums_;
+    launch.partial_outputs = partial_outputs_;
+    launch.first_context_tokens = first_position + 1U;
+    launch.rows = rows;
+    launch.device_page_layer = index;
+    launch.device_page_tokens = g_.kv_page_tokens;
+    launch.query_heads = g_.query_heads;
+    launch.kv_heads = g_.kv_heads;
+    launch.head_dim = g_.head_dim;
+    launch.split_tokens = split_tokens_;
+    launch.maximum_splits = maximum_splits_;
+    launch.query_stride = query_stride;
+    launch.output_gated = g_.output_gated;
+    launch.output_kind = QLLM_OUT_BF16;
+    launch.stream = stream;
+    status_check(qllm_attention_paged_f16(&launch));
+  }
+}
+
 void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                            std::uint32_t rows,
                                            std::uint32_t first_position,
@@ -768,74 +849,8 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
     status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
                                           hidden_bytes, projections, 3U, rows,
                                           stream));
-    if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-      if (deferred_positions)
-        status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
-            query_, query_stride, key_, value_, layer.query_norm,
-            layer.key_norm, const_cast<const void* const*>(device_page_table_),
-            index, g_.kv_page_tokens, positions_, rows, g_.query_heads,
-            g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
-            g_.rope_theta, 0, stream));
-      else
-        status_check(qllm_qkv_rope_cache_paged_q4h_batch(
-            query_, query_stride, key_, value_, layer.query_norm,
-            layer.key_norm, const_cast<const void* const*>(device_page_table_),
-            index, g_.kv_page_tokens, first_position, first_position, rows,
-            g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
-            g_.norm_epsilon, g_.rope_theta, 0, stream));
-      qllm_q4h_attention_launch launch{};
-      launch.query = query_;
-      launch.page_table = const_cast<const void* const*>(device_page_table_);
-      launch.output = attention_;
-      launch.partial_maxima = partial_maxima_;
-      launch.partial_sums = partial_sums_;
-      launch.partial_outputs = partial_outputs_;
-      launch.first_context_tokens = first_position + 1U;  // :7915
-      launch.rows = rows;
-      launch.full_attention_layer = index;
-      launch.page_tokens = g_.kv_page_tokens;
-      launch.query_heads = g_.query_heads;
-      launch.kv_heads = g_.kv_heads;
-      launch.head_dim = g_.head_dim;
-      launch.split_tokens = split_tokens_;
-      launch.maximum_splits = maximum_splits_;
-      launch.query_stride = query_stride;
-      launch.output_gated = g_.output_gated;
-      launch.output_kind = QLLM_OUT_BF16;
-      launch.stream = stream;
-      launch.device_positions = deferred_positions ? positions_ : nullptr;
-      status_check(qllm_attention_paged_q4h(&launch));
-    } else {
-      status_check(qllm_qkv_rope_batch(
-          query_, query_stride, key_, layer.query_norm, layer.key_norm,
-          first_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
-          g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
-      status_check(qllm_store_kv_paged_f16_batch(
-          key_, value_, const_cast<const void* const*>(device_page_table_),
-          index, g_.kv_page_tokens, first_position, rows, g_.kv_heads,
-          g_.head_dim, stream));
-      qllm_f16_attention_launch launch{};
-      launch.query = query_;
-      launch.device_pages = const_cast<const void* const*>(device_page_table_);
-      launch.output = attention_;
-      launch.partial_maxima = partial_maxima_;
-      launch.partial_sums = partial_sums_;
-      launch.partial_outputs = partial_outputs_;
-      launch.first_context_tokens = first_position + 1U;
-      launch.rows = rows;
-      launch.device_page_layer = index;
-      launch.device_page_tokens = g_.kv_page_tokens;
-      launch.query_heads = g_.query_heads;
-      launch.kv_heads = g_.kv_heads;
-      launch.head_dim = g_.head_dim;
-      launch.split_tokens = split_tokens_;
-      launch.maximum_splits = maximum_splits_;
-      launch.query_stride = query_stride;
-      launch.output_gated = g_.output_gated;
-      launch.output_kind = QLLM_OUT_BF16;
-      launch.stream = stream;
-      status_check(qllm_attention_paged_f16(&launch));
-    }
+    enqueue_attention(index, rows, first_position, deferred_positions, query_,
+                      key_, value_, attention_);
     status_check(qllm_fp4_gemm_bf16(&layer.output.descriptor, attention_,
                                     attention_bytes, hidden_, QLLM_OUT_F32,
                                     hidden_, rows, stream));
@@ -861,6 +876,196 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
   status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
                                  select_workspace_, select_workspace_bytes_,
                                  stream));
+}
+
+void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
+  if (rows <= prefill_rows_) return;
+  if (prefill_rows_)
+    throw std::runtime_error("prefill workspace is already allocated smaller");
+  const auto allocate = [this](std::size_t bytes) {
+    void* pointer{};
+    hip_check(hipMalloc(&pointer, bytes), "allocate prefill workspace");
+    allocations_.push_back(pointer);
+    return pointer;
+  };
+  const std::size_t n = rows;
+  const std::size_t query_width =
+      std::size_t{g_.query_heads} * g_.head_dim * (g_.output_gated ? 2U : 1U);
+  const std::size_t kv_width = std::size_t{g_.kv_heads} * g_.head_dim;
+  prefill_tokens_ = static_cast<std::uint32_t*>(allocate(n * 4U));
+  prefill_hidden_ = static_cast<float*>(allocate(n * g_.hidden * 4U));
+  prefill_normalized_ =
+      static_cast<std::uint16_t*>(allocate(n * g_.hidden * 2U));
+  prefill_query_ = static_cast<float*>(allocate(n * query_width * 4U));
+  prefill_key_ = static_cast<float*>(allocate(n * kv_width * 4U));
+  prefill_value_ = static_cast<float*>(allocate(n * kv_width * 4U));
+  prefill_attention_ = static_cast<std::uint16_t*>(
+      allocate(n * g_.query_heads * g_.head_dim * 2U));
+  prefill_gate_ = static_cast<float*>(allocate(n * g_.intermediate * 4U));
+  prefill_up_ = static_cast<float*>(allocate(n * g_.intermediate * 4U));
+  prefill_activation_ =
+      static_cast<std::uint16_t*>(allocate(n * g_.intermediate * 2U));
+  prefill_rows_ = rows;
+}
+
+Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    std::span<const std::uint32_t> tokens, std::uint32_t first_position,
+    const er::ProgramRequestContext& request) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto state =
+        std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+    if (tokens.empty() || tokens.size() > g_.max_context ||
+        first_position > g_.max_context - tokens.size() ||
+        (opaque_state && !state))
+      return {{er::ErrorCode::invalid_argument, "prompt rows are invalid"}, 0U};
+    if (!embedding_ready_ || !head_ready_ || attention_ops_ != g_.layers ||
+        ffn_ops_ != g_.layers)
+      return {{er::ErrorCode::invalid_argument, "target program is not prepared"},
+              0U};
+    for (const auto token : tokens)
+      if (token >= g_.vocabulary)
+        return {{er::ErrorCode::invalid_argument,
+                 "prompt token is outside the vocabulary"},
+                0U};
+    const auto count = static_cast<std::uint32_t>(tokens.size());
+    const std::uint32_t chunk_rows = std::min(count, prefill_chunk_rows());
+    ensure_prefill_workspace(prefill_rows_ ? prefill_rows_ : chunk_rows);
+    ensure_pages(first_position + count - 1U);
+    void* const stream = stream_;
+    const auto hip_stream = static_cast<hipStream_t>(stream_);
+    const std::size_t query_width =
+        std::size_t{g_.query_heads} * g_.head_dim * (g_.output_gated ? 2U : 1U);
+    const std::size_t kv_width = std::size_t{g_.kv_heads} * g_.head_dim;
+    const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
+    const bool feed_proposer = state && mtp_.ready;
+    if (state) {
+      state->draft_valid = false;
+      state->draft_predictions.clear();
+      state->mtp_length = first_position;
+    }
+
+    for (std::uint32_t done = 0; done < count;) {
+      const std::uint32_t rows = std::min(prefill_rows_, count - done);
+      const std::uint32_t position = first_position + done;
+      hip_check(hipMemcpyAsync(prefill_tokens_, tokens.data() + done, rows * 4U,
+                               hipMemcpyHostToDevice, hip_stream),
+                "upload prompt tokens");
+      status_check(qllm_fp4_embedding_batch(&embedding_.descriptor,
+                                            prefill_tokens_, prefill_hidden_,
+                                            rows, stream));
+      const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
+      for (std::uint32_t index = 0; index < g_.layers; ++index) {
+        const auto& layer = layers_[index];
+        status_check(qllm_rms_norm_batch(
+            prefill_hidden_, layer.input_norm, nullptr, prefill_normalized_,
+            g_.hidden, rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm,
+            stream));
+        const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+        const qllm_gemm_segment projections[3] = {
+            {prefill_query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+            {prefill_key_, kv_rows, QLLM_OUT_F32},
+            {prefill_value_, kv_rows, QLLM_OUT_F32}};
+        status_check(qllm_fp4_gemm_bf16_tall_split(
+            &layer.qkv.descriptor, prefill_normalized_, hidden_bytes,
+            projections, 3U, rows, stream));
+        // attention in row batches of the verify step's size: each batch sees
+        // the cache up to and including its own rows
+        for (std::uint32_t row = 0; row < rows; row += max_rows_) {
+          const std::uint32_t batch = std::min(max_rows_, rows - row);
+          enqueue_attention(index, batch, position + row, false,
+                            prefill_query_ + row * query_width,
+                            prefill_key_ + row * kv_width,
+                            prefill_value_ + row * kv_width,
+                            prefill_attention_ + row * attention_width);
+        }
+        status_check(qllm_fp4_gemm_bf16_tall(
+            &layer.output.descriptor, prefill_attention_,
+            std::size_t{rows} * attention_width * 2U, prefill_hidden_,
+            QLLM_OUT_F32, prefill_hidden_, rows, stream));
+        status_check(qllm_rms_norm_batch(
+            prefill_hidden_, layer.post_attention_norm, nullptr,
+            prefill_normalized_, g_.hidden, rows, g_.hidden, g_.norm_epsilon,
+            g_.zero_centered_norm, stream));
+        status_check(qllm_fp4_gemm_bf16_tall(
+            &layer.gate.descriptor, prefill_normalized_, hidden_bytes,
+            prefill_gate_, QLLM_OUT_F32, nullptr, rows, stream));
+        status_check(qllm_fp4_gemm_bf16_tall(
+            &layer.up.descriptor, prefill_normalized_, hidden_bytes, prefill_up_,
+            QLLM_OUT_F32, nullptr, rows, stream));
+        // silu(gate) * up with the verify step's bf16 rounding points; the
+        // result is exact in bf16, so the conversion moves bits only
+        status_check(qllm_silu_product(prefill_gate_, prefill_up_, prefill_gate_,
+                                       rows * g_.intermediate, 1, stream));
+        status_check(qllm_convert_f32_to_bf16_batch(
+            prefill_gate_, prefill_activation_,
+            std::size_t{rows} * g_.intermediate * 2U, rows, g_.intermediate,
+            g_.intermediate, stream));
+        status_check(qllm_fp4_gemm_bf16_tall(
+            &layer.down.descriptor, prefill_activation_,
+            std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_,
+            QLLM_OUT_F32, prefill_hidden_, rows, stream));
+      }
+      // the proposer sees (token at p + 1, target hidden at p) for every prompt
+      // position but the last, whose successor is not known yet
+      if (feed_proposer) {
+        const std::uint32_t pairs = done + rows == count ? rows - 1U : rows;
+        for (std::uint32_t row = 0; row < pairs; row += max_rows_) {
+          const std::uint32_t batch = std::min(max_rows_, pairs - row);
+          (void)run_mtp(*state, tokens.subspan(done + row + 1U, batch),
+                        prefill_hidden_ + std::size_t{row} * g_.hidden, false,
+                        nullptr, 0U, 0U);
+        }
+      }
+      done += rows;
+      if (done == count) {
+        // last row -> the verify step's buffers, then the head on that row
+        hip_check(hipMemcpyAsync(
+                      hidden_, prefill_hidden_ + std::size_t{rows - 1U} * g_.hidden,
+                      g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
+                  "retain the prompt's last hidden state");
+      }
+    }
+    status_check(qllm_rms_norm_batch(hidden_, final_norm_, nullptr, normalized_,
+                                     g_.hidden, 1U, g_.hidden, g_.norm_epsilon,
+                                     g_.zero_centered_norm, stream));
+    status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
+                                    std::size_t{g_.hidden} * 2U, logits_,
+                                    QLLM_OUT_F32, nullptr, 1U, stream));
+    status_check(qllm_argmax_batch(logits_, g_.vocabulary, 1U, argmax_tokens_,
+                                   select_workspace_, select_workspace_bytes_,
+                                   stream));
+    std::uint32_t predicted{};
+    hip_check(hipMemcpyAsync(&predicted, argmax_tokens_, sizeof(predicted),
+                             hipMemcpyDeviceToHost, hip_stream),
+              "copy the prompt's prediction");
+    hip_check(hipStreamSynchronize(hip_stream), "prompt prefill");
+    prefill_tokens_total_ += count;
+    if (state) {
+      state->synchronized_token = predicted;
+      if (feed_proposer) {
+        // the last pair, then the first drafts (as synchronize does)
+        const std::uint32_t last[1] = {predicted};
+        const auto sample_position = first_position + count;
+        auto draft = run_mtp(*state, last, hidden_, true, &request,
+                             sample_position, 1U);
+        if (!draft) throw std::runtime_error("prompt prefill produced no draft");
+        const auto reserved = request.parameters.find("reserved_context_tokens");
+        const auto context_limit =
+            reserved == request.parameters.end()
+                ? g_.max_context
+                : static_cast<std::uint32_t>(reserved->second);
+        if (state->mtp_length + 1U < context_limit)
+          extend_mtp_rollout(*state, request, std::move(*draft), context_limit);
+      } else {
+        state->mtp_length = first_position + count;
+      }
+    }
+    return {er::Status::success(), predicted};
+  } catch (const std::exception& error) {
+    return {{er::ErrorCode::internal, error.what()}, 0U};
+  }
 }
 
 er::Status Mi355DenseFp4Provider::run_target(const std::uint32_t* tokens,

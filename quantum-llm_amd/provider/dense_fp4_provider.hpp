@@ -182,6 +182,27 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   [[nodiscard]] std::map<std::string, std::uint64_t, std::less<>> telemetry()
       const;
   [[nodiscard]] er::ServiceContract service_contract() const;
+
+  // Prompt prefill: runs `tokens` (positions first_position ..) through the
+  // target in chunks of up to prefill_chunk_rows() rows - the linears on the
+  // tall-batch GEMM, attention and the K/V store in row batches of the verify
+  // step's size - and returns the greedy prediction for the position after
+  // the prompt.  With a request state the proposer is fed the prompt as the
+  // worker's feed does through synchronize_exact_decode_batch
+  // (runtime/tools/moe_vm_runner.cpp:682-745), and the first drafts are rolled
+  // out: the state is then ready for execute_exact_decode at
+  // first_position + tokens.size() with the prediction as guaranteed token.
+  struct PrefillResult final {
+    er::Status status;
+    std::uint32_t predicted{};
+  };
+  [[nodiscard]] PrefillResult prefill(
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      std::span<const std::uint32_t> tokens, std::uint32_t first_position,
+      const er::ProgramRequestContext& request);
+  [[nodiscard]] static constexpr std::uint32_t prefill_chunk_rows() noexcept {
+    return 1024U;
+  }
   [[nodiscard]] std::uint64_t weight_bytes() const noexcept {
     return weight_bytes_;
   }
@@ -220,6 +241,12 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       const float* previous_hidden, bool produce_logits,
       const er::ProgramRequestContext* request, std::uint32_t sample_position,
       std::uint32_t random_stream);
+  void enqueue_attention(std::uint32_t index, std::uint32_t rows,
+                         std::uint32_t first_position, bool deferred_positions,
+                         float* query, float* key, const float* value,
+                         std::uint16_t* attention_out);
+  // buffers for `rows` prompt rows at a time (allocated on first use)
+  void ensure_prefill_workspace(std::uint32_t rows);
   void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
                    bool produce_logits, std::uint32_t cache_position,
                    bool deferred_positions);
@@ -290,6 +317,19 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* mtp_last_hidden_{};
   float* mtp_logits_{};
   std::uint32_t* mtp_argmax_{};
+  // prompt prefill workspace
+  std::uint32_t prefill_rows_{};
+  std::uint32_t* prefill_tokens_{};
+  float* prefill_hidden_{};
+  std::uint16_t* prefill_normalized_{};   // bf16 [rows, hidden]
+  float* prefill_query_{};
+  float* prefill_key_{};
+  float* prefill_value_{};
+  std::uint16_t* prefill_attention_{};    // bf16 [rows, query_heads * head_dim]
+  float* prefill_gate_{};
+  float* prefill_up_{};
+  std::uint16_t* prefill_activation_{};   // bf16 [rows, intermediate]
+  std::uint64_t prefill_tokens_total_{};
   std::uint32_t* mtp_positions_{};      // cache, rotary, context, draft slot
   std::uint32_t* mtp_draft_tokens_{};
   std::vector<void*> mtp_graphs_;       // hipGraphExec_t at 2*rows + chained

@@ -253,6 +253,19 @@ extern "C" int32_t qllm_provider_synchronize(qllm_provider* provider,
       *provider->exact, provider->state, batch));
 }
 
+extern "C" int32_t qllm_provider_prefill(qllm_provider* provider,
+                                         const uint32_t* tokens, uint32_t count,
+                                         uint32_t first_position,
+                                         uint32_t* predicted) {
+  if (!provider || !tokens || !count || !predicted)
+    return fail(QLLM_INVALID_ARGUMENT, "prompt arguments are invalid");
+  const auto result = provider->provider->prefill(
+      provider->state, {tokens, count}, first_position, provider->request);
+  if (!result.status.ok()) return from_status(result.status);
+  *predicted = result.predicted;
+  return QLLM_OK;
+}
+
 extern "C" int32_t qllm_provider_set_drafts(
     qllm_provider* provider, const uint32_t* draft_tokens, uint32_t draft_count,
     const uint32_t* distribution_counts, const uint32_t* distribution_tokens,

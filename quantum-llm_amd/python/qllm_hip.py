@@ -87,6 +87,8 @@ SIGNATURES = {
     "qllm_fp4_gemv_q8_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_fp4_gemm_bf16": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
     "qllm_fp4_gemm_bf16_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_bf16_tall": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_bf16_tall_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_swiglu_bf16": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
     "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32, c_uint32]),

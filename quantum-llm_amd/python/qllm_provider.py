@@ -67,6 +67,7 @@ SIGNATURES = {
     "qllm_sampling_rejection": (c_int32, [c_uint32, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_double, c_double, POINTER(c_int32), POINTER(c_uint32), POINTER(c_double), POINTER(c_double)]),
     "qllm_sampling_counter_uniform": (c_double, [c_uint64, c_uint32, c_uint32, c_uint32]),
     "qllm_provider_create_from_artifact": (c_void_p, [c_char_p, c_uint32, c_uint32, c_char_p, c_uint32]),
+    "qllm_provider_prefill": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, POINTER(c_uint32)]),
     "qllm_sha256": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_sha256_portable": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_model_descriptor_parse": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
@@ -164,6 +165,15 @@ class Provider:
                       min_p_ppm=0, seed=0):
         _check(self.lib.qllm_provider_begin_request(
             self.handle, temperature_ppm, top_p_ppm, top_k, min_p_ppm, seed))
+
+    def prefill(self, tokens, first_position=0):
+        """Prompt prefill; returns the greedy prediction after the prompt."""
+        import numpy as np
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        predicted = c_uint32()
+        _check(self.lib.qllm_provider_prefill(self.handle, tokens.ctypes.data, tokens.size,
+                                              first_position, ctypes.byref(predicted)))
+        return predicted.value
 
     def synchronize(self, token, position):
         _check(self.lib.qllm_provider_synchronize(self.handle, token, position))

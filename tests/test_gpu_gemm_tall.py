@@ -1,0 +1,117 @@
+"""The FP4 GEMM for tall batches (prompt prefill) against the CPU oracle, and
+against the small-batch kernel on the same rows."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as gu
+import oracle_lib as ol
+import qllm_hip as qh
+import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def tall(device, codes, scales, scheme, rows, padded, act, out_kind=qh.OUT_F32,
+         residual=None):
+    batch = act.shape[0]
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    matrix, keep = qh.prepack(qh.fp4_matrix(d_codes, d_scales, rows, padded, padded, scheme),
+                              device)
+    dtype = torch.bfloat16 if out_kind == qh.OUT_BF16 else torch.float32
+    out = torch.zeros((batch, rows), dtype=dtype, device=device)
+    d_residual = None if residual is None else gu.device_tensor(residual, device)
+    qh.call("qllm_fp4_gemm_bf16_tall", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(out), out_kind, qh.ptr(d_residual), batch, None)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("rows,padded,batch", [
+    (256, 64, 128), (300, 1024, 9), (1024, 5120, 200), (77, 128, 333),
+    (2048, 1024, 1024), (512, 8192, 130)])
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_tall_gemm_matches_oracle(device, scheme, rows, padded, batch):
+    """Ragged shapes: batches that are no multiple of 128, weight rows that are
+    no multiple of 256 or 32, a single chunk of K."""
+    rng = np.random.default_rng(rows + batch)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
+    got = tall(device, codes, scales, scheme, rows, padded, act)
+    gu.assert_close(got, want, what="tall GEMM")
+    if scheme == ol.SCALE_UE8M0_BLOCK32:
+        # exact bf16 operands: only the F32 summation order separates the two
+        error = np.abs(got - want).max() / np.abs(want).max()
+        assert error < 2e-6 * np.sqrt(padded)
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_tall_gemm_residual_and_bf16_output(device, scheme):
+    rng = np.random.default_rng(5)
+    rows, padded, batch = 640, 1024, 150
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    residual = rng.standard_normal((batch, rows)).astype(np.float32)
+    want = ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act)
+    got = tall(device, codes, scales, scheme, rows, padded, act, residual=residual)
+    gu.assert_close(got, want + residual, what="tall GEMM + residual")
+    got = tall(device, codes, scales, scheme, rows, padded, act, out_kind=qh.OUT_BF16)
+    gu.assert_close(got, want, rtol=1e-2, atol=1e-3, what="tall GEMM bf16")
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_tall_gemm_rows_equal_the_small_batch_kernel(device, scheme):
+    """The same five rows through the verify-step kernel and through the tall
+    one (as rows 123..127 of a batch of 128)."""
+    rng = np.random.default_rng(8)
+    rows, padded = 1024, 5120
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((128, padded)).astype(np.float32))
+    small = gu.gemm(device, codes, scales, scheme, rows, padded, act[123:128])
+    big = tall(device, codes, scales, scheme, rows, padded, act)[123:128]
+    gu.assert_close(big, small, rtol=2e-3, atol=2e-4, what="tall vs small-batch rows")
+
+
+def test_tall_split_outputs(device):
+    rng = np.random.default_rng(9)
+    scheme, padded, batch = ol.SCALE_F16_BLOCK16, 1024, 140
+    parts = [512, 64, 64]
+    rows = sum(parts)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    whole = tall(device, codes, scales, scheme, rows, padded, act)
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    matrix, keep = qh.prepack(qh.fp4_matrix(d_codes, d_scales, rows, padded, padded, scheme),
+                              device)
+    outs = [torch.zeros((batch, part), device=device) for part in parts]
+    segments = (qh.GemmSegment * 3)(*[qh.GemmSegment(qh.ptr(o), part, qh.OUT_F32)
+                                      for o, part in zip(outs, parts)])
+    qh.call("qllm_fp4_gemm_bf16_tall_split", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            segments, 3, batch, None)
+    torch.cuda.synchronize()
+    first = 0
+    for out, part in zip(outs, parts):
+        assert np.array_equal(out.cpu().numpy(), whole[:, first:first + part])
+        first += part
+    bad = (qh.GemmSegment * 2)(qh.GemmSegment(qh.ptr(outs[0]), 520, qh.OUT_F32),
+                               qh.GemmSegment(qh.ptr(outs[1]), 120, qh.OUT_F32))
+    with pytest.raises(qh.QllmError, match="multiples of 32"):
+        qh.call("qllm_fp4_gemm_bf16_tall_split", matrix, qh.ptr(d_act), d_act.numel() * 2,
+                bad, 2, batch, None)
+
+
+def test_tall_gemm_rejects_row_major(device):
+    rng = np.random.default_rng(1)
+    codes, scales = synth.fp4_matrix(rng, 64, 64, 0)
+    d = [gu.device_tensor(x, device) for x in (codes, scales)]
+    act = torch.zeros((16, 64), dtype=torch.bfloat16, device=device)
+    out = torch.zeros((16, 64), device=device)
+    matrix = qh.fp4_matrix(d[0], d[1], 64, 64, 64, 0)
+    with pytest.raises(qh.QllmError, match="invalid tall"):
+        qh.call("qllm_fp4_gemm_bf16_tall", matrix, qh.ptr(act), act.numel() * 2,
+                qh.ptr(out), qh.OUT_F32, None, 16, None)
