@@ -165,7 +165,7 @@ def measure_decode_cycle(qp, np, rows, steps, warmup):
 
 def measure_prefill(qp, np, prompt_tokens):
     """Prompt prefill of the same model: `prompt_tokens` synthetic tokens from
-    position 0 - the linears on the tall-batch GEMM (1024 rows at a time),
+    position 0 - the linears on the tall-batch GEMM (2048 rows at a time),
     attention and the Q4H store in row batches of five - timed from the call
     to the prediction of the token after the prompt (time to first token)."""
     geometry = dict(MODEL)
@@ -175,7 +175,7 @@ def measure_prefill(qp, np, prompt_tokens):
     provider.prepare_exact_decode("decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2")
     rng = np.random.default_rng(11)
     tokens = rng.integers(0, MODEL["vocabulary"], prompt_tokens).astype(np.uint32)
-    provider.prefill(tokens[:min(prompt_tokens, 1024)], 0)      # warm-up, allocates
+    provider.prefill(tokens[:min(prompt_tokens, 2048)], 0)      # warm-up, allocates
     provider.synchronize_stream()
     begin = time.perf_counter()
     provider.prefill(tokens, 0)

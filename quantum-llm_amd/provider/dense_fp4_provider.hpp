@@ -201,7 +201,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       std::span<const std::uint32_t> tokens, std::uint32_t first_position,
       const er::ProgramRequestContext& request);
   [[nodiscard]] static constexpr std::uint32_t prefill_chunk_rows() noexcept {
-    return 1024U;
+    return 2048U;
   }
   [[nodiscard]] std::uint64_t weight_bytes() const noexcept {
     return weight_bytes_;
