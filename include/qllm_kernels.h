@@ -348,6 +348,17 @@ typedef struct qllm_q4h_attention_launch {
  * head_dim in {128, 256}, page_tokens % 64 == 0, split_tokens % 64 == 0.
  * The pages must hold every 64-token tile that overlaps the context. */
 int32_t qllm_attention_paged_q4h(const qllm_q4h_attention_launch* launch);
+/* Many micro-batches in one launch (prompt prefill): the launch's `rows` rows
+ * are attended in batches of `batch_rows` consecutive rows, batch b exactly as
+ * a launch of its own with first_context_tokens + b * batch_rows would be
+ * (row r of the whole attends tokens [0, first_context_tokens + r)), all
+ * batches side by side in one grid.  query, output and the partial buffers
+ * hold `rows` rows; batch_rows * (query_heads/kv_heads) <= 48 (32 at head_dim
+ * 256); rows <= 65535; device_positions must be NULL.  No counterpart in the
+ * reference, whose prefill attention is a kernel of its own
+ * (transformer_kernels.cu:9906-10153). */
+int32_t qllm_attention_paged_q4h_batched(const qllm_q4h_attention_launch* launch,
+                                         uint32_t batch_rows);
 
 /* ---- attention: exact F16 paged cache ---------------------------------------- */
 

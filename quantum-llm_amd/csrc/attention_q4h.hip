@@ -25,6 +25,7 @@
 // merges the splits.  Maxima are kept in the log2 domain.
 #include "attention_common.hpp"
 
+#include <algorithm>
 #include <utility>
 
 namespace qllm {
@@ -76,6 +77,10 @@ struct SplitArgs {
   uint32_t split_tokens;
   uint32_t maximum_splits;
   const uint32_t* device_positions;  // optional: [2] = first_context_tokens
+  // Batched launch (prompt prefill): workgroups of grid layer z take rows
+  // [z * batch_rows, +batch_rows) of `rows`, each layer a launch of its own as
+  // far as the kernel is concerned.  0 = one batch holds all rows.
+  uint32_t batch_rows;
 };
 
 
@@ -210,7 +215,23 @@ __device__ __forceinline__ uint32_t lds_address(const void* pointer) {
 // loads fly while the matrix cores and the softmax work on registers.
 template <int D, int RT>
 __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
-    const SplitArgs args) {
+    const SplitArgs launch_args) {
+  // a batched launch narrows the arguments to the batch of this grid layer
+  SplitArgs args = launch_args;
+  if (launch_args.batch_rows) {
+    const uint32_t first_row = blockIdx.z * launch_args.batch_rows;
+    const size_t first_partial = static_cast<size_t>(first_row) *
+                                 launch_args.maximum_splits *
+                                 launch_args.query_heads;
+    args.rows = min(launch_args.batch_rows, launch_args.rows - first_row);
+    args.first_context_tokens = launch_args.first_context_tokens + first_row;
+    args.query = launch_args.query + static_cast<size_t>(first_row) *
+                                         launch_args.query_heads *
+                                         launch_args.query_stride;
+    args.partial_maxima = launch_args.partial_maxima + first_partial;
+    args.partial_sums = launch_args.partial_sums + first_partial;
+    args.partial_outputs = launch_args.partial_outputs + first_partial * D;
+  }
   constexpr int KSTEPS = D / 64;      // int8 MFMA k-steps over head_dim
   constexpr int DT = D / 16;          // 16-wide tiles of head_dim
   constexpr int ROW = D / 2;          // bytes of codes per token
@@ -1086,6 +1107,73 @@ extern "C" int32_t qllm_quantize_gqa_queries_q8(
                                as_stream(stream)>>>(
       query, query_stride, q8, query_scales, query_heads, head_dim);
   return launched("GQA query Q8 quantization");
+}
+
+extern "C" int32_t qllm_attention_paged_q4h_batched(
+    const qllm_q4h_attention_launch* launch, uint32_t batch_rows) {
+  if (!launch || !launch->query || !launch->page_table || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      !launch->first_context_tokens || !launch->rows || !batch_rows ||
+      launch->device_positions || !launch->page_tokens ||
+      launch->page_tokens % 64u || !launch->query_heads || !launch->kv_heads ||
+      launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      launch->split_tokens % 64u || !launch->maximum_splits ||
+      launch->maximum_splits > kCombineSplitCapacity ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->rows > 65535u ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid batched Q4H paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t row_tiles = (std::min(batch_rows, launch->rows) * group + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched Q4H paged attention: batch_rows * (query_heads/kv_heads) "
+                "exceeds 48 (32 at head_dim 256)");
+  const uint32_t batches = (launch->rows + batch_rows - 1u) / batch_rows;
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      !launch->split_tokens
+          ? launch->maximum_splits
+          : (last_context + launch->split_tokens - 1u) / launch->split_tokens;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched Q4H paged attention: context needs more splits than "
+                "maximum_splits");
+  SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.page_table = launch->page_table;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.layer = launch->full_attention_layer;
+  args.page_tokens = launch->page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  args.batch_rows = batch_rows;
+  const dim3 grid(launch->kv_heads, splits, batches);
+  const hipStream_t stream = as_stream(launch->stream);
+  int32_t status = launch->head_dim == 128u
+                       ? launch_split<128>(args, row_tiles, grid, stream)
+                       : launch_split<256>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  // partials are laid out by global row, which is what the combine indexes
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, nullptr, stream);
 }
 
 extern "C" int32_t qllm_attention_paged_q4h(

@@ -329,6 +329,11 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* prefill_gate_{};
   float* prefill_up_{};
   std::uint16_t* prefill_activation_{};   // bf16 [rows, intermediate]
+  // split partials of the batched prompt attention: [rows, splits, heads(, d)]
+  std::uint32_t prefill_splits_{};
+  float* prefill_partial_maxima_{};
+  float* prefill_partial_sums_{};
+  float* prefill_partial_outputs_{};
   std::uint64_t prefill_tokens_total_{};
   std::uint32_t* mtp_positions_{};      // cache, rotary, context, draft slot
   std::uint32_t* mtp_draft_tokens_{};

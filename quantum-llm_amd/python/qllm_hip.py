@@ -106,6 +106,7 @@ SIGNATURES = {
     "qllm_store_kv_paged_q4h_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_quantize_gqa_queries_q8": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_q4h": (c_int32, [POINTER(Q4hAttentionLaunch)]),
+    "qllm_attention_paged_q4h_batched": (c_int32, [POINTER(Q4hAttentionLaunch), c_uint32]),
     "qllm_store_kv_paged_f16_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),
     "qllm_q8_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),

@@ -168,3 +168,48 @@ def test_attention_rejects_unsupported_geometry(device):
     with pytest.raises(qh.QllmError) as error:   # 5 rows x 10 grouped heads > 48
         qh.call("qllm_attention_paged_q4h", launch)
     assert error.value.code == 4
+
+
+@pytest.mark.parametrize("total,first,Q,KV,d,gated,batch", [
+    (23, 300, 64, 8, 128, False, 5),     # last batch has 3 rows
+    (40, 1, 8, 2, 256, True, 5),         # the prompt starts the cache; d = 256
+    (64, 4000, 64, 8, 128, False, 6),    # six rows per batch (48 matrix rows)
+    (7, 70, 16, 8, 128, False, 1)])      # one row per batch
+def test_batched_launch_equals_one_launch_per_batch(device, total, first, Q, KV, d,
+                                                     gated, batch):
+    """Prompt prefill attends `total` consecutive rows in one launch, in
+    batches of `batch` rows that each see the cache up to their own rows: bit
+    for bit what one launch per batch computes, and the oracle's attention."""
+    rng = np.random.default_rng(total + first)
+    page_tokens, splits = 64, 8
+    tokens = first + total - 1
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, page_tokens, 1, 0)
+    stride = d * (2 if gated else 1)
+    query = ol.bf16_round(rng.standard_normal((total, Q, stride)).astype(np.float32))
+    d_pages = [gu.device_tensor(page, device) for page in pages]
+    table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
+                         device=device)
+    d_query = gu.device_tensor(query, device)
+    maxima = torch.zeros((total, splits, Q), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((total, splits, Q, d), device=device)
+    out = torch.zeros((total, Q, d), device=device)
+    launch = qh.Q4hAttentionLaunch(
+        qh.ptr(d_query), 0, 0, qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), first, total, 0, page_tokens, Q, KV, d, 0, splits, stride,
+        int(gated), qh.OUT_F32, None)
+    qh.call("qllm_attention_paged_q4h_batched", launch, batch)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for row in range(0, total, batch):
+        rows = min(batch, total - row)
+        single = gu.q4h_attention(device, pages, query[row:row + rows], rows, Q, KV, d,
+                                  first + row, page_tokens, 0, gated, balanced_splits=splits)
+        assert np.array_equal(got[row:row + rows], single), row
+    shape = ol.AttentionShape(total, Q, KV, d, first, page_tokens, 0, int(gated))
+    gu.assert_close(got, ol.attention_q4h(shape, query, pages, "f64"), what="batched attention")
+    if total * (Q // KV) > (32 if d == 256 else 48):
+        with pytest.raises(qh.QllmError, match="exceeds"):     # one batch of everything
+            qh.call("qllm_attention_paged_q4h_batched", launch, total)
