@@ -158,7 +158,7 @@ struct Operand<kSchemeF16> {
 // consecutive positions within one XCD's share of the grid, so that the tile's
 // weights are fetched from HBM once per XCD rather than once per workgroup.
 template <int SCHEME>
-__global__ __launch_bounds__(kWaves * 64) void fp4_gemm_tall_kernel(
+__global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
     const TallArgs args) {
   using Op = Operand<SCHEME>;
   using Vector = typename Op::Vector;
