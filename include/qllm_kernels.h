@@ -401,6 +401,9 @@ typedef struct qllm_f16_attention_launch {
 } qllm_f16_attention_launch;
 
 int32_t qllm_attention_paged_f16(const qllm_f16_attention_launch* launch);
+/* The batched form for prompt prefill, as qllm_attention_paged_q4h_batched. */
+int32_t qllm_attention_paged_f16_batched(const qllm_f16_attention_launch* launch,
+                                         uint32_t batch_rows);
 
 /* ---- attention: Q8 paged cache (the proposer's) ------------------------------- */
 

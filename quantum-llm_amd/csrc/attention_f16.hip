@@ -132,6 +132,9 @@ struct F16SplitArgs {
   uint32_t maximum_splits;
   size_t page_offset;   // Q8: byte offset of the layer inside a page
   const uint32_t* device_positions;  // optional: [2] = first_context_tokens
+  // Batched launch (prompt prefill): grid layer z takes rows
+  // [z * batch_rows, +batch_rows) of `rows`.  0 = one batch holds all rows.
+  uint32_t batch_rows;
 };
 
 constexpr uint32_t kF16Tile = 32;  // tokens per wave step
@@ -150,7 +153,23 @@ constexpr uint32_t kF16Tile = 32;  // tokens per wave step
 // Q8 = the cache holds int8 codes and per-record scales instead of binary16.
 template <int D, int RT, bool Q8>
 __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
-    const F16SplitArgs args) {
+    const F16SplitArgs launch_args) {
+  // a batched launch narrows the arguments to the batch of this grid layer
+  F16SplitArgs args = launch_args;
+  if (launch_args.batch_rows) {
+    const uint32_t first_row = blockIdx.z * launch_args.batch_rows;
+    const size_t first_partial = static_cast<size_t>(first_row) *
+                                 launch_args.maximum_splits *
+                                 launch_args.query_heads;
+    args.rows = min(launch_args.batch_rows, launch_args.rows - first_row);
+    args.first_context_tokens = launch_args.first_context_tokens + first_row;
+    args.query = launch_args.query + static_cast<size_t>(first_row) *
+                                         launch_args.query_heads *
+                                         launch_args.query_stride;
+    args.partial_maxima = launch_args.partial_maxima + first_partial;
+    args.partial_sums = launch_args.partial_sums + first_partial;
+    args.partial_outputs = launch_args.partial_outputs + first_partial * D;
+  }
   constexpr int KSTEPS = D / 32;  // k-steps of the score MFMA over head_dim
   constexpr int DT = D / 16;      // 16-wide tiles of head_dim
   constexpr int GR = D / 8;       // 16-byte granules per V row
@@ -536,6 +555,73 @@ extern "C" int32_t qllm_attention_paged_f16(
   args.split_tokens = launch->split_tokens;
   args.maximum_splits = launch->maximum_splits;
   const dim3 grid(launch->kv_heads, splits);
+  const hipStream_t stream = as_stream(launch->stream);
+  const int32_t status =
+      launch->head_dim == 128u ? launch_f16_split<128>(args, row_tiles, grid, stream)
+                               : launch_f16_split<256>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, nullptr, stream);
+}
+
+extern "C" int32_t qllm_attention_paged_f16_batched(
+    const qllm_f16_attention_launch* launch, uint32_t batch_rows) {
+  if (!launch || !launch->query || !launch->device_pages || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      !launch->first_context_tokens || !launch->rows || !batch_rows ||
+      !launch->device_page_tokens || launch->device_page_tokens % kF16Tile ||
+      !launch->query_heads || !launch->kv_heads ||
+      launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      launch->split_tokens % kF16Tile || !launch->maximum_splits ||
+      launch->maximum_splits > 2048u ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->rows > 65535u ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid batched F16 paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t row_tiles =
+      ((batch_rows < launch->rows ? batch_rows : launch->rows) * group + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched F16 paged attention: batch_rows * (query_heads/kv_heads) "
+                "exceeds 48 (32 at head_dim 256)");
+  const uint32_t batches = (launch->rows + batch_rows - 1u) / batch_rows;
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      launch->split_tokens
+          ? (last_context + launch->split_tokens - 1u) / launch->split_tokens
+          : launch->maximum_splits;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched F16 paged attention: context needs more splits than "
+                "maximum_splits");
+  F16SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.pages = launch->device_pages;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.layer = launch->device_page_layer;
+  args.page_tokens = launch->device_page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  args.batch_rows = batch_rows;
+  const dim3 grid(launch->kv_heads, splits, batches);
   const hipStream_t stream = as_stream(launch->stream);
   const int32_t status =
       launch->head_dim == 128u ? launch_f16_split<128>(args, row_tiles, grid, stream)

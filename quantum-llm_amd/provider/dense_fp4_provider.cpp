@@ -905,7 +905,7 @@ void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
   prefill_up_ = static_cast<float*>(allocate(n * g_.intermediate * 4U));
   prefill_activation_ =
       static_cast<std::uint16_t*>(allocate(n * g_.intermediate * 2U));
-  if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
+  {
     // fewer splits than the verify step: the row batches of a chunk already
     // fill the GPU, and the partials are per row
     prefill_splits_ = std::min<std::uint32_t>(maximum_splits_, 8U);
@@ -1014,14 +1014,38 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.stream = stream;
           status_check(qllm_attention_paged_q4h_batched(&launch, max_rows_));
         } else {
-          for (std::uint32_t row = 0; row < rows; row += max_rows_) {
-            const std::uint32_t batch = std::min(max_rows_, rows - row);
-            enqueue_attention(index, batch, position + row, false,
-                              prefill_query_ + row * query_width,
-                              prefill_key_ + row * kv_width,
-                              prefill_value_ + row * kv_width,
-                              prefill_attention_ + row * attention_width);
-          }
+          const std::uint32_t query_stride =
+              g_.head_dim * (g_.output_gated ? 2U : 1U);
+          const auto pages = const_cast<const void* const*>(device_page_table_);
+          status_check(qllm_qkv_rope_batch(
+              prefill_query_, query_stride, prefill_key_, layer.query_norm,
+              layer.key_norm, position, rows, g_.query_heads, g_.kv_heads,
+              g_.head_dim, g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0,
+              stream));
+          status_check(qllm_store_kv_paged_f16_batch(
+              prefill_key_, prefill_value_, pages, index, g_.kv_page_tokens,
+              position, rows, g_.kv_heads, g_.head_dim, stream));
+          qllm_f16_attention_launch launch{};
+          launch.query = prefill_query_;
+          launch.device_pages = pages;
+          launch.output = prefill_attention_;
+          launch.partial_maxima = prefill_partial_maxima_;
+          launch.partial_sums = prefill_partial_sums_;
+          launch.partial_outputs = prefill_partial_outputs_;
+          launch.first_context_tokens = position + 1U;
+          launch.rows = rows;
+          launch.device_page_layer = index;
+          launch.device_page_tokens = g_.kv_page_tokens;
+          launch.query_heads = g_.query_heads;
+          launch.kv_heads = g_.kv_heads;
+          launch.head_dim = g_.head_dim;
+          launch.split_tokens = 0U;
+          launch.maximum_splits = prefill_splits_;
+          launch.query_stride = query_stride;
+          launch.output_gated = g_.output_gated;
+          launch.output_kind = QLLM_OUT_BF16;
+          launch.stream = stream;
+          status_check(qllm_attention_paged_f16_batched(&launch, max_rows_));
         }
         status_check(qllm_fp4_gemm_bf16_tall(
             &layer.output.descriptor, prefill_attention_,

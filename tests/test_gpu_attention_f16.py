@@ -130,3 +130,35 @@ def test_f16_attention_rejects_unsupported_geometry(device):
         run_case(device, rng, 40, 3, 32, 2, 32, 32, 32, False)
     with pytest.raises(qh.QllmError):   # 6 rows x 8 heads per KV head = 3 tiles, 4th row tile
         run_case(device, rng, 40, 7, 8, 1, 128, 32, 32, False)
+
+
+def test_batched_launch_equals_one_launch_per_batch(device):
+    """All row batches of a prompt chunk in one launch: bit for bit what one
+    launch per batch computes."""
+    rng = np.random.default_rng(77)
+    total, first, Q, KV, d, page_tokens, splits, batch = 23, 200, 16, 4, 128, 64, 8, 5
+    tokens = first + total - 1
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.f16_pages(keys, values, page_tokens, 1, 0)
+    query = ol.bf16_round(rng.standard_normal((total, Q, d)).astype(np.float32))
+    d_pages = [gu.device_tensor(page, device) for page in pages]
+    table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
+                         device=device)
+    d_query = gu.device_tensor(query, device)
+    maxima = torch.zeros((total, splits, Q), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((total, splits, Q, d), device=device)
+    out = torch.zeros((total, Q, d), device=device)
+    launch = qh.F16AttentionLaunch(
+        qh.ptr(d_query), qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), first, total, 0, page_tokens, Q, KV, d, 0, splits, d, 0,
+        qh.OUT_F32, None)
+    qh.call("qllm_attention_paged_f16_batched", launch, batch)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for row in range(0, total, batch):
+        rows = min(batch, total - row)
+        single = gu.f16_attention(device, pages, query[row:row + rows], rows, Q, KV, d,
+                                  first + row, page_tokens, 0, False, balanced_splits=splits)
+        assert np.array_equal(got[row:row + rows], single), row
