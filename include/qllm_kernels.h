@@ -157,6 +157,19 @@ int32_t qllm_fp4_gemm_bf16_split(const qllm_fp4_matrix* matrix,
                                  uint32_t segment_count, uint32_t batch,
                                  void* stream);
 
+/* The same product with K cut over k_splits workgroups per tile (tiled layout
+ * only, 1 <= k_splits <= 16): partials f32 [k_splits][batch][rows], split s
+ * holding the sum over its share of the 64-column chunks.  For matrices with
+ * too few rows to occupy the GPU (o and down projections); the consumer adds
+ * the partials in index order (qllm_rms_norm_residual_batch does), which
+ * keeps the result independent of the launch's timing.  The reference has one
+ * thread block per output row group and no such cut
+ * (transformer_kernels.cu:7559-7593). */
+int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,
+                                   const void* input, size_t input_bytes,
+                                   float* partials, uint32_t k_splits,
+                                   uint32_t batch, void* stream);
+
 /* Gate and up projections of one SwiGLU block in a single pass over a shared
  * BF16 input: out[m,n] = bf16(bf16(silu(gate[m,n])) * up[m,n]) stored as
  * bf16 [batch, rows].  Fuses two qllm_fp4_gemm_bf16 calls with silu_product
@@ -205,6 +218,20 @@ int32_t qllm_rms_norm_batch(const float* input, const float* weight,
                             uint32_t bf16_padded_columns, uint32_t rows,
                             uint32_t elements, float epsilon,
                             int32_t zero_centered, void* stream);
+
+/* The residual add of a projection computed as K-split partials
+ * (qllm_fp4_gemm_bf16_partial) folded into the RMSNorm that follows:
+ * hidden[r] += partials[0][r] + ... + partials[count-1][r] (in that order;
+ * partials f32 [count][rows][elements]), output_bf16[r] = RMSNorm(hidden[r]).
+ * Replaces add_kernel + rms_batch_kernel of the reference
+ * (transformer_kernels.cu:2522-2528, 2469-2503) for that case.  elements % 4
+ * == 0, at most 16384; pointers 16-byte aligned; 1 <= count <= 16. */
+int32_t qllm_rms_norm_residual_batch(float* hidden, const float* partials,
+                                     uint32_t partial_count,
+                                     const float* weight, void* output_bf16,
+                                     uint32_t rows, uint32_t elements,
+                                     float epsilon, int32_t zero_centered,
+                                     void* stream);
 
 /* Two normalisations into one bf16 batch: output row r, of 2 * elements
  * columns, is [RMSNorm(first[r]) | RMSNorm(second[r])], each half with its own

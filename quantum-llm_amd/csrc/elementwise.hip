@@ -172,10 +172,16 @@ __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
 // One row of up to 16384 elements (a multiple of four) on 1024 threads:
 // `out_f32` / `out_bf16` point at the row's outputs (either may be null) and
 // bf16 columns [elements, bf16_columns) are zeroed.
+// With `partial_count` > 0 the row normalised is input_row + partials[0] +
+// partials[1] + ... (added in that order; partial p of the row lies
+// `partial_stride` floats after partial p - 1) and that sum is also written
+// back to `sum_out`.
 __device__ __forceinline__ void rms_norm_row_wide(
     const float* input_row, const float* weight, float* out_f32,
     uint16_t* out_bf16, uint32_t bf16_columns, uint32_t elements,
-    float epsilon, bool zero_centered, float* scratch) {
+    float epsilon, bool zero_centered, float* scratch,
+    const float* partial_row = nullptr, uint32_t partial_count = 0u,
+    size_t partial_stride = 0u, float* sum_out = nullptr) {
   const float4* x = reinterpret_cast<const float4*>(input_row);
   const uint32_t vectors = elements / 4u;
   // the row and its weights are fetched together, before the reduction
@@ -189,6 +195,20 @@ __device__ __forceinline__ void rms_norm_row_wide(
     factors[slot] = make_float4(1.f, 1.f, 1.f, 1.f);
     if (weight && index < vectors)
       factors[slot] = reinterpret_cast<const float4*>(weight)[index];
+  }
+  if (partial_count) {
+#pragma unroll
+    for (int slot = 0; slot < 4; ++slot) {
+      const uint32_t index = slot * 1024u + threadIdx.x;
+      if (index >= vectors) continue;
+      for (uint32_t p = 0; p < partial_count; ++p) {
+        const float4 part =
+            reinterpret_cast<const float4*>(partial_row + p * partial_stride)[index];
+        values[slot].x += part.x; values[slot].y += part.y;
+        values[slot].z += part.z; values[slot].w += part.w;
+      }
+      reinterpret_cast<float4*>(sum_out)[index] = values[slot];
+    }
   }
 #pragma unroll
   for (int slot = 0; slot < 4; ++slot) {
@@ -238,6 +258,22 @@ __global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
       output_f32 ? output_f32 + row * elements : nullptr,
       output_bf16 ? output_bf16 + row * bf16_padded_columns : nullptr,
       bf16_padded_columns, elements, epsilon, zero_centered, scratch);
+}
+
+// hidden[r] += partials[0][r] + ... + partials[count-1][r], then its RMSNorm in
+// bf16: the residual add of a projection whose K was cut over workgroups
+// (qllm_fp4_gemm_bf16_partial) folded into the norm that follows it.
+__global__ __launch_bounds__(1024) void rms_norm_residual_kernel(
+    float* hidden, const float* partials, uint32_t partial_count,
+    const float* weight, uint16_t* output_bf16, uint32_t elements,
+    float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  rms_norm_row_wide(hidden + row * elements, weight, nullptr,
+                    output_bf16 + row * elements, elements, elements, epsilon,
+                    zero_centered, scratch, partials + row * elements,
+                    partial_count, static_cast<size_t>(gridDim.x) * elements,
+                    hidden + row * elements);
 }
 
 // Row r of the output is [RMSNorm(first[r]) | RMSNorm(second[r])] in bf16:
@@ -408,6 +444,24 @@ extern "C" int32_t qllm_rms_norm_batch(const float* input, const float* weight,
         input, weight, output_f32, static_cast<uint16_t*>(output_bf16),
         bf16_padded_columns, elements, epsilon, zero_centered != 0);
   return launched("RMSNorm batch");
+}
+
+extern "C" int32_t qllm_rms_norm_residual_batch(
+    float* hidden, const float* partials, uint32_t partial_count,
+    const float* weight, void* output_bf16, uint32_t rows, uint32_t elements,
+    float epsilon, int32_t zero_centered, void* stream) {
+  const auto aligned = [](const void* pointer) {
+    return reinterpret_cast<uintptr_t>(pointer) % 16u == 0u;
+  };
+  if (!hidden || !partials || !partial_count || partial_count > 16u ||
+      !output_bf16 || !rows || rows > 65535u || !elements ||
+      elements % 4u != 0u || elements > 16384u || !aligned(hidden) ||
+      !aligned(partials) || !aligned(output_bf16) || (weight && !aligned(weight)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid residual RMSNorm");
+  rms_norm_residual_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+      hidden, partials, partial_count, weight,
+      static_cast<uint16_t*>(output_bf16), elements, epsilon, zero_centered != 0);
+  return launched("residual RMSNorm");
 }
 
 extern "C" int32_t qllm_rms_norm_concat_batch(

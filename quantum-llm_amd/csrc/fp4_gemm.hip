@@ -72,6 +72,11 @@ struct GemmArgs {
   // Optional split of the output rows over up to three buffers (the q, k and
   // v projections stored as one matrix): segment s takes the next
   // segment_rows[s] rows.  segments == 0: everything goes to `output`.
+  // Cut of K over several workgroups per tile: workgroup (tile, split) sums the
+  // split's share of the 64-column chunks and writes an F32 partial to
+  // output + split * batch * rows (no residual, no segments); the consumer
+  // adds the partials.  0 or 1: one workgroup per tile.
+  uint32_t k_splits;
   uint32_t segments;
   uint32_t segment_rows[3];
   uint32_t segment_kind[3];
@@ -166,7 +171,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint32_t h = args.tile_rows;
   const uint32_t half_rows = h / 2u;
   const uint32_t tile_lane = n < half_rows ? n : half_rows - 1u;
-  const uint32_t first_row = blockIdx.x * h;
+  const uint32_t splits = args.k_splits > 1u ? args.k_splits : 1u;
+  const uint32_t tile_index = blockIdx.x / splits;
+  const uint32_t split = blockIdx.x - tile_index * splits;
+  const uint32_t first_row = tile_index * h;
 
   // Weight and scale streams: wave-uniform start of the tile's stream plus a
   // 32-bit lane offset; consecutive chunks are weight_step / scale_step apart.
@@ -188,7 +196,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
   for (int t = 0; t < TILES; ++t) {
     if (TILED) {
-      const size_t first_chunk = static_cast<size_t>(blockIdx.x) * (K / kChunk);
+      const size_t first_chunk = static_cast<size_t>(tile_index) * (K / kChunk);
       weight_base[t] = args.tile[t].weights + first_chunk * weight_step;
       scale_base[t] = args.tile[t].scales + first_chunk * scale_step;
     } else {
@@ -245,7 +253,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
       for (int i = 0; i < REGS; ++i) acc[t][j][i] = 0.0f;
 
-  const uint32_t chunks = K / kChunk;
+  // this workgroup's chunks: [first_chunk_of_split, + chunks)
+  const uint32_t all_chunks = K / kChunk;
+  const uint32_t first_chunk_of_split = split * all_chunks / splits;
+  const uint32_t chunks = (split + 1u) * all_chunks / splits - first_chunk_of_split;
   const uint32_t my_chunks =
       chunks > wave ? (chunks - wave + WAVES - 1u) / WAVES : 0u;
   // Prefetch is unconditional: indices past the wave's last chunk are clamped
@@ -257,7 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   uint32_t scales[PF][TILES][SCALE_WORDS];
   uint4 activation[PF];
   auto issue = [&](int slot, uint32_t index) {
-    const uint32_t chunk = wave + index * WAVES;   // uniform
+    const uint32_t chunk = first_chunk_of_split + wave + index * WAVES;   // uniform
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       codes[slot][t] = load_stream16(
@@ -416,6 +427,9 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     store_output(args.segment_output[segment], args.segment_kind[segment],
                  static_cast<size_t>(item_batch) * args.segment_rows[segment] + local,
                  total);
+  } else if (splits > 1u) {
+    static_cast<float*>(args.output)[static_cast<size_t>(split) * BATCH * args.rows +
+                                     item_index] = total;
   } else {
     store_output(args.output, args.output_kind, item_index, total + residual_value);
   }
@@ -554,11 +568,13 @@ int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
 }
 
 // One tile per workgroup (a gate tile and its up tile for the fused SwiGLU
-// pair); four waves split K, eight when the matrix has too few tiles to give
-// every CU one.
+// pair), or k_splits workgroups per tile; four waves split K, eight when the
+// launch has too few workgroups to give every CU one.
 int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
                     bool swiglu, hipStream_t stream) {
-  const uint32_t tiles = (args.rows + args.tile_rows - 1u) / args.tile_rows;
+  const uint32_t splits = args.k_splits > 1u ? args.k_splits : 1u;
+  const uint32_t tiles =
+      (args.rows + args.tile_rows - 1u) / args.tile_rows * splits;
   const uint32_t waves = tiles <= 256u && !swiglu ? 8u : 4u;
 #define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
   return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
@@ -694,6 +710,31 @@ extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
             input, nullptr, output, residual, matrix->rows,
             matrix->padded_columns, batch, output_kind);
   return launched("FP4 BF16 GEMV");
+}
+
+extern "C" int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,
+                                              const void* input,
+                                              size_t input_bytes,
+                                              float* partials,
+                                              uint32_t k_splits, uint32_t batch,
+                                              void* stream) {
+  if (!matrix_ok(matrix) || matrix->layout != QLLM_LAYOUT_TILED || !input ||
+      !partials || !batch || batch > 8u || !k_splits ||
+      k_splits > matrix->padded_columns / kChunk || k_splits > 16u ||
+      input_bytes < static_cast<size_t>(batch) * matrix->padded_columns * 2u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 BF16 partial GEMM");
+  GemmArgs args{};
+  args.tile[0] = {matrix->weights, static_cast<const uint8_t*>(matrix->scales)};
+  args.tile[1] = args.tile[0];
+  args.activations = static_cast<const uint16_t*>(input);
+  args.output = partials;
+  args.rows = matrix->rows;
+  args.padded_columns = matrix->padded_columns;
+  args.output_kind = QLLM_OUT_F32;
+  args.tile_rows = matrix_tile_rows(matrix);
+  args.k_splits = k_splits;
+  return launch_mfma(args, static_cast<int>(matrix->scale_scheme), true, batch,
+                     false, as_stream(stream));
 }
 
 extern "C" int32_t qllm_fp4_gemm_bf16_split(

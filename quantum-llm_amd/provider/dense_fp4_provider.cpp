@@ -223,6 +223,16 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   activation_ =
       static_cast<std::uint16_t*>(device_alloc(rows * g_.intermediate * 2U));
   logits_ = static_cast<float*>(device_alloc(rows * g_.vocabulary * 4U));
+  // The o and down projections have too few rows to occupy the GPU: K is cut
+  // over projection_splits_ workgroups per tile and the norm that follows
+  // adds the partials to the residual stream.
+  if (const char* text = std::getenv("QLLM_PROVIDER_K_SPLITS"))
+    projection_splits_ = static_cast<std::uint32_t>(
+        std::clamp(std::atoi(text), 0, 16));
+  if (g_.hidden % 4U != 0U || g_.hidden > 16384U) projection_splits_ = 0U;
+  if (projection_splits_ > 1U)
+    projection_partials_ = static_cast<float*>(
+        device_alloc(projection_splits_ * rows * g_.hidden * 4U));
 
   // Context splits: kv_heads * splits workgroups fill the 256 CUs; the
   // attention kernels deal the context's tiles evenly over them themselves
@@ -833,13 +843,41 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
       std::size_t{rows} * g_.query_heads * g_.head_dim * 2U;
   status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
                                         hidden_, rows, stream));
+  // Partials of the last residual projection that hidden_ does not hold yet;
+  // the next norm adds them.
+  std::uint32_t pending_partials = 0U;
+  const auto normalise = [&](const float* weight) {
+    if (pending_partials)
+      status_check(qllm_rms_norm_residual_batch(
+          hidden_, projection_partials_, pending_partials, weight, normalized_,
+          rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm, stream));
+    else
+      status_check(qllm_rms_norm_batch(hidden_, weight, nullptr, normalized_,
+                                       g_.hidden, rows, g_.hidden,
+                                       g_.norm_epsilon, g_.zero_centered_norm,
+                                       stream));
+    pending_partials = 0U;
+  };
+  // hidden_ += matrix * input, either in the projection's epilogue or as
+  // partials left for the next norm
+  const auto project_residual = [&](const qllm_fp4_matrix& matrix,
+                                    const std::uint16_t* input,
+                                    std::size_t input_bytes) {
+    if (projection_splits_ > 1U && matrix.layout == QLLM_LAYOUT_TILED &&
+        matrix.padded_columns / 64U >= projection_splits_) {
+      status_check(qllm_fp4_gemm_bf16_partial(&matrix, input, input_bytes,
+                                              projection_partials_,
+                                              projection_splits_, rows, stream));
+      pending_partials = projection_splits_;
+    } else {
+      status_check(qllm_fp4_gemm_bf16(&matrix, input, input_bytes, hidden_,
+                                      QLLM_OUT_F32, hidden_, rows, stream));
+    }
+  };
   for (std::uint32_t index = 0; index < g_.layers; ++index) {
     const auto& layer = layers_[index];
     // full attention block (run_full_attention, :6892)
-    status_check(qllm_rms_norm_batch(hidden_, layer.input_norm, nullptr,
-                                     normalized_, g_.hidden, rows, g_.hidden,
-                                     g_.norm_epsilon, g_.zero_centered_norm,
-                                     stream));
+    normalise(layer.input_norm);
     // query, key and value projections (:7004-7011) in one launch
     const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
     const qllm_gemm_segment projections[3] = {
@@ -851,26 +889,18 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                           stream));
     enqueue_attention(index, rows, first_position, deferred_positions, query_,
                       key_, value_, attention_);
-    status_check(qllm_fp4_gemm_bf16(&layer.output.descriptor, attention_,
-                                    attention_bytes, hidden_, QLLM_OUT_F32,
-                                    hidden_, rows, stream));
+    project_residual(layer.output.descriptor, attention_, attention_bytes);
     // dense SwiGLU block (run_ffn, :8250-8293)
-    status_check(qllm_rms_norm_batch(hidden_, layer.post_attention_norm,
-                                     nullptr, normalized_, g_.hidden, rows,
-                                     g_.hidden, g_.norm_epsilon,
-                                     g_.zero_centered_norm, stream));
+    normalise(layer.post_attention_norm);
     status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
                                       &layer.up.descriptor, normalized_,
                                       hidden_bytes, activation_, rows, stream));
-    status_check(qllm_fp4_gemm_bf16(
-        &layer.down.descriptor, activation_,
-        std::size_t{rows} * g_.intermediate * 2U, hidden_, QLLM_OUT_F32,
-        hidden_, rows, stream));
+    project_residual(layer.down.descriptor, activation_,
+                     std::size_t{rows} * g_.intermediate * 2U);
   }
-  // head (run_head, :8393-8527)
-  status_check(qllm_rms_norm_batch(hidden_, final_norm_, nullptr, normalized_,
-                                   g_.hidden, rows, g_.hidden, g_.norm_epsilon,
-                                   g_.zero_centered_norm, stream));
+  // head (run_head, :8393-8527); the norm also completes hidden_, which the
+  // proposer reads
+  normalise(final_norm_);
   status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_, hidden_bytes,
                                   logits_, QLLM_OUT_F32, nullptr, rows, stream));
   status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
@@ -1248,10 +1278,17 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
                                           hidden_bytes, activation_, rows,
                                           stream_));
       } else if (which == "ffn_down") {
-        status_check(qllm_fp4_gemm_bf16(
-            &layer.down.descriptor, activation_,
-            std::size_t{rows} * g_.intermediate * 2U, query_, QLLM_OUT_F32,
-            nullptr, rows, stream_));
+        // as the target pass launches it
+        const auto& down = layer.down.descriptor;
+        if (projection_splits_ > 1U && down.layout == QLLM_LAYOUT_TILED &&
+            down.padded_columns / 64U >= projection_splits_)
+          status_check(qllm_fp4_gemm_bf16_partial(
+              &down, activation_, std::size_t{rows} * g_.intermediate * 2U,
+              projection_partials_, projection_splits_, rows, stream_));
+        else
+          status_check(qllm_fp4_gemm_bf16(
+              &down, activation_, std::size_t{rows} * g_.intermediate * 2U,
+              query_, QLLM_OUT_F32, nullptr, rows, stream_));
       } else if (which == "lm_head") {
         status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
                                         hidden_bytes, logits_, QLLM_OUT_F32,

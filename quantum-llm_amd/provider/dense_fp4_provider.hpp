@@ -303,6 +303,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* partial_maxima_{};
   float* partial_sums_{};
   float* partial_outputs_{};
+  float* projection_partials_ = nullptr;   // [splits][rows][hidden]
+  std::uint32_t projection_splits_ = 3U;   // 0 / 1: residual in the epilogue
   void* select_workspace_{};
   std::size_t select_workspace_bytes_{};
   std::uint32_t* argmax_tokens_{};

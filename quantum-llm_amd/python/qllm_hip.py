@@ -86,6 +86,7 @@ SIGNATURES = {
     "qllm_convert_f32_to_bf16_batch": (c_int32, [c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_gemv_q8_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_fp4_gemm_bf16": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_bf16_partial": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_gemm_bf16_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_gemm_bf16_tall": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
     "qllm_fp4_gemm_bf16_tall_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
@@ -95,6 +96,7 @@ SIGNATURES = {
     "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
     "qllm_fp4_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_uint32, c_void_p]),
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_residual_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_silu_product": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),

@@ -201,3 +201,55 @@ def test_invalid_arguments_are_rejected(device):
     with pytest.raises(qh.QllmError):   # batch > 8
         qh.call("qllm_fp4_gemm_bf16", qh.fp4_matrix(codes, scales, 64, 64, 64, 0),
                 qh.ptr(act), act.numel() * 2, qh.ptr(out), 0, None, 9, None)
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_F16_BLOCK16, ol.SCALE_UE8M0_BLOCK32])
+@pytest.mark.parametrize("rows,padded,batch,splits", [
+    (5120, 17408, 5, 3), (5120, 8192, 5, 3), (333, 5120, 8, 2), (64, 128, 1, 2),
+    (100, 320, 3, 5), (512, 1024, 5, 16), (40, 64, 2, 1)])
+def test_k_split_partials_add_up_to_the_product(device, scheme, rows, padded, batch, splits):
+    """K cut over several workgroups per tile: partial s is the product over
+    the split's own chunks of 64 columns (checked against the oracle on that
+    column range), so the partials add up to the whole product."""
+    rng = np.random.default_rng(rows + padded + splits + scheme)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    tensors = (gu.device_tensor(codes, device), gu.device_tensor(scales, device))
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                                            scheme), device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    partials = torch.full((splits, batch, rows), np.nan, device=device)
+    qh.call("qllm_fp4_gemm_bf16_partial", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(partials), splits, batch, None)
+    torch.cuda.synchronize()
+    got = partials.cpu().numpy()
+    chunks = padded // 64
+    pick = rng.choice(rows, min(rows, 48), replace=False)
+    for split in range(splits):
+        first, last = split * chunks // splits * 64, (split + 1) * chunks // splits * 64
+        masked = np.zeros_like(act)
+        masked[:, first:last] = act[:, first:last]
+        want = ol.fp4_linear_f64(codes[pick], scales[pick], scheme, len(pick), padded, masked)
+        gu.assert_close(got[split][:, pick], want, what=f"partial {split}")
+    whole = gu.gemm(device, codes, scales, scheme, rows, padded, act, tiled=True)
+    # F32 sums of up to 17408 terms of magnitude ~10 in two different orders
+    gu.assert_close(got.astype(np.float64).sum(axis=0), whole, rtol=1e-5, atol=2e-3,
+                    what="sum of the partials")
+
+
+def test_k_split_rejects_what_it_does_not_take(device):
+    rng = np.random.default_rng(9)
+    rows, padded, batch = 64, 128, 5
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_F16_BLOCK16)
+    tensors = (gu.device_tensor(codes, device), gu.device_tensor(scales, device))
+    row_major = qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                              ol.SCALE_F16_BLOCK16)
+    tiled, keep = qh.prepack(row_major, device)
+    d_act = torch.zeros((batch, padded), dtype=torch.bfloat16, device=device)
+    partials = torch.zeros((16, batch, rows), device=device)
+    for matrix, splits, rows_in_batch in ((row_major, 2, batch), (tiled, 0, batch),
+                                          (tiled, 3, batch), (tiled, 17, batch),
+                                          (tiled, 2, 9)):
+        with pytest.raises(qh.QllmError):
+            qh.call("qllm_fp4_gemm_bf16_partial", matrix, qh.ptr(d_act), d_act.numel() * 2,
+                    qh.ptr(partials), splits, rows_in_batch, None)

@@ -186,3 +186,37 @@ def test_query_q8_quantisation_is_byte_exact(device):
     torch.cuda.synchronize()
     assert np.array_equal(q8.cpu().numpy(), want_q8)
     assert np.array_equal(scales.cpu().numpy(), want_scales)
+
+
+@pytest.mark.parametrize("elements,count", [(5120, 3), (256, 1), (16384, 16), (5124, 2)])
+def test_rms_norm_residual_adds_partials_in_order(device, elements, count):
+    """hidden += partial 0 + partial 1 + ... (that order, F32) and the RMSNorm
+    of the sum in bf16: the sum bit for bit, the norm equal to the plain norm
+    kernel's on the same sum and within the reference's 2e-5 of the oracle."""
+    rng = np.random.default_rng(elements + count)
+    rows = 5
+    hidden = (rng.standard_normal((rows, elements)) * 2).astype(np.float32)
+    partials = rng.standard_normal((count, rows, elements)).astype(np.float32)
+    w = (0.1 * rng.standard_normal(elements)).astype(np.float32)
+    d_hidden, d_partials, d_w = (gu.device_tensor(x, device) for x in (hidden, partials, w))
+    out = torch.zeros((rows, elements), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_residual_batch", qh.ptr(d_hidden), qh.ptr(d_partials), count,
+            qh.ptr(d_w), qh.ptr(out), rows, elements, 1e-6, 1, None)
+    total = hidden.copy()
+    for part in partials:
+        total = total + part
+    torch.cuda.synchronize()
+    assert np.array_equal(d_hidden.cpu().numpy(), total)
+    plain = torch.zeros((rows, elements), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_batch", qh.ptr(d_hidden), qh.ptr(d_w), None, qh.ptr(plain),
+            elements, rows, elements, 1e-6, 1, None)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert np.array_equal(got, plain.float().cpu().numpy())
+    want = ol.rms_norm_rows(total, w, 1e-6, True)
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 2e-5).all()
+    for bad_elements, bad_count in ((elements + 2, count), (16388, count), (elements, 0),
+                                    (elements, 17)):
+        with pytest.raises(qh.QllmError):
+            qh.call("qllm_rms_norm_residual_batch", qh.ptr(d_hidden), qh.ptr(d_partials),
+                    bad_count, qh.ptr(d_w), qh.ptr(out), rows, bad_elements, 1e-6, 1, None)
