@@ -177,6 +177,10 @@ void Mi355DenseFp4Provider::release() {
   if (stream_) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
   for (void* pointer : allocations_) (void)hipFree(pointer);
   allocations_.clear();
+  if (staging_) {
+    (void)hipHostFree(staging_);
+    staging_ = nullptr;
+  }
   for (void* page : pages_)
     if (page) (void)hipFree(page);
   pages_.clear();
@@ -206,8 +210,17 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   const std::size_t widest =
       std::max<std::size_t>({g_.hidden, g_.intermediate,
                              std::size_t{g_.query_heads} * g_.head_dim});
-  tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
-  positions_ = static_cast<std::uint32_t*>(device_alloc(4U * 4U));
+  // tokens (up to 8) and the four position words of a pass lie side by side,
+  // so that one copy from pinned host memory uploads both
+  tokens_ = static_cast<std::uint32_t*>(device_alloc((8U + 4U) * 4U));
+  positions_ = tokens_ + 8U;
+  {
+    void* pinned = nullptr;
+    hip_check(hipHostMalloc(&pinned, sizeof(HostStaging), hipHostMallocDefault),
+              "allocate pinned staging");
+    staging_ = static_cast<HostStaging*>(pinned);
+    *staging_ = HostStaging{};
+  }
   graphs_.assign(max_rows_ + 1U, nullptr);
   if (const char* eager = std::getenv("QLLM_PROVIDER_EAGER"))
     use_graphs_ = eager[0] == '0';
@@ -258,7 +271,8 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
       static_cast<std::uint32_t*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
 
   if (g_.mtp_layers) {
-    mtp_tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+    mtp_tokens_ = static_cast<std::uint32_t*>(device_alloc((8U + 4U) * 4U));
+    mtp_positions_ = mtp_tokens_ + 8U;
     mtp_embedding_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
     mtp_fusion_input_ =
         static_cast<std::uint16_t*>(device_alloc(rows * 2U * g_.hidden * 2U));
@@ -268,7 +282,6 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
               "clear proposer hidden state");
     mtp_logits_ = static_cast<float*>(device_alloc(g_.draft_vocabulary * 4U));
     mtp_argmax_ = static_cast<std::uint32_t*>(device_alloc(4U));
-    mtp_positions_ = static_cast<std::uint32_t*>(device_alloc(4U * 4U));
     mtp_draft_tokens_ =
         static_cast<std::uint32_t*>(device_alloc(kMaximumDraftDepth * 4U));
     mtp_graphs_.assign(2U * (max_rows_ + 1U), nullptr);
@@ -1199,14 +1212,15 @@ er::Status Mi355DenseFp4Provider::run_target_graph(const std::uint32_t* tokens,
       return {er::ErrorCode::invalid_argument, "target program is not prepared"};
     ensure_pages(first_position + rows - 1U);
     const auto stream = static_cast<hipStream_t>(stream_);
+    // The stream is idle here (every pass ends with a wait), so the pinned
+    // words of the previous pass have been read.
+    std::copy(tokens, tokens + rows, staging_->target);
     const std::uint32_t positions[4] = {first_position, first_position,
                                         first_position + 1U, rows};
-    hip_check(hipMemcpyAsync(tokens_, tokens, rows * sizeof(std::uint32_t),
+    std::copy(positions, positions + 4, staging_->target + 8);
+    hip_check(hipMemcpyAsync(tokens_, staging_->target, sizeof(staging_->target),
                              hipMemcpyHostToDevice, stream),
-              "upload target tokens");
-    hip_check(hipMemcpyAsync(positions_, positions, sizeof(positions),
-                             hipMemcpyHostToDevice, stream),
-              "upload target positions");
+              "upload target tokens and positions");
     if (!graphs_[rows]) {
       hip_check(hipStreamSynchronize(stream), "drain stream before capture");
       hipGraph_t graph{};
@@ -1687,12 +1701,12 @@ void Mi355DenseFp4Provider::propose_with_graphs(
   ensure_pages(committed_length + drafts - 2U);
   const std::uint32_t positions[4] = {first_position, first_position + 1U,
                                       first_position + 1U, 0U};
-  hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
-                           hipMemcpyHostToDevice, stream),
-            "upload MTP token batch");
-  hip_check(hipMemcpyAsync(mtp_positions_, positions, sizeof(positions),
-                           hipMemcpyHostToDevice, stream),
-            "upload MTP positions");
+  std::copy(tokens.begin(), tokens.end(), staging_->proposer);
+  std::copy(positions, positions + 4, staging_->proposer + 8);
+  hip_check(hipMemcpyAsync(mtp_tokens_, staging_->proposer,
+                           sizeof(staging_->proposer), hipMemcpyHostToDevice,
+                           stream),
+            "upload MTP tokens and positions");
   state.draft_predictions.clear();
   state.draft_predictions.reserve(drafts);
   const bool greedy =
@@ -1701,7 +1715,7 @@ void Mi355DenseFp4Provider::propose_with_graphs(
     launch_mtp_graph(rows, false);
     for (std::uint32_t pass = 1; pass < drafts; ++pass)
       launch_mtp_graph(1U, true);
-    std::uint32_t chosen[kMaximumDraftDepth]{};
+    std::uint32_t* const chosen = staging_->download;
     hip_check(hipMemcpyAsync(chosen, mtp_draft_tokens_, drafts * 4U,
                              hipMemcpyDeviceToHost, stream),
               "copy MTP draft tokens");
@@ -1808,10 +1822,22 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
 
     std::vector<er::SamplingDistribution> target_distributions;
     target_distributions.reserve(rows);
-    for (std::uint32_t row = 0; row < rows; ++row)
-      target_distributions.push_back(distribution_from_logits(
-          logits_ + std::size_t{row} * g_.vocabulary, g_.vocabulary,
-          argmax_tokens_ + row, invocation.request));
+    if (request_parameter(invocation.request, "sampling_temperature_ppm") == 0U) {
+      // greedy: the rows' arg-max tokens in one copy and one wait
+      const auto stream = static_cast<hipStream_t>(stream_);
+      hip_check(hipMemcpyAsync(staging_->download, argmax_tokens_,
+                               rows * sizeof(std::uint32_t),
+                               hipMemcpyDeviceToHost, stream),
+                "copy exact greedy tokens");
+      hip_check(hipStreamSynchronize(stream), "copy exact greedy tokens");
+      for (std::uint32_t row = 0; row < rows; ++row)
+        target_distributions.push_back({{{staging_->download[row], 1.0}}});
+    } else {
+      for (std::uint32_t row = 0; row < rows; ++row)
+        target_distributions.push_back(distribution_from_logits(
+            logits_ + std::size_t{row} * g_.vocabulary, g_.vocabulary,
+            argmax_tokens_ + row, invocation.request));
+    }
 
     const auto seed = request_parameter(invocation.request, "sampling_seed");
     std::size_t accepted{};

@@ -303,6 +303,14 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* partial_maxima_{};
   float* partial_sums_{};
   float* partial_outputs_{};
+  // Pinned host words for the small per-pass transfers: 8 tokens + 4
+  // position words up (target pass, proposer pass), 8 chosen tokens down.
+  struct HostStaging {
+    std::uint32_t target[12];
+    std::uint32_t proposer[12];
+    std::uint32_t download[8];
+  };
+  HostStaging* staging_ = nullptr;
   float* projection_partials_ = nullptr;   // [splits][rows][hidden]
   std::uint32_t projection_splits_ = 3U;   // 0 / 1: residual in the epilogue
   void* select_workspace_{};
