@@ -117,13 +117,15 @@ def cpu_baseline(rows):
     }
 
 
-def measure_decode_cycle(qp, np, rows, steps, warmup):
+def measure_decode_cycle(qp, np, rows, steps, warmup, sampled=False):
     """The whole decode cycle of the same model with the proposer inside the
     provider: verify step, proposer advance over the emitted tokens, rollout of
     the next four drafts (1 + 3 proposer passes over its Q8 cache, each ending
     in the 65536-row draft head).  Random-init weights accept almost nothing,
     so a cycle emits one token; the time per cycle is what real weights would
-    see as well."""
+    see as well.  `sampled`: temperature 0.7, top-p 0.95, top-k 64 instead of
+    greedy (rejection sampling on the host from the rows' top-k logits, the
+    proposer returning to the host after every pass)."""
     geometry = dict(MODEL)
     geometry["mtp_layers"] = 1
     needed = CONTEXT + (steps + warmup + 2) * rows + 8
@@ -132,7 +134,11 @@ def measure_decode_cycle(qp, np, rows, steps, warmup):
     provider.load_synthetic_weights(20241125)
     provider.prefill_synthetic_kv(CONTEXT, 7)
     provider.prepare_exact_decode("decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2")
-    provider.begin_request(temperature_ppm=0)
+    if sampled:
+        provider.begin_request(temperature_ppm=700000, top_p_ppm=950000, top_k=64,
+                               seed=20241125)
+    else:
+        provider.begin_request(temperature_ppm=0)
     token, position = 1, CONTEXT
     provider.synchronize(token, position)
     emitted = 0
@@ -376,6 +382,11 @@ def main():
         provider.close()
         provider = None
         decode_cycle = measure_decode_cycle(qp, np, rows, min(steps, 20), min(warmup, 3))
+        sampled = measure_decode_cycle(qp, np, rows, min(steps, 20), min(warmup, 3),
+                                       sampled=True)
+        decode_cycle["sampled_t0.7_top_p0.95_top_k64"] = {
+            key: sampled[key] for key in ("tok_s", "ms_per_cycle", "emitted_tokens",
+                                          "accepted_drafts")}
     if arguments.layers == MODEL["layers"] and not arguments.skip_long_contexts:
         if provider is not None:
             provider.close()

@@ -527,6 +527,19 @@ int32_t qllm_topk_logits(const float* values, uint32_t count, uint32_t top_k,
                          void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* The same selection for `rows` rows of logits in two launches (k <= 64):
+ * values f32 [rows][row_stride] (the first `count` of each row), outputs
+ * [rows][top_k].  Same order, ties and padding as qllm_topk_logits.  The
+ * reference selects row by row (topk_logits, transformer_kernels.cu:7096-7178,
+ * one call per target row, dense_fp4_provider.cpp:8331-8391). */
+size_t qllm_topk_batch_workspace_bytes(uint32_t count, uint32_t top_k,
+                                       uint32_t rows);
+int32_t qllm_topk_logits_batch(const float* values, uint32_t count,
+                               size_t row_stride, uint32_t top_k, uint32_t rows,
+                               float* output_values, uint32_t* output_indices,
+                               void* workspace, size_t workspace_bytes,
+                               void* stream);
+
 /* replaces apply_presence_penalty (transformer_kernels.hpp:1292-1294). */
 int32_t qllm_apply_presence_penalty(float* logits, const uint8_t* emitted,
                                     uint32_t count, float penalty,

@@ -219,6 +219,160 @@ __global__ __launch_bounds__(kMergeThreads) void topk_merge_kernel(
                                  output_indices, shared_values, shared_indices);
 }
 
+// ---- batched top-k by threshold ------------------------------------------------
+//
+// The k rounds above cost a block reduction each.  For k <= 64 the rows of a
+// batch are served by two launches instead:
+//   1. the maximum of every chunk of `chunk` items (one wave per chunk);
+//   2. per row, one workgroup: the k-th largest chunk maximum is a threshold
+//      that at least k items reach (the chunk maxima themselves), so the top k
+//      lie among the items >= threshold; those - a few hundred for logits
+//      whose large values are spread over the vocabulary - are gathered into
+//      LDS and ranked against each other, rank r going to output slot r.
+// With fewer chunks than k the threshold is -inf (every item is a candidate).
+// If more candidates turn up than LDS holds (large values packed into a few
+// chunks), the workgroup falls back to k rounds over the whole row.  Results
+// are those of the rounds: same order, same ties, NaN excluded, missing ranks
+// padded with (-inf, no index).
+constexpr uint32_t kSelectThreads = 1024;
+constexpr uint32_t kSelectCandidates = 4096;
+constexpr uint32_t kSelectMaxChunks = 4096;
+constexpr uint32_t kSelectMaxK = 64;
+
+__global__ __launch_bounds__(256) void chunk_max_kernel(
+    const float* values, uint32_t count, size_t row_stride, uint32_t chunk,
+    uint32_t chunks_per_row, float* maxima) {
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t index = blockIdx.x * 4u + (threadIdx.x >> 6);
+  if (index >= chunks_per_row) return;
+  const float* row = values + blockIdx.y * row_stride;
+  const uint32_t first = index * chunk;
+  const uint32_t last = min(count, first + chunk);
+  float best = -INFINITY;
+  for (uint32_t item = first + lane; item < last; item += 64u) {
+    const float value = row[item];
+    if (value > best) best = value;   // NaN never wins
+  }
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1)
+    best = fmaxf(best, __shfl_xor(best, offset, 64));
+  if (lane == 0u) maxima[blockIdx.y * chunks_per_row + index] = best;
+}
+
+__global__ __launch_bounds__(kSelectThreads) void topk_threshold_kernel(
+    const float* values, uint32_t count, size_t row_stride, uint32_t top_k,
+    const float* maxima, uint32_t chunks_per_row, float* output_values,
+    uint32_t* output_indices) {
+  __shared__ float candidate_values[kSelectCandidates];
+  __shared__ uint32_t candidate_indices[kSelectCandidates];
+  __shared__ float threshold;
+  __shared__ uint32_t candidates;
+  __shared__ float shared_values[16];
+  __shared__ uint32_t shared_indices[16];
+  const float* row = values + blockIdx.x * row_stride;
+  float* out_values = output_values + static_cast<size_t>(blockIdx.x) * top_k;
+  uint32_t* out_indices = output_indices + static_cast<size_t>(blockIdx.x) * top_k;
+
+  // the k-th largest chunk maximum (staged in candidate_values)
+  if (threadIdx.x == 0u) {
+    threshold = -INFINITY;
+    candidates = 0u;
+  }
+  for (uint32_t item = threadIdx.x; item < chunks_per_row; item += kSelectThreads)
+    candidate_values[item] = maxima[blockIdx.x * chunks_per_row + item];
+  __syncthreads();
+  if (chunks_per_row >= top_k)
+    for (uint32_t item = threadIdx.x; item < chunks_per_row; item += kSelectThreads) {
+      const float mine = candidate_values[item];
+      uint32_t rank = 0;
+      for (uint32_t other = 0; other < chunks_per_row; ++other) {
+        const float value = candidate_values[other];
+        rank += value > mine || (value == mine && other < item) ? 1u : 0u;
+      }
+      if (rank == top_k - 1u) threshold = mine;
+    }
+  __syncthreads();
+  const float limit = threshold;
+  __syncthreads();   // the staged maxima are overwritten from here on
+
+  for (uint32_t item = threadIdx.x; item < count; item += kSelectThreads) {
+    const float value = row[item];
+    if (value >= limit) {   // false for NaN
+      const uint32_t slot = atomicAdd(&candidates, 1u);
+      if (slot < kSelectCandidates) {
+        candidate_values[slot] = value;
+        candidate_indices[slot] = item;
+      }
+    }
+  }
+  __syncthreads();
+  const uint32_t found = candidates;
+
+  if (found <= kSelectCandidates) {
+    for (uint32_t item = threadIdx.x; item < found; item += kSelectThreads) {
+      const float mine = candidate_values[item];
+      const uint32_t mine_index = candidate_indices[item];
+      uint32_t rank = 0;
+      for (uint32_t other = 0; other < found; ++other)
+        rank += better(candidate_values[other], candidate_indices[other], mine,
+                       mine_index) ? 1u : 0u;
+      if (rank < top_k) {
+        out_values[rank] = mine;
+        out_indices[rank] = mine_index;
+      }
+    }
+    for (uint32_t rank = found + threadIdx.x; rank < top_k; rank += kSelectThreads) {
+      out_values[rank] = -INFINITY;
+      out_indices[rank] = kNoIndex;
+    }
+    return;
+  }
+
+  // More candidates than LDS holds: k rounds over the row, each taking the
+  // best item that comes after the previous winner in the order.
+  float previous = INFINITY;
+  uint32_t previous_index = 0u;
+  bool first_round = true;
+  for (uint32_t rank = 0; rank < top_k; ++rank) {
+    float best = -INFINITY;
+    uint32_t best_index = kNoIndex;
+    for (uint32_t item = threadIdx.x; item < count; item += kSelectThreads) {
+      const float value = row[item];
+      if (isnan(value)) continue;
+      if (!first_round && !better(previous, previous_index, value, item)) continue;
+      if (best_index == kNoIndex || better(value, item, best, best_index)) {
+        best = value;
+        best_index = item;
+      }
+    }
+    block_best(best, best_index, shared_values, shared_indices);
+    if (threadIdx.x == 0u) {
+      out_values[rank] = best_index == kNoIndex ? -INFINITY : best;
+      out_indices[rank] = best_index;
+    }
+    if (best_index == kNoIndex) {
+      for (uint32_t rest = rank + 1u + threadIdx.x; rest < top_k;
+           rest += kSelectThreads) {
+        out_values[rest] = -INFINITY;
+        out_indices[rest] = kNoIndex;
+      }
+      return;
+    }
+    previous = best;
+    previous_index = best_index;
+    first_round = false;
+  }
+}
+
+// chunk size: a power of two >= 64 aiming at 4 k chunks per row, at most
+// kSelectMaxChunks chunks
+uint32_t select_chunk(uint32_t count, uint32_t top_k) {
+  uint32_t chunk = 64u;
+  while (chunk * 2u <= count / (4u * top_k)) chunk *= 2u;
+  while ((count + chunk - 1u) / chunk > kSelectMaxChunks) chunk *= 2u;
+  return chunk;
+}
+
 // transformer_kernels.cu:7180-7186
 __global__ void presence_penalty_kernel(float* logits, const uint8_t* emitted,
                                         uint32_t count, float penalty) {
@@ -294,6 +448,37 @@ extern "C" int32_t qllm_topk_logits(const float* values, uint32_t count,
       partial_values, partial_indices, static_cast<uint32_t>(survivors), top_k,
       output_values, output_indices);
   return launched("top-k logits");
+}
+
+extern "C" size_t qllm_topk_batch_workspace_bytes(uint32_t count,
+                                                  uint32_t top_k,
+                                                  uint32_t rows) {
+  if (!count || !top_k || top_k > kSelectMaxK || !rows) return 0;
+  const uint32_t chunk = select_chunk(count, top_k);
+  return static_cast<size_t>((count + chunk - 1u) / chunk) * rows * sizeof(float);
+}
+
+extern "C" int32_t qllm_topk_logits_batch(const float* values, uint32_t count,
+                                          size_t row_stride, uint32_t top_k,
+                                          uint32_t rows, float* output_values,
+                                          uint32_t* output_indices,
+                                          void* workspace,
+                                          size_t workspace_bytes,
+                                          void* stream) {
+  if (!values || !count || !top_k || top_k > kSelectMaxK || top_k > count ||
+      !rows || rows > 65535u || row_stride < count || !output_values ||
+      !output_indices || !workspace ||
+      workspace_bytes < qllm_topk_batch_workspace_bytes(count, top_k, rows))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid batched top-k logits");
+  const uint32_t chunk = select_chunk(count, top_k);
+  const uint32_t chunks = (count + chunk - 1u) / chunk;
+  float* maxima = static_cast<float*>(workspace);
+  chunk_max_kernel<<<dim3((chunks + 3u) / 4u, rows), 256, 0, as_stream(stream)>>>(
+      values, count, row_stride, chunk, chunks, maxima);
+  topk_threshold_kernel<<<rows, kSelectThreads, 0, as_stream(stream)>>>(
+      values, count, row_stride, top_k, maxima, chunks, output_values,
+      output_indices);
+  return launched("batched top-k logits");
 }
 
 extern "C" int32_t qllm_apply_presence_penalty(float* logits,

@@ -263,12 +263,16 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
 
   select_workspace_bytes_ = std::max(
       qllm_argmax_workspace_bytes(g_.vocabulary, max_rows_),
-      qllm_topk_workspace_bytes(g_.vocabulary, kMaximumGpuSamplingTopK));
+      std::max(qllm_topk_workspace_bytes(g_.vocabulary, kMaximumGpuSamplingTopK),
+               qllm_topk_batch_workspace_bytes(g_.vocabulary,
+                                               kMaximumGpuSamplingTopK, max_rows_)));
   select_workspace_ = device_alloc(select_workspace_bytes_);
   argmax_tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
-  top_logits_ = static_cast<float*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
-  top_tokens_ =
-      static_cast<std::uint32_t*>(device_alloc(kMaximumGpuSamplingTopK * 4U));
+  // top-k logits of up to 8 rows, then their tokens: one buffer, one readback
+  top_logits_ = static_cast<float*>(
+      device_alloc(8U * kMaximumGpuSamplingTopK * (4U + 4U)));
+  top_tokens_ = reinterpret_cast<std::uint32_t*>(
+      top_logits_ + 8U * kMaximumGpuSamplingTopK);
 
   if (g_.mtp_layers) {
     mtp_tokens_ = static_cast<std::uint32_t*>(device_alloc((8U + 4U) * 4U));
@@ -1434,25 +1438,61 @@ er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
     for (const auto token : host_tokens) host_logits.push_back(full[token]);
     sampling_logit_transfer_bytes_ += full.size() * 4U;
   } else {
-    status_check(qllm_topk_logits(row_logits, vocabulary,
-                                  static_cast<std::uint32_t>(top_k), top_logits_,
-                                  top_tokens_, select_workspace_,
-                                  select_workspace_bytes_, stream_));
-    host_logits.resize(top_k);
-    host_tokens.resize(top_k);
-    hip_check(hipMemcpyAsync(host_logits.data(), top_logits_, top_k * 4U,
-                             hipMemcpyDeviceToHost, stream),
-              "copy speculative top-k logits");
-    hip_check(hipMemcpyAsync(host_tokens.data(), top_tokens_, top_k * 4U,
-                             hipMemcpyDeviceToHost, stream),
-              "copy speculative top-k tokens");
-    hip_check(hipStreamSynchronize(stream), "copy speculative top-k");
-    ++sampling_gpu_calls_;
-    sampling_logit_transfer_bytes_ += top_k * 8U;
+    return std::move(distributions_from_top_k(row_logits, vocabulary, vocabulary,
+                                              1U, request)
+                         .front());
   }
   return er::make_sampling_distribution(
       host_logits, host_tokens, static_cast<std::uint32_t>(temperature), top_p,
       min_p);
+}
+
+// The distributions of `rows` rows of logits (row r at logits + r * stride)
+// for a sampled request with 1 <= top_k <= 64: one selection launch for all
+// rows, one readback, then make_sampling_distribution per row
+// (distribution_from_logits, dense_fp4_provider.cpp:8331-8391, which selects
+// and reads back row by row).
+std::vector<er::SamplingDistribution>
+Mi355DenseFp4Provider::distributions_from_top_k(
+    const float* logits, std::uint32_t vocabulary, std::size_t stride,
+    std::uint32_t rows, const er::ProgramRequestContext& request) {
+  const auto stream = static_cast<hipStream_t>(stream_);
+  const auto temperature = request_parameter(request, "sampling_temperature_ppm");
+  const auto top_p = static_cast<std::uint32_t>(
+      request_parameter(request, "sampling_top_p_ppm"));
+  const auto min_p = static_cast<std::uint32_t>(
+      request_parameter(request, "sampling_min_p_ppm"));
+  const auto top_k =
+      static_cast<std::uint32_t>(request_parameter(request, "sampling_top_k"));
+  if (!rows || rows > 8U || !top_k || top_k > kMaximumGpuSamplingTopK ||
+      top_k > vocabulary)
+    throw std::runtime_error(
+        "sampled exact decode requires top-k of at most 64 (0 = whole row)");
+  status_check(qllm_topk_logits_batch(logits, vocabulary, stride, top_k, rows,
+                                      top_logits_, top_tokens_, select_workspace_,
+                                      select_workspace_bytes_, stream_));
+  // logits of all rows, then tokens of all rows (the device buffers are
+  // adjacent with room for 8 rows of 64)
+  constexpr std::size_t kCapacity = 8U * kMaximumGpuSamplingTopK;
+  hip_check(hipMemcpyAsync(staging_->top_logits, top_logits_,
+                           kCapacity * 4U + std::size_t{rows} * top_k * 4U,
+                           hipMemcpyDeviceToHost, stream),
+            "copy speculative top-k");
+  hip_check(hipStreamSynchronize(stream), "copy speculative top-k");
+  ++sampling_gpu_calls_;
+  sampling_logit_transfer_bytes_ += std::size_t{rows} * top_k * 8U;
+  std::vector<er::SamplingDistribution> result;
+  result.reserve(rows);
+  for (std::uint32_t row = 0; row < rows; ++row) {
+    const std::span<const float> row_logits(
+        staging_->top_logits + std::size_t{row} * top_k, top_k);
+    const std::span<const std::uint32_t> row_tokens(
+        staging_->top_tokens + std::size_t{row} * top_k, top_k);
+    result.push_back(er::make_sampling_distribution(
+        row_logits, row_tokens, static_cast<std::uint32_t>(temperature), top_p,
+        min_p));
+  }
+  return result;
 }
 
 // ---- the proposer (run_mtp / extend_mtp_rollout, :8681-8852) -----------------
@@ -1731,11 +1771,13 @@ void Mi355DenseFp4Provider::propose_with_graphs(
     for (std::uint32_t depth = 0; depth < drafts; ++depth) {
       if (depth) {
         // the device chained its own argmax; the sampled draft replaces it
-        const std::uint32_t token = state.draft_predictions.back().token;
-        hip_check(hipMemcpyAsync(mtp_tokens_, &token, sizeof(token),
-                                 hipMemcpyHostToDevice, stream),
+        // (pinned word: the previous pass ended with a wait, and the copy is
+        // ordered before the pass launched next)
+        staging_->proposer[0] = state.draft_predictions.back().token;
+        hip_check(hipMemcpyAsync(mtp_tokens_, staging_->proposer,
+                                 sizeof(std::uint32_t), hipMemcpyHostToDevice,
+                                 stream),
                   "upload sampled MTP draft");
-        hip_check(hipStreamSynchronize(stream), "upload sampled MTP draft");
       }
       launch_mtp_graph(depth ? 1U : rows, depth != 0U);
       DraftPrediction prediction;
@@ -1832,6 +1874,9 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       hip_check(hipStreamSynchronize(stream), "copy exact greedy tokens");
       for (std::uint32_t row = 0; row < rows; ++row)
         target_distributions.push_back({{{staging_->download[row], 1.0}}});
+    } else if (request_parameter(invocation.request, "sampling_top_k") != 0U) {
+      target_distributions = distributions_from_top_k(
+          logits_, g_.vocabulary, g_.vocabulary, rows, invocation.request);
     } else {
       for (std::uint32_t row = 0; row < rows; ++row)
         target_distributions.push_back(distribution_from_logits(

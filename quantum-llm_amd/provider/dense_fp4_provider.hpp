@@ -228,6 +228,9 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                    std::uint64_t seed, bool tiled);
   void enqueue_target(const std::uint32_t* device_tokens, std::uint32_t rows,
                       std::uint32_t first_position, bool deferred_positions);
+  std::vector<er::SamplingDistribution> distributions_from_top_k(
+      const float* logits, std::uint32_t vocabulary, std::size_t stride,
+      std::uint32_t rows, const er::ProgramRequestContext& request);
   er::SamplingDistribution distribution_from_logits(
       const float* row_logits, std::uint32_t vocabulary,
       const std::uint32_t* device_argmax,
@@ -309,6 +312,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
     std::uint32_t target[12];
     std::uint32_t proposer[12];
     std::uint32_t download[8];
+    float top_logits[8 * 64];            // top-k readback: logits of all rows,
+    std::uint32_t top_tokens[8 * 64];    // then their tokens
   };
   HostStaging* staging_ = nullptr;
   float* projection_partials_ = nullptr;   // [splits][rows][hidden]

@@ -220,3 +220,86 @@ def test_rms_norm_residual_adds_partials_in_order(device, elements, count):
         with pytest.raises(qh.QllmError):
             qh.call("qllm_rms_norm_residual_batch", qh.ptr(d_hidden), qh.ptr(d_partials),
                     bad_count, qh.ptr(d_w), qh.ptr(out), rows, bad_elements, 1e-6, 1, None)
+
+
+def batched_topk(device, rows_of_values, k, stride=None):
+    values = np.stack(rows_of_values).astype(np.float32)
+    rows, count = values.shape
+    stride = stride or count
+    padded = np.full((rows, stride), 1e30, dtype=np.float32)   # never read
+    padded[:, :count] = values
+    d_values = gu.device_tensor(padded, device)
+    out_v = torch.zeros((rows, k), device=device)
+    out_i = torch.zeros((rows, k), dtype=torch.int32, device=device)
+    size = qh.call("qllm_topk_batch_workspace_bytes", count, k, rows)
+    workspace = torch.zeros(max(size, 4), dtype=torch.uint8, device=device)
+    qh.call("qllm_topk_logits_batch", qh.ptr(d_values), count, stride, k, rows,
+            qh.ptr(out_v), qh.ptr(out_i), qh.ptr(workspace), size, None)
+    torch.cuda.synchronize()
+    return out_v.cpu().numpy(), out_i.cpu().numpy().astype(np.uint32)
+
+
+def check_against_oracle(device, rows_of_values, k, stride=None):
+    values, indices = batched_topk(device, rows_of_values, k, stride)
+    for row, source in enumerate(rows_of_values):
+        want_v, want_i = ol.topk(np.asarray(source, dtype=np.float32), k)
+        assert indices[row].tolist() == want_i.tolist(), row
+        assert np.array_equal(values[row], want_v), row
+
+
+def test_batched_topk_equals_the_oracle_row_by_row(device):
+    """Threshold selection for all rows of a batch: bit-equal to the exact
+    descending top-k of the oracle (ties to the lower id, NaN excluded)."""
+    nan = float("nan")
+    # runtime/tools/dense_fp4_cuda_smoke.cpp:4313-4335
+    check_against_oracle(device, [[1.0, 7.0, nan, 7.0, -2.0, 4.5, 4.5, 9.0, 0.0]], 5)
+    # :4337-4359, beside three other rows of the same length
+    v = 248320
+    i = np.arange(v, dtype=np.float32)
+    big = (np.sin(i * np.float32(0.0137)) + np.float32(0.37) * np.cos(i * np.float32(0.0071))
+           ).astype(np.float32)
+    big[19] = big[127] = 7.0
+    big[1021] = nan
+    rng = np.random.default_rng(5)
+    check_against_oracle(device, [big, rng.standard_normal(v), -big, np.sort(big)], 20)
+    # the verify step's shape: 5 rows of the vocabulary inside a wider buffer
+    logits = [rng.standard_normal(151936) * 3 for _ in range(5)]
+    logits[1][1000:1064] = 50.0            # 64 equal winners
+    logits[2][::7] = nan
+    logits[3][:] = np.round(logits[3])     # many ties at the threshold
+    check_against_oracle(device, logits, 64, stride=151936 + 64)
+    check_against_oracle(device, logits[:2], 1)
+    # the draft vocabulary, a short row, fewer chunks than k
+    check_against_oracle(device, [rng.standard_normal(65536)], 64)
+    check_against_oracle(device, [rng.standard_normal(4097), rng.standard_normal(4097)], 64)
+    check_against_oracle(device, [rng.standard_normal(300)], 64)
+
+
+def test_batched_topk_when_the_threshold_does_not_filter(device):
+    """Large values packed into few chunks, or all values equal: more items
+    reach the threshold than the candidate list holds and the rows fall back
+    to the k rounds; fewer valid items than k pad with (-inf, no index)."""
+    rng = np.random.default_rng(6)
+    flat = np.zeros(151936, dtype=np.float32)
+    ramp = np.arange(151936, dtype=np.float32)          # the top k end the row
+    plateau = rng.standard_normal(151936).astype(np.float32)
+    plateau[plateau > -1.0] = 2.5                       # most items tie for first
+    check_against_oracle(device, [flat, ramp, -ramp, plateau], 64)
+    few = np.full(9000, np.nan, dtype=np.float32)
+    few[[3, 4000, 8999]] = [1.0, -np.inf, 1.0]
+    values, indices = batched_topk(device, [few], 8)
+    assert indices[0].tolist() == [3, 8999, 4000] + [0xffffffff] * 5
+    assert values[0][:3].tolist() == [1.0, 1.0, -np.inf] and np.all(np.isneginf(values[0][3:]))
+
+
+def test_batched_topk_rejects_what_it_does_not_take(device):
+    values = torch.zeros((2, 1000), device=device)
+    out_v = torch.zeros((2, 64), device=device)
+    out_i = torch.zeros((2, 64), dtype=torch.int32, device=device)
+    workspace = torch.zeros(1 << 16, dtype=torch.uint8, device=device)
+    for count, stride, k, rows, bytes_ in ((1000, 1000, 65, 2, 1 << 16), (1000, 999, 8, 2, 1 << 16),
+                                           (1000, 1000, 0, 2, 1 << 16), (1000, 1000, 8, 0, 1 << 16),
+                                           (1000, 1000, 8, 2, 8), (7, 1000, 8, 2, 1 << 16)):
+        with pytest.raises(qh.QllmError):
+            qh.call("qllm_topk_logits_batch", qh.ptr(values), count, stride, k, rows,
+                    qh.ptr(out_v), qh.ptr(out_i), qh.ptr(workspace), bytes_, None)
