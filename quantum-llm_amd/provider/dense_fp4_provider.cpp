@@ -997,6 +997,10 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
     const std::size_t kv_width = std::size_t{g_.kv_heads} * g_.head_dim;
     const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
     const bool feed_proposer = state && mtp_.ready;
+    // query rows per attention workgroup: as many as the kernels' three (two at
+    // head_dim 256) 16-row tiles hold for one KV head's group of query heads
+    const std::uint32_t attention_batch = std::max(
+        1U, (g_.head_dim == 256U ? 32U : 48U) / (g_.query_heads / g_.kv_heads));
     if (state) {
       state->draft_valid = false;
       state->draft_predictions.clear();
@@ -1059,7 +1063,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.output_gated = g_.output_gated;
           launch.output_kind = QLLM_OUT_BF16;
           launch.stream = stream;
-          status_check(qllm_attention_paged_q4h_batched(&launch, max_rows_));
+          status_check(qllm_attention_paged_q4h_batched(&launch, attention_batch));
         } else {
           const std::uint32_t query_stride =
               g_.head_dim * (g_.output_gated ? 2U : 1U);
@@ -1092,7 +1096,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.output_gated = g_.output_gated;
           launch.output_kind = QLLM_OUT_BF16;
           launch.stream = stream;
-          status_check(qllm_attention_paged_f16_batched(&launch, max_rows_));
+          status_check(qllm_attention_paged_f16_batched(&launch, attention_batch));
         }
         status_check(qllm_fp4_gemm_bf16_tall(
             &layer.output.descriptor, prefill_attention_,
