@@ -288,7 +288,12 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
     mtp_argmax_ = static_cast<std::uint32_t*>(device_alloc(4U));
     mtp_draft_tokens_ =
         static_cast<std::uint32_t*>(device_alloc(kMaximumDraftDepth * 4U));
-    mtp_graphs_.assign(2U * (max_rows_ + 1U), nullptr);
+    // a captured pass at 2 * rows + chained, then the captured greedy rollouts
+    // (first pass of `rows` rows + drafts - 1 chained single-row passes) at
+    // 2 * (max_rows + 1) + rows * (kMaximumDraftDepth + 1) + drafts
+    mtp_graphs_.assign(2U * (max_rows_ + 1U) +
+                           (max_rows_ + 1U) * (kMaximumDraftDepth + 1U),
+                       nullptr);
   }
 
   // Page geometry: every page holds all target layers back to back, then the
@@ -1647,9 +1652,16 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
 // Replays the proposer pass captured for (rows, source of the previous hidden
 // state); the first use captures it.  `chained` passes read the proposer's own
 // last hidden state, the others the target's.
-void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained) {
+// `drafts` == 0: one pass of `rows` rows (on the target's hidden state, or
+// `chained` on the proposer's own).  `drafts` >= 1: a whole greedy rollout in
+// one graph - the pass of `rows` rows on the target's hidden state followed by
+// drafts - 1 chained single-row passes.
+void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained,
+                                             std::uint32_t drafts) {
   const auto stream = static_cast<hipStream_t>(stream_);
-  void*& slot = mtp_graphs_.at(2U * rows + (chained ? 1U : 0U));
+  void*& slot = mtp_graphs_.at(
+      drafts ? 2U * (max_rows_ + 1U) + rows * (kMaximumDraftDepth + 1U) + drafts
+             : 2U * rows + (chained ? 1U : 0U));
   if (!slot) {
     hip_check(hipStreamSynchronize(stream), "drain stream before capture");
     hipGraph_t graph{};
@@ -1657,6 +1669,8 @@ void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained) {
               "begin proposer capture");
     try {
       enqueue_mtp(rows, chained ? mtp_last_hidden_ : hidden_, true, 0U, true);
+      for (std::uint32_t pass = 1; pass < drafts; ++pass)
+        enqueue_mtp(1U, mtp_last_hidden_, true, 0U, true);
     } catch (...) {
       (void)hipStreamEndCapture(stream, &graph);
       if (graph) (void)hipGraphDestroy(graph);
@@ -1756,9 +1770,7 @@ void Mi355DenseFp4Provider::propose_with_graphs(
   const bool greedy =
       request_parameter(request, "sampling_temperature_ppm") == 0U;
   if (greedy) {
-    launch_mtp_graph(rows, false);
-    for (std::uint32_t pass = 1; pass < drafts; ++pass)
-      launch_mtp_graph(1U, true);
+    launch_mtp_graph(rows, false, drafts);
     std::uint32_t* const chosen = staging_->download;
     hip_check(hipMemcpyAsync(chosen, mtp_draft_tokens_, drafts * 4U,
                              hipMemcpyDeviceToHost, stream),

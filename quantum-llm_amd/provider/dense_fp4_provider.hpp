@@ -253,7 +253,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
                    bool produce_logits, std::uint32_t cache_position,
                    bool deferred_positions);
-  void launch_mtp_graph(std::uint32_t rows, bool chained);
+  void launch_mtp_graph(std::uint32_t rows, bool chained,
+                        std::uint32_t drafts = 0U);
   // run_mtp + extend_mtp_rollout replayed from captured graphs
   void propose_with_graphs(DenseFp4RequestState& state,
                            std::span<const std::uint32_t> tokens,
@@ -352,7 +353,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   std::uint64_t prefill_tokens_total_{};
   std::uint32_t* mtp_positions_{};      // cache, rotary, context, draft slot
   std::uint32_t* mtp_draft_tokens_{};
-  std::vector<void*> mtp_graphs_;       // hipGraphExec_t at 2*rows + chained
+  std::vector<void*> mtp_graphs_;       // hipGraphExec_t: passes, then rollouts
 
   std::uint32_t* positions_{};   // device: cache, rotary, first-context
   std::vector<void*> graphs_;    // hipGraphExec_t per row count
