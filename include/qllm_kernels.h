@@ -498,6 +498,15 @@ typedef struct qllm_q8_attention_launch {
 
 int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launch);
 
+/* qllm_attention_paged_q8 for a prompt chunk: `rows` query rows served in
+ * batches of batch_rows (grid layer z = rows z*batch_rows ..., each row with
+ * its own context first_context_tokens + row), one launch and one combine.
+ * Partials are laid out by global row.  rows <= 65535; device_positions must
+ * be NULL.  No counterpart in the reference, which feeds the proposer five
+ * rows at a time (dense_fp4_provider.cpp:8681-8792). */
+int32_t qllm_attention_paged_q8_batched(const qllm_q8_attention_launch* launch,
+                                        uint32_t batch_rows);
+
 /* ---- token selection ------------------------------------------------------------ */
 
 /* Chains greedy proposer passes on the device (no counterpart in the

@@ -735,3 +735,71 @@ extern "C" int32_t qllm_attention_paged_q8(const qllm_q8_attention_launch* launc
       launch->maximum_splits, launch->split_tokens, launch->rows,
       launch->query_heads, launch->head_dim, launch->device_positions, stream);
 }
+
+extern "C" int32_t qllm_attention_paged_q8_batched(
+    const qllm_q8_attention_launch* launch, uint32_t batch_rows) {
+  if (!launch || !launch->query || !launch->device_pages || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      launch->device_positions || !launch->first_context_tokens ||
+      !launch->rows || !batch_rows || launch->rows > 65535u ||
+      !launch->page_tokens || launch->page_tokens % kF16Tile ||
+      launch->page_offset_bytes % 16u || !launch->query_heads ||
+      !launch->kv_heads || launch->query_heads % launch->kv_heads ||
+      (launch->head_dim != 128u && launch->head_dim != 256u) ||
+      launch->split_tokens % kF16Tile || !launch->maximum_splits ||
+      launch->maximum_splits > 2048u ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid batched Q8 paged attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  const uint32_t row_tiles =
+      ((batch_rows < launch->rows ? batch_rows : launch->rows) * group + 15u) / 16u;
+  if (row_tiles > 3u || (launch->head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched Q8 paged attention: batch_rows * (query_heads/kv_heads) "
+                "exceeds 48 (32 at head_dim 256)");
+  const uint32_t batches = (launch->rows + batch_rows - 1u) / batch_rows;
+  const uint32_t last_context = launch->first_context_tokens + launch->rows - 1u;
+  const uint32_t splits =
+      launch->split_tokens
+          ? (last_context + launch->split_tokens - 1u) / launch->split_tokens
+          : launch->maximum_splits;
+  if (splits > launch->maximum_splits)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "batched Q8 paged attention: context needs more splits than "
+                "maximum_splits");
+  F16SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.pages = launch->device_pages;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.page_tokens = launch->page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.split_tokens = launch->split_tokens;
+  args.maximum_splits = launch->maximum_splits;
+  args.page_offset = launch->page_offset_bytes;
+  args.batch_rows = batch_rows;
+  const dim3 grid(launch->kv_heads, splits, batches);
+  const hipStream_t stream = as_stream(launch->stream);
+  const int32_t status =
+      launch->head_dim == 128u
+          ? launch_f16_split<128, true>(args, row_tiles, grid, stream)
+          : launch_f16_split<256, true>(args, row_tiles, grid, stream);
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, launch->split_tokens, launch->rows,
+      launch->query_heads, launch->head_dim, nullptr, stream);
+}

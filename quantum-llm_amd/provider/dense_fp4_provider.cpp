@@ -930,6 +930,107 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                  stream));
 }
 
+// The proposer's pass over a prompt chunk: row r pairs tokens[r] (the token
+// after prompt position `position` + r) with the target's hidden state of that
+// position, which prefill() left in prefill_hidden_.  Same operations as
+// enqueue_mtp without the draft head, on the tall-batch GEMM and the batched
+// Q8 attention; writes the proposer's cache records position .. position +
+// rows - 1 and reuses the prefill buffers (prefill_hidden_ becomes the
+// proposer's residual stream).
+void Mi355DenseFp4Provider::enqueue_mtp_prefill(
+    std::span<const std::uint32_t> tokens, std::uint32_t position,
+    std::uint32_t attention_batch) {
+  void* const stream = stream_;
+  const auto hip_stream = static_cast<hipStream_t>(stream_);
+  const auto rows = static_cast<std::uint32_t>(tokens.size());
+  const auto& layer = mtp_.layer;
+  const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
+  const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
+  const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+  float* const embedding = prefill_gate_;                 // f32 [rows, hidden]
+  std::uint16_t* const fusion_input = prefill_activation_;  // bf16 [rows, 2 hidden]
+  hip_check(hipMemcpyAsync(prefill_tokens_, tokens.data(), rows * 4U,
+                           hipMemcpyHostToDevice, hip_stream),
+            "upload the proposer's prompt tokens");
+  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, prefill_tokens_,
+                                        embedding, rows, stream));
+  status_check(qllm_rms_norm_concat_batch(
+      embedding, mtp_.embedding_norm, prefill_hidden_, mtp_.hidden_norm,
+      fusion_input, rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm,
+      stream));
+  status_check(qllm_fp4_gemm_bf16_tall(&mtp_.fusion.descriptor, fusion_input,
+                                       2U * hidden_bytes, prefill_hidden_,
+                                       QLLM_OUT_F32, nullptr, rows, stream));
+  status_check(qllm_rms_norm_batch(prefill_hidden_, layer.input_norm, nullptr,
+                                   prefill_normalized_, g_.hidden, rows,
+                                   g_.hidden, g_.norm_epsilon,
+                                   g_.zero_centered_norm, stream));
+  const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+  const qllm_gemm_segment projections[3] = {
+      {prefill_query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+      {prefill_key_, kv_rows, QLLM_OUT_F32},
+      {prefill_value_, kv_rows, QLLM_OUT_F32}};
+  status_check(qllm_fp4_gemm_bf16_tall_split(&layer.qkv.descriptor,
+                                             prefill_normalized_, hidden_bytes,
+                                             projections, 3U, rows, stream));
+  const auto pages = const_cast<const void* const*>(device_page_table_);
+  // the proposer's cache lags the target's by one token: record `position`
+  // carries rotary position `position` + 1 (enqueue_mtp)
+  status_check(qllm_qkv_rope_batch(
+      prefill_query_, query_stride, prefill_key_, layer.query_norm,
+      layer.key_norm, position + 1U, rows, g_.query_heads, g_.kv_heads,
+      g_.head_dim, g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
+  status_check(qllm_store_kv_paged_q8_batch(
+      prefill_key_, prefill_value_, pages, mtp_page_offset_, g_.kv_page_tokens,
+      position, rows, g_.kv_heads, g_.head_dim, stream));
+  qllm_q8_attention_launch launch{};
+  launch.query = prefill_query_;
+  launch.device_pages = pages;
+  launch.output = prefill_attention_;
+  launch.partial_maxima = prefill_partial_maxima_;
+  launch.partial_sums = prefill_partial_sums_;
+  launch.partial_outputs = prefill_partial_outputs_;
+  launch.page_offset_bytes = mtp_page_offset_;
+  launch.first_context_tokens = position + 1U;
+  launch.rows = rows;
+  launch.page_tokens = g_.kv_page_tokens;
+  launch.query_heads = g_.query_heads;
+  launch.kv_heads = g_.kv_heads;
+  launch.head_dim = g_.head_dim;
+  launch.split_tokens = 0U;
+  launch.maximum_splits = prefill_splits_;
+  launch.query_stride = query_stride;
+  launch.output_gated = g_.output_gated;
+  launch.output_kind = QLLM_OUT_BF16;
+  launch.stream = stream;
+  status_check(qllm_attention_paged_q8_batched(&launch, attention_batch));
+  status_check(qllm_fp4_gemm_bf16_tall(
+      &layer.output.descriptor, prefill_attention_,
+      std::size_t{rows} * attention_width * 2U, prefill_hidden_, QLLM_OUT_F32,
+      prefill_hidden_, rows, stream));
+  status_check(qllm_rms_norm_batch(prefill_hidden_, layer.post_attention_norm,
+                                   nullptr, prefill_normalized_, g_.hidden, rows,
+                                   g_.hidden, g_.norm_epsilon,
+                                   g_.zero_centered_norm, stream));
+  status_check(qllm_fp4_gemm_bf16_tall(&layer.gate.descriptor,
+                                       prefill_normalized_, hidden_bytes,
+                                       prefill_gate_, QLLM_OUT_F32, nullptr, rows,
+                                       stream));
+  status_check(qllm_fp4_gemm_bf16_tall(&layer.up.descriptor, prefill_normalized_,
+                                       hidden_bytes, prefill_up_, QLLM_OUT_F32,
+                                       nullptr, rows, stream));
+  status_check(qllm_silu_product(prefill_gate_, prefill_up_, prefill_gate_,
+                                 rows * g_.intermediate, 1, stream));
+  status_check(qllm_convert_f32_to_bf16_batch(
+      prefill_gate_, prefill_activation_,
+      std::size_t{rows} * g_.intermediate * 2U, rows, g_.intermediate,
+      g_.intermediate, stream));
+  status_check(qllm_fp4_gemm_bf16_tall(
+      &layer.down.descriptor, prefill_activation_,
+      std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_, QLLM_OUT_F32,
+      prefill_hidden_, rows, stream));
+}
+
 void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
   if (rows <= prefill_rows_) return;
   if (prefill_rows_)
@@ -1130,25 +1231,35 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
             std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_,
             QLLM_OUT_F32, prefill_hidden_, rows, stream));
       }
-      // the proposer sees (token at p + 1, target hidden at p) for every prompt
-      // position but the last, whose successor is not known yet
-      if (feed_proposer) {
-        const std::uint32_t pairs = done + rows == count ? rows - 1U : rows;
-        for (std::uint32_t row = 0; row < pairs; row += max_rows_) {
-          const std::uint32_t batch = std::min(max_rows_, pairs - row);
-          (void)run_mtp(*state, tokens.subspan(done + row + 1U, batch),
-                        prefill_hidden_ + std::size_t{row} * g_.hidden, false,
-                        nullptr, 0U, 0U);
-        }
-      }
-      done += rows;
-      if (done == count) {
+      if (done + rows == count) {
         // last row -> the verify step's buffers, then the head on that row
         hip_check(hipMemcpyAsync(
                       hidden_, prefill_hidden_ + std::size_t{rows - 1U} * g_.hidden,
                       g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
                   "retain the prompt's last hidden state");
       }
+      // the proposer sees (token at p + 1, target hidden at p) for every prompt
+      // position but the last, whose successor is not known yet
+      if (feed_proposer) {
+        const std::uint32_t pairs = done + rows == count ? rows - 1U : rows;
+        const bool tall = g_.hidden <= 16384U && g_.intermediate >= 2U * g_.hidden &&
+                          mtp_.fusion.descriptor.layout == QLLM_LAYOUT_TILED;
+        if (pairs && tall) {
+          enqueue_mtp_prefill(tokens.subspan(done + 1U, pairs), position,
+                              attention_batch);
+          state->mtp_length += pairs;
+          ++mtp_passes_;
+          mtp_rows_ += pairs;
+        } else {
+          for (std::uint32_t row = 0; row < pairs; row += max_rows_) {
+            const std::uint32_t batch = std::min(max_rows_, pairs - row);
+            (void)run_mtp(*state, tokens.subspan(done + row + 1U, batch),
+                          prefill_hidden_ + std::size_t{row} * g_.hidden, false,
+                          nullptr, 0U, 0U);
+          }
+        }
+      }
+      done += rows;
     }
     status_check(qllm_rms_norm_batch(hidden_, final_norm_, nullptr, normalized_,
                                      g_.hidden, 1U, g_.hidden, g_.norm_epsilon,

@@ -253,6 +253,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
                    bool produce_logits, std::uint32_t cache_position,
                    bool deferred_positions);
+  void enqueue_mtp_prefill(std::span<const std::uint32_t> tokens,
+                           std::uint32_t position, std::uint32_t attention_batch);
   void launch_mtp_graph(std::uint32_t rows, bool chained,
                         std::uint32_t drafts = 0U);
   // run_mtp + extend_mtp_rollout replayed from captured graphs

@@ -112,6 +112,7 @@ SIGNATURES = {
     "qllm_store_kv_paged_f16_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),
     "qllm_attention_paged_f16_batched": (c_int32, [POINTER(F16AttentionLaunch), c_uint32]),
+    "qllm_attention_paged_q8_batched": (c_int32, [POINTER(Q8AttentionLaunch), c_uint32]),
     "qllm_q8_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_store_kv_paged_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_store_kv_paged_q8_batch_deferred": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),

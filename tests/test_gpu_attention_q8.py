@@ -148,3 +148,39 @@ def test_q8_entry_points_reject_bad_arguments(device):
     launch.page_tokens, launch.head_dim = 32, 64
     with pytest.raises(qh.QllmError):          # head_dim
         qh.call("qllm_attention_paged_q8", launch)
+
+
+@pytest.mark.parametrize("total,first,Q,KV,d,batch,gated", [
+    (23, 200, 16, 4, 128, 5, False), (40, 1, 64, 8, 128, 6, False),
+    (9, 300, 24, 4, 256, 4, True)])
+def test_q8_batched_launch_equals_one_launch_per_batch(device, total, first, Q, KV, d,
+                                                       batch, gated):
+    """All row batches of a prompt chunk in one launch: bit for bit what one
+    launch per batch computes."""
+    rng = np.random.default_rng(total + first)
+    page_tokens, offset, splits = 64, 512, 8
+    tokens = first + total - 1
+    d_pages, table, pages = build_cache(device, rng, tokens, KV, d, page_tokens, offset)
+    stride = d * (2 if gated else 1)
+    query = rng.standard_normal((total, Q, stride)).astype(np.float32)
+    d_query = gu.device_tensor(query, device)
+    maxima = torch.zeros((total, splits, Q), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((total, splits, Q, d), device=device)
+    out = torch.zeros((total, Q, d), device=device)
+    launch = qh.Q8AttentionLaunch(
+        qh.ptr(d_query), qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), offset, first, total, page_tokens, Q, KV, d, 0, splits, stride,
+        int(gated), qh.OUT_F32, None)
+    qh.call("qllm_attention_paged_q8_batched", launch, batch)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for row in range(0, total, batch):
+        rows = min(batch, total - row)
+        single = gu.q8_attention(device, d_pages, table, offset, query[row:row + rows], rows,
+                                 Q, KV, d, first + row, page_tokens, 0, gated,
+                                 balanced_splits=splits)
+        assert np.array_equal(got[row:row + rows], single), row
+    if total * (Q // KV) > (32 if d == 256 else 48):
+        with pytest.raises(qh.QllmError):
+            qh.call("qllm_attention_paged_q8_batched", launch, total)

@@ -75,6 +75,9 @@ def test_prefill_feeds_the_proposer_and_decoding_continues(device, count):
     drafts = fast.drafts()
     assert len(drafts) == 4
     assert fast.telemetry("provider_mtp_rows") >= count
+    # the prompt's pairs go through the proposer in one tall pass per chunk
+    # (then the last pair and three rollout passes), not five rows at a time
+    assert fast.telemetry("provider_mtp_passes") == (5 if count > 1 else 4)
     # the same stream token by token: target row, then the proposer's pair
     slow.begin_request(temperature_ppm=0)
     for index in range(count):
