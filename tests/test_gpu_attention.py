@@ -213,3 +213,26 @@ def test_batched_launch_equals_one_launch_per_batch(device, total, first, Q, KV,
     if total * (Q // KV) > (32 if d == 256 else 48):
         with pytest.raises(qh.QllmError, match="exceeds"):     # one batch of everything
             qh.call("qllm_attention_paged_q4h_batched", launch, total)
+
+
+def test_attention_at_131072_tokens_on_one_kv_head(device):
+    """The long-context benchmark shape cut down to one KV head and its eight
+    query heads (the heads are independent, so this is one eighth of the full
+    launch): against the oracle in double precision, and the same result for
+    every context partition."""
+    rng = np.random.default_rng(131072)
+    tokens, rows, Q, KV, d, page = 131072, 5, 8, 1, 128, 256
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, page)
+    query = ol.bf16_round(rng.standard_normal((rows, Q, d)).astype(np.float32))
+    first = tokens - 4
+    results = [gu.q4h_attention(device, pages, query, rows, Q, KV, d, first, page,
+                                split, False) for split in (4096, 16384, 0)]
+    for other in results[1:]:
+        assert np.abs(other - results[0]).max() < 2e-5
+    shape = ol.AttentionShape(rows, Q, KV, d, first, page, 0, 0)
+    want = ol.attention_q4h(shape, query, pages, "f64")
+    gu.assert_close(results[0], want, what="131072-token attention")
+    # the rows are causal among themselves: each sees one token more
+    assert all(np.abs(results[0][r] - results[0][r + 1]).max() > 0 for r in range(rows - 1))

@@ -162,3 +162,23 @@ def test_batched_launch_equals_one_launch_per_batch(device):
         single = gu.f16_attention(device, pages, query[row:row + rows], rows, Q, KV, d,
                                   first + row, page_tokens, 0, False, balanced_splits=splits)
         assert np.array_equal(got[row:row + rows], single), row
+
+
+def test_f16_attention_at_262144_tokens_on_one_kv_head(device):
+    """The exact-F16 benchmark shape cut down to one KV head and its eight
+    query heads: against the oracle (reference rounding points and exact), and
+    the same result for every context partition."""
+    rng = np.random.default_rng(262144)
+    tokens, rows, Q, KV, d, page = 262144, 5, 8, 1, 128, 256
+    first = tokens - (rows - 1)
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.f16_pages(keys, values, page)
+    query = rng.standard_normal((rows, Q, d)).astype(np.float32)
+    results = [gu.f16_attention(device, pages, query, rows, Q, KV, d, first, page, split,
+                                False) for split in (8192, 65536, 0)]
+    for other in results[1:]:
+        assert np.abs(other - results[0]).max() < 2e-5
+    shape = ol.AttentionShape(rows, Q, KV, d, first, page, 0, 0)
+    gu.assert_close(results[0], ol.attention_f16(shape, query, pages, False),
+                    what="262144-token F16 attention (exact)")
