@@ -528,6 +528,20 @@ int32_t qllm_argmax_batch(const float* values, uint32_t count,
                           uint32_t batch, uint32_t* output, void* workspace,
                           size_t workspace_bytes, void* stream);
 
+/* qllm_argmax_batch for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it): the same
+ * kernels and results, the stage-1 partials in a fixed 64 KiB array inside
+ * the library's code object instead of a workspace.  No counterpart in the
+ * reference.  Calls no allocating routine.  Limit: ceil(count / 2048) * batch
+ * <= 8192 (qllm_argmax_workspace_bytes(count, batch) <=
+ * qllm_argmax_static_capacity_bytes()); larger requests fail with
+ * QLLM_INVALID_ARGUMENT.  Every call on a GPU shares that GPU's array: calls
+ * that overlap on one GPU (different streams or threads) race. */
+size_t qllm_argmax_static_capacity_bytes(void);
+int32_t qllm_argmax_batch_static(const float* values, uint32_t count,
+                                 uint32_t batch, uint32_t* output,
+                                 void* stream);
+
 /* replaces topk_logits (transformer_kernels.hpp:1271-1290): exact descending
  * top-k of one row, ties to the lower id, NaN excluded, k <= 1024. */
 size_t qllm_topk_workspace_bytes(uint32_t count, uint32_t top_k);

@@ -6,6 +6,8 @@
 // NaN never selected.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace qllm {
 namespace {
 
@@ -406,6 +408,75 @@ extern "C" int32_t qllm_argmax_batch(const float* values, uint32_t count,
   argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
       partial_values, partial_indices, blocks, output);
   return launched("argmax batch");
+}
+
+// ---- argmax without an allocation -------------------------------------------
+// The stage-1 partials of qllm_argmax_batch in a fixed array inside the code
+// object instead of a caller's workspace.  Each device that loads the library
+// holds its own copy; host code reaches it through the address
+// hipGetSymbolAddress reports for the current device, never through the
+// array's name.
+namespace qllm {
+namespace {
+
+constexpr size_t kStaticArgmaxBytes = 64u * 1024u;
+constexpr int kStaticArgmaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticArgmaxBytes];
+
+std::mutex static_argmax_mutex;
+void* static_argmax_address[kStaticArgmaxDevices] = {};
+
+// Address of `scratch` on the current device, looked up once per device.
+int32_t static_argmax_scratch(void** address) {
+  int device = -1;
+  if (const int32_t status = checked(hipGetDevice(&device), "hipGetDevice"))
+    return status;
+  if (device < 0 || device >= kStaticArgmaxDevices)
+    return fail(QLLM_INVALID_ARGUMENT, "argmax static: device index above 63");
+  std::lock_guard<std::mutex> guard(static_argmax_mutex);
+  if (!static_argmax_address[device]) {
+    void* found = nullptr;
+    if (const int32_t status =
+            checked(hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)),
+                    "hipGetSymbolAddress(argmax scratch)"))
+      return status;
+    if (!found) return fail(QLLM_INTERNAL, "argmax static: no scratch address");
+    static_argmax_address[device] = found;
+  }
+  *address = static_argmax_address[device];
+  return QLLM_OK;
+}
+
+}  // namespace
+}  // namespace qllm
+
+extern "C" size_t qllm_argmax_static_capacity_bytes(void) {
+  return kStaticArgmaxBytes;
+}
+
+extern "C" int32_t qllm_argmax_batch_static(const float* values, uint32_t count,
+                                            uint32_t batch, uint32_t* output,
+                                            void* stream) {
+  if (!values || !count || !batch || !output)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid argmax batch");
+  if (qllm_argmax_workspace_bytes(count, batch) > kStaticArgmaxBytes)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "argmax static: ceil(count / 2048) * batch exceeds 8192 "
+                "(the 64 KiB scratch array); use qllm_argmax_batch with a "
+                "workspace");
+  void* workspace = nullptr;
+  if (const int32_t status = static_argmax_scratch(&workspace)) return status;
+  const uint32_t blocks = (count + kArgmaxChunk - 1u) / kArgmaxChunk;
+  float* partial_values = static_cast<float*>(workspace);
+  uint32_t* partial_indices = reinterpret_cast<uint32_t*>(
+      partial_values + static_cast<size_t>(blocks) * batch);
+  // every partial the final kernel reads is written by this call's first
+  // kernel, so nothing left by an earlier call needs clearing
+  argmax_partial_kernel<<<dim3(blocks, batch), 256, 0, as_stream(stream)>>>(
+      values, count, partial_values, partial_indices, blocks);
+  argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
+      partial_values, partial_indices, blocks, output);
+  return launched("argmax batch static");
 }
 
 extern "C" int32_t qllm_rollout_advance(const uint32_t* selected,

@@ -120,6 +120,8 @@ SIGNATURES = {
     "qllm_attention_paged_q8": (c_int32, [POINTER(Q8AttentionLaunch)]),
     "qllm_argmax_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "qllm_argmax_batch": (c_int32, [c_void_p, c_uint32, c_uint32, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "qllm_argmax_static_capacity_bytes": (c_size_t, []),
+    "qllm_argmax_batch_static": (c_int32, [c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "qllm_topk_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "qllm_topk_logits": (c_int32, [c_void_p, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "qllm_topk_batch_workspace_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
