@@ -202,7 +202,10 @@ int32_t qllm_fp4_gemm_bf16_tall_split(const qllm_fp4_matrix* matrix,
                                       uint32_t segment_count, uint32_t batch,
                                       void* stream);
 
-/* replaces fp4_embedding_batch (transformer_kernels.hpp:68-70). */
+/* replaces fp4_embedding_batch (transformer_kernels.hpp:68-70).  A token
+ * outside the matrix (tokens[r] >= rows; a device-side selection over logits
+ * without a finite maximum yields 0xffffffff) reads nothing and gives a row of
+ * zeros; host callers validate tokens themselves, as the reference does. */
 int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
                                  const uint32_t* tokens, float* output,
                                  uint32_t batch, void* stream);
@@ -567,6 +570,25 @@ int32_t qllm_topk_logits_batch(const float* values, uint32_t count,
 int32_t qllm_apply_presence_penalty(float* logits, const uint8_t* emitted,
                                     uint32_t count, float penalty,
                                     void* stream);
+
+/* The same penalty for the `rows` rows of one verify step in one launch
+ * (logits f32 [rows][row_stride], the first `count` of each row): row r is
+ * penalised at the tokens marked in `emitted` and at drafts[0 .. r-1], the
+ * tokens the rows before it carry (drafts: device, rows - 1 entries).  The
+ * reference penalises row by row and marks draft r in a scratch copy of the
+ * presence bytes in between (runtime/tools/dense_fp4_provider.cpp:
+ * 11182-11202). */
+int32_t qllm_apply_presence_penalty_rows(float* logits, size_t row_stride,
+                                         const uint8_t* emitted,
+                                         const uint32_t* drafts, uint32_t rows,
+                                         uint32_t count, float penalty,
+                                         void* stream);
+
+/* emitted[tokens[i]] = 1 for up to 64 device-resident tokens (entries >= count
+ * are ignored).  Replaces the per-token cudaMemset of the reference
+ * (dense_fp4_provider.cpp:11261-11270, 8822-8847). */
+int32_t qllm_mark_presence(uint8_t* emitted, const uint32_t* tokens,
+                           uint32_t token_count, uint32_t count, void* stream);
 
 /* ---- synthetic data (benchmarks and tests) ------------------------------------- */
 

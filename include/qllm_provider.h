@@ -112,6 +112,19 @@ int32_t qllm_provider_begin_request(qllm_provider* provider,
                                     uint32_t top_p_ppm, uint32_t top_k,
                                     uint32_t min_p_ppm, uint64_t seed);
 
+/* The same with the request's parameter map spelled out, name by name, as the
+ * runner builds it (moe_vm_runner.cpp:318-347): reserved_context_tokens,
+ * sampling_temperature_ppm, sampling_top_p_ppm, sampling_top_k,
+ * sampling_min_p_ppm, sampling_presence_penalty_biased_ppm (penalty in ppm +
+ * 2,000,000), sampling_first_output_position, sampling_seed,
+ * exact_decode_enabled.  A sampled request (temperature != 0) without a first
+ * output position or with a penalty parameter above 4,000,000 is turned down
+ * (dense_fp4_provider.cpp:5502-5513). */
+int32_t qllm_provider_begin_request_with(qllm_provider* provider,
+                                         const char* const* names,
+                                         const uint64_t* values,
+                                         uint32_t count);
+
 /* synchronize_exact_decode_batch with one token: the stream stands at
  * `position` with `token` guaranteed (the batch starts at position - 1, the
  * target position the token was chosen from).  With an MTP layer this feeds

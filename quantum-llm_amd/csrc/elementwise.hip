@@ -73,9 +73,16 @@ __global__ __launch_bounds__(256) void convert_f32_to_bf16_batch_kernel(
 __global__ __launch_bounds__(256) void fp4_embedding_batch_kernel(
     const uint8_t* weights, const uint8_t* scales, uint32_t scheme,
     const uint32_t* tokens, float* output, uint32_t columns,
-    uint32_t padded_columns) {
+    uint32_t padded_columns, uint32_t vocabulary) {
   const uint32_t request = blockIdx.x;
   const size_t token = tokens[request];
+  if (token >= vocabulary) {
+    // a token chosen on the device from logits without a finite maximum: no
+    // row to read, the caller rejects the token when it sees it
+    for (uint32_t column = threadIdx.x; column < columns; column += blockDim.x)
+      output[static_cast<size_t>(request) * columns + column] = 0.0f;
+    return;
+  }
   const uint8_t* row_codes = weights + token * (padded_columns / 2u);
   for (uint32_t column = threadIdx.x; column < columns; column += blockDim.x) {
     const uint8_t byte = row_codes[column / 2u];
@@ -103,11 +110,18 @@ __global__ __launch_bounds__(256) void fp4_embedding_batch_kernel(
 __global__ __launch_bounds__(256) void fp4_embedding_batch_wide_kernel(
     const uint8_t* weights, const uint8_t* scales, uint32_t scheme,
     const uint32_t* tokens, float* output, uint32_t columns,
-    uint32_t padded_columns) {
+    uint32_t padded_columns, uint32_t vocabulary) {
   const uint32_t request = blockIdx.x;
   const uint32_t column = (blockIdx.y * blockDim.x + threadIdx.x) * 8u;
   if (column >= columns) return;
   const size_t token = tokens[request];
+  if (token >= vocabulary) {   // see fp4_embedding_batch_kernel
+    float4* destination = reinterpret_cast<float4*>(
+        output + static_cast<size_t>(request) * columns + column);
+    destination[0] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    destination[1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    return;
+  }
   const uint32_t codes = *reinterpret_cast<const uint32_t*>(
       weights + token * (padded_columns / 2u) + column / 2u);
   float scale;
@@ -410,12 +424,12 @@ extern "C" int32_t qllm_fp4_embedding_batch(const qllm_fp4_matrix* matrix,
                                       256, 0, as_stream(stream)>>>(
         matrix->weights, static_cast<const uint8_t*>(matrix->scales),
         matrix->scale_scheme, tokens, output, matrix->columns,
-        matrix->padded_columns);
+        matrix->padded_columns, matrix->rows);
   else
     fp4_embedding_batch_kernel<<<batch, 256, 0, as_stream(stream)>>>(
         matrix->weights, static_cast<const uint8_t*>(matrix->scales),
         matrix->scale_scheme, tokens, output, matrix->columns,
-        matrix->padded_columns);
+        matrix->padded_columns, matrix->rows);
   return launched("FP4 embedding batch");
 }
 

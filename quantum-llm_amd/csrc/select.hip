@@ -382,6 +382,29 @@ __global__ void presence_penalty_kernel(float* logits, const uint8_t* emitted,
   if (index < count && emitted[index] != 0u) logits[index] -= penalty;
 }
 
+// The verify step's rows in one launch: row r is penalised where a token was
+// emitted before the step or is one of the drafts the rows before r carry
+// (the reference penalises row by row and marks draft r in a scratch copy of
+// the presence bytes in between, dense_fp4_provider.cpp:11182-11202).
+__global__ __launch_bounds__(256) void presence_penalty_rows_kernel(
+    float* logits, size_t row_stride, const uint8_t* emitted,
+    const uint32_t* drafts, uint32_t rows, uint32_t count, float penalty) {
+  const uint32_t index = blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= count) return;
+  bool present = emitted[index] != 0u;
+  for (uint32_t row = 0; row < rows; ++row) {
+    if (present) logits[row * row_stride + index] -= penalty;
+    if (row + 1u < rows && drafts[row] == index) present = true;
+  }
+}
+
+__global__ __launch_bounds__(64) void mark_presence_kernel(
+    uint8_t* emitted, const uint32_t* tokens, uint32_t token_count,
+    uint32_t count) {
+  if (threadIdx.x < token_count && tokens[threadIdx.x] < count)
+    emitted[tokens[threadIdx.x]] = 1u;
+}
+
 }  // namespace
 }  // namespace qllm
 
@@ -561,4 +584,27 @@ extern "C" int32_t qllm_apply_presence_penalty(float* logits,
   presence_penalty_kernel<<<(count + 255u) / 256u, 256, 0, as_stream(stream)>>>(
       logits, emitted, count, penalty);
   return launched("presence penalty");
+}
+
+extern "C" int32_t qllm_apply_presence_penalty_rows(
+    float* logits, size_t row_stride, const uint8_t* emitted,
+    const uint32_t* drafts, uint32_t rows, uint32_t count, float penalty,
+    void* stream) {
+  if (!logits || !emitted || !count || !rows || row_stride < count ||
+      (rows > 1u && !drafts))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid presence penalty rows");
+  presence_penalty_rows_kernel<<<(count + 255u) / 256u, 256, 0,
+                                 as_stream(stream)>>>(
+      logits, row_stride, emitted, drafts, rows, count, penalty);
+  return launched("presence penalty rows");
+}
+
+extern "C" int32_t qllm_mark_presence(uint8_t* emitted, const uint32_t* tokens,
+                                      uint32_t token_count, uint32_t count,
+                                      void* stream) {
+  if (!emitted || !tokens || !token_count || token_count > 64u || !count)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid presence marks");
+  mark_presence_kernel<<<1, 64, 0, as_stream(stream)>>>(emitted, tokens,
+                                                        token_count, count);
+  return launched("presence marks");
 }

@@ -28,6 +28,28 @@ void status_check(std::int32_t status) {
 
 std::uint32_t pad32(std::uint32_t value) { return (value + 31U) / 32U * 32U; }
 
+// A device allocation that is freed unless release() hands it on.
+class DeviceBuffer final {
+ public:
+  DeviceBuffer(std::size_t bytes, const char* what) {
+    hip_check(hipMalloc(&pointer_, bytes), what);
+  }
+  ~DeviceBuffer() {
+    if (pointer_) (void)hipFree(pointer_);
+  }
+  DeviceBuffer(const DeviceBuffer&) = delete;
+  DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+  [[nodiscard]] void* get() const noexcept { return pointer_; }
+  [[nodiscard]] void* release() noexcept {
+    void* pointer = pointer_;
+    pointer_ = nullptr;
+    return pointer;
+  }
+
+ private:
+  void* pointer_{};
+};
+
 std::uint64_t request_parameter(const er::ProgramRequestContext& request,
                                 std::string_view name) {
   const auto found = request.parameters.find(name);
@@ -35,6 +57,17 @@ std::uint64_t request_parameter(const er::ProgramRequestContext& request,
     throw std::runtime_error("request parameter is absent: " +
                              std::string(name));
   return found->second;
+}
+
+// The penalty a request asks for: the parameter is biased by 2,000,000 ppm so
+// that negative penalties travel as unsigned values
+// (runtime/tools/moe_vm_runner.cpp:318-347, dense_fp4_provider.cpp:8336-8341).
+double presence_penalty_of(const er::ProgramRequestContext& request) {
+  const auto biased =
+      request_parameter(request, "sampling_presence_penalty_biased_ppm");
+  if (biased > 4'000'000U)
+    throw std::runtime_error("sampling presence penalty is invalid");
+  return (static_cast<double>(biased) - 2'000'000.0) / 1'000'000.0;
 }
 
 er::ExactDecodeExecutionHandle completed_exact(
@@ -151,6 +184,13 @@ Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
   if (g_.kv_encoding == KvEncoding::fp16 &&
       g_.query_heads / g_.kv_heads > 16U)
     throw std::invalid_argument("exact F16 KV supports at most 16 grouped heads");
+  // what one attention workgroup holds: three 16-row tiles of (row, grouped
+  // query head) pairs, two at head_dim 256 - for every cache kind
+  if ((g_.draft_depth + 1U) * (g_.query_heads / g_.kv_heads) >
+      (g_.head_dim == 256U ? 32U : 48U))
+    throw std::invalid_argument(
+        "(draft_depth + 1) * (query_heads / kv_heads) exceeds the attention "
+        "kernels' 48 rows (32 at head_dim 256)");
   hipStream_t stream{};
   hip_check(hipStreamCreate(&stream), "create provider stream");
   stream_ = stream;
@@ -268,6 +308,12 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
                                                kMaximumGpuSamplingTopK, max_rows_)));
   select_workspace_ = device_alloc(select_workspace_bytes_);
   argmax_tokens_ = static_cast<std::uint32_t*>(device_alloc(rows * 4U));
+  presence_ = static_cast<std::uint8_t*>(device_alloc(g_.vocabulary));
+  proposal_presence_ = static_cast<std::uint8_t*>(device_alloc(g_.vocabulary));
+  hip_check(hipMemset(presence_, 0, g_.vocabulary), "clear presence bytes");
+  hip_check(hipMemset(proposal_presence_, 0, g_.vocabulary),
+            "clear presence bytes");
+  mark_tokens_ = static_cast<std::uint32_t*>(device_alloc(8U * 4U));
   // top-k logits of up to 8 rows, then their tokens: one buffer, one readback
   top_logits_ = static_cast<float*>(
       device_alloc(8U * kMaximumGpuSamplingTopK * (4U + 4U)));
@@ -351,19 +397,18 @@ DeviceFp4Matrix Mi355DenseFp4Provider::upload_matrix(
       tensor.scale_offset + scale_bytes > tensor.value.bytes)
     throw std::runtime_error("FP4 tensor geometry mismatch: " + tensor.name);
 
-  void* staged_codes{};
-  void* staged_scales{};
-  hip_check(hipMalloc(&staged_codes, code_bytes), "allocate FP4 weights");
-  hip_check(hipMalloc(&staged_scales, scale_bytes), "allocate FP4 scales");
-  hip_check(hipMemcpy(staged_codes, tensor.value.data + tensor.data_offset,
+  DeviceBuffer staged_codes(code_bytes, "allocate FP4 weights");
+  DeviceBuffer staged_scales(scale_bytes, "allocate FP4 scales");
+  hip_check(hipMemcpy(staged_codes.get(), tensor.value.data + tensor.data_offset,
                       code_bytes, hipMemcpyHostToDevice),
             "upload FP4 weights");
-  hip_check(hipMemcpy(staged_scales, tensor.value.data + tensor.scale_offset,
-                      scale_bytes, hipMemcpyHostToDevice),
+  hip_check(hipMemcpy(staged_scales.get(),
+                      tensor.value.data + tensor.scale_offset, scale_bytes,
+                      hipMemcpyHostToDevice),
             "upload FP4 scales");
   DeviceFp4Matrix matrix;
-  matrix.descriptor = {static_cast<const std::uint8_t*>(staged_codes),
-                       staged_scales,
+  matrix.descriptor = {static_cast<const std::uint8_t*>(staged_codes.get()),
+                       staged_scales.get(),
                        rows,
                        columns,
                        padded,
@@ -371,32 +416,31 @@ DeviceFp4Matrix Mi355DenseFp4Provider::upload_matrix(
                                : std::uint32_t{QLLM_SCALE_UE8M0_BLOCK32},
                        QLLM_LAYOUT_ROW_MAJOR,
                        0U};
+  const auto keep = [this, &matrix](DeviceBuffer& codes, DeviceBuffer& scales) {
+    allocations_.reserve(allocations_.size() + 2U);
+    matrix.weights = codes.get();
+    matrix.scales = scales.get();
+    allocations_.push_back(codes.release());
+    allocations_.push_back(scales.release());
+  };
   if (tiled && padded % 64U == 0U) {
-    void* packed_codes{};
-    void* packed_scales{};
     // tile height 0: full 32-row tiles
-    hip_check(hipMalloc(&packed_codes,
-                        qllm_fp4_packed_weight_bytes(rows, padded, 0U)),
-              "allocate tiled FP4 weights");
-    hip_check(hipMalloc(&packed_scales,
-                        qllm_fp4_packed_scale_bytes(
-                            rows, padded, matrix.descriptor.scale_scheme, 0U)),
-              "allocate tiled FP4 scales");
+    DeviceBuffer packed_codes(qllm_fp4_packed_weight_bytes(rows, padded, 0U),
+                              "allocate tiled FP4 weights");
+    DeviceBuffer packed_scales(
+        qllm_fp4_packed_scale_bytes(rows, padded,
+                                    matrix.descriptor.scale_scheme, 0U),
+        "allocate tiled FP4 scales");
     qllm_fp4_matrix packed{};
-    status_check(qllm_fp4_prepack(&matrix.descriptor, 0U, packed_codes,
-                                  packed_scales, &packed, stream_));
+    status_check(qllm_fp4_prepack(&matrix.descriptor, 0U, packed_codes.get(),
+                                  packed_scales.get(), &packed, stream_));
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
               "prepack FP4 weights");
-    (void)hipFree(staged_codes);
-    (void)hipFree(staged_scales);
     matrix.descriptor = packed;
-    staged_codes = packed_codes;
-    staged_scales = packed_scales;
+    keep(packed_codes, packed_scales);   // the row-major copies are freed
+  } else {
+    keep(staged_codes, staged_scales);
   }
-  matrix.weights = staged_codes;
-  matrix.scales = staged_scales;
-  allocations_.push_back(staged_codes);
-  allocations_.push_back(staged_scales);
   weight_bytes_ += code_bytes + scale_bytes;
   return matrix;
 }
@@ -418,18 +462,18 @@ DeviceFp4Matrix Mi355DenseFp4Provider::concatenate_rows(
   const std::size_t row_code_bytes = padded / 2U;
   const std::size_t row_scale_bytes =
       block16 ? std::size_t{padded / 16U} * 2U : padded / 32U;
-  void* codes{};
-  void* scales{};
-  hip_check(hipMalloc(&codes, rows * row_code_bytes), "allocate joined weights");
-  hip_check(hipMalloc(&scales, rows * row_scale_bytes), "allocate joined scales");
+  DeviceBuffer codes(rows * row_code_bytes, "allocate joined weights");
+  DeviceBuffer scales(rows * row_scale_bytes, "allocate joined scales");
   std::size_t row = 0;
   for (const auto& part : parts) {
     const std::uint32_t part_rows = part.descriptor.rows;
-    hip_check(hipMemcpy(static_cast<std::uint8_t*>(codes) + row * row_code_bytes,
+    hip_check(hipMemcpy(static_cast<std::uint8_t*>(codes.get()) +
+                            row * row_code_bytes,
                         part.weights, part_rows * row_code_bytes,
                         hipMemcpyDeviceToDevice),
               "join weights");
-    hip_check(hipMemcpy(static_cast<std::uint8_t*>(scales) + row * row_scale_bytes,
+    hip_check(hipMemcpy(static_cast<std::uint8_t*>(scales.get()) +
+                            row * row_scale_bytes,
                         part.scales, part_rows * row_scale_bytes,
                         hipMemcpyDeviceToDevice),
               "join scales");
@@ -442,34 +486,33 @@ DeviceFp4Matrix Mi355DenseFp4Provider::concatenate_rows(
   }
   DeviceFp4Matrix joined;
   joined.descriptor = first;
-  joined.descriptor.weights = static_cast<const std::uint8_t*>(codes);
-  joined.descriptor.scales = scales;
+  joined.descriptor.weights = static_cast<const std::uint8_t*>(codes.get());
+  joined.descriptor.scales = scales.get();
   joined.descriptor.rows = rows;
+  const auto keep = [this, &joined](DeviceBuffer& kept_codes,
+                                    DeviceBuffer& kept_scales) {
+    allocations_.reserve(allocations_.size() + 2U);
+    joined.weights = kept_codes.get();
+    joined.scales = kept_scales.get();
+    allocations_.push_back(kept_codes.release());
+    allocations_.push_back(kept_scales.release());
+  };
   if (padded % 64U == 0U) {
-    void* packed_codes{};
-    void* packed_scales{};
-    hip_check(hipMalloc(&packed_codes,
-                        qllm_fp4_packed_weight_bytes(rows, padded, 0U)),
-              "allocate tiled FP4 weights");
-    hip_check(hipMalloc(&packed_scales,
-                        qllm_fp4_packed_scale_bytes(rows, padded,
-                                                    first.scale_scheme, 0U)),
-              "allocate tiled FP4 scales");
+    DeviceBuffer packed_codes(qllm_fp4_packed_weight_bytes(rows, padded, 0U),
+                              "allocate tiled FP4 weights");
+    DeviceBuffer packed_scales(
+        qllm_fp4_packed_scale_bytes(rows, padded, first.scale_scheme, 0U),
+        "allocate tiled FP4 scales");
     qllm_fp4_matrix packed{};
-    status_check(qllm_fp4_prepack(&joined.descriptor, 0U, packed_codes,
-                                  packed_scales, &packed, stream_));
+    status_check(qllm_fp4_prepack(&joined.descriptor, 0U, packed_codes.get(),
+                                  packed_scales.get(), &packed, stream_));
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
               "prepack joined FP4 weights");
-    (void)hipFree(codes);
-    (void)hipFree(scales);
     joined.descriptor = packed;
-    codes = packed_codes;
-    scales = packed_scales;
+    keep(packed_codes, packed_scales);
+  } else {
+    keep(codes, scales);
   }
-  joined.weights = codes;
-  joined.scales = scales;
-  allocations_.push_back(codes);
-  allocations_.push_back(scales);
   return joined;
 }
 
@@ -669,12 +712,42 @@ void Mi355DenseFp4Provider::finish_mtp_weights() {
 }
 
 er::CreateOperationRequestStateResult
-Mi355DenseFp4Provider::create_request_state(const er::ProgramRequestContext&) {
+Mi355DenseFp4Provider::create_request_state(
+    const er::ProgramRequestContext& request) {
   try {
+    std::lock_guard lock(mutex_);
+    // the sampling profile check of dense_fp4_provider.cpp:5502-5513
+    const auto temperature = request.parameters.find("sampling_temperature_ppm");
+    if (temperature != request.parameters.end() && temperature->second != 0U) {
+      const auto first = request.parameters.find("sampling_first_output_position");
+      const auto presence =
+          request.parameters.find("sampling_presence_penalty_biased_ppm");
+      if (first == request.parameters.end() || first->second >= g_.max_context ||
+          presence == request.parameters.end() || presence->second > 4'000'000U)
+        throw std::runtime_error("request has an invalid sampling profile");
+    }
+    hip_check(hipMemsetAsync(presence_, 0, g_.vocabulary,
+                             static_cast<hipStream_t>(stream_)),
+              "zero request sampling presence");
     return {er::Status::success(), std::make_shared<DenseFp4RequestState>()};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
   }
+}
+
+void Mi355DenseFp4Provider::mark_presence(
+    std::uint8_t* emitted, std::span<const std::uint32_t> tokens) {
+  if (tokens.empty()) return;
+  if (tokens.size() > 8U) throw std::runtime_error("too many presence marks");
+  const auto stream = static_cast<hipStream_t>(stream_);
+  // the pinned words are free: every pass that used them ended with a wait
+  std::copy(tokens.begin(), tokens.end(), staging_->marks);
+  hip_check(hipMemcpyAsync(mark_tokens_, staging_->marks, tokens.size() * 4U,
+                           hipMemcpyHostToDevice, stream),
+            "upload presence marks");
+  status_check(qllm_mark_presence(emitted, mark_tokens_,
+                                  static_cast<std::uint32_t>(tokens.size()),
+                                  g_.vocabulary, stream_));
 }
 
 // Records where the verified stream stands after prefill / a previous step
@@ -712,10 +785,18 @@ er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
     state->mtp_length = synchronization.first_target_position;
     if (mtp_.ready) {
       const auto sample_position = synchronization.first_target_position + rows;
+      if (synchronization.produce_final_draft)
+        hip_check(hipMemcpyAsync(proposal_presence_, presence_, g_.vocabulary,
+                                 hipMemcpyDeviceToDevice,
+                                 static_cast<hipStream_t>(stream_)),
+                  "initialize speculative proposal presence");
       auto draft = run_mtp(*state, synchronization.next_tokens, hidden_,
                            synchronization.produce_final_draft,
                            synchronization.produce_final_draft
                                ? &synchronization.request
+                               : nullptr,
+                           synchronization.produce_final_draft
+                               ? proposal_presence_
                                : nullptr,
                            sample_position, 1U);
       if (synchronization.produce_final_draft) {
@@ -1255,7 +1336,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
             const std::uint32_t batch = std::min(max_rows_, pairs - row);
             (void)run_mtp(*state, tokens.subspan(done + row + 1U, batch),
                           prefill_hidden_ + std::size_t{row} * g_.hidden, false,
-                          nullptr, 0U, 0U);
+                          nullptr, nullptr, 0U, 0U);
           }
         }
       }
@@ -1282,8 +1363,11 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
         // the last pair, then the first drafts (as synchronize does)
         const std::uint32_t last[1] = {predicted};
         const auto sample_position = first_position + count;
+        hip_check(hipMemcpyAsync(proposal_presence_, presence_, g_.vocabulary,
+                                 hipMemcpyDeviceToDevice, hip_stream),
+                  "initialize speculative proposal presence");
         auto draft = run_mtp(*state, last, hidden_, true, &request,
-                             sample_position, 1U);
+                             proposal_presence_, sample_position, 1U);
         if (!draft) throw std::runtime_error("prompt prefill produced no draft");
         const auto reserved = request.parameters.find("reserved_context_tokens");
         const auto context_limit =
@@ -1515,11 +1599,22 @@ er::Status Mi355DenseFp4Provider::synchronize() {
 // selects the whole-vocabulary path of the scalar sampler (sample_token,
 // :773-799): the row is copied to the host and ordered there.
 er::SamplingDistribution Mi355DenseFp4Provider::distribution_from_logits(
-    const float* row_logits, std::uint32_t vocabulary,
-    const std::uint32_t* device_argmax,
-    const er::ProgramRequestContext& request) {
+    float* row_logits, std::uint32_t vocabulary, std::uint32_t* device_argmax,
+    const er::ProgramRequestContext& request, const std::uint8_t* presence) {
   const auto stream = static_cast<hipStream_t>(stream_);
+  const auto penalty = presence_penalty_of(request);
   const auto temperature = request_parameter(request, "sampling_temperature_ppm");
+  if (penalty != 0.0) {
+    if (!presence) throw std::runtime_error("sampling presence state is absent");
+    status_check(qllm_apply_presence_penalty(row_logits, presence, vocabulary,
+                                             static_cast<float>(penalty),
+                                             stream_));
+    // the arg-max the pass left behind was taken before the penalty
+    if (temperature == 0U)
+      status_check(qllm_argmax_batch(row_logits, vocabulary, 1U, device_argmax,
+                                     select_workspace_, select_workspace_bytes_,
+                                     stream_));
+  }
   if (temperature == 0U) {
     std::uint32_t token{};
     hip_check(hipMemcpyAsync(&token, device_argmax, sizeof(token),
@@ -1801,8 +1896,8 @@ void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained,
 std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
     DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
     const float* previous_hidden, bool produce_logits,
-    const er::ProgramRequestContext* request, std::uint32_t sample_position,
-    std::uint32_t random_stream) {
+    const er::ProgramRequestContext* request, const std::uint8_t* presence,
+    std::uint32_t sample_position, std::uint32_t random_stream) {
   if (!mtp_.ready || tokens.empty() || tokens.size() > max_rows_ ||
       !previous_hidden || state.mtp_length + tokens.size() > g_.max_context)
     throw std::runtime_error("invalid MTP microbatch");
@@ -1825,7 +1920,7 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
   DraftPrediction result;
   if (request) {
     result.distribution = distribution_from_logits(
-        mtp_logits_, g_.draft_vocabulary, mtp_argmax_, *request);
+        mtp_logits_, g_.draft_vocabulary, mtp_argmax_, *request, presence);
     result.token = er::sample_distribution(
         result.distribution,
         er::counter_uniform(request_parameter(*request, "sampling_seed"),
@@ -1837,6 +1932,9 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
     hip_check(hipStreamSynchronize(hip_stream), "copy final MTP draft token");
     result.distribution.entries.push_back({result.token, 1.0});
   }
+  // logits without a finite maximum select no token
+  if (result.token >= g_.draft_vocabulary)
+    throw std::runtime_error("MTP draft token is outside the draft vocabulary");
   return result;
 }
 
@@ -1888,6 +1986,11 @@ void Mi355DenseFp4Provider::propose_with_graphs(
               "copy MTP draft tokens");
     hip_check(hipStreamSynchronize(stream), "copy MTP draft tokens");
     for (std::uint32_t depth = 0; depth < drafts; ++depth) {
+      // logits without a finite maximum select no token (0xffffffff); the
+      // chained pass embedded a row of zeros for it and every kernel ran
+      if (chosen[depth] >= g_.draft_vocabulary)
+        throw std::runtime_error(
+            "MTP draft token is outside the draft vocabulary");
       DraftPrediction prediction;
       prediction.token = chosen[depth];
       prediction.distribution.entries.push_back({chosen[depth], 1.0});
@@ -1908,8 +2011,9 @@ void Mi355DenseFp4Provider::propose_with_graphs(
       }
       launch_mtp_graph(depth ? 1U : rows, depth != 0U);
       DraftPrediction prediction;
+      // a request with a presence penalty takes the uncaptured passes
       prediction.distribution = distribution_from_logits(
-          mtp_logits_, g_.draft_vocabulary, mtp_argmax_, request);
+          mtp_logits_, g_.draft_vocabulary, mtp_argmax_, request, nullptr);
       prediction.token = er::sample_distribution(
           prediction.distribution,
           er::counter_uniform(seed, committed_length + (depth ? depth - 1U : 0U),
@@ -1938,6 +2042,9 @@ void Mi355DenseFp4Provider::extend_mtp_rollout(
   if (committed_length + 1U >= context_limit)
     throw std::runtime_error("MTP rollout root exceeds context");
   state.draft_predictions.push_back(std::move(first));
+  // every draft is present for the drafts after it (:8822-8847)
+  const std::uint32_t root[1] = {state.draft_predictions.back().token};
+  mark_presence(proposal_presence_, root);
   while (state.draft_predictions.size() < g_.draft_depth &&
          state.mtp_length + 2U < context_limit) {
     // the next pass reads the proposer's own last hidden state before it
@@ -1945,10 +2052,13 @@ void Mi355DenseFp4Provider::extend_mtp_rollout(
     const auto sample_position = state.mtp_length;
     const std::uint32_t token[1] = {state.draft_predictions.back().token};
     auto prediction = run_mtp(
-        state, token, mtp_last_hidden_, true, &request, sample_position,
+        state, token, mtp_last_hidden_, true, &request, proposal_presence_,
+        sample_position,
         1U + static_cast<std::uint32_t>(state.draft_predictions.size()));
     if (!prediction) throw std::runtime_error("MTP rollout produced no proposal");
     state.draft_predictions.push_back(std::move(*prediction));
+    const std::uint32_t drafted[1] = {state.draft_predictions.back().token};
+    mark_presence(proposal_presence_, drafted);
   }
   state.draft_valid = !state.draft_predictions.empty();
   // speculative rows of the proposer's cache are overwritten by the next pass
@@ -1989,9 +2099,23 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
                                            invocation.position);
     if (!status.ok()) throw std::runtime_error(std::string(status.message()));
 
+    // Row r is penalised at the tokens emitted before this step and at the
+    // drafts of the rows before it (:11182-11202); tokens_[1..] are the drafts.
+    const auto penalty = presence_penalty_of(invocation.request);
+    const bool greedy =
+        request_parameter(invocation.request, "sampling_temperature_ppm") == 0U;
+    if (penalty != 0.0) {
+      status_check(qllm_apply_presence_penalty_rows(
+          logits_, g_.vocabulary, presence_, tokens_ + 1, rows, g_.vocabulary,
+          static_cast<float>(penalty), stream_));
+      if (greedy)
+        status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows,
+                                       argmax_tokens_, select_workspace_,
+                                       select_workspace_bytes_, stream_));
+    }
     std::vector<er::SamplingDistribution> target_distributions;
     target_distributions.reserve(rows);
-    if (request_parameter(invocation.request, "sampling_temperature_ppm") == 0U) {
+    if (greedy) {
       // greedy: the rows' arg-max tokens in one copy and one wait
       const auto stream = static_cast<hipStream_t>(stream_);
       hip_check(hipMemcpyAsync(staging_->download, argmax_tokens_,
@@ -2005,10 +2129,13 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       target_distributions = distributions_from_top_k(
           logits_, g_.vocabulary, g_.vocabulary, rows, invocation.request);
     } else {
+      // whole-vocabulary candidates; the penalty has been applied above
+      er::ProgramRequestContext unpenalised = invocation.request;
+      unpenalised.parameters["sampling_presence_penalty_biased_ppm"] = 2'000'000U;
       for (std::uint32_t row = 0; row < rows; ++row)
         target_distributions.push_back(distribution_from_logits(
             logits_ + std::size_t{row} * g_.vocabulary, g_.vocabulary,
-            argmax_tokens_ + row, invocation.request));
+            argmax_tokens_ + row, unpenalised, nullptr));
     }
 
     const auto seed = request_parameter(invocation.request, "sampling_seed");
@@ -2036,6 +2163,15 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
               300U));
 
     const auto positions_advanced = static_cast<std::uint32_t>(accepted + 1U);
+    {
+      // accepted drafts and the next token are emitted tokens from here on
+      // (:11261-11270)
+      std::vector<std::uint32_t> emitted_now;
+      for (std::size_t index = 0; index < accepted; ++index)
+        emitted_now.push_back(state->draft_predictions[index].token);
+      emitted_now.push_back(next_token);
+      mark_presence(presence_, emitted_now);
+    }
     if (mtp_.ready) {
       // advance the proposer over the accepted drafts and the next token (row r
       // pairs the token at position + r + 1 with the target's hidden state at
@@ -2049,12 +2185,19 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       state->mtp_length = invocation.position;
       state->draft_valid = false;
       state->draft_predictions.clear();
-      if (future_exact && use_graphs_) {
+      // The captured passes select their drafts on the device without the
+      // presence bytes; a request with a penalty takes the uncaptured ones.
+      if (future_exact && use_graphs_ && penalty == 0.0) {
         propose_with_graphs(*state, mtp_tokens, invocation.request,
                             invocation.context_limit);
       } else {
+        hip_check(hipMemcpyAsync(proposal_presence_, presence_, g_.vocabulary,
+                                 hipMemcpyDeviceToDevice,
+                                 static_cast<hipStream_t>(stream_)),
+                  "initialize next MTP rollout presence");
         auto first = run_mtp(*state, mtp_tokens, hidden_, future_exact,
                              future_exact ? &invocation.request : nullptr,
+                             future_exact ? proposal_presence_ : nullptr,
                              invocation.position + positions_advanced, 1U);
         if (future_exact) {
           if (!first)

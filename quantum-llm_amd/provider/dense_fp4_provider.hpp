@@ -232,9 +232,11 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       const float* logits, std::uint32_t vocabulary, std::size_t stride,
       std::uint32_t rows, const er::ProgramRequestContext& request);
   er::SamplingDistribution distribution_from_logits(
-      const float* row_logits, std::uint32_t vocabulary,
-      const std::uint32_t* device_argmax,
-      const er::ProgramRequestContext& request);
+      float* row_logits, std::uint32_t vocabulary, std::uint32_t* device_argmax,
+      const er::ProgramRequestContext& request, const std::uint8_t* presence);
+  // emitted[token] = 1 for every token (one upload, one launch)
+  void mark_presence(std::uint8_t* emitted,
+                     std::span<const std::uint32_t> tokens);
   // One proposer pass over `tokens` (run_mtp, dense_fp4_provider.cpp:8681-
   // 8792): row r embeds tokens[r], takes previous_hidden row r (device, F32),
   // is cached at position mtp_length + r and rotated at mtp_length + r + 1.
@@ -242,8 +244,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   std::optional<DraftPrediction> run_mtp(
       DenseFp4RequestState& state, std::span<const std::uint32_t> tokens,
       const float* previous_hidden, bool produce_logits,
-      const er::ProgramRequestContext* request, std::uint32_t sample_position,
-      std::uint32_t random_stream);
+      const er::ProgramRequestContext* request, const std::uint8_t* presence,
+      std::uint32_t sample_position, std::uint32_t random_stream);
   void enqueue_attention(std::uint32_t index, std::uint32_t rows,
                          std::uint32_t first_position, bool deferred_positions,
                          float* query, float* key, const float* value,
@@ -317,6 +319,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
     std::uint32_t download[8];
     float top_logits[8 * 64];            // top-k readback: logits of all rows,
     std::uint32_t top_tokens[8 * 64];    // then their tokens
+    std::uint32_t marks[8];              // tokens whose presence byte is set
   };
   HostStaging* staging_ = nullptr;
   float* projection_partials_ = nullptr;   // [splits][rows][hidden]
@@ -324,6 +327,13 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void* select_workspace_{};
   std::size_t select_workspace_bytes_{};
   std::uint32_t* argmax_tokens_{};
+  // Presence bytes of the request's emitted tokens and the scratch copy that
+  // also carries the drafts of the rollout in progress (sampling_presence_,
+  // sampling_proposal_presence_, dense_fp4_provider.cpp:4242-4243); one
+  // request at a time, as the KV cache is.
+  std::uint8_t* presence_{};
+  std::uint8_t* proposal_presence_{};
+  std::uint32_t* mark_tokens_{};
   float* top_logits_{};
   std::uint32_t* top_tokens_{};
 

@@ -229,11 +229,34 @@ extern "C" int32_t qllm_provider_begin_request(qllm_provider* provider,
   provider->request.parameters["sampling_seed"] = seed;
   provider->request.parameters["sampling_presence_penalty_biased_ppm"] =
       2'000'000U;
+  provider->request.parameters["sampling_first_output_position"] = 0U;
   provider->request.parameters["exact_decode_enabled"] = 1U;
   auto result = provider->provider->create_request_state(provider->request);
   if (!result.status.ok()) return from_status(result.status);
   provider->state = result.state;
   return QLLM_OK;
+}
+
+extern "C" int32_t qllm_provider_begin_request_with(qllm_provider* provider,
+                                                    const char* const* names,
+                                                    const uint64_t* values,
+                                                    uint32_t count) {
+  if (!provider || (count && (!names || !values)))
+    return fail(QLLM_INVALID_ARGUMENT, "request parameters are invalid");
+  try {
+    provider->request = {};
+    for (uint32_t index = 0; index < count; ++index) {
+      if (!names[index])
+        return fail(QLLM_INVALID_ARGUMENT, "request parameter name is null");
+      provider->request.parameters[names[index]] = values[index];
+    }
+    auto result = provider->provider->create_request_state(provider->request);
+    if (!result.status.ok()) return from_status(result.status);
+    provider->state = result.state;
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
 }
 
 extern "C" int32_t qllm_provider_synchronize(qllm_provider* provider,

@@ -127,6 +127,8 @@ SIGNATURES = {
     "qllm_topk_batch_workspace_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_topk_logits_batch": (c_int32, [c_void_p, c_uint32, c_size_t, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "qllm_apply_presence_penalty": (c_int32, [c_void_p, c_void_p, c_uint32, c_float, c_void_p]),
+    "qllm_apply_presence_penalty_rows": (c_int32, [c_void_p, c_size_t, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_void_p]),
+    "qllm_mark_presence": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fill_random": (c_int32, [c_void_p, c_size_t, c_uint32, c_uint64, c_void_p]),
 }
 

@@ -42,6 +42,7 @@ SIGNATURES = {
     "qllm_provider_load_synthetic_weights": (c_int32, [c_void_p, c_uint64]),
     "qllm_provider_prefill_synthetic_kv": (c_int32, [c_void_p, c_uint32, c_uint64]),
     "qllm_provider_begin_request": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint64]),
+    "qllm_provider_begin_request_with": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32]),
     "qllm_provider_synchronize": (c_int32, [c_void_p, c_uint32, c_uint32]),
     "qllm_provider_set_drafts": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_void_p]),
     "qllm_provider_verify": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint32)]),
@@ -165,6 +166,14 @@ class Provider:
                       min_p_ppm=0, seed=0):
         _check(self.lib.qllm_provider_begin_request(
             self.handle, temperature_ppm, top_p_ppm, top_k, min_p_ppm, seed))
+
+    def begin_request_with(self, **parameters):
+        """create_request_state with the request's parameter map given by name."""
+        import numpy as np
+        names = (c_char_p * len(parameters))(*[n.encode() for n in parameters])
+        values = np.array(list(parameters.values()), dtype=np.uint64)
+        _check(self.lib.qllm_provider_begin_request_with(
+            self.handle, names, values.ctypes.data, len(parameters)))
 
     def prefill(self, tokens, first_position=0):
         """Prompt prefill; returns the greedy prediction after the prompt."""

@@ -333,6 +333,15 @@ def argmax(values):
     return oracle().qo_argmax(_p(values), c_uint32(values.size))
 
 
+def presence_penalty(logits, emitted, penalty):
+    """logits - penalty where emitted (a copy; qo_presence_penalty)."""
+    out = np.ascontiguousarray(logits, dtype=np.float32).copy()
+    emitted = np.ascontiguousarray(emitted, dtype=np.uint8)
+    oracle().qo_presence_penalty(_p(out), _p(emitted), c_uint32(out.size),
+                                 ctypes.c_float(penalty))
+    return out
+
+
 def topk(values, k):
     values = np.ascontiguousarray(values, dtype=np.float32)
     out_v = np.empty(k, dtype=np.float32)

@@ -188,6 +188,75 @@ def test_captured_proposer_passes_equal_the_eager_ones(device, monkeypatch,
         assert np.array_equal(eager_step[4], graph_step[4])
 
 
+@pytest.mark.parametrize("temperature,top_k", [(0, 0), (800000, 20)])
+def test_decode_cycle_with_a_presence_penalty(device, temperature, top_k):
+    """The proposer penalises its draft logits at the emitted tokens and at the
+    drafts of the rollout so far (dense_fp4_provider.cpp:8822-8847, 11290-11296):
+    the last draft is the arg-max of the penalised logits it left behind, the
+    target's acceptance is the oracle's on the penalised target logits, and a
+    repeated run gives the same stream."""
+    streams = []
+    for attempt in range(2):
+        rng, model, provider = make("reference", 31)
+        V = model.vocabulary
+        provider.run_target(rng.integers(0, V, 5).astype(np.uint32), 0)
+        position, token = 5, 7
+        provider.begin_request_with(
+            reserved_context_tokens=256, sampling_temperature_ppm=temperature,
+            sampling_top_p_ppm=950000, sampling_top_k=top_k, sampling_min_p_ppm=0,
+            sampling_presence_penalty_biased_ppm=4000000,      # penalty 2.0
+            sampling_first_output_position=0, sampling_seed=77, exact_decode_enabled=1)
+        provider.synchronize(token, position)
+        stream, emitted_tokens = [], set()
+        for step in range(6):
+            drafts = provider.drafts()
+            assert len(drafts) == 4
+            if temperature == 0:
+                _, draft_logits = provider.mtp_state()
+                assert drafts[-1] == ol.argmax(draft_logits)
+            emitted, next_token, advanced = provider.verify(token, position, 256)
+            if temperature == 0:
+                accepted, want_next = ol.accept_greedy(
+                    provider.logits(5), np.array(drafts, dtype=np.uint32))
+                assert advanced == accepted + 1 and next_token == want_next
+            assert emitted == [token, *drafts[:advanced - 1]]
+            stream += emitted
+            token, position = next_token, position + advanced
+        streams.append(stream)
+        provider.close()
+    assert streams[0] == streams[1]
+
+
+def test_draft_logits_without_a_finite_maximum_are_reported(device):
+    """A draft norm full of NaN makes every draft logit NaN: the device-side
+    arg-max selects no token, the chained pass embeds zeros for it, every
+    kernel runs to its end and the step reports the failure."""
+    rng = np.random.default_rng(5)
+    c = CONFIGS["baseline"]
+    model = step_oracle.TinyModel(
+        rng, 256, 512, 2, 8, 2, c["head_dim"], 256, c["scheme"],
+        output_gated=c["output_gated"], qk_norm=c["qk_norm"],
+        zero_centered=c["zero_centered"], rotary_dim=c["rotary_dim"])
+    model.mtp["draft_norm"][:] = np.nan
+    provider = step_oracle.build_provider(model, qp, mtp=True,
+                                          draft_vocabulary=DRAFT_VOCABULARY)
+    provider.run_target(rng.integers(0, 256, 5).astype(np.uint32), 0)
+    provider.begin_request(temperature_ppm=0)
+    with pytest.raises(qp.ProviderError) as error:      # uncaptured passes
+        provider.synchronize(3, 5)
+    assert "draft" in str(error.value)
+    # the captured rollout at the end of a verify step chains its four passes on
+    # the device: the token nobody selected (0xffffffff) is embedded as zeros
+    provider.set_drafts(np.array([1, 2, 3, 4], dtype=np.uint32))
+    with pytest.raises(qp.ProviderError) as error:
+        provider.verify(3, 5, 256)
+    assert "draft" in str(error.value)
+    # the device is intact: the target still runs and gives finite logits
+    provider.run_target(rng.integers(0, 256, 5).astype(np.uint32), 0)
+    assert np.isfinite(provider.logits(5)).all()
+    provider.close()
+
+
 def test_rollout_stops_at_the_context_limit(device):
     rng, model, provider = make("baseline", 37, max_context=64)
     V = model.vocabulary

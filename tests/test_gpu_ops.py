@@ -173,6 +173,35 @@ def test_presence_penalty_known_answer(device):
     assert logits.cpu().numpy().tolist() == [3.0, 0.5, -0.5, -1.0]
 
 
+def test_presence_penalty_over_the_rows_of_a_verify_step(device):
+    """Row r is penalised at the emitted tokens and at the drafts of the rows
+    before it; the oracle does it row by row, marking a draft in between."""
+    rng = np.random.default_rng(8)
+    V, stride, rows = 151936, 151936 + 64, 5
+    logits = rng.standard_normal((rows, stride)).astype(np.float32)
+    emitted = (rng.random(V) < 0.01).astype(np.uint8)
+    drafts = np.array([17, 90000, 17, V - 1], dtype=np.uint32)   # a repeated draft
+    want = logits.copy()
+    present = emitted.copy()
+    for row in range(rows):
+        want[row, :V] = ol.presence_penalty(logits[row, :V], present, 1.5)
+        if row < rows - 1:
+            present[drafts[row]] = 1
+    d_logits = gu.device_tensor(logits, device)
+    d_emitted = gu.device_tensor(emitted, device)
+    d_drafts = gu.device_tensor(drafts, device)
+    qh.call("qllm_apply_presence_penalty_rows", qh.ptr(d_logits), stride,
+            qh.ptr(d_emitted), qh.ptr(d_drafts), rows, V, 1.5, None)
+    # marks: tokens on the device, entries outside the vocabulary ignored
+    marks = gu.device_tensor(np.array([5, V - 1, 0xffffffff, 5], np.uint32), device)
+    qh.call("qllm_mark_presence", qh.ptr(d_emitted), qh.ptr(marks), 4, V, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_logits.cpu().numpy(), want)      # padding untouched too
+    marked = emitted.copy()
+    marked[[5, V - 1]] = 1
+    assert np.array_equal(d_emitted.cpu().numpy(), marked)
+
+
 def test_query_q8_quantisation_is_byte_exact(device):
     rng = np.random.default_rng(6)
     rows, Q, d = 5, 24, 256

@@ -170,6 +170,108 @@ def test_acceptance_is_bit_exact_on_the_same_logits(device, name):
     provider.close()
 
 
+def request_with(temperature_ppm, top_k, seed, penalty_ppm, **extra):
+    return dict(reserved_context_tokens=256, sampling_temperature_ppm=temperature_ppm,
+                sampling_top_p_ppm=950000, sampling_top_k=top_k, sampling_min_p_ppm=0,
+                sampling_presence_penalty_biased_ppm=2000000 + penalty_ppm,
+                sampling_first_output_position=0, sampling_seed=seed,
+                exact_decode_enabled=1, **extra)
+
+
+@pytest.mark.parametrize("temperature_ppm,top_k", [(0, 0), (900000, 20), (700000, 0)])
+def test_presence_penalty_in_the_verify_step(device, temperature_ppm, top_k):
+    """A request with a presence penalty of 1.5 (and one of -0.75): every row's
+    logits are penalised at the tokens emitted so far and at the drafts of the
+    rows before it, before arg-max / top-k (dense_fp4_provider.cpp:8331-8349,
+    11182-11202, 11261-11270); tokens bit-exact against the oracle applying
+    qo_presence_penalty to the logits the GPU produced."""
+    for penalty_ppm in (1500000, -750000):
+        rng, model, provider = make("baseline", 17)
+        V = model.vocabulary
+        penalty = np.float32(penalty_ppm / 1e6)
+        provider.run_target(rng.integers(0, V, 5).astype(np.uint32), 0)
+        position, token, seed = 5, int(rng.integers(0, V)), 4242
+        provider.begin_request_with(**request_with(temperature_ppm, top_k, seed, penalty_ppm))
+        provider.synchronize(token, position)
+        emitted_so_far = np.zeros(V, dtype=np.uint8)
+        for step in range(4):
+            drafts = rng.integers(0, V, 4).astype(np.uint32)
+            if step:
+                drafts[0] = drafts[2]          # a draft that repeats inside the step
+            rows = np.array([token, *drafts], dtype=np.uint32)
+            provider.run_target(rows, position)
+            raw = provider.logits(5)
+            if temperature_ppm == 0:
+                # make the first draft the penalised arg-max so that it is accepted
+                drafts[0] = ol.argmax(ol.presence_penalty(raw[0], emitted_so_far, penalty))
+                rows[1] = drafts[0]
+                provider.run_target(rows, position)
+                raw = provider.logits(5)
+            if temperature_ppm == 0:
+                provider.set_drafts(drafts)
+                draft_distributions = [(np.array([t], np.uint32), np.array([1.0]))
+                                       for t in drafts]
+            else:
+                draft_distributions = []
+                for t in drafts:
+                    q = rng.dirichlet(np.full(V, 0.1)); q /= q.sum()
+                    q_tokens = np.arange(V, dtype=np.uint32)
+                    if q[t] == 0.0:
+                        q[t] = 1e-6; q /= q.sum()
+                    draft_distributions.append((q_tokens, q))
+                provider.set_drafts(drafts, draft_distributions)
+            got_emitted, got_next, advanced = provider.verify(token, position, 256)
+            # the oracle's statement on the raw logits
+            present = emitted_so_far.copy()
+            penalised = np.empty_like(raw)
+            for row in range(5):
+                penalised[row] = ol.presence_penalty(raw[row], present, penalty)
+                if row < 4:
+                    present[drafts[row]] = 1
+            assert np.array_equal(provider.logits(5), penalised), (penalty_ppm, step)
+            if temperature_ppm == 0:
+                accepted, want_next = ol.accept_greedy(penalised, drafts)
+                assert accepted >= 1
+            else:
+                targets = []
+                for row in range(5):
+                    if top_k:
+                        values, indices = ol.topk(penalised[row], top_k)
+                    else:
+                        indices = np.lexsort((np.arange(V), -penalised[row].astype(np.float64))).astype(np.uint32)
+                        values = penalised[row][indices]
+                    status, t, p = ol.make_sampling_distribution(
+                        values, indices, temperature_ppm, 950000, 0)
+                    assert status == 0
+                    targets.append((t, p))
+                status, accepted, want_next = ol.accept_stochastic(
+                    targets, draft_distributions, drafts.tolist(), seed, position)
+                assert status == 0
+            assert advanced == accepted + 1 and got_next == want_next, (penalty_ppm, step)
+            assert got_emitted == [token, *drafts[:accepted].tolist()]
+            emitted_so_far[drafts[:accepted]] = 1
+            emitted_so_far[got_next] = 1
+            token, position = got_next, position + advanced
+        provider.close()
+
+
+def test_request_profiles_the_provider_turns_down(device):
+    rng, model, provider = make("baseline", 3)
+    with pytest.raises(qp.ProviderError):      # sampled, penalty parameter above 4,000,000
+        provider.begin_request_with(**request_with(700000, 20, 1, 2000001))
+    bad = request_with(700000, 20, 1, 0)
+    del bad["sampling_first_output_position"]
+    with pytest.raises(qp.ProviderError):      # sampled without a first output position
+        provider.begin_request_with(**bad)
+    # a greedy request carries the parameter too, and it is checked when used
+    provider.begin_request_with(**request_with(0, 0, 1, 2000001))
+    provider.synchronize(5, 10)
+    provider.set_drafts(np.array([1, 2, 3, 4], dtype=np.uint32))
+    with pytest.raises(qp.ProviderError):
+        provider.verify(5, 10, 256)
+    provider.close()
+
+
 def test_provider_rejects_invalid_streams(device):
     rng, model, provider = make("baseline", 3)
     provider.begin_request(temperature_ppm=0)
