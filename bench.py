@@ -374,7 +374,12 @@ def main():
         "launches_timed": launches,
     }
     other_kernels = {}
+    qkv_rows = (MODEL["query_heads"] + 2 * MODEL["kv_heads"]) * MODEL["head_dim"]
+    attention_width = MODEL["query_heads"] * MODEL["head_dim"]
     for name, bytes_per_launch in (
+            ("qkv", fp4_bytes(qkv_rows, H) + rows * H * 2 + rows * qkv_rows * 4),
+            ("attention_output", fp4_bytes(H, attention_width) + rows * attention_width * 2
+             + rows * H * 4),
             ("ffn_down", fp4_bytes(H, I) + rows * I * 2 + rows * H * 4),
             ("lm_head", fp4_bytes(vocabulary, H) + rows * H * 2 + rows * vocabulary * 4),
             ("attention", CONTEXT * MODEL["kv_heads"] * 2 * (MODEL["head_dim"] // 2 + 2)

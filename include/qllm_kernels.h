@@ -296,6 +296,27 @@ int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
     uint32_t rotary_dim, float epsilon, float rope_theta,
     int32_t bf16_activations, void* stream);
 
+/* The same operation fed by a q/k/v projection that was computed as K-split
+ * partials (qllm_fp4_gemm_bf16_partial on the matrix holding the query, key
+ * and value rows in that order): partials f32 [partial_count][rows]
+ * [query_heads * query_stride + 2 * kv_heads * head_dim].  Every (row, head)
+ * workgroup first adds its slice of the partials in index order into `query`
+ * (dense rows of query_heads * query_stride floats), `key` and `value`, then
+ * goes on as qllm_qkv_rope_cache_paged_q4h_batch; device_positions, when not
+ * NULL, replaces the two positions as in the deferred form.  The reference
+ * has one thread block per output row group in its projection and no such cut
+ * (runtime/tools/dense_fp4_provider.cpp:7004-7011). */
+int32_t qllm_qkv_rope_cache_paged_q4h_from_partials(
+    const float* partials, uint32_t partial_count, float* query,
+    uint32_t query_stride, float* key, float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, const uint32_t* device_positions,
+    uint32_t rows, uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, void* stream);
+
 /* The same per-head RMSNorm + rotary without the K/V store, for caches that
  * store K/V separately.  replaces gated_gqa_qkv_rope_fp16_batch
  * (runtime/src/cuda/transformer_kernels.cu:3645-3726). */

@@ -147,6 +147,28 @@ int32_t qllm_provider_prefill(qllm_provider* provider, const uint32_t* tokens,
                               uint32_t count, uint32_t first_position,
                               uint32_t* predicted);
 
+/* One batch through the prepared program, operation by operation, the way
+ * the common VM drives a provider (IOperationProvider::execute,
+ * runtime/include/expert/runtime/program_executor.hpp:251-254; the reference's
+ * execute, runtime/tools/dense_fp4_provider.cpp:10680-10992): `rows` tokens at
+ * consecutive `positions` (host arrays), `*next_token` = the head's selection
+ * for the last row under the request's sampling parameters.  With exact decode
+ * enabled in the request the batch then awaits qllm_provider_synchronize_batch. */
+int32_t qllm_provider_execute_program(qllm_provider* provider,
+                                      const uint32_t* tokens,
+                                      const uint32_t* positions, uint32_t rows,
+                                      uint32_t* next_token);
+
+/* synchronize_exact_decode_batch (program_executor.hpp:340-362): next_tokens[r]
+ * is the token after target position first_target_position + r; the proposer
+ * is fed (token, target hidden state) pairs from the batch the program last
+ * executed, and with produce_final_draft the drafts are rolled out. */
+int32_t qllm_provider_synchronize_batch(qllm_provider* provider,
+                                        const uint32_t* next_tokens,
+                                        uint32_t count,
+                                        uint32_t first_target_position,
+                                        int32_t produce_final_draft);
+
 /* Drafts for the next verify step.  distribution_counts[i] entries of
  * (tokens, probabilities) describe draft i's proposal distribution q; a count
  * of 0 means the one-hot distribution on the draft token (greedy). */
@@ -278,6 +300,20 @@ int32_t qllm_model_descriptor_parse(const char* text, size_t text_bytes,
                                     const uint8_t* content_sha256,
                                     uint64_t namespace_base, char* dump,
                                     size_t capacity, size_t* dump_bytes);
+/* Binds a model program against providers described in text ("provider
+ * <name> <priority> <callable 0|1>" lines, each followed by its "capability
+ * <name> <minimum_abi> <maximum_abi>" lines, tab separated) and writes a
+ * canonical report: registration statuses, the bind status, the providers of
+ * the plan and the compiled program (ExecutionProviderRegistry::add / bind,
+ * runtime/src/execution_provider.cpp:10-131; compile_model_program,
+ * runtime/src/model_descriptor.cpp:374-490).  executable != 0 binds callable
+ * providers only. */
+int32_t qllm_model_program_bind(const char* text, size_t text_bytes,
+                                const uint8_t* content_sha256,
+                                uint64_t namespace_base, const char* providers,
+                                int32_t executable, char* dump, size_t capacity,
+                                size_t* dump_bytes);
+
 /* load_model_descriptor_artifact (model_descriptor.hpp:282-285): the file
  * must have expected_bytes bytes and the expected SHA-256. */
 int32_t qllm_model_descriptor_load(const char* path, uint64_t expected_bytes,

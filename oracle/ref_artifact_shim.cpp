@@ -1,7 +1,8 @@
 // C-callable shim over the reference's own artifact reader.  TEST
 // INFRASTRUCTURE ONLY.  Compiled together with the reference sources
-// runtime/src/{model_descriptor,model_artifact,model_tensor_store,sha256,
-// expert_catalog,expert_record}.cpp and core/src/json.cpp, read where they lie
+// runtime/src/{model_descriptor,execution_provider,model_artifact,
+// model_tensor_store,sha256,expert_catalog,expert_record}.cpp and
+// core/src/json.cpp, read where they lie
 // in the reference tree, into oracle/_ref/libqllm_ref_artifact.so.  The shim
 // adds no logic: it calls the reference's functions and prints their results
 // with the same writer (descriptor_dump.hpp) the product uses on its own types.
@@ -11,6 +12,7 @@
 #include "expert/runtime/sha256.hpp"
 
 #include "descriptor_dump.hpp"
+#include "registry_probe.hpp"
 
 #include <algorithm>
 #include <cstdint>
@@ -83,6 +85,18 @@ int qref_model_descriptor_load(const char* path, std::uint64_t expected_bytes,
   copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
             dump_bytes);
   return 0;
+}
+
+// the reference's ExecutionProviderRegistry and compile_model_program
+// (runtime/src/execution_provider.cpp, model_descriptor.cpp:374-490)
+void qref_model_program_bind(const char* text, std::size_t text_bytes,
+                             const std::uint8_t* content_sha256,
+                             std::uint64_t namespace_base, const char* providers,
+                             int executable, char* dump, std::size_t capacity,
+                             std::size_t* dump_bytes) {
+  copy_text(qllm::dump::bind_report({text, text_bytes}, digest_of(content_sha256),
+                                    namespace_base, providers, executable != 0),
+            dump, capacity, dump_bytes);
 }
 
 int qref_artifact_open(const char* root, std::uint32_t mtp_draft_depth,

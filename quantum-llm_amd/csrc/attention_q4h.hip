@@ -875,7 +875,8 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     uint32_t first_cache_position, uint32_t first_rotary_position,
     uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
     uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations,
-    const uint32_t* device_positions) {
+    const uint32_t* device_positions, const float* partials,
+    uint32_t partial_count, uint32_t rows) {
   __shared__ float shared[256];
   __shared__ float rotated[256];
   if (device_positions) {
@@ -884,6 +885,41 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
   }
   const uint32_t row = blockIdx.y;
   const uint32_t lane = threadIdx.x;
+  if (partials) {
+    // The projection arrived as K-split partials f32 [partial_count][rows]
+    // [q rows | k rows | v rows]: this block's slice of query (with its gate
+    // half, if any), or of key and value, is summed in index order first.
+    const uint32_t query_rows = query_heads * query_stride;
+    const uint32_t kv_rows = kv_heads * head_dim;
+    const size_t width = static_cast<size_t>(query_rows) + 2u * kv_rows;
+    const size_t slab = static_cast<size_t>(rows) * width;
+    const float* source = partials + static_cast<size_t>(row) * width;
+    if (blockIdx.x < query_heads) {
+      const uint32_t first = blockIdx.x * query_stride;
+      float* q = query + static_cast<size_t>(row) * query_rows + first;
+      for (uint32_t index = lane; index < query_stride; index += 64u) {
+        float sum = source[first + index];
+        for (uint32_t part = 1; part < partial_count; ++part)
+          sum += source[part * slab + first + index];
+        q[index] = sum;
+      }
+    } else {
+      const uint32_t first = (blockIdx.x - query_heads) * head_dim;
+      float* k = key + static_cast<size_t>(row) * kv_rows + first;
+      float* v = const_cast<float*>(value) + static_cast<size_t>(row) * kv_rows + first;
+      for (uint32_t index = lane; index < head_dim; index += 64u) {
+        float k_sum = source[query_rows + first + index];
+        float v_sum = source[query_rows + kv_rows + first + index];
+        for (uint32_t part = 1; part < partial_count; ++part) {
+          k_sum += source[part * slab + query_rows + first + index];
+          v_sum += source[part * slab + query_rows + kv_rows + first + index];
+        }
+        k[index] = k_sum;
+        v[index] = v_sum;
+      }
+    }
+    __syncthreads();   // one wave: its stores are visible to all its lanes
+  }
   const uint32_t rotary_position = first_rotary_position + row;
   if (blockIdx.x < query_heads) {
     const uint32_t head = blockIdx.x;
@@ -1027,7 +1063,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
-      epsilon, rope_theta, bf16_activations != 0, nullptr);
+      epsilon, rope_theta, bf16_activations != 0, nullptr, nullptr, 0u, rows);
   return launched("Q4H QKV rope cache batch");
 }
 
@@ -1052,8 +1088,39 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, 0u, 0u, query_heads, kv_heads,
       head_dim, rotary_dim, epsilon, rope_theta, bf16_activations != 0,
-      device_positions);
+      device_positions, nullptr, 0u, rows);
   return launched("deferred Q4H QKV rope cache batch");
+}
+
+extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_from_partials(
+    const float* partials, uint32_t partial_count, float* query,
+    uint32_t query_stride, float* key, float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, const uint32_t* device_positions,
+    uint32_t rows, uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, void* stream) {
+  if (!partials || !partial_count || partial_count > 16u || !query || !key ||
+      !value || !page_table || !page_tokens || !rows || !query_heads ||
+      !kv_heads || query_heads < kv_heads || query_heads % kv_heads ||
+      !head_dim || head_dim > 256u || head_dim % 2u ||
+      query_stride < head_dim || !rotary_dim || rotary_dim > head_dim ||
+      rotary_dim % 2u || !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
+      (!device_positions &&
+       (first_cache_position > 0xffffffffu - (rows - 1u) ||
+        first_rotary_position > 0xffffffffu - (rows - 1u))))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "invalid Q4H QKV rope cache batch from partials");
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
+      query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
+      full_attention_layer, page_tokens, first_cache_position,
+      first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
+      epsilon, rope_theta, bf16_activations != 0, device_positions, partials,
+      partial_count, rows);
+  return launched("Q4H QKV rope cache batch from partials");
 }
 
 extern "C" int32_t qllm_qkv_rope_batch(
@@ -1073,7 +1140,8 @@ extern "C" int32_t qllm_qkv_rope_batch(
                         as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
-      rotary_dim, epsilon, rope_theta, bf16_activations != 0, nullptr);
+      rotary_dim, epsilon, rope_theta, bf16_activations != 0, nullptr, nullptr,
+      0u, rows);
   return launched("QKV rope batch");
 }
 
@@ -1093,7 +1161,7 @@ extern "C" int32_t qllm_qkv_rope_batch_deferred(
                         as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, 0u, query_heads, kv_heads, head_dim, rotary_dim, epsilon,
-      rope_theta, bf16_activations != 0, device_positions);
+      rope_theta, bf16_activations != 0, device_positions, nullptr, 0u, rows);
   return launched("deferred QKV rope batch");
 }
 

@@ -1,5 +1,7 @@
 #include "artifact_provider.hpp"
 
+#include "dense_record.hpp"
+
 #include <algorithm>
 #include <bit>
 #include <cmath>
@@ -45,7 +47,8 @@ class TensorBinder final {
  public:
   explicit TensorBinder(er::IModelTensorStore& store) : store_(store) {}
 
-  er::Status bind(const er::BindingMap& bindings,
+  er::Status bind(
+      const std::map<std::string, std::string, std::less<>>& bindings,
                   std::vector<er::PreparedTensorBinding>& out, const char* what) {
     out.clear();
     out.reserve(bindings.size());
@@ -185,17 +188,15 @@ er::Status dense_geometry_from_artifact(const er::ModelDescriptor& model,
   }
 }
 
-CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
-    const std::filesystem::path& artifact_root,
+er::CreateExecutionProviderModuleResult make_mi355_dense_fp4_module(
+    std::shared_ptr<er::ModelArtifact> artifact,
     const ArtifactProviderOptions& options) {
   try {
-    auto artifact = std::make_shared<er::ModelArtifact>();
-    if (auto status = er::ModelArtifact::load(artifact_root, *artifact); !status.ok())
-      return {status, {}};
-    if (options.mtp_draft_depth)
-      if (auto status = artifact->configure_mtp_draft_depth(options.mtp_draft_depth);
-          !status.ok())
-        return {status, {}};
+    if (!artifact) return {invalid("artifact is absent"), {}};
+    if (options.routed_vram_policy != "fixed")
+      return {invalid("a dense resident provider has no routed VRAM policy but "
+                      "\"fixed\""),
+              {}};
     auto store = std::make_shared<er::MappedModelTensorStore>();
     if (auto status = er::MappedModelTensorStore::create(*artifact, *store);
         !status.ok())
@@ -211,8 +212,8 @@ CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
     }
 
     const er::ModelDescriptor& model = artifact->model();
-    auto definition = make_mi355_dense_fp4_provider();
-    if (auto status = er::provider_supports_model(model, definition.capabilities);
+    auto metadata = make_mi355_dense_fp4_provider();
+    if (auto status = er::provider_supports_model(model, metadata.capabilities);
         !status.ok())
       return {status, {}};
     DenseGeometry geometry;
@@ -220,55 +221,123 @@ CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
         !status.ok())
       return {status, {}};
 
-    ExecutionProviderModule module;
-    module.implementation = std::make_shared<Mi355DenseFp4Provider>(geometry);
-    TensorBinder binder(*store);
-    std::vector<er::PreparedTensorBinding> bound;
-    for (std::size_t index = 0; index < model.operation_program.size(); ++index) {
-      const auto& operation = model.operation_program[index];
-      if (operation.logical_operation != index)
-        return {invalid("compiled operation order or kernel binding is invalid"), {}};
-      if (auto status = binder.bind(operation.tensor_bindings, bound, "tensor");
-          !status.ok())
-        return {status, {}};
-      er::OperationPreparationContext context;
-      context.capability = operation.capability;
-      context.abi = operation.abi_version;
-      context.parameters = operation.parameters;
-      context.tensors = bound;
-      auto prepared = module.implementation->prepare(context);
-      if (!prepared.status.ok()) return {prepared.status, {}};
-      if (!prepared.operation)
-        return {invalid("callable provider returned no prepared operation"), {}};
-      module.operations.push_back(std::move(prepared.operation));
-    }
-    if (model.exact_decode_program) {
-      const auto& decode = *model.exact_decode_program;
-      if (auto status =
-              binder.bind(decode.tensor_bindings, bound, "exact decode tensor");
-          !status.ok())
-        return {status, {}};
-      er::ExactDecodePreparationContext context;
-      context.capability = decode.capability;
-      context.abi = decode.abi_version;
-      context.parameters = decode.parameters;
-      context.tensors = bound;
-      auto prepared = module.implementation->prepare_exact_decode(context);
-      if (!prepared.status.ok()) return {prepared.status, {}};
-      if (!prepared.operation)
-        return {invalid("callable provider returned no exact decode program"), {}};
-      module.exact_decode = std::move(prepared.operation);
-    }
-    definition.entry = module.implementation.get();
-    module.definition = std::move(definition);
-    module.service = module.implementation->service_contract();
-    module.artifact = std::move(artifact);
+    auto implementation = std::make_shared<Mi355DenseFp4Provider>(geometry);
+    er::ExecutionProviderModule module;
+    module.definition = {metadata.name, metadata.priority,
+                         std::move(metadata.capabilities), implementation};
     module.tensor_store = std::move(store);
+    module.service = implementation->service_contract();
+    const bool mtp = model.exact_decode_program.has_value();
+    module.service.mtp_resource_available = mtp;
+    module.service.mtp_runtime_ready = mtp;
+    module.service.mtp_enabled = mtp;
+    module.service.vram_cache_bytes = options.vram_cache_bytes;
+    module.service.routed_vram_policy = options.routed_vram_policy;
+    module.telemetry = [implementation] { return implementation->telemetry(); };
+    // nothing to fit after the tensors are bound: weights and workspaces are
+    // resident, KV pages are allocated on demand
+    module.finalize_service =
+        [](er::ExecutionProviderModule::ServiceContract&) {
+          return er::Status::success();
+        };
     return {er::Status::success(), std::move(module)};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal,
              std::string("dense FP4 provider creation failed: ") + error.what()},
             {}};
+  }
+}
+
+er::CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
+    const std::filesystem::path& artifact_root, std::uint32_t max_context,
+    std::uint32_t capacity, std::uint64_t /*ram_cache_bytes*/,
+    std::uint64_t vram_cache_bytes, std::uint64_t kv_cache_bytes,
+    std::uint32_t kv_page_tokens, std::string_view kv_cache_dtype,
+    std::string_view /*placement_profile*/, std::string_view routed_vram_policy,
+    bool /*profile_gpu_phases*/, bool /*discover_active_expert_devices*/,
+    std::vector<int> /*active_expert_devices*/,
+    std::uint64_t /*active_expert_device_cache_bytes*/,
+    std::uint64_t /*active_expert_host_cache_bytes*/,
+    std::uint32_t mtp_draft_depth) {
+  try {
+    // the launch contract of dense_fp4_provider.cpp:2330-2336; one request at
+    // a time owns the KV cache here
+    if (!capacity || !max_context || !kv_cache_bytes || !kv_page_tokens)
+      return {invalid("invalid dense FP4 provider launch contract"), {}};
+    if (capacity != 1U)
+      return {invalid("this provider serves one request at a time (capacity 1)"),
+              {}};
+    auto artifact = std::make_shared<er::ModelArtifact>();
+    if (auto status = er::ModelArtifact::load(artifact_root, *artifact); !status.ok())
+      return {status, {}};
+    if (mtp_draft_depth != 0U)
+      if (auto status = artifact->configure_mtp_draft_depth(mtp_draft_depth);
+          !status.ok())
+        return {status, {}};
+    ArtifactProviderOptions options;
+    options.max_context = max_context;
+    options.kv_page_tokens = kv_page_tokens;
+    options.kv_cache_dtype = std::string(kv_cache_dtype);
+    options.vram_cache_bytes = vram_cache_bytes ? vram_cache_bytes : 1U;
+    options.routed_vram_policy = std::string(routed_vram_policy);
+    return make_mi355_dense_fp4_module(std::move(artifact), options);
+  } catch (const std::exception& error) {
+    return {{er::ErrorCode::internal, error.what()}, {}};
+  }
+}
+
+er::Status prepare_program(const er::ModelDescriptor& model,
+                           const er::ExecutionProviderModule& module,
+                           PreparedProgram& prepared) {
+  try {
+    if (!module.definition.implementation || !module.tensor_store)
+      return invalid("provider module is incomplete");
+    er::ExecutionProviderRegistry registry;
+    if (auto status = registry.add(module.definition); !status.ok()) return status;
+    auto bound = registry.bind(model, er::ExecutionProviderBindingMode::executable);
+    if (!bound.status.ok()) return bound.status;
+    prepared = PreparedProgram{};
+    prepared.bound = std::move(bound.provider);
+    const auto& program = prepared.bound.program;
+    auto& provider = *module.definition.implementation;
+    if (program.operations.size() != model.operation_program.size())
+      return invalid("compiled operation order or kernel binding is invalid");
+    TensorBinder binder(*module.tensor_store);
+    std::vector<er::PreparedTensorBinding> tensors;
+    for (std::size_t index = 0; index < model.operation_program.size(); ++index) {
+      const auto& operation = model.operation_program[index];
+      const auto& compiled = program.operations[index];
+      if (compiled.logical_operation != index ||
+          compiled.kernel_binding >= program.kernels.size())
+        return invalid("compiled operation order or kernel binding is invalid");
+      if (auto status = binder.bind(operation.tensor_bindings, tensors, "tensor");
+          !status.ok())
+        return status;
+      auto result = provider.prepare({model, operation, compiled, tensors});
+      if (!result.status.ok()) return result.status;
+      if (!result.operation)
+        return invalid("callable provider returned no prepared operation");
+      prepared.operations.push_back(std::move(result.operation));
+    }
+    if (model.exact_decode_program) {
+      if (!program.exact_decode)
+        return invalid("exact decode program was not compiled");
+      const auto& decode = *model.exact_decode_program;
+      if (auto status =
+              binder.bind(decode.tensor_bindings, tensors, "exact decode tensor");
+          !status.ok())
+        return status;
+      auto result = provider.prepare_exact_decode(
+          {model, decode, *program.exact_decode, tensors});
+      if (!result.status.ok()) return result.status;
+      if (!result.operation)
+        return invalid("callable provider returned no exact decode program");
+      prepared.exact_decode = std::move(result.operation);
+    }
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal,
+            std::string("program preparation failed: ") + error.what()};
   }
 }
 

@@ -80,7 +80,7 @@ er::ExactDecodeExecutionHandle completed_exact(
         shared->reset();
         return value;
       },
-      []() {});
+      [shared]() { shared->reset(); });
 }
 
 const er::ImmutableModelTensor& tensor_for(
@@ -108,15 +108,40 @@ const er::ImmutableModelTensor& tensor_for_either(
   throw std::runtime_error("tensor role is not bound: " + std::string(role));
 }
 
-class PreparedMarker final : public er::IPreparedOperation {
- public:
-  explicit PreparedMarker(std::string capability)
-      : capability_(std::move(capability)) {}
-  const std::string& capability() const noexcept { return capability_; }
+// Value ABIs between operations as the artifact declares them
+// (dense_fp4_provider.cpp:59-74).  The hidden-state ABI string names F32 rows
+// in device memory; the memory domain says whose device.
+constexpr std::string_view kHiddenAbi = "batch.hidden.f32.cuda.v1";
+constexpr std::string_view kTokenAbi = "batch.token-id.u32.host.v1";
+constexpr std::string_view kPositionAbi = "batch.position.u32.host.v1";
+constexpr std::string_view kDeviceDomain = "hip.device";
 
- private:
-  std::string capability_;
-};
+// :550-564
+std::span<const std::uint32_t> host_u32_batch(const er::ExecutionValue& value,
+                                              std::string_view abi,
+                                              std::string_view description) {
+  if (!value.valid() || value.abi != abi || value.memory_domain != "host" ||
+      value.bytes % sizeof(std::uint32_t) != 0U ||
+      value.bytes / sizeof(std::uint32_t) > 1024U ||
+      reinterpret_cast<std::uintptr_t>(value.data) % alignof(std::uint32_t) != 0U)
+    throw std::runtime_error(std::string(description) + " ABI mismatch");
+  return {reinterpret_cast<const std::uint32_t*>(value.data),
+          static_cast<std::size_t>(value.bytes / sizeof(std::uint32_t))};
+}
+
+// :5605-5620
+er::OperationExecutionHandle completed_operation(
+    er::OperationExecutionResult result) {
+  auto shared = std::make_shared<std::optional<er::OperationExecutionResult>>(
+      std::move(result));
+  return er::OperationExecutionHandle::from_callbacks(
+      [shared]() {
+        auto value = std::move(*shared);
+        shared->reset();
+        return value;
+      },
+      [shared]() { shared->reset(); });
+}
 
 er::Status validate_parameters(
     const std::map<std::string, std::uint64_t, std::less<>>& parameters) {
@@ -134,7 +159,19 @@ er::Status validate_parameters(
 
 }  // namespace
 
-struct Mi355DenseFp4Provider::PreparedOp {};
+// What prepare() leaves behind for execute() (PreparedOperation,
+// dense_fp4_provider.cpp:2273-2291): which block this is, where its inputs sit
+// in an invocation and which output ports, with which ABI, it must fill.
+struct Mi355DenseFp4Provider::PreparedOperation final : er::IPreparedOperation {
+  enum class Kind { embedding, attention, ffn, head, exact_decode };
+  Kind kind{};
+  std::string capability;
+  std::uint32_t abi_version{};
+  std::uint32_t logical_operation{};
+  std::uint32_t layer{};   // attention / ffn: index among the blocks of its kind
+  std::map<std::string, std::size_t, std::less<>> input_indices;
+  std::vector<std::pair<std::string, std::string>> outputs;
+};
 
 er::WorkerProviderDefinition make_mi355_dense_fp4_provider() {
   const auto validator = [](const er::ModelDescriptor& model) {
@@ -145,12 +182,12 @@ er::WorkerProviderDefinition make_mi355_dense_fp4_provider() {
   // compiler/expert_pack/adapters.py:1682-1697) plus the block-16 variants.
   return {"mi355-dense-fp4",
           200U,
-          {{"embedding.lookup.fp4-block32.v1", 1U, 2U, validator},
+          {{"embedding.lookup.fp4-block32.v1", 1U, 1U, validator},
            {"dense.activation-input.bfloat16.v1", 1U, 1U, validator},
-           {"block.full-attention.output-gated.v1", 1U, 2U, validator},
+           {"block.full-attention.output-gated.v1", 1U, 1U, validator},
            {"block.full-attention.standard-gqa.v1", 1U, 1U, validator},
-           {"ffn.swiglu.dense.fp4-block32.v1", 1U, 2U, validator},
-           {"head.rmsnorm.token-select.fp4-block32.v1", 1U, 2U, validator},
+           {"ffn.swiglu.dense.fp4-block32.v1", 1U, 1U, validator},
+           {"head.rmsnorm.token-select.fp4-block32.v1", 1U, 1U, validator},
            {"decode.mtp.dense-full-attention.fp4-block32.exact.v2", 2U, 2U,
             validator},
            {"embedding.lookup.fp4-f16-block16.v1", 1U, 1U, validator},
@@ -194,6 +231,7 @@ Mi355DenseFp4Provider::Mi355DenseFp4Provider(const DenseGeometry& geometry)
   hipStream_t stream{};
   hip_check(hipStreamCreate(&stream), "create provider stream");
   stream_ = stream;
+  device_lifetime_ = std::make_shared<std::uint8_t>(std::uint8_t{0});
   layers_.resize(g_.layers);
   accepted_depth_calls_.assign(g_.draft_depth + 1U, 0U);
   max_rows_ = g_.draft_depth + 1U;
@@ -286,6 +324,14 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   if (projection_splits_ > 1U)
     projection_partials_ = static_cast<float*>(
         device_alloc(projection_splits_ * rows * g_.hidden * 4U));
+
+  if (const char* text = std::getenv("QLLM_PROVIDER_QKV_SPLITS"))
+    qkv_splits_ =
+        static_cast<std::uint32_t>(std::clamp(std::atoi(text), 0, 16));
+  if (g_.kv_encoding != KvEncoding::q4_f16_per_head) qkv_splits_ = 0U;
+  if (qkv_splits_ > 1U)
+    qkv_partials_ = static_cast<float*>(device_alloc(
+        qkv_splits_ * rows * (query_width + 2U * kv_width) * 4U));
 
   // Context splits: kv_heads * splits workgroups fill the 256 CUs; the
   // attention kernels deal the context's tiles evenly over them themselves
@@ -535,9 +581,25 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
     const er::OperationPreparationContext& context) {
   try {
     std::lock_guard lock(mutex_);
-    auto status = validate_parameters(context.parameters);
+    auto status = validate_parameters(context.operation.parameters);
     if (!status.ok()) return {status, {}};
-    const std::string& capability = context.capability;
+    const std::string& capability = context.operation.capability;
+    auto prepared = std::make_shared<PreparedOperation>();
+    prepared->capability = capability;
+    prepared->abi_version = context.operation.abi_version;
+    prepared->logical_operation = context.compiled.logical_operation;
+    // ports: inputs arrive in the compiled order, outputs leave with the ABI
+    // the artifact declares for the port (:2912-2923)
+    for (std::size_t index = 0; index < context.compiled.input_values.size();
+         ++index)
+      prepared->input_indices.emplace(context.compiled.input_values[index].port,
+                                      index);
+    for (const auto& binding : context.compiled.output_values) {
+      const auto output = context.operation.output_bindings.find(binding.port);
+      if (output == context.operation.output_bindings.end())
+        throw std::runtime_error("compiled output port is absent");
+      prepared->outputs.emplace_back(binding.port, output->second.abi);
+    }
     const auto query_rows =
         g_.query_heads * g_.head_dim * (g_.output_gated ? 2U : 1U);
     const auto require_shape = [](const DeviceFp4Matrix& matrix,
@@ -551,6 +613,7 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
           tensor_for_either(context.tensors, "weight", "token_embedding"), false);
       require_shape(embedding_, g_.vocabulary, g_.hidden, "token_embedding");
       embedding_ready_ = true;
+      prepared->kind = PreparedOperation::Kind::embedding;
     } else if (capability.starts_with("block.full-attention.")) {
       const bool gated = capability.find("output-gated") != std::string::npos;
       if (gated != g_.output_gated)
@@ -583,6 +646,8 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
         layer.key_norm =
             upload_f32(tensor_for(context.tensors, "key_norm"), g_.head_dim);
       }
+      prepared->kind = PreparedOperation::Kind::attention;
+      prepared->layer = attention_ops_;
       ++attention_ops_;
     } else if (capability.starts_with("ffn.swiglu.dense.")) {
       if (ffn_ops_ >= g_.layers)
@@ -600,6 +665,8 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
       require_shape(layer.gate, g_.intermediate, g_.hidden, "gate_projection");
       require_shape(layer.up, g_.intermediate, g_.hidden, "up_projection");
       require_shape(layer.down, g_.hidden, g_.intermediate, "down_projection");
+      prepared->kind = PreparedOperation::Kind::ffn;
+      prepared->layer = ffn_ops_;
       ++ffn_ops_;
     } else if (capability.starts_with("head.rmsnorm.token-select.")) {
       final_norm_ = upload_f32(
@@ -608,13 +675,13 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare(
           tensor_for_either(context.tensors, "weight", "output_head"), true);
       require_shape(head_, g_.vocabulary, g_.hidden, "output_head");
       head_ready_ = true;
+      prepared->kind = PreparedOperation::Kind::head;
     } else {
       return {{er::ErrorCode::invalid_argument,
                "capability is not provided: " + capability},
               {}};
     }
-    return {er::Status::success(),
-            std::make_shared<PreparedMarker>(capability)};
+    return {er::Status::success(), std::move(prepared)};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
   }
@@ -624,13 +691,17 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare_exact_decode(
     const er::ExactDecodePreparationContext& context) {
   try {
     std::lock_guard lock(mutex_);
-    if (!context.capability.starts_with("decode.mtp.dense-full-attention.") ||
-        context.abi != 2U)
+    if (!context.program.capability.starts_with(
+            "decode.mtp.dense-full-attention.") ||
+        context.program.abi_version != 2U)
       return {{er::ErrorCode::invalid_argument,
                "exact decode capability or ABI is not provided"},
               {}};
-    const auto depth = context.parameters.find("draft_depth");
-    if (depth == context.parameters.end() || depth->second != g_.draft_depth)
+    // the artifact contract of the exact-decode program (:2934-2966)
+    const auto& parameters = context.program.parameters;
+    const auto depth = parameters.find("draft_depth");
+    if (depth == parameters.end() || depth->second != g_.draft_depth ||
+        context.program.maximum_emitted_tokens != g_.draft_depth + 1U)
       return {{er::ErrorCode::invalid_argument,
                "exact decode draft depth does not match the provider"},
               {}};
@@ -644,7 +715,11 @@ er::PrepareOperationResult Mi355DenseFp4Provider::prepare_exact_decode(
       return {{er::ErrorCode::invalid_argument,
                "exact decode with an MTP layer needs the proposer's tensors"},
               {}};
-    exact_ = std::make_shared<PreparedMarker>(context.capability);
+    auto prepared = std::make_shared<PreparedOperation>();
+    prepared->kind = PreparedOperation::Kind::exact_decode;
+    prepared->capability = context.program.capability;
+    prepared->abi_version = context.program.abi_version;
+    exact_ = prepared;
     return {er::Status::success(), exact_};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
@@ -750,6 +825,270 @@ void Mi355DenseFp4Provider::mark_presence(
                                   g_.vocabulary, stream_));
 }
 
+er::Status Mi355DenseFp4Provider::rebind_request_state(
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    const er::ProgramRequestContext& request) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto state =
+        std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+    const auto first = request.parameters.find("sampling_first_output_position");
+    const auto presence =
+        request.parameters.find("sampling_presence_penalty_biased_ppm");
+    if (!state || first == request.parameters.end() ||
+        first->second >= g_.max_context ||
+        presence == request.parameters.end() || presence->second > 4'000'000U)
+      throw std::runtime_error("sampling request rebind is invalid");
+    hip_check(hipMemsetAsync(presence_, 0, g_.vocabulary,
+                             static_cast<hipStream_t>(stream_)),
+              "reset request sampling presence");
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
+// :5579-5586
+er::ExecutionValue Mi355DenseFp4Provider::device_hidden_value(
+    std::uint32_t rows) const {
+  if (!rows || rows > max_rows_)
+    throw std::runtime_error("invalid FP4 hidden batch size");
+  return {std::string(kHiddenAbi), std::string(kDeviceDomain), device_lifetime_,
+          reinterpret_cast<const std::byte*>(hidden_),
+          std::uint64_t{rows} * g_.hidden * sizeof(float)};
+}
+
+// :5649-5660
+std::uint32_t Mi355DenseFp4Provider::require_hidden_value(
+    const er::ExecutionValue& value) const {
+  const auto row_bytes = std::uint64_t{g_.hidden} * sizeof(float);
+  if (value.abi != kHiddenAbi || value.memory_domain != kDeviceDomain ||
+      value.data != reinterpret_cast<const std::byte*>(hidden_) ||
+      value.bytes % row_bytes != 0U || value.bytes / row_bytes == 0U ||
+      value.bytes / row_bytes > max_rows_)
+    throw std::runtime_error("hidden-state execution ABI mismatch");
+  return static_cast<std::uint32_t>(value.bytes / row_bytes);
+}
+
+// The head's token for a request (run_head with a request, :8433-8517): the
+// presence penalty from the first output position on, arg-max at temperature
+// zero, otherwise top-k or whole-row candidates ordered on the host and one
+// draw from stream 0; an output token is marked as emitted.  logits_ row 0.
+std::uint32_t Mi355DenseFp4Provider::select_head_token(
+    const er::ProgramRequestContext& request, std::uint32_t sample_position) {
+  const auto stream = static_cast<hipStream_t>(stream_);
+  const auto first_output =
+      request_parameter(request, "sampling_first_output_position");
+  const bool output_sampling = sample_position >= first_output;
+  const auto penalty = presence_penalty_of(request);
+  if (output_sampling && penalty != 0.0) {
+    status_check(qllm_apply_presence_penalty(logits_, presence_, g_.vocabulary,
+                                             static_cast<float>(penalty),
+                                             stream_));
+    status_check(qllm_argmax_batch(logits_, g_.vocabulary, 1U, argmax_tokens_,
+                                   select_workspace_, select_workspace_bytes_,
+                                   stream_));
+  }
+  const auto temperature = request_parameter(request, "sampling_temperature_ppm");
+  std::uint32_t selected{};
+  if (temperature == 0U) {
+    hip_check(hipMemcpyAsync(&selected, argmax_tokens_, sizeof(selected),
+                             hipMemcpyDeviceToHost, stream),
+              "copy dense FP4 greedy token");
+    hip_check(hipStreamSynchronize(stream), "copy dense FP4 greedy token");
+  } else {
+    // the penalty, if any, has been applied: the distribution is taken from
+    // the row as it stands
+    er::ProgramRequestContext unpenalised = request;
+    unpenalised.parameters["sampling_presence_penalty_biased_ppm"] = 2'000'000U;
+    const auto top_k = request_parameter(request, "sampling_top_k");
+    if (top_k > kMaximumGpuSamplingTopK) {
+      // the scalar sampler orders that many candidates on the host
+      // (sample_token, :773-799)
+      std::vector<float> row(g_.vocabulary);
+      hip_check(hipMemcpyAsync(row.data(), logits_, row.size() * 4U,
+                               hipMemcpyDeviceToHost, stream),
+                "copy dense FP4 sampling logits");
+      hip_check(hipStreamSynchronize(stream), "copy dense FP4 sampling logits");
+      if (top_k > row.size())
+        throw std::runtime_error("invalid token sampling contract");
+      std::vector<std::uint32_t> candidates(row.size());
+      std::iota(candidates.begin(), candidates.end(), 0U);
+      const auto before = [&](std::uint32_t left, std::uint32_t right) {
+        const float a = row[left];
+        const float b = row[right];
+        if (std::isnan(a)) return false;
+        if (std::isnan(b)) return true;
+        return a == b ? left < right : a > b;
+      };
+      std::partial_sort(candidates.begin(), candidates.begin() + top_k,
+                        candidates.end(), before);
+      candidates.resize(top_k);
+      std::vector<float> ordered;
+      for (const auto candidate : candidates) ordered.push_back(row[candidate]);
+      sampling_logit_transfer_bytes_ += row.size() * 4U;
+      const auto distribution = er::make_sampling_distribution(
+          ordered, candidates, static_cast<std::uint32_t>(temperature),
+          static_cast<std::uint32_t>(
+              request_parameter(request, "sampling_top_p_ppm")),
+          static_cast<std::uint32_t>(
+              request_parameter(request, "sampling_min_p_ppm")));
+      selected = er::sample_distribution(
+          distribution,
+          er::counter_uniform(request_parameter(request, "sampling_seed"),
+                              sample_position, 0U));
+    } else {
+      const auto distribution = distribution_from_logits(
+          logits_, g_.vocabulary, argmax_tokens_, unpenalised, nullptr);
+      selected = er::sample_distribution(
+          distribution,
+          er::counter_uniform(request_parameter(request, "sampling_seed"),
+                              sample_position, 0U));
+    }
+  }
+  if (output_sampling) {
+    const std::uint32_t token[1] = {selected};
+    mark_presence(presence_, token);
+  }
+  return selected;
+}
+
+// One operation of the artifact's program (execute, :10680-10992).
+er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
+    const er::IPreparedOperation& opaque_operation,
+    const std::shared_ptr<er::IOperationProviderRequestState>& opaque_state,
+    const er::OperationInvocation& invocation) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto* operation =
+        dynamic_cast<const PreparedOperation*>(&opaque_operation);
+    const auto state =
+        std::dynamic_pointer_cast<DenseFp4RequestState>(opaque_state);
+    if (!operation || !state ||
+        operation->kind == PreparedOperation::Kind::exact_decode)
+      throw std::runtime_error("dense FP4 invocation state is invalid");
+    const auto input = [&](std::string_view port) -> const er::ExecutionValue& {
+      const auto found = operation->input_indices.find(port);
+      if (found == operation->input_indices.end() ||
+          found->second >= invocation.inputs.size())
+        throw std::runtime_error("operation input port is absent");
+      return invocation.inputs[found->second];
+    };
+    const auto stream = static_cast<hipStream_t>(stream_);
+    std::map<std::string, er::ExecutionValue, std::less<>> outputs;
+    switch (operation->kind) {
+      case PreparedOperation::Kind::embedding: {
+        state->exact_decode_enabled =
+            exact_ &&
+            request_parameter(invocation.request, "exact_decode_enabled") != 0U;
+        if (state->synchronization_rows != 0U)
+          throw std::runtime_error("previous target batch was not synchronized");
+        const auto tokens =
+            host_u32_batch(input("token_ids"), kTokenAbi, "embedding token batch");
+        if (tokens.empty() || tokens.size() > max_rows_)
+          throw std::runtime_error("invalid FP4 hidden batch size");
+        for (const auto token : tokens)
+          if (token >= g_.vocabulary)
+            throw std::runtime_error("embedding token exceeds vocabulary");
+        const auto rows = static_cast<std::uint32_t>(tokens.size());
+        // a pageable source: the copy has read it when the call returns
+        hip_check(hipMemcpyAsync(tokens_, tokens.data(), rows * 4U,
+                                 hipMemcpyHostToDevice, stream),
+                  "upload target tokens");
+        status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, tokens_,
+                                              hidden_, rows, stream_));
+        pending_partials_ = 0U;
+        state->current_batch_rows = rows;
+        outputs.emplace("hidden", device_hidden_value(rows));
+        break;
+      }
+      case PreparedOperation::Kind::attention: {
+        const auto rows = require_hidden_value(input("hidden"));
+        const auto positions = host_u32_batch(input("positions"), kPositionAbi,
+                                              "attention position batch");
+        if (positions.size() != rows || rows != state->current_batch_rows)
+          throw std::runtime_error("attention batch width changed in program");
+        for (std::uint32_t row = 0; row < rows; ++row)
+          if (positions[row] >= g_.max_context ||
+              (row != 0U && positions[row] != positions[0] + row))
+            throw std::runtime_error("attention position batch is not contiguous");
+        state->current_batch_first = positions.front();
+        state->current_position = positions.back();
+        ensure_pages(positions.back());
+        enqueue_attention_block(operation->layer, rows, positions.front(), false,
+                                false);
+        outputs.emplace("hidden", device_hidden_value(rows));
+        break;
+      }
+      case PreparedOperation::Kind::ffn: {
+        const auto rows = require_hidden_value(input("hidden"));
+        if (rows != state->current_batch_rows)
+          throw std::runtime_error("FFN batch width changed in program");
+        enqueue_ffn_block(operation->layer, rows, false);
+        outputs.emplace("hidden", device_hidden_value(rows));
+        break;
+      }
+      case PreparedOperation::Kind::head: {
+        const auto rows = require_hidden_value(input("hidden"));
+        if (rows != state->current_batch_rows)
+          throw std::runtime_error("head batch width changed in program");
+        // hidden_ keeps the batch: the proposer is synchronised from it
+        if (state->exact_decode_enabled) {
+          state->synchronization_first = state->current_batch_first;
+          state->synchronization_rows = rows;
+          state->synchronization_consumed = 0U;
+        } else {
+          state->synchronization_first = 0U;
+          state->synchronization_rows = 0U;
+          state->synchronization_consumed = 0U;
+          state->mtp_length = state->current_position + 1U;
+          state->draft_valid = false;
+          state->draft_predictions.clear();
+        }
+        // a batch selects for its last row only (terminal_only, :8397-8402)
+        enqueue_head(rows - 1U, 1U);
+        auto owner = std::make_shared<std::vector<std::uint32_t>>(
+            1U, select_head_token(invocation.request, state->current_position));
+        outputs.emplace(
+            "token_ids",
+            er::ExecutionValue{std::string(kTokenAbi), "host", owner,
+                               reinterpret_cast<const std::byte*>(owner->data()),
+                               owner->size() * sizeof(std::uint32_t)});
+        program_steps_ += rows;
+        if (rows > 1U) prefill_tokens_total_ += rows;
+        break;
+      }
+      case PreparedOperation::Kind::exact_decode:
+        throw std::runtime_error("exact decode entered scalar execution");
+    }
+    er::OperationExecutionResult result;
+    result.status = er::Status::success();
+    result.outputs.reserve(operation->outputs.size());
+    for (const auto& [port, abi] : operation->outputs) {
+      const auto found = outputs.find(port);
+      if (found == outputs.end() || found->second.abi != abi)
+        throw std::runtime_error("dense FP4 output ABI mismatch");
+      result.outputs.push_back(std::move(found->second));
+    }
+    return completed_operation(std::move(result));
+  } catch (const std::exception& error) {
+    return completed_operation({{er::ErrorCode::internal, error.what()}, {}});
+  }
+}
+
+// :10994-11009
+er::Status Mi355DenseFp4Provider::synchronize_exact_decode(
+    const er::IPreparedOperation& operation,
+    const std::shared_ptr<er::IOperationProviderRequestState>& state,
+    const er::ExactDecodeSynchronization& synchronization) {
+  const std::uint32_t tokens[1] = {synchronization.next_token};
+  return synchronize_exact_decode_batch(
+      operation, state,
+      er::ExactDecodeSynchronizationBatch{synchronization.request, tokens,
+                                          synchronization.target_position,
+                                          synchronization.produce_draft});
+}
+
 // Records where the verified stream stands after prefill / a previous step
 // (dense_fp4_provider.cpp:11011-11130).  Producing the drafts themselves is
 // the proposer's job; they arrive through set_draft_predictions().
@@ -775,6 +1114,23 @@ er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
         synchronization.first_target_position > g_.max_context - rows)
       return {er::ErrorCode::invalid_argument,
               "exact decode synchronization is invalid"};
+    // Rows of the last head execute() ran are consumed in order (:11020-11036);
+    // a host that runs the target through run_target() has no such window and
+    // synchronises from row 0 of that pass.
+    const float* previous_hidden = hidden_;
+    if (state->synchronization_rows != 0U) {
+      if (state->synchronization_consumed >= state->synchronization_rows ||
+          rows > state->synchronization_rows - state->synchronization_consumed ||
+          state->mtp_length != synchronization.first_target_position ||
+          synchronization.first_target_position !=
+              state->synchronization_first + state->synchronization_consumed)
+        throw std::runtime_error("MTP synchronization stream is invalid");
+      previous_hidden =
+          hidden_ + std::size_t{state->synchronization_consumed} * g_.hidden;
+      state->synchronization_consumed += rows;
+      if (state->synchronization_consumed == state->synchronization_rows)
+        state->synchronization_rows = state->synchronization_consumed = 0U;
+    }
     state->synchronized_token = synchronization.next_tokens.back();
     state->draft_valid = false;
     state->draft_predictions.clear();
@@ -790,7 +1146,7 @@ er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
                                  hipMemcpyDeviceToDevice,
                                  static_cast<hipStream_t>(stream_)),
                   "initialize speculative proposal presence");
-      auto draft = run_mtp(*state, synchronization.next_tokens, hidden_,
+      auto draft = run_mtp(*state, synchronization.next_tokens, previous_hidden,
                            synchronization.produce_final_draft,
                            synchronization.produce_final_draft
                                ? &synchronization.request
@@ -860,13 +1216,23 @@ er::Status Mi355DenseFp4Provider::set_draft_predictions(
 // starting at `first_position`; the result goes to `attention_out` in bf16.
 void Mi355DenseFp4Provider::enqueue_attention(
     std::uint32_t index, std::uint32_t rows, std::uint32_t first_position,
-    bool deferred_positions, float* query, float* key, const float* value,
-    std::uint16_t* attention_out) {
+    bool deferred_positions, float* query, float* key, float* value,
+    std::uint16_t* attention_out, const float* qkv_partials,
+    std::uint32_t qkv_partial_count) {
   void* const stream = stream_;
   const auto& layer = layers_[index];
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-    if (deferred_positions)
+    if (qkv_partials)
+      status_check(qllm_qkv_rope_cache_paged_q4h_from_partials(
+          qkv_partials, qkv_partial_count, query, query_stride, key, value,
+          layer.query_norm, layer.key_norm,
+          const_cast<const void* const*>(device_page_table_), index,
+          g_.kv_page_tokens, first_position, first_position,
+          deferred_positions ? positions_ : nullptr, rows, g_.query_heads,
+          g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
+          g_.rope_theta, 0, stream));
+    else if (deferred_positions)
       status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
           query, query_stride, key, value, layer.query_norm,
           layer.key_norm, const_cast<const void* const*>(device_page_table_),
@@ -935,80 +1301,128 @@ void Mi355DenseFp4Provider::enqueue_attention(
   }
 }
 
-void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
-                                           std::uint32_t rows,
-                                           std::uint32_t first_position,
-                                           bool deferred_positions) {
-  void* const stream = stream_;
-  const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
+// RMSNorm of hidden_ into normalized_ (bf16), first adding the partials a
+// K-split residual projection left behind.
+void Mi355DenseFp4Provider::enqueue_normalise(const float* weight,
+                                              std::uint32_t rows) {
+  if (pending_partials_)
+    status_check(qllm_rms_norm_residual_batch(
+        hidden_, projection_partials_, pending_partials_, weight, normalized_,
+        rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm, stream_));
+  else
+    status_check(qllm_rms_norm_batch(hidden_, weight, nullptr, normalized_,
+                                     g_.hidden, rows, g_.hidden, g_.norm_epsilon,
+                                     g_.zero_centered_norm, stream_));
+  pending_partials_ = 0U;
+}
+
+// hidden_ += matrix * input, in the projection's epilogue or - when the
+// caller lets the next norm finish the sum - as K-split partials.
+void Mi355DenseFp4Provider::enqueue_residual_projection(
+    const qllm_fp4_matrix& matrix, const std::uint16_t* input,
+    std::size_t input_bytes, std::uint32_t rows, bool leave_partials) {
+  if (leave_partials && projection_splits_ > 1U &&
+      matrix.layout == QLLM_LAYOUT_TILED &&
+      matrix.padded_columns / 64U >= projection_splits_) {
+    status_check(qllm_fp4_gemm_bf16_partial(&matrix, input, input_bytes,
+                                            projection_partials_,
+                                            projection_splits_, rows, stream_));
+    pending_partials_ = projection_splits_;
+  } else {
+    status_check(qllm_fp4_gemm_bf16(&matrix, input, input_bytes, hidden_,
+                                    QLLM_OUT_F32, hidden_, rows, stream_));
+  }
+}
+
+// full attention block (run_full_attention, :6892)
+void Mi355DenseFp4Provider::enqueue_attention_block(std::uint32_t index,
+                                                    std::uint32_t rows,
+                                                    std::uint32_t first_position,
+                                                    bool deferred_positions,
+                                                    bool leave_partials) {
+  const auto& layer = layers_[index];
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
   const std::size_t attention_bytes =
       std::size_t{rows} * g_.query_heads * g_.head_dim * 2U;
-  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
-                                        hidden_, rows, stream));
-  // Partials of the last residual projection that hidden_ does not hold yet;
-  // the next norm adds them.
-  std::uint32_t pending_partials = 0U;
-  const auto normalise = [&](const float* weight) {
-    if (pending_partials)
-      status_check(qllm_rms_norm_residual_batch(
-          hidden_, projection_partials_, pending_partials, weight, normalized_,
-          rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm, stream));
-    else
-      status_check(qllm_rms_norm_batch(hidden_, weight, nullptr, normalized_,
-                                       g_.hidden, rows, g_.hidden,
-                                       g_.norm_epsilon, g_.zero_centered_norm,
-                                       stream));
-    pending_partials = 0U;
-  };
-  // hidden_ += matrix * input, either in the projection's epilogue or as
-  // partials left for the next norm
-  const auto project_residual = [&](const qllm_fp4_matrix& matrix,
-                                    const std::uint16_t* input,
-                                    std::size_t input_bytes) {
-    if (projection_splits_ > 1U && matrix.layout == QLLM_LAYOUT_TILED &&
-        matrix.padded_columns / 64U >= projection_splits_) {
-      status_check(qllm_fp4_gemm_bf16_partial(&matrix, input, input_bytes,
-                                              projection_partials_,
-                                              projection_splits_, rows, stream));
-      pending_partials = projection_splits_;
-    } else {
-      status_check(qllm_fp4_gemm_bf16(&matrix, input, input_bytes, hidden_,
-                                      QLLM_OUT_F32, hidden_, rows, stream));
-    }
-  };
-  for (std::uint32_t index = 0; index < g_.layers; ++index) {
-    const auto& layer = layers_[index];
-    // full attention block (run_full_attention, :6892)
-    normalise(layer.input_norm);
-    // query, key and value projections (:7004-7011) in one launch
-    const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+  enqueue_normalise(layer.input_norm, rows);
+  // query, key and value projections (:7004-7011) in one launch
+  const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+  const bool cut_qkv = qkv_splits_ > 1U &&
+                       layer.qkv.descriptor.layout == QLLM_LAYOUT_TILED &&
+                       layer.qkv.descriptor.padded_columns / 64U >= qkv_splits_;
+  if (cut_qkv) {
+    status_check(qllm_fp4_gemm_bf16_partial(&layer.qkv.descriptor, normalized_,
+                                            hidden_bytes, qkv_partials_,
+                                            qkv_splits_, rows, stream_));
+    enqueue_attention(index, rows, first_position, deferred_positions, query_,
+                      key_, value_, attention_, qkv_partials_, qkv_splits_);
+  } else {
     const qllm_gemm_segment projections[3] = {
         {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
         {key_, kv_rows, QLLM_OUT_F32},
         {value_, kv_rows, QLLM_OUT_F32}};
     status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
                                           hidden_bytes, projections, 3U, rows,
-                                          stream));
+                                          stream_));
     enqueue_attention(index, rows, first_position, deferred_positions, query_,
                       key_, value_, attention_);
-    project_residual(layer.output.descriptor, attention_, attention_bytes);
-    // dense SwiGLU block (run_ffn, :8250-8293)
-    normalise(layer.post_attention_norm);
-    status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
-                                      &layer.up.descriptor, normalized_,
-                                      hidden_bytes, activation_, rows, stream));
-    project_residual(layer.down.descriptor, activation_,
-                     std::size_t{rows} * g_.intermediate * 2U);
   }
-  // head (run_head, :8393-8527); the norm also completes hidden_, which the
-  // proposer reads
-  normalise(final_norm_);
-  status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_, hidden_bytes,
-                                  logits_, QLLM_OUT_F32, nullptr, rows, stream));
+  enqueue_residual_projection(layer.output.descriptor, attention_,
+                              attention_bytes, rows, leave_partials);
+}
+
+// dense SwiGLU block (run_ffn, :8250-8293)
+void Mi355DenseFp4Provider::enqueue_ffn_block(std::uint32_t index,
+                                              std::uint32_t rows,
+                                              bool leave_partials) {
+  const auto& layer = layers_[index];
+  enqueue_normalise(layer.post_attention_norm, rows);
+  status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor, &layer.up.descriptor,
+                                    normalized_,
+                                    std::size_t{rows} * g_.hidden * 2U,
+                                    activation_, rows, stream_));
+  enqueue_residual_projection(layer.down.descriptor, activation_,
+                              std::size_t{rows} * g_.intermediate * 2U, rows,
+                              leave_partials);
+}
+
+// head (run_head, :8393-8432) on rows [first_row, first_row + rows) of
+// hidden_: logits_ [rows, vocabulary] and their arg-max tokens.  The norm
+// also completes hidden_ when partials are pending, which is only so for a
+// head over all rows.
+void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
+                                         std::uint32_t rows) {
+  if (pending_partials_ && first_row != 0U)
+    throw std::runtime_error("head over a row range needs a complete hidden state");
+  if (first_row == 0U) {
+    enqueue_normalise(final_norm_, rows);
+  } else {
+    status_check(qllm_rms_norm_batch(
+        hidden_ + std::size_t{first_row} * g_.hidden, final_norm_, nullptr,
+        normalized_, g_.hidden, rows, g_.hidden, g_.norm_epsilon,
+        g_.zero_centered_norm, stream_));
+  }
+  status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
+                                  std::size_t{rows} * g_.hidden * 2U, logits_,
+                                  QLLM_OUT_F32, nullptr, rows, stream_));
   status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
                                  select_workspace_, select_workspace_bytes_,
-                                 stream));
+                                 stream_));
+}
+
+void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
+                                           std::uint32_t rows,
+                                           std::uint32_t first_position,
+                                           bool deferred_positions) {
+  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
+                                        hidden_, rows, stream_));
+  pending_partials_ = 0U;
+  for (std::uint32_t index = 0; index < g_.layers; ++index) {
+    enqueue_attention_block(index, rows, first_position, deferred_positions,
+                            true);
+    enqueue_ffn_block(index, rows, true);
+  }
+  enqueue_head(0U, rows);
 }
 
 // The proposer's pass over a prompt chunk: row r pairs tokens[r] (the token
@@ -1511,6 +1925,36 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
           status_check(qllm_fp4_gemm_bf16(
               &down, activation_, std::size_t{rows} * g_.intermediate * 2U,
               query_, QLLM_OUT_F32, nullptr, rows, stream_));
+      } else if (which == "qkv") {
+        // as the target pass launches it
+        const auto& qkv = layer.qkv.descriptor;
+        const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+        if (qkv_splits_ > 1U && qkv.layout == QLLM_LAYOUT_TILED &&
+            qkv.padded_columns / 64U >= qkv_splits_) {
+          status_check(qllm_fp4_gemm_bf16_partial(&qkv, normalized_, hidden_bytes,
+                                                  qkv_partials_, qkv_splits_,
+                                                  rows, stream_));
+        } else {
+          const qllm_gemm_segment projections[3] = {
+              {query_, qkv.rows - 2U * kv_rows, QLLM_OUT_F32},
+              {key_, kv_rows, QLLM_OUT_F32},
+              {value_, kv_rows, QLLM_OUT_F32}};
+          status_check(qllm_fp4_gemm_bf16_split(&qkv, normalized_, hidden_bytes,
+                                                projections, 3U, rows, stream_));
+        }
+      } else if (which == "attention_output") {
+        const auto& output = layer.output.descriptor;
+        const std::size_t bytes =
+            std::size_t{rows} * g_.query_heads * g_.head_dim * 2U;
+        if (projection_splits_ > 1U && output.layout == QLLM_LAYOUT_TILED &&
+            output.padded_columns / 64U >= projection_splits_)
+          status_check(qllm_fp4_gemm_bf16_partial(&output, attention_, bytes,
+                                                  projection_partials_,
+                                                  projection_splits_, rows,
+                                                  stream_));
+        else
+          status_check(qllm_fp4_gemm_bf16(&output, attention_, bytes, query_,
+                                          QLLM_OUT_F32, nullptr, rows, stream_));
       } else if (which == "lm_head") {
         status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
                                         hidden_bytes, logits_, QLLM_OUT_F32,
@@ -2460,18 +2904,34 @@ Mi355DenseFp4Provider::telemetry() const {
   return values;
 }
 
-er::ServiceContract Mi355DenseFp4Provider::service_contract() const {
-  er::ServiceContract contract;
+// The contract the runner validates and publishes (values of
+// dense_fp4_provider.cpp:11447-11486 for a dense resident model).
+er::ExecutionProviderModule::ServiceContract
+Mi355DenseFp4Provider::service_contract() const {
+  er::ExecutionProviderModule::ServiceContract contract;
+  contract.prefill_mode = "causal_layer_major";
+  contract.prefill_chunk_tokens = max_rows_;   // rows one execute() batch holds
+  contract.session_retention = false;
+  contract.request_stream_mode = "per_request_nonblocking";
+  contract.rope_mode = "artifact";
   contract.kv_dtype = g_.kv_encoding == KvEncoding::fp16 ? "fp16"
                                                           : "q4-f16-per-head";
-  contract.kv_allocation = "on-demand-pages";
+  contract.kv_allocation = "paged_on_demand";
   contract.kv_page_tokens = g_.kv_page_tokens;
   contract.kv_page_bytes = kv_page_bytes_;
   contract.kv_page_capacity = pages_.size();
   contract.placement_mode = "resident";
-  contract.mtp_resource_available = true;
+  contract.placement_profile = "resident";
+  contract.ram_cache_bytes = 0U;
+  contract.vram_cache_bytes = std::max<std::uint64_t>(weight_bytes_, 1U);
+  contract.placement_prefetch_enabled = false;
+  contract.placement_prefetch_state = "disabled";
+  contract.placement_minimum_observations = 0U;
+  contract.mtp_resource_available = static_cast<bool>(exact_);
   contract.mtp_runtime_ready = static_cast<bool>(exact_);
   contract.mtp_enabled = static_cast<bool>(exact_);
+  contract.retain_previous_route = false;
+  contract.cpu_hybrid_enabled = false;
   contract.sampling_supported = true;
   return contract;
 }

@@ -19,8 +19,9 @@
 #include <vector>
 
 #include "qllm_kernels.h"
-#include "runtime_interface.hpp"
-#include "speculative_sampling.hpp"
+#include "expert/runtime/program_executor.hpp"
+#include "expert/runtime/worker_provider.hpp"
+#include "expert/runtime/speculative_sampling.hpp"
 
 namespace qllm {
 
@@ -73,6 +74,17 @@ class DenseFp4RequestState final : public er::IOperationProviderRequestState {
   std::uint32_t mtp_length{};   // position of the guaranteed token
   bool draft_valid{};
   std::vector<DraftPrediction> draft_predictions;
+  // the batch execute() is walking through the program
+  // (RequestState, dense_fp4_provider.cpp:2195-2260)
+  std::uint32_t current_batch_rows{};
+  std::uint32_t current_batch_first{};
+  std::uint32_t current_position{};
+  bool exact_decode_enabled{};
+  // target rows of the last head whose successors the proposer has not been
+  // told yet: positions synchronization_first .. + synchronization_rows
+  std::uint32_t synchronization_first{};
+  std::uint32_t synchronization_rows{};
+  std::uint32_t synchronization_consumed{};
 };
 
 struct DeviceFp4Matrix final {
@@ -117,8 +129,23 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       const er::OperationPreparationContext& context) override;
   [[nodiscard]] er::CreateOperationRequestStateResult create_request_state(
       const er::ProgramRequestContext& request) override;
+  // One operation of the program on the batch the embedding started
+  // (dense_fp4_provider.cpp:10680-10992): token ids and positions arrive as
+  // host values, the hidden state travels between operations as a device
+  // value, the head returns token ids as a host value.
+  [[nodiscard]] er::OperationExecutionHandle execute(
+      const er::IPreparedOperation& operation,
+      const std::shared_ptr<er::IOperationProviderRequestState>& request_state,
+      const er::OperationInvocation& invocation) override;
+  [[nodiscard]] er::Status rebind_request_state(
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      const er::ProgramRequestContext& request) override;
   [[nodiscard]] er::PrepareOperationResult prepare_exact_decode(
       const er::ExactDecodePreparationContext& context) override;
+  [[nodiscard]] er::Status synchronize_exact_decode(
+      const er::IPreparedOperation& operation,
+      const std::shared_ptr<er::IOperationProviderRequestState>& state,
+      const er::ExactDecodeSynchronization& synchronization) override;
   [[nodiscard]] er::Status synchronize_exact_decode_batch(
       const er::IPreparedOperation& operation,
       const std::shared_ptr<er::IOperationProviderRequestState>& state,
@@ -166,7 +193,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   // Average duration, in microseconds, of one launch of a hot kernel measured
   // with HIP events on the provider's stream: the kernel is launched once per
   // layer (distinct weights / KV each time) for `rounds` passes over the
-  // layers.  which: "ffn_gate_up", "ffn_down", "attention", "lm_head".
+  // layers.  which: "ffn_gate_up", "ffn_down", "qkv", "attention_output",
+  // "attention", "lm_head".
   [[nodiscard]] er::Status time_kernel(const std::string& which,
                                        std::uint32_t rounds,
                                        std::uint32_t context_tokens,
@@ -181,7 +209,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   [[nodiscard]] const DenseGeometry& geometry() const noexcept { return g_; }
   [[nodiscard]] std::map<std::string, std::uint64_t, std::less<>> telemetry()
       const;
-  [[nodiscard]] er::ServiceContract service_contract() const;
+  [[nodiscard]] er::ExecutionProviderModule::ServiceContract service_contract()
+      const;
 
   // Prompt prefill: runs `tokens` (positions first_position ..) through the
   // target in chunks of up to prefill_chunk_rows() rows - the linears on the
@@ -214,8 +243,35 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                         void* host_output);
 
  private:
-  struct PreparedOp;
+  struct PreparedOperation;
   void allocate_workspaces();
+  // the blocks of a target pass on rows [0, rows) of hidden_; with
+  // `leave_partials` a residual projection may end as K-split partials that
+  // the next norm adds (pending_partials_), otherwise hidden_ is complete
+  // when the block returns
+  void enqueue_normalise(const float* weight, std::uint32_t rows);
+  void enqueue_residual_projection(const qllm_fp4_matrix& matrix,
+                                   const std::uint16_t* input,
+                                   std::size_t input_bytes, std::uint32_t rows,
+                                   bool leave_partials);
+  void enqueue_attention_block(std::uint32_t index, std::uint32_t rows,
+                               std::uint32_t first_position,
+                               bool deferred_positions, bool leave_partials);
+  void enqueue_ffn_block(std::uint32_t index, std::uint32_t rows,
+                         bool leave_partials);
+  void enqueue_head(std::uint32_t first_row, std::uint32_t rows);
+  // run_head with a request (dense_fp4_provider.cpp:8433-8517): presence
+  // penalty, arg-max or sampling of the single head row in logits_, the
+  // emitted token marked
+  std::uint32_t select_head_token(const er::ProgramRequestContext& request,
+                                  std::uint32_t sample_position);
+  [[nodiscard]] er::ExecutionValue device_hidden_value(std::uint32_t rows) const;
+  [[nodiscard]] std::uint32_t require_hidden_value(
+      const er::ExecutionValue& value) const;
+  std::uint32_t pending_partials_{};
+  std::shared_ptr<const void> device_lifetime_;
+  std::vector<std::shared_ptr<const PreparedOperation>> prepared_attention_;
+  std::vector<std::shared_ptr<const PreparedOperation>> prepared_ffn_;
   void ensure_pages(std::uint32_t last_position);
   DeviceFp4Matrix upload_matrix(const er::ImmutableModelTensor& tensor,
                                 bool tiled);
@@ -248,8 +304,10 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       std::uint32_t sample_position, std::uint32_t random_stream);
   void enqueue_attention(std::uint32_t index, std::uint32_t rows,
                          std::uint32_t first_position, bool deferred_positions,
-                         float* query, float* key, const float* value,
-                         std::uint16_t* attention_out);
+                         float* query, float* key, float* value,
+                         std::uint16_t* attention_out,
+                         const float* qkv_partials = nullptr,
+                         std::uint32_t qkv_partial_count = 0U);
   // buffers for `rows` prompt rows at a time (allocated on first use)
   void ensure_prefill_workspace(std::uint32_t rows);
   void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
@@ -324,6 +382,12 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   HostStaging* staging_ = nullptr;
   float* projection_partials_ = nullptr;   // [splits][rows][hidden]
   std::uint32_t projection_splits_ = 3U;   // 0 / 1: residual in the epilogue
+  // The q/k/v projection cut along K the same way (QLLM_PROVIDER_QKV_SPLITS);
+  // the rope + store kernel adds the partials.  0 / 1: one workgroup per
+  // tile, the default - its 320 tiles already cover the GPU, and 2..8 cuts
+  // measured 11.4-14.5 us against 11.7 us uncut.
+  float* qkv_partials_ = nullptr;          // [splits][rows][q + k + v rows]
+  std::uint32_t qkv_splits_ = 0U;
   void* select_workspace_{};
   std::size_t select_workspace_bytes_{};
   std::uint32_t* argmax_tokens_{};

@@ -3,14 +3,10 @@
 // files and, per dense tensor, its record inside a pack.  Dense-only: an
 // artifact whose program declares routed expert components is rejected, since
 // this provider executes none.  Names and meanings follow
-// runtime/include/expert/runtime/model_artifact.hpp:15-92 and
-// model_tensor_store.hpp:15-34; the record layout is
-// docs/expert-pack-v1.md:20-36 with the header of
-// compiler/expert_pack/constants.py:72-92.
+// runtime/include/expert/runtime/model_artifact.hpp:15-92.
 #pragma once
 
-#include "model_descriptor.hpp"
-#include "runtime_interface.hpp"
+#include "expert/runtime/model_descriptor.hpp"
 
 #include <cstdint>
 #include <filesystem>
@@ -81,36 +77,5 @@ class ModelArtifact final {
   std::vector<ArtifactPack> packs_;
   std::vector<ArtifactDenseTensor> dense_tensors_;
 };
-
-// Read-only memory mapping of the dense packs, each checked against the
-// manifest's SHA-256 when it is mapped.  resolve() hands out views into the
-// mapping; they stay valid while the store or any resolved tensor lives.
-class MappedModelTensorStore final : public IModelTensorStore {
- public:
-  MappedModelTensorStore();
-  MappedModelTensorStore(const MappedModelTensorStore&) = delete;
-  MappedModelTensorStore& operator=(const MappedModelTensorStore&) = delete;
-  MappedModelTensorStore(MappedModelTensorStore&&) noexcept;
-  MappedModelTensorStore& operator=(MappedModelTensorStore&&) noexcept;
-  ~MappedModelTensorStore() override;
-
-  [[nodiscard]] static Status create(const ModelArtifact& artifact,
-                                     MappedModelTensorStore& destination) noexcept;
-  [[nodiscard]] ResolveModelTensorResult resolve(std::string_view name) override;
-  [[nodiscard]] bool valid() const noexcept;
-
- private:
-  struct Core;
-  std::shared_ptr<Core> core_;
-};
-
-// Checks the 256-byte header of a dense record against its index entry:
-// magic, version, sizes, row-major flag, rank and shape, SHA-256 of the name,
-// section ranges, and the byte counts the quantisation ABI implies
-// (compiler/expert_pack/validate.py:148-325, without re-hashing the payload,
-// which the pack's own checksum covers).  `record` points at the header.
-[[nodiscard]] Status validate_dense_record(const ArtifactDenseTensor& entry,
-                                           const std::byte* record,
-                                           std::uint64_t available_bytes) noexcept;
 
 }  // namespace expert::runtime

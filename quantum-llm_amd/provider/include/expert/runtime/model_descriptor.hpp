@@ -2,13 +2,11 @@
 // needs (kernel capabilities and ABIs), its operations in order with their
 // integer parameters, tensor roles and SSA values, and the optional exact
 // (speculative) decode service.  Types and functions carry the names and
-// meanings of runtime/include/expert/runtime/model_descriptor.hpp:18-293; the
-// compiled form (CompiledModelProgram, :195-262) belongs to the reference's
-// program executor and has no counterpart here.
+// meanings of runtime/include/expert/runtime/model_descriptor.hpp:18-293,
+// the compiled form (CompiledModelProgram, :195-262) included.
 #pragma once
 
-#include "sha256.hpp"
-#include "status.hpp"
+#include "expert/runtime/storage.hpp"
 
 #include <cstdint>
 #include <filesystem>
@@ -109,6 +107,25 @@ struct OperationProgramDescriptor final {
   // provider port -> artifact-declared SSA value and its ABI
   std::map<std::string, ValueBinding, std::less<>> input_bindings;
   std::map<std::string, ValueBinding, std::less<>> output_bindings;
+
+  OperationProgramDescriptor() = default;
+  OperationProgramDescriptor(
+      std::uint32_t logical_operation_value, std::uint32_t logical_layer_value,
+      std::string capability_value, std::uint32_t abi_version_value,
+      std::string routed_component_value, std::uint32_t component_layer_value,
+      ParameterMap parameters_value = {}, BindingMap tensor_bindings_value = {},
+      std::map<std::string, ValueBinding, std::less<>> input_bindings_value = {},
+      std::map<std::string, ValueBinding, std::less<>> output_bindings_value = {})
+      : logical_operation(logical_operation_value),
+        logical_layer(logical_layer_value),
+        capability(std::move(capability_value)),
+        abi_version(abi_version_value),
+        routed_component(std::move(routed_component_value)),
+        component_layer(component_layer_value),
+        parameters(std::move(parameters_value)),
+        tensor_bindings(std::move(tensor_bindings_value)),
+        input_bindings(std::move(input_bindings_value)),
+        output_bindings(std::move(output_bindings_value)) {}
 };
 
 // :149-152
@@ -145,6 +162,73 @@ struct ModelDescriptor final {
   std::optional<ExactDecodeProgramDescriptor> exact_decode_program;
 };
 
+// The program with every name resolved to an index, once, at start-up
+// (:195-262): which capability of which provider serves a required kernel,
+// which SSA value a port reads or writes.
+struct CompiledKernelBinding final {
+  std::uint32_t requirement_index{};
+  // filled in by ExecutionProviderRegistry::bind; compile_model_program()
+  // compiles against one capability table and leaves it zero
+  std::uint32_t provider_registry_index{};
+  std::uint32_t provider_capability_index{};
+};
+
+struct CompiledLayerProgram final {
+  std::uint32_t logical_layer{};
+  std::uint32_t block_kernel_binding{};
+  std::optional<std::uint32_t> routed_component_index;
+  std::uint32_t component_layer{};
+  ParameterMap parameters;
+};
+
+struct CompiledOperationProgram final {
+  std::uint32_t logical_operation{};
+  std::uint32_t logical_layer{};
+  std::uint32_t kernel_binding{};
+  std::optional<std::uint32_t> routed_component_index;
+  std::uint32_t component_layer{};
+  ParameterMap parameters;
+  BindingMap tensor_bindings;
+  struct ValueBinding final {
+    std::string port;
+    std::uint32_t value_index{};
+  };
+  std::vector<ValueBinding> input_values;
+  std::vector<ValueBinding> output_values;
+};
+
+struct CompiledProgramValue final {
+  std::string name;
+  std::string abi;
+};
+
+struct CompiledProgramEndpoint final {
+  std::string role;
+  std::uint32_t value_index{};
+};
+
+struct CompiledExactDecodeProgram final {
+  std::uint32_t kernel_binding{};
+  std::uint32_t maximum_emitted_tokens{};
+  ParameterMap parameters;
+  BindingMap tensor_bindings;
+};
+
+struct CompiledModelProgram final {
+  std::vector<CompiledKernelBinding> kernels;
+  std::vector<CompiledLayerProgram> layers;
+  std::vector<CompiledOperationProgram> operations;
+  std::vector<CompiledProgramValue> values;
+  std::vector<CompiledProgramEndpoint> inputs;
+  std::vector<CompiledProgramEndpoint> outputs;
+  std::optional<CompiledExactDecodeProgram> exact_decode;
+};
+
+struct CompileModelProgramResult final {
+  Status status;
+  CompiledModelProgram program;
+};
+
 struct ParseModelDescriptorResult final {
   Status status;
   ModelDescriptor descriptor;
@@ -157,6 +241,9 @@ struct ParseModelDescriptorResult final {
     const RoutedExpertComponentDescriptor& component,
     std::uint32_t model_hidden_size) noexcept;
 [[nodiscard]] Status provider_supports_model(
+    const ModelDescriptor& descriptor,
+    std::span<const KernelCapability> capabilities) noexcept;
+[[nodiscard]] CompileModelProgramResult compile_model_program(
     const ModelDescriptor& descriptor,
     std::span<const KernelCapability> capabilities) noexcept;
 // Parses the line-oriented program text.  Component namespace offsets are

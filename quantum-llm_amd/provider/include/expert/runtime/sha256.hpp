@@ -5,15 +5,14 @@
 // (runtime/include/expert/runtime/sha256.hpp:26-28).
 #pragma once
 
+#include "expert/runtime/storage.hpp"
+
 #include <array>
 #include <cstddef>
 #include <cstdint>
 #include <span>
 
 namespace expert::runtime {
-
-// storage.hpp:47
-using Sha256Digest = std::array<std::byte, 32>;
 
 // Incremental form: feed() any number of times, then digest().
 class Sha256Stream final {

@@ -1,7 +1,10 @@
-// Status and error codes of the common runtime
-// (runtime/include/expert/runtime/storage.hpp:17-45).
+// Status and error codes of the common runtime and the digest type
+// (runtime/include/expert/runtime/storage.hpp:17-47); the storage requests
+// of that header belong to routed-expert paging and are not restated.
 #pragma once
 
+#include <array>
+#include <cstddef>
 #include <cstdint>
 #include <string>
 #include <string_view>
@@ -38,5 +41,8 @@ class Status final {
   ErrorCode code_{ErrorCode::ok};
   std::string message_;
 };
+
+// storage.hpp:47
+using Sha256Digest = std::array<std::byte, 32>;
 
 }  // namespace expert::runtime

@@ -1,7 +1,8 @@
 // Parser and validator of the artifact's model program.  Behaviour (what is
 // accepted, what is rejected and with which message) follows
 // runtime/src/model_descriptor.cpp:107-723 of the reference.
-#include "model_descriptor.hpp"
+#include "expert/runtime/model_descriptor.hpp"
+#include "expert/runtime/sha256.hpp"
 
 #include <algorithm>
 #include <charconv>
@@ -578,6 +579,106 @@ Status provider_supports_model(
   } catch (const std::exception& error) {
     return {ErrorCode::internal,
             std::string("execution provider validation failed: ") + error.what()};
+  }
+}
+
+// Names resolved to indices once (runtime/src/model_descriptor.cpp:374-490):
+// kernel binding k stands for required kernel k and the position of the first
+// capability that serves it; layers and operations refer to their kernel
+// binding and component by index; under schema 3 every SSA value gets a slot -
+// program inputs first (in role order), then each operation's outputs in
+// program order - and ports refer to slots.
+CompileModelProgramResult compile_model_program(
+    const ModelDescriptor& descriptor,
+    std::span<const KernelCapability> capabilities) noexcept {
+  if (auto supported = provider_supports_model(descriptor, capabilities);
+      !supported.ok())
+    return {std::move(supported), {}};
+  try {
+    CompiledModelProgram program;
+    const auto binding_of = [&](const std::string& capability,
+                                std::uint32_t abi) -> std::uint32_t {
+      for (std::uint32_t k = 0; k < descriptor.required_kernels.size(); ++k)
+        if (descriptor.required_kernels[k].capability == capability &&
+            descriptor.required_kernels[k].abi_version == abi)
+          return k;
+      throw std::out_of_range("kernel requirement is not declared");
+    };
+    const auto component_of =
+        [&](const std::string& name) -> std::optional<std::uint32_t> {
+      if (name.empty()) return std::nullopt;
+      for (std::uint32_t c = 0; c < descriptor.routed_components.size(); ++c)
+        if (descriptor.routed_components[c].name == name) return c;
+      throw std::out_of_range("routed component is not declared");
+    };
+    for (std::uint32_t k = 0; k < descriptor.required_kernels.size(); ++k) {
+      const auto& required = descriptor.required_kernels[k];
+      std::uint32_t offered = 0;
+      while (offered < capabilities.size() &&
+             !(capabilities[offered].capability == required.capability &&
+               required.abi_version >= capabilities[offered].minimum_abi &&
+               required.abi_version <= capabilities[offered].maximum_abi))
+        ++offered;
+      program.kernels.push_back({k, 0U, offered});
+    }
+    for (const auto& layer : descriptor.layer_program)
+      program.layers.push_back(
+          {layer.logical_layer,
+           binding_of(layer.block_capability, layer.block_abi_version),
+           component_of(layer.routed_component), layer.component_layer,
+           layer.parameters});
+    if (descriptor.operation_program.empty()) {
+      // schema 1: one block per layer stands for the operation program
+      for (const auto& layer : descriptor.layer_program)
+        program.operations.push_back(
+            {static_cast<std::uint32_t>(program.operations.size()),
+             layer.logical_layer,
+             binding_of(layer.block_capability, layer.block_abi_version),
+             component_of(layer.routed_component), layer.component_layer,
+             layer.parameters, {}, {}, {}});
+    } else {
+      for (const auto& operation : descriptor.operation_program)
+        program.operations.push_back(
+            {operation.logical_operation, operation.logical_layer,
+             binding_of(operation.capability, operation.abi_version),
+             component_of(operation.routed_component), operation.component_layer,
+             operation.parameters, operation.tensor_bindings, {}, {}});
+    }
+    if (descriptor.schema_version >= 3U) {
+      std::map<std::string, std::uint32_t, std::less<>> slots;
+      const auto new_slot = [&](const std::string& name, const std::string& abi) {
+        const auto slot = static_cast<std::uint32_t>(program.values.size());
+        program.values.push_back({name, abi});
+        slots.emplace(name, slot);
+        return slot;
+      };
+      for (const auto& [role, endpoint] : descriptor.program_inputs)
+        program.inputs.push_back({role, new_slot(endpoint.value, endpoint.abi)});
+      for (std::size_t index = 0; index < descriptor.operation_program.size();
+           ++index) {
+        const auto& source = descriptor.operation_program[index];
+        auto& compiled = program.operations[index];
+        for (const auto& [port, bound] : source.input_bindings)
+          compiled.input_values.push_back({port, slots.at(bound.value)});
+        for (const auto& [port, bound] : source.output_bindings)
+          compiled.output_values.push_back(
+              {port, new_slot(bound.value, bound.abi)});
+      }
+      for (const auto& [role, endpoint] : descriptor.program_outputs)
+        program.outputs.push_back({role, slots.at(endpoint.value)});
+    }
+    if (descriptor.exact_decode_program) {
+      const auto& decode = *descriptor.exact_decode_program;
+      program.exact_decode = CompiledExactDecodeProgram{
+          binding_of(decode.capability, decode.abi_version),
+          decode.maximum_emitted_tokens, decode.parameters,
+          decode.tensor_bindings};
+    }
+    return {Status::success(), std::move(program)};
+  } catch (const std::exception& error) {
+    return {{ErrorCode::internal,
+             std::string("model program compilation failed: ") + error.what()},
+            {}};
   }
 }
 

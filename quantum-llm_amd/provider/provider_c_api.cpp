@@ -13,7 +13,10 @@
 
 #include "artifact_provider.hpp"
 #include "dense_fp4_provider.hpp"
+#include "dense_record.hpp"
+#include "expert/runtime/sha256.hpp"
 #include "descriptor_dump.hpp"
+#include "registry_probe.hpp"
 
 namespace er = expert::runtime;
 
@@ -22,6 +25,9 @@ struct qllm_provider {
   // set when the provider was created from an artifact directory
   std::shared_ptr<er::ModelArtifact> artifact;
   std::shared_ptr<er::IModelTensorStore> tensor_store;
+  // the compiled form of every prepared operation, in program order: what
+  // execute() is invoked with
+  std::vector<er::CompiledOperationProgram> compiled;
   std::vector<er::PreparedTensorBinding> staged;
   std::vector<std::shared_ptr<const er::IPreparedOperation>> operations;
   std::shared_ptr<const er::IPreparedOperation> exact;
@@ -99,18 +105,40 @@ extern "C" qllm_provider* qllm_provider_create_from_artifact(
     if (kv_page_tokens) options.kv_page_tokens = kv_page_tokens;
     if (kv_cache_dtype) options.kv_cache_dtype = kv_cache_dtype;
     options.mtp_draft_depth = mtp_draft_depth;
-    auto created =
-        qllm::make_mi355_dense_fp4_callable_provider(artifact_root, options);
+    // what the runner's main does (moe_vm_runner.cpp:1501-1528): load the
+    // artifact, create the one module that serves its program, bind, prepare
+    auto artifact = std::make_shared<er::ModelArtifact>();
+    if (auto status = er::ModelArtifact::load(artifact_root, *artifact);
+        !status.ok()) {
+      from_status(status);
+      return nullptr;
+    }
+    if (mtp_draft_depth)
+      if (auto status = artifact->configure_mtp_draft_depth(mtp_draft_depth);
+          !status.ok()) {
+        from_status(status);
+        return nullptr;
+      }
+    auto created = qllm::make_mi355_dense_fp4_module(artifact, options);
     if (!created.status.ok()) {
       from_status(created.status);
       return nullptr;
     }
+    qllm::PreparedProgram prepared;
+    if (auto status =
+            qllm::prepare_program(artifact->model(), created.module, prepared);
+        !status.ok()) {
+      from_status(status);
+      return nullptr;
+    }
     auto handle = std::make_unique<qllm_provider>();
-    handle->provider = std::move(created.module.implementation);
-    handle->artifact = std::move(created.module.artifact);
+    handle->provider = std::dynamic_pointer_cast<qllm::Mi355DenseFp4Provider>(
+        created.module.definition.implementation);
+    handle->artifact = std::move(artifact);
     handle->tensor_store = std::move(created.module.tensor_store);
-    handle->operations = std::move(created.module.operations);
-    handle->exact = std::move(created.module.exact_decode);
+    handle->operations = std::move(prepared.operations);
+    handle->compiled = std::move(prepared.bound.program.operations);
+    handle->exact = std::move(prepared.exact_decode);
     return handle.release();
   } catch (const std::exception& error) {
     fail(QLLM_INTERNAL, error.what());
@@ -173,32 +201,89 @@ extern "C" int32_t qllm_provider_prepare(qllm_provider* provider,
                                          const char* capability) {
   if (!provider || !capability)
     return fail(QLLM_INVALID_ARGUMENT, "prepare arguments are invalid");
-  er::OperationPreparationContext context;
-  context.capability = capability;
-  context.abi = 1U;
-  context.tensors = provider->staged;
-  auto result = provider->provider->prepare(context);
-  provider->staged.clear();
-  if (!result.status.ok()) return from_status(result.status);
-  provider->operations.push_back(result.operation);
-  return QLLM_OK;
+  try {
+    // A one-operation program description for the staged tensors: the ports
+    // and value ABIs the artifact compiler declares for this kind of block
+    // (compiler/expert_pack/adapters.py:1422-1602).
+    const std::string name = capability;
+    const std::string hidden = "batch.hidden.f32.cuda.v1";
+    const std::string token = "batch.token-id.u32.host.v1";
+    const std::string position = "batch.position.u32.host.v1";
+    const auto index = static_cast<uint32_t>(provider->operations.size());
+    er::OperationProgramDescriptor operation;
+    operation.logical_operation = index;
+    operation.logical_layer = er::kModelLevelOperationLayer;
+    operation.capability = name;
+    operation.abi_version = 1U;
+    const auto in = [&](const char* port, const std::string& abi) {
+      operation.input_bindings[port] = {std::string("staged.") + port, abi};
+    };
+    const auto out = [&](const char* port, const std::string& abi) {
+      operation.output_bindings[port] = {std::string("staged.out.") + port, abi};
+    };
+    if (name.starts_with("embedding.")) {
+      in("token_ids", token);
+      out("hidden", hidden);
+    } else if (name.starts_with("block.")) {
+      in("hidden", hidden);
+      in("positions", position);
+      out("hidden", hidden);
+    } else if (name.starts_with("head.")) {
+      in("hidden", hidden);
+      out("token_ids", token);
+    } else {
+      in("hidden", hidden);
+      out("hidden", hidden);
+    }
+    er::CompiledOperationProgram compiled;
+    compiled.logical_operation = index;
+    compiled.logical_layer = operation.logical_layer;
+    uint32_t slot = 0;
+    for (const auto& [port, binding] : operation.input_bindings)
+      compiled.input_values.push_back({port, slot++});
+    for (const auto& [port, binding] : operation.output_bindings)
+      compiled.output_values.push_back({port, slot++});
+    const er::ModelDescriptor model{};
+    auto result = provider->provider->prepare(
+        {model, operation, compiled, provider->staged});
+    provider->staged.clear();
+    if (!result.status.ok()) return from_status(result.status);
+    provider->operations.push_back(result.operation);
+    provider->compiled.push_back(std::move(compiled));
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    provider->staged.clear();
+    return fail(QLLM_INTERNAL, error.what());
+  }
 }
 
 extern "C" int32_t qllm_provider_prepare_exact_decode(qllm_provider* provider,
                                                       const char* capability) {
   if (!provider || !capability)
     return fail(QLLM_INVALID_ARGUMENT, "prepare arguments are invalid");
-  er::ExactDecodePreparationContext context;
-  context.capability = capability;
-  context.abi = 2U;
-  context.parameters["draft_depth"] = provider->provider->geometry().draft_depth;
-  context.parameters["source_mtp_layers"] = 1U;
-  context.tensors = provider->staged;
-  auto result = provider->provider->prepare_exact_decode(context);
-  provider->staged.clear();
-  if (!result.status.ok()) return from_status(result.status);
-  provider->exact = result.operation;
-  return QLLM_OK;
+  try {
+    // the exact-decode contract the artifact declares (:2934-2966)
+    const auto& geometry = provider->provider->geometry();
+    er::ExactDecodeProgramDescriptor program;
+    program.capability = capability;
+    program.abi_version = 2U;
+    program.maximum_emitted_tokens = geometry.draft_depth + 1U;
+    program.parameters["draft_depth"] = geometry.draft_depth;
+    program.parameters["source_mtp_layers"] = 1U;
+    er::CompiledExactDecodeProgram compiled;
+    compiled.maximum_emitted_tokens = program.maximum_emitted_tokens;
+    compiled.parameters = program.parameters;
+    const er::ModelDescriptor model{};
+    auto result = provider->provider->prepare_exact_decode(
+        {model, program, compiled, provider->staged});
+    provider->staged.clear();
+    if (!result.status.ok()) return from_status(result.status);
+    provider->exact = result.operation;
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    provider->staged.clear();
+    return fail(QLLM_INTERNAL, error.what());
+  }
 }
 
 extern "C" int32_t qllm_provider_load_synthetic_weights(qllm_provider* provider,
@@ -355,6 +440,87 @@ extern "C" int32_t qllm_provider_run_target(qllm_provider* provider,
                                             uint32_t first_position) {
   if (!provider) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
   return from_status(provider->provider->run_target(tokens, rows, first_position));
+}
+
+extern "C" int32_t qllm_provider_execute_program(qllm_provider* provider,
+                                                 const uint32_t* tokens,
+                                                 const uint32_t* positions,
+                                                 uint32_t rows,
+                                                 uint32_t* next_token) {
+  if (!provider || !tokens || !positions || !rows || !next_token ||
+      !provider->state || provider->operations.empty() ||
+      provider->operations.size() != provider->compiled.size())
+    return fail(QLLM_INVALID_ARGUMENT, "program execution arguments are invalid");
+  try {
+    // The operations in program order, each fed through its ports: token ids
+    // and positions are the program's inputs, the hidden state is whatever
+    // the operation before produced (the dense program is a chain).
+    const auto host_value = [](const char* abi, const uint32_t* words,
+                               uint32_t count) {
+      auto owner = std::make_shared<std::vector<uint32_t>>(words, words + count);
+      return er::ExecutionValue{abi, "host", owner,
+                                reinterpret_cast<const std::byte*>(owner->data()),
+                                owner->size() * sizeof(uint32_t)};
+    };
+    const auto token_value = host_value("batch.token-id.u32.host.v1", tokens, rows);
+    const auto position_value =
+        host_value("batch.position.u32.host.v1", positions, rows);
+    er::ExecutionValue hidden;
+    er::ExecutionValue selected;
+    for (size_t index = 0; index < provider->operations.size(); ++index) {
+      const auto& compiled = provider->compiled[index];
+      std::vector<er::ExecutionValue> inputs;
+      for (const auto& binding : compiled.input_values) {
+        if (binding.port == "token_ids")
+          inputs.push_back(token_value);
+        else if (binding.port == "positions")
+          inputs.push_back(position_value);
+        else if (binding.port == "hidden")
+          inputs.push_back(hidden);
+        else
+          return fail(QLLM_INVALID_ARGUMENT,
+                      "operation input port is not part of a dense program: " +
+                          binding.port);
+      }
+      auto handle = provider->provider->execute(
+          *provider->operations[index], provider->state,
+          er::OperationInvocation{provider->request, compiled, inputs});
+      if (!handle.valid())
+        return fail(QLLM_INVALID_ARGUMENT, "operation invocation was rejected");
+      auto result = handle.poll();
+      if (!result) return fail(QLLM_INTERNAL, "operation did not complete");
+      if (!result->status.ok()) return from_status(result->status);
+      if (result->outputs.size() != compiled.output_values.size())
+        return fail(QLLM_INTERNAL, "operation returned a partial output set");
+      for (size_t port = 0; port < compiled.output_values.size(); ++port) {
+        if (compiled.output_values[port].port == "hidden")
+          hidden = result->outputs[port];
+        else if (compiled.output_values[port].port == "token_ids")
+          selected = result->outputs[port];
+      }
+    }
+    if (!selected.valid() || selected.bytes < sizeof(uint32_t))
+      return fail(QLLM_INTERNAL, "program produced no token");
+    std::memcpy(next_token, selected.data + selected.bytes - sizeof(uint32_t),
+                sizeof(uint32_t));
+    return QLLM_OK;
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
+}
+
+extern "C" int32_t qllm_provider_synchronize_batch(qllm_provider* provider,
+                                                   const uint32_t* next_tokens,
+                                                   uint32_t count,
+                                                   uint32_t first_target_position,
+                                                   int32_t produce_final_draft) {
+  if (!provider || !provider->exact || !provider->state || !next_tokens || !count)
+    return fail(QLLM_INVALID_ARGUMENT, "exact decode is not prepared");
+  er::ExactDecodeSynchronizationBatch batch{
+      provider->request, {next_tokens, count}, first_target_position,
+      produce_final_draft != 0};
+  return from_status(provider->provider->synchronize_exact_decode_batch(
+      *provider->exact, provider->state, batch));
 }
 
 extern "C" int32_t qllm_provider_capture_target(qllm_provider* provider,
@@ -627,6 +793,22 @@ extern "C" int32_t qllm_model_descriptor_parse(
   if (!parsed.status.ok()) return from_status(parsed.status);
   return copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
                    dump_bytes);
+}
+
+extern "C" int32_t qllm_model_program_bind(
+    const char* text, size_t text_bytes, const uint8_t* content_sha256,
+    uint64_t namespace_base, const char* providers, int32_t executable,
+    char* dump, size_t capacity, size_t* dump_bytes) {
+  if ((!text && text_bytes) || !providers)
+    return fail(QLLM_INVALID_ARGUMENT, "model program or providers are null");
+  try {
+    return copy_text(
+        qllm::dump::bind_report({text, text_bytes}, digest_of(content_sha256),
+                                namespace_base, providers, executable != 0),
+        dump, capacity, dump_bytes);
+  } catch (const std::exception& error) {
+    return fail(QLLM_INTERNAL, error.what());
+  }
 }
 
 extern "C" int32_t qllm_model_descriptor_load(

@@ -1,4 +1,4 @@
-#include "sha256.hpp"
+#include "expert/runtime/sha256.hpp"
 
 #include <algorithm>
 #include <bit>

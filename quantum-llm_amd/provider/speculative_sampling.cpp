@@ -1,4 +1,4 @@
-#include "speculative_sampling.hpp"
+#include "expert/runtime/speculative_sampling.hpp"
 
 #include <algorithm>
 #include <cmath>

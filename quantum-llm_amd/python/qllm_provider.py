@@ -44,6 +44,8 @@ SIGNATURES = {
     "qllm_provider_begin_request": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint64]),
     "qllm_provider_begin_request_with": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32]),
     "qllm_provider_synchronize": (c_int32, [c_void_p, c_uint32, c_uint32]),
+    "qllm_provider_execute_program": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, POINTER(c_uint32)]),
+    "qllm_provider_synchronize_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_int32]),
     "qllm_provider_set_drafts": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_void_p]),
     "qllm_provider_verify": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint32)]),
     "qllm_provider_run_target": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32]),
@@ -72,6 +74,7 @@ SIGNATURES = {
     "qllm_sha256": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_sha256_portable": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_model_descriptor_parse": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
+    "qllm_model_program_bind": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_int32, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_model_descriptor_load": (c_int32, [c_char_p, c_uint64, c_char_p, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_artifact_open": (c_int32, [c_char_p, c_uint32, c_int32, POINTER(c_void_p)]),
     "qllm_artifact_close": (None, [c_void_p]),
@@ -183,6 +186,26 @@ class Provider:
         _check(self.lib.qllm_provider_prefill(self.handle, tokens.ctypes.data, tokens.size,
                                               first_position, ctypes.byref(predicted)))
         return predicted.value
+
+    def execute_program(self, tokens, first_position):
+        """The prepared program, operation by operation, on `tokens` at
+        consecutive positions; returns the head's token for the last row."""
+        import numpy as np
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        positions = np.arange(first_position, first_position + len(tokens),
+                              dtype=np.uint32)
+        selected = c_uint32()
+        _check(self.lib.qllm_provider_execute_program(
+            self.handle, tokens.ctypes.data, positions.ctypes.data, len(tokens),
+            ctypes.byref(selected)))
+        return selected.value
+
+    def synchronize_batch(self, next_tokens, first_target_position, produce_final_draft):
+        import numpy as np
+        next_tokens = np.ascontiguousarray(next_tokens, dtype=np.uint32)
+        _check(self.lib.qllm_provider_synchronize_batch(
+            self.handle, next_tokens.ctypes.data, len(next_tokens),
+            first_target_position, int(produce_final_draft)))
 
     def synchronize(self, token, position):
         _check(self.lib.qllm_provider_synchronize(self.handle, token, position))

@@ -33,6 +33,9 @@ def reference():
         lib.qref_model_descriptor_load.argtypes = [
             c_char_p, c_uint64, c_char_p, c_char_p, c_uint64, c_char_p, c_size_t,
             POINTER(c_size_t)]
+        lib.qref_model_program_bind.argtypes = [
+            c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_int, c_char_p, c_size_t,
+            POINTER(c_size_t)]
         lib.qref_artifact_open.argtypes = [c_char_p, c_uint32, c_int, POINTER(c_void_p),
                                            c_char_p, c_size_t]
         lib.qref_artifact_close.argtypes = [c_void_p]
@@ -80,6 +83,18 @@ class Product:
                                               byref(length))
         return (code, _text(buffer, length)) if code == 0 else (
             code, lib.qllm_provider_last_error().decode())
+
+    @staticmethod
+    def bind(text: bytes, content_hash: bytes, namespace_base: int, providers: str,
+             executable: bool):
+        """Report of registering `providers` and binding the program to them."""
+        lib = product()
+        buffer, length = create_string_buffer(CAPACITY), c_size_t()
+        code = lib.qllm_model_program_bind(text, len(text), content_hash, namespace_base,
+                                           providers.encode(), int(executable), buffer,
+                                           CAPACITY, byref(length))
+        assert code == 0, lib.qllm_provider_last_error().decode()
+        return _text(buffer, length)
 
     class Artifact:
         def __init__(self, root, mtp_draft_depth=0, map_tensors=True):
@@ -131,6 +146,15 @@ class Reference:
             os.fsencode(path), expected_bytes, expected_sha, content_hash, namespace_base,
             buffer, CAPACITY, byref(length))
         return code, _text(buffer, length)
+
+    @staticmethod
+    def bind(text: bytes, content_hash: bytes, namespace_base: int, providers: str,
+             executable: bool):
+        buffer, length = create_string_buffer(CAPACITY), c_size_t()
+        reference().qref_model_program_bind(text, len(text), content_hash, namespace_base,
+                                            providers.encode(), int(executable), buffer,
+                                            CAPACITY, byref(length))
+        return _text(buffer, length)
 
     class Artifact:
         def __init__(self, root, mtp_draft_depth=0, map_tensors=True):

@@ -25,9 +25,10 @@ HEADER_BYTES = 256
 DENSE_HEADER = struct.Struct("<8sHHIIIIIIIIQQQQQ32s32s")
 FLAG_ROW_MAJOR, FLAG_SYMMETRIC, FLAG_PER_ROW_SCALES = 1, 4, 8
 
-TOKEN_ABI = "token.batch.u32.v1"
-POSITION_ABI = "position.batch.u32.v1"
-HIDDEN_ABI = "hidden.batch.f32.v1"
+# the value ABIs the artifact compiler declares (compiler/expert_pack/adapters.py:111-113)
+TOKEN_ABI = "batch.token-id.u32.host.v1"
+POSITION_ABI = "batch.position.u32.host.v1"
+HIDDEN_ABI = "batch.hidden.f32.cuda.v1"
 
 
 def _align(value, alignment):

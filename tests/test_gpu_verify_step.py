@@ -31,8 +31,12 @@ def make(name, seed):
     return rng, model, step_oracle.build_provider(model, qp)
 
 
+@pytest.mark.parametrize("qkv_splits", ["0", "4"])
 @pytest.mark.parametrize("name", list(CONFIGS))
-def test_target_pass_matches_composed_oracle(device, name):
+def test_target_pass_matches_composed_oracle(device, monkeypatch, name, qkv_splits):
+    # qkv_splits 4: the q/k/v projection as four K-split partials that the
+    # rope + store kernel adds up (off by default)
+    monkeypatch.setenv("QLLM_PROVIDER_QKV_SPLITS", qkv_splits)
     rng, model, provider = make(name, 7)
     page_tokens = 64
     layer_bytes = ol.q4h_layer_bytes(page_tokens, model.kv_heads, model.head_dim)
