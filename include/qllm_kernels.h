@@ -100,6 +100,17 @@ int32_t qllm_fp4_prepack(const qllm_fp4_matrix* source, uint32_t tile_rows,
                          void* packed_weights, void* packed_scales,
                          qllm_fp4_matrix* packed, void* stream);
 
+/* The inverse for a row range: rows [first_row, first_row + row_count) of a
+ * matrix in either layout, as row-major codes [row_count, padded_columns/2] and
+ * scales (u8 [row_count, padded/32] or f16 [row_count, padded/16]) in device
+ * memory.  For tools and tests that need the values a provider holds (a
+ * random-init model is generated directly in the tiled layout); moves bytes
+ * and changes no value.  No counterpart in the reference, whose device layout
+ * is the artifact's. */
+int32_t qllm_fp4_unpack_rows(const qllm_fp4_matrix* matrix, uint32_t first_row,
+                             uint32_t row_count, void* weights, void* scales,
+                             void* stream);
+
 enum qllm_output_kind {
   QLLM_OUT_F32 = 0,         /* float [batch, rows] */
   QLLM_OUT_F32_BF16_ROUNDED = 1, /* float storage, values rounded to bf16

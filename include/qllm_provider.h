@@ -147,6 +147,16 @@ int32_t qllm_provider_prefill(qllm_provider* provider, const uint32_t* tokens,
                               uint32_t count, uint32_t first_position,
                               uint32_t* predicted);
 
+/* Rows [first_row, first_row + rows) of one of the provider's FP4 matrices as
+ * row-major codes [rows, padded_columns/2] and scales in host memory, whatever
+ * layout the device copy has (tools and tests; a random-init model exists on
+ * the device only).  name: "token_embedding", "output_head",
+ * "layer.<n>.qkv|output|gate|up|down" (qkv: query, key and value rows in that
+ * order), "mtp.fusion", "mtp.layer.qkv|output|gate|up|down". */
+int32_t qllm_provider_copy_matrix_rows(qllm_provider* provider, const char* name,
+                                       uint32_t first_row, uint32_t rows,
+                                       void* host_codes, void* host_scales);
+
 /* One batch through the prepared program, operation by operation, the way
  * the common VM drives a provider (IOperationProvider::execute,
  * runtime/include/expert/runtime/program_executor.hpp:251-254; the reference's

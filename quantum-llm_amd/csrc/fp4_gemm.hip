@@ -659,10 +659,109 @@ __global__ void fp4_prepack_kernel(const uint8_t* weights,
   }
 }
 
+// The inverse of fp4_prepack_kernel for rows [first_row, first_row + count):
+// every piece of the tiles that overlap the range puts its four dwords back
+// where the row-major layout has them.
+__global__ void fp4_unpack_kernel(const uint8_t* tiled_weights,
+                                  const uint8_t* tiled_scales,
+                                  uint8_t* out_weights, uint8_t* out_scales,
+                                  uint32_t first_row, uint32_t count,
+                                  uint32_t padded_columns, uint32_t f16_scales,
+                                  uint32_t h) {
+  const uint32_t chunks = padded_columns / kChunk;
+  const uint32_t half_rows = h / 2u;
+  const uint32_t first_tile = first_row / h;
+  const uint32_t last_tile = (first_row + count - 1u) / h;
+  const size_t pieces =
+      static_cast<size_t>(last_tile - first_tile + 1u) * chunks * 2u * h;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const uint32_t scale_chunk_bytes = f16_scales ? 8u : 2u;
+  const uint32_t scale_entries = f16_scales ? h : half_rows;
+  for (size_t local = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+       local < pieces; local += stride) {
+    const size_t piece =
+        local + static_cast<size_t>(first_tile) * chunks * 2u * h;
+    const uint32_t within = static_cast<uint32_t>(piece % (2u * h));
+    const size_t block = piece / (2u * h);
+    const uint32_t g = within / half_rows;
+    const uint32_t n = within % half_rows;
+    const uint32_t chunk = static_cast<uint32_t>(block % chunks);
+    const uint32_t tile = static_cast<uint32_t>(block / chunks);
+    const uint4 packed = *reinterpret_cast<const uint4*>(tiled_weights + piece * 16u);
+    const uint32_t value[4] = {packed.x, packed.y, packed.z, packed.w};
+    for (uint32_t j = 0; j < 2u; ++j)
+      for (uint32_t s = 0; s < 2u; ++s) {
+        const uint32_t row = tile * h + j * half_rows + n;
+        if (row < first_row || row >= first_row + count) continue;
+        *reinterpret_cast<uint32_t*>(
+            out_weights +
+            static_cast<size_t>(row - first_row) * (padded_columns / 2u) +
+            chunk * 32u + s * 16u + g * 4u) = value[2u * j + s];
+      }
+    if (within >= scale_entries) continue;
+    const uint32_t p = within / half_rows;
+    for (uint32_t j = 0; j < 2u; ++j)
+      for (uint32_t s = 0; s < 2u; ++s) {
+        const uint32_t row = tile * h + j * half_rows + n;
+        if (row < first_row || row >= first_row + count) continue;
+        uint8_t* target =
+            out_scales +
+            static_cast<size_t>(row - first_row) * (chunks * scale_chunk_bytes) +
+            chunk * scale_chunk_bytes;
+        if (f16_scales)
+          reinterpret_cast<uint16_t*>(target)[2u * s + p] =
+              reinterpret_cast<const uint16_t*>(
+                  tiled_scales + (block * h + within) * 8u)[2u * j + s];
+        else
+          target[s] = (tiled_scales + (block * half_rows + within) * 4u)[2u * j + s];
+      }
+  }
+}
+
 }  // namespace
 }  // namespace qllm
 
 using namespace qllm;
+
+extern "C" int32_t qllm_fp4_unpack_rows(const qllm_fp4_matrix* matrix,
+                                        uint32_t first_row, uint32_t row_count,
+                                        void* weights, void* scales,
+                                        void* stream) {
+  if (!matrix_ok(matrix) || !row_count || first_row >= matrix->rows ||
+      row_count > matrix->rows - first_row || !weights || !scales)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 row read-back");
+  const bool f16 = matrix->scale_scheme == QLLM_SCALE_F16_BLOCK16;
+  const size_t row_bytes = matrix->padded_columns / 2u;
+  const size_t scale_row_bytes =
+      f16 ? matrix->padded_columns / 8u : matrix->padded_columns / 32u;
+  if (matrix->layout == QLLM_LAYOUT_ROW_MAJOR) {
+    if (const int32_t status = checked(
+            hipMemcpyAsync(weights, matrix->weights + first_row * row_bytes,
+                           row_count * row_bytes, hipMemcpyDeviceToDevice,
+                           as_stream(stream)),
+            "copy FP4 rows"))
+      return status;
+    return checked(
+        hipMemcpyAsync(scales,
+                       static_cast<const uint8_t*>(matrix->scales) +
+                           first_row * scale_row_bytes,
+                       row_count * scale_row_bytes, hipMemcpyDeviceToDevice,
+                       as_stream(stream)),
+        "copy FP4 row scales");
+  }
+  if (matrix->padded_columns % kChunk != 0u)
+    return fail(QLLM_INVALID_ARGUMENT, "tiled FP4 matrix needs K % 64 == 0");
+  const uint32_t h = matrix_tile_rows(matrix);
+  const size_t tiles = (first_row + row_count - 1u) / h - first_row / h + 1u;
+  const size_t pieces = tiles * (matrix->padded_columns / kChunk) * 2u * h;
+  const uint32_t grid =
+      static_cast<uint32_t>(pieces / 256u < 16384u ? pieces / 256u + 1u : 16384u);
+  fp4_unpack_kernel<<<grid, 256, 0, as_stream(stream)>>>(
+      matrix->weights, static_cast<const uint8_t*>(matrix->scales),
+      static_cast<uint8_t*>(weights), static_cast<uint8_t*>(scales), first_row,
+      row_count, matrix->padded_columns, f16 ? 1u : 0u, h);
+  return launched("FP4 row read-back");
+}
 
 extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
                                       const void* input, size_t input_bytes,

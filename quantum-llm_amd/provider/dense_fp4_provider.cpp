@@ -2904,6 +2904,69 @@ Mi355DenseFp4Provider::telemetry() const {
   return values;
 }
 
+er::Status Mi355DenseFp4Provider::copy_matrix_rows(std::string_view name,
+                                                   std::uint32_t first_row,
+                                                   std::uint32_t rows,
+                                                   void* host_codes,
+                                                   void* host_scales) {
+  try {
+    std::lock_guard lock(mutex_);
+    const auto of_layer = [](const LayerWeights& layer,
+                             std::string_view which) -> const DeviceFp4Matrix* {
+      if (which == "qkv") return &layer.qkv;
+      if (which == "output") return &layer.output;
+      if (which == "gate") return &layer.gate;
+      if (which == "up") return &layer.up;
+      if (which == "down") return &layer.down;
+      return nullptr;
+    };
+    const DeviceFp4Matrix* matrix = nullptr;
+    if (name == "token_embedding") {
+      matrix = &embedding_;
+    } else if (name == "output_head") {
+      matrix = &head_;
+    } else if (name == "mtp.fusion") {
+      matrix = &mtp_.fusion;
+    } else if (name.starts_with("mtp.layer.")) {
+      matrix = of_layer(mtp_.layer, name.substr(10));
+    } else if (name.starts_with("layer.")) {
+      const auto rest = name.substr(6);
+      const auto dot = rest.find('.');
+      if (dot != std::string_view::npos) {
+        const auto index = std::stoul(std::string(rest.substr(0, dot)));
+        if (index < layers_.size())
+          matrix = of_layer(layers_[index], rest.substr(dot + 1U));
+      }
+    }
+    if (!matrix || !matrix->weights || !host_codes || !host_scales || !rows ||
+        first_row >= matrix->descriptor.rows ||
+        rows > matrix->descriptor.rows - first_row)
+      return {er::ErrorCode::invalid_argument,
+              "matrix name or row range is invalid: " + std::string(name)};
+    const auto& d = matrix->descriptor;
+    const std::size_t code_bytes = std::size_t{rows} * d.padded_columns / 2U;
+    const std::size_t scale_bytes =
+        d.scale_scheme == QLLM_SCALE_F16_BLOCK16
+            ? std::size_t{rows} * (d.padded_columns / 16U) * 2U
+            : std::size_t{rows} * (d.padded_columns / 32U);
+    DeviceBuffer codes(code_bytes, "allocate row read-back");
+    DeviceBuffer scales(scale_bytes, "allocate row read-back");
+    status_check(qllm_fp4_unpack_rows(&d, first_row, rows, codes.get(),
+                                      scales.get(), stream_));
+    const auto stream = static_cast<hipStream_t>(stream_);
+    hip_check(hipMemcpyAsync(host_codes, codes.get(), code_bytes,
+                             hipMemcpyDeviceToHost, stream),
+              "copy matrix rows");
+    hip_check(hipMemcpyAsync(host_scales, scales.get(), scale_bytes,
+                             hipMemcpyDeviceToHost, stream),
+              "copy matrix row scales");
+    hip_check(hipStreamSynchronize(stream), "copy matrix rows");
+    return er::Status::success();
+  } catch (const std::exception& error) {
+    return {er::ErrorCode::internal, error.what()};
+  }
+}
+
 // The contract the runner validates and publishes (values of
 // dense_fp4_provider.cpp:11447-11486 for a dense resident model).
 er::ExecutionProviderModule::ServiceContract

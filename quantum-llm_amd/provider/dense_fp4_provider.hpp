@@ -241,6 +241,14 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   }
   [[nodiscard]] er::Status copy_kv_page(std::uint32_t page_index,
                                         void* host_output);
+  // Rows [first_row, first_row + rows) of a weight matrix as row-major codes
+  // and scales in host memory, whatever layout the device copy has.  Names:
+  // "token_embedding", "output_head", "layer.<n>.qkv|output|gate|up|down",
+  // "mtp.fusion", "mtp.layer.qkv|output|gate|up|down".
+  [[nodiscard]] er::Status copy_matrix_rows(std::string_view name,
+                                            std::uint32_t first_row,
+                                            std::uint32_t rows, void* host_codes,
+                                            void* host_scales);
 
  private:
   struct PreparedOperation;

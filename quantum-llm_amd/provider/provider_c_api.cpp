@@ -523,6 +523,16 @@ extern "C" int32_t qllm_provider_synchronize_batch(qllm_provider* provider,
       *provider->exact, provider->state, batch));
 }
 
+extern "C" int32_t qllm_provider_copy_matrix_rows(qllm_provider* provider,
+                                                  const char* name,
+                                                  uint32_t first_row,
+                                                  uint32_t rows, void* host_codes,
+                                                  void* host_scales) {
+  if (!provider || !name) return fail(QLLM_INVALID_ARGUMENT, "provider is null");
+  return from_status(provider->provider->copy_matrix_rows(
+      name, first_row, rows, host_codes, host_scales));
+}
+
 extern "C" int32_t qllm_provider_capture_target(qllm_provider* provider,
                                                 const uint32_t* tokens,
                                                 uint32_t rows,

@@ -46,6 +46,7 @@ SIGNATURES = {
     "qllm_provider_synchronize": (c_int32, [c_void_p, c_uint32, c_uint32]),
     "qllm_provider_execute_program": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, POINTER(c_uint32)]),
     "qllm_provider_synchronize_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, c_int32]),
+    "qllm_provider_copy_matrix_rows": (c_int32, [c_void_p, c_char_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "qllm_provider_set_drafts": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_void_p]),
     "qllm_provider_verify": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_void_p, POINTER(c_uint32), POINTER(c_uint32), POINTER(c_uint32)]),
     "qllm_provider_run_target": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32]),
@@ -287,6 +288,17 @@ class Provider:
         _check(self.lib.qllm_provider_copy_kv_page(self.handle, page_index,
                                                    out.ctypes.data))
         return out
+
+    def matrix_rows(self, name, first_row, rows, padded_columns, scheme):
+        """(codes [rows, K/2] u8, scales) of a weight matrix's rows, row-major."""
+        import numpy as np
+        codes = np.empty((rows, padded_columns // 2), dtype=np.uint8)
+        scales = (np.empty((rows, padded_columns // 16), dtype=np.uint16) if scheme == 1
+                  else np.empty((rows, padded_columns // 32), dtype=np.uint8))
+        _check(self.lib.qllm_provider_copy_matrix_rows(
+            self.handle, name.encode(), first_row, rows, codes.ctypes.data,
+            scales.ctypes.data))
+        return codes, scales
 
     def mtp_state(self):
         """(last hidden [hidden], draft logits [draft_vocabulary]) of the proposer."""

@@ -1,0 +1,229 @@
+"""The benchmark configurations at their full sizes through the C ABI.
+
+* the 64-layer, hidden-5120 verify step at 32768 tokens of Q4H context: graph
+  replay bit-equal to kernel-by-kernel launches, greedy acceptance on the very
+  logits the GPU produced, the head against the oracle on sampled vocabulary
+  rows, and a whole layer of that model (same weights: the generator's seeds
+  run matrix by matrix) against the composed oracle;
+* the long-context attention launches with all eight KV heads: 131072 tokens
+  of Q4H and 262144 tokens of exact F16, split-invariant and against the oracle
+  on one KV head of the same launch;
+* lm_head over the 151936-token vocabulary with stochastic acceptance against
+  Dirichlet(0.1) draft distributions over the whole vocabulary.
+"""
+import numpy as np
+import pytest
+
+import gpu_util as gu
+import oracle_lib as ol
+import qllm_provider as qp
+import step_oracle
+import synth
+
+pytestmark = pytest.mark.gpu
+
+MODEL = dict(hidden=5120, intermediate=17408, layers=64, query_heads=64, kv_heads=8,
+             head_dim=128, rotary_dim=128, vocabulary=151936, rope_theta=1.0e6,
+             norm_epsilon=1.0e-6, output_gated=0, qk_norm=0, zero_centered_norm=0,
+             scale_scheme=1, kv_encoding=0, kv_page_tokens=256, draft_depth=4)
+CONTEXT = 32768
+SEED = 20241125
+TAG = "decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2"
+
+
+def provider_with(layers, context=CONTEXT, kv_seed=7):
+    geometry = dict(MODEL, layers=layers, max_context=context + 256)
+    provider = qp.Provider(**geometry)
+    provider.load_synthetic_weights(SEED)
+    if context:
+        provider.prefill_synthetic_kv(context, kv_seed)
+    provider.prepare_exact_decode(TAG)
+    return provider
+
+
+class HostLayerModel(step_oracle.TinyModel):
+    """The first layer of the provider's random-init model as host tensors, a
+    few rows of the embedding and a sample of the head's rows."""
+
+    def __init__(self, provider, tokens, head_rows):
+        H, I, Q, KV, d = (MODEL["hidden"], MODEL["intermediate"], MODEL["query_heads"],
+                          MODEL["kv_heads"], MODEL["head_dim"])
+        self.hidden, self.intermediate, self.layers = H, I, 1
+        self.query_heads, self.kv_heads, self.head_dim = Q, KV, d
+        self.rotary_dim, self.rope_theta, self.eps = d, MODEL["rope_theta"], MODEL["norm_epsilon"]
+        self.scheme, self.output_gated, self.qk_norm, self.zero_centered = 1, False, False, False
+        rows = lambda name, first, count, columns: provider.matrix_rows(  # noqa: E731
+            name, first, count, columns, 1)
+        embedded = [rows("token_embedding", int(t), 1, H) for t in tokens]
+        self.embedding = (np.concatenate([e[0] for e in embedded]),
+                          np.concatenate([e[1] for e in embedded]))
+        ones = np.ones(H, dtype=np.float32)
+        qkv = rows("layer.0.qkv", 0, (Q + 2 * KV) * d, H)
+        cut = lambda pair, a, b: (pair[0][a:b], pair[1][a:b])  # noqa: E731
+        self.blocks = [dict(
+            input_norm=ones, post_attention_norm=ones,
+            query=cut(qkv, 0, Q * d), key=cut(qkv, Q * d, (Q + KV) * d),
+            value=cut(qkv, (Q + KV) * d, (Q + 2 * KV) * d),
+            output=rows("layer.0.output", 0, H, Q * d),
+            gate=rows("layer.0.gate", 0, I, H), up=rows("layer.0.up", 0, I, H),
+            down=rows("layer.0.down", 0, H, I))]
+        self.final_norm = ones
+        sampled = [rows("output_head", int(r), 1, H) for r in head_rows]
+        self.head = (np.concatenate([s[0] for s in sampled]),
+                     np.concatenate([s[1] for s in sampled]))
+        self.vocabulary = len(head_rows)
+
+
+def test_one_layer_of_the_27b_model_at_32k_against_the_composed_oracle(device):
+    """Hidden 5120, 64Q/8KV heads of 128, FFN 17408, vocabulary 151936, 32768
+    cached tokens: every operation of a layer at its benchmark shape, composed,
+    against the CPU oracle on the weights read back from the device."""
+    rng = np.random.default_rng(3)
+    provider = provider_with(1)
+    tokens = rng.integers(0, MODEL["vocabulary"], 5).astype(np.uint32)
+    head_rows = np.sort(rng.choice(MODEL["vocabulary"], 384, replace=False))
+    pages_before = [provider.kv_page(index) for index in range(CONTEXT // 256 + 1)]
+    provider.run_target(tokens, CONTEXT)
+    logits, hidden = provider.logits(5), provider.hidden(5)
+    observed = [provider.kv_page(index) for index in range(CONTEXT // 256 + 1)]
+    model = HostLayerModel(provider, tokens, head_rows)
+    report = {}
+    want_logits, want_hidden = step_oracle.run_target(
+        model, np.arange(5, dtype=np.uint32), CONTEXT, pages_before, 256, observed, report)
+    assert report["record_byte_diffs"] <= 0.03 * report["record_bytes"]
+    relative = np.linalg.norm(hidden - want_hidden) / np.linalg.norm(want_hidden)
+    assert relative < 1e-2, relative
+    assert np.abs(hidden - want_hidden).max() < 0.05 * np.abs(want_hidden).max()
+    sampled = logits[:, head_rows]
+    relative = np.linalg.norm(sampled - want_logits) / np.linalg.norm(want_logits)
+    assert relative < 2e-2, relative
+    provider.close()
+
+
+def test_the_64_layer_verify_step_at_32k(device):
+    rng = np.random.default_rng(5)
+    provider = provider_with(64)
+    V = MODEL["vocabulary"]
+    token, position = int(rng.integers(0, V)), CONTEXT
+    provider.begin_request(temperature_ppm=0)
+    provider.synchronize(token, position)
+    drafts = rng.integers(0, V, 4).astype(np.uint32)
+    rows = np.array([token, *drafts], dtype=np.uint32)
+    # kernel by kernel, then make the first draft the target's own choice
+    provider.run_target(rows, position)
+    drafts[0] = rows[1] = provider.logits(5)[0].argmax()
+    provider.run_target(rows, position)
+    eager_logits, eager_hidden = provider.logits(5), provider.hidden(5)
+    assert np.isfinite(eager_logits).all()
+    # the captured graph: the same bits, replay after replay
+    provider.capture_target(rows, position)
+    for _ in range(2):
+        provider.replay_target()
+        provider.synchronize_stream()
+        assert np.array_equal(provider.logits(5), eager_logits)
+        assert np.array_equal(provider.hidden(5), eager_hidden)
+    # the verify step (graph path) and the oracle's acceptance on its logits
+    provider.set_drafts(drafts)
+    emitted, next_token, advanced = provider.verify(token, position, position + 64)
+    logits = provider.logits(5)
+    assert np.array_equal(logits, eager_logits)
+    accepted, want_next = ol.accept_greedy(logits, drafts)
+    assert accepted >= 1
+    assert advanced == accepted + 1 and next_token == want_next
+    assert emitted == [token, *drafts[:accepted].tolist()]
+    # the head on the GPU's own final hidden state, 512 sampled vocabulary rows
+    sample = np.sort(rng.choice(V, 512, replace=False))
+    codes, scales = zip(*[provider.matrix_rows("output_head", int(r), 1, MODEL["hidden"], 1)
+                          for r in sample])
+    x = ol.rms_norm_rows(eager_hidden, np.ones(MODEL["hidden"], np.float32),
+                         MODEL["norm_epsilon"], False, True)
+    want = ol.fp4_linear_f64(np.concatenate(codes), np.concatenate(scales), 1, len(sample),
+                             MODEL["hidden"], x)
+    gu.assert_close(logits[:, sample], want, what="lm_head after 64 layers")
+    provider.close()
+
+
+def test_lm_head_and_stochastic_acceptance_over_the_whole_vocabulary(device):
+    """Hidden [5, 5120] through the 151936-row head, then min(1, p/q) acceptance
+    with q ~ Dirichlet(0.1) over the whole vocabulary, temperature 0.7, top-p
+    0.95, every candidate ordered on the host (top_k = 0): bit-exact against the
+    oracle on the GPU's logits."""
+    rng = np.random.default_rng(9)
+    provider = provider_with(1, context=1024)
+    V = MODEL["vocabulary"]
+    position, token = 1024, int(rng.integers(0, V))
+    for seed in (11, 12):
+        provider.begin_request(temperature_ppm=700000, top_p_ppm=950000, top_k=0,
+                               min_p_ppm=0, seed=seed)
+        provider.synchronize(token, position)
+        tokens, distributions = [], []
+        for _ in range(4):
+            q = rng.dirichlet(np.full(V, 0.1))
+            q = q / q.sum()
+            tokens.append(int(rng.choice(V, p=q)))
+            distributions.append((np.arange(V, dtype=np.uint32), q))
+        provider.set_drafts(np.array(tokens, dtype=np.uint32), distributions)
+        emitted, following, advanced = provider.verify(token, position, position + 64)
+        logits = provider.logits(5)
+        targets = []
+        for row in range(5):
+            order = np.lexsort((np.arange(V), -logits[row].astype(np.float64)))
+            status, t, p = ol.make_sampling_distribution(
+                logits[row][order], order.astype(np.uint32), 700000, 950000, 0)
+            assert status == 0
+            targets.append((t, p))
+        status, accepted, want_next = ol.accept_stochastic(
+            targets, distributions, tokens, seed, position)
+        assert status == 0
+        assert advanced == accepted + 1 and following == want_next
+        assert emitted == [token, *tokens[:accepted]]
+        token, position = following, position + advanced
+    provider.close()
+
+
+def eight_heads(rng, tokens, d):
+    """K and V for eight KV heads: one head's N(0,1) rows, shifted along the
+    context by a different amount per head."""
+    base_k = rng.standard_normal((tokens, d)).astype(np.float32)
+    base_v = rng.standard_normal((tokens, d)).astype(np.float32)
+    keys = np.stack([np.roll(base_k, 977 * h, axis=0) for h in range(8)], axis=1)
+    values = np.stack([np.roll(base_v, 1361 * h, axis=0) for h in range(8)], axis=1)
+    return keys, values
+
+
+def test_q4h_attention_at_131072_tokens_with_eight_kv_heads(device):
+    rng = np.random.default_rng(131)
+    tokens, rows, Q, KV, d, page = 131072, 5, 64, 8, 128, 256
+    keys, values = eight_heads(rng, tokens, d)
+    pages = synth.q4h_pages(keys, values, page)
+    query = ol.bf16_round(rng.standard_normal((rows, Q, d)).astype(np.float32))
+    first = tokens - 4
+    results = [gu.q4h_attention(device, pages, query, rows, Q, KV, d, first, page, split,
+                                False) for split in (4096, 16384, 0)]
+    for other in results[1:]:
+        assert np.abs(other - results[0]).max() < 2e-5
+    for head in (0, 5):          # one KV head of the same launch against the oracle
+        one = synth.q4h_pages(keys[:, head:head + 1], values[:, head:head + 1], page)
+        shape = ol.AttentionShape(rows, 8, 1, d, first, page, 0, 0)
+        want = ol.attention_q4h(shape, query[:, 8 * head:8 * head + 8], one, "f64")
+        gu.assert_close(results[2][:, 8 * head:8 * head + 8], want,
+                        what=f"131072-token attention, KV head {head}")
+
+
+def test_f16_attention_at_262144_tokens_with_eight_kv_heads(device):
+    rng = np.random.default_rng(262)
+    tokens, rows, Q, KV, d, page = 262144, 5, 64, 8, 128, 256
+    keys, values = eight_heads(rng, tokens, d)
+    pages = synth.f16_pages(keys, values, page)
+    query = rng.standard_normal((rows, Q, d)).astype(np.float32)
+    first = tokens - (rows - 1)
+    results = [gu.f16_attention(device, pages, query, rows, Q, KV, d, first, page, split,
+                                False) for split in (8192, 65536, 0)]
+    for other in results[1:]:
+        assert np.abs(other - results[0]).max() < 2e-5
+    head = 3
+    one = synth.f16_pages(keys[:, head:head + 1], values[:, head:head + 1], page)
+    shape = ol.AttentionShape(rows, 8, 1, d, first, page, 0, 0)
+    want = ol.attention_f16(shape, query[:, 8 * head:8 * head + 8], one, False)
+    gu.assert_close(results[2][:, 8 * head:8 * head + 8], want,
+                    what="262144-token F16 attention, KV head 3")

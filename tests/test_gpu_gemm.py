@@ -44,6 +44,33 @@ def test_gemm_tile_heights(device, scheme, tile_rows, rows, padded, batch):
     gu.assert_close(got, want, what=f"tile height {tile_rows}")
 
 
+@pytest.mark.parametrize("tile_rows", [8, 20, 32])
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_rows_read_back_from_the_tiled_layout(device, scheme, tile_rows):
+    """qllm_fp4_unpack_rows undoes qllm_fp4_prepack for any row range (and is a
+    plain copy for a row-major matrix)."""
+    rng = np.random.default_rng(tile_rows + scheme)
+    rows, padded = 333, 1024
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    plain = qh.fp4_matrix(d_codes, d_scales, rows, padded, padded, scheme)
+    tiled, keep = qh.prepack(plain, device, tile_rows)
+    for matrix in (tiled, plain):
+        for first, count in ((0, rows), (0, 1), (rows - 1, 1), (17, 40), (31, 2), (300, 33)):
+            out_codes = torch.full((count, padded // 2), 0xee, dtype=torch.uint8, device=device)
+            out_scales = torch.full((count, scales.shape[1] * scales.itemsize), 0xee,
+                                    dtype=torch.uint8, device=device)
+            qh.call("qllm_fp4_unpack_rows", matrix, first, count, qh.ptr(out_codes),
+                    qh.ptr(out_scales), None)
+            torch.cuda.synchronize()
+            assert np.array_equal(out_codes.cpu().numpy(), codes[first:first + count])
+            assert np.array_equal(out_scales.cpu().numpy().view(scales.dtype),
+                                  scales[first:first + count])
+    with pytest.raises(qh.QllmError):
+        qh.call("qllm_fp4_unpack_rows", tiled, rows, 1, qh.ptr(d_codes), qh.ptr(d_scales), None)
+    del keep
+
+
 @pytest.mark.parametrize("padded,tiled", [(5120, True), (5120, False), (96, False)])
 def test_split_gemm_equals_separate_calls(device, padded, tiled):
     """q, k and v stored as one matrix: each output segment carries exactly the
