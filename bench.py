@@ -384,7 +384,7 @@ def main():
             ("lm_head", fp4_bytes(vocabulary, H) + rows * H * 2 + rows * vocabulary * 4),
             ("attention", CONTEXT * MODEL["kv_heads"] * 2 * (MODEL["head_dim"] // 2 + 2)
              + 2 * rows * MODEL["query_heads"] * MODEL["head_dim"] * 2)):
-        us, _ = provider.time_kernel(name, 4, CONTEXT)
+        us, _ = provider.time_kernel(name, 16 if name == "lm_head" else 4, CONTEXT)
         other_kernels[name] = {"avg_launch_us": round(us, 3),
                                "achieved_GBps": round(bytes_per_launch / us / 1e3, 1),
                                "frac": round(bytes_per_launch / us / 1e3 / HBM_PEAK_GBS, 4)}
@@ -450,7 +450,10 @@ def main():
             "step_roofline_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 /
                                         HBM_PEAK_GBS, 4),
             "reference_published_tok_s_rtx3090": 54.54,
-            "projected_tok_s_at_reference_acceptance_2.6667": round(
+            # the verify step alone: no proposer passes in the timed region (the
+            # decode cycle below has them and carries the projection that can be
+            # set next to the reference's end-to-end figure)
+            "verify_only_projected_tok_s_at_reference_acceptance_2.6667": round(
                 2.6667 * 1000.0 / ms_per_step, 1),
         },
         "roofline": roofline,

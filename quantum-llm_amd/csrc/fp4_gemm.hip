@@ -7,14 +7,21 @@
 // Two kernels:
 //  * fp4_gemm_mfma_kernel  - the hot path.  At M=5 a verify step needs
 //    16 flop per weight byte; at HBM speed that is ~130 TFLOP/s, above what
-//    the vector ALUs deliver, so the contraction runs on the matrix cores
-//    (v_mfma_f32_32x32x16_bf16) with the batch as the 32-wide M side (rows
-//    >= batch are don't-care) and 32 weight rows as the N side.  Packed
-//    nibbles stream from HBM with one 16-byte load per lane, are expanded in
-//    registers by v_cvt_scalef32_pk_bf16_fp4 (exact), and activations are
-//    staged once per workgroup in LDS in MFMA fragment order.
-//  * fp4_gemv_generic_kernel - any shape/scheme/activation type, one wave per
-//    output row; used for shapes the MFMA kernel does not take.
+//    the vector ALUs deliver, so the contraction runs on the matrix cores,
+//    on v_mfma_f32_16x16x32_bf16: 16 weight rows on the N side, 32 columns of
+//    K - two 16-blocks with scales of their own - which are kept apart on the
+//    M side (MFMA rows 0..7 carry the batch for the first block, rows 8..15
+//    for the second), so that each block sum is scaled by its own scale before
+//    the halves are added.  Packed nibbles stream from HBM with one 16-byte
+//    load per lane (one contiguous KiB per wave in the tiled layout), are
+//    expanded in registers by v_cvt_scalef32_pk_bf16_fp4 (exact), and the
+//    activations of a chunk ride along through a wave-private LDS ring; a
+//    workgroup's waves interleave over the 64-column chunks of K and meet in
+//    LDS once, after the loop.
+//  * fp4_gemv_generic_kernel - any shape/scheme/activation type (the Q8
+//    integer form of the reference included), one wave per output row; used
+//    for shapes the MFMA kernel does not take.  The provider never selects it
+//    for a K that is a multiple of 64.
 #include "common.hpp"
 
 #include <cstdlib>

@@ -1597,7 +1597,13 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
         std::size_t{g_.query_heads} * g_.head_dim * (g_.output_gated ? 2U : 1U);
     const std::size_t kv_width = std::size_t{g_.kv_heads} * g_.head_dim;
     const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
-    const bool feed_proposer = state && mtp_.ready;
+    // a request that will not be decoded speculatively keeps the proposer out
+    // (the runner synchronises only exact-eligible requests,
+    // runtime/tools/moe_vm_runner.cpp:735-745)
+    const auto exact_enabled = request.parameters.find("exact_decode_enabled");
+    const bool feed_proposer =
+        state && mtp_.ready &&
+        (exact_enabled == request.parameters.end() || exact_enabled->second != 0U);
     // query rows per attention workgroup: as many as the kernels' three (two at
     // head_dim 256) 16-row tiles hold for one KV head's group of query heads
     const std::uint32_t attention_batch = std::max(
@@ -1766,10 +1772,16 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
                                    select_workspace_, select_workspace_bytes_,
                                    stream));
     std::uint32_t predicted{};
-    hip_check(hipMemcpyAsync(&predicted, argmax_tokens_, sizeof(predicted),
-                             hipMemcpyDeviceToHost, hip_stream),
-              "copy the prompt's prediction");
-    hip_check(hipStreamSynchronize(hip_stream), "prompt prefill");
+    if (request.parameters.contains("sampling_temperature_ppm")) {
+      // the head under the request's sampling profile, at the position of the
+      // prompt's last token (run_head with a request, :8433-8517)
+      predicted = select_head_token(request, first_position + count - 1U);
+    } else {
+      hip_check(hipMemcpyAsync(&predicted, argmax_tokens_, sizeof(predicted),
+                               hipMemcpyDeviceToHost, hip_stream),
+                "copy the prompt's prediction");
+      hip_check(hipStreamSynchronize(hip_stream), "prompt prefill");
+    }
     prefill_tokens_total_ += count;
     if (state) {
       state->synchronized_token = predicted;
@@ -2007,23 +2019,66 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
         throw std::runtime_error("unknown kernel name: " + which);
       }
     };
-    const std::uint32_t per_round = which == "lm_head" ? 1U : g_.layers;
-    for (std::uint32_t index = 0; index < per_round; ++index) launch_one(index);
     hipEvent_t begin{};
     hipEvent_t end{};
     hip_check(hipEventCreate(&begin), "create timing event");
     hip_check(hipEventCreate(&end), "create timing event");
-    hip_check(hipEventRecord(begin, stream), "record timing event");
-    for (std::uint32_t round = 0; round < rounds; ++round)
+    const auto timed = [&](const auto& body) {
+      hip_check(hipEventRecord(begin, stream), "record timing event");
+      body();
+      hip_check(hipEventRecord(end, stream), "record timing event");
+      hip_check(hipEventSynchronize(end), "wait for timing event");
+      float milliseconds{};
+      hip_check(hipEventElapsedTime(&milliseconds, begin, end), "read timing");
+      return static_cast<double>(milliseconds);
+    };
+    if (which == "lm_head") {
+      // There is one head, and it nearly fits the last-level cache: launched
+      // back to back it would be timed on cached weights.  Every timed launch
+      // therefore follows the gate/up launches of several layers - more than
+      // twice the cache's size of other weights, as in a step - and the time of
+      // those launches alone is taken off.
+      const std::uint64_t filler_bytes =
+          2U * qllm_fp4_packed_weight_bytes(g_.intermediate, pad32(g_.hidden), 0U);
+      const std::uint32_t fillers = std::min<std::uint32_t>(
+          g_.layers, static_cast<std::uint32_t>(
+                         (std::uint64_t{640} << 20U) / std::max<std::uint64_t>(
+                                                           filler_bytes, 1U) + 1U));
+      const auto filler = [&](std::uint32_t round) {
+        for (std::uint32_t index = 0; index < fillers; ++index) {
+          const auto& layer = layers_[(round * fillers + index) % g_.layers];
+          status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
+                                            &layer.up.descriptor, normalized_,
+                                            hidden_bytes, activation_, rows,
+                                            stream_));
+        }
+      };
+      filler(0U);
+      launch_one(0U);
+      const double with_head = timed([&] {
+        for (std::uint32_t round = 0; round < rounds; ++round) {
+          filler(round);
+          launch_one(0U);
+        }
+      });
+      const double without = timed([&] {
+        for (std::uint32_t round = 0; round < rounds; ++round) filler(round);
+      });
+      *launches = rounds;
+      *microseconds = 1000.0 * (with_head - without) / static_cast<double>(rounds);
+    } else {
+      const std::uint32_t per_round = g_.layers;
       for (std::uint32_t index = 0; index < per_round; ++index) launch_one(index);
-    hip_check(hipEventRecord(end, stream), "record timing event");
-    hip_check(hipEventSynchronize(end), "wait for timing event");
-    float milliseconds{};
-    hip_check(hipEventElapsedTime(&milliseconds, begin, end), "read timing");
+      const double milliseconds = timed([&] {
+        for (std::uint32_t round = 0; round < rounds; ++round)
+          for (std::uint32_t index = 0; index < per_round; ++index)
+            launch_one(index);
+      });
+      *launches = std::uint64_t{rounds} * per_round;
+      *microseconds = 1000.0 * milliseconds / static_cast<double>(*launches);
+    }
     (void)hipEventDestroy(begin);
     (void)hipEventDestroy(end);
-    *launches = std::uint64_t{rounds} * per_round;
-    *microseconds = 1000.0 * milliseconds / static_cast<double>(*launches);
     return er::Status::success();
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};

@@ -193,7 +193,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   // Average duration, in microseconds, of one launch of a hot kernel measured
   // with HIP events on the provider's stream: the kernel is launched once per
   // layer (distinct weights / KV each time) for `rounds` passes over the
-  // layers.  which: "ffn_gate_up", "ffn_down", "qkv", "attention_output",
+  // layers; the head, of which there is one, is timed on weights that other
+  // launches have pushed out of the last-level cache.  which: "ffn_gate_up", "ffn_down", "qkv", "attention_output",
   // "attention", "lm_head".
   [[nodiscard]] er::Status time_kernel(const std::string& which,
                                        std::uint32_t rounds,
@@ -215,8 +216,10 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   // Prompt prefill: runs `tokens` (positions first_position ..) through the
   // target in chunks of up to prefill_chunk_rows() rows - the linears on the
   // tall-batch GEMM, attention and the K/V store in row batches of the verify
-  // step's size - and returns the greedy prediction for the position after
-  // the prompt.  With a request state the proposer is fed the prompt as the
+  // step's size - and returns the head's token for the position after the
+  // prompt: selected under the request's sampling profile when the request
+  // carries one, the arg-max otherwise.  With a request state (and unless the
+  // request says exact_decode_enabled = 0) the proposer is fed the prompt as the
   // worker's feed does through synchronize_exact_decode_batch
   // (runtime/tools/moe_vm_runner.cpp:682-745), and the first drafts are rolled
   // out: the state is then ready for execute_exact_decode at

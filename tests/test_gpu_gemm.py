@@ -216,6 +216,37 @@ def test_q8_gemv_matches_reference_integer_statement(device):
     assert np.abs(out.cpu().numpy() - want).max() < 2e-4
 
 
+@pytest.mark.parametrize("rows,columns,batch", [(17408, 5120, 5), (1000, 5100, 8),
+                                                (64, 33, 1)])
+def test_q8_gemv_at_model_shapes_and_ragged_k(device, rows, columns, batch):
+    """The Q8-activation form (the reference's default arithmetic: integer
+    block sums, one F32 scale FMA per 32-block) at the SwiGLU projection's
+    shape and with a K that is not a multiple of the block: against the integer
+    statement of the oracle, 2e-4 as the reference's own gate."""
+    rng = np.random.default_rng(rows + columns)
+    padded = (columns + 31) // 32 * 32
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    x = rng.standard_normal((batch, columns)).astype(np.float32)
+    want_q8, want_scales = ol.quantize_q8_rows(x, padded)
+    d_x = gu.device_tensor(x, device)
+    d_q8 = torch.zeros((batch, padded), dtype=torch.int8, device=device)
+    d_s = torch.zeros(batch, device=device)
+    qh.call("qllm_quantize_q8_batch", qh.ptr(d_x), qh.ptr(d_q8), qh.ptr(d_s), batch,
+            columns, padded, 0, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_q8.cpu().numpy(), want_q8)
+    assert not want_q8[:, columns:].any()                       # padding quantises to 0
+    want = ol.fp4_linear_block32_q8(codes, scales, rows, padded, want_q8, want_scales)
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    out = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemv_q8_batch",
+            qh.fp4_matrix(d_codes, d_scales, rows, columns, padded, 0), qh.ptr(d_q8),
+            qh.ptr(d_s), qh.ptr(out), batch, 0, None)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.abs(got - want).max() <= 2e-4 * max(1.0, np.abs(want).max())
+
+
 def test_invalid_arguments_are_rejected(device):
     with pytest.raises(qh.QllmError) as error:
         qh.call("qllm_fp4_gemm_bf16", qh.fp4_matrix(None, None, 4, 4, 32, 0), None, 0,
