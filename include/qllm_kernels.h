@@ -328,6 +328,33 @@ int32_t qllm_qkv_rope_cache_paged_q4h_from_partials(
     uint32_t rotary_dim, float epsilon, float rope_theta,
     int32_t bf16_activations, void* stream);
 
+/* The same operation (partials may be NULL: query, key and value then hold the
+ * projection already), which also leaves the rotated queries as the operands
+ * of qllm_attention_paged_q4h: per KV head and 16-row tile of its rows *
+ * (query_heads / kv_heads) matrix rows (row r, head h of the group at r *
+ * group + h) and per 64 elements of head_dim, a high and a low int8 plane of
+ * 1 KiB in matrix-core order, query = scale * (128 * high + low) to 15 bits of
+ * the row's largest magnitude; query_operand_scales holds 16 floats per row
+ * tile and KV head, the scale times log2(e) / (16 sqrt(head_dim)).
+ * query_operands: qllm_q4h_query_operand_bytes() bytes, 16-byte aligned; rows
+ * of a tile past the batch are left untouched.  head_dim in {128, 256},
+ * rows * (query_heads / kv_heads) <= 48 (32 at head_dim 256).  The reference
+ * quantises its queries in a kernel of its own
+ * (quantize_gqa_queries_q8_kernel, transformer_kernels.cu:4391-4416). */
+size_t qllm_q4h_query_operand_bytes(uint32_t rows, uint32_t query_heads,
+                                    uint32_t kv_heads, uint32_t head_dim);
+int32_t qllm_qkv_rope_cache_paged_q4h_prepared(
+    const float* partials, uint32_t partial_count, float* query,
+    uint32_t query_stride, float* key, float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, const uint32_t* device_positions,
+    uint32_t rows, uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, int8_t* query_operands,
+    float* query_operand_scales, void* stream);
+
 /* The same per-head RMSNorm + rotary without the K/V store, for caches that
  * store K/V separately.  replaces gated_gqa_qkv_rope_fp16_batch
  * (runtime/src/cuda/transformer_kernels.cu:3645-3726). */
@@ -373,10 +400,13 @@ int32_t qllm_quantize_gqa_queries_q8(const float* query,
  * for gated_gqa_attention_microbatch_paged_q4_per_head_tensor_core. */
 typedef struct qllm_q4h_attention_launch {
   const float* query;           /* [rows, query_heads, query_stride], 16-byte
-                                   aligned; the kernel quantises it itself */
-  const int8_t* q8_queries;     /* accepted for layout parity with the
-                                   reference struct; may be NULL, unused */
-  const float* query_scales;    /* as above */
+                                   aligned; the kernel quantises it itself
+                                   unless the next two fields are set */
+  const int8_t* q8_queries;     /* NULL, or the query operands that
+                                   qllm_qkv_rope_cache_paged_q4h_prepared left
+                                   for these rows (two int8 planes, not the
+                                   reference's single Q8 plane) */
+  const float* query_scales;    /* NULL, or the operand scales of the same call */
   const void* const* page_table;
   void* output;                 /* [rows, query_heads, head_dim] */
   float* partial_maxima;        /* [rows, maximum_splits, query_heads] */

@@ -61,8 +61,27 @@ __device__ __forceinline__ Q4hPlanes q4h_planes(const void* page,
   return planes;
 }
 
+// Prepared query operands of one KV head: for every 16-row tile of its
+// rows * group matrix rows and every 64-wide k-step of head_dim a high and a
+// low int8 plane of 1 KiB in matrix-core operand order (lane (col, quad) owns
+// bytes [16 * (16 * quad + col), +16) of a plane), q = scale * (128 * high +
+// low); the scales, already multiplied by log2(e) / (16 sqrt(head_dim)), are
+// a separate array of 16 floats per row tile.
+__host__ __device__ inline uint32_t q4h_row_tiles(uint32_t rows, uint32_t group) {
+  return (rows * group + 15u) / 16u;
+}
+__host__ __device__ inline size_t q4h_operand_plane_bytes(uint32_t row_tiles,
+                                                          uint32_t head_dim) {
+  return static_cast<size_t>(row_tiles) * (head_dim / 64u) * 2u * 1024u;
+}
+
 struct SplitArgs {
   const float* query;
+  // Optional: the query operands as qkv_rope_q4h_kernel prepares them (see
+  // q4h_query_operand_bytes); the kernel then copies them instead of
+  // quantising `query`.
+  const uint8_t* query_operands;
+  const float* query_operand_scales;
   uint32_t query_stride;
   const void* const* page_table;
   float* partial_maxima;
@@ -339,13 +358,40 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // so the integer scores carry the query to ~3e-5 relative instead of the
   // 4e-3 of a single Q8 plane.  The operands are published in MFMA order.
   static_assert(RT * KSTEPS <= kSplitWaves, "one wave per operand pair");
-  // the wave's first tile sets out before anything else: its flight time covers
-  // the query work below
+  if (args.query_operands) {
+    // prepared by the rotary kernel: the planes go straight to LDS, one KiB
+    // per wave and load, the scales with them
+    constexpr uint32_t kPlanes = RT * KSTEPS * 2;
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t exchange_lds =
+        __builtin_amdgcn_readfirstlane(lds_address(exchange));
+    const uint8_t* planes = uniform_pointer(
+        args.query_operands + static_cast<size_t>(kv_head) * kPlanes * 1024u);
+#pragma unroll
+    for (uint32_t plane = 0; plane < (kPlanes + kSplitWaves - 1u) / kSplitWaves;
+         ++plane) {
+      const uint32_t index = plane * kSplitWaves + wave;
+      if (index < kPlanes)
+        copy16_to_lds(planes + index * 1024u, lane_now * 16u,
+                      exchange_lds + index * 1024u);
+    }
+    if (wave == kSplitWaves - 1u && lane_now < RT * 16u) {
+      const uint8_t* scales = uniform_pointer(reinterpret_cast<const uint8_t*>(
+          args.query_operand_scales + static_cast<size_t>(kv_head) * RT * 16u));
+      copy4_to_lds(scales, lane_now * 4u, exchange_lds + kPlanes * 1024u);
+      const uint32_t row = lane_now < matrix_rows ? lane_now / group : 0u;
+      exchange_limit[lane_now] = first_context_tokens + row;
+    }
+  }
+  // the wave's first tile sets out before the query work below, which its
+  // flight time covers
   if (tile_first < tile_last) {
     stage_keys(tile_first);
     stage_values(tile_first);
   }
-  if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
+  if (args.query_operands) {
+    vmem_wait<0>();
+  } else if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
     // wave u builds k-step u % KSTEPS of row tile u / KSTEPS (the row's scale
     // needs the whole row, so every such wave reads all of it)
     const uint32_t rt = wave / KSTEPS;
@@ -725,12 +771,50 @@ __global__ void attention_combine_kernel(
   // The first kCombinePrefetch partial outputs are fetched before anything
   // depends on them, so that they travel together with the maxima and sums.
   constexpr uint32_t kCombinePrefetch = 32;
-  const float* source = partial_outputs + first_partial * head_dim + dimension;
-  const size_t stride = static_cast<size_t>(query_heads) * head_dim;
+  // (wave-uniform row address + the thread's dimension: the address arithmetic
+  // stays on the scalar unit and no load waits for another)
+  const float* partial_rows = partial_outputs + first_partial * head_dim;
+  const uint32_t stride = query_heads * head_dim;
+  const float* source = partial_rows + dimension;
   float fetched[kCombinePrefetch];
 #pragma unroll
-  for (uint32_t split = 0; split < kCombinePrefetch; ++split)
-    fetched[split] = split < active ? source[split * stride] : 0.0f;
+  for (uint32_t split = 0; split < kCombinePrefetch; ++split) {
+    // past the last split: that split once more (finite), weighted by zero
+    const float* row_of_split =
+        partial_rows + static_cast<size_t>(min(split, active - 1u)) * stride;
+    fetched[split] = row_of_split[dimension];
+  }
+  const size_t record = static_cast<size_t>(row) * query_heads + head;
+  if (active <= kCombinePrefetch) {
+    // Few splits: every wave takes one split per lane, so maximum, weights and
+    // their sum come from lane exchanges alone and everything the result needs
+    // is requested in one round trip.
+    const uint32_t lane = threadIdx.x & 63u;
+    const size_t partial = first_partial + static_cast<size_t>(lane) * query_heads;
+    const float split_max = lane < active ? partial_maxima[partial] : kMaskedMax;
+    const float split_sum = lane < active ? partial_sums[partial] : 0.0f;
+    float gate = 0.0f;
+    if (output_gated) gate = query[record * query_stride + head_dim + dimension];
+    const float maximum = wave_max(split_max);
+    const float weight = __builtin_amdgcn_exp2f(split_max - maximum);
+    const float sum = wave_sum(split_sum * weight);
+    float result = 0.0f;
+#pragma unroll
+    for (uint32_t split = 0; split < kCombinePrefetch; ++split)
+      result = fmaf(fetched[split],
+                    __uint_as_float(__builtin_amdgcn_readlane(
+                        __float_as_uint(weight), split)),
+                    result);
+    result /= sum;
+    if (output_gated) result *= 1.0f / (1.0f + expf(-gate));
+    const size_t index = record * head_dim + dimension;
+    if (output_kind == QLLM_OUT_BF16)
+      static_cast<uint16_t*>(output)[index] =
+          static_cast<uint16_t>(f32_to_bf16_bits(result));
+    else
+      static_cast<float*>(output)[index] = result;
+    return;
+  }
   float local_max = kMaskedMax;
   for (uint32_t split = threadIdx.x; split < active; split += blockDim.x)
     local_max = fmaxf(local_max,
@@ -751,9 +835,8 @@ __global__ void attention_combine_kernel(
   for (uint32_t split = 0; split < kCombinePrefetch; ++split)
     if (split < active) result = fmaf(fetched[split], weights[split], result);
   for (uint32_t split = kCombinePrefetch; split < active; ++split)
-    result = fmaf(source[split * stride], weights[split], result);
+    result = fmaf(source[static_cast<size_t>(split) * stride], weights[split], result);
   result /= sum;
-  const size_t record = static_cast<size_t>(row) * query_heads + head;
   if (output_gated) {
     const float gate = query[record * query_stride + head_dim + dimension];
     result *= 1.0f / (1.0f + expf(-gate));
@@ -876,7 +959,8 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
     uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations,
     const uint32_t* device_positions, const float* partials,
-    uint32_t partial_count, uint32_t rows) {
+    uint32_t partial_count, uint32_t rows, uint8_t* operands,
+    float* operand_scales) {
   __shared__ float shared[256];
   __shared__ float rotated[256];
   if (device_positions) {
@@ -927,6 +1011,47 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
         query + (static_cast<size_t>(row) * query_heads + head) * query_stride;
     head_norm_rope(q, q_weight, head_dim, rotary_dim, rotary_position, epsilon,
                    theta, bf16_activations, shared, rotated, lane);
+    if (!operands) return;
+    // The attention kernel's query operands (same arithmetic as its own
+    // quantisation): 15 bits against the row's largest magnitude, split into
+    // a high and a low int8 plane, each byte dropped where the matrix core
+    // wants it.  Element d of the row belongs to k-step h = 2 (d / 128) +
+    // (d % 32) / 16, lane quad (d % 128) / 32, and inside the lane's 16 bytes
+    // to slot (j < 8: even j first, then odd j; likewise for j >= 8), j = d % 16.
+    const uint32_t group = query_heads / kv_heads;
+    const uint32_t matrix_row = row * group + head % group;
+    const uint32_t row_tile = matrix_row / 16u;
+    const uint32_t column = matrix_row % 16u;
+    const uint32_t k_steps = head_dim / 64u;
+    const uint32_t row_tiles = q4h_row_tiles(rows, group);
+    float maximum = 0.0f;
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      maximum = fmaxf(maximum, fabsf(rotated[index]));
+    maximum = wave_max(maximum);
+    const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
+    const float inverse = 1.0f / scale;
+    uint8_t* planes = operands + (head / group) *
+                                     q4h_operand_plane_bytes(row_tiles, head_dim);
+    for (uint32_t index = lane; index < head_dim; index += 64u) {
+      int quantized = __float2int_rn(rotated[index] * inverse);
+      quantized = max(-16319, min(16319, quantized));
+      const int high = (quantized + 64) >> 7;  // floor((v + 64) / 128)
+      const int low = quantized - (high << 7);
+      const uint32_t within = index % 128u;
+      const uint32_t step = 2u * (index / 128u) + (within % 32u) / 16u;
+      const uint32_t quad = within / 32u;
+      const uint32_t j = index % 16u;
+      const uint32_t slot = (j & 8u) + ((j & 1u) << 2) + ((j & 7u) >> 1);
+      uint8_t* piece = planes +
+                       static_cast<size_t>(row_tile * k_steps + step) * 2048u +
+                       (16u * quad + column) * 16u + slot;
+      piece[0] = static_cast<uint8_t>(high);
+      piece[1024] = static_cast<uint8_t>(low);
+    }
+    if (lane == 0u)
+      operand_scales[(head / group) * row_tiles * 16u + matrix_row] =
+          scale * (1.4426950408889634f /
+                   (16.0f * sqrtf(static_cast<float>(head_dim))));
     return;
   }
   const uint32_t head = blockIdx.x - query_heads;
@@ -1063,7 +1188,8 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
-      epsilon, rope_theta, bf16_activations != 0, nullptr, nullptr, 0u, rows);
+      epsilon, rope_theta, bf16_activations != 0, nullptr, nullptr, 0u, rows,
+      nullptr, nullptr);
   return launched("Q4H QKV rope cache batch");
 }
 
@@ -1088,7 +1214,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, 0u, 0u, query_heads, kv_heads,
       head_dim, rotary_dim, epsilon, rope_theta, bf16_activations != 0,
-      device_positions, nullptr, 0u, rows);
+      device_positions, nullptr, 0u, rows, nullptr, nullptr);
   return launched("deferred Q4H QKV rope cache batch");
 }
 
@@ -1119,8 +1245,60 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_from_partials(
       full_attention_layer, page_tokens, first_cache_position,
       first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
       epsilon, rope_theta, bf16_activations != 0, device_positions, partials,
-      partial_count, rows);
+      partial_count, rows, nullptr, nullptr);
   return launched("Q4H QKV rope cache batch from partials");
+}
+
+extern "C" size_t qllm_q4h_query_operand_bytes(uint32_t rows,
+                                               uint32_t query_heads,
+                                               uint32_t kv_heads,
+                                               uint32_t head_dim) {
+  if (!rows || !kv_heads || !query_heads || query_heads % kv_heads ||
+      (head_dim != 128u && head_dim != 256u))
+    return 0;
+  return kv_heads *
+         q4h_operand_plane_bytes(q4h_row_tiles(rows, query_heads / kv_heads),
+                                 head_dim);
+}
+
+extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_prepared(
+    const float* partials, uint32_t partial_count, float* query,
+    uint32_t query_stride, float* key, float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, uint32_t full_attention_layer,
+    uint32_t page_tokens, uint32_t first_cache_position,
+    uint32_t first_rotary_position, const uint32_t* device_positions,
+    uint32_t rows, uint32_t query_heads, uint32_t kv_heads, uint32_t head_dim,
+    uint32_t rotary_dim, float epsilon, float rope_theta,
+    int32_t bf16_activations, int8_t* query_operands,
+    float* query_operand_scales, void* stream) {
+  if ((partials && (!partial_count || partial_count > 16u)) || !query || !key ||
+      !value || !page_table || !page_tokens || !rows || !query_heads ||
+      !kv_heads || query_heads < kv_heads || query_heads % kv_heads ||
+      (head_dim != 128u && head_dim != 256u) || query_stride < head_dim ||
+      !rotary_dim || rotary_dim > head_dim || rotary_dim % 2u ||
+      !(epsilon > 0.0f) || !(rope_theta > 0.0f) || !query_operands ||
+      !query_operand_scales ||
+      (reinterpret_cast<uintptr_t>(query_operands) & 15u) ||
+      (!device_positions &&
+       (first_cache_position > 0xffffffffu - (rows - 1u) ||
+        first_rotary_position > 0xffffffffu - (rows - 1u))))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "invalid Q4H QKV rope cache batch with query operands");
+  const uint32_t row_tiles = q4h_row_tiles(rows, query_heads / kv_heads);
+  if (row_tiles > 3u || (head_dim == 256u && row_tiles > 2u))
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q4H query operands: rows * (query_heads/kv_heads) exceeds 48 "
+                "(32 at head_dim 256)");
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+                        as_stream(stream)>>>(
+      query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
+      full_attention_layer, page_tokens, first_cache_position,
+      first_rotary_position, query_heads, kv_heads, head_dim, rotary_dim,
+      epsilon, rope_theta, bf16_activations != 0, device_positions, partials,
+      partials ? partial_count : 0u, rows,
+      reinterpret_cast<uint8_t*>(query_operands), query_operand_scales);
+  return launched("Q4H QKV rope cache batch with query operands");
 }
 
 extern "C" int32_t qllm_qkv_rope_batch(
@@ -1141,7 +1319,7 @@ extern "C" int32_t qllm_qkv_rope_batch(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
       rotary_dim, epsilon, rope_theta, bf16_activations != 0, nullptr, nullptr,
-      0u, rows);
+      0u, rows, nullptr, nullptr);
   return launched("QKV rope batch");
 }
 
@@ -1161,7 +1339,8 @@ extern "C" int32_t qllm_qkv_rope_batch_deferred(
                         as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, 0u, query_heads, kv_heads, head_dim, rotary_dim, epsilon,
-      rope_theta, bf16_activations != 0, device_positions, nullptr, 0u, rows);
+      rope_theta, bf16_activations != 0, device_positions, nullptr, 0u, rows,
+      nullptr, nullptr);
   return launched("deferred QKV rope batch");
 }
 
@@ -1283,6 +1462,13 @@ extern "C" int32_t qllm_attention_paged_q4h(
                 "maximum_splits");
   SplitArgs args{};
   args.query = launch->query;
+  if (launch->q8_queries && launch->query_scales) {
+    if (reinterpret_cast<uintptr_t>(launch->q8_queries) & 15u)
+      return fail(QLLM_INVALID_ARGUMENT,
+                  "Q4H paged attention: query operands must be 16-byte aligned");
+    args.query_operands = reinterpret_cast<const uint8_t*>(launch->q8_queries);
+    args.query_operand_scales = launch->query_scales;
+  }
   args.query_stride = launch->query_stride;
   args.page_table = launch->page_table;
   args.partial_maxima = launch->partial_maxima;

@@ -346,6 +346,20 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   partial_sums_ = static_cast<float*>(device_alloc(partials * 4U));
   partial_outputs_ =
       static_cast<float*>(device_alloc(partials * g_.head_dim * 4U));
+  if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
+    // The rotary kernel hands the attention kernel its query operands (two
+    // int8 planes in matrix-core order and the row scales).  Rows past the
+    // batch are never written: they stay zero.
+    const std::size_t operand_bytes = qllm_q4h_query_operand_bytes(
+        max_rows_, g_.query_heads, g_.kv_heads, g_.head_dim);
+    const std::size_t scale_bytes = std::size_t{g_.kv_heads} * 3U * 16U * 4U;
+    query_operands_ = static_cast<std::int8_t*>(device_alloc(operand_bytes));
+    query_operand_scales_ = static_cast<float*>(device_alloc(scale_bytes));
+    hip_check(hipMemset(query_operands_, 0, operand_bytes),
+              "clear query operands");
+    hip_check(hipMemset(query_operand_scales_, 0, scale_bytes),
+              "clear query operand scales");
+  }
 
   select_workspace_bytes_ = std::max(
       qllm_argmax_workspace_bytes(g_.vocabulary, max_rows_),
@@ -1223,31 +1237,20 @@ void Mi355DenseFp4Provider::enqueue_attention(
   const auto& layer = layers_[index];
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-    if (qkv_partials)
-      status_check(qllm_qkv_rope_cache_paged_q4h_from_partials(
-          qkv_partials, qkv_partial_count, query, query_stride, key, value,
-          layer.query_norm, layer.key_norm,
-          const_cast<const void* const*>(device_page_table_), index,
-          g_.kv_page_tokens, first_position, first_position,
-          deferred_positions ? positions_ : nullptr, rows, g_.query_heads,
-          g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
-          g_.rope_theta, 0, stream));
-    else if (deferred_positions)
-      status_check(qllm_qkv_rope_cache_paged_q4h_batch_deferred(
-          query, query_stride, key, value, layer.query_norm,
-          layer.key_norm, const_cast<const void* const*>(device_page_table_),
-          index, g_.kv_page_tokens, positions_, rows, g_.query_heads,
-          g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
-          g_.rope_theta, 0, stream));
-    else
-      status_check(qllm_qkv_rope_cache_paged_q4h_batch(
-          query, query_stride, key, value, layer.query_norm,
-          layer.key_norm, const_cast<const void* const*>(device_page_table_),
-          index, g_.kv_page_tokens, first_position, first_position, rows,
-          g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
-          g_.norm_epsilon, g_.rope_theta, 0, stream));
+    // rotary + K/V store; the queries also leave as the attention kernel's
+    // int8 operands, so that it starts on its tiles at once
+    status_check(qllm_qkv_rope_cache_paged_q4h_prepared(
+        qkv_partials, qkv_partial_count, query, query_stride, key, value,
+        layer.query_norm, layer.key_norm,
+        const_cast<const void* const*>(device_page_table_), index,
+        g_.kv_page_tokens, first_position, first_position,
+        deferred_positions ? positions_ : nullptr, rows, g_.query_heads,
+        g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
+        g_.rope_theta, 0, query_operands_, query_operand_scales_, stream));
     qllm_q4h_attention_launch launch{};
     launch.query = query;
+    launch.q8_queries = query_operands_;
+    launch.query_scales = query_operand_scales_;
     launch.page_table = const_cast<const void* const*>(device_page_table_);
     launch.output = attention_out;
     launch.partial_maxima = partial_maxima_;
@@ -1917,6 +1920,16 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
       if (!context_tokens || context_tokens + rows > g_.max_context)
         return {er::ErrorCode::invalid_argument, "timing context is invalid"};
       ensure_pages(context_tokens + rows - 1U);
+      // the attention launches read the query operands a rotary launch leaves
+      if (g_.kv_encoding == KvEncoding::q4_f16_per_head)
+        status_check(qllm_qkv_rope_cache_paged_q4h_prepared(
+            nullptr, 0U, query_, query_stride, key_, value_,
+            layers_[0].query_norm, layers_[0].key_norm,
+            const_cast<const void* const*>(device_page_table_), 0U,
+            g_.kv_page_tokens, context_tokens, context_tokens, nullptr, rows,
+            g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
+            g_.norm_epsilon, g_.rope_theta, 0, query_operands_,
+            query_operand_scales_, stream_));
     }
     const auto launch_one = [&](std::uint32_t index) {
       const auto& layer = layers_[index % g_.layers];
@@ -1996,6 +2009,8 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
       } else if (which == "attention") {
         qllm_q4h_attention_launch launch{};
         launch.query = query_;
+        launch.q8_queries = query_operands_;   // as the target pass launches it
+        launch.query_scales = query_operand_scales_;
         launch.page_table = const_cast<const void* const*>(device_page_table_);
         launch.output = attention_;
         launch.partial_maxima = partial_maxima_;

@@ -380,6 +380,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* partial_maxima_{};
   float* partial_sums_{};
   float* partial_outputs_{};
+  std::int8_t* query_operands_{};       // Q4H attention operands of a batch
+  float* query_operand_scales_{};
   // Pinned host words for the small per-pass transfers: 8 tokens + 4
   // position words up (target pass, proposer pass), 8 chosen tokens down.
   struct HostStaging {

@@ -236,3 +236,92 @@ def test_attention_at_131072_tokens_on_one_kv_head(device):
     gu.assert_close(results[0], want, what="131072-token attention")
     # the rows are causal among themselves: each sees one token more
     assert all(np.abs(results[0][r] - results[0][r + 1]).max() > 0 for r in range(rows - 1))
+
+
+def unpack_query_operands(planes, scales, rows, Q, KV, d):
+    """The prepared operands of qllm_qkv_rope_cache_paged_q4h_prepared back as
+    (high, low) int8 [rows, Q, d] and the scale per (row, head)."""
+    group = Q // KV
+    row_tiles = (rows * group + 15) // 16
+    steps = d // 64
+    planes = planes.reshape(KV, row_tiles, steps, 2, 64, 16).view(np.int8)
+    scales = scales.reshape(KV, row_tiles * 16)
+    high = np.zeros((rows, Q, d), dtype=np.int8)
+    low = np.zeros_like(high)
+    scale = np.zeros((rows, Q), dtype=np.float32)
+    for row in range(rows):
+        for head in range(Q):
+            kv, m = head // group, row * group + head % group
+            scale[row, head] = scales[kv, m]
+            for index in range(d):
+                within, j = index % 128, index % 16
+                step = 2 * (index // 128) + (within % 32) // 16
+                lane = 16 * (within // 32) + m % 16
+                slot = (j & 8) + ((j & 1) << 2) + ((j & 7) >> 1)
+                high[row, head, index] = planes[kv, m // 16, step, 0, lane, slot]
+                low[row, head, index] = planes[kv, m // 16, step, 1, lane, slot]
+    return high, low, scale
+
+
+@pytest.mark.parametrize("tokens,rows,Q,KV,d,page,gated", [
+    (1000, 5, 64, 8, 128, 256, False),
+    (700, 4, 24, 4, 256, 256, True),
+    (300, 1, 16, 8, 128, 64, False),
+    (130, 3, 16, 2, 128, 64, True)])
+def test_prepared_query_operands_give_the_same_attention(device, tokens, rows, Q, KV, d,
+                                                         page, gated):
+    """The rotary kernel's query operands are what the attention kernel would
+    have built from the rotated queries itself: same bytes, same output."""
+    rng = np.random.default_rng(tokens + Q)
+    first = tokens - (rows - 1)           # context of the first row, new tokens included
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, page, 1, 0)
+    stride = d * (2 if gated else 1)
+    q = rng.standard_normal((rows, Q, stride)).astype(np.float32)
+    q[1 % rows, 3] *= 37.0                # rows of very different magnitude
+    k = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    v = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    d_pages = [gu.device_tensor(p, device) for p in pages]
+    table = torch.tensor([p.data_ptr() for p in d_pages], dtype=torch.int64, device=device)
+    d_q, d_k, d_v = (gu.device_tensor(x, device) for x in (q, k, v))
+    operand_bytes = qh.call("qllm_q4h_query_operand_bytes", rows, Q, KV, d)
+    group = Q // KV
+    row_tiles = (rows * group + 15) // 16
+    assert operand_bytes == KV * row_tiles * (d // 64) * 2048
+    operands = torch.zeros(operand_bytes, dtype=torch.uint8, device=device)
+    scales = torch.zeros(KV * row_tiles * 16, dtype=torch.float32, device=device)
+    qh.call("qllm_qkv_rope_cache_paged_q4h_prepared", None, 0, qh.ptr(d_q), stride,
+            qh.ptr(d_k), qh.ptr(d_v), None, None, qh.ptr(table), 0, page, first - 1,
+            first - 1, None, rows, Q, KV, d, d, 1e-6, 1e6, 0, qh.ptr(operands),
+            qh.ptr(scales), None)
+    torch.cuda.synchronize()
+    rotated = d_q.cpu().numpy()
+    high, low, scale = unpack_query_operands(operands.cpu().numpy(), scales.cpu().numpy(),
+                                             rows, Q, KV, d)
+    # 15 bits of each row's largest magnitude, exactly as the kernel rounds
+    largest = np.abs(rotated[..., :d]).max(axis=-1)
+    step = np.maximum(largest * np.float32(1.0 / 16319.0), np.float32(2.0 ** -100))
+    quantized = np.rint(rotated[..., :d] * (np.float32(1.0) / step)[..., None])
+    quantized = np.clip(quantized, -16319, 16319).astype(np.int32)
+    assert np.array_equal(128 * high.astype(np.int32) + low, quantized)
+    assert low.min() >= -64 and low.max() <= 63 and np.abs(high).max() <= 127
+    factor = np.float32(1.4426950408889634 / (16.0 * np.sqrt(np.float32(d))))
+    assert np.allclose(scale, step * factor, rtol=1e-6, atol=0)
+
+    def attend(prepared):
+        splits = 32
+        maxima = torch.zeros((rows, splits, Q), device=device)
+        sums = torch.zeros_like(maxima)
+        outputs = torch.zeros((rows, splits, Q, d), device=device)
+        out = torch.zeros((rows, Q, d), device=device)
+        launch = qh.Q4hAttentionLaunch(
+            qh.ptr(d_q), qh.ptr(operands) if prepared else 0,
+            qh.ptr(scales) if prepared else 0, qh.ptr(table), qh.ptr(out),
+            qh.ptr(maxima), qh.ptr(sums), qh.ptr(outputs), first, rows, 0, page, Q, KV,
+            d, 0, splits, stride, int(gated), qh.OUT_F32, None)
+        qh.call("qllm_attention_paged_q4h", launch)
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+
+    assert np.array_equal(attend(True), attend(False))
