@@ -42,6 +42,66 @@ __device__ __forceinline__ const void* uniform_page(
   return ((constant_table)page_table)[index];
 }
 
+// Tells the compiler that a pointer every lane computes alike is wave-uniform,
+// so that it can live in scalar registers.
+__device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* pointer) {
+  const uint64_t bits = reinterpret_cast<uint64_t>(pointer);
+  const uint32_t low =
+      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits));
+  const uint32_t high =
+      __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(bits >> 32));
+  return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(high) << 32) | low);
+}
+
+// Direct global -> LDS loads (no VGPRs): lane l of the wave fetches 16 (4)
+// bytes at base + offset[l] and they land at lds + 16*l (4*l).  `base` and
+// `lds` are wave-uniform.  Written as assembly so that the address stays in
+// the scalar-base + 32-bit-lane-offset form (one VGPR for all loads of a tile)
+// and so that the compiler, which would otherwise wait for every outstanding
+// load before any later LDS access, leaves the waiting to this kernel.
+__device__ __forceinline__ void copy16_to_lds(const uint8_t* base,
+                                              uint32_t lane_offset,
+                                              uint32_t lds) {
+  uint32_t saved_m0;  // M0 carries the LDS address; it is put back afterwards
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0) : "v"(lane_offset), "s"(base), "s"(lds) : "memory");
+}
+__device__ __forceinline__ void copy4_to_lds(const uint8_t* base,
+                                             uint32_t lane_offset,
+                                             uint32_t lds) {
+  uint32_t saved_m0;  // M0 carries the LDS address; it is put back afterwards
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0) : "v"(lane_offset), "s"(base), "s"(lds) : "memory");
+}
+
+// at most COUNT vmem loads (direct-to-LDS loads included) still in flight
+template <int COUNT>
+__device__ __forceinline__ void vmem_wait() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(COUNT) : "memory");
+}
+// Lane index recomputed where it is needed (two instructions) instead of
+// being kept in a register across the tile loop.
+__device__ __forceinline__ uint32_t fresh_lane_index() {
+  uint32_t lane;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0"
+               : "=v"(lane));
+  return lane;
+}
+__device__ __forceinline__ uint32_t lds_address(const void* pointer) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) const void*)pointer));
+}
+
 // Tiles [first, last) of the context that wave `wave` of split `split` walks.
 // split_tokens == 0: balanced - the context's tiles are dealt evenly over
 // every wave of the grid row, whatever the context length.  Otherwise split

@@ -445,6 +445,297 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
                            target);
 }
 
+// The binary16 cache at head_dim 128, software-pipelined: the kernel above
+// asks for a tile when it needs it and so leaves the memory system idle while
+// it computes.  Here a tile's K rows and V rows travel global -> LDS with
+// direct loads (no registers) into wave-private staging areas, and each area is
+// refilled with the next tile as soon as the current one has been read out of
+// it, so a wave always has a K or a V tile in flight.  Arithmetic, tile size and
+// the order of every sum are those of the kernel above: results are bit-equal.
+//
+// LDS granules (16 bytes) are swizzled against bank conflicts on the way in, by
+// the choice of which global granule a lane fetches for its LDS slot: K row r
+// keeps granule g at g ^ (r & 15) (the A-operand read takes one granule from
+// each of 16 consecutive rows), V row t at g ^ (2 * (t & 7)) as above.
+template <int RT>
+__global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_d128_kernel(
+    const F16SplitArgs args) {
+  constexpr int D = 128;
+  constexpr int KSTEPS = D / 32;
+  constexpr int DT = D / 16;
+  constexpr int GR = D / 8;                    // 16-byte granules per row
+  constexpr int TILE_BYTES = kF16Tile * D * 2;  // K (or V) rows of a tile
+  constexpr int STAGE = 2 * TILE_BYTES;        // a wave's K area, then its V area
+  constexpr int LOADS = TILE_BYTES / 1024;     // direct loads per area and tile
+  constexpr int UNITS = RT * KSTEPS;
+  constexpr int EXCHANGE_Q = UNITS * 1024 + RT * 64;
+  constexpr int EXCHANGE_MERGE = kSplitWaves * RT * 512;
+  static_assert(kSplitWaves * STAGE >= kSplitWaves * kSplitWaves * 1024,
+                "the merge pool fits the staging memory");
+  __shared__ __attribute__((aligned(16))) uint8_t stage[kSplitWaves * STAGE];
+  __shared__ __attribute__((aligned(16)))
+  uint8_t exchange[EXCHANGE_Q > EXCHANGE_MERGE ? EXCHANGE_Q : EXCHANGE_MERGE];
+
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t col = lane & 15u;
+  const uint32_t quad = lane >> 4;
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t split = blockIdx.y;
+  const uint32_t group = args.query_heads / args.kv_heads;
+  const uint32_t matrix_rows = args.rows * group;
+  const uint32_t first_context_tokens =
+      args.device_positions ? args.device_positions[2]
+                            : args.first_context_tokens;
+  const uint32_t last_context = first_context_tokens + args.rows - 1u;
+  const uint32_t context_tiles = (last_context + kF16Tile - 1u) / kF16Tile;
+  uint32_t tile_first, tile_last;
+  wave_tile_range(context_tiles, kF16Tile, args.split_tokens, split, gridDim.y,
+                  wave, tile_first, tile_last);
+
+  uint8_t* stage_k = stage + wave * STAGE;
+  uint8_t* stage_v = stage_k + TILE_BYTES;
+  const uint32_t stage_k_lds =
+      __builtin_amdgcn_readfirstlane(lds_address(stage_k));
+  const uint32_t stage_v_lds = stage_k_lds + TILE_BYTES;
+  const uint32_t row_bytes = args.kv_heads * D * 2u;   // bytes between tokens
+  const size_t page_bytes =
+      static_cast<size_t>(args.page_tokens) * row_bytes;   // K (or V) of a layer
+
+  // Load `pass` of an area fills LDS slots [64 * pass, +64): lane l holds row
+  // 4 * pass + l / 16, slot granule l % 16, and fetches the global granule that
+  // the swizzle puts there.  The lane's share of the address depends on
+  // pass % 4 (K) or pass % 2 (V) only.
+  auto stage_rows = [&](uint32_t tile, bool values) {
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t lane_row = lane_now >> 4;
+    const uint32_t granule = lane_now & 15u;
+    const uint32_t tile_begin = tile * kF16Tile;
+    const uint8_t* page = static_cast<const uint8_t*>(
+        uniform_page(args.pages, tile_begin / args.page_tokens));
+    const uint8_t* rows = uniform_pointer(
+        page + (static_cast<size_t>(args.layer) * 2u + (values ? 1u : 0u)) * page_bytes +
+        static_cast<size_t>(tile_begin % args.page_tokens) * row_bytes +
+        kv_head * (D * 2u));
+    const uint32_t target = values ? stage_v_lds : stage_k_lds;
+#pragma unroll
+    for (int pass = 0; pass < LOADS; ++pass) {
+      const uint32_t row = 4u * (pass % 4) + lane_row;   // row & 15
+      const uint32_t source_granule =
+          values ? granule ^ (2u * (row & 7u)) : granule ^ row;
+      copy16_to_lds(rows + static_cast<size_t>(4 * pass) * row_bytes,
+                    lane_row * row_bytes + source_granule * 16u,
+                    target + pass * 1024);
+    }
+  };
+  // the wave's first tile sets out before the query work below
+  if (tile_first < tile_last) {
+    stage_rows(tile_first, false);
+    stage_rows(tile_first, true);
+  }
+
+  // ---- query operands (B side of S = K.Q) in binary16, built once -------------
+  uint32_t* exchange_limit = reinterpret_cast<uint32_t*>(exchange + UNITS * 1024);
+  for (uint32_t unit = wave; unit < static_cast<uint32_t>(UNITS);
+       unit += kSplitWaves) {
+    const uint32_t rt = unit / KSTEPS;
+    const uint32_t step = unit % KSTEPS;
+    const uint32_t matrix_row = 16u * rt + col;
+    const bool valid = matrix_row < matrix_rows;
+    const uint32_t row = valid ? matrix_row / group : 0u;
+    const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
+    const float* source =
+        args.query +
+        (static_cast<size_t>(row) * args.query_heads + head) * args.query_stride +
+        32u * step + 8u * quad;
+    f16x8 operand;
+#pragma unroll
+    for (int piece = 0; piece < 2; ++piece) {
+      float4 loaded = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      if (valid) loaded = *reinterpret_cast<const float4*>(source + 4 * piece);
+      operand[4 * piece + 0] = static_cast<_Float16>(loaded.x);
+      operand[4 * piece + 1] = static_cast<_Float16>(loaded.y);
+      operand[4 * piece + 2] = static_cast<_Float16>(loaded.z);
+      operand[4 * piece + 3] = static_cast<_Float16>(loaded.w);
+    }
+    *reinterpret_cast<f16x8*>(exchange + unit * 1024u + lane * 16u) = operand;
+    if (step == 0u && quad == 0u)
+      exchange_limit[16u * rt + col] = first_context_tokens + row;
+  }
+  __syncthreads();
+  const uint8_t* q_operands = exchange + lane * 16u;
+  const float score_unit =
+      1.4426950408889634f / sqrtf(static_cast<float>(D));  // log2 units
+
+  // K operand of (st, ks): row 16 * st + col, granule 4 * ks + quad
+  const uint8_t* key_read = stage_k + col * (GR * 16u);
+  // V, transposing read: see the kernel above
+  const uint32_t read_token = 4u * quad + (col >> 2);
+  const uint32_t read_swizzle = read_token & 7u;
+  const uint32_t read_base =
+      read_token * (GR * 16u) + ((col >> 1) & 1u) * 16u + (col & 1u) * 8u;
+
+  float running_max[RT];
+  float running_sum[RT];
+  f32x4 out[DT][RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    running_max[rt] = kMaskedMax;
+    running_sum[rt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
+  }
+
+  // Loads in flight at the top of an iteration, oldest first: this tile's K,
+  // this tile's V.
+  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+    const uint32_t tile_begin = tile * kF16Tile;
+    const bool needs_mask = tile_begin + kF16Tile > first_context_tokens;
+    const bool has_next = tile + 1u < tile_last;
+
+    // ---- K rows out of LDS, the next tile's K on its way ------------------------
+    vmem_wait<LOADS>();
+    f16x8 key_operand[2][KSTEPS];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        key_operand[st][ks] = *reinterpret_cast<const f16x8*>(
+            key_read + st * 16 * (GR * 16) + (((4u * ks + quad) ^ col) * 16u));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (has_next) stage_rows(tile + 1u, false);
+
+    // ---- S = K . Q, online softmax, probabilities per row tile ------------------
+    f16x4 p_operand[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      asm volatile("" ::: "memory");  // one row tile's query operands at a time
+      float score[2][4];
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        f32x4 dot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          const f16x8 q = *reinterpret_cast<const f16x8*>(
+              q_operands + (rt * KSTEPS + ks) * 1024);
+          dot = __builtin_amdgcn_mfma_f32_16x16x32_f16(key_operand[st][ks], q,
+                                                       dot, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) score[st][i] = dot[i] * score_unit;
+      }
+      if (needs_mask) {
+        const uint32_t first_token = tile_begin + 4u * quad;
+        const uint32_t limit = exchange_limit[16 * rt + col];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (first_token + 16u * st + i >= limit) score[st][i] = -INFINITY;
+      }
+      float tile_max = score[0][0];
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tile_max = fmaxf(tile_max, score[st][i]);
+      tile_max = quad_row_max(tile_max);
+      const bool grew = tile_max - running_max[rt] > 8.0f;
+      if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+        const float new_max = fmaxf(running_max[rt], tile_max);
+        if (tile != tile_first) {
+          const float factor = __builtin_amdgcn_exp2f(running_max[rt] - new_max);
+          running_sum[rt] *= factor;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+        }
+        running_max[rt] = new_max;
+      }
+      float sum = 0.0f;
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const _Float16 p = static_cast<_Float16>(
+              __builtin_amdgcn_exp2f(score[st][i] - running_max[rt]));
+          p_operand[rt][st][i] = p;
+          sum += static_cast<float>(p);
+        }
+      running_sum[rt] += sum;
+    }
+
+    // ---- V rows have arrived; O^T += V^T . P^T ----------------------------------
+    // in flight, oldest first: this tile's V, the next tile's K
+    if (has_next)
+      vmem_wait<LOADS>();
+    else
+      vmem_wait<0>();
+    if (needs_mask) {
+      // records no row can see may be uninitialised: a NaN there would
+      // survive its zero probability
+#pragma unroll
+      for (int pass = 0; pass < LOADS; ++pass) {
+        const uint32_t token = 4u * pass + quad;
+        if (tile_begin + token >= last_context)
+          *reinterpret_cast<uint4*>(stage_v + (pass * 64u + lane) * 16u) =
+              make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const uint32_t address = st * 16u * (GR * 16u) + read_base +
+                                 ((2u * dt) ^ (2u * read_swizzle)) * 16u;
+        typedef short i16x4 __attribute__((ext_vector_type(4)));
+        const f16x4 v = __builtin_bit_cast(
+            f16x4, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                       (__attribute__((address_space(3))) i16x4*)(stage_v +
+                                                                  address)));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          out[dt][rt] = __builtin_amdgcn_mfma_f32_16x16x16f16(
+              v, p_operand[rt][st], out[dt][rt], 0, 0, 0);
+      }
+    }
+    // every V read has returned before the area is refilled
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (has_next) stage_rows(tile + 1u, true);
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) running_sum[rt] = quad_row_sum(running_sum[rt]);
+
+  const PartialTarget target{args.partial_maxima, args.partial_sums,
+                             args.partial_outputs, args.maximum_splits,
+                             args.query_heads, kv_head, split, group,
+                             matrix_rows};
+  merge_wave_states<D, RT>(running_max, running_sum, out,
+                           reinterpret_cast<float*>(stage),
+                           reinterpret_cast<float2*>(exchange), wave, lane,
+                           target);
+}
+
+int32_t launch_f16_split_d128(const F16SplitArgs& args, uint32_t row_tiles,
+                              dim3 grid, hipStream_t stream) {
+  switch (row_tiles) {
+    case 1:
+      f16_attention_split_d128_kernel<1><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      break;
+    case 2:
+      f16_attention_split_d128_kernel<2><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      break;
+    default:
+      f16_attention_split_d128_kernel<3><<<grid, kSplitWaves * 64, 0, stream>>>(args);
+      break;
+  }
+  return launched("F16 attention split");
+}
+
 template <int D, bool Q8 = false>
 int32_t launch_f16_split(const F16SplitArgs& args, uint32_t row_tiles, dim3 grid,
                          hipStream_t stream) {
@@ -557,8 +848,9 @@ extern "C" int32_t qllm_attention_paged_f16(
   const dim3 grid(launch->kv_heads, splits);
   const hipStream_t stream = as_stream(launch->stream);
   const int32_t status =
-      launch->head_dim == 128u ? launch_f16_split<128>(args, row_tiles, grid, stream)
-                               : launch_f16_split<256>(args, row_tiles, grid, stream);
+      launch->head_dim == 128u
+          ? launch_f16_split_d128(args, row_tiles, grid, stream)
+          : launch_f16_split<256>(args, row_tiles, grid, stream);
   if (status != QLLM_OK) return status;
   return launch_attention_combine(
       launch->query, launch->query_stride, launch->output_gated,

@@ -182,3 +182,38 @@ def test_f16_attention_at_262144_tokens_on_one_kv_head(device):
     shape = ol.AttentionShape(rows, Q, KV, d, first, page, 0, 0)
     gu.assert_close(results[0], ol.attention_f16(shape, query, pages, False),
                     what="262144-token F16 attention (exact)")
+
+
+@pytest.mark.parametrize("tokens,rows,Q,KV,splits,gated", [
+    (6000, 5, 64, 8, 4, False),      # six tiles per wave, three row tiles
+    (2051, 3, 16, 8, 2, True),       # one row tile, ragged tail tile
+    (40000, 4, 32, 4, 32, False)])   # two row tiles at 40K tokens
+def test_pipelined_kernel_equals_the_plain_one(device, tokens, rows, Q, KV, splits, gated):
+    """head_dim 128 launches take the kernel that keeps the next tile in flight;
+    the batched entry point still runs the plain one.  Same tiles, same order
+    of every sum: the outputs are bit-equal."""
+    rng = np.random.default_rng(tokens)
+    d, page_tokens = 128, 256
+    first = tokens - (rows - 1)
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.f16_pages(keys, values, page_tokens, 1, 0)
+    stride = d * (2 if gated else 1)
+    query = rng.standard_normal((rows, Q, stride)).astype(np.float32)
+    pipelined = gu.f16_attention(device, pages, query, rows, Q, KV, d, first, page_tokens,
+                                 0, gated, balanced_splits=splits)
+    d_pages = [gu.device_tensor(page, device) for page in pages]
+    table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
+                         device=device)
+    d_query = gu.device_tensor(query, device)
+    maxima = torch.zeros((rows, splits, Q), device=device)
+    sums = torch.zeros_like(maxima)
+    outputs = torch.zeros((rows, splits, Q, d), device=device)
+    out = torch.zeros((rows, Q, d), device=device)
+    launch = qh.F16AttentionLaunch(
+        qh.ptr(d_query), qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), first, rows, 0, page_tokens, Q, KV, d, 0, splits, stride,
+        int(gated), qh.OUT_F32, None)
+    qh.call("qllm_attention_paged_f16_batched", launch, rows)
+    torch.cuda.synchronize()
+    assert np.array_equal(pipelined, out.cpu().numpy())
