@@ -440,6 +440,41 @@ typedef struct qllm_q4h_attention_launch {
  * head_dim in {128, 256}, page_tokens % 64 == 0, split_tokens % 64 == 0.
  * The pages must hold every 64-token tile that overlaps the context. */
 int32_t qllm_attention_paged_q4h(const qllm_q4h_attention_launch* launch);
+/* The same launch doing the rotary kernel's work for the batch as well (the
+ * reference keeps them apart: gated_gqa_qkv_rope_paged_batch_kernel,
+ * transformer_kernels.cu:3550-3643, then the attention kernel).  launch->query
+ * holds the projection's raw query rows and is left as it is; key / value
+ * [rows, kv_heads, head_dim] the raw K and V rows.  Every workgroup normalises
+ * (weights may be NULL) and rotates the query rows of its KV head with the
+ * (cos, sin) pairs of rope_table - qllm_rope_table, [rows][rotary_dim / 2][2] -
+ * and quantises them as qllm_qkv_rope_cache_paged_q4h_prepared does; the
+ * batch's K/V records (cache positions first_cache_position .. + rows - 1, the
+ * last `rows` tokens of the context: first_cache_position + 1 ==
+ * first_context_tokens) are encoded by the workgroups that attend them and
+ * written to their pages by one of them.  With launch->device_positions the
+ * cache position is device_positions[0].  Outputs and page bytes equal those of
+ * the two separate launches. */
+typedef struct qllm_q4h_fused_rope {
+  const float* key;
+  const float* value;
+  const float* q_norm_weight;   /* NULL: no per-head norm */
+  const float* k_norm_weight;
+  const float* rope_table;
+  uint32_t rotary_dim;
+  float epsilon;
+  uint32_t first_cache_position;
+  int32_t bf16_activations;
+} qllm_q4h_fused_rope;
+int32_t qllm_attention_paged_q4h_fused(const qllm_q4h_attention_launch* launch,
+                                       const qllm_q4h_fused_rope* rope);
+/* (cos, sin) of the rotary angles of rows at positions first_rotary_position
+ * .. + rows - 1 (or from device_positions[1]), pair p of row r at
+ * table[(r * rotary_dim / 2 + p) * 2]: the values the rotary kernels compute
+ * for themselves (angle = position * theta^(-2p / rotary_dim)). */
+int32_t qllm_rope_table(float* table, uint32_t rows, uint32_t rotary_dim,
+                        uint32_t first_rotary_position, float rope_theta,
+                        int32_t bf16_activations,
+                        const uint32_t* device_positions, void* stream);
 /* Many micro-batches in one launch (prompt prefill): the launch's `rows` rows
  * are attended in batches of `batch_rows` consecutive rows, batch b exactly as
  * a launch of its own with first_context_tokens + b * batch_rows would be

@@ -5,6 +5,8 @@
 
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace qllm {
 
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
@@ -22,6 +24,22 @@ __device__ __forceinline__ float quad_row_max(float value) {
   auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(value),
                                             __float_as_uint(value), false, false);
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+// max over all 64 lanes without the LDS pipeline: four cross-lane steps inside
+// each row of 16 lanes, then the rows
+__device__ __forceinline__ float wave_max_in_registers(float value) {
+  const auto step = [](float v, auto control) {
+    const int moved = __builtin_amdgcn_update_dpp(
+        __float_as_int(v), __float_as_int(v), decltype(control)::value, 0xf, 0xf,
+        false);
+    return fmaxf(v, __int_as_float(moved));
+  };
+  value = step(value, std::integral_constant<int, 0xb1>{});    // quad_perm 1,0,3,2
+  value = step(value, std::integral_constant<int, 0x4e>{});    // quad_perm 2,3,0,1
+  value = step(value, std::integral_constant<int, 0x141>{});   // row_half_mirror
+  value = step(value, std::integral_constant<int, 0x140>{});   // row_mirror
+  return quad_row_max(value);
 }
 
 __device__ __forceinline__ float quad_row_sum(float value) {
@@ -102,6 +120,14 @@ __device__ __forceinline__ uint32_t lds_address(const void* pointer) {
       (__attribute__((address_space(3))) const void*)pointer));
 }
 
+// A word of a small device-side parameter block (step positions) that no
+// kernel writes: fetched with a scalar load, like the page table.
+__device__ __forceinline__ uint32_t uniform_word(const uint32_t* words,
+                                                 uint32_t index) {
+  typedef const uint32_t __attribute__((address_space(4)))* constant_words;
+  return ((constant_words)words)[index];
+}
+
 // Tiles [first, last) of the context that wave `wave` of split `split` walks.
 // split_tokens == 0: balanced - the context's tiles are dealt evenly over
 // every wave of the grid row, whatever the context length.  Otherwise split
@@ -115,12 +141,14 @@ __device__ __forceinline__ void wave_tile_range(uint32_t context_tiles,
                                                 uint32_t& tile_first,
                                                 uint32_t& tile_last) {
   if (split_tokens == 0u) {
+    // floor(slot * tiles / slots) in 32-bit arithmetic: with tiles = q * slots
+    // + r it is slot * q + floor(slot * r / slots), and slot * r < slots^2
     const uint32_t slots = splits * kSplitWaves;
     const uint32_t slot = split * kSplitWaves + wave;
-    tile_first = static_cast<uint32_t>(
-        static_cast<uint64_t>(slot) * context_tiles / slots);
-    tile_last = static_cast<uint32_t>(
-        static_cast<uint64_t>(slot + 1u) * context_tiles / slots);
+    const uint32_t quotient = context_tiles / slots;
+    const uint32_t remainder = context_tiles - quotient * slots;
+    tile_first = slot * quotient + slot * remainder / slots;
+    tile_last = (slot + 1u) * quotient + (slot + 1u) * remainder / slots;
   } else {
     const uint32_t split_tiles = split_tokens / tile_tokens;
     const uint32_t begin = min(split * split_tiles, context_tiles);

@@ -63,7 +63,8 @@ __global__ __launch_bounds__(64) void q8_store_kernel(
   const uint32_t lane = threadIdx.x;
   const uint32_t kv_head = blockIdx.x;
   const uint32_t row = blockIdx.y;
-  if (device_positions) first_cache_position = device_positions[0];
+  if (device_positions)
+    first_cache_position = uniform_word(device_positions, 0u);
   const uint32_t position = first_cache_position + row;
   uint8_t* page = static_cast<uint8_t*>(const_cast<void*>(
                       page_table[position / page_tokens])) + page_offset;
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
   const uint32_t group = args.query_heads / args.kv_heads;
   const uint32_t matrix_rows = args.rows * group;
   const uint32_t first_context_tokens =
-      args.device_positions ? args.device_positions[2]
+      args.device_positions ? uniform_word(args.device_positions, 2u)
                             : args.first_context_tokens;
   const uint32_t last_context = first_context_tokens + args.rows - 1u;
   const uint32_t context_tiles = (last_context + kF16Tile - 1u) / kF16Tile;
@@ -485,7 +486,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_d128_ker
   const uint32_t group = args.query_heads / args.kv_heads;
   const uint32_t matrix_rows = args.rows * group;
   const uint32_t first_context_tokens =
-      args.device_positions ? args.device_positions[2]
+      args.device_positions ? uniform_word(args.device_positions, 2u)
                             : args.first_context_tokens;
   const uint32_t last_context = first_context_tokens + args.rows - 1u;
   const uint32_t context_tiles = (last_context + kF16Tile - 1u) / kF16Tile;

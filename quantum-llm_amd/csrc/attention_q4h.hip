@@ -100,6 +100,18 @@ struct SplitArgs {
   // [z * batch_rows, +batch_rows) of `rows`, each layer a launch of its own as
   // far as the kernel is concerned.  0 = one batch holds all rows.
   uint32_t batch_rows;
+  // Fused rotary and K/V store (the FUSED instantiation): `query` then holds
+  // the projection's raw rows, raw_key / raw_value the batch's K and V rows,
+  // rope_table the rows' (cos, sin) as rope_table_kernel leaves them.
+  const float* raw_key;
+  const float* raw_value;
+  const float* q_weight;
+  const float* k_weight;
+  const float2* rope_table;
+  uint32_t rotary_dim;
+  float epsilon;
+  uint32_t first_cache_position;   // or device_positions[0]
+  uint32_t bf16_activations;
 };
 
 
@@ -165,6 +177,210 @@ __device__ __forceinline__ uint32_t insert_bits(uint32_t mask, uint32_t value,
   asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(result) : "s"(mask), "v"(value), "v"(base));
   return result;
 }
+// One wave encodes one (token, kv head) K or V vector.
+__device__ __forceinline__ void q4h_encode_record(const float* source,
+                                                  uint32_t head_dim,
+                                                  uint8_t* codes,
+                                                  uint8_t* scale_slot,
+                                                  uint32_t lane) {
+  float maximum = 0.0f;
+  for (uint32_t index = lane; index < head_dim; index += 64u)
+    maximum = fmaxf(maximum, fabsf(source[index]));
+  maximum = wave_max(maximum);
+  const uint32_t scale_bits =
+      f32_to_f16_bits(fmaxf(__fdiv_rn(maximum, 7.0f), 0x1p-24f));
+  const float scale = f16_bits_to_f32(scale_bits);
+  if (lane == 0u)
+    *reinterpret_cast<uint16_t*>(scale_slot) = static_cast<uint16_t>(scale_bits);
+  for (uint32_t pair = lane; pair < head_dim / 2u; pair += 64u) {
+    const int low = max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair], scale))));
+    const int high =
+        max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair + 1u], scale))));
+    codes[pair] = static_cast<uint8_t>((low & 0x0f) | ((high & 0x0f) << 4));
+  }
+}
+
+// Per-head RMSNorm(1+w) and NeoX rotary; one wave per (head, row).  The
+// rotated row is left in `rotated` (LDS) for a caller that goes on to encode
+// it, and written to `write_back` unless that is null.  TABLE: cosine and sine
+// of the row's position come from `table_row` [rotary_dim / 2] (as
+// rope_table_kernel leaves them) instead of being computed here.
+template <bool TABLE>
+__device__ __forceinline__ void head_norm_rope_impl(
+    const float* x, float* write_back, const float* weight, uint32_t head_dim,
+    uint32_t rotary_dim, uint32_t position, float epsilon, float theta,
+    bool bf16_activations, const float2* table_row, float* shared,
+    float* rotated, uint32_t lane) {
+  if (weight) {
+    float square = 0.0f;
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      square = fmaf(x[index], x[index], square);
+    square = wave_sum(square);
+    const float inverse =
+        rsqrtf(square / static_cast<float>(head_dim) + epsilon);
+    for (uint32_t index = lane; index < head_dim; index += 64u) {
+      const float value = x[index] * inverse * (1.0f + weight[index]);
+      shared[index] = bf16_activations ? bf16_round(value) : value;
+    }
+  } else {
+    for (uint32_t index = lane; index < head_dim; index += 64u)
+      shared[index] = x[index];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t half = rotary_dim / 2u;
+  for (uint32_t index = lane; index < head_dim; index += 64u) {
+    float result = shared[index];
+    if (index < rotary_dim) {
+      const uint32_t pair = index % half;
+      const float other =
+          index < half ? -shared[index + half] : shared[index - half];
+      float sine, cosine;
+      if constexpr (TABLE) {
+        const float2 entry = table_row[pair];
+        cosine = entry.x;
+        sine = entry.y;
+      } else {
+        const float angle =
+            static_cast<float>(position) *
+            powf(theta, -2.0f * static_cast<float>(pair) /
+                            static_cast<float>(rotary_dim));
+        sincosf(angle, &sine, &cosine);
+        if (bf16_activations) {
+          cosine = bf16_round(cosine);
+          sine = bf16_round(sine);
+        }
+      }
+      // one rounding order wherever this is compiled in
+      result = __fmaf_rn(shared[index], cosine, __fmul_rn(other, sine));
+    }
+    result = bf16_activations ? bf16_round(result) : result;
+    if (write_back) write_back[index] = result;
+    rotated[index] = result;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+__device__ __forceinline__ void head_norm_rope(float* x, const float* weight,
+                                               uint32_t head_dim,
+                                               uint32_t rotary_dim,
+                                               uint32_t position, float epsilon,
+                                               float theta, bool bf16_activations,
+                                               float* shared, float* rotated,
+                                               uint32_t lane) {
+  head_norm_rope_impl<false>(x, x, weight, head_dim, rotary_dim, position,
+                             epsilon, theta, bf16_activations, nullptr, shared,
+                             rotated, lane);
+}
+
+// The same arithmetic on a row that is already in registers (lane l holds
+// elements l, l + 64, ...: x, the norm weights and the (cos, sin) of each
+// element's pair), so that a caller can fetch several rows at once and pay one
+// memory round trip for all of them.  The rotated row is left in `rotated`.
+template <int N>
+__device__ __forceinline__ void head_norm_rope_registers(
+    const float (&x)[N], const float (&weight)[N], bool has_weight,
+    uint32_t rotary_dim, const float2 (&entry)[N], float epsilon,
+    bool bf16_activations, float* shared, float* rotated, uint32_t lane) {
+  constexpr uint32_t head_dim = 64u * N;
+  if (has_weight) {
+    float square = 0.0f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) square = fmaf(x[k], x[k], square);
+    square = wave_sum(square);
+    const float inverse =
+        rsqrtf(square / static_cast<float>(head_dim) + epsilon);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const float value = x[k] * inverse * (1.0f + weight[k]);
+      shared[lane + 64u * k] = bf16_activations ? bf16_round(value) : value;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < N; ++k) shared[lane + 64u * k] = x[k];
+  }
+  __builtin_amdgcn_wave_barrier();
+  const uint32_t half = rotary_dim / 2u;
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    const uint32_t index = lane + 64u * k;
+    float result = shared[index];
+    if (index < rotary_dim) {
+      const float other =
+          index < half ? -shared[index + half] : shared[index - half];
+      result = __fmaf_rn(shared[index], entry[k].x, __fmul_rn(other, entry[k].y));
+    }
+    rotated[index] = bf16_activations ? bf16_round(result) : result;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// The same once more without LDS, for rotary halves that are a multiple of 64
+// elements: both elements of a pair then sit in the same lane.  The rotated
+// row is returned in `rotated` (registers).
+template <int N>
+__device__ __forceinline__ void head_norm_rope_in_lane(
+    const float (&x)[N], const float (&weight)[N], bool has_weight,
+    uint32_t rotary_dim, const float2 (&entry)[N], float epsilon,
+    bool bf16_activations, float (&rotated)[N], uint32_t lane) {
+  constexpr uint32_t head_dim = 64u * N;
+  float value[N];
+  if (has_weight) {
+    float square = 0.0f;
+#pragma unroll
+    for (int k = 0; k < N; ++k) square = fmaf(x[k], x[k], square);
+    square = wave_sum(square);
+    const float inverse =
+        rsqrtf(square / static_cast<float>(head_dim) + epsilon);
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const float scaled = x[k] * inverse * (1.0f + weight[k]);
+      value[k] = bf16_activations ? bf16_round(scaled) : scaled;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < N; ++k) value[k] = x[k];
+  }
+  const int shift = static_cast<int>(rotary_dim / 128u);   // pair distance in k
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    float result = value[k];
+    if (k < 2 * shift) {
+      float partner = 0.0f;
+#pragma unroll
+      for (int j = 0; j < N; ++j)
+        if (k < shift ? j == k + shift : j + shift == k) partner = value[j];
+      const float other = k < shift ? -partner : partner;
+      result = __fmaf_rn(value[k], entry[k].x, __fmul_rn(other, entry[k].y));
+    }
+    rotated[k] = bf16_activations ? bf16_round(result) : result;
+  }
+}
+
+// Cosine and sine of rows' rotary angles, one (cos, sin) per (row, pair): what
+// head_norm_rope computes for itself, once per step instead of once per layer.
+__global__ void rope_table_kernel(float2* table, uint32_t rotary_dim,
+                                  uint32_t first_rotary_position, float theta,
+                                  bool bf16_activations,
+                                  const uint32_t* device_positions) {
+  if (device_positions)
+    first_rotary_position = uniform_word(device_positions, 1u);
+  const uint32_t half = rotary_dim / 2u;
+  const uint32_t row = blockIdx.x;
+  for (uint32_t pair = threadIdx.x; pair < half; pair += blockDim.x) {
+    const float angle =
+        static_cast<float>(first_rotary_position + row) *
+        powf(theta, -2.0f * static_cast<float>(pair) /
+                        static_cast<float>(rotary_dim));
+    float sine, cosine;
+    sincosf(angle, &sine, &cosine);
+    if (bf16_activations) {
+      cosine = bf16_round(cosine);
+      sine = bf16_round(sine);
+    }
+    table[row * half + pair] = make_float2(cosine, sine);
+  }
+}
+
 // D = head_dim (128 or 256), RT = number of 16-row tiles (rows*group <= 16*RT).
 //
 // Each wave owns a contiguous run of 64-token tiles.  A tile's K codes, V
@@ -172,12 +388,21 @@ __device__ __forceinline__ uint32_t insert_bits(uint32_t mask, uint32_t value,
 // staging area [K codes + scales | V codes]; each half is refilled with the
 // next tile as soon as the current tile has been read out of it, so the
 // loads fly while the matrix cores and the softmax work on registers.
-template <int D, int RT>
+//
+// FUSED: the kernel also does what qkv_rope_q4h_kernel does for the batch.
+// Every workgroup rotates (and, with weights, normalises) the query rows of
+// its KV head itself and quantises them straight into the operand area - this
+// work hides behind the flight of the first tile.  The batch's own K/V records
+// are encoded by the workgroups whose tiles reach them, into LDS, and laid over
+// the staged tile before it is read (the cache pages need not hold them yet);
+// the workgroup that owns the context's last tile also writes them to the
+// pages for later steps.
+template <int D, int RT, bool FUSED = false>
 __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     const SplitArgs launch_args) {
   // a batched launch narrows the arguments to the batch of this grid layer
   SplitArgs args = launch_args;
-  if (launch_args.batch_rows) {
+  if (!FUSED && launch_args.batch_rows) {
     const uint32_t first_row = blockIdx.z * launch_args.batch_rows;
     const size_t first_partial = static_cast<size_t>(first_row) *
                                  launch_args.maximum_splits *
@@ -191,6 +416,18 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     args.partial_sums = launch_args.partial_sums + first_partial;
     args.partial_outputs = launch_args.partial_outputs + first_partial * D;
   }
+  // Everything the prologue reads from the argument block is asked for here,
+  // in one round trip, not piece by piece along its chain of dependencies.
+  asm volatile("" ::"s"(args.query), "s"(args.page_table),
+               "s"(args.device_positions), "s"(args.query_operands),
+               "s"(args.query_operand_scales), "s"(args.query_stride),
+               "s"(args.first_context_tokens), "s"(args.rows), "s"(args.layer),
+               "s"(args.page_tokens), "s"(args.query_heads), "s"(args.kv_heads),
+               "s"(args.split_tokens));
+  if constexpr (FUSED)
+    asm volatile("" ::"s"(args.raw_key), "s"(args.raw_value), "s"(args.q_weight),
+                 "s"(args.k_weight), "s"(args.rope_table), "s"(args.rotary_dim),
+                 "s"(args.first_cache_position), "s"(args.bf16_activations));
   constexpr int KSTEPS = D / 64;      // int8 MFMA k-steps over head_dim
   constexpr int DT = D / 16;          // 16-wide tiles of head_dim
   constexpr int ROW = D / 2;          // bytes of codes per token
@@ -215,7 +452,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   const uint32_t group = args.query_heads / args.kv_heads;
   const uint32_t matrix_rows = args.rows * group;
   const uint32_t first_context_tokens =
-      args.device_positions ? args.device_positions[2]
+      args.device_positions ? uniform_word(args.device_positions, 2u)
                             : args.first_context_tokens;
   const uint32_t last_context = first_context_tokens + args.rows - 1u;
   const uint32_t context_tiles = (last_context + 63u) / 64u;
@@ -298,7 +535,254 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // so the integer scores carry the query to ~3e-5 relative instead of the
   // 4e-3 of a single Q8 plane.  The operands are published in MFMA order.
   static_assert(RT * KSTEPS <= kSplitWaves, "one wave per operand pair");
-  if (args.query_operands) {
+  // fused mode: scratch of the per-wave rotary, then the batch's fresh K/V
+  // records [K codes | V codes | K scale | V scale] of this KV head
+  constexpr int RECORD = D + 16;
+  constexpr int FRESH_ROWS = FUSED ? RT * 16 : 1;
+  // at head_dim 256 the rotary scratch lies in the (still empty) staging area
+  // and the first tile sets out after the query work: LDS has no room for both
+  constexpr bool SCRATCH_IN_STAGE = D == 256;
+  __shared__ float rope_scratch[FUSED && !SCRATCH_IN_STAGE ? kSplitWaves * 2 * D : 1];
+  __shared__ __attribute__((aligned(16))) uint8_t fresh[FRESH_ROWS * RECORD];
+  uint32_t first_cache_position = 0u;
+  bool reaches_batch = false;   // some tile of this workgroup holds batch tokens
+  if constexpr (FUSED) {
+    first_cache_position = args.device_positions ? uniform_word(args.device_positions, 0u)
+                                                 : args.first_cache_position;
+    float* shared = SCRATCH_IN_STAGE ? reinterpret_cast<float*>(stage_k)
+                                     : rope_scratch + wave * (2 * D);
+    float* rotated = shared + D;
+    const uint32_t half = args.rotary_dim / 2u;
+    constexpr int N = D / 64;                       // elements of a row per lane
+    constexpr int ROWS_PER_WAVE = RT * 16 / kSplitWaves;
+    // Everything the wave will need comes in one round trip: its query rows
+    // (matrix rows wave, wave + 8, ...), the batch's K/V row it encodes, norm
+    // weights and the rows' (cos, sin).
+    float q_values[ROWS_PER_WAVE][N];
+    float2 q_entry[ROWS_PER_WAVE][N];
+    float weights[2][N];                            // query norm, key norm
+    // (without norm weights the loads read the query buffer instead and their
+    // values go unused: no branch, no wait of its own)
+    const float* q_weight = args.q_weight ? args.q_weight : args.query;
+    const float* k_weight = args.k_weight ? args.k_weight : args.query;
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      weights[0][k] = q_weight[lane + 64u * k];
+      weights[1][k] = k_weight[lane + 64u * k];
+    }
+    // (rows past the batch fetch the last row again; nothing uses the values.
+    // Row and head of matrix row wave + 8 item follow from those of the row
+    // before, all on the scalar unit)
+    uint32_t pair_of_lane[N];
+    if ((half & (half - 1u)) == 0u) {
+#pragma unroll
+      for (int k = 0; k < N; ++k) pair_of_lane[k] = (lane + 64u * k) & (half - 1u);
+    } else {
+#pragma unroll
+      for (int k = 0; k < N; ++k) pair_of_lane[k] = (lane + 64u * k) % half;
+    }
+    {
+      uint32_t row = wave / group;
+      uint32_t member = wave % group;
+      const uint32_t row_step = kSplitWaves / group;
+      const uint32_t member_step = kSplitWaves % group;
+#pragma unroll
+      for (int item = 0; item < ROWS_PER_WAVE; ++item) {
+        const uint32_t fetched_row = min(row, args.rows - 1u);
+        const float* source = reinterpret_cast<const float*>(uniform_pointer(
+            reinterpret_cast<const uint8_t*>(
+                args.query + (fetched_row * args.query_heads + kv_head * group +
+                              member) * args.query_stride)));
+        const float2* entries = reinterpret_cast<const float2*>(uniform_pointer(
+            reinterpret_cast<const uint8_t*>(args.rope_table + fetched_row * half)));
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+          q_values[item][k] = source[lane + 64u * k];
+          q_entry[item][k] = entries[pair_of_lane[k]];
+        }
+        member += member_step;
+        row += row_step;
+        if (member >= group) {
+          member -= group;
+          ++row;
+        }
+      }
+    }
+    uint32_t workgroup_first, workgroup_last, unused;
+    wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y, 0u,
+                    workgroup_first, unused);
+    wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y,
+                    kSplitWaves - 1u, unused, workgroup_last);
+    reaches_batch = workgroup_first < workgroup_last &&
+                    workgroup_last * 64u > first_cache_position;
+    // the wave's first tile sets out first: the work below hides behind it
+    if (!SCRATCH_IN_STAGE && tile_first < tile_last) {
+      stage_keys(tile_first);
+      stage_values(tile_first);
+    }
+    // batch rows wave, wave + 8, ... are this wave's to encode (one for the
+    // usual batches; the rest, if any, are fetched when their turn comes)
+    const bool writes_pages = reaches_batch && workgroup_last == context_tiles;
+    float k_values[N], v_values[N];
+    float2 k_entry[N];
+    const auto fetch_record = [&](uint32_t row) {
+      const size_t source = (static_cast<size_t>(row) * args.kv_heads + kv_head) * D;
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        const uint32_t index = lane + 64u * k;
+        k_values[k] = args.raw_key[source + index];
+        v_values[k] = args.raw_value[source + index];
+        k_entry[k] = args.rope_table[row * half + pair_of_lane[k]];
+      }
+    };
+    if (reaches_batch && wave < args.rows) fetch_record(wave);
+    // where element lane + 64 k of a row goes inside the row's operand bytes:
+    // k-step 2 (d / 128) + (d % 32) / 16, lane quad (d % 128) / 32, byte slot
+    // (even elements of each half of 8 first, then the odd ones)
+    uint32_t piece_of_lane[N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      const uint32_t index = lane + 64u * k;
+      const uint32_t within = index % 128u;
+      const uint32_t step = 2u * (index / 128u) + (within % 32u) / 16u;
+      const uint32_t j = index % 16u;
+      piece_of_lane[k] = step * 2048u + (within / 32u) * 256u + (j & 8u) +
+                         ((j & 1u) << 2) + ((j & 7u) >> 1);
+    }
+    const bool pairs_in_lane = half % 64u == 0u;
+
+    // Rows past the batch go through the same arithmetic as zero rows (zero
+    // operands, the smallest scale, the first row's limit): no branch between
+    // the rows, so their instruction streams interleave.
+    const bool has_q_weight = args.q_weight != nullptr;
+    const bool bf16_rounding = args.bf16_activations != 0u;
+    const auto quantise_rows = [&](auto rotate) {
+#pragma unroll
+      for (int item = 0; item < ROWS_PER_WAVE; ++item) {
+        const uint32_t matrix_row = wave + kSplitWaves * item;
+        const uint32_t row_tile = matrix_row / 16u;
+        const uint32_t column = matrix_row % 16u;
+        const bool valid = matrix_row < matrix_rows;
+        float source[N];
+#pragma unroll
+        for (int k = 0; k < N; ++k) source[k] = valid ? q_values[item][k] : 0.0f;
+        float row_values[N];
+        rotate(source, q_entry[item], row_values);
+        float maximum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < N; ++k) maximum = fmaxf(maximum, fabsf(row_values[k]));
+        maximum = wave_max_in_registers(maximum);
+        const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
+        const float inverse = 1.0f / scale;
+        uint8_t* row_pieces =
+            exchange + row_tile * (KSTEPS * 2048u) + column * 16u;   // wave-uniform
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+          int quantized = __float2int_rn(row_values[k] * inverse);
+          quantized = max(-16319, min(16319, quantized));
+          const int high = (quantized + 64) >> 7;  // floor((v + 64) / 128)
+          const int low = quantized - (high << 7);
+          row_pieces[piece_of_lane[k]] = static_cast<uint8_t>(high);
+          row_pieces[piece_of_lane[k] + 1024u] = static_cast<uint8_t>(low);
+        }
+        if (lane == 0u) {
+          exchange_scale[matrix_row] =
+              scale *
+              (1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D))));
+          exchange_limit[matrix_row] =
+              first_context_tokens + (valid ? matrix_row / group : 0u);
+        }
+      }
+    };
+    if (pairs_in_lane && !has_q_weight && !bf16_rounding) {
+      // the usual case, straight-line: rotary only, both halves of a pair in
+      // the lane
+      const int shift = static_cast<int>(args.rotary_dim / 128u);
+      quantise_rows([&](const float (&x)[N], const float2 (&entry)[N],
+                        float (&result)[N]) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+          result[k] = x[k];
+          if (k < 2 * shift) {
+            float partner = 0.0f;
+#pragma unroll
+            for (int j = 0; j < N; ++j)
+              if (k < shift ? j == k + shift : j + shift == k) partner = x[j];
+            const float other = k < shift ? -partner : partner;
+            result[k] = __fmaf_rn(x[k], entry[k].x, __fmul_rn(other, entry[k].y));
+          }
+        }
+      });
+    } else if (pairs_in_lane) {
+      quantise_rows([&](const float (&x)[N], const float2 (&entry)[N],
+                        float (&result)[N]) {
+        head_norm_rope_in_lane<N>(x, weights[0], has_q_weight, args.rotary_dim, entry,
+                                  args.epsilon, bf16_rounding, result, lane);
+      });
+    } else {
+      quantise_rows([&](const float (&x)[N], const float2 (&entry)[N],
+                        float (&result)[N]) {
+        head_norm_rope_registers<N>(x, weights[0], has_q_weight, args.rotary_dim,
+                                    entry, args.epsilon, bf16_rounding, shared,
+                                    rotated, lane);
+#pragma unroll
+        for (int k = 0; k < N; ++k) result[k] = rotated[lane + 64u * k];
+        __builtin_amdgcn_wave_barrier();   // `rotated` is reused by the next row
+      });
+    }
+    if (reaches_batch) {
+      for (uint32_t row = wave; row < args.rows; row += kSplitWaves) {
+        if (row != wave) fetch_record(row);
+        uint8_t* record = fresh + row * RECORD;
+        head_norm_rope_registers<N>(k_values, weights[1], args.k_weight != nullptr,
+                                    args.rotary_dim, k_entry, args.epsilon,
+                                    args.bf16_activations != 0u, shared, rotated,
+                                    lane);
+        q4h_encode_record(rotated, D, record, record + D, lane);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int k = 0; k < N; ++k) shared[lane + 64u * k] = v_values[k];
+        __builtin_amdgcn_wave_barrier();
+        q4h_encode_record(shared, D, record + ROW, record + D + 2, lane);
+        __builtin_amdgcn_wave_barrier();
+        if (writes_pages) {
+          // the record goes to its page for the steps to come
+          const uint32_t position = first_cache_position + row;
+          uint8_t* page = static_cast<uint8_t*>(const_cast<void*>(
+              args.page_table[position / args.page_tokens]));
+          const Q4hPlanes planes =
+              q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
+          const size_t slot = static_cast<size_t>(kv_head) * args.page_tokens +
+                              position % args.page_tokens;
+          constexpr uint32_t kWords = ROW / 4u;   // dwords of codes per record
+          if (lane < kWords)
+            reinterpret_cast<uint32_t*>(
+                const_cast<uint8_t*>(planes.key_codes) + slot * ROW)[lane] =
+                reinterpret_cast<const uint32_t*>(record)[lane];
+          if (lane < kWords)
+            reinterpret_cast<uint32_t*>(
+                const_cast<uint8_t*>(planes.value_codes) + slot * ROW)[lane] =
+                reinterpret_cast<const uint32_t*>(record + ROW)[lane];
+          if (lane == 0u)
+            *reinterpret_cast<uint16_t*>(
+                const_cast<uint8_t*>(planes.key_scales) + slot * 2u) =
+                *reinterpret_cast<const uint16_t*>(record + D);
+          if (lane == 1u)
+            *reinterpret_cast<uint16_t*>(
+                const_cast<uint8_t*>(planes.value_scales) + slot * 2u) =
+                *reinterpret_cast<const uint16_t*>(record + D + 2);
+        }
+      }
+    }
+    if (SCRATCH_IN_STAGE && tile_first < tile_last) {
+      // every lane is done with the scratch before the tile lands on it
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      __builtin_amdgcn_wave_barrier();
+      stage_keys(tile_first);
+      stage_values(tile_first);
+    }
+    vmem_wait<0>();
+  } else if (args.query_operands) {
     // prepared by the rotary kernel: the planes go straight to LDS, one KiB
     // per wave and load, the scales with them
     constexpr uint32_t kPlanes = RT * KSTEPS * 2;
@@ -325,11 +809,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   }
   // the wave's first tile sets out before the query work below, which its
   // flight time covers
-  if (tile_first < tile_last) {
+  if (!FUSED && tile_first < tile_last) {
     stage_keys(tile_first);
     stage_values(tile_first);
   }
-  if (args.query_operands) {
+  if (FUSED) {
+  } else if (args.query_operands) {
     vmem_wait<0>();
   } else if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
     // wave u builds k-step u % KSTEPS of row tile u / KSTEPS (the row's scale
@@ -445,6 +930,30 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
     // ---- K codes and scales out of LDS ----------------------------------------
     vmem_wait<V_LOADS>();
+    // the batch's own tokens inside this tile, [batch_first, batch_last)
+    uint32_t batch_first = 0u, batch_last = 0u;
+    if constexpr (FUSED) {
+      batch_first = max(first_cache_position, tile_begin);
+      batch_last = min(first_cache_position + args.rows, tile_begin + 64u);
+      if (batch_first < batch_last) {
+        // their fresh K records go over whatever the pages held
+        const uint32_t count = batch_last - batch_first;
+        for (uint32_t piece = lane; piece < count * kParts; piece += 64u) {
+          const uint32_t token = batch_first + piece / kParts;
+          const uint32_t part = piece % kParts;
+          *reinterpret_cast<uint4*>(stage_k + (token - tile_begin) * ROW + part * 16u) =
+              *reinterpret_cast<const uint4*>(
+                  fresh + (token - first_cache_position) * RECORD + part * 16u);
+        }
+        for (uint32_t index = lane; index < count; index += 64u) {
+          const uint32_t token = batch_first + index;
+          *reinterpret_cast<uint16_t*>(stage_k + CODES + 2u * (token - tile_begin)) =
+              *reinterpret_cast<const uint16_t*>(
+                  fresh + (token - first_cache_position) * RECORD + D);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+    }
     u32x4 key_raw[4 * (D / 128)];
     u32x2 scale_raw[4];  // K scales of sub-tile st
     [&]<int... I>(std::integer_sequence<int, I...>) {
@@ -545,6 +1054,30 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
           vmem_wait<KS_LOADS>();
         else
           vmem_wait<0>();
+        if constexpr (FUSED) {
+          if (batch_first < batch_last) {
+            // and their fresh V records (LDS row of token t: see stage_values)
+            uint8_t* stage_v = stage_k + CODES + 256;
+            const uint32_t count = batch_last - batch_first;
+            for (uint32_t piece = lane; piece < count * kParts; piece += 64u) {
+              const uint32_t token = batch_first + piece / kParts;
+              const uint32_t part = piece % kParts;
+              const uint32_t t = token - tile_begin;
+              const uint32_t lds_row = 16u * ((t >> 2) & 3u) + 4u * (t >> 4) + (t & 3u);
+              *reinterpret_cast<uint4*>(stage_v + lds_row * ROW + part * 16u) =
+                  *reinterpret_cast<const uint4*>(
+                      fresh + (token - first_cache_position) * RECORD + ROW +
+                      part * 16u);
+            }
+            for (uint32_t index = lane; index < count; index += 64u) {
+              const uint32_t token = batch_first + index;
+              *reinterpret_cast<uint16_t*>(stage_v + CODES + 2u * (token - tile_begin)) =
+                  *reinterpret_cast<const uint16_t*>(
+                      fresh + (token - first_cache_position) * RECORD + D + 2);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          }
+        }
         u32x2 value_scale_raw[4];
         [&]<int... I>(std::integer_sequence<int, I...>) {
           ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
@@ -698,7 +1231,8 @@ __global__ void attention_combine_kernel(
     const uint32_t* device_positions) {
   __shared__ float weights[kCombineSplitCapacity];
   __shared__ float scratch[4];
-  if (device_positions) first_context_tokens = device_positions[2];
+  if (device_positions)
+    first_context_tokens = uniform_word(device_positions, 2u);
   const uint32_t head = blockIdx.x;
   const uint32_t row = blockIdx.y;
   const uint32_t dimension = threadIdx.x;
@@ -791,29 +1325,6 @@ __global__ void attention_combine_kernel(
 
 // ---- K/V store ----------------------------------------------------------------
 
-// One wave encodes one (token, kv head) K or V vector.
-__device__ __forceinline__ void q4h_encode_record(const float* source,
-                                                  uint32_t head_dim,
-                                                  uint8_t* codes,
-                                                  uint8_t* scale_slot,
-                                                  uint32_t lane) {
-  float maximum = 0.0f;
-  for (uint32_t index = lane; index < head_dim; index += 64u)
-    maximum = fmaxf(maximum, fabsf(source[index]));
-  maximum = wave_max(maximum);
-  const uint32_t scale_bits =
-      f32_to_f16_bits(fmaxf(__fdiv_rn(maximum, 7.0f), 0x1p-24f));
-  const float scale = f16_bits_to_f32(scale_bits);
-  if (lane == 0u)
-    *reinterpret_cast<uint16_t*>(scale_slot) = static_cast<uint16_t>(scale_bits);
-  for (uint32_t pair = lane; pair < head_dim / 2u; pair += 64u) {
-    const int low = max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair], scale))));
-    const int high =
-        max(-7, min(7, __float2int_rn(__fdiv_rn(source[2u * pair + 1u], scale))));
-    codes[pair] = static_cast<uint8_t>((low & 0x0f) | ((high & 0x0f) << 4));
-  }
-}
-
 __global__ __launch_bounds__(64) void q4h_store_kernel(
     const float* key, const float* value, const void* const* page_table,
     uint32_t layer, uint32_t page_tokens, uint32_t first_cache_position,
@@ -837,58 +1348,6 @@ __global__ __launch_bounds__(64) void q4h_store_kernel(
                     const_cast<uint8_t*>(planes.value_scales) + record * 2u, lane);
 }
 
-// Per-head RMSNorm(1+w) and NeoX rotary, in place; one wave per (head, row).
-// The rotated row is also left in `rotated` (LDS) for a caller that goes on to
-// encode it.
-__device__ __forceinline__ void head_norm_rope(float* x, const float* weight,
-                                               uint32_t head_dim,
-                                               uint32_t rotary_dim,
-                                               uint32_t position, float epsilon,
-                                               float theta, bool bf16_activations,
-                                               float* shared, float* rotated,
-                                               uint32_t lane) {
-  if (weight) {
-    float square = 0.0f;
-    for (uint32_t index = lane; index < head_dim; index += 64u)
-      square = fmaf(x[index], x[index], square);
-    square = wave_sum(square);
-    const float inverse =
-        rsqrtf(square / static_cast<float>(head_dim) + epsilon);
-    for (uint32_t index = lane; index < head_dim; index += 64u) {
-      const float value = x[index] * inverse * (1.0f + weight[index]);
-      shared[index] = bf16_activations ? bf16_round(value) : value;
-    }
-  } else {
-    for (uint32_t index = lane; index < head_dim; index += 64u)
-      shared[index] = x[index];
-  }
-  __builtin_amdgcn_wave_barrier();
-  const uint32_t half = rotary_dim / 2u;
-  for (uint32_t index = lane; index < head_dim; index += 64u) {
-    float result = shared[index];
-    if (index < rotary_dim) {
-      const uint32_t pair = index % half;
-      const float angle =
-          static_cast<float>(position) *
-          powf(theta, -2.0f * static_cast<float>(pair) /
-                          static_cast<float>(rotary_dim));
-      const float other =
-          index < half ? -shared[index + half] : shared[index - half];
-      float sine, cosine;
-      sincosf(angle, &sine, &cosine);
-      if (bf16_activations) {
-        cosine = bf16_round(cosine);
-        sine = bf16_round(sine);
-      }
-      result = shared[index] * cosine + other * sine;
-    }
-    result = bf16_activations ? bf16_round(result) : result;
-    x[index] = result;
-    rotated[index] = result;
-  }
-  __builtin_amdgcn_wave_barrier();
-}
-
 // grid (query_heads + kv_heads, rows): blocks [0, query_heads) rotate a query
 // head, the others rotate a key head and encode that K/V record.
 __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
@@ -904,8 +1363,8 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
   __shared__ float shared[256];
   __shared__ float rotated[256];
   if (device_positions) {
-    first_cache_position = device_positions[0];
-    first_rotary_position = device_positions[1];
+    first_cache_position = uniform_word(device_positions, 0u);
+    first_rotary_position = uniform_word(device_positions, 1u);
   }
   const uint32_t row = blockIdx.y;
   const uint32_t lane = threadIdx.x;
@@ -1037,20 +1496,22 @@ __global__ __launch_bounds__(64) void quantize_queries_q8_kernel(
   }
 }
 
-template <int D>
+template <int D, bool FUSED = false>
 int32_t launch_split(const SplitArgs& args, uint32_t row_tiles, dim3 grid,
                      hipStream_t stream) {
   const size_t lds = 0;  // all LDS of the split kernel is static
   switch (row_tiles) {
     case 1:
-      q4h_attention_split_kernel<D, 1><<<grid, kSplitWaves * 64, lds, stream>>>(args);
+      q4h_attention_split_kernel<D, 1, FUSED>
+          <<<grid, kSplitWaves * 64, lds, stream>>>(args);
       break;
     case 2:
-      q4h_attention_split_kernel<D, 2><<<grid, kSplitWaves * 64, lds, stream>>>(args);
+      q4h_attention_split_kernel<D, 2, FUSED>
+          <<<grid, kSplitWaves * 64, lds, stream>>>(args);
       break;
     default:
       if constexpr (D == 128) {
-        q4h_attention_split_kernel<D, 3>
+        q4h_attention_split_kernel<D, 3, FUSED>
             <<<grid, kSplitWaves * 64, lds, stream>>>(args);
         break;
       } else {
@@ -1363,8 +1824,9 @@ extern "C" int32_t qllm_attention_paged_q4h_batched(
       launch->query_heads, launch->head_dim, nullptr, stream);
 }
 
-extern "C" int32_t qllm_attention_paged_q4h(
-    const qllm_q4h_attention_launch* launch) {
+namespace {
+int32_t launch_q4h_attention(const qllm_q4h_attention_launch* launch,
+                             const qllm_q4h_fused_rope* rope) {
   if (!launch || !launch->query || !launch->page_table || !launch->output ||
       (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
       launch->query_stride % 4u ||
@@ -1425,9 +1887,32 @@ extern "C" int32_t qllm_attention_paged_q4h(
   args.device_positions = launch->device_positions;
   const dim3 grid(launch->kv_heads, splits);
   const hipStream_t stream = as_stream(launch->stream);
-  int32_t status = launch->head_dim == 128u
-                       ? launch_split<128>(args, row_tiles, grid, stream)
-                       : launch_split<256>(args, row_tiles, grid, stream);
+  int32_t status;
+  if (rope) {
+    if (!rope->key || !rope->value || !rope->rope_table || !rope->rotary_dim ||
+        rope->rotary_dim > launch->head_dim || rope->rotary_dim % 2u ||
+        !(rope->epsilon > 0.0f) ||
+        (!launch->device_positions &&
+         rope->first_cache_position + 1u != launch->first_context_tokens))
+      return fail(QLLM_INVALID_ARGUMENT, "invalid fused rotary inputs");
+    args.query_operands = nullptr;
+    args.raw_key = rope->key;
+    args.raw_value = rope->value;
+    args.q_weight = rope->q_norm_weight;
+    args.k_weight = rope->k_norm_weight;
+    args.rope_table = reinterpret_cast<const float2*>(rope->rope_table);
+    args.rotary_dim = rope->rotary_dim;
+    args.epsilon = rope->epsilon;
+    args.first_cache_position = rope->first_cache_position;
+    args.bf16_activations = rope->bf16_activations != 0 ? 1u : 0u;
+    status = launch->head_dim == 128u
+                 ? launch_split<128, true>(args, row_tiles, grid, stream)
+                 : launch_split<256, true>(args, row_tiles, grid, stream);
+  } else {
+    status = launch->head_dim == 128u
+                 ? launch_split<128>(args, row_tiles, grid, stream)
+                 : launch_split<256>(args, row_tiles, grid, stream);
+  }
   if (status != QLLM_OK) return status;
   return launch_attention_combine(
       launch->query, launch->query_stride, launch->output_gated,
@@ -1435,4 +1920,32 @@ extern "C" int32_t qllm_attention_paged_q4h(
       launch->output, launch->output_kind, launch->first_context_tokens,
       launch->maximum_splits, launch->split_tokens, launch->rows,
       launch->query_heads, launch->head_dim, launch->device_positions, stream);
+}
+}  // namespace
+
+extern "C" int32_t qllm_attention_paged_q4h(
+    const qllm_q4h_attention_launch* launch) {
+  return launch_q4h_attention(launch, nullptr);
+}
+
+extern "C" int32_t qllm_attention_paged_q4h_fused(
+    const qllm_q4h_attention_launch* launch, const qllm_q4h_fused_rope* rope) {
+  if (!rope) return fail(QLLM_INVALID_ARGUMENT, "invalid fused rotary inputs");
+  return launch_q4h_attention(launch, rope);
+}
+
+extern "C" int32_t qllm_rope_table(float* table, uint32_t rows,
+                                   uint32_t rotary_dim,
+                                   uint32_t first_rotary_position,
+                                   float rope_theta, int32_t bf16_activations,
+                                   const uint32_t* device_positions,
+                                   void* stream) {
+  if (!table || !rows || !rotary_dim || rotary_dim % 2u || rotary_dim > 256u ||
+      !(rope_theta > 0.0f) ||
+      (!device_positions && first_rotary_position > 0xffffffffu - (rows - 1u)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid rotary table request");
+  rope_table_kernel<<<rows, 128, 0, as_stream(stream)>>>(
+      reinterpret_cast<float2*>(table), rotary_dim, first_rotary_position,
+      rope_theta, bf16_activations != 0, device_positions);
+  return launched("rotary table");
 }

@@ -359,6 +359,9 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
               "clear query operands");
     hip_check(hipMemset(query_operand_scales_, 0, scale_bytes),
               "clear query operand scales");
+    // (cos, sin) of a batch's rotary angles, computed once per pass
+    rope_table_ = static_cast<float*>(
+        device_alloc(std::size_t{max_rows_} * g_.rotary_dim * 4U));
   }
 
   select_workspace_bytes_ = std::max(
@@ -1029,6 +1032,7 @@ er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
         state->current_batch_first = positions.front();
         state->current_position = positions.back();
         ensure_pages(positions.back());
+        enqueue_rope_table(rows, positions.front(), false);
         enqueue_attention_block(operation->layer, rows, positions.front(), false,
                                 false);
         outputs.emplace("hidden", device_hidden_value(rows));
@@ -1237,20 +1241,25 @@ void Mi355DenseFp4Provider::enqueue_attention(
   const auto& layer = layers_[index];
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   if (g_.kv_encoding == KvEncoding::q4_f16_per_head) {
-    // rotary + K/V store; the queries also leave as the attention kernel's
-    // int8 operands, so that it starts on its tiles at once
-    status_check(qllm_qkv_rope_cache_paged_q4h_prepared(
-        qkv_partials, qkv_partial_count, query, query_stride, key, value,
-        layer.query_norm, layer.key_norm,
-        const_cast<const void* const*>(device_page_table_), index,
-        g_.kv_page_tokens, first_position, first_position,
-        deferred_positions ? positions_ : nullptr, rows, g_.query_heads,
-        g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
-        g_.rope_theta, 0, query_operands_, query_operand_scales_, stream));
+    // With the projection in one piece the attention kernel does the rotary
+    // and the K/V store itself (cos / sin from rope_table_, see
+    // enqueue_rope_table); K-split partials go through the rotary kernel,
+    // which sums them and leaves the queries as the attention kernel's int8
+    // operands.
+    const bool fused = qkv_partials == nullptr;
+    if (!fused)
+      status_check(qllm_qkv_rope_cache_paged_q4h_prepared(
+          qkv_partials, qkv_partial_count, query, query_stride, key, value,
+          layer.query_norm, layer.key_norm,
+          const_cast<const void* const*>(device_page_table_), index,
+          g_.kv_page_tokens, first_position, first_position,
+          deferred_positions ? positions_ : nullptr, rows, g_.query_heads,
+          g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon,
+          g_.rope_theta, 0, query_operands_, query_operand_scales_, stream));
     qllm_q4h_attention_launch launch{};
     launch.query = query;
-    launch.q8_queries = query_operands_;
-    launch.query_scales = query_operand_scales_;
+    launch.q8_queries = fused ? nullptr : query_operands_;
+    launch.query_scales = fused ? nullptr : query_operand_scales_;
     launch.page_table = const_cast<const void* const*>(device_page_table_);
     launch.output = attention_out;
     launch.partial_maxima = partial_maxima_;
@@ -1270,7 +1279,21 @@ void Mi355DenseFp4Provider::enqueue_attention(
     launch.output_kind = QLLM_OUT_BF16;
     launch.stream = stream;
     launch.device_positions = deferred_positions ? positions_ : nullptr;
-    status_check(qllm_attention_paged_q4h(&launch));
+    if (fused) {
+      qllm_q4h_fused_rope rope{};
+      rope.key = key;
+      rope.value = value;
+      rope.q_norm_weight = layer.query_norm;
+      rope.k_norm_weight = layer.key_norm;
+      rope.rope_table = rope_table_;
+      rope.rotary_dim = g_.rotary_dim;
+      rope.epsilon = g_.norm_epsilon;
+      rope.first_cache_position = first_position;
+      rope.bf16_activations = 0;
+      status_check(qllm_attention_paged_q4h_fused(&launch, &rope));
+    } else {
+      status_check(qllm_attention_paged_q4h(&launch));
+    }
   } else {
     status_check(qllm_qkv_rope_batch(
         query, query_stride, key, layer.query_norm, layer.key_norm,
@@ -1302,6 +1325,18 @@ void Mi355DenseFp4Provider::enqueue_attention(
     launch.stream = stream;
     status_check(qllm_attention_paged_f16(&launch));
   }
+}
+
+// (cos, sin) of the rotary angles of a batch at first_position .. + rows - 1
+// (or at the device-side positions), for the attention launches of a pass.
+void Mi355DenseFp4Provider::enqueue_rope_table(std::uint32_t rows,
+                                               std::uint32_t first_position,
+                                               bool deferred_positions) {
+  if (!rope_table_) return;
+  status_check(qllm_rope_table(rope_table_, rows, g_.rotary_dim, first_position,
+                               g_.rope_theta, 0,
+                               deferred_positions ? positions_ : nullptr,
+                               stream_));
 }
 
 // RMSNorm of hidden_ into normalized_ (bf16), first adding the partials a
@@ -1419,6 +1454,7 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                            bool deferred_positions) {
   status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
                                         hidden_, rows, stream_));
+  enqueue_rope_table(rows, first_position, deferred_positions);
   pending_partials_ = 0U;
   for (std::uint32_t index = 0; index < g_.layers; ++index) {
     enqueue_attention_block(index, rows, first_position, deferred_positions,
@@ -1920,16 +1956,8 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
       if (!context_tokens || context_tokens + rows > g_.max_context)
         return {er::ErrorCode::invalid_argument, "timing context is invalid"};
       ensure_pages(context_tokens + rows - 1U);
-      // the attention launches read the query operands a rotary launch leaves
-      if (g_.kv_encoding == KvEncoding::q4_f16_per_head)
-        status_check(qllm_qkv_rope_cache_paged_q4h_prepared(
-            nullptr, 0U, query_, query_stride, key_, value_,
-            layers_[0].query_norm, layers_[0].key_norm,
-            const_cast<const void* const*>(device_page_table_), 0U,
-            g_.kv_page_tokens, context_tokens, context_tokens, nullptr, rows,
-            g_.query_heads, g_.kv_heads, g_.head_dim, g_.rotary_dim,
-            g_.norm_epsilon, g_.rope_theta, 0, query_operands_,
-            query_operand_scales_, stream_));
+      // the attention launches rotate and store the batch themselves
+      enqueue_rope_table(rows, context_tokens, false);
     }
     const auto launch_one = [&](std::uint32_t index) {
       const auto& layer = layers_[index % g_.layers];
@@ -2009,8 +2037,6 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
       } else if (which == "attention") {
         qllm_q4h_attention_launch launch{};
         launch.query = query_;
-        launch.q8_queries = query_operands_;   // as the target pass launches it
-        launch.query_scales = query_operand_scales_;
         launch.page_table = const_cast<const void* const*>(device_page_table_);
         launch.output = attention_;
         launch.partial_maxima = partial_maxima_;
@@ -2029,7 +2055,17 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
         launch.output_gated = g_.output_gated;
         launch.output_kind = QLLM_OUT_BF16;
         launch.stream = stream_;
-        status_check(qllm_attention_paged_q4h(&launch));
+        // as the target pass launches it
+        qllm_q4h_fused_rope rope{};
+        rope.key = key_;
+        rope.value = value_;
+        rope.q_norm_weight = layer.query_norm;
+        rope.k_norm_weight = layer.key_norm;
+        rope.rope_table = rope_table_;
+        rope.rotary_dim = g_.rotary_dim;
+        rope.epsilon = g_.norm_epsilon;
+        rope.first_cache_position = context_tokens;
+        status_check(qllm_attention_paged_q4h_fused(&launch, &rope));
       } else {
         throw std::runtime_error("unknown kernel name: " + which);
       }

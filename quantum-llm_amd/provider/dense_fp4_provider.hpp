@@ -265,6 +265,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                    const std::uint16_t* input,
                                    std::size_t input_bytes, std::uint32_t rows,
                                    bool leave_partials);
+  void enqueue_rope_table(std::uint32_t rows, std::uint32_t first_position,
+                          bool deferred_positions);
   void enqueue_attention_block(std::uint32_t index, std::uint32_t rows,
                                std::uint32_t first_position,
                                bool deferred_positions, bool leave_partials);
@@ -382,6 +384,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* partial_outputs_{};
   std::int8_t* query_operands_{};       // Q4H attention operands of a batch
   float* query_operand_scales_{};
+  float* rope_table_{};                 // [max_rows, rotary_dim / 2] (cos, sin)
   // Pinned host words for the small per-pass transfers: 8 tokens + 4
   // position words up (target pass, proposer pass), 8 chosen tokens down.
   struct HostStaging {

@@ -51,6 +51,13 @@ class Q4hAttentionLaunch(Structure):
                 ("stream", c_void_p), ("device_positions", c_void_p)]
 
 
+class Q4hFusedRope(Structure):
+    _fields_ = [("key", c_void_p), ("value", c_void_p), ("q_norm_weight", c_void_p),
+                ("k_norm_weight", c_void_p), ("rope_table", c_void_p),
+                ("rotary_dim", c_uint32), ("epsilon", c_float),
+                ("first_cache_position", c_uint32), ("bf16_activations", c_int32)]
+
+
 class F16AttentionLaunch(Structure):
     _fields_ = [("query", c_void_p), ("device_pages", c_void_p),
                 ("output", c_void_p), ("partial_maxima", c_void_p),
@@ -112,6 +119,8 @@ SIGNATURES = {
     "qllm_store_kv_paged_q4h_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_quantize_gqa_queries_q8": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_q4h": (c_int32, [POINTER(Q4hAttentionLaunch)]),
+    "qllm_attention_paged_q4h_fused": (c_int32, [POINTER(Q4hAttentionLaunch), POINTER(Q4hFusedRope)]),
+    "qllm_rope_table": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p, c_void_p]),
     "qllm_attention_paged_q4h_batched": (c_int32, [POINTER(Q4hAttentionLaunch), c_uint32]),
     "qllm_store_kv_paged_f16_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),

@@ -325,3 +325,70 @@ def test_prepared_query_operands_give_the_same_attention(device, tokens, rows, Q
         return out.cpu().numpy()
 
     assert np.array_equal(attend(True), attend(False))
+
+
+@pytest.mark.parametrize("tokens,rows,Q,KV,d,page,gated,qk_norm,rotary,splits", [
+    (1000, 5, 64, 8, 128, 256, False, False, 128, 32),
+    (5, 5, 8, 2, 128, 64, False, True, 128, 32),       # the batch is the whole context
+    (66, 5, 16, 2, 128, 64, True, True, 64, 32),       # batch across a tile and page edge
+    (258, 4, 24, 4, 256, 256, True, True, 64, 32),     # reference geometry, page edge
+    (4100, 1, 64, 8, 128, 256, False, False, 128, 32),
+    (20000, 5, 64, 8, 128, 256, False, True, 128, 32),
+    (700, 6, 8, 8, 128, 64, False, False, 128, 4)])    # one query head per KV head
+def test_fused_rotary_attention_equals_the_two_launches(device, tokens, rows, Q, KV, d, page,
+                                                        gated, qk_norm, rotary, splits):
+    """qllm_attention_paged_q4h_fused (rotary, K/V store and attention in one
+    launch, cos/sin from qllm_rope_table) against the rotary kernel followed by
+    the attention kernel: same output bits, same page bytes."""
+    rng = np.random.default_rng(tokens + rows + Q)
+    first = tokens - (rows - 1)
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, page, 2, 1)
+    stride = d * (2 if gated else 1)
+    q = rng.standard_normal((rows, Q, stride)).astype(np.float32)
+    k = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    v = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    qw = (0.1 * rng.standard_normal(d)).astype(np.float32) if qk_norm else None
+    kw = (0.1 * rng.standard_normal(d)).astype(np.float32) if qk_norm else None
+    d_qw = None if qw is None else gu.device_tensor(qw, device)
+    d_kw = None if kw is None else gu.device_tensor(kw, device)
+    group = Q // KV
+    row_tiles = (rows * group + 15) // 16
+    results = []
+    for fused in (False, True):
+        d_pages = [gu.device_tensor(p, device) for p in pages]
+        table = torch.tensor([p.data_ptr() for p in d_pages], dtype=torch.int64,
+                             device=device)
+        d_q, d_k, d_v = (gu.device_tensor(x, device) for x in (q, k, v))
+        maxima = torch.zeros((rows, splits, Q), device=device)
+        sums = torch.zeros_like(maxima)
+        outputs = torch.zeros((rows, splits, Q, d), device=device)
+        out = torch.zeros((rows, Q, d), device=device)
+        operands = torch.zeros(KV * row_tiles * (d // 64) * 2048, dtype=torch.uint8,
+                               device=device)
+        scales = torch.zeros(KV * row_tiles * 16, dtype=torch.float32, device=device)
+        launch = qh.Q4hAttentionLaunch(
+            qh.ptr(d_q), 0 if fused else qh.ptr(operands), 0 if fused else qh.ptr(scales),
+            qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums), qh.ptr(outputs),
+            first, rows, 1, page, Q, KV, d, 0, splits, stride, int(gated), qh.OUT_F32, None)
+        if fused:
+            cos_sin = torch.zeros((rows, rotary // 2, 2), device=device)
+            qh.call("qllm_rope_table", qh.ptr(cos_sin), rows, rotary, first - 1, 1e6, 0,
+                    None, None)
+            rope = qh.Q4hFusedRope(qh.ptr(d_k), qh.ptr(d_v), qh.ptr(d_qw), qh.ptr(d_kw),
+                                   qh.ptr(cos_sin), rotary, 1e-6, first - 1, 0)
+            qh.call("qllm_attention_paged_q4h_fused", launch, rope)
+        else:
+            qh.call("qllm_qkv_rope_cache_paged_q4h_prepared", None, 0, qh.ptr(d_q), stride,
+                    qh.ptr(d_k), qh.ptr(d_v), qh.ptr(d_qw), qh.ptr(d_kw), qh.ptr(table), 1,
+                    page, first - 1, first - 1, None, rows, Q, KV, d, rotary, 1e-6, 1e6, 0,
+                    qh.ptr(operands), qh.ptr(scales), None)
+            qh.call("qllm_attention_paged_q4h", launch)
+        torch.cuda.synchronize()
+        results.append((out.cpu().numpy(), [p.cpu().numpy() for p in d_pages]))
+    (plain, plain_pages), (fused, fused_pages) = results
+    assert np.array_equal(plain, fused)
+    for index, (a, b) in enumerate(zip(plain_pages, fused_pages)):
+        assert np.array_equal(a, b), index
+    assert not np.array_equal(plain_pages[-1], pages[-1])   # the batch was stored
