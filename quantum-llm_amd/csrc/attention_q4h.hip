@@ -656,10 +656,28 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     // the rows, so their instruction streams interleave.
     const bool has_q_weight = args.q_weight != nullptr;
     const bool bf16_rounding = args.bf16_activations != 0u;
+    // The wave's last row is past the batch in the usual shapes (40 matrix rows
+    // in 48 slots): it alone sits behind a branch, which leaves it out then.
+    const bool last_item_live =
+        wave + kSplitWaves * (ROWS_PER_WAVE - 1) < matrix_rows;
     const auto quantise_rows = [&](auto rotate) {
 #pragma unroll
       for (int item = 0; item < ROWS_PER_WAVE; ++item) {
         const uint32_t matrix_row = wave + kSplitWaves * item;
+        if (item == ROWS_PER_WAVE - 1 && !last_item_live) {
+          if (lane < KSTEPS * 2u * 4u)
+            *reinterpret_cast<uint4*>(
+                exchange + ((matrix_row / 16u) * KSTEPS * 2u + lane / 4u) * 1024u +
+                (16u * (lane % 4u) + matrix_row % 16u) * 16u) =
+                make_uint4(0u, 0u, 0u, 0u);
+          if (lane == 0u) {
+            exchange_scale[matrix_row] =
+                0x1p-100f *
+                (1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D))));
+            exchange_limit[matrix_row] = first_context_tokens;
+          }
+          continue;
+        }
         const uint32_t row_tile = matrix_row / 16u;
         const uint32_t column = matrix_row % 16u;
         const bool valid = matrix_row < matrix_rows;
@@ -930,26 +948,39 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
     // ---- K codes and scales out of LDS ----------------------------------------
     vmem_wait<V_LOADS>();
-    // the batch's own tokens inside this tile, [batch_first, batch_last)
-    uint32_t batch_first = 0u, batch_last = 0u;
     if constexpr (FUSED) {
-      batch_first = max(first_cache_position, tile_begin);
-      batch_last = min(first_cache_position + args.rows, tile_begin + 64u);
+      // the batch's own tokens inside this tile, [batch_first, batch_last):
+      // their fresh records go over whatever the pages held, once the whole
+      // tile has landed (a tile or two per launch pay this wait)
+      const uint32_t batch_first = max(first_cache_position, tile_begin);
+      const uint32_t batch_last =
+          min(first_cache_position + args.rows, tile_begin + 64u);
       if (batch_first < batch_last) {
-        // their fresh K records go over whatever the pages held
+        vmem_wait<0>();
+        const uint32_t lane_now = fresh_lane_index();
+        uint8_t* stage_v = stage_k + CODES + 256;
         const uint32_t count = batch_last - batch_first;
-        for (uint32_t piece = lane; piece < count * kParts; piece += 64u) {
+#pragma clang loop vectorize(disable) unroll(disable)
+        for (uint32_t piece = lane_now; piece < count * kParts; piece += 64u) {
           const uint32_t token = batch_first + piece / kParts;
           const uint32_t part = piece % kParts;
-          *reinterpret_cast<uint4*>(stage_k + (token - tile_begin) * ROW + part * 16u) =
-              *reinterpret_cast<const uint4*>(
-                  fresh + (token - first_cache_position) * RECORD + part * 16u);
+          const uint32_t t = token - tile_begin;
+          const uint8_t* record = fresh + (token - first_cache_position) * RECORD;
+          *reinterpret_cast<uint4*>(stage_k + t * ROW + part * 16u) =
+              *reinterpret_cast<const uint4*>(record + part * 16u);
+          // LDS row of token t in the V area: see stage_values
+          const uint32_t lds_row = 16u * ((t >> 2) & 3u) + 4u * (t >> 4) + (t & 3u);
+          *reinterpret_cast<uint4*>(stage_v + lds_row * ROW + part * 16u) =
+              *reinterpret_cast<const uint4*>(record + ROW + part * 16u);
         }
-        for (uint32_t index = lane; index < count; index += 64u) {
+#pragma clang loop vectorize(disable) unroll(disable)
+        for (uint32_t index = lane_now; index < count; index += 64u) {
           const uint32_t token = batch_first + index;
+          const uint8_t* record = fresh + (token - first_cache_position) * RECORD;
           *reinterpret_cast<uint16_t*>(stage_k + CODES + 2u * (token - tile_begin)) =
-              *reinterpret_cast<const uint16_t*>(
-                  fresh + (token - first_cache_position) * RECORD + D);
+              *reinterpret_cast<const uint16_t*>(record + D);
+          *reinterpret_cast<uint16_t*>(stage_v + CODES + 2u * (token - tile_begin)) =
+              *reinterpret_cast<const uint16_t*>(record + D + 2);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       }
@@ -1054,30 +1085,6 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
           vmem_wait<KS_LOADS>();
         else
           vmem_wait<0>();
-        if constexpr (FUSED) {
-          if (batch_first < batch_last) {
-            // and their fresh V records (LDS row of token t: see stage_values)
-            uint8_t* stage_v = stage_k + CODES + 256;
-            const uint32_t count = batch_last - batch_first;
-            for (uint32_t piece = lane; piece < count * kParts; piece += 64u) {
-              const uint32_t token = batch_first + piece / kParts;
-              const uint32_t part = piece % kParts;
-              const uint32_t t = token - tile_begin;
-              const uint32_t lds_row = 16u * ((t >> 2) & 3u) + 4u * (t >> 4) + (t & 3u);
-              *reinterpret_cast<uint4*>(stage_v + lds_row * ROW + part * 16u) =
-                  *reinterpret_cast<const uint4*>(
-                      fresh + (token - first_cache_position) * RECORD + ROW +
-                      part * 16u);
-            }
-            for (uint32_t index = lane; index < count; index += 64u) {
-              const uint32_t token = batch_first + index;
-              *reinterpret_cast<uint16_t*>(stage_v + CODES + 2u * (token - tile_begin)) =
-                  *reinterpret_cast<const uint16_t*>(
-                      fresh + (token - first_cache_position) * RECORD + D + 2);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          }
-        }
         u32x2 value_scale_raw[4];
         [&]<int... I>(std::integer_sequence<int, I...>) {
           ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
