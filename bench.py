@@ -388,6 +388,11 @@ def main():
         other_kernels[name] = {"avg_launch_us": round(us, 3),
                                "achieved_GBps": round(bytes_per_launch / us / 1e3, 1),
                                "frac": round(bytes_per_launch / us / 1e3 / HBM_PEAK_GBS, 4)}
+    other_kernels["attention"]["launches"] = (
+        "rotary + Q4H store + query quantisation + attention split in one launch, then "
+        "the split combine; the separate rotary launch it replaces took 5.2 us")
+    other_kernels["lm_head"]["weights"] = (
+        "cold: every timed launch follows > 640 MB of other weight reads")
 
     # the other contexts of the metric: the same step at 131072 tokens (Q4H) and
     # the exact-F16 attention kernel at 262144 tokens, on providers of their own
