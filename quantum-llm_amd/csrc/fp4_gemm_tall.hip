@@ -27,6 +27,8 @@
 //    twice the matrix instructions.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace qllm {
 namespace {
 
@@ -119,26 +121,30 @@ struct Operand<kSchemeF16> {
   static constexpr int kParts = 2;
   // `scale_bits` = the block's binary16 scale; out[0] = hi, out[1] = lo with
   // hi + lo = weight x scale exactly
+  // An E2M1 weight is (1 or 1.5) x a power of two: w = a + b with a = its leading
+  // power of two (the binary16 value with the mantissa cleared) and b = w - a,
+  // zero or half of a.  a x scale and b x scale are then both exact in binary16
+  // (a scale's 11 bits times a power of two), so hi = a x scale, lo = b x scale
+  // need five packed instructions per pair of weights.
   static __device__ __forceinline__ void weights(uint32_t packed, float,
                                                  uint32_t scale_bits,
                                                  Vector (&out)[2]) {
-    const float scale = f16_bits_to_f32(scale_bits);
+    const f16x2 scale =
+        __builtin_bit_cast(f16x2, scale_bits | (scale_bits << 16));
     Vector hi, lo;
 #pragma unroll
     for (int pair = 0; pair < 4; ++pair) {
-      f32x2 w;
+      f16x2 w;
       switch (pair) {
-        case 0: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(packed, 1.0f, 0); break;
-        case 1: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(packed, 1.0f, 1); break;
-        case 2: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(packed, 1.0f, 2); break;
-        default: w = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(packed, 1.0f, 3); break;
+        case 0: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 0); break;
+        case 1: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 1); break;
+        case 2: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2); break;
+        default: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3); break;
       }
-      const float p0 = w[0] * scale;   // exact: at most 13 significant bits
-      const float p1 = w[1] * scale;
-      const f16x2 top = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(p0, p1));
-      const float r0 = p0 - static_cast<float>(top[0]);
-      const float r1 = p1 - static_cast<float>(top[1]);
-      const f16x2 rest = __builtin_bit_cast(f16x2, __builtin_amdgcn_cvt_pkrtz(r0, r1));
+      const f16x2 leading = __builtin_bit_cast(
+          f16x2, __builtin_bit_cast(uint32_t, w) & 0xfc00fc00u);
+      const f16x2 top = leading * scale;
+      const f16x2 rest = (w - leading) * scale;
       hi[2 * pair] = top[0]; hi[2 * pair + 1] = top[1];
       lo[2 * pair] = rest[0]; lo[2 * pair + 1] = rest[1];
     }
@@ -235,9 +241,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
       *reinterpret_cast<uint4*>(&tile[buffer][stage_target + piece * 16u]) = v;
     }
   };
+  // (slot indices are compile-time constants throughout: an array indexed by a
+  // run-time slot would live in scratch memory, and every reload from there
+  // would wait for the prefetch that was just issued)
   uint4 codes[2][kTilesPerWave];
   uint2 scales[2][kTilesPerWave];
-  const auto fetch_weights = [&](uint32_t slot, uint32_t chunk) {
+  const auto fetch_weights = [&]<int slot>(std::integral_constant<int, slot>,
+                                           uint32_t chunk) {
 #pragma unroll
     for (uint32_t t = 0; t < kTilesPerWave; ++t) {
       codes[slot][t] = *reinterpret_cast<const uint4*>(
@@ -254,15 +264,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
   };
 
   fetch_activations(0u);
-  fetch_weights(0u, 0u);
+  fetch_weights(std::integral_constant<int, 0>{}, 0u);
   store_activations(0u);
 
-  for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-    const uint32_t slot = chunk & 1u;
+  const auto step = [&]<int slot>(std::integral_constant<int, slot>,
+                                  uint32_t chunk) {
     __syncthreads();   // tile[slot] is complete; tile[slot ^ 1] is free
     const uint32_t next = chunk + 1u < chunks ? chunk + 1u : chunk;
     fetch_activations(next);
-    fetch_weights(slot ^ 1u, next);
+    fetch_weights(std::integral_constant<int, slot ^ 1>{}, next);
 
     const uint8_t* current = tile[slot];
 #pragma unroll
@@ -296,6 +306,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
       }
     }
     if (chunk + 1u < chunks) store_activations(slot ^ 1u);
+  };
+  for (uint32_t chunk = 0; chunk < chunks; chunk += 2u) {
+    step(std::integral_constant<int, 0>{}, chunk);
+    if (chunk + 1u < chunks) step(std::integral_constant<int, 1>{}, chunk + 1u);
   }
 
   // D register i of lane (n, g): activation row 16 mt + 4 g + i, weight row
