@@ -1327,6 +1327,18 @@ void Mi355DenseFp4Provider::enqueue_attention(
   }
 }
 
+// Context splits of a batched (prompt) attention launch.  Every workgroup pays
+// a prologue and a merge of its eight wave states whatever its share of the
+// context, so the context is cut only as far as it takes to give every CU a
+// workgroup: a full chunk's row batches need no cut at all (a 32768-token
+// prompt: 5.50 s with eight splits, 5.09 / 4.91 / 4.79 s with four / two / one).
+std::uint32_t Mi355DenseFp4Provider::prefill_splits_for(
+    std::uint32_t rows, std::uint32_t attention_batch) const noexcept {
+  const std::uint32_t batches = (rows + attention_batch - 1U) / attention_batch;
+  const std::uint32_t workgroups = std::max(1U, batches * g_.kv_heads);
+  return std::clamp((256U + workgroups - 1U) / workgroups, 1U, prefill_splits_);
+}
+
 // (cos, sin) of the rotary angles of a batch at first_position .. + rows - 1
 // (or at the device-side positions), for the attention launches of a pass.
 void Mi355DenseFp4Provider::enqueue_rope_table(std::uint32_t rows,
@@ -1532,7 +1544,7 @@ void Mi355DenseFp4Provider::enqueue_mtp_prefill(
   launch.kv_heads = g_.kv_heads;
   launch.head_dim = g_.head_dim;
   launch.split_tokens = 0U;
-  launch.maximum_splits = prefill_splits_;
+  launch.maximum_splits = prefill_splits_for(rows, attention_batch);
   launch.query_stride = query_stride;
   launch.output_gated = g_.output_gated;
   launch.output_kind = QLLM_OUT_BF16;
@@ -1704,7 +1716,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.kv_heads = g_.kv_heads;
           launch.head_dim = g_.head_dim;
           launch.split_tokens = 0U;
-          launch.maximum_splits = prefill_splits_;
+          launch.maximum_splits = prefill_splits_for(rows, attention_batch);
           launch.query_stride = query_stride;
           launch.output_gated = g_.output_gated;
           launch.output_kind = QLLM_OUT_BF16;
@@ -1737,7 +1749,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.kv_heads = g_.kv_heads;
           launch.head_dim = g_.head_dim;
           launch.split_tokens = 0U;
-          launch.maximum_splits = prefill_splits_;
+          launch.maximum_splits = prefill_splits_for(rows, attention_batch);
           launch.query_stride = query_stride;
           launch.output_gated = g_.output_gated;
           launch.output_kind = QLLM_OUT_BF16;

@@ -265,6 +265,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                    const std::uint16_t* input,
                                    std::size_t input_bytes, std::uint32_t rows,
                                    bool leave_partials);
+  [[nodiscard]] std::uint32_t prefill_splits_for(
+      std::uint32_t rows, std::uint32_t attention_batch) const noexcept;
   void enqueue_rope_table(std::uint32_t rows, std::uint32_t first_position,
                           bool deferred_positions);
   void enqueue_attention_block(std::uint32_t index, std::uint32_t rows,
