@@ -204,6 +204,17 @@ int32_t qllm_fp4_gemm_bf16_tall(const qllm_fp4_matrix* matrix, const void* input
                                 size_t input_bytes, void* output,
                                 uint32_t output_kind, const float* residual,
                                 uint32_t batch, void* stream);
+/* The tall GEMM on the gate and the up matrix of a SwiGLU block at once (same
+ * shape, scheme and tiled layout): output bf16 [batch, rows] =
+ * bf16(bf16(silu(gate . x)) * (up . x)), the rounding points of
+ * qllm_silu_product with bf16 activations.  The tall counterpart of
+ * qllm_fp4_swiglu_bf16; the reference runs two GEMMs and swiglu_kernel
+ * (runtime/tools/dense_fp4_provider.cpp:8250-8293). */
+int32_t qllm_fp4_swiglu_bf16_tall(const qllm_fp4_matrix* gate,
+                                  const qllm_fp4_matrix* up, const void* input,
+                                  size_t input_bytes, void* output_bf16,
+                                  uint32_t batch, void* stream);
+
 /* The same with the output columns split over up to three buffers, each a
  * multiple of 32 weight rows (the q, k and v projections stored as one
  * matrix). */

@@ -52,6 +52,10 @@ typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 struct TallArgs {
   const uint8_t* weights;        // streaming layout, 32-row tiles
   const uint8_t* scales;
+  // SWIGLU form: `weights` / `scales` are the gate matrix, these the up matrix
+  // of the same shape; output = bf16(bf16(silu(gate . x)) * (up . x))
+  const uint8_t* up_weights;
+  const uint8_t* up_scales;
   const uint16_t* activations;   // bf16 [batch, padded_columns]
   uint32_t rows;                 // weight rows = output columns
   uint32_t padded_columns;
@@ -163,7 +167,12 @@ struct Operand<kSchemeF16> {
 // [256 n_tile, +256).  Workgroups that share weights (same n_tile) are given
 // consecutive positions within one XCD's share of the grid, so that the tile's
 // weights are fetched from HBM once per XCD rather than once per workgroup.
-template <int SCHEME>
+//
+// SWIGLU: a wave's two tiles are the same 32 rows of the gate and of the up
+// matrix (a workgroup covers 128 rows of each), and the epilogue writes
+// silu(gate) * up in bf16 with the rounding points of the separate
+// SiLU-product launch - no F32 round trip of the two projections.
+template <int SCHEME, bool SWIGLU = false>
 __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
     const TallArgs args) {
   using Op = Operand<SCHEME>;
@@ -193,12 +202,14 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
   uint32_t tile_index[kTilesPerWave];
 #pragma unroll
   for (uint32_t t = 0; t < kTilesPerWave; ++t) {
-    tile_index[t] = n_tile * kTilesN + wave * kTilesPerWave + t;
+    tile_index[t] = SWIGLU ? n_tile * kWaves + wave
+                           : n_tile * kTilesN + wave * kTilesPerWave + t;
     const size_t stream = min(tile_index[t], tile_count - 1u);
-    weight_stream[t] = args.weights + stream * chunks * (kTileRows * 32u) +
-                       (g * 16u + n) * 16u;
+    weight_stream[t] = (SWIGLU && t ? args.up_weights : args.weights) +
+                       stream * chunks * (kTileRows * 32u) + (g * 16u + n) * 16u;
     scale_stream[t] =
-        args.scales + stream * chunks * (kTileRows * (F16 ? 8u : 2u)) +
+        (SWIGLU && t ? args.up_scales : args.scales) +
+        stream * chunks * (kTileRows * (F16 ? 8u : 2u)) +
         (F16 ? ((g >> 1) * 16u + n) * 8u : n * 4u);
   }
 
@@ -314,6 +325,27 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
 
   // D register i of lane (n, g): activation row 16 mt + 4 g + i, weight row
   // 32 tile + 16 j + n
+  if constexpr (SWIGLU) {
+    if (tile_index[0] >= tile_count) return;
+#pragma unroll
+    for (uint32_t j = 0; j < 2u; ++j) {
+      const uint32_t column = tile_index[0] * kTileRows + 16u * j + n;
+      if (column >= args.rows) continue;
+#pragma unroll
+      for (uint32_t mt = 0; mt < kTilesM; ++mt)
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) {
+          const uint32_t row = first_m + 16u * mt + 4u * g + i;
+          if (row >= args.batch) continue;
+          const float gate = acc[mt][0][j][i];
+          const float activated = bf16_round(gate / (1.0f + expf(-gate)));
+          static_cast<uint16_t*>(args.output)[static_cast<size_t>(row) * args.rows +
+                                              column] =
+              static_cast<uint16_t>(f32_to_bf16_bits(activated * acc[mt][1][j][i]));
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (uint32_t t = 0; t < kTilesPerWave; ++t) {
     if (tile_index[t] >= tile_count) continue;
@@ -366,9 +398,15 @@ bool tall_matrix_ok(const qllm_fp4_matrix* m) {
 
 int32_t launch_tall(TallArgs args, uint32_t scheme, hipStream_t stream) {
   args.m_tiles = (args.batch + kRowsM - 1u) / kRowsM;
-  args.n_tiles = (args.rows + kTilesN * kTileRows - 1u) / (kTilesN * kTileRows);
+  const bool swiglu = args.up_weights != nullptr;
+  const uint32_t rows_per_workgroup = (swiglu ? kWaves : kTilesN) * kTileRows;
+  args.n_tiles = (args.rows + rows_per_workgroup - 1u) / rows_per_workgroup;
   const uint32_t grid = args.m_tiles * args.n_tiles;
-  if (scheme == QLLM_SCALE_F16_BLOCK16)
+  if (swiglu && scheme == QLLM_SCALE_F16_BLOCK16)
+    fp4_gemm_tall_kernel<kSchemeF16, true><<<grid, kWaves * 64, 0, stream>>>(args);
+  else if (swiglu)
+    fp4_gemm_tall_kernel<kSchemeUe8m0, true><<<grid, kWaves * 64, 0, stream>>>(args);
+  else if (scheme == QLLM_SCALE_F16_BLOCK16)
     fp4_gemm_tall_kernel<kSchemeF16><<<grid, kWaves * 64, 0, stream>>>(args);
   else
     fp4_gemm_tall_kernel<kSchemeUe8m0><<<grid, kWaves * 64, 0, stream>>>(args);
@@ -405,6 +443,32 @@ extern "C" int32_t qllm_fp4_gemm_bf16_tall(const qllm_fp4_matrix* matrix,
   args.output_kind = output_kind;
   args.residual = residual;
   return launch_tall(args, matrix->scale_scheme, as_stream(stream));
+}
+
+extern "C" int32_t qllm_fp4_swiglu_bf16_tall(const qllm_fp4_matrix* gate,
+                                             const qllm_fp4_matrix* up,
+                                             const void* input, size_t input_bytes,
+                                             void* output_bf16, uint32_t batch,
+                                             void* stream) {
+  if (!tall_matrix_ok(gate) || !tall_matrix_ok(up) || gate->rows != up->rows ||
+      gate->padded_columns != up->padded_columns ||
+      gate->scale_scheme != up->scale_scheme || !input || !output_bf16 ||
+      !batch || batch > (1u << 20) ||
+      (reinterpret_cast<uintptr_t>(input) & 15u) ||
+      input_bytes < static_cast<size_t>(batch) * gate->padded_columns * 2u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid tall FP4 SwiGLU");
+  TallArgs args{};
+  args.weights = gate->weights;
+  args.scales = static_cast<const uint8_t*>(gate->scales);
+  args.up_weights = up->weights;
+  args.up_scales = static_cast<const uint8_t*>(up->scales);
+  args.activations = static_cast<const uint16_t*>(input);
+  args.rows = gate->rows;
+  args.padded_columns = gate->padded_columns;
+  args.batch = batch;
+  args.output = output_bf16;
+  args.output_kind = QLLM_OUT_BF16;
+  return launch_tall(args, gate->scale_scheme, as_stream(stream));
 }
 
 extern "C" int32_t qllm_fp4_gemm_bf16_tall_split(

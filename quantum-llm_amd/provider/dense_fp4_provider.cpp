@@ -1493,7 +1493,7 @@ void Mi355DenseFp4Provider::enqueue_mtp_prefill(
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
   const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
-  float* const embedding = prefill_gate_;                 // f32 [rows, hidden]
+  float* const embedding = prefill_embedding_;            // f32 [rows, hidden]
   std::uint16_t* const fusion_input = prefill_activation_;  // bf16 [rows, 2 hidden]
   hip_check(hipMemcpyAsync(prefill_tokens_, tokens.data(), rows * 4U,
                            hipMemcpyHostToDevice, hip_stream),
@@ -1558,19 +1558,9 @@ void Mi355DenseFp4Provider::enqueue_mtp_prefill(
                                    nullptr, prefill_normalized_, g_.hidden, rows,
                                    g_.hidden, g_.norm_epsilon,
                                    g_.zero_centered_norm, stream));
-  status_check(qllm_fp4_gemm_bf16_tall(&layer.gate.descriptor,
-                                       prefill_normalized_, hidden_bytes,
-                                       prefill_gate_, QLLM_OUT_F32, nullptr, rows,
-                                       stream));
-  status_check(qllm_fp4_gemm_bf16_tall(&layer.up.descriptor, prefill_normalized_,
-                                       hidden_bytes, prefill_up_, QLLM_OUT_F32,
-                                       nullptr, rows, stream));
-  status_check(qllm_silu_product(prefill_gate_, prefill_up_, prefill_gate_,
-                                 rows * g_.intermediate, 1, stream));
-  status_check(qllm_convert_f32_to_bf16_batch(
-      prefill_gate_, prefill_activation_,
-      std::size_t{rows} * g_.intermediate * 2U, rows, g_.intermediate,
-      g_.intermediate, stream));
+  status_check(qllm_fp4_swiglu_bf16_tall(
+      &layer.gate.descriptor, &layer.up.descriptor, prefill_normalized_,
+      hidden_bytes, prefill_activation_, rows, stream));
   status_check(qllm_fp4_gemm_bf16_tall(
       &layer.down.descriptor, prefill_activation_,
       std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_, QLLM_OUT_F32,
@@ -1600,10 +1590,10 @@ void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
   prefill_value_ = static_cast<float*>(allocate(n * kv_width * 4U));
   prefill_attention_ = static_cast<std::uint16_t*>(
       allocate(n * g_.query_heads * g_.head_dim * 2U));
-  prefill_gate_ = static_cast<float*>(allocate(n * g_.intermediate * 4U));
-  prefill_up_ = static_cast<float*>(allocate(n * g_.intermediate * 4U));
-  prefill_activation_ =
-      static_cast<std::uint16_t*>(allocate(n * g_.intermediate * 2U));
+  prefill_embedding_ = static_cast<float*>(allocate(n * g_.hidden * 4U));
+  // the MLP's activation; the proposer's fusion input [rows, 2 hidden] too
+  prefill_activation_ = static_cast<std::uint16_t*>(allocate(
+      n * std::max<std::size_t>(g_.intermediate, 2U * g_.hidden) * 2U));
   {
     // fewer splits than the verify step: the row batches of a chunk already
     // fill the GPU, and the partials are per row
@@ -1764,20 +1754,11 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
             prefill_hidden_, layer.post_attention_norm, nullptr,
             prefill_normalized_, g_.hidden, rows, g_.hidden, g_.norm_epsilon,
             g_.zero_centered_norm, stream));
-        status_check(qllm_fp4_gemm_bf16_tall(
-            &layer.gate.descriptor, prefill_normalized_, hidden_bytes,
-            prefill_gate_, QLLM_OUT_F32, nullptr, rows, stream));
-        status_check(qllm_fp4_gemm_bf16_tall(
-            &layer.up.descriptor, prefill_normalized_, hidden_bytes, prefill_up_,
-            QLLM_OUT_F32, nullptr, rows, stream));
-        // silu(gate) * up with the verify step's bf16 rounding points; the
-        // result is exact in bf16, so the conversion moves bits only
-        status_check(qllm_silu_product(prefill_gate_, prefill_up_, prefill_gate_,
-                                       rows * g_.intermediate, 1, stream));
-        status_check(qllm_convert_f32_to_bf16_batch(
-            prefill_gate_, prefill_activation_,
-            std::size_t{rows} * g_.intermediate * 2U, rows, g_.intermediate,
-            g_.intermediate, stream));
+        // gate and up in one launch; silu(gate) * up leaves it in bf16 with
+        // the verify step's rounding points
+        status_check(qllm_fp4_swiglu_bf16_tall(
+            &layer.gate.descriptor, &layer.up.descriptor, prefill_normalized_,
+            hidden_bytes, prefill_activation_, rows, stream));
         status_check(qllm_fp4_gemm_bf16_tall(
             &layer.down.descriptor, prefill_activation_,
             std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_,

@@ -436,8 +436,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   float* prefill_key_{};
   float* prefill_value_{};
   std::uint16_t* prefill_attention_{};    // bf16 [rows, query_heads * head_dim]
-  float* prefill_gate_{};
-  float* prefill_up_{};
+  float* prefill_embedding_{};
   std::uint16_t* prefill_activation_{};   // bf16 [rows, intermediate]
   // split partials of the batched prompt attention: [rows, splits, heads(, d)]
   std::uint32_t prefill_splits_{};

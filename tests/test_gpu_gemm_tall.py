@@ -105,6 +105,40 @@ def test_tall_split_outputs(device):
                 bad, 2, batch, None)
 
 
+@pytest.mark.parametrize("rows,padded,batch", [(1024, 1024, 200), (300, 128, 77), (96, 64, 129)])
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+def test_tall_swiglu_equals_two_gemms_and_the_product(device, scheme, rows, padded, batch):
+    """One launch over the gate and the up matrix against two tall GEMMs and
+    the SiLU-product launch with bf16 rounding points: bit-equal, and against
+    the oracle's F64 projections within bf16 rounding."""
+    rng = np.random.default_rng(rows + padded + batch)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    matrices, keep, f32, f64 = [], [], [], []
+    for _ in range(2):
+        codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+        tensors = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+        matrix, packed = qh.prepack(qh.fp4_matrix(*tensors, rows, padded, padded, scheme), device)
+        out = torch.zeros((batch, rows), device=device)
+        qh.call("qllm_fp4_gemm_bf16_tall", matrix, qh.ptr(d_act), d_act.numel() * 2,
+                qh.ptr(out), qh.OUT_F32, None, batch, None)
+        matrices.append(matrix); keep.append((tensors, packed)); f32.append(out)
+        f64.append(ol.fp4_linear_f64(codes, scales, scheme, rows, padded, act))
+    qh.call("qllm_silu_product", qh.ptr(f32[0]), qh.ptr(f32[1]), qh.ptr(f32[0]),
+            batch * rows, 1, None)
+    fused = torch.zeros((batch, rows), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_fp4_swiglu_bf16_tall", matrices[0], matrices[1], qh.ptr(d_act),
+            d_act.numel() * 2, qh.ptr(fused), batch, None)
+    torch.cuda.synchronize()
+    got = fused.float().cpu().numpy()
+    assert np.array_equal(got, f32[0].cpu().numpy())
+    want = f64[0] / (1.0 + np.exp(np.minimum(-f64[0], 700.0))) * f64[1]
+    gu.assert_close(got, want, rtol=2e-2, atol=2e-2 * np.abs(want).max(), what="tall SwiGLU")
+    with pytest.raises(qh.QllmError, match="invalid tall FP4 SwiGLU"):
+        qh.call("qllm_fp4_swiglu_bf16_tall", matrices[0], None, qh.ptr(d_act),
+                d_act.numel() * 2, qh.ptr(fused), batch, None)
+
+
 def test_tall_gemm_rejects_row_major(device):
     rng = np.random.default_rng(1)
     codes, scales = synth.fp4_matrix(rng, 64, 64, 0)
