@@ -53,6 +53,10 @@ typedef struct qllm_dense_geometry {
   /* Head rows the proposer scores (project_prefix :6280-6308); 0 =
    * min(vocabulary, 65536). */
   uint32_t draft_vocabulary;
+  /* Rows of a prompt that go through the tall linears at a time
+   * (qllm_provider_prefill); 0 = 4096.  The reference's prompt path runs
+   * prefill_chunk_tokens rows per program step (moe_vm_runner.cpp:682-745). */
+  uint32_t prefill_chunk_rows;
 } qllm_dense_geometry;
 
 const char* qllm_provider_last_error(void);

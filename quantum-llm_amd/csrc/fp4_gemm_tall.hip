@@ -42,6 +42,7 @@ constexpr uint32_t kWaves = 4;
 constexpr uint32_t kTilesPerWave = 2;    // 32-row weight tiles per wave
 constexpr uint32_t kTilesN = kWaves * kTilesPerWave;   // per workgroup
 constexpr uint32_t kTileRows = 32;
+constexpr uint32_t kBand = 8;            // activation tiles per band of the grid
 // LDS row of the activation tile: 64 values of 16 bits plus 16 bytes, so that
 // the sixteen rows a fragment load touches fall on different banks
 constexpr uint32_t kLdsRow = kChunk * 2u + 16u;
@@ -125,11 +126,9 @@ struct Operand<kSchemeF16> {
   static constexpr int kParts = 2;
   // `scale_bits` = the block's binary16 scale; out[0] = hi, out[1] = lo with
   // hi + lo = weight x scale exactly
-  // An E2M1 weight is (1 or 1.5) x a power of two: w = a + b with a = its leading
-  // power of two (the binary16 value with the mantissa cleared) and b = w - a,
-  // zero or half of a.  a x scale and b x scale are then both exact in binary16
-  // (a scale's 11 bits times a power of two), so hi = a x scale, lo = b x scale
-  // need five packed instructions per pair of weights.
+  // hi = the product rounded to binary16, lo = the rounding error, which a
+  // fused multiply-add returns exactly (it has at most two significant bits):
+  // three packed instructions per pair of weights.
   static __device__ __forceinline__ void weights(uint32_t packed, float,
                                                  uint32_t scale_bits,
                                                  Vector (&out)[2]) {
@@ -145,10 +144,8 @@ struct Operand<kSchemeF16> {
         case 2: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 2); break;
         default: w = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(packed, 1.0f, 3); break;
       }
-      const f16x2 leading = __builtin_bit_cast(
-          f16x2, __builtin_bit_cast(uint32_t, w) & 0xfc00fc00u);
-      const f16x2 top = leading * scale;
-      const f16x2 rest = (w - leading) * scale;
+      const f16x2 top = w * scale;
+      const f16x2 rest = __builtin_elementwise_fma(w, scale, -top);
       hi[2 * pair] = top[0]; hi[2 * pair + 1] = top[1];
       lo[2 * pair] = rest[0]; lo[2 * pair + 1] = rest[1];
     }
@@ -164,9 +161,7 @@ struct Operand<kSchemeF16> {
 };
 
 // Workgroup (m_tile, n_tile): activation rows [128 m_tile, +128), weight rows
-// [256 n_tile, +256).  Workgroups that share weights (same n_tile) are given
-// consecutive positions within one XCD's share of the grid, so that the tile's
-// weights are fetched from HBM once per XCD rather than once per workgroup.
+// [256 n_tile, +256).
 //
 // SWIGLU: a wave's two tiles are the same 32 rows of the gate and of the up
 // matrix (a workgroup covers 128 rows of each), and the epilogue writes
@@ -187,11 +182,21 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
   const uint32_t K = args.padded_columns;
   const uint32_t chunks = K / kChunk;
 
+  // Workgroups are dealt to the eight XCDs in turn, so XCD x runs the ids
+  // x, x + 8, ...: give it a contiguous range of tiles instead.  Within the
+  // range the tiles go band by band (kBand activation tiles high), column by
+  // column: the 64 workgroups an XCD runs at a time then cover about 8 x 8
+  // tiles and fetch 8 + 8 operand tiles per K step into its L2 rather than
+  // 64 + 1.
   const uint32_t total = args.m_tiles * args.n_tiles;
-  uint32_t id = blockIdx.x;
-  if (total % 8u == 0u) id = (blockIdx.x % 8u) * (total / 8u) + blockIdx.x / 8u;
-  const uint32_t m_tile = id % args.m_tiles;
-  const uint32_t n_tile = id / args.m_tiles;
+  const uint32_t xcd = blockIdx.x % 8u;
+  const uint32_t id = xcd * (total / 8u) + min(xcd, total % 8u) + blockIdx.x / 8u;
+  const uint32_t band_tiles = kBand * args.n_tiles;
+  const uint32_t band = id / band_tiles;
+  const uint32_t in_band = id - band * band_tiles;
+  const uint32_t height = min(kBand, args.m_tiles - band * kBand);
+  const uint32_t m_tile = band * kBand + in_band % height;
+  const uint32_t n_tile = in_band / height;
   const uint32_t first_m = m_tile * kRowsM;
 
   // weight streams of this wave's tiles (tiles past the matrix repeat the last
@@ -213,7 +218,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
         (F16 ? ((g >> 1) * 16u + n) * 8u : n * 4u);
   }
 
-  // activation tile: thread -> (row, half of the 64 columns), 64 bytes
+  // activation tile: thread -> (row, half of the 64 columns), 64 bytes.  Rows
+  // past the batch stage row 0 again: their results are never stored, and a
+  // load under a branch would make every wait for the weights conservative.
   const uint32_t stage_row = threadIdx.x >> 1;
   const uint32_t stage_half = threadIdx.x & 1u;
   const bool stage_live = first_m + stage_row < args.batch;
@@ -237,11 +244,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
   const auto fetch_activations = [&](uint32_t chunk) {
 #pragma unroll
     for (uint32_t piece = 0; piece < 4u; ++piece)
-      staged[piece] = stage_live
-                          ? *reinterpret_cast<const uint4*>(
-                                stage_source + static_cast<size_t>(chunk) * 128u +
-                                piece * 16u)
-                          : make_uint4(0u, 0u, 0u, 0u);
+      staged[piece] = *reinterpret_cast<const uint4*>(
+          stage_source + static_cast<size_t>(chunk) * 128u + piece * 16u);
   };
   const auto store_activations = [&](uint32_t buffer) {
 #pragma unroll
@@ -284,6 +288,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void fp4_gemm_tall_kernel(
     const uint32_t next = chunk + 1u < chunks ? chunk + 1u : chunk;
     fetch_activations(next);
     fetch_weights(std::integral_constant<int, slot ^ 1>{}, next);
+    // the loads stay here, a whole step ahead of their use (left alone, the
+    // scheduler sinks them to the end of the step to shorten live ranges)
+    __builtin_amdgcn_sched_barrier(0);
 
     const uint8_t* current = tile[slot];
 #pragma unroll

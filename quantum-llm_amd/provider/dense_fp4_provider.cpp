@@ -1629,8 +1629,9 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
                  "prompt token is outside the vocabulary"},
                 0U};
     const auto count = static_cast<std::uint32_t>(tokens.size());
-    const std::uint32_t chunk_rows = std::min(count, prefill_chunk_rows());
-    ensure_prefill_workspace(prefill_rows_ ? prefill_rows_ : chunk_rows);
+    // sized for a whole chunk whatever the first prompt's length: the
+    // workspace does not grow
+    ensure_prefill_workspace(std::min(prefill_chunk_rows(), g_.max_context));
     ensure_pages(first_position + count - 1U);
     void* const stream = stream_;
     const auto hip_stream = static_cast<hipStream_t>(stream_);
@@ -1775,7 +1776,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
       // position but the last, whose successor is not known yet
       if (feed_proposer) {
         const std::uint32_t pairs = done + rows == count ? rows - 1U : rows;
-        const bool tall = g_.hidden <= 16384U && g_.intermediate >= 2U * g_.hidden &&
+        const bool tall = g_.hidden <= 16384U &&
                           mtp_.fusion.descriptor.layout == QLLM_LAYOUT_TILED;
         if (pairs && tall) {
           enqueue_mtp_prefill(tokens.subspan(done + 1U, pairs), position,

@@ -28,7 +28,8 @@ class DenseGeometry(Structure):
                 ("zero_centered_norm", c_int32), ("scale_scheme", c_uint32),
                 ("kv_encoding", c_uint32), ("kv_page_tokens", c_uint32),
                 ("max_context", c_uint32), ("draft_depth", c_uint32),
-                ("mtp_layers", c_uint32), ("draft_vocabulary", c_uint32)]
+                ("mtp_layers", c_uint32), ("draft_vocabulary", c_uint32),
+                ("prefill_chunk_rows", c_uint32)]
 
 
 SIGNATURES = {

@@ -245,7 +245,7 @@ def run_mtp(model: TinyModel, tokens, previous_hidden, mtp_length, q8_pages,
 
 
 def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
-                   kv_encoding=0, mtp=False, draft_vocabulary=0):
+                   kv_encoding=0, mtp=False, draft_vocabulary=0, prefill_chunk_rows=0):
     """Hands the host tensors to the provider operation by operation, the way
     the common VM calls prepare() in artifact order."""
     m = model
@@ -256,7 +256,8 @@ def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
         norm_epsilon=m.eps, output_gated=int(m.output_gated), qk_norm=int(m.qk_norm),
         zero_centered_norm=int(m.zero_centered), scale_scheme=m.scheme,
         kv_encoding=kv_encoding, kv_page_tokens=page_tokens, max_context=max_context,
-        draft_depth=4, mtp_layers=int(mtp), draft_vocabulary=draft_vocabulary)
+        draft_depth=4, mtp_layers=int(mtp), draft_vocabulary=draft_vocabulary,
+        prefill_chunk_rows=prefill_chunk_rows)
     abi = 16 if m.scheme == ol.SCALE_F16_BLOCK16 else 3
     tag = "fp4-f16-block16" if m.scheme == ol.SCALE_F16_BLOCK16 else "fp4-block32"
     d, Q, KV, H, I, V = m.head_dim, m.query_heads, m.kv_heads, m.hidden, m.intermediate, m.vocabulary

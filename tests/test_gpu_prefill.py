@@ -103,6 +103,37 @@ def test_prefill_feeds_the_proposer_and_decoding_continues(device, count):
     slow.close()
 
 
+@pytest.mark.parametrize("kv_encoding", [0, 1])
+def test_chunked_prefill_equals_one_pass(device, kv_encoding):
+    """A prompt cut into chunks of 64 and 17 rows (the last one ragged) against
+    the same prompt in one pass: the chunks see the earlier ones through the
+    cache only, so logits and hidden state agree within the end-to-end bound
+    and the proposer ends in the same state."""
+    rng, model, _ = make("reference", 77)
+    tokens = rng.integers(0, model.vocabulary, 150).astype(np.uint32)
+    results = []
+    for chunk_rows in (0, 64, 17):
+        provider = step_oracle.build_provider(
+            model, qp, mtp=True, draft_vocabulary=128, kv_encoding=kv_encoding,
+            max_context=512, prefill_chunk_rows=chunk_rows)
+        provider.begin_request(temperature_ppm=0)
+        predicted = provider.prefill(tokens, 2)
+        passes = provider.telemetry("provider_mtp_passes")
+        chunks = 1 if chunk_rows == 0 else -(-150 // chunk_rows)
+        assert passes == chunks + 4            # a tall pass per chunk, last pair, 3 rollouts
+        results.append((predicted, provider.logits(1)[0], provider.hidden(1)[0],
+                        provider.mtp_state(), provider.drafts()))
+        provider.close()
+    want = results[0]
+    for got in results[1:]:
+        assert (np.linalg.norm(got[1] - want[1]) / np.linalg.norm(want[1])) < 2e-2
+        assert np.abs(got[2] - want[2]).max() < 2e-2 * np.abs(want[2]).max()
+        assert got[0] == want[0] or (
+            want[1].max() - want[1][got[0]] < 1e-2 * np.abs(want[1]).max())
+        assert (np.linalg.norm(got[3][1] - want[3][1]) / np.linalg.norm(want[3][1])) < 3e-2
+        assert len(got[4]) == 4
+
+
 def test_prefill_rejects_bad_prompts(device):
     rng, model, build = make("baseline", 3, max_context=128)
     provider = build()
