@@ -1330,6 +1330,41 @@ __global__ void attention_combine_kernel(
     static_cast<float*>(output)[index] = result;
 }
 
+// The combine of a launch with a single split (the prompt's chunks): the
+// split's weight is one, so the result is its output over its sum - the same
+// operations as above, four dimensions per thread and no per-split loads.
+__global__ __launch_bounds__(256) void attention_single_split_kernel(
+    const float* query, uint32_t query_stride, int output_gated,
+    const float* partial_sums, const float* partial_outputs, void* output,
+    uint32_t output_kind, uint32_t head_dim, size_t elements) {
+  const size_t index =
+      (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4u;
+  if (index >= elements) return;
+  const size_t record = index / head_dim;
+  const uint32_t dimension = static_cast<uint32_t>(index - record * head_dim);
+  const float4 partial = *reinterpret_cast<const float4*>(partial_outputs + index);
+  const float sum = partial_sums[record];
+  float result[4] = {partial.x / sum, partial.y / sum, partial.z / sum,
+                     partial.w / sum};
+  if (output_gated) {
+    const float4 gate = *reinterpret_cast<const float4*>(
+        query + record * query_stride + head_dim + dimension);
+    result[0] *= 1.0f / (1.0f + expf(-gate.x));
+    result[1] *= 1.0f / (1.0f + expf(-gate.y));
+    result[2] *= 1.0f / (1.0f + expf(-gate.z));
+    result[3] *= 1.0f / (1.0f + expf(-gate.w));
+  }
+  if (output_kind == QLLM_OUT_BF16) {
+    uint2 packed;
+    packed.x = f32_to_bf16_bits(result[0]) | (f32_to_bf16_bits(result[1]) << 16);
+    packed.y = f32_to_bf16_bits(result[2]) | (f32_to_bf16_bits(result[3]) << 16);
+    *reinterpret_cast<uint2*>(static_cast<uint16_t*>(output) + index) = packed;
+  } else {
+    *reinterpret_cast<float4*>(static_cast<float*>(output) + index) =
+        make_float4(result[0], result[1], result[2], result[3]);
+  }
+}
+
 // ---- K/V store ----------------------------------------------------------------
 
 __global__ __launch_bounds__(64) void q4h_store_kernel(
@@ -1543,6 +1578,15 @@ int32_t launch_attention_combine(const float* query, uint32_t query_stride,
                                  uint32_t head_dim,
                                  const uint32_t* device_positions,
                                  hipStream_t stream) {
+  if (maximum_splits == 1u && !split_tokens && head_dim % 4u == 0u &&
+      query_stride % 4u == 0u && !(reinterpret_cast<uintptr_t>(query) & 15u)) {
+    const size_t elements = static_cast<size_t>(rows) * query_heads * head_dim;
+    attention_single_split_kernel<<<static_cast<unsigned>((elements / 4u + 255u) / 256u),
+                                    256, 0, stream>>>(
+        query, query_stride, output_gated, partial_sums, partial_outputs, output,
+        output_kind, head_dim, elements);
+    return launched("attention single-split combine");
+  }
   const dim3 grid(query_heads, rows);
   attention_combine_kernel<<<grid, head_dim, 0, stream>>>(
       query, query_stride, output_gated, partial_maxima, partial_sums,

@@ -175,13 +175,14 @@ def test_attention_rejects_unsupported_geometry(device):
     (40, 1, 8, 2, 256, True, 5),         # the prompt starts the cache; d = 256
     (64, 4000, 64, 8, 128, False, 6),    # six rows per batch (48 matrix rows)
     (7, 70, 16, 8, 128, False, 1)])      # one row per batch
+@pytest.mark.parametrize("splits", [8, 1])   # 1: the combine's single-split form
 def test_batched_launch_equals_one_launch_per_batch(device, total, first, Q, KV, d,
-                                                     gated, batch):
+                                                     gated, batch, splits):
     """Prompt prefill attends `total` consecutive rows in one launch, in
     batches of `batch` rows that each see the cache up to their own rows: bit
     for bit what one launch per batch computes, and the oracle's attention."""
     rng = np.random.default_rng(total + first)
-    page_tokens, splits = 64, 8
+    page_tokens = 64
     tokens = first + total - 1
     keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
     values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
