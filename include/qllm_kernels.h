@@ -498,6 +498,19 @@ int32_t qllm_rope_table(float* table, uint32_t rows, uint32_t rotary_dim,
 int32_t qllm_attention_paged_q4h_batched(const qllm_q4h_attention_launch* launch,
                                          uint32_t batch_rows);
 
+/* The same attention for a long run of prompt rows (head_dim 128,
+ * split_tokens 0): eight consecutive batches share a workgroup, which fetches
+ * every cache tile once for the eight and converts its V codes and scales to
+ * matrix-core operands once; every batch (one wave) walks the tiles of its
+ * own context in order, so sums differ from the batched launch's in the last
+ * bits (other order of F32 additions), the records read and the arithmetic per
+ * score are the same.  maximum_splits cuts the tiles of a workgroup's longest
+ * context evenly (1 when rows / (8 batch_rows) * kv_heads workgroups fill the
+ * GPU).  Replaces the reference's prefill attention
+ * (transformer_kernels.cu:9906-10153: 64-row query blocks per cache tile). */
+int32_t qllm_attention_paged_q4h_prompt(const qllm_q4h_attention_launch* launch,
+                                        uint32_t batch_rows);
+
 /* ---- attention: exact F16 paged cache ---------------------------------------- */
 
 /* Per-layer page layout: K [page_tokens][kv_heads][head_dim] then

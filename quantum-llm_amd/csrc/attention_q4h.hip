@@ -1223,6 +1223,473 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
                            target);
 }
 
+// ---- prompt attention: eight row batches share every cache tile -------------
+// A prompt chunk's row batches walk the same cache tiles, and the tile loop
+// above is bound by vector instructions, a good part of them the nibble ->
+// binary16 conversion of the tile's V codes and the scale handling.  Here a
+// workgroup's eight waves each own one row batch (48 matrix rows: quantised
+// queries, scores, softmax and accumulators as above), fetch every tile once
+// for all of them and convert its V side once: the V operands of a tile lie in
+// LDS in matrix-core order, the K scales as F32 and the V scales as the
+// binary16 pairs the probabilities are multiplied with, and every wave reads
+// them from there (the K codes stay raw: widening them is cheap, and LDS has
+// no room for a second copy next to eight batches' query operands).
+//
+// Per tile t the workgroup meets one barrier.  Between two barriers a wave
+//   1. sends its share of later tiles on their way, global -> LDS: waves 0..3
+//      a quarter each of the V codes of tile t + 2 (waves 0 and 1 also its K
+//      and V scales), waves 4..7 a quarter each of the K codes of tile t + 1,
+//   2. converts its share of tile t + 1: V row tile `wave` from the raw codes
+//      (read transposed), wave 6 the K scales, wave 7 the V scale pairs,
+//   3. runs its batch over tile t.
+// The tiles of the workgroup's longest context are dealt evenly over the grid's
+// splits; a batch stops at its own last tile.  Every wave writes its batch's
+// split partial itself - no states are merged.
+constexpr int kPromptBatches = 8;
+
+template <int D>
+__global__ __launch_bounds__(kPromptBatches * 64) void q4h_prompt_attention_kernel(
+    const SplitArgs args) {
+  static_assert(D == 128, "LDS holds eight batches' query operands at 128 only");
+  constexpr int RT = 3;
+  constexpr int KSTEPS = D / 64;
+  constexpr int DT = D / 16;
+  constexpr int ROW = D / 2;
+  constexpr int CODES = 64 * ROW;
+  constexpr int Q_BYTES = RT * KSTEPS * 2 * 1024;   // query operands of a batch
+  constexpr int RAW_V = CODES + 512;                // V codes | K scales | V scales
+  constexpr int CONV_V = DT * 2 * 1024;             // V operands of a tile
+  constexpr int CONV_KS = CONV_V;                   // K scales, F32 per token
+  constexpr int CONV_VS = CONV_KS + 256;            // V scale pairs
+  constexpr int CONV = CONV_VS + 128;
+  __shared__ __attribute__((aligned(16))) uint8_t q_operands_all[kPromptBatches * Q_BYTES];
+  __shared__ float q_scales[kPromptBatches * RT * 16];
+  __shared__ uint32_t q_limits[kPromptBatches * RT * 16];
+  __shared__ __attribute__((aligned(16))) uint8_t converted[2 * CONV];
+  __shared__ __attribute__((aligned(16))) uint8_t raw_values[2 * RAW_V];
+  __shared__ __attribute__((aligned(16))) uint8_t raw_keys[2 * CODES];
+
+  const uint32_t lane = threadIdx.x & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t col = lane & 15u;
+  const uint32_t quad = lane >> 4;
+  const uint32_t kv_head = blockIdx.x;
+  const uint32_t split = blockIdx.y;
+  const uint32_t splits = gridDim.y;
+  const uint32_t group = args.query_heads / args.kv_heads;
+
+  // this wave's batch
+  const uint32_t batches = (args.rows + args.batch_rows - 1u) / args.batch_rows;
+  const uint32_t first_batch = blockIdx.z * kPromptBatches;
+  const uint32_t batch = first_batch + wave;
+  const bool live = batch < batches;
+  const uint32_t first_row = live ? batch * args.batch_rows : 0u;
+  const uint32_t batch_rows = live ? min(args.batch_rows, args.rows - first_row) : 0u;
+  const uint32_t matrix_rows = batch_rows * group;
+  const uint32_t first_context_tokens = args.first_context_tokens + first_row;
+  const uint32_t batch_tiles =
+      live ? (first_context_tokens + batch_rows - 1u + 63u) / 64u : 0u;
+  // the workgroup's tiles: those of its last batch, cut by the grid's splits
+  const uint32_t last_batch = min(first_batch + kPromptBatches, batches) - 1u;
+  const uint32_t workgroup_context =
+      args.first_context_tokens +
+      min((last_batch + 1u) * args.batch_rows, args.rows) - 1u;
+  const uint32_t workgroup_tiles = (workgroup_context + 63u) / 64u;
+  const uint32_t quotient = workgroup_tiles / splits;
+  const uint32_t remainder = workgroup_tiles - quotient * splits;
+  const uint32_t tile_first = split * quotient + split * remainder / splits;
+  const uint32_t tile_last =
+      (split + 1u) * quotient + (split + 1u) * remainder / splits;
+  // records from here on were never written: their scales stay away from the
+  // matrix cores
+  const uint32_t launch_context = args.first_context_tokens + args.rows - 1u;
+
+  const uint32_t raw_values_lds =
+      __builtin_amdgcn_readfirstlane(lds_address(raw_values));
+  const uint32_t raw_keys_lds =
+      __builtin_amdgcn_readfirstlane(lds_address(raw_keys));
+  const uint32_t value_scale_distance =
+      args.page_tokens * args.kv_heads * (ROW + 2u);
+
+  // ---- a wave's share of fetching and converting a tile -----------------------
+  // waves 0..3: V codes, LDS rows 16 wave .. + 15 of the permuted tile (row R
+  // holds token 16 ((R / 4) % 4) + 4 (R / 16) + R % 4); waves 0 and 1 also the
+  // tile's K and V scales (lanes 0..31 fetch tokens 2l, 2l + 1; the others
+  // repeat them)
+  const auto send_values = [&](uint32_t tile) {
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t lane_row = lane_now >> 2;
+    const uint32_t tile_begin = tile * 64u;
+    const void* page = uniform_page(args.page_table, tile_begin / args.page_tokens);
+    const Q4hPlanes planes =
+        q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
+    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
+                           tile_begin % args.page_tokens;
+    const uint32_t target = raw_values_lds + (tile & 1u) * RAW_V;
+    const uint8_t* rows = uniform_pointer(planes.value_codes +
+                                          (record0 + 4u * wave) * ROW);
+    copy16_to_lds(rows,
+                  (16u * ((lane_row >> 2) & 3u) + (lane_row & 3u)) * ROW +
+                      (lane_now & 3u) * 16u,
+                  target + wave * 1024u);
+    if (wave < 2u) {
+      const uint8_t* scales = uniform_pointer(
+          planes.key_scales + record0 * 2u + wave * value_scale_distance);
+      copy4_to_lds(scales, 4u * (lane_now & 31u), target + CODES + wave * 256u);
+    }
+  };
+  // waves 4..7: a quarter of the tile's K codes each
+  const auto send_keys = [&](uint32_t tile) {
+    const uint32_t lane_now = fresh_lane_index();
+    const uint32_t tile_begin = tile * 64u;
+    const void* page = uniform_page(args.page_table, tile_begin / args.page_tokens);
+    const Q4hPlanes planes =
+        q4h_planes(page, args.layer, args.page_tokens, args.kv_heads, D);
+    const size_t record0 = static_cast<size_t>(kv_head) * args.page_tokens +
+                           tile_begin % args.page_tokens;
+    const uint8_t* rows = uniform_pointer(planes.key_codes + record0 * ROW +
+                                          (wave - 4u) * 1024u);
+    copy16_to_lds(rows, lane_now * 16u,
+                  raw_keys_lds + (tile & 1u) * CODES + (wave - 4u) * 1024u);
+  };
+  const auto convert = [&](uint32_t tile) {
+    uint8_t* target = converted + (tile & 1u) * CONV;
+    const uint32_t source = raw_values_lds + (tile & 1u) * RAW_V;
+    const uint32_t lane_now = fresh_lane_index();
+    // V: row tile `wave` of head_dim, both halves of the 64 tokens
+    u32x2 transposed;
+    {
+      const uint32_t address =
+          source + (16u * (lane_now >> 4) + (lane_now & 15u)) * ROW + wave * 8u;
+      asm volatile("ds_read_b64_tr_b4 %0, %1" : "=v"(transposed) : "v"(address));
+    }
+    uint32_t first_scale = 0u, second_scale = 0u;
+    if (wave == 6u) {
+      // K scale of token lane_now
+      const uint32_t address = source + CODES + 2u * lane_now;
+      asm volatile("ds_read_u16 %0, %1" : "=v"(first_scale) : "v"(address));
+    } else if (wave == 7u) {
+      // V scales of tokens (32 u + 4 q + c, + 16) for lane = 16 u + 4 q + c < 32
+      const uint32_t low_token = 32u * ((lane_now >> 4) & 1u) + (lane_now & 15u);
+      const uint32_t address = source + CODES + 256u + 2u * low_token;
+      asm volatile("ds_read_u16 %0, %1" : "=v"(first_scale) : "v"(address));
+      asm volatile("ds_read_u16 %0, %1 offset:32" : "=v"(second_scale) : "v"(address));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(transposed), "+v"(first_scale), "+v"(second_scale)
+                 :: "memory");
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const uint32_t x = transposed[u] ^ 0x88888888u;
+      const uint32_t y = x >> 8;
+      const f16x2 bias_low = {static_cast<_Float16>(-1032.0f),
+                              static_cast<_Float16>(-1032.0f)};
+      const f16x2 bias_high = {static_cast<_Float16>(-72.0f),
+                               static_cast<_Float16>(-72.0f)};
+      const f16x2 e0 = __builtin_bit_cast(
+          f16x2, insert_bits(0x000f000fu, x, 0x64006400u)) + bias_low;
+      const f16x2 e1 = __builtin_bit_cast(
+          f16x2, insert_bits(0x00f000f0u, x, 0x54005400u)) + bias_high;
+      const f16x2 e2 = __builtin_bit_cast(
+          f16x2, insert_bits(0x000f000fu, y, 0x64006400u)) + bias_low;
+      const f16x2 e3 = __builtin_bit_cast(
+          f16x2, insert_bits(0x00f000f0u, y, 0x54005400u)) + bias_high;
+      u32x4 operand;
+      operand[0] = __builtin_bit_cast(uint32_t, e0);
+      operand[1] = __builtin_bit_cast(uint32_t, e1);
+      operand[2] = __builtin_bit_cast(uint32_t, e2);
+      operand[3] = __builtin_bit_cast(uint32_t, e3);
+      *reinterpret_cast<u32x4*>(target + (wave * 2u + u) * 1024u + lane_now * 16u) =
+          operand;
+    }
+    if (wave == 6u) {
+      *reinterpret_cast<float*>(target + CONV_KS + lane_now * 4u) =
+          f16_bits_to_f32(first_scale);
+    } else if (wave == 7u && lane_now < 32u) {
+      const uint32_t low_token = 32u * (lane_now >> 4) + (lane_now & 15u);
+      const uint32_t tile_begin = tile * 64u;
+      if (tile_begin + low_token >= launch_context) first_scale = 0u;
+      if (tile_begin + low_token + 16u >= launch_context) second_scale = 0u;
+      *reinterpret_cast<uint32_t*>(target + CONV_VS + lane_now * 4u) =
+          first_scale | (second_scale << 16);
+    }
+  };
+
+  // ---- the first tiles set out, the queries are quantised meanwhile -----------
+  const bool any_tile = tile_first < tile_last;
+  if (any_tile) {
+    if (wave < 4u) send_values(tile_first);
+    else send_keys(tile_first);
+  }
+  uint8_t* q_operands_mine = q_operands_all + wave * Q_BYTES;
+  float* exchange_scale = q_scales + wave * RT * 16;
+  uint32_t* exchange_limit = q_limits + wave * RT * 16;
+  if (live) {
+#pragma unroll 1
+    for (uint32_t pair = 0; pair < static_cast<uint32_t>(RT * KSTEPS); ++pair) {
+      // k-step pair % KSTEPS of row tile pair / KSTEPS, as in the split kernel
+      const uint32_t rt = pair / KSTEPS;
+      const uint32_t step = pair % KSTEPS;
+      const uint32_t matrix_row = 16u * rt + col;
+      const bool valid = matrix_row < matrix_rows;
+      const uint32_t row = valid ? matrix_row / group : 0u;
+      const uint32_t head = kv_head * group + (valid ? matrix_row % group : 0u);
+      const size_t record =
+          static_cast<size_t>(first_row + row) * args.query_heads + head;
+      float values[16];
+      float maximum = 0.0f;
+#pragma unroll
+      for (int h = 0; h < KSTEPS; ++h) {
+        const uint32_t d0 = 128u * (h / 2) + 32u * quad + 16u * (h % 2);
+#pragma unroll
+        for (int piece = 0; piece < 4; ++piece) {
+          float4 loaded = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          if (valid)
+            loaded = *reinterpret_cast<const float4*>(
+                args.query + record * args.query_stride + d0 + 4u * piece);
+          if (static_cast<uint32_t>(h) == step) {
+            values[4 * piece + 0] = loaded.x;
+            values[4 * piece + 1] = loaded.y;
+            values[4 * piece + 2] = loaded.z;
+            values[4 * piece + 3] = loaded.w;
+          }
+          maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(loaded.x), fabsf(loaded.y)),
+                                         fmaxf(fabsf(loaded.z), fabsf(loaded.w))));
+        }
+      }
+      maximum = quad_row_max(maximum);
+      const float scale = fmaxf(maximum * (1.0f / 16319.0f), 0x1p-100f);
+      const float inverse = 1.0f / scale;
+      if (quad == 0u && step == 0u) {
+        exchange_scale[16 * rt + col] =
+            scale * (1.4426950408889634f / (16.0f * sqrtf(static_cast<float>(D))));
+        exchange_limit[16 * rt + col] = first_context_tokens + row;
+      }
+      uint32_t high_bytes[16], low_bytes[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        int quantized = __float2int_rn(values[j] * inverse);
+        quantized = max(-16319, min(16319, quantized));
+        const int high = (quantized + 64) >> 7;
+        const int low = quantized - (high << 7);
+        high_bytes[j] = static_cast<uint32_t>(high) & 0xffu;
+        low_bytes[j] = static_cast<uint32_t>(low) & 0xffu;
+      }
+      const int order[16] = {0, 2, 4, 6, 1, 3, 5, 7, 8, 10, 12, 14, 9, 11, 13, 15};
+      i32x4 high_operand, low_operand;
+#pragma unroll
+      for (int word = 0; word < 4; ++word) {
+        uint32_t high_word = 0u, low_word = 0u;
+#pragma unroll
+        for (int byte = 0; byte < 4; ++byte) {
+          high_word |= high_bytes[order[4 * word + byte]] << (8 * byte);
+          low_word |= low_bytes[order[4 * word + byte]] << (8 * byte);
+        }
+        high_operand[word] = static_cast<int>(high_word);
+        low_operand[word] = static_cast<int>(low_word);
+      }
+      *reinterpret_cast<i32x4*>(q_operands_mine + (pair * 2u + 0u) * 1024u +
+                                lane * 16u) = high_operand;
+      *reinterpret_cast<i32x4*>(q_operands_mine + (pair * 2u + 1u) * 1024u +
+                                lane * 16u) = low_operand;
+    }
+  }
+  vmem_wait<0>();
+  __syncthreads();   // the first tile's raw codes and scales are in LDS
+  if (any_tile) {
+    if (wave < 4u && tile_first + 1u < tile_last) send_values(tile_first + 1u);
+    convert(tile_first);
+  }
+  vmem_wait<0>();
+  __syncthreads();   // V operands of the first tile, raw V of the second
+
+  const uint8_t* q_operands = q_operands_mine + lane * 16u;
+  float running_max[RT];
+  float running_sum[RT];
+  f32x4 out[DT][RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    running_max[rt] = kMaskedMax;
+    running_sum[rt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
+  }
+
+  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+    if (wave < 4u) {
+      if (tile + 2u < tile_last) send_values(tile + 2u);
+    } else if (tile + 1u < tile_last) {
+      send_keys(tile + 1u);
+    }
+    if (tile + 1u < tile_last) convert(tile + 1u);
+    if (tile < batch_tiles) {
+      const uint32_t tile_begin = tile * 64u;
+      const bool needs_mask = tile_begin + 64u > first_context_tokens;
+      const uint8_t* operands = converted + (tile & 1u) * CONV;
+      // K codes out of LDS (raw), widened to int8 * 16
+      u32x4 key_raw[4];
+      {
+        const uint32_t key_address =
+            raw_keys_lds + (tile & 1u) * CODES + col * ROW + 16u * quad;
+        key_raw[0] = lds_read16<0 * 16 * ROW>(key_address);
+        key_raw[1] = lds_read16<1 * 16 * ROW>(key_address);
+        key_raw[2] = lds_read16<2 * 16 * ROW>(key_address);
+        key_raw[3] = lds_read16<3 * 16 * ROW>(key_address);
+        lds_wait(key_raw);
+      }
+      i32x4 key_operand[4][KSTEPS];
+      float k_scale[4][4];
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const u32x4 x = key_raw[st];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          i32x4 operand;
+          operand[0] = static_cast<int>((x[2 * half] << 4) & 0xf0f0f0f0u);
+          operand[1] = static_cast<int>(x[2 * half] & 0xf0f0f0f0u);
+          operand[2] = static_cast<int>((x[2 * half + 1] << 4) & 0xf0f0f0f0u);
+          operand[3] = static_cast<int>(x[2 * half + 1] & 0xf0f0f0f0u);
+          key_operand[st][half] = operand;
+        }
+        const float4 scales = *reinterpret_cast<const float4*>(
+            operands + CONV_KS + (16u * st + 4u * quad) * 4u);
+        k_scale[st][0] = scales.x; k_scale[st][1] = scales.y;
+        k_scale[st][2] = scales.z; k_scale[st][3] = scales.w;
+      }
+      f16x2 v_scale[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const uint4 pairs = *reinterpret_cast<const uint4*>(
+            operands + CONV_VS + (16u * u + 4u * quad) * 4u);
+        v_scale[u][0] = __builtin_bit_cast(f16x2, pairs.x);
+        v_scale[u][1] = __builtin_bit_cast(f16x2, pairs.y);
+        v_scale[u][2] = __builtin_bit_cast(f16x2, pairs.z);
+        v_scale[u][3] = __builtin_bit_cast(f16x2, pairs.w);
+      }
+      f16x8 p_operand[RT][2];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        asm volatile("" ::: "memory");
+        i32x4 q_high[KSTEPS], q_low[KSTEPS];
+#pragma unroll
+        for (int h = 0; h < KSTEPS; ++h) {
+          q_high[h] = *reinterpret_cast<const i32x4*>(
+              q_operands + ((rt * KSTEPS + h) * 2 + 0) * 1024);
+          q_low[h] = *reinterpret_cast<const i32x4*>(
+              q_operands + ((rt * KSTEPS + h) * 2 + 1) * 1024);
+        }
+        const float q_scale = exchange_scale[16 * rt + col];
+        float score[4][4];
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+          i32x4 dot_high = {0, 0, 0, 0};
+          i32x4 dot_low = {0, 0, 0, 0};
+#pragma unroll
+          for (int h = 0; h < KSTEPS; ++h) {
+            dot_high = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                key_operand[st][h], q_high[h], dot_high, 0, 0, 0);
+            dot_low = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                key_operand[st][h], q_low[h], dot_low, 0, 0, 0);
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int dot = (dot_high[i] << 7) + dot_low[i];
+            score[st][i] = static_cast<float>(dot) * k_scale[st][i];
+          }
+        }
+        if (needs_mask) {
+          const uint32_t first_token = tile_begin + 4u * quad;
+          const uint32_t limit = exchange_limit[16 * rt + col];
+#pragma unroll
+          for (int st = 0; st < 4; ++st)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (first_token + 16u * st + i >= limit) score[st][i] = -INFINITY;
+        }
+        // online softmax, as in the split kernel
+        float tile_max = score[0][0];
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) tile_max = fmaxf(tile_max, score[st][i]);
+        tile_max = quad_row_max(tile_max);
+        const bool grew = (tile_max - running_max[rt]) * q_scale > 8.0f;
+        if (__builtin_amdgcn_ballot_w64(grew) != 0ull) {
+          const float new_max = fmaxf(running_max[rt], tile_max);
+          if (tile != tile_first) {
+            const float factor =
+                __builtin_amdgcn_exp2f((running_max[rt] - new_max) * q_scale);
+            running_sum[rt] *= factor;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) out[dt][rt][i] *= factor;
+          }
+          running_max[rt] = new_max;
+        }
+        const float offset = -running_max[rt] * q_scale;
+        float sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const float p0 =
+                __builtin_amdgcn_exp2f(fmaf(score[2 * u][c], q_scale, offset));
+            const float p1 =
+                __builtin_amdgcn_exp2f(fmaf(score[2 * u + 1][c], q_scale, offset));
+            sum += p0 + p1;
+            f16x2 pair = {static_cast<_Float16>(p0), static_cast<_Float16>(p1)};
+            pair *= v_scale[u][c];
+            p_operand[rt][u][2 * c] = pair[0];
+            p_operand[rt][u][2 * c + 1] = pair[1];
+          }
+        running_sum[rt] += sum;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const f16x8 v_operand = *reinterpret_cast<const f16x8*>(
+              operands + (dt * 2 + u) * 1024 + lane * 16u);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            out[dt][rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                v_operand, p_operand[rt][u], out[dt][rt], 0, 0, 0);
+        }
+      }
+    }
+    vmem_wait<0>();
+    __syncthreads();
+  }
+  if (!live) return;
+
+  // ---- the batch's split partial ------------------------------------------------
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    running_sum[rt] = quad_row_sum(running_sum[rt]);
+    running_max[rt] = running_max[rt] > 0.5f * kMaskedMax
+                          ? running_max[rt] * exchange_scale[16 * rt + col]
+                          : kMaskedMax;
+    const uint32_t matrix_row = 16u * rt + col;
+    if (matrix_row >= matrix_rows) continue;
+    const uint32_t row = first_row + matrix_row / group;
+    const uint32_t head = kv_head * group + matrix_row % group;
+    const size_t partial =
+        (static_cast<size_t>(row) * args.maximum_splits + split) * args.query_heads +
+        head;
+    if (quad == 0u) {
+      args.partial_maxima[partial] = running_max[rt];
+      args.partial_sums[partial] = running_sum[rt];
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<f32x4*>(args.partial_outputs + partial * D + 16u * dt +
+                                4u * quad) = out[dt][rt];
+  }
+}
+
 // Split-K merge (maxima in log2 units), optional sigmoid output gate.
 // One workgroup per (query head, row), one thread per output dimension.  The
 // per-split weights exp2(m_s - M) are computed once, cooperatively, into LDS;
@@ -1873,6 +2340,60 @@ extern "C" int32_t qllm_attention_paged_q4h_batched(
       launch->output, launch->output_kind, launch->first_context_tokens,
       launch->maximum_splits, launch->split_tokens, launch->rows,
       launch->query_heads, launch->head_dim, nullptr, stream);
+}
+
+extern "C" int32_t qllm_attention_paged_q4h_prompt(
+    const qllm_q4h_attention_launch* launch, uint32_t batch_rows) {
+  if (!launch || !launch->query || !launch->page_table || !launch->output ||
+      (reinterpret_cast<uintptr_t>(launch->query) & 15u) ||
+      launch->query_stride % 4u || !launch->partial_maxima ||
+      !launch->partial_sums || !launch->partial_outputs ||
+      !launch->first_context_tokens || !launch->rows || !batch_rows ||
+      launch->device_positions || !launch->page_tokens ||
+      launch->page_tokens % 64u || !launch->query_heads || !launch->kv_heads ||
+      launch->query_heads % launch->kv_heads || launch->head_dim != 128u ||
+      launch->split_tokens || !launch->maximum_splits ||
+      launch->maximum_splits > kCombineSplitCapacity ||
+      launch->query_stride <
+          (launch->output_gated ? 2u : 1u) * launch->head_dim ||
+      (launch->output_kind != QLLM_OUT_F32 &&
+       launch->output_kind != QLLM_OUT_BF16) ||
+      launch->rows > 65535u * kPromptBatches ||
+      launch->first_context_tokens > 0xffffffffu - (launch->rows - 1u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H prompt attention");
+  const uint32_t group = launch->query_heads / launch->kv_heads;
+  if (std::min(batch_rows, launch->rows) * group > 48u)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "Q4H prompt attention: batch_rows * (query_heads/kv_heads) "
+                "exceeds 48");
+  const uint32_t batches = (launch->rows + batch_rows - 1u) / batch_rows;
+  SplitArgs args{};
+  args.query = launch->query;
+  args.query_stride = launch->query_stride;
+  args.page_table = launch->page_table;
+  args.partial_maxima = launch->partial_maxima;
+  args.partial_sums = launch->partial_sums;
+  args.partial_outputs = launch->partial_outputs;
+  args.first_context_tokens = launch->first_context_tokens;
+  args.rows = launch->rows;
+  args.layer = launch->full_attention_layer;
+  args.page_tokens = launch->page_tokens;
+  args.query_heads = launch->query_heads;
+  args.kv_heads = launch->kv_heads;
+  args.maximum_splits = launch->maximum_splits;
+  args.batch_rows = batch_rows;
+  const dim3 grid(launch->kv_heads, launch->maximum_splits,
+                  (batches + kPromptBatches - 1u) / kPromptBatches);
+  const hipStream_t stream = as_stream(launch->stream);
+  q4h_prompt_attention_kernel<128><<<grid, kPromptBatches * 64, 0, stream>>>(args);
+  const int32_t status = launched("Q4H prompt attention");
+  if (status != QLLM_OK) return status;
+  return launch_attention_combine(
+      launch->query, launch->query_stride, launch->output_gated,
+      launch->partial_maxima, launch->partial_sums, launch->partial_outputs,
+      launch->output, launch->output_kind, launch->first_context_tokens,
+      launch->maximum_splits, 0u, launch->rows, launch->query_heads,
+      launch->head_dim, nullptr, stream);
 }
 
 namespace {

@@ -1707,12 +1707,25 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           launch.kv_heads = g_.kv_heads;
           launch.head_dim = g_.head_dim;
           launch.split_tokens = 0U;
-          launch.maximum_splits = prefill_splits_for(rows, attention_batch);
           launch.query_stride = query_stride;
           launch.output_gated = g_.output_gated;
           launch.output_kind = QLLM_OUT_BF16;
           launch.stream = stream;
-          status_check(qllm_attention_paged_q4h_batched(&launch, attention_batch));
+          // From 32 row batches on, eight batches share a workgroup and every
+          // cache tile it fetches and converts; the context is then cut as far
+          // as it takes to give every CU one of those workgroups.
+          const std::uint32_t batches =
+              (rows + attention_batch - 1U) / attention_batch;
+          if (g_.head_dim == 128U && batches >= 32U) {
+            const std::uint32_t workgroups = (batches + 7U) / 8U * g_.kv_heads;
+            launch.maximum_splits = std::clamp(
+                (256U + workgroups - 1U) / workgroups, 1U, prefill_splits_);
+            status_check(qllm_attention_paged_q4h_prompt(&launch, attention_batch));
+          } else {
+            launch.maximum_splits = prefill_splits_for(rows, attention_batch);
+            status_check(
+                qllm_attention_paged_q4h_batched(&launch, attention_batch));
+          }
         } else {
           const std::uint32_t query_stride =
               g_.head_dim * (g_.output_gated ? 2U : 1U);

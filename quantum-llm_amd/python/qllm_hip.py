@@ -123,6 +123,7 @@ SIGNATURES = {
     "qllm_attention_paged_q4h_fused": (c_int32, [POINTER(Q4hAttentionLaunch), POINTER(Q4hFusedRope)]),
     "qllm_rope_table": (c_int32, [c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p, c_void_p]),
     "qllm_attention_paged_q4h_batched": (c_int32, [POINTER(Q4hAttentionLaunch), c_uint32]),
+    "qllm_attention_paged_q4h_prompt": (c_int32, [POINTER(Q4hAttentionLaunch), c_uint32]),
     "qllm_store_kv_paged_f16_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_attention_paged_f16": (c_int32, [POINTER(F16AttentionLaunch)]),
     "qllm_attention_paged_f16_batched": (c_int32, [POINTER(F16AttentionLaunch), c_uint32]),

@@ -216,6 +216,55 @@ def test_batched_launch_equals_one_launch_per_batch(device, total, first, Q, KV,
             qh.call("qllm_attention_paged_q4h_batched", launch, total)
 
 
+@pytest.mark.parametrize("total,first,Q,KV,gated,batch,splits", [
+    (100, 300, 64, 8, False, 6, 1),      # 17 batches: three workgroup layers, the last part empty
+    (100, 300, 64, 8, False, 6, 3),      # the tiles cut over three splits
+    (55, 1, 16, 8, True, 5, 1),          # the prompt starts the cache; gated; small groups
+    (20, 4000, 64, 8, False, 6, 5),      # fewer than eight batches
+    (300, 70, 40, 8, False, 6, 2)])      # group of five: 30 of 48 matrix rows
+def test_prompt_attention_equals_the_batched_launch(device, total, first, Q, KV, gated,
+                                                    batch, splits):
+    """Eight batches per workgroup on shared tiles: the oracle's attention, and
+    the batched launch's result up to the rounding of the probabilities."""
+    d, page_tokens = 128, 64
+    rng = np.random.default_rng(total * 7 + first)
+    tokens = first + total - 1
+    keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    values = rng.standard_normal((tokens, KV, d)).astype(np.float32)
+    pages = synth.q4h_pages(keys, values, page_tokens, 1, 0)
+    stride = d * (2 if gated else 1)
+    query = ol.bf16_round(rng.standard_normal((total, Q, stride)).astype(np.float32))
+    d_pages = [gu.device_tensor(page, device) for page in pages]
+    table = torch.tensor([page.data_ptr() for page in d_pages], dtype=torch.int64,
+                         device=device)
+    d_query = gu.device_tensor(query, device)
+    results = {}
+    for name in ("qllm_attention_paged_q4h_prompt", "qllm_attention_paged_q4h_batched"):
+        maxima = torch.zeros((total, splits, Q), device=device)
+        sums = torch.zeros_like(maxima)
+        outputs = torch.zeros((total, splits, Q, d), device=device)
+        out = torch.full((total, Q, d), float("nan"), device=device)
+        launch = qh.Q4hAttentionLaunch(
+            qh.ptr(d_query), 0, 0, qh.ptr(table), qh.ptr(out), qh.ptr(maxima),
+            qh.ptr(sums), qh.ptr(outputs), first, total, 0, page_tokens, Q, KV, d, 0,
+            splits, stride, int(gated), qh.OUT_F32, None)
+        qh.call(name, launch, batch)
+        torch.cuda.synchronize()
+        results[name] = out.cpu().numpy()
+    got, batched = results.values()
+    shape = ol.AttentionShape(total, Q, KV, d, first, page_tokens, 0, int(gated))
+    gu.assert_close(got, ol.attention_q4h(shape, query, pages, "f64"), what="prompt attention")
+    # (binary16 probabilities are rounded relative to each wave's running
+    # maximum, which the two launches reach by different routes: a few 1e-4)
+    gu.assert_close(got, batched, rtol=3e-3, atol=3e-4, what="prompt vs batched")
+    bad = qh.Q4hAttentionLaunch(
+        qh.ptr(d_query), 0, 0, qh.ptr(table), qh.ptr(out), qh.ptr(maxima), qh.ptr(sums),
+        qh.ptr(outputs), first, total, 0, page_tokens, Q, KV, d, 64, splits, stride,
+        int(gated), qh.OUT_F32, None)
+    with pytest.raises(qh.QllmError, match="invalid Q4H prompt attention"):
+        qh.call("qllm_attention_paged_q4h_prompt", bad, batch)   # fixed split_tokens
+
+
 def test_attention_at_131072_tokens_on_one_kv_head(device):
     """The long-context benchmark shape cut down to one KV head and its eight
     query heads (the heads are independent, so this is one eighth of the full
