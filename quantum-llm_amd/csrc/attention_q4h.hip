@@ -1875,7 +1875,9 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     first_cache_position = uniform_word(device_positions, 0u);
     first_rotary_position = uniform_word(device_positions, 1u);
   }
-  const uint32_t row = blockIdx.y;
+  // grid layer y takes rows y, y + gridDim.y, ... (one row each for a verify
+  // step; a prompt chunk's thousands of rows go eight to a block)
+  const auto process = [&](const uint32_t row) {
   const uint32_t lane = threadIdx.x;
   if (partials) {
     // The projection arrived as K-split partials f32 [partial_count][rows]
@@ -1981,6 +1983,11 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
                     head_dim,
                     const_cast<uint8_t*>(planes.value_codes) + record * (head_dim / 2u),
                     const_cast<uint8_t*>(planes.value_scales) + record * 2u, lane);
+  };
+  for (uint32_t row = blockIdx.y; row < rows; row += gridDim.y) {
+    process(row);
+    __syncthreads();   // the scratch rows are free again
+  }
 }
 
 // transformer_kernels.cu:4391-4416
@@ -2062,6 +2069,13 @@ int32_t launch_attention_combine(const float* query, uint32_t query_stride,
   return launched("attention split combine");
 }
 
+// grid layers of the rotary kernels: a block per row up to 64 rows, beyond
+// that eight rows per block (a block is one wave; hundreds of thousands of
+// them cost more to dispatch than to run)
+inline uint32_t rope_grid_rows(uint32_t rows) {
+  return rows <= 64u ? rows : (rows + 7u) / 8u;
+}
+
 }  // namespace qllm
 
 using namespace qllm;
@@ -2102,7 +2116,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch(
       first_cache_position > 0xffffffffu - (rows - 1u) ||
       first_rotary_position > 0xffffffffu - (rows - 1u))
     return fail(QLLM_INVALID_ARGUMENT, "invalid Q4H QKV rope cache batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
@@ -2128,7 +2142,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_batch_deferred(
       !(epsilon > 0.0f) || !(rope_theta > 0.0f))
     return fail(QLLM_INVALID_ARGUMENT,
                 "invalid deferred Q4H QKV rope cache batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, 0u, 0u, query_heads, kv_heads,
@@ -2158,7 +2172,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_from_partials(
         first_rotary_position > 0xffffffffu - (rows - 1u))))
     return fail(QLLM_INVALID_ARGUMENT,
                 "invalid Q4H QKV rope cache batch from partials");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
@@ -2209,7 +2223,7 @@ extern "C" int32_t qllm_qkv_rope_cache_paged_q4h_prepared(
     return fail(QLLM_INVALID_ARGUMENT,
                 "Q4H query operands: rows * (query_heads/kv_heads) exceeds 48 "
                 "(32 at head_dim 256)");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, value, q_norm_weight, k_norm_weight, page_table,
       full_attention_layer, page_tokens, first_cache_position,
@@ -2233,7 +2247,7 @@ extern "C" int32_t qllm_qkv_rope_batch(
       !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
       first_rotary_position > 0xffffffffu - (rows - 1u))
     return fail(QLLM_INVALID_ARGUMENT, "invalid QKV rope batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, first_rotary_position, query_heads, kv_heads, head_dim,
@@ -2254,7 +2268,7 @@ extern "C" int32_t qllm_qkv_rope_batch_deferred(
       query_stride < head_dim || !rotary_dim || rotary_dim > head_dim ||
       rotary_dim % 2u || !(epsilon > 0.0f) || !(rope_theta > 0.0f))
     return fail(QLLM_INVALID_ARGUMENT, "invalid deferred QKV rope batch");
-  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rows), 64, 0,
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
                         as_stream(stream)>>>(
       query, query_stride, key, nullptr, q_norm_weight, k_norm_weight, nullptr,
       0u, 1u, 0u, 0u, query_heads, kv_heads, head_dim, rotary_dim, epsilon,
