@@ -226,7 +226,7 @@ def test_prompt_attention_equals_the_batched_launch(device, total, first, Q, KV,
                                                     batch, splits):
     """Eight batches per workgroup on shared tiles: the oracle's attention, and
     the batched launch's result up to the rounding of the probabilities."""
-    d, page_tokens = 128, 64
+    d, page_tokens = 128, (256 if total == 300 else 64)   # tiles inside and across pages
     rng = np.random.default_rng(total * 7 + first)
     tokens = first + total - 1
     keys = rng.standard_normal((tokens, KV, d)).astype(np.float32)
