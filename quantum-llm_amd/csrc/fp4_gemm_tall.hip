@@ -17,10 +17,10 @@
 //  * UE8M0 per 32: the power-of-two scale is folded into the nibble -> bf16
 //    conversion, which stays exact; bf16 matrix instructions.
 //  * binary16 per 16: weight x scale has up to 13 significant bits (a 3-bit
-//    weight times an 11-bit scale).  It is formed exactly in F32 and split
-//    into two binary16 values, hi (the top 11 bits) and lo (the rest, exact),
-//    which go through the matrix cores one after the other into the same F32
-//    accumulator; the bf16 activations are converted to binary16 (exact
+//    weight times an 11-bit scale).  It is split into two binary16 values,
+//    hi = the product rounded to binary16 and lo = its rounding error, which
+//    a fused multiply-add returns exactly; they go through the matrix cores
+//    one after the other into the same F32 accumulator; the bf16 activations are converted to binary16 (exact
 //    between 6.1e-5 and 65504 in magnitude - the range of a decoder's
 //    normalised activations; beyond it they saturate or lose low bits).  The
 //    products are therefore the exact ones, as in the small-batch kernel, at
