@@ -169,11 +169,12 @@ def measure_decode_cycle(qp, np, rows, steps, warmup, sampled=False):
     return report
 
 
-def measure_prefill(qp, np, prompt_tokens):
+def measure_prefill(qp, np, prompt_tokens, chunk_rows=0):
     """Prompt prefill of the same model: `prompt_tokens` synthetic tokens from
-    position 0 - the linears on the tall-batch GEMM (2048 rows at a time),
-    attention in six-row batches, one launch per chunk - timed from the call
-    to the prediction of the token after the prompt (time to first token)."""
+    position 0 - the linears on the tall-batch GEMM (`chunk_rows` rows at a
+    time, 0 = the provider's 32768), attention in six-row batches, one launch
+    per chunk - timed from the call to the prediction of the token after the
+    prompt (time to first token)."""
     rng = np.random.default_rng(11)
     tokens = rng.integers(0, MODEL["vocabulary"], prompt_tokens).astype(np.uint32)
 
@@ -181,6 +182,7 @@ def measure_prefill(qp, np, prompt_tokens):
         geometry = dict(MODEL)
         geometry["mtp_layers"] = mtp_layers
         geometry["max_context"] = (prompt_tokens + 16 + 255) // 256 * 256
+        geometry["prefill_chunk_rows"] = chunk_rows
         provider = qp.Provider(**geometry)
         provider.load_synthetic_weights(20241125)
         provider.prepare_exact_decode(
@@ -292,6 +294,9 @@ def main():
     parser.add_argument("--skip-decode-cycle", action="store_true",
                         help="leave out the decode cycle with the proposer (a second "
                              "provider with the MTP layer)")
+    parser.add_argument("--prefill-chunk-rows", type=int, default=0,
+                        help="prompt rows per pass of the tall linears (0 = the "
+                             "provider's default)")
     parser.add_argument("--prefill-tokens", type=int, default=2048,
                         help="prompt length of the prefill leg (0 skips it; 32768 "
                              "is the context of the headline metric)")
@@ -419,7 +424,8 @@ def main():
         if provider is not None:
             provider.close()
         provider = None
-        prefill = measure_prefill(qp, np, arguments.prefill_tokens)
+        prefill = measure_prefill(qp, np, arguments.prefill_tokens,
+                                  arguments.prefill_chunk_rows)
     layers = geometry["layers"]
     step_bytes = (layers * (fp4_bytes(MODEL["query_heads"] * 128, H) +
                             2 * fp4_bytes(MODEL["kv_heads"] * 128, H) +

@@ -54,7 +54,7 @@ typedef struct qllm_dense_geometry {
    * min(vocabulary, 65536). */
   uint32_t draft_vocabulary;
   /* Rows of a prompt that go through the tall linears at a time
-   * (qllm_provider_prefill); 0 = 4096.  The reference's prompt path runs
+   * (qllm_provider_prefill); 0 = 32768.  The reference's prompt path runs
    * prefill_chunk_tokens rows per program step (moe_vm_runner.cpp:682-745). */
   uint32_t prefill_chunk_rows;
 } qllm_dense_geometry;

@@ -1280,7 +1280,8 @@ __global__ __launch_bounds__(kPromptBatches * 64) void q4h_prompt_attention_kern
 
   // this wave's batch
   const uint32_t batches = (args.rows + args.batch_rows - 1u) / args.batch_rows;
-  const uint32_t first_batch = blockIdx.z * kPromptBatches;
+  // (the workgroups with the longest contexts are dispatched first)
+  const uint32_t first_batch = (gridDim.z - 1u - blockIdx.z) * kPromptBatches;
   const uint32_t batch = first_batch + wave;
   const bool live = batch < batches;
   const uint32_t first_row = live ? batch * args.batch_rows : 0u;

@@ -1339,6 +1339,17 @@ std::uint32_t Mi355DenseFp4Provider::prefill_splits_for(
   return std::clamp((256U + workgroups - 1U) / workgroups, 1U, prefill_splits_);
 }
 
+// Context splits of the shared-tile prompt attention (eight row batches per
+// workgroup), or 0 where the batched launch of the verify step's kernel serves:
+// fewer than 32 row batches, head_dim 256.
+std::uint32_t Mi355DenseFp4Provider::prompt_attention_splits(
+    std::uint32_t rows, std::uint32_t attention_batch) const noexcept {
+  const std::uint32_t batches = (rows + attention_batch - 1U) / attention_batch;
+  if (g_.head_dim != 128U || batches < 32U) return 0U;
+  const std::uint32_t workgroups = (batches + 7U) / 8U * g_.kv_heads;
+  return std::clamp((256U + workgroups - 1U) / workgroups, 1U, prefill_splits_);
+}
+
 // (cos, sin) of the rotary angles of a batch at first_position .. + rows - 1
 // (or at the device-side positions), for the attention launches of a pass.
 void Mi355DenseFp4Provider::enqueue_rope_table(std::uint32_t rows,
@@ -1598,7 +1609,18 @@ void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
     // fewer splits than the verify step: the row batches of a chunk already
     // fill the GPU, and the partials are per row
     prefill_splits_ = std::min<std::uint32_t>(maximum_splits_, 8U);
-    const std::size_t partials = n * prefill_splits_ * g_.query_heads;
+    // partial rows: the most rows x splits any chunk of up to n rows asks for
+    // (long chunks are not cut, short ones have few rows)
+    const std::uint32_t attention_batch = std::max(
+        1U, (g_.head_dim == 256U ? 32U : 48U) / (g_.query_heads / g_.kv_heads));
+    std::size_t partial_rows = 0;
+    for (std::uint32_t chunk = 1; chunk <= rows; ++chunk)
+      partial_rows = std::max<std::size_t>(
+          partial_rows,
+          std::size_t{chunk} *
+              std::max(prefill_splits_for(chunk, attention_batch),
+                       prompt_attention_splits(chunk, attention_batch)));
+    const std::size_t partials = partial_rows * g_.query_heads;
     prefill_partial_maxima_ = static_cast<float*>(allocate(partials * 4U));
     prefill_partial_sums_ = static_cast<float*>(allocate(partials * 4U));
     prefill_partial_outputs_ =
@@ -1714,12 +1736,9 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
           // From 32 row batches on, eight batches share a workgroup and every
           // cache tile it fetches and converts; the context is then cut as far
           // as it takes to give every CU one of those workgroups.
-          const std::uint32_t batches =
-              (rows + attention_batch - 1U) / attention_batch;
-          if (g_.head_dim == 128U && batches >= 32U) {
-            const std::uint32_t workgroups = (batches + 7U) / 8U * g_.kv_heads;
-            launch.maximum_splits = std::clamp(
-                (256U + workgroups - 1U) / workgroups, 1U, prefill_splits_);
+          if (const std::uint32_t splits =
+                  prompt_attention_splits(rows, attention_batch)) {
+            launch.maximum_splits = splits;
             status_check(qllm_attention_paged_q4h_prompt(&launch, attention_batch));
           } else {
             launch.maximum_splits = prefill_splits_for(rows, attention_batch);

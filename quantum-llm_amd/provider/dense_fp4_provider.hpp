@@ -56,9 +56,10 @@ struct DenseGeometry final {
   // Rows of the output head the proposer scores (project_prefix); 0 stands
   // for min(vocabulary, 65536).  A multiple of 32.
   std::uint32_t draft_vocabulary{0};
-  // Prompt rows per pass of the tall linears; 0 stands for 4096 (measured on a
-  // 27B-class model: 3200 and 4096 within 0.5 %, 2048 8 % and 8192 1.5 %
-  // slower over a 32768-token prompt).
+  // Prompt rows per pass of the tall linears; 0 stands for 32768 (measured on
+  // a 27B-class model over a 32768-token prompt: 3.42 s in one pass, 3.64 s in
+  // passes of 4096 rows, whose o and down projections load the CUs unevenly;
+  // the workspace of a pass is about 200 KB per row).
   std::uint32_t prefill_chunk_rows{0};
 };
 
@@ -237,7 +238,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
       std::span<const std::uint32_t> tokens, std::uint32_t first_position,
       const er::ProgramRequestContext& request);
   [[nodiscard]] std::uint32_t prefill_chunk_rows() const noexcept {
-    return g_.prefill_chunk_rows ? g_.prefill_chunk_rows : 4096U;
+    return g_.prefill_chunk_rows ? g_.prefill_chunk_rows : 32768U;
   }
   [[nodiscard]] std::uint64_t weight_bytes() const noexcept {
     return weight_bytes_;
@@ -270,6 +271,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                                    std::size_t input_bytes, std::uint32_t rows,
                                    bool leave_partials);
   [[nodiscard]] std::uint32_t prefill_splits_for(
+      std::uint32_t rows, std::uint32_t attention_batch) const noexcept;
+  [[nodiscard]] std::uint32_t prompt_attention_splits(
       std::uint32_t rows, std::uint32_t attention_batch) const noexcept;
   void enqueue_rope_table(std::uint32_t rows, std::uint32_t first_position,
                           bool deferred_positions);
