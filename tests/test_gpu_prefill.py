@@ -134,6 +134,33 @@ def test_chunked_prefill_equals_one_pass(device, kv_encoding):
         assert len(got[4]) == 4
 
 
+def test_long_prompt_in_one_pass_equals_chunks(device):
+    """5000 prompt rows in one pass (834 row batches: 105 layers of the prompt
+    attention's grid, the longest contexts first) against passes of 1024 rows:
+    the same logits and hidden state within the end-to-end bound, the same
+    cache records up to the quantiser's one-step flips."""
+    rng, model, _ = make("reference", 123)
+    count = 5000
+    tokens = rng.integers(0, model.vocabulary, count).astype(np.uint32)
+    results = []
+    for chunk_rows in (0, 1024):
+        provider = step_oracle.build_provider(
+            model, qp, draft_vocabulary=128, max_context=5120, page_tokens=256,
+            prefill_chunk_rows=chunk_rows)
+        predicted = provider.prefill(tokens, 0)
+        pages = [provider.kv_page(page) for page in range((count + 255) // 256)]
+        results.append((predicted, provider.logits(1)[0], provider.hidden(1)[0], pages))
+        provider.close()
+    (want_token, want_logits, want_hidden, want_pages), \
+        (got_token, got_logits, got_hidden, got_pages) = results
+    assert (np.linalg.norm(got_logits - want_logits) / np.linalg.norm(want_logits)) < 2e-2
+    assert np.abs(got_hidden - want_hidden).max() < 2e-2 * np.abs(want_hidden).max()
+    assert got_token == want_token or (
+        want_logits.max() - want_logits[got_token] < 1e-2 * np.abs(want_logits).max())
+    differing = sum(int((a != b).sum()) for a, b in zip(got_pages, want_pages))
+    assert differing <= 0.03 * sum(a.size for a in want_pages)
+
+
 def test_prefill_rejects_bad_prompts(device):
     rng, model, build = make("baseline", 3, max_context=128)
     provider = build()
