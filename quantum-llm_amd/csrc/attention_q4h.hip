@@ -403,7 +403,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // a batched launch narrows the arguments to the batch of this grid layer
   SplitArgs args = launch_args;
   if (!FUSED && launch_args.batch_rows) {
-    const uint32_t first_row = blockIdx.z * launch_args.batch_rows;
+    // (the batches with the longest contexts, the last rows, are dispatched first)
+    const uint32_t first_row =
+        (gridDim.z - 1u - blockIdx.z) * launch_args.batch_rows;
     const size_t first_partial = static_cast<size_t>(first_row) *
                                  launch_args.maximum_splits *
                                  launch_args.query_heads;
