@@ -297,9 +297,10 @@ def main():
     parser.add_argument("--prefill-chunk-rows", type=int, default=0,
                         help="prompt rows per pass of the tall linears (0 = the "
                              "provider's default)")
-    parser.add_argument("--prefill-tokens", type=int, default=2048,
-                        help="prompt length of the prefill leg (0 skips it; 32768 "
-                             "is the context of the headline metric)")
+    parser.add_argument("--prefill-tokens", type=int, default=32768,
+                        help="prompt length of the prefill leg (0 skips it; the "
+                             "default is the context of the headline metric, for "
+                             "which the reference publishes its time to first token)")
     parser.add_argument("--calibration-copy", action="store_true",
                         help="also run one 256 MiB device copy (a kernel of known "
                              "traffic to scale hardware counters by)")
