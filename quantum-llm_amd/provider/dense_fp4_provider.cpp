@@ -821,6 +821,13 @@ Mi355DenseFp4Provider::create_request_state(
     hip_check(hipMemsetAsync(presence_, 0, g_.vocabulary,
                              static_cast<hipStream_t>(stream_)),
               "zero request sampling presence");
+    // The KV pages of the request's reserved context are allocated and cleared
+    // here, not page by page inside the decode loop (an allocation, a clearing
+    // and a blocking copy at every page boundary).
+    const auto reserved = request.parameters.find("reserved_context_tokens");
+    if (reserved != request.parameters.end() && reserved->second != 0U)
+      ensure_pages(static_cast<std::uint32_t>(
+          std::min<std::uint64_t>(reserved->second, g_.max_context) - 1U));
     return {er::Status::success(), std::make_shared<DenseFp4RequestState>()};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
