@@ -255,6 +255,8 @@ void Mi355DenseFp4Provider::release() {
   if (stream_) (void)hipStreamSynchronize(static_cast<hipStream_t>(stream_));
   for (void* pointer : allocations_) (void)hipFree(pointer);
   allocations_.clear();
+  for (void* pointer : prefill_allocations_) (void)hipFree(pointer);
+  prefill_allocations_.clear();
   if (staging_) {
     (void)hipHostFree(staging_);
     staging_ = nullptr;
@@ -1585,14 +1587,21 @@ void Mi355DenseFp4Provider::enqueue_mtp_prefill(
       prefill_hidden_, rows, stream));
 }
 
+// The buffers of a prompt pass of up to `rows` rows.  A longer prompt than any
+// before replaces them by larger ones (the stream is idle between prefills).
 void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
   if (rows <= prefill_rows_) return;
-  if (prefill_rows_)
-    throw std::runtime_error("prefill workspace is already allocated smaller");
+  if (prefill_rows_) {
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "drain the stream before the prefill workspace grows");
+    for (void* pointer : prefill_allocations_) (void)hipFree(pointer);
+    prefill_allocations_.clear();
+    prefill_rows_ = 0U;
+  }
   const auto allocate = [this](std::size_t bytes) {
     void* pointer{};
     hip_check(hipMalloc(&pointer, bytes), "allocate prefill workspace");
-    allocations_.push_back(pointer);
+    prefill_allocations_.push_back(pointer);
     return pointer;
   };
   const std::size_t n = rows;
@@ -1658,9 +1667,10 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
                  "prompt token is outside the vocabulary"},
                 0U};
     const auto count = static_cast<std::uint32_t>(tokens.size());
-    // sized for a whole chunk whatever the first prompt's length: the
-    // workspace does not grow
-    ensure_prefill_workspace(std::min(prefill_chunk_rows(), g_.max_context));
+    // sized for the pass this prompt needs, in steps of 4096 rows
+    ensure_prefill_workspace(std::min(
+        std::min(prefill_chunk_rows(), g_.max_context),
+        (std::min(count, prefill_chunk_rows()) + 4095U) / 4096U * 4096U));
     ensure_pages(first_position + count - 1U);
     void* const stream = stream_;
     const auto hip_stream = static_cast<hipStream_t>(stream_);

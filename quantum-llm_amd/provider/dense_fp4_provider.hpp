@@ -436,6 +436,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   std::uint32_t* mtp_argmax_{};
   // prompt prefill workspace
   std::uint32_t prefill_rows_{};
+  std::vector<void*> prefill_allocations_;
   std::uint32_t* prefill_tokens_{};
   float* prefill_hidden_{};
   std::uint16_t* prefill_normalized_{};   // bf16 [rows, hidden]

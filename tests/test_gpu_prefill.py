@@ -147,6 +147,8 @@ def test_long_prompt_in_one_pass_equals_chunks(device):
         provider = step_oracle.build_provider(
             model, qp, draft_vocabulary=128, max_context=5120, page_tokens=256,
             prefill_chunk_rows=chunk_rows)
+        if chunk_rows == 0:
+            provider.prefill(tokens[:10], 0)     # a short prompt first: the workspace grows
         predicted = provider.prefill(tokens, 0)
         pages = [provider.kv_page(page) for page in range((count + 255) // 256)]
         results.append((predicted, provider.logits(1)[0], provider.hidden(1)[0], pages))
