@@ -38,7 +38,11 @@ struct Machine {
   er::ModelArtifact artifact;
   er::ExecutionProviderModule module;
   er::MoeProgramExecutor executor;
-  er::ProgramExecutionSession session;
+  // one session per request slot and one more, so that a test can ask for a
+  // request the provider has no slot for; `session` is the selected one
+  std::vector<er::ProgramExecutionSession> sessions;
+  std::size_t selected = 0;
+  er::ProgramExecutionSession& session() { return sessions[selected]; }
   std::string error;
 };
 
@@ -64,8 +68,10 @@ const char* qvm_error(void* machine) {
 
 void* qvm_open(const char* root, std::uint32_t max_context,
                std::uint32_t kv_page_tokens, const char* kv_cache_dtype,
-               std::uint32_t mtp_draft_depth, char* message, std::size_t capacity) {
+               std::uint32_t mtp_draft_depth, std::uint32_t request_capacity,
+               char* message, std::size_t capacity) {
   auto machine = std::make_unique<Machine>();
+  machine->sessions.resize(std::size_t{request_capacity} + 1U);
   const auto give_up = [&](const er::Status& status) -> void* {
     if (message && capacity) {
       const auto text = std::string(status.message());
@@ -81,7 +87,7 @@ void* qvm_open(const char* root, std::uint32_t max_context,
   }
   // the factory with the runner's sixteen arguments (moe_vm_runner.cpp:459-468)
   auto created = qllm::make_mi355_dense_fp4_callable_provider(
-      root, max_context, 1U, std::uint64_t{1} << 30U, std::uint64_t{1} << 30U,
+      root, max_context, request_capacity, std::uint64_t{1} << 30U, std::uint64_t{1} << 30U,
       std::uint64_t{64} << 20U, kv_page_tokens, kv_cache_dtype, "latency", "fixed",
       false, false, {}, 0U, 0U, mtp_draft_depth);
   if (!created.status.ok()) return give_up(created.status);
@@ -106,7 +112,9 @@ void* qvm_open(const char* root, std::uint32_t max_context,
 
 void qvm_close(void* opaque) {
   auto* machine = static_cast<Machine*>(opaque);
-  if (machine && machine->session.valid()) machine->session.cancel();
+  if (machine)
+    for (auto& session : machine->sessions)
+      if (session.valid()) session.cancel();
   delete machine;
 }
 
@@ -127,14 +135,34 @@ int qvm_service(void* opaque, char* kv_dtype, std::size_t capacity,
 int qvm_begin_session(void* opaque, const char* const* names,
                       const std::uint64_t* values, std::uint32_t count) {
   auto* machine = static_cast<Machine*>(opaque);
-  if (machine->session.valid()) machine->session.cancel();
+  // the selected session's previous request ends (and gives its slot back)
+  // before the new one begins
+  if (machine->session().valid()) machine->session().cancel();
+  machine->session() = er::ProgramExecutionSession{};
   er::ProgramRequestContext request;
-  request.request_id = 1U;
+  request.request_id = machine->selected + 1U;
   for (std::uint32_t index = 0; index < count; ++index)
     request.parameters[names[index]] = values[index];
   auto begun = machine->executor.begin_session(std::move(request));
   if (!begun.status.ok()) return fail(machine, begun.status);
-  machine->session = std::move(begun.session);
+  machine->session() = std::move(begun.session);
+  return 0;
+}
+
+// which session the calls below address
+int qvm_select_session(void* opaque, std::uint32_t index) {
+  auto* machine = static_cast<Machine*>(opaque);
+  if (index >= machine->sessions.size())
+    return fail(machine, {er::ErrorCode::invalid_argument, "no such session"});
+  machine->selected = index;
+  return 0;
+}
+
+// ends the selected session's request
+int qvm_end_session(void* opaque) {
+  auto* machine = static_cast<Machine*>(opaque);
+  if (machine->session().valid()) machine->session().cancel();
+  machine->session() = er::ProgramExecutionSession{};
   return 0;
 }
 
@@ -150,7 +178,7 @@ int qvm_execute(void* opaque, const std::uint32_t* tokens,
     else if (endpoint.abi == kPositionAbi)
       inputs.emplace(role, host_words(kPositionAbi, positions, rows));
   }
-  auto started = machine->session.execute(std::move(inputs));
+  auto started = machine->session().execute(std::move(inputs));
   if (!started.status.ok()) return fail(machine, started.status);
   std::optional<er::ProgramExecutionResult> result;
   for (int attempt = 0; attempt < 1000000 && !result; ++attempt)
@@ -164,14 +192,14 @@ int qvm_execute(void* opaque, const std::uint32_t* tokens,
 }
 
 int qvm_exact_available(void* opaque) {
-  return static_cast<Machine*>(opaque)->session.exact_decode_available() ? 1 : 0;
+  return static_cast<Machine*>(opaque)->session().exact_decode_available() ? 1 : 0;
 }
 
 int qvm_synchronize(void* opaque, const std::uint32_t* next_tokens,
                     std::uint32_t count, std::uint32_t first_target_position,
                     int produce_final_draft) {
   auto* machine = static_cast<Machine*>(opaque);
-  const auto status = machine->session.synchronize_exact_decode_batch(
+  const auto status = machine->session().synchronize_exact_decode_batch(
       {next_tokens, count}, first_target_position, produce_final_draft != 0);
   return status.ok() ? 0 : fail(machine, status);
 }
@@ -182,7 +210,7 @@ int qvm_exact_decode(void* opaque, std::uint32_t guaranteed_token,
                      std::uint32_t* next_token, std::uint32_t* positions_advanced) {
   auto* machine = static_cast<Machine*>(opaque);
   auto started =
-      machine->session.execute_exact_decode(guaranteed_token, position, context_limit);
+      machine->session().execute_exact_decode(guaranteed_token, position, context_limit);
   if (!started.status.ok()) return fail(machine, started.status);
   std::optional<er::ExactDecodeExecutionResult> result;
   for (int attempt = 0; attempt < 1000000 && !result; ++attempt)

@@ -124,6 +124,8 @@ er::Status dense_geometry_from_artifact(const er::ModelDescriptor& model,
     if (g.max_context > model.max_context_tokens)
       return invalid("requested context exceeds the artifact's maximum");
     g.kv_page_tokens = options.kv_page_tokens;
+    g.capacity = std::max(1U, options.capacity);
+    g.profile_gpu_phases = options.profile_gpu_phases;
     if (options.kv_cache_dtype == "artifact" ||
         options.kv_cache_dtype == "q4-f16-per-head")
       g.kv_encoding = KvEncoding::q4_f16_per_head;
@@ -254,19 +256,15 @@ er::CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
     std::uint64_t vram_cache_bytes, std::uint64_t kv_cache_bytes,
     std::uint32_t kv_page_tokens, std::string_view kv_cache_dtype,
     std::string_view /*placement_profile*/, std::string_view routed_vram_policy,
-    bool /*profile_gpu_phases*/, bool /*discover_active_expert_devices*/,
+    bool profile_gpu_phases, bool /*discover_active_expert_devices*/,
     std::vector<int> /*active_expert_devices*/,
     std::uint64_t /*active_expert_device_cache_bytes*/,
     std::uint64_t /*active_expert_host_cache_bytes*/,
     std::uint32_t mtp_draft_depth) {
   try {
-    // the launch contract of dense_fp4_provider.cpp:2330-2336; one request at
-    // a time owns the KV cache here
+    // the launch contract of dense_fp4_provider.cpp:2330-2336
     if (!capacity || !max_context || !kv_cache_bytes || !kv_page_tokens)
       return {invalid("invalid dense FP4 provider launch contract"), {}};
-    if (capacity != 1U)
-      return {invalid("this provider serves one request at a time (capacity 1)"),
-              {}};
     auto artifact = std::make_shared<er::ModelArtifact>();
     if (auto status = er::ModelArtifact::load(artifact_root, *artifact); !status.ok())
       return {status, {}};
@@ -280,6 +278,8 @@ er::CreateExecutionProviderModuleResult make_mi355_dense_fp4_callable_provider(
     options.kv_cache_dtype = std::string(kv_cache_dtype);
     options.vram_cache_bytes = vram_cache_bytes ? vram_cache_bytes : 1U;
     options.routed_vram_policy = std::string(routed_vram_policy);
+    options.capacity = capacity;
+    options.profile_gpu_phases = profile_gpu_phases;
     return make_mi355_dense_fp4_module(std::move(artifact), options);
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};

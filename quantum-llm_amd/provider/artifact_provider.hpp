@@ -29,6 +29,8 @@ struct ArtifactProviderOptions final {
   std::uint32_t mtp_draft_depth{};  // 0 = the artifact's declared depth
   std::uint64_t vram_cache_bytes{1};  // echoed in the service contract
   std::string routed_vram_policy{"fixed"};
+  std::uint32_t capacity{1};        // request slots
+  bool profile_gpu_phases{};        // provider_gpu_*_ns telemetry, uncaptured passes
 };
 
 // The descriptor check behind every capability of this provider: the slice of

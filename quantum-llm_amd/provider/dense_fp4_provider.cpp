@@ -261,9 +261,15 @@ void Mi355DenseFp4Provider::release() {
     (void)hipHostFree(staging_);
     staging_ = nullptr;
   }
-  for (void* page : pages_)
-    if (page) (void)hipFree(page);
-  pages_.clear();
+  for (auto& slot : slots_)
+    for (void* page : slot.pages)
+      if (page) (void)hipFree(page);
+  slots_.clear();
+  for (auto& events : gpu_event_pool_) {
+    (void)hipEventDestroy(static_cast<hipEvent_t>(events.start));
+    (void)hipEventDestroy(static_cast<hipEvent_t>(events.stop));
+  }
+  gpu_event_pool_.clear();
   if (stream_) {
     (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
     stream_ = nullptr;
@@ -304,6 +310,7 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   graphs_.assign(max_rows_ + 1U, nullptr);
   if (const char* eager = std::getenv("QLLM_PROVIDER_EAGER"))
     use_graphs_ = eager[0] == '0';
+  if (g_.profile_gpu_phases) use_graphs_ = false;
   hidden_ = static_cast<float*>(device_alloc(rows * g_.hidden * 4U));
   // read by the proposer when a stream is synchronised before any target pass
   hip_check(hipMemset(hidden_, 0, rows * g_.hidden * 4U), "clear hidden state");
@@ -417,23 +424,119 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
                      qllm_q8_layer_bytes(g_.kv_page_tokens, g_.kv_heads, g_.head_dim);
   const std::size_t page_count =
       (g_.max_context + g_.kv_page_tokens - 1U) / g_.kv_page_tokens;
-  pages_.assign(page_count, nullptr);
+  slots_.resize(std::max(1U, g_.capacity));
+  for (auto& slot : slots_) {
+    slot.leased = std::make_shared<std::atomic<bool>>(false);
+    slot.pages.assign(page_count, nullptr);
+    if (slots_.size() > 1U) {
+      slot.saved_presence = static_cast<std::uint8_t*>(device_alloc(g_.vocabulary));
+      hip_check(hipMemset(slot.saved_presence, 0, g_.vocabulary),
+                "clear slot presence bytes");
+      if (g_.mtp_layers) {
+        slot.saved_last_hidden = static_cast<float*>(device_alloc(g_.hidden * 4U));
+        hip_check(hipMemset(slot.saved_last_hidden, 0, g_.hidden * 4U),
+                  "clear slot proposer state");
+      }
+    }
+  }
   device_page_table_ =
       static_cast<void**>(device_alloc(page_count * sizeof(void*)));
   hip_check(hipMemset(device_page_table_, 0, page_count * sizeof(void*)),
             "clear device page table");
 }
 
+// Makes `slot` the one whose pages, presence bytes and proposer state the
+// kernels address.  Everything is ordered on the provider's stream, so work
+// already enqueued for the outgoing slot still sees its own table.
+void Mi355DenseFp4Provider::activate(std::uint32_t slot) {
+  if (slot >= slots_.size()) throw std::runtime_error("request slot is invalid");
+  if (slot == active_slot_) return;
+  const auto stream = static_cast<hipStream_t>(stream_);
+  auto& outgoing = slots_[active_slot_];
+  auto& incoming = slots_[slot];
+  hip_check(hipMemcpyAsync(outgoing.saved_presence, presence_, g_.vocabulary,
+                           hipMemcpyDeviceToDevice, stream),
+            "save request presence bytes");
+  hip_check(hipMemcpyAsync(presence_, incoming.saved_presence, g_.vocabulary,
+                           hipMemcpyDeviceToDevice, stream),
+            "load request presence bytes");
+  if (mtp_last_hidden_) {
+    hip_check(hipMemcpyAsync(outgoing.saved_last_hidden, mtp_last_hidden_,
+                             g_.hidden * 4U, hipMemcpyDeviceToDevice, stream),
+              "save proposer state");
+    hip_check(hipMemcpyAsync(mtp_last_hidden_, incoming.saved_last_hidden,
+                             g_.hidden * 4U, hipMemcpyDeviceToDevice, stream),
+              "load proposer state");
+  }
+  // a pageable source: the copy has read it when the call returns
+  hip_check(hipMemcpyAsync(device_page_table_, incoming.pages.data(),
+                           incoming.pages.size() * sizeof(void*),
+                           hipMemcpyHostToDevice, stream),
+            "load request page table");
+  active_slot_ = slot;
+}
+
+// ---- GPU phase timing (dense_fp4_provider.cpp:5691-5738) ---------------------
+// An event pair per operation of a pass, from a pool that grows on demand; the
+// pass's last operation reads them all back and adds each to its phase's total.
+std::size_t Mi355DenseFp4Provider::begin_gpu_phase(GpuPhase phase) {
+  if (!g_.profile_gpu_phases) return ~std::size_t{0};
+  if (active_gpu_events_ == gpu_event_pool_.size()) {
+    hipEvent_t start{}, stop{};
+    hip_check(hipEventCreate(&start), "create GPU phase start event");
+    if (const auto status = hipEventCreate(&stop); status != hipSuccess) {
+      (void)hipEventDestroy(start);
+      hip_check(status, "create GPU phase stop event");
+    }
+    gpu_event_pool_.push_back({start, stop, phase});
+  }
+  auto& events = gpu_event_pool_[active_gpu_events_];
+  events.phase = phase;
+  hip_check(hipEventRecord(static_cast<hipEvent_t>(events.start),
+                           static_cast<hipStream_t>(stream_)),
+            "record GPU phase start");
+  return active_gpu_events_++;
+}
+
+void Mi355DenseFp4Provider::end_gpu_phase(std::size_t index) {
+  if (!g_.profile_gpu_phases) return;
+  if (index >= active_gpu_events_)
+    throw std::runtime_error("GPU phase event index is invalid");
+  hip_check(hipEventRecord(static_cast<hipEvent_t>(gpu_event_pool_[index].stop),
+                           static_cast<hipStream_t>(stream_)),
+            "record GPU phase stop");
+}
+
+void Mi355DenseFp4Provider::collect_gpu_phases() {
+  if (!g_.profile_gpu_phases || active_gpu_events_ == 0U) return;
+  hip_check(hipEventSynchronize(static_cast<hipEvent_t>(
+                gpu_event_pool_[active_gpu_events_ - 1U].stop)),
+            "synchronize GPU phase events");
+  for (std::size_t index = 0; index < active_gpu_events_; ++index) {
+    const auto& events = gpu_event_pool_[index];
+    float milliseconds{};
+    hip_check(hipEventElapsedTime(&milliseconds,
+                                  static_cast<hipEvent_t>(events.start),
+                                  static_cast<hipEvent_t>(events.stop)),
+              "read GPU phase elapsed time");
+    gpu_phase_ns_[static_cast<std::size_t>(events.phase)] +=
+        static_cast<std::uint64_t>(std::llround(double{milliseconds} * 1.0e6));
+  }
+  active_gpu_events_ = 0U;
+  ++gpu_measured_batches_;
+}
+
 void Mi355DenseFp4Provider::ensure_pages(std::uint32_t last_position) {
+  auto& pages = slots_[active_slot_].pages;
   const std::size_t last_page = last_position / g_.kv_page_tokens;
-  if (last_page >= pages_.size())
+  if (last_page >= pages.size())
     throw std::runtime_error("KV position exceeds the configured context");
   for (std::size_t page = 0; page <= last_page; ++page) {
-    if (pages_[page]) continue;
+    if (pages[page]) continue;
     void* pointer{};
     hip_check(hipMalloc(&pointer, kv_page_bytes_), "allocate KV page");
     hip_check(hipMemset(pointer, 0, kv_page_bytes_), "clear KV page");
-    pages_[page] = pointer;
+    pages[page] = pointer;
     hip_check(hipMemcpy(device_page_table_ + page, &pointer, sizeof(pointer),
                         hipMemcpyHostToDevice),
               "publish KV page");
@@ -820,6 +923,17 @@ Mi355DenseFp4Provider::create_request_state(
           presence == request.parameters.end() || presence->second > 4'000'000U)
         throw std::runtime_error("request has an invalid sampling profile");
     }
+    // a free slot, or the reference's answer when every slot is taken
+    // (dense_fp4_provider.cpp:5514-5518)
+    std::uint32_t slot = 0U;
+    while (slot < slots_.size() &&
+           slots_[slot].leased->load(std::memory_order_acquire))
+      ++slot;
+    if (slot == slots_.size())
+      return {{er::ErrorCode::backpressure,
+               "dense FP4 provider has no free request slot"},
+              {}};
+    activate(slot);
     hip_check(hipMemsetAsync(presence_, 0, g_.vocabulary,
                              static_cast<hipStream_t>(stream_)),
               "zero request sampling presence");
@@ -830,7 +944,11 @@ Mi355DenseFp4Provider::create_request_state(
     if (reserved != request.parameters.end() && reserved->second != 0U)
       ensure_pages(static_cast<std::uint32_t>(
           std::min<std::uint64_t>(reserved->second, g_.max_context) - 1U));
-    return {er::Status::success(), std::make_shared<DenseFp4RequestState>()};
+    auto state = std::make_shared<DenseFp4RequestState>();
+    state->slot = slot;
+    state->lease = slots_[slot].leased;
+    state->lease->store(true, std::memory_order_release);
+    return {er::Status::success(), std::move(state)};
   } catch (const std::exception& error) {
     return {{er::ErrorCode::internal, error.what()}, {}};
   }
@@ -865,6 +983,7 @@ er::Status Mi355DenseFp4Provider::rebind_request_state(
         first->second >= g_.max_context ||
         presence == request.parameters.end() || presence->second > 4'000'000U)
       throw std::runtime_error("sampling request rebind is invalid");
+    activate(state->slot);
     hip_check(hipMemsetAsync(presence_, 0, g_.vocabulary,
                              static_cast<hipStream_t>(stream_)),
               "reset request sampling presence");
@@ -993,6 +1112,7 @@ er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
     if (!operation || !state ||
         operation->kind == PreparedOperation::Kind::exact_decode)
       throw std::runtime_error("dense FP4 invocation state is invalid");
+    activate(state->slot);
     const auto input = [&](std::string_view port) -> const er::ExecutionValue& {
       const auto found = operation->input_indices.find(port);
       if (found == operation->input_indices.end() ||
@@ -1002,6 +1122,16 @@ er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
     };
     const auto stream = static_cast<hipStream_t>(stream_);
     std::map<std::string, er::ExecutionValue, std::less<>> outputs;
+    const auto phase_of = [](PreparedOperation::Kind kind) {
+      switch (kind) {
+        case PreparedOperation::Kind::embedding: return GpuPhase::embedding;
+        case PreparedOperation::Kind::attention: return GpuPhase::full_attention;
+        case PreparedOperation::Kind::ffn: return GpuPhase::ffn;
+        case PreparedOperation::Kind::head: return GpuPhase::head;
+        default: return GpuPhase::mtp;
+      }
+    };
+    const auto phase_events = begin_gpu_phase(phase_of(operation->kind));
     switch (operation->kind) {
       case PreparedOperation::Kind::embedding: {
         state->exact_decode_enabled =
@@ -1074,6 +1204,8 @@ er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
         }
         // a batch selects for its last row only (terminal_only, :8397-8402)
         enqueue_head(rows - 1U, 1U);
+        end_gpu_phase(phase_events);
+        collect_gpu_phases();
         auto owner = std::make_shared<std::vector<std::uint32_t>>(
             1U, select_head_token(invocation.request, state->current_position));
         outputs.emplace(
@@ -1088,6 +1220,8 @@ er::OperationExecutionHandle Mi355DenseFp4Provider::execute(
       case PreparedOperation::Kind::exact_decode:
         throw std::runtime_error("exact decode entered scalar execution");
     }
+    if (operation->kind != PreparedOperation::Kind::head)
+      end_gpu_phase(phase_events);
     er::OperationExecutionResult result;
     result.status = er::Status::success();
     result.outputs.reserve(operation->outputs.size());
@@ -1135,6 +1269,7 @@ er::Status Mi355DenseFp4Provider::synchronize_exact_decode_batch(
       if (token >= g_.vocabulary)
         return {er::ErrorCode::invalid_argument,
                 "synchronized token is outside the vocabulary"};
+    activate(state->slot);
     const auto rows =
         static_cast<std::uint32_t>(synchronization.next_tokens.size());
     if (rows > max_rows_ ||
@@ -1484,16 +1619,28 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
                                            std::uint32_t rows,
                                            std::uint32_t first_position,
                                            bool deferred_positions) {
-  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
-                                        hidden_, rows, stream_));
-  enqueue_rope_table(rows, first_position, deferred_positions);
+  // with phase timing on, an event pair around every operation (nothing is
+  // recorded otherwise, and never into a captured graph: profiling passes run
+  // uncaptured)
+  const auto timed = [this](GpuPhase phase, auto&& enqueue) {
+    const auto events = begin_gpu_phase(phase);
+    enqueue();
+    end_gpu_phase(events);
+  };
+  timed(GpuPhase::embedding, [&] {
+    status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, device_tokens,
+                                          hidden_, rows, stream_));
+    enqueue_rope_table(rows, first_position, deferred_positions);
+  });
   pending_partials_ = 0U;
   for (std::uint32_t index = 0; index < g_.layers; ++index) {
-    enqueue_attention_block(index, rows, first_position, deferred_positions,
-                            true);
-    enqueue_ffn_block(index, rows, true);
+    timed(GpuPhase::full_attention, [&] {
+      enqueue_attention_block(index, rows, first_position, deferred_positions,
+                              true);
+    });
+    timed(GpuPhase::ffn, [&] { enqueue_ffn_block(index, rows, true); });
   }
-  enqueue_head(0U, rows);
+  timed(GpuPhase::head, [&] { enqueue_head(0U, rows); });
 }
 
 // The proposer's pass over a prompt chunk: row r pairs tokens[r] (the token
@@ -1666,6 +1813,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
         return {{er::ErrorCode::invalid_argument,
                  "prompt token is outside the vocabulary"},
                 0U};
+    if (state) activate(state->slot);
     const auto count = static_cast<std::uint32_t>(tokens.size());
     // sized for the pass this prompt needs, in steps of 4096 rows
     ensure_prefill_workspace(std::min(
@@ -1909,6 +2057,7 @@ er::Status Mi355DenseFp4Provider::run_target(const std::uint32_t* tokens,
                              static_cast<hipStream_t>(stream_)),
               "upload target tokens");
     enqueue_target(tokens_, rows, first_position, false);
+    collect_gpu_phases();
     return er::Status::success();
   } catch (const std::exception& error) {
     return {er::ErrorCode::internal, error.what()};
@@ -2504,7 +2653,12 @@ std::optional<DraftPrediction> Mi355DenseFp4Provider::run_mtp(
   hip_check(hipMemcpyAsync(mtp_tokens_, tokens.data(), rows * 4U,
                            hipMemcpyHostToDevice, hip_stream),
             "upload MTP token batch");
-  enqueue_mtp(rows, previous_hidden, produce_logits, cache_position, false);
+  {
+    const auto events = begin_gpu_phase(GpuPhase::mtp);
+    enqueue_mtp(rows, previous_hidden, produce_logits, cache_position, false);
+    end_gpu_phase(events);
+    collect_gpu_phases();
+  }
   state.mtp_length += rows;
   ++mtp_passes_;
   mtp_rows_ += rows;
@@ -2674,6 +2828,7 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
         invocation.position + 1U >= invocation.context_limit ||
         invocation.context_limit > g_.max_context)
       throw std::runtime_error("exact MTP invocation stream is invalid");
+    activate(state->slot);
     const auto proposal_count = state->draft_predictions.size();
     if (proposal_count == 0U || proposal_count > g_.draft_depth ||
         invocation.position + proposal_count >= invocation.context_limit)
@@ -3017,6 +3172,7 @@ er::Status Mi355DenseFp4Provider::copy_mtp_state(float* host_last_hidden,
 er::Status Mi355DenseFp4Provider::copy_kv_page(std::uint32_t page_index,
                                                void* host_output) {
   std::lock_guard lock(mutex_);
+  const auto& pages_ = slots_[active_slot_].pages;
   if (!host_output || page_index >= pages_.size())
     return {er::ErrorCode::invalid_argument, "KV page index is invalid"};
   auto status = hipStreamSynchronize(static_cast<hipStream_t>(stream_));
@@ -3050,6 +3206,18 @@ Mi355DenseFp4Provider::telemetry() const {
   values["provider_mtp_kv_page_offset"] = mtp_page_offset_;
   values["provider_weight_bytes"] = weight_bytes_;
   values["provider_kv_page_bytes"] = kv_page_bytes_;
+  // dense_fp4_provider.cpp:3170-3200
+  if (g_.profile_gpu_phases) {
+    const auto phase = [this](GpuPhase which) {
+      return gpu_phase_ns_[static_cast<std::size_t>(which)];
+    };
+    values["provider_gpu_embedding_ns"] = phase(GpuPhase::embedding);
+    values["provider_gpu_full_attention_ns"] = phase(GpuPhase::full_attention);
+    values["provider_gpu_ffn_ns"] = phase(GpuPhase::ffn);
+    values["provider_gpu_head_ns"] = phase(GpuPhase::head);
+    values["provider_gpu_mtp_ns"] = phase(GpuPhase::mtp);
+    values["provider_gpu_measured_batches"] = gpu_measured_batches_;
+  }
   return values;
 }
 
@@ -3131,7 +3299,7 @@ Mi355DenseFp4Provider::service_contract() const {
   contract.kv_allocation = "paged_on_demand";
   contract.kv_page_tokens = g_.kv_page_tokens;
   contract.kv_page_bytes = kv_page_bytes_;
-  contract.kv_page_capacity = pages_.size();
+  contract.kv_page_capacity = slots_.size() * slots_.front().pages.size();
   contract.placement_mode = "resident";
   contract.placement_profile = "resident";
   contract.ram_cache_bytes = 0U;

@@ -9,6 +9,7 @@
 // the gfx950 kernels of include/qllm_kernels.h on one HIP stream.
 #pragma once
 
+#include <atomic>
 #include <cstdint>
 #include <map>
 #include <memory>
@@ -61,6 +62,14 @@ struct DenseGeometry final {
   // passes of 4096 rows, whose o and down projections load the CUs unevenly;
   // the workspace of a pass is about 200 KB per row).
   std::uint32_t prefill_chunk_rows{0};
+  // Requests that may be open at once (request slots,
+  // dense_fp4_provider.cpp:5514-5518, 6554-6588): each owns its KV pages, its
+  // presence bytes and its proposer state.
+  std::uint32_t capacity{1};
+  // Opt-in hipEvent pairs around every operation kind, accumulated into the
+  // provider_gpu_*_ns telemetry (dense_fp4_provider.cpp:5661-5738).  Passes run
+  // one launch at a time then: a captured graph has no place for the events.
+  bool profile_gpu_phases{};
 };
 
 // Defined with the artifact factory: the descriptor check behind every
@@ -75,6 +84,13 @@ struct DraftPrediction final {
 
 class DenseFp4RequestState final : public er::IOperationProviderRequestState {
  public:
+  ~DenseFp4RequestState() override {
+    if (lease) lease->store(false, std::memory_order_release);
+  }
+  // The request slot this state holds until it is destroyed: its index and
+  // the slot's in-use flag (shared with the provider, which may be gone first).
+  std::uint32_t slot{};
+  std::shared_ptr<std::atomic<bool>> lease;
   std::uint32_t synchronized_token{};
   std::uint32_t mtp_length{};   // position of the guaranteed token
   bool draft_valid{};
@@ -213,6 +229,9 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   [[nodiscard]] const float* hidden() const noexcept { return hidden_; }
   [[nodiscard]] void* stream() const noexcept { return stream_; }
   [[nodiscard]] const DenseGeometry& geometry() const noexcept { return g_; }
+  [[nodiscard]] bool profiles_gpu_phases() const noexcept {
+    return g_.profile_gpu_phases;
+  }
   [[nodiscard]] std::map<std::string, std::uint64_t, std::less<>> telemetry()
       const;
   [[nodiscard]] er::ExecutionProviderModule::ServiceContract service_contract()
@@ -294,7 +313,34 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   std::shared_ptr<const void> device_lifetime_;
   std::vector<std::shared_ptr<const PreparedOperation>> prepared_attention_;
   std::vector<std::shared_ptr<const PreparedOperation>> prepared_ffn_;
+  // What a request keeps on the device between calls.  Kernels and captured
+  // graphs address one working set (device_page_table_, presence_,
+  // mtp_last_hidden_); when a call arrives for another slot the working set
+  // is saved into the outgoing slot and loaded from the incoming one - a page
+  // table upload and two small device copies on the provider's stream.
+  struct RequestSlot final {
+    std::shared_ptr<std::atomic<bool>> leased;
+    std::vector<void*> pages;        // this slot's page pointers (host view)
+    std::uint8_t* saved_presence{};  // [vocabulary], capacity > 1 only
+    float* saved_last_hidden{};      // [hidden], proposer, capacity > 1 only
+  };
+  void activate(std::uint32_t slot);
   void ensure_pages(std::uint32_t last_position);
+  // GPU phase timing (begin_gpu_phase / end_gpu_phase / collect_gpu_phases,
+  // dense_fp4_provider.cpp:5691-5738)
+  enum class GpuPhase : std::uint32_t { embedding, full_attention, ffn, head, mtp, count };
+  struct GpuPhaseEvents final {
+    void* start{};
+    void* stop{};
+    GpuPhase phase{};
+  };
+  [[nodiscard]] std::size_t begin_gpu_phase(GpuPhase phase);
+  void end_gpu_phase(std::size_t index);
+  void collect_gpu_phases();
+  std::vector<GpuPhaseEvents> gpu_event_pool_;
+  std::size_t active_gpu_events_{};
+  std::uint64_t gpu_phase_ns_[static_cast<std::size_t>(GpuPhase::count)]{};
+  std::uint64_t gpu_measured_batches_{};
   DeviceFp4Matrix upload_matrix(const er::ImmutableModelTensor& tensor,
                                 bool tiled);
   // One tiled matrix holding the rows of the given row-major matrices in
@@ -370,7 +416,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   MtpWeights mtp_;
 
   // KV cache
-  std::vector<void*> pages_;
+  std::vector<RequestSlot> slots_;
+  std::uint32_t active_slot_{};
   void** device_page_table_{};
   std::uint64_t kv_page_bytes_{};
   std::uint64_t mtp_page_offset_{};   // the proposer's Q8 layer inside a page

@@ -317,6 +317,8 @@ extern "C" int32_t qllm_provider_begin_request(qllm_provider* provider,
       2'000'000U;
   provider->request.parameters["sampling_first_output_position"] = 0U;
   provider->request.parameters["exact_decode_enabled"] = 1U;
+  // the handle's previous request gives its slot back first
+  provider->state.reset();
   auto result = provider->provider->create_request_state(provider->request);
   if (!result.status.ok()) return from_status(result.status);
   provider->state = result.state;
@@ -336,6 +338,7 @@ extern "C" int32_t qllm_provider_begin_request_with(qllm_provider* provider,
         return fail(QLLM_INVALID_ARGUMENT, "request parameter name is null");
       provider->request.parameters[names[index]] = values[index];
     }
+    provider->state.reset();
     auto result = provider->provider->create_request_state(provider->request);
     if (!result.status.ok()) return from_status(result.status);
     provider->state = result.state;

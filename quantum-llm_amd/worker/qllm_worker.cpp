@@ -4,732 +4,694 @@
 // CudaWorker :489) talks to this worker unchanged.
 //
 //   usage: qllm-worker <artifact> --worker --max-context=N --ram-cache-gib=N
-//            --vram-cache-gib=N --capacity=1 --kv-cache-mib=N --kv-page-tokens=N
+//            --vram-cache-gib=N --capacity=N --kv-cache-mib=N --kv-page-tokens=N
 //            --placement-profile=latency|balanced|capacity
 //            [--kv-cache-dtype=artifact|q4-f16-per-head|fp16]
 //            [--mtp-draft-depth=N] [--routed-vram-policy=fixed]
+//            [--prefill-chunk-limit=N] [--profile-gpu-phases]
 //
-// Start-up follows main() of the runner (:1472-1538): artifact load, the one
-// module whose capability table covers the program, registry add + bind,
-// preparation of every operation, service contract check, the ready line
-// (:577-652).  Commands (worker_loop, :655-1470): PING, BEGIN <id> <context>
-// <t,t,...> [SAMPLING <temperature_ppm> <top_p_ppm> <top_k> <min_p_ppm>
-// <presence_ppm> <seed>], STEP <id>,<mode>..., NEXT <id> <mode>, CANCEL <id>,
-// END <id>, STATS, SHUTDOWN; modes: 0 = decode (an exact-decode step when the
-// request is eligible), 1 = emit the pending token and close, 2 = one plain
-// program step.  Session retention, parking and persistence are not offered
-// (the ready line says so), so RESUME / CHECKPOINT / RETAIN / DROP / SAVE /
-// LOAD / PRUNE answer with the runner's "does not support" errors; MULTIMODAL
-// needs a program input this provider's programs do not have.  Every failure
-// is one {"type":"error"} line; the process keeps serving.
+// Structure: Engine is what every request runs on (model, prepared program,
+// provider, the program's token ports); Request owns one conversation - its
+// program session, the token the model has predicted but not yet emitted, its
+// position and limit - and moves it forward by prompt, by speculative step,
+// by plain step or by its closing token; Service maps each command verb to a
+// handler through a table, reads the handler's arguments with a typed field
+// cursor and answers with one JSON line.  Every failure is an
+// {"type":"error"} line; the process keeps serving.
+//
+// Commands: PING, BEGIN <id> <context> <t,t,...> [SAMPLING <temperature_ppm>
+// <top_p_ppm> <top_k> <min_p_ppm> <presence_ppm> <seed>], STEP <id>,<mode>...,
+// NEXT <id> <mode>, CANCEL <id>, END <id>, STATS, SHUTDOWN; modes: 0 = decode
+// (an exact-decode step when the request is eligible), 1 = emit the pending
+// token and close, 2 = one plain program step.  Session retention, parking and
+// persistence are not offered (the ready line says so), so RESUME / CHECKPOINT
+// / RETAIN / DROP / SAVE / LOAD / PRUNE answer with the runner's "does not
+// support" errors; MULTIMODAL needs a program input this provider's programs
+// do not have.
 #include "expert/runtime/model_artifact.hpp"
 #include "expert/runtime/program_executor.hpp"
 
 #include "artifact_provider.hpp"
 #include "dense_fp4_provider.hpp"
+#include "launch_contract.hpp"
 #include "program_session.hpp"
+#include "wire.hpp"
 
 #include <algorithm>
+#include <array>
 #include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <filesystem>
 #include <iostream>
-#include <limits>
 #include <map>
 #include <memory>
-#include <optional>
-#include <set>
 #include <span>
 #include <stdexcept>
 #include <string>
 #include <string_view>
-#include <unordered_map>
 #include <vector>
 
 namespace er = expert::runtime;
 
+namespace qllm::worker {
 namespace {
+
+using wire::expect;
+using wire::FieldCursor;
+using wire::JsonLine;
 
 constexpr std::string_view kTokenAbi = "batch.token-id.u32.host.v1";
 constexpr std::string_view kPositionAbi = "batch.position.u32.host.v1";
+constexpr char kNoRetention[] = "callable provider does not support session retention";
+constexpr char kNoPersistence[] =
+    "callable provider does not support session persistence";
 
-void require(bool condition, std::string_view message) {
-  if (!condition) throw std::runtime_error(std::string(message));
-}
+void expect_ok(const er::Status& status) { expect(status.ok(), status.message()); }
 
-// ---- launch options (worker_contract.cpp:67-180) ---------------------------
+class Stopwatch final {
+ public:
+  [[nodiscard]] std::uint64_t nanoseconds() const {
+    return static_cast<std::uint64_t>(
+        std::chrono::duration_cast<std::chrono::nanoseconds>(
+            std::chrono::steady_clock::now() - start_)
+            .count());
+  }
 
-struct LaunchOptions final {
-  std::uint32_t max_context{};
-  std::uint64_t ram_cache_gib{};
-  std::uint64_t vram_cache_gib{};
-  std::string routed_vram_policy{"fixed"};
-  std::uint32_t capacity{};
-  std::uint64_t kv_cache_mib{};
-  std::uint32_t kv_page_tokens{};
-  std::string kv_cache_dtype{"artifact"};
-  std::string placement_profile;
-  bool profile_gpu_phases{};
-  std::optional<std::uint32_t> mtp_draft_depth;
+ private:
+  std::chrono::steady_clock::time_point start_{std::chrono::steady_clock::now()};
 };
 
-std::uint64_t unsigned_integer(const std::string& text) {
-  require(!text.empty() &&
-              std::all_of(text.begin(), text.end(),
-                          [](char c) { return c >= '0' && c <= '9'; }) &&
-              text.size() <= 19U,
-          "invalid worker launch contract: worker option is not an unsigned integer");
-  return std::stoull(text);
-}
+// What the worker counts itself; the provider's own telemetry joins it in the
+// STATS reply.
+struct Counters final {
+  std::uint64_t program_steps{};
+  std::uint64_t program_step_ns{};
+  std::uint64_t useful_tokens{};
+  std::uint64_t exact_calls{};
+  std::uint64_t exact_positions{};
+  std::uint64_t exact_accepted{};
+  std::uint64_t cancelled{};
+};
 
-LaunchOptions parse_launch_options(int argc, char** argv) {
-  std::map<std::string, std::optional<std::string>, std::less<>> raw;
-  for (int index = 3; index < argc; ++index) {
-    const std::string_view argument(argv[index]);
-    require(argument.starts_with("--") && argument.size() > 2U,
-            "invalid worker launch contract: worker launch contains a positional "
-            "option");
-    const auto separator = argument.find('=');
-    const auto name = argument.substr(
-        2U, separator == std::string_view::npos ? std::string_view::npos
-                                                : separator - 2U);
-    const auto canonical = [](char c) {
-      return (c >= 'a' && c <= 'z') || (c >= '0' && c <= '9') || c == '-';
-    };
-    require(!name.empty() && name.front() != '-' && name.back() != '-' &&
-                std::all_of(name.begin(), name.end(), canonical),
-            "invalid worker launch contract: worker option name is not canonical");
-    std::optional<std::string> value;
-    if (separator != std::string_view::npos) {
-      require(separator + 1U < argument.size(),
-              "invalid worker launch contract: worker option value is empty");
-      value = std::string(argument.substr(separator + 1U));
-    }
-    require(raw.emplace(std::string(name), std::move(value)).second,
-            "invalid worker launch contract: worker option is duplicated");
-  }
-  const auto value_of = [&](const char* name) -> const std::string& {
-    const auto found = raw.find(name);
-    require(found != raw.end() && found->second.has_value(),
-            std::string("invalid worker launch contract: missing worker option --") +
-                name);
-    return *found->second;
-  };
-  const auto u32 = [&](const char* name) {
-    const auto value = unsigned_integer(value_of(name));
-    require(value != 0U && value <= std::numeric_limits<std::uint32_t>::max(),
-            "invalid worker launch contract: worker option is out of range");
-    return static_cast<std::uint32_t>(value);
-  };
-  LaunchOptions options;
-  options.max_context = u32("max-context");
-  options.ram_cache_gib = unsigned_integer(value_of("ram-cache-gib"));
-  options.vram_cache_gib = unsigned_integer(value_of("vram-cache-gib"));
-  if (raw.contains("routed-vram-policy"))
-    options.routed_vram_policy = value_of("routed-vram-policy");
-  options.capacity = u32("capacity");
-  options.kv_cache_mib = unsigned_integer(value_of("kv-cache-mib"));
-  options.kv_page_tokens = u32("kv-page-tokens");
-  if (raw.contains("kv-cache-dtype"))
-    options.kv_cache_dtype = value_of("kv-cache-dtype");
-  options.placement_profile = value_of("placement-profile");
-  if (raw.contains("mtp-draft-depth"))
-    options.mtp_draft_depth = u32("mtp-draft-depth");
-  require(options.ram_cache_gib != 0U && options.vram_cache_gib != 0U &&
-              options.kv_cache_mib != 0U &&
-              (options.routed_vram_policy == "fixed" ||
-               options.routed_vram_policy == "fit") &&
-              (options.placement_profile == "latency" ||
-               options.placement_profile == "balanced" ||
-               options.placement_profile == "capacity"),
-          "invalid worker launch contract: worker resource contract is invalid");
-  if (const auto found = raw.find("profile-gpu-phases"); found != raw.end()) {
-    require(!found->second.has_value(),
-            "invalid worker launch contract: boolean worker option "
-            "profile-gpu-phases has a value");
-    options.profile_gpu_phases = true;
-  }
-  constexpr std::string_view known[]{
-      "max-context",       "ram-cache-gib",      "vram-cache-gib",
-      "routed-vram-policy", "capacity",          "kv-cache-mib",
-      "kv-page-tokens",    "kv-cache-dtype",     "mtp-draft-depth",
-      "placement-profile", "profile-gpu-phases"};
-  for (const auto& [name, value] : raw)
-    require(std::find(std::begin(known), std::end(known), name) != std::end(known),
-            "callable VM service does not accept provider-specific launch flags");
-  require(options.ram_cache_gib <= (std::numeric_limits<std::uint64_t>::max() >> 30U) &&
-              options.vram_cache_gib <=
-                  (std::numeric_limits<std::uint64_t>::max() >> 30U) &&
-              options.kv_cache_mib <=
-                  (std::numeric_limits<std::uint64_t>::max() >> 20U),
-          "worker resource byte count overflows");
-  return options;
-}
-
-// ---- protocol helpers --------------------------------------------------------
-
-std::vector<std::string_view> split_tabs(std::string_view line) {
-  std::vector<std::string_view> fields;
-  for (;;) {
-    const auto tab = line.find('\t');
-    fields.push_back(line.substr(0U, tab));
-    if (tab == std::string_view::npos) return fields;
-    line.remove_prefix(tab + 1U);
-  }
-}
-
-std::vector<std::uint32_t> parse_tokens(std::string_view text,
-                                        std::uint32_t vocabulary) {
-  std::vector<std::uint32_t> tokens;
-  while (!text.empty()) {
-    const auto comma = text.find(',');
-    const auto value = std::stoull(std::string(text.substr(0U, comma)));
-    require(value < vocabulary, "token is outside model vocabulary");
-    tokens.push_back(static_cast<std::uint32_t>(value));
-    if (comma == std::string_view::npos) break;
-    text.remove_prefix(comma + 1U);
-  }
-  return tokens;
-}
-
-std::string json_text(std::string_view value) {
-  std::string text;
-  for (const char c : value) {
-    if (c == '"' || c == '\\') {
-      text.push_back('\\');
-      text.push_back(c);
-    } else if (c == '\n' || c == '\r' || c == '\t') {
-      text.push_back(' ');
-    } else {
-      text.push_back(c);
-    }
-  }
-  return text;
-}
-
-er::ExecutionValue host_words(std::span<const std::uint32_t> words,
-                              std::string_view abi) {
-  auto owner = std::make_shared<std::vector<std::uint32_t>>(words.begin(), words.end());
-  return {std::string(abi), "host", owner,
-          reinterpret_cast<const std::byte*>(owner->data()),
-          owner->size() * sizeof(std::uint32_t)};
-}
-
-struct Sampling final {
+// The SAMPLING group of a BEGIN line; without one a request is greedy.
+struct SamplingProfile final {
   std::uint32_t temperature_ppm{};
   std::uint32_t top_p_ppm{1000000U};
   std::uint32_t top_k{};
   std::uint32_t min_p_ppm{};
   std::int32_t presence_penalty_ppm{};
   std::uint64_t seed{};
-  [[nodiscard]] bool enabled() const noexcept { return temperature_ppm != 0U; }
+
+  [[nodiscard]] bool greedy() const noexcept { return temperature_ppm == 0U; }
+
+  static SamplingProfile read(FieldCursor& fields, std::uint32_t vocabulary) {
+    expect(fields.left() >= 6U, "invalid BEGIN sampling marker");
+    const auto temperature = fields.natural();
+    const auto top_p = fields.natural();
+    const auto top_k = fields.natural();
+    const auto min_p = fields.natural();
+    const auto presence = fields.integer();
+    SamplingProfile profile;
+    profile.seed = fields.natural();
+    expect(temperature <= 2000000U && top_p >= 1U && top_p <= 1000000U &&
+               top_k <= vocabulary && min_p <= 1000000U && presence >= -2000000 &&
+               presence <= 2000000,
+           "invalid BEGIN sampling values");
+    profile.temperature_ppm = static_cast<std::uint32_t>(temperature);
+    profile.top_p_ppm = static_cast<std::uint32_t>(top_p);
+    profile.top_k = static_cast<std::uint32_t>(top_k);
+    profile.min_p_ppm = static_cast<std::uint32_t>(min_p);
+    profile.presence_penalty_ppm = static_cast<std::int32_t>(presence);
+    return profile;
+  }
+
+  // the request parameters a provider reads (moe_vm_runner.cpp:318-347)
+  void publish(std::map<std::string, std::uint64_t, std::less<>>& parameters) const {
+    parameters["sampling_temperature_ppm"] = temperature_ppm;
+    parameters["sampling_top_p_ppm"] = top_p_ppm;
+    parameters["sampling_top_k"] = top_k;
+    parameters["sampling_min_p_ppm"] = min_p_ppm;
+    parameters["sampling_presence_penalty_biased_ppm"] = static_cast<std::uint64_t>(
+        std::int64_t{presence_penalty_ppm} + 2'000'000);
+    parameters["sampling_seed"] = seed;
+  }
 };
 
-// moe_vm_runner.cpp:318-347
-er::ProgramRequestContext request_context(std::uint64_t id, std::uint32_t reserved,
-                                          std::uint32_t first_output_position,
-                                          const Sampling& sampling, bool exact) {
-  er::ProgramRequestContext request;
-  request.request_id = id;
-  request.parameters.emplace("reserved_context_tokens", reserved);
-  request.parameters.emplace("sampling_temperature_ppm", sampling.temperature_ppm);
-  request.parameters.emplace("sampling_top_p_ppm", sampling.top_p_ppm);
-  request.parameters.emplace("sampling_top_k", sampling.top_k);
-  request.parameters.emplace("sampling_min_p_ppm", sampling.min_p_ppm);
-  request.parameters.emplace(
-      "sampling_presence_penalty_biased_ppm",
-      static_cast<std::uint64_t>(
-          static_cast<std::int64_t>(sampling.presence_penalty_ppm) + 2'000'000LL));
-  request.parameters.emplace("sampling_first_output_position", first_output_position);
-  request.parameters.emplace("sampling_seed", sampling.seed);
-  request.parameters.emplace("exact_decode_enabled", exact ? 1U : 0U);
-  return request;
+enum class StepMode : std::uint8_t { decode = 0, finish = 1, plain = 2 };
+
+[[nodiscard]] StepMode step_mode(std::string_view text) {
+  expect(text.size() == 1U && text[0] >= '0' && text[0] <= '2',
+         "STEP request mismatch");
+  return static_cast<StepMode>(text[0] - '0');
 }
 
-struct Ports final {
-  std::string token_input;
-  std::string position_input;
-  std::string token_output;
-};
+// The model, its prepared program and the provider behind it: shared by all
+// requests, changed by none.
+class Engine final {
+ public:
+  Engine(const er::ModelDescriptor& model, const er::ExecutionProviderModule& module,
+         const PreparedProgram& prepared, const LaunchOptions& options)
+      : model_(model), module_(module), prepared_(prepared) {
+    provider_ = std::dynamic_pointer_cast<Mi355DenseFp4Provider>(
+        module.definition.implementation);
+    expect(provider_ != nullptr, "callable provider module has no implementation");
+    find_ports();
+    chunk_ = std::max<std::uint32_t>(1U, module.service.prefill_chunk_tokens);
+    if (options.prefill_chunk_limit)
+      chunk_ = std::min(chunk_, *options.prefill_chunk_limit);
+  }
 
-// :297-316
-Ports service_ports(const er::ModelDescriptor& model) {
-  Ports ports;
-  for (const auto& [role, endpoint] : model.program_inputs) {
-    if (endpoint.abi == kTokenAbi) {
-      require(ports.token_input.empty(), "multiple token program inputs");
-      ports.token_input = role;
-    } else if (endpoint.abi == kPositionAbi) {
-      require(ports.position_input.empty(), "multiple position program inputs");
-      ports.position_input = role;
+  [[nodiscard]] const er::ModelDescriptor& model() const noexcept { return model_; }
+  [[nodiscard]] const er::ExecutionProviderModule& module() const noexcept {
+    return module_;
+  }
+  [[nodiscard]] const PreparedProgram& prepared() const noexcept { return prepared_; }
+  [[nodiscard]] Mi355DenseFp4Provider& provider() const noexcept { return *provider_; }
+  [[nodiscard]] std::uint32_t chunk_tokens() const noexcept { return chunk_; }
+
+  // Whether a request with this profile may be decoded speculatively
+  // (moe_vm_runner.cpp:670-676): greedy always, sampled only through the
+  // version-2 exact-decode contract with a top-k the device selection serves.
+  [[nodiscard]] bool speculative(const SamplingProfile& profile) const noexcept {
+    const auto& decode = model_.exact_decode_program;
+    if (!decode) return false;
+    if (profile.greedy()) return true;
+    return decode->abi_version >= 2U && profile.top_k >= 1U && profile.top_k <= 64U;
+  }
+
+  // One pass of the program over `tokens` at first_position, first_position +
+  // 1, ...; returns the token the head selected for the last row.
+  [[nodiscard]] std::uint32_t run(ProgramSession& session,
+                                  std::span<const std::uint32_t> tokens,
+                                  std::uint32_t first_position) const {
+    std::vector<std::uint32_t> positions(tokens.size());
+    for (std::uint32_t row = 0U; row < positions.size(); ++row)
+      positions[row] = first_position + row;
+    std::map<std::string, er::ExecutionValue, std::less<>> inputs;
+    inputs.emplace(token_input_, words(tokens, kTokenAbi));
+    inputs.emplace(position_input_, words(positions, kPositionAbi));
+    auto outputs = session.execute(std::move(inputs));
+    expect_ok(outputs.status);
+    const auto found = outputs.values.find(token_output_);
+    expect(found != outputs.values.end(),
+           "model program did not publish its token output");
+    const er::ExecutionValue& value = found->second;
+    expect(value.valid() && value.abi == kTokenAbi && value.memory_domain == "host" &&
+               value.bytes != 0U && value.bytes % sizeof(std::uint32_t) == 0U,
+           "callable VM returned an invalid token value");
+    std::uint32_t last{};
+    std::memcpy(&last, value.data + (value.bytes - sizeof(last)), sizeof(last));
+    return last;
+  }
+
+ private:
+  static er::ExecutionValue words(std::span<const std::uint32_t> values,
+                                  std::string_view abi) {
+    auto storage =
+        std::make_shared<std::vector<std::uint32_t>>(values.begin(), values.end());
+    const auto* bytes = reinterpret_cast<const std::byte*>(storage->data());
+    return {std::string(abi), "host", storage, bytes,
+            storage->size() * sizeof(std::uint32_t)};
+  }
+
+  // The token-step service ABI (moe_vm_runner.cpp:297-316): exactly a token
+  // and a position input and one token output.
+  void find_ports() {
+    const auto claim = [](std::string& port, const std::string& role,
+                          std::string_view complaint) {
+      expect(port.empty(), complaint);
+      port = role;
+    };
+    for (const auto& [role, endpoint] : model_.program_inputs) {
+      if (endpoint.abi == kTokenAbi)
+        claim(token_input_, role, "multiple token program inputs");
+      else if (endpoint.abi == kPositionAbi)
+        claim(position_input_, role, "multiple position program inputs");
     }
+    for (const auto& [role, endpoint] : model_.program_outputs)
+      if (endpoint.abi == kTokenAbi)
+        claim(token_output_, role, "multiple token program outputs");
+    expect(model_.program_inputs.size() == 2U && !token_input_.empty() &&
+               !position_input_.empty() && !token_output_.empty(),
+           "artifact does not implement the token-step service ABI");
   }
-  for (const auto& [role, endpoint] : model.program_outputs) {
-    if (endpoint.abi != kTokenAbi) continue;
-    require(ports.token_output.empty(), "multiple token program outputs");
-    ports.token_output = role;
-  }
-  require(!ports.token_input.empty() && !ports.position_input.empty() &&
-              !ports.token_output.empty() && model.program_inputs.size() == 2U,
-          "artifact does not implement the token-step service ABI");
-  return ports;
-}
 
-struct ActiveRequest final {
-  std::unique_ptr<qllm::ProgramSession> session;
-  std::uint32_t predicted{};
-  std::uint32_t next_position{};
-  std::uint32_t context_limit{};
-  Sampling sampling;
+  const er::ModelDescriptor& model_;
+  const er::ExecutionProviderModule& module_;
+  const PreparedProgram& prepared_;
+  std::shared_ptr<Mi355DenseFp4Provider> provider_;
+  std::string token_input_, position_input_, token_output_;
+  std::uint32_t chunk_{1U};
 };
 
-// :540-568, the checks that apply to a resident provider without retention
-void validate_service_contract(const er::ModelDescriptor& model,
-                               const er::ExecutionProviderModule& module,
-                               const LaunchOptions& options) {
-  const auto& service = module.service;
-  const auto& provider = module.definition.implementation;
-  require(!service.prefill_mode.empty() && service.prefill_chunk_tokens != 0U &&
-              provider != nullptr &&
-              service.session_retention ==
-                  provider->supports_request_state_retention() &&
-              service.session_parking ==
-                  provider->supports_request_state_parking() &&
-              service.session_persistence ==
-                  provider->supports_request_state_persistence() &&
-              !service.session_parking && service.session_park_ram_bytes == 0U &&
-              service.session_park_page_capacity == 0U &&
-              !service.request_stream_mode.empty() && !service.rope_mode.empty() &&
-              !service.kv_dtype.empty() &&
-              (options.kv_cache_dtype == "artifact" ||
-               service.kv_dtype == options.kv_cache_dtype) &&
-              !service.kv_allocation.empty() &&
-              service.kv_page_tokens == options.kv_page_tokens &&
-              service.kv_page_bytes != 0U && service.kv_page_capacity != 0U &&
-              service.routed_vram_policy == options.routed_vram_policy &&
-              service.placement_mode == "resident" &&
-              service.placement_profile == "resident" &&
-              service.ram_cache_bytes == 0U && service.vram_cache_bytes != 0U &&
-              !service.placement_prefetch_enabled &&
-              service.placement_minimum_observations == 0U &&
-              !service.placement_prefetch_state.empty() &&
-              service.mtp_enabled == model.exact_decode_program.has_value() &&
-              (!service.mtp_enabled ||
-               (service.mtp_resource_available && service.mtp_runtime_ready)),
+// One conversation.  `pending_` is the token the model has chosen for
+// position `position_` and the service has not been given yet.
+class Request final {
+ public:
+  Request(const Engine& engine, std::uint64_t id, std::uint32_t context_limit,
+          const SamplingProfile& profile, std::size_t prompt_tokens)
+      : engine_(engine), limit_(context_limit), speculative_(engine.speculative(profile)) {
+    er::ProgramRequestContext context;
+    context.request_id = id;
+    context.parameters["reserved_context_tokens"] = context_limit;
+    context.parameters["sampling_first_output_position"] = prompt_tokens - 1U;
+    context.parameters["exact_decode_enabled"] = speculative_ ? 1U : 0U;
+    profile.publish(context.parameters);
+    expect_ok(ProgramSession::begin(engine.model(), engine.module(), engine.prepared(),
+                                    std::move(context), session_));
+    speculative_ = speculative_ && session_->exact_decode_available();
+  }
+
+  [[nodiscard]] std::uint32_t position() const noexcept { return position_; }
+
+  // The prompt (the runner's feed, moe_vm_runner.cpp:679-857).  Prompts longer
+  // than one program batch take the provider's tall prefill, which also feeds
+  // the proposer and rolls the first drafts out; short ones walk the program
+  // batch by batch and tell the proposer each batch's successors.
+  void ingest(std::span<const std::uint32_t> prompt, Counters& counters) {
+    const Stopwatch watch;
+    const std::size_t batch = engine_.chunk_tokens();
+    if (prompt.size() > batch) {
+      const auto result = engine_.provider().prefill(session_->state(), prompt,
+                                                     position_, session_->request());
+      expect_ok(result.status);
+      pending_ = result.predicted;
+    } else {
+      for (std::size_t done = 0U; done < prompt.size(); done += batch) {
+        const auto rows = prompt.subspan(done, std::min(batch, prompt.size() - done));
+        const auto first = position_ + static_cast<std::uint32_t>(done);
+        pending_ = engine_.run(*session_, rows, first);
+        if (!speculative_) continue;
+        // row r's successor is the next prompt token; the last row's is the
+        // head's prediction
+        std::vector<std::uint32_t> successors(rows.begin() + 1, rows.end());
+        const bool last = done + rows.size() == prompt.size();
+        successors.push_back(last ? pending_ : prompt[done + rows.size()]);
+        expect_ok(session_->synchronize_exact_decode_batch(successors, first, last));
+      }
+    }
+    position_ += static_cast<std::uint32_t>(prompt.size());
+    counters.program_steps += prompt.size();
+    counters.program_step_ns += watch.nanoseconds();
+  }
+
+  // The tokens one step hands to the service.
+  [[nodiscard]] std::vector<std::uint32_t> advance(StepMode mode, Counters& counters) {
+    if (mode == StepMode::finish) return {pending_};
+    expect(position_ < limit_, "request context is exhausted");
+    // a verify step needs room for the guaranteed token and one more
+    if (mode == StepMode::decode && speculative_ && position_ + 1U < limit_)
+      return verify(counters);
+    // the position is taken once the program has run: a proposer that cannot
+    // follow (its rollout would start past the context) fails the step, and
+    // the request still stands one token further
+    const std::uint32_t emitted = pending_;
+    const std::uint32_t here = position_;
+    pending_ = engine_.run(*session_, {&emitted, 1U}, here);
+    position_ = here + 1U;
+    if (speculative_)
+      expect_ok(session_->synchronize_exact_decode_batch({&pending_, 1U}, here, true));
+    ++counters.program_steps;
+    return {emitted};
+  }
+
+ private:
+  std::vector<std::uint32_t> verify(Counters& counters) {
+    auto result = session_->execute_exact_decode(pending_, position_, limit_);
+    expect_ok(result.status);
+    pending_ = result.next_token;
+    position_ += result.positions_advanced;
+    counters.program_steps += result.positions_advanced;
+    counters.exact_calls += 1U;
+    counters.exact_positions += result.positions_advanced;
+    counters.exact_accepted += result.positions_advanced - 1U;
+    return std::move(result.emitted_tokens);
+  }
+
+  const Engine& engine_;
+  std::unique_ptr<ProgramSession> session_;
+  std::uint32_t pending_{};
+  std::uint32_t position_{};
+  std::uint32_t limit_{};
+  bool speculative_{};
+};
+
+// The service contract a resident provider without retention must return
+// (moe_vm_runner.cpp:540-568).
+void check_service_contract(const er::ModelDescriptor& model,
+                            const er::ExecutionProviderModule& module,
+                            const LaunchOptions& options) {
+  const auto& s = module.service;
+  const auto* provider = module.definition.implementation.get();
+  const bool retention_agrees =
+      provider != nullptr &&
+      s.session_retention == provider->supports_request_state_retention() &&
+      s.session_parking == provider->supports_request_state_parking() &&
+      s.session_persistence == provider->supports_request_state_persistence() &&
+      !s.session_parking && s.session_park_ram_bytes == 0U &&
+      s.session_park_page_capacity == 0U;
+  const bool kv_agrees =
+      !s.kv_dtype.empty() && !s.kv_allocation.empty() &&
+      (options.kv_cache_dtype == "artifact" || s.kv_dtype == options.kv_cache_dtype) &&
+      s.kv_page_tokens == options.kv_page_tokens && s.kv_page_bytes != 0U &&
+      s.kv_page_capacity != 0U;
+  const bool placement_agrees =
+      s.placement_mode == "resident" && s.placement_profile == "resident" &&
+      s.routed_vram_policy == options.routed_vram_policy && s.ram_cache_bytes == 0U &&
+      s.vram_cache_bytes != 0U && !s.placement_prefetch_enabled &&
+      s.placement_minimum_observations == 0U && !s.placement_prefetch_state.empty();
+  const bool mtp_agrees =
+      s.mtp_enabled == model.exact_decode_program.has_value() &&
+      (!s.mtp_enabled || (s.mtp_resource_available && s.mtp_runtime_ready));
+  require(!s.prefill_mode.empty() && s.prefill_chunk_tokens != 0U &&
+              !s.request_stream_mode.empty() && !s.rope_mode.empty() &&
+              retention_agrees && kv_agrees && placement_agrees && mtp_agrees,
           "callable provider returned an invalid service contract");
 }
 
-// :577-652
-void print_ready(const er::ModelDescriptor& model,
-                 const er::ExecutionProviderModule::ServiceContract& service,
-                 const LaunchOptions& options) {
-  const auto flag = [](bool value) { return value ? "true" : "false"; };
-  std::uint64_t draft_depth = 0U;
-  if (model.exact_decode_program) {
-    const auto found = model.exact_decode_program->parameters.find("draft_depth");
-    if (found != model.exact_decode_program->parameters.end())
-      draft_depth = found->second;
-  }
-  auto& out = std::cout;
-  out << "{\"type\":\"ready\",\"protocol\":13,\"capacity\":" << options.capacity
-      << ",\"architecture_id\":\"" << json_text(model.architecture_id)
-      << "\",\"vocab_size\":" << model.vocab_size
-      << ",\"max_context_tokens\":" << model.max_context_tokens
-      << ",\"routed_layers\":0,\"experts_per_layer\":0,\"route_width\":0"
-      << ",\"expert_encoding\":\"\",\"operation_capabilities\":[";
-  for (std::size_t index = 0; index < model.required_kernels.size(); ++index)
-    out << (index ? "," : "") << '"'
-        << json_text(model.required_kernels[index].capability) << '"';
-  out << "],\"prefill_mode\":\"" << service.prefill_mode
-      << "\",\"prefill_chunk_tokens\":" << service.prefill_chunk_tokens
-      << ",\"session_retention\":" << flag(service.session_retention)
-      << ",\"session_parking\":" << flag(service.session_parking)
-      << ",\"session_persistence\":" << flag(service.session_persistence)
-      << ",\"session_park_ram_bytes\":" << service.session_park_ram_bytes
-      << ",\"session_park_page_capacity\":" << service.session_park_page_capacity
-      << ",\"request_stream_mode\":\"" << service.request_stream_mode
-      << "\",\"gpu_phase_timing\":" << flag(options.profile_gpu_phases)
-      << ",\"sampling_supported\":" << flag(service.sampling_supported)
-      << ",\"sampling_presence_penalty_supported\":" << flag(service.sampling_supported)
-      << ",\"mtp_resource_available\":" << flag(service.mtp_resource_available)
-      << ",\"mtp_runtime_ready\":" << flag(service.mtp_runtime_ready)
-      << ",\"mtp_enabled\":" << flag(service.mtp_enabled)
-      << ",\"mtp_draft_depth\":" << draft_depth
-      << ",\"retain_previous_route\":" << flag(service.retain_previous_route)
-      << ",\"cpu_hybrid_enabled\":" << flag(service.cpu_hybrid_enabled)
-      << ",\"rope_mode\":\"" << service.rope_mode << "\",\"kv_dtype\":\""
-      << service.kv_dtype << "\",\"kv_allocation\":\"" << service.kv_allocation
-      << "\",\"kv_page_tokens\":" << service.kv_page_tokens
-      << ",\"kv_page_bytes\":" << service.kv_page_bytes
-      << ",\"kv_page_capacity\":" << service.kv_page_capacity
-      << ",\"placement_mode\":\"" << service.placement_mode
-      << "\",\"placement_profile\":\"" << service.placement_profile
-      << "\",\"ram_cache_bytes\":" << service.ram_cache_bytes
-      << ",\"vram_cache_bytes\":" << service.vram_cache_bytes
-      << ",\"routed_vram_policy\":\"" << service.routed_vram_policy << '"'
-      << ",\"placement_prefetch_enabled\":"
-      << flag(service.placement_prefetch_enabled)
-      << ",\"placement_prefetch_state\":\"" << service.placement_prefetch_state
-      << "\",\"placement_minimum_observations\":"
-      << service.placement_minimum_observations << "}\n"
-      << std::flush;
-}
+class Service final {
+ public:
+  Service(const Engine& engine, const LaunchOptions& options)
+      : engine_(engine), options_(options) {}
 
-int worker_loop(const er::ModelDescriptor& model,
-                const er::ExecutionProviderModule& module,
-                const qllm::PreparedProgram& prepared,
-                const LaunchOptions& options) {
-  const auto ports = service_ports(model);
-  const auto provider = std::dynamic_pointer_cast<qllm::Mi355DenseFp4Provider>(
-      module.definition.implementation);
-  require(provider != nullptr, "callable provider module has no implementation");
-  std::unordered_map<std::uint64_t, ActiveRequest> active;
-  std::uint64_t program_steps{}, program_step_ns{}, useful_tokens{};
-  std::uint64_t exact_calls{}, exact_positions{}, exact_accepted{}, cancelled{};
-  // :670-676
-  const auto exact_eligible = [&](const Sampling& sampling) {
-    if (!model.exact_decode_program) return false;
-    if (!sampling.enabled()) return true;
-    return model.exact_decode_program->abi_version >= 2U && sampling.top_k != 0U &&
-           sampling.top_k <= 64U;
-  };
-  const auto page_count = [&](std::uint32_t tokens) {
-    return (std::uint64_t{tokens} + module.service.kv_page_tokens - 1U) /
-           module.service.kv_page_tokens;
-  };
-  print_ready(model, module.service, options);
-
-  // one program step on `tokens` at consecutive positions; the head's token
-  const auto run_program = [&](ActiveRequest& request,
-                               std::span<const std::uint32_t> tokens,
-                               std::uint32_t first_position) {
-    std::vector<std::uint32_t> positions(tokens.size());
-    for (std::size_t index = 0; index < positions.size(); ++index)
-      positions[index] = first_position + static_cast<std::uint32_t>(index);
-    std::map<std::string, er::ExecutionValue, std::less<>> inputs;
-    inputs.emplace(ports.token_input, host_words(tokens, kTokenAbi));
-    inputs.emplace(ports.position_input, host_words(positions, kPositionAbi));
-    auto result = request.session->execute(std::move(inputs));
-    require(result.status.ok(), result.status.message());
-    const auto output = result.values.find(ports.token_output);
-    require(output != result.values.end(),
-            "model program did not publish its token output");
-    const auto& value = output->second;
-    require(value.valid() && value.abi == kTokenAbi && value.memory_domain == "host" &&
-                value.bytes >= sizeof(std::uint32_t) &&
-                value.bytes % sizeof(std::uint32_t) == 0U,
-            "callable VM returned an invalid token value");
-    std::uint32_t token{};
-    std::memcpy(&token, value.data + value.bytes - sizeof(token), sizeof(token));
-    return token;
-  };
-
-  // The prompt (feed, :679-857).  Long prompts go through the provider's tall
-  // prefill, which also feeds the proposer and rolls the first drafts out when
-  // the request will be decoded speculatively; short ones take the program in
-  // batches of prefill_chunk_tokens with a synchronisation after each.
-  const auto feed = [&](ActiveRequest& request,
-                        std::span<const std::uint32_t> tokens,
-                        std::uint32_t first_position) {
-    const auto began = std::chrono::steady_clock::now();
-    const bool exact = exact_eligible(request.sampling) &&
-                       request.session->exact_decode_available();
-    const std::uint32_t chunk =
-        std::max<std::uint32_t>(1U, module.service.prefill_chunk_tokens);
-    if (tokens.size() > chunk) {
-      const auto result = provider->prefill(request.session->state(), tokens,
-                                            first_position,
-                                            request.session->request());
-      require(result.status.ok(), result.status.message());
-      request.predicted = result.predicted;
-    } else {
-      for (std::size_t offset = 0; offset < tokens.size();) {
-        const auto count = std::min<std::size_t>(chunk, tokens.size() - offset);
-        const auto position = first_position + static_cast<std::uint32_t>(offset);
-        request.predicted = run_program(request, tokens.subspan(offset, count), position);
-        if (exact) {
-          std::vector<std::uint32_t> successors(count);
-          for (std::size_t row = 0; row < count; ++row)
-            successors[row] = offset + row + 1U == tokens.size()
-                                  ? request.predicted
-                                  : tokens[offset + row + 1U];
-          const auto status = request.session->synchronize_exact_decode_batch(
-              successors, position, offset + count == tokens.size());
-          require(status.ok(), status.message());
-        }
-        offset += count;
+  int serve(std::istream& in, std::ostream& out) {
+    out_ = &out;
+    announce();
+    std::string line;
+    while (open_ && std::getline(in, line)) {
+      try {
+        dispatch(line);
+      } catch (const std::exception& error) {
+        JsonLine("error").string("message", error.what()).send(out);
       }
     }
-    program_steps += tokens.size();
-    program_step_ns += static_cast<std::uint64_t>(
-        std::chrono::duration_cast<std::chrono::nanoseconds>(
-            std::chrono::steady_clock::now() - began)
-            .count());
-    request.next_position = first_position + static_cast<std::uint32_t>(tokens.size());
+    return 0;
+  }
+
+ private:
+  using Handler = void (Service::*)(FieldCursor&);
+  struct Command final {
+    std::string_view verb;
+    Handler handler;
+  };
+  void dispatch(std::string_view line) {
+    static constexpr std::array<Command, 12> kCommands{{
+        {"PING", &Service::ping},
+        {"BEGIN", &Service::begin},
+        {"STEP", &Service::step},
+        {"NEXT", &Service::next},
+        {"CANCEL", &Service::cancel},
+        {"END", &Service::end},
+        {"DROP", &Service::drop},
+        {"SAVE", &Service::persistence},
+        {"LOAD", &Service::persistence},
+        {"PRUNE", &Service::persistence},
+        {"STATS", &Service::stats},
+        {"SHUTDOWN", &Service::shutdown},
+    }};
+    FieldCursor fields(line);
+    verb_ = fields.text();
+    for (const auto& command : kCommands)
+      if (command.verb == verb_) return (this->*command.handler)(fields);
+    wire::fail("unknown worker command");
+  }
+
+  // the ready line: every field the service's worker client reads
+  // (ops/python/expert_server.py:575-700)
+  void announce() {
+    const auto& model = engine_.model();
+    const auto& s = engine_.module().service;
+    std::uint64_t draft_depth = 0U;
+    if (const auto& decode = model.exact_decode_program)
+      if (const auto found = decode->parameters.find("draft_depth");
+          found != decode->parameters.end())
+        draft_depth = found->second;
+    std::vector<std::string> capabilities;
+    for (const auto& kernel : model.required_kernels)
+      capabilities.push_back(kernel.capability);
+    JsonLine("ready")
+        .number("protocol", 13U)
+        .number("capacity", options_.capacity)
+        .string("architecture_id", model.architecture_id)
+        .number("vocab_size", model.vocab_size)
+        .number("max_context_tokens", model.max_context_tokens)
+        .number("routed_layers", 0U)
+        .number("experts_per_layer", 0U)
+        .number("route_width", 0U)
+        .string("expert_encoding", "")
+        .strings("operation_capabilities", capabilities)
+        .string("prefill_mode", s.prefill_mode)
+        .number("prefill_chunk_tokens", engine_.chunk_tokens())
+        .boolean("session_retention", s.session_retention)
+        .boolean("session_parking", s.session_parking)
+        .boolean("session_persistence", s.session_persistence)
+        .number("session_park_ram_bytes", s.session_park_ram_bytes)
+        .number("session_park_page_capacity", s.session_park_page_capacity)
+        .string("request_stream_mode", s.request_stream_mode)
+        .boolean("gpu_phase_timing", engine_.provider().profiles_gpu_phases())
+        .boolean("sampling_supported", s.sampling_supported)
+        .boolean("sampling_presence_penalty_supported", s.sampling_supported)
+        .boolean("mtp_resource_available", s.mtp_resource_available)
+        .boolean("mtp_runtime_ready", s.mtp_runtime_ready)
+        .boolean("mtp_enabled", s.mtp_enabled)
+        .number("mtp_draft_depth", draft_depth)
+        .boolean("retain_previous_route", s.retain_previous_route)
+        .boolean("cpu_hybrid_enabled", s.cpu_hybrid_enabled)
+        .string("rope_mode", s.rope_mode)
+        .string("kv_dtype", s.kv_dtype)
+        .string("kv_allocation", s.kv_allocation)
+        .number("kv_page_tokens", s.kv_page_tokens)
+        .number("kv_page_bytes", s.kv_page_bytes)
+        .number("kv_page_capacity", s.kv_page_capacity)
+        .string("placement_mode", s.placement_mode)
+        .string("placement_profile", s.placement_profile)
+        .number("ram_cache_bytes", s.ram_cache_bytes)
+        .number("vram_cache_bytes", s.vram_cache_bytes)
+        .string("routed_vram_policy", s.routed_vram_policy)
+        .boolean("placement_prefetch_enabled", s.placement_prefetch_enabled)
+        .string("placement_prefetch_state", s.placement_prefetch_state)
+        .number("placement_minimum_observations", s.placement_minimum_observations)
+        .send(*out_);
+  }
+
+  void ping(FieldCursor& fields) {
+    expect(fields.done(), "invalid PING");
+    JsonLine("pong").send(*out_);
+  }
+
+  // BEGIN <id> <context> <tokens> [RESUME ..|MULTIMODAL ..|CHECKPOINT ..]
+  //       [SAMPLING t p k m presence seed]
+  void begin(FieldCursor& fields) {
+    expect(fields.left() >= 3U, "invalid BEGIN");
+    const auto id = fields.natural();
+    const auto context = fields.natural();
+    expect(id != 0U && requests_.find(id) == requests_.end() && context >= 2U &&
+               context <= options_.max_context,
+           "invalid BEGIN request identity or context");
+    const auto prompt = wire::token_list(fields.text(), engine_.model().vocab_size);
+    expect(prompt.size() < context, "prompt exhausts request context");
+    if (fields.keyword("RESUME")) wire::fail(kNoRetention);
+    expect(!prompt.empty(), "fresh BEGIN has no prompt");
+    if (fields.keyword("MULTIMODAL"))
+      wire::fail("artifact does not accept multimodal input");
+    if (fields.keyword("CHECKPOINT")) wire::fail(kNoRetention);
+    SamplingProfile profile;
+    if (fields.keyword("SAMPLING"))
+      profile = SamplingProfile::read(fields, engine_.model().vocab_size);
+    expect(fields.done(), "unknown BEGIN request fields");
+    expect(requests_.size() < options_.capacity,
+           "callable provider capacity is exhausted");
+    auto request = std::make_unique<Request>(
+        engine_, id, static_cast<std::uint32_t>(context), profile, prompt.size());
+    request->ingest(prompt, counters_);
+    requests_.emplace(id, std::move(request));
+    JsonLine("begun").number("id", id).send(*out_);
+  }
+
+  struct Turn final {
+    std::uint64_t id{};
+    StepMode mode{};
+    std::vector<std::uint32_t> emitted;
   };
 
-  std::string line;
-  while (std::getline(std::cin, line)) {
-    try {
-      const auto fields = split_tabs(line);
-      require(!fields.empty(), "empty worker command");
-      if (fields[0] == "PING") {
-        require(fields.size() == 1U, "invalid PING");
-        std::cout << "{\"type\":\"pong\"}\n" << std::flush;
-      } else if (fields[0] == "BEGIN") {
-        require(fields.size() >= 4U, "invalid BEGIN");
-        const auto id = std::stoull(std::string(fields[1]));
-        const auto context = std::stoull(std::string(fields[2]));
-        require(id != 0U && !active.contains(id) && context >= 2U &&
-                    context <= options.max_context,
-                "invalid BEGIN request identity or context");
-        const auto prompt = parse_tokens(fields[3], model.vocab_size);
-        require(prompt.size() < context, "prompt exhausts request context");
-        std::size_t field = 4U;
-        if (field < fields.size() && fields[field] == "RESUME")
-          throw std::runtime_error(
-              "callable provider does not support session retention");
-        require(!prompt.empty(), "fresh BEGIN has no prompt");
-        if (field < fields.size() && fields[field] == "MULTIMODAL")
-          throw std::runtime_error("artifact does not accept multimodal input");
-        if (field < fields.size() && fields[field] == "CHECKPOINT")
-          throw std::runtime_error(
-              "callable provider does not support session retention");
-        Sampling sampling;
-        if (field < fields.size() && fields[field] == "SAMPLING") {
-          require(field + 6U < fields.size(), "invalid BEGIN sampling marker");
-          const auto temperature = std::stoull(std::string(fields[field + 1U]));
-          const auto top_p = std::stoull(std::string(fields[field + 2U]));
-          const auto top_k = std::stoull(std::string(fields[field + 3U]));
-          const auto min_p = std::stoull(std::string(fields[field + 4U]));
-          const auto presence = std::stoll(std::string(fields[field + 5U]));
-          sampling.seed = std::stoull(std::string(fields[field + 6U]));
-          require(temperature <= 2000000U && top_p != 0U && top_p <= 1000000U &&
-                      top_k <= model.vocab_size && min_p <= 1000000U &&
-                      presence >= -2000000LL && presence <= 2000000LL,
-                  "invalid BEGIN sampling values");
-          sampling.temperature_ppm = static_cast<std::uint32_t>(temperature);
-          sampling.top_p_ppm = static_cast<std::uint32_t>(top_p);
-          sampling.top_k = static_cast<std::uint32_t>(top_k);
-          sampling.min_p_ppm = static_cast<std::uint32_t>(min_p);
-          sampling.presence_penalty_ppm = static_cast<std::int32_t>(presence);
-          field += 7U;
-        }
-        require(field == fields.size(), "unknown BEGIN request fields");
-        require(active.size() < options.capacity,
-                "callable provider capacity is exhausted");
-        ActiveRequest request;
-        request.sampling = sampling;
-        const auto status = qllm::ProgramSession::begin(
-            model, module, prepared,
-            request_context(id, static_cast<std::uint32_t>(context),
-                            static_cast<std::uint32_t>(prompt.size() - 1U), sampling,
-                            exact_eligible(sampling)),
-            request.session);
-        require(status.ok(), status.message());
-        feed(request, prompt, 0U);
-        request.context_limit = static_cast<std::uint32_t>(context);
-        active.emplace(id, std::move(request));
-        std::cout << "{\"type\":\"begun\",\"id\":" << id << "}\n" << std::flush;
-      } else if (fields[0] == "STEP" || fields[0] == "NEXT") {
-        std::vector<std::pair<std::uint64_t, std::uint32_t>> items;
-        std::set<std::uint64_t> unique;
-        const auto parse_item = [&](std::string_view item) {
-          const auto comma = item.find(',');
-          require(comma != std::string_view::npos, "invalid STEP item");
-          const auto id = std::stoull(std::string(item.substr(0U, comma)));
-          const auto mode = item.substr(comma + 1U);
-          require(active.contains(id) && unique.insert(id).second &&
-                      (mode == "0" || mode == "1" || mode == "2"),
-                  "STEP request mismatch");
-          items.emplace_back(id, mode == "1" ? 1U : mode == "2" ? 2U : 0U);
-        };
-        if (fields[0] == "NEXT") {
-          require(fields.size() == 3U, "invalid NEXT");
-          parse_item(std::string(fields[1]) + "," + std::string(fields[2]));
-        } else {
-          require(fields.size() >= 2U && fields.size() <= options.capacity + 1U,
-                  "invalid STEP");
-          for (std::size_t index = 1U; index < fields.size(); ++index)
-            parse_item(fields[index]);
-        }
-        std::vector<std::vector<std::uint32_t>> emitted(items.size());
-        const auto began = std::chrono::steady_clock::now();
-        for (std::size_t index = 0; index < items.size(); ++index) {
-          const auto [id, mode] = items[index];
-          auto& request = active.at(id);
-          if (mode == 1U) {
-            emitted[index] = {request.predicted};
-            continue;
-          }
-          require(request.next_position < request.context_limit,
-                  "request context is exhausted");
-          const bool exact = exact_eligible(request.sampling) &&
-                             request.session->exact_decode_available();
-          if (mode == 0U && exact &&
-              request.next_position + 1U < request.context_limit) {
-            auto result = request.session->execute_exact_decode(
-                request.predicted, request.next_position, request.context_limit);
-            require(result.status.ok(), result.status.message());
-            emitted[index] = std::move(result.emitted_tokens);
-            request.predicted = result.next_token;
-            request.next_position += result.positions_advanced;
-            program_steps += result.positions_advanced;
-            ++exact_calls;
-            exact_positions += result.positions_advanced;
-            exact_accepted += result.positions_advanced - 1U;
-            continue;
-          }
-          emitted[index] = {request.predicted};
-          const std::uint32_t token[1] = {request.predicted};
-          request.predicted = run_program(request, token, request.next_position);
-          ++request.next_position;
-          if (exact) {
-            const std::uint32_t successor[1] = {request.predicted};
-            const auto status = request.session->synchronize_exact_decode_batch(
-                successor, request.next_position - 1U, true);
-            require(status.ok(), status.message());
-          }
-          ++program_steps;
-        }
-        program_step_ns += static_cast<std::uint64_t>(
-            std::chrono::duration_cast<std::chrono::nanoseconds>(
-                std::chrono::steady_clock::now() - began)
-                .count());
-        for (const auto& tokens : emitted) useful_tokens += tokens.size();
-        const auto print_tokens = [](const std::vector<std::uint32_t>& tokens) {
-          for (std::size_t index = 0; index < tokens.size(); ++index)
-            std::cout << (index ? "," : "") << tokens[index];
-        };
-        if (fields[0] == "NEXT") {
-          std::cout << "{\"type\":\"token\",\"id\":" << items[0].first
-                    << ",\"tokens\":[";
-          print_tokens(emitted[0]);
-          std::cout << "]}\n";
-        } else {
-          std::cout << "{\"type\":\"batch\",\"items\":[";
-          for (std::size_t index = 0; index < items.size(); ++index) {
-            std::cout << (index ? "," : "") << "{\"id\":" << items[index].first
-                      << ",\"tokens\":[";
-            print_tokens(emitted[index]);
-            std::cout << "]}";
-          }
-          std::cout << "]}\n";
-        }
-        std::cout << std::flush;
-        for (const auto [id, mode] : items)
-          if (mode == 1U) active.erase(id);
-      } else if (fields[0] == "CANCEL") {
-        require(fields.size() == 2U, "invalid CANCEL");
-        if (active.erase(std::stoull(std::string(fields[1])))) ++cancelled;
-      } else if (fields[0] == "END") {
-        require(fields.size() == 2U || fields.size() == 4U || fields.size() == 6U,
-                "invalid END");
-        const auto id = std::stoull(std::string(fields[1]));
-        const auto found = active.find(id);
-        require(found != active.end(), "unknown active request");
-        require(fields.size() == 2U,
-                "callable provider does not support session retention");
-        active.erase(found);
-        ++cancelled;
-        std::cout << "{\"type\":\"ended\",\"id\":" << id << "}\n" << std::flush;
-      } else if (fields[0] == "DROP") {
-        require(fields.size() == 2U, "invalid DROP");
-        throw std::runtime_error(
-            "callable provider does not support session retention");
-      } else if (fields[0] == "SAVE" || fields[0] == "LOAD" || fields[0] == "PRUNE") {
-        require(fields.size() == (fields[0] == "LOAD" ? 15U : 4U),
-                std::string("invalid ") + std::string(fields[0]));
-        throw std::runtime_error(
-            "callable provider does not support session persistence");
-      } else if (fields[0] == "STATS") {
-        require(fields.size() == 1U, "invalid STATS");
-        std::uint64_t reserved_pages{};
-        for (const auto& [id, request] : active)
-          reserved_pages += page_count(request.next_position);
-        auto telemetry = module.telemetry
-                             ? module.telemetry()
-                             : std::map<std::string, std::uint64_t, std::less<>>{};
-        telemetry["program_steps"] = program_steps;
-        telemetry["program_step_ns"] = program_step_ns;
-        telemetry["useful_tokens"] = useful_tokens;
-        telemetry["exact_decode_calls"] = exact_calls;
-        telemetry["exact_decode_positions"] = exact_positions;
-        telemetry["exact_decode_accepted_tokens"] = exact_accepted;
-        telemetry["cancelled_requests"] = cancelled;
-        telemetry["active_requests"] = active.size();
-        telemetry["retained_sessions"] = 0U;
-        telemetry["parked_sessions"] = 0U;
-        telemetry["parked_pages"] = 0U;
-        telemetry.try_emplace("kv_allocated_pages", reserved_pages);
-        telemetry["kv_reserved_pages"] = reserved_pages;
-        std::cout << "{\"type\":\"stats\"";
-        for (const auto& [name, value] : telemetry)
-          std::cout << ",\"" << json_text(name) << "\":" << value;
-        std::cout << "}\n" << std::flush;
-      } else if (fields[0] == "SHUTDOWN") {
-        require(fields.size() == 1U && active.empty(),
-                "SHUTDOWN requires no retained state");
-        std::cout << "{\"type\":\"shutdown\"}\n" << std::flush;
-        return 0;
-      } else {
-        throw std::runtime_error("unknown worker command");
-      }
-    } catch (const std::exception& error) {
-      std::cout << "{\"type\":\"error\",\"message\":\"" << json_text(error.what())
-                << "\"}\n"
-                << std::flush;
-    }
+  Turn turn(std::string_view id_text, std::string_view mode_text,
+            std::span<const Turn> earlier) const {
+    Turn next;
+    next.id = wire::decimal<std::uint64_t>(id_text);
+    const bool repeated = std::any_of(
+        earlier.begin(), earlier.end(),
+        [&](const Turn& other) { return other.id == next.id; });
+    expect(!repeated && requests_.find(next.id) != requests_.end(),
+           "STEP request mismatch");
+    next.mode = step_mode(mode_text);
+    return next;
   }
-  return 0;
+
+  // runs the turns in order, then retires the requests that emitted their
+  // closing token
+  void take_turns(std::vector<Turn>& turns) {
+    const Stopwatch watch;
+    for (auto& item : turns)
+      item.emitted = requests_.at(item.id)->advance(item.mode, counters_);
+    counters_.program_step_ns += watch.nanoseconds();
+    for (const auto& item : turns) counters_.useful_tokens += item.emitted.size();
+  }
+
+  void retire(std::span<const Turn> turns) {
+    for (const auto& item : turns)
+      if (item.mode == StepMode::finish) requests_.erase(item.id);
+  }
+
+  // STEP <id>,<mode> [<id>,<mode> ...]: one batch reply for all of them
+  void step(FieldCursor& fields) {
+    expect(fields.left() >= 1U && fields.left() <= options_.capacity, "invalid STEP");
+    std::vector<Turn> turns;
+    while (!fields.done()) {
+      const auto item = fields.text();
+      const auto comma = item.find(',');
+      expect(comma != std::string_view::npos, "invalid STEP item");
+      turns.push_back(turn(item.substr(0U, comma), item.substr(comma + 1U), turns));
+    }
+    take_turns(turns);
+    JsonLine reply("batch");
+    reply.begin_items("items");
+    for (const auto& item : turns) reply.item(item.id, item.emitted);
+    reply.end_items().send(*out_);
+    retire(turns);
+  }
+
+  // NEXT <id> <mode>: the single-request form, answered with a token line
+  void next(FieldCursor& fields) {
+    expect(fields.left() == 2U, "invalid NEXT");
+    const auto id_text = fields.text();
+    std::vector<Turn> turns{turn(id_text, fields.text(), {})};
+    take_turns(turns);
+    JsonLine("token").number("id", turns[0].id).numbers("tokens", turns[0].emitted)
+        .send(*out_);
+    retire(turns);
+  }
+
+  // CANCEL <id>: no reply line; an unknown id is not an error (the request
+  // may have ended on its own meanwhile)
+  void cancel(FieldCursor& fields) {
+    expect(fields.left() == 1U, "invalid CANCEL");
+    counters_.cancelled += requests_.erase(fields.natural());
+  }
+
+  // END <id> [RETAIN <key> [AT <tokens>]]
+  void end(FieldCursor& fields) {
+    expect(fields.left() == 1U || fields.left() == 3U || fields.left() == 5U,
+           "invalid END");
+    const auto id = fields.natural();
+    const auto found = requests_.find(id);
+    expect(found != requests_.end(), "unknown active request");
+    expect(fields.done(), kNoRetention);
+    requests_.erase(found);
+    ++counters_.cancelled;
+    JsonLine("ended").number("id", id).send(*out_);
+  }
+
+  void drop(FieldCursor& fields) {
+    expect(fields.left() == 1U, "invalid DROP");
+    wire::fail(kNoRetention);
+  }
+
+  // SAVE / PRUNE <a> <b> <c>, LOAD with its fourteen fields
+  void persistence(FieldCursor& fields) {
+    const std::size_t arguments = verb_ == "LOAD" ? 14U : 3U;
+    expect(fields.left() == arguments, "invalid " + std::string(verb_));
+    wire::fail(kNoPersistence);
+  }
+
+  void stats(FieldCursor& fields) {
+    expect(fields.done(), "invalid STATS");
+    const std::uint64_t page_tokens = engine_.module().service.kv_page_tokens;
+    std::uint64_t reserved_pages = 0U;
+    for (const auto& [id, request] : requests_)
+      reserved_pages += (request->position() + page_tokens - 1U) / page_tokens;
+    std::map<std::string, std::uint64_t, std::less<>> figures;
+    if (engine_.module().telemetry) figures = engine_.module().telemetry();
+    figures.try_emplace("kv_allocated_pages", reserved_pages);
+    const std::pair<const char*, std::uint64_t> own[] = {
+        {"program_steps", counters_.program_steps},
+        {"program_step_ns", counters_.program_step_ns},
+        {"useful_tokens", counters_.useful_tokens},
+        {"exact_decode_calls", counters_.exact_calls},
+        {"exact_decode_positions", counters_.exact_positions},
+        {"exact_decode_accepted_tokens", counters_.exact_accepted},
+        {"cancelled_requests", counters_.cancelled},
+        {"active_requests", requests_.size()},
+        {"retained_sessions", 0U},
+        {"parked_sessions", 0U},
+        {"parked_pages", 0U},
+        {"kv_reserved_pages", reserved_pages},
+    };
+    for (const auto& [name, value] : own) figures[name] = value;
+    JsonLine reply("stats");
+    for (const auto& [name, value] : figures) reply.number(name, value);
+    reply.send(*out_);
+  }
+
+  void shutdown(FieldCursor& fields) {
+    expect(fields.done() && requests_.empty(), "SHUTDOWN requires no retained state");
+    JsonLine("shutdown").send(*out_);
+    open_ = false;
+  }
+
+  const Engine& engine_;
+  const LaunchOptions& options_;
+  std::ostream* out_{};
+  std::string_view verb_;
+  std::map<std::uint64_t, std::unique_ptr<Request>> requests_;
+  Counters counters_;
+  bool open_{true};
+};
+
+int run(int argc, char** argv) {
+  const auto options = parse_launch_options(argc, argv);
+  auto artifact = std::make_shared<er::ModelArtifact>();
+  expect_ok(er::ModelArtifact::load(std::filesystem::path(argv[1]), *artifact));
+  if (options.mtp_draft_depth)
+    expect_ok(artifact->configure_mtp_draft_depth(*options.mtp_draft_depth));
+  const er::ModelDescriptor& model = artifact->model();
+  require(model.schema_version >= 3U,
+          "callable VM service requires a schema v3 artifact");
+  // exactly one module must cover the program (moe_vm_runner.cpp:431-497);
+  // this worker links one
+  require(er::provider_supports_model(model,
+                                      make_mi355_dense_fp4_provider().capabilities)
+              .ok(),
+          "no callable provider implements the artifact program");
+  ArtifactProviderOptions provider_options;
+  provider_options.max_context = options.max_context;
+  provider_options.capacity = options.capacity;
+  provider_options.kv_page_tokens = options.kv_page_tokens;
+  provider_options.kv_cache_dtype = options.kv_cache_dtype;
+  provider_options.vram_cache_bytes = options.vram_cache_gib << 30U;
+  provider_options.routed_vram_policy = options.routed_vram_policy;
+  provider_options.profile_gpu_phases = options.profile_gpu_phases;
+  auto created = make_mi355_dense_fp4_module(artifact, provider_options);
+  expect_ok(created.status);
+  PreparedProgram prepared;
+  expect_ok(prepare_program(model, created.module, prepared));
+  if (created.module.finalize_service)
+    expect_ok(created.module.finalize_service(created.module.service));
+  check_service_contract(model, created.module, options);
+  const Engine engine(model, created.module, prepared, options);
+  return Service(engine, options).serve(std::cin, std::cout);
 }
 
 }  // namespace
+}  // namespace qllm::worker
 
 int main(int argc, char** argv) {
+  if (argc < 3 || std::string_view(argv[2]) != "--worker") {
+    std::cerr << "usage: qllm-worker <artifact> --worker <resource-options>\n";
+    return 64;
+  }
   try {
-    if (argc < 3 || std::string_view(argv[2]) != "--worker") {
-      std::cerr << "usage: qllm-worker <artifact> --worker <resource-options>\n";
-      return 64;
-    }
-    const auto options = parse_launch_options(argc, argv);
-    const std::filesystem::path root(argv[1]);
-    auto artifact = std::make_shared<er::ModelArtifact>();
-    auto status = er::ModelArtifact::load(root, *artifact);
-    require(status.ok(), status.message());
-    if (options.mtp_draft_depth) {
-      status = artifact->configure_mtp_draft_depth(*options.mtp_draft_depth);
-      require(status.ok(), status.message());
-    }
-    require(artifact->model().schema_version >= 3U,
-            "callable VM service requires a schema v3 artifact");
-    // create_module (:431-497): exactly one module must cover the program;
-    // this worker links one
-    const auto metadata = qllm::make_mi355_dense_fp4_provider();
-    require(er::provider_supports_model(artifact->model(), metadata.capabilities).ok(),
-            "no callable provider implements the artifact program");
-    qllm::ArtifactProviderOptions provider_options;
-    provider_options.max_context = options.max_context;
-    provider_options.kv_page_tokens = options.kv_page_tokens;
-    provider_options.kv_cache_dtype = options.kv_cache_dtype;
-    provider_options.vram_cache_bytes = options.vram_cache_gib << 30U;
-    provider_options.routed_vram_policy = options.routed_vram_policy;
-    require(options.capacity == 1U,
-            "this provider serves one request at a time (--capacity=1)");
-    auto created = qllm::make_mi355_dense_fp4_module(artifact, provider_options);
-    require(created.status.ok(), created.status.message());
-    require(created.module.definition.implementation != nullptr,
-            "callable provider module has no implementation");
-    qllm::PreparedProgram prepared;
-    status = qllm::prepare_program(artifact->model(), created.module, prepared);
-    require(status.ok(), status.message());
-    if (created.module.finalize_service) {
-      status = created.module.finalize_service(created.module.service);
-      require(status.ok(), status.message());
-    }
-    validate_service_contract(artifact->model(), created.module, options);
-    return worker_loop(artifact->model(), created.module, prepared, options);
+    return qllm::worker::run(argc, argv);
   } catch (const std::exception& error) {
     std::cerr << "qllm worker: " << error.what() << '\n';
     return 1;

@@ -31,7 +31,9 @@ def library():
         lib = ctypes.CDLL(LIBRARY)
         lib.qvm_open.restype = c_void_p
         lib.qvm_open.argtypes = [c_char_p, c_uint32, c_uint32, c_char_p, c_uint32,
-                                 c_char_p, c_size_t]
+                                 c_uint32, c_char_p, c_size_t]
+        lib.qvm_select_session.argtypes = [c_void_p, c_uint32]
+        lib.qvm_end_session.argtypes = [c_void_p]
         lib.qvm_close.argtypes = [c_void_p]
         lib.qvm_error.restype = c_char_p
         lib.qvm_error.argtypes = [c_void_p]
@@ -54,12 +56,13 @@ def library():
 
 class Machine:
     def __init__(self, root, max_context, kv_page_tokens, kv_cache_dtype="artifact",
-                 mtp_draft_depth=0, vocabulary=0):
+                 mtp_draft_depth=0, vocabulary=0, capacity=1):
         self.lib = library()
         self.vocabulary = vocabulary
         message = create_string_buffer(2048)
         self.handle = self.lib.qvm_open(os.fsencode(root), max_context, kv_page_tokens,
-                                        kv_cache_dtype.encode(), mtp_draft_depth, message, 2048)
+                                        kv_cache_dtype.encode(), mtp_draft_depth, capacity,
+                                        message, 2048)
         if not self.handle:
             raise VmError(message.value.decode())
 
@@ -80,6 +83,14 @@ class Machine:
         return dict(kv_dtype=dtype.value.decode(), kv_page_tokens=page.value,
                     prefill_chunk_tokens=chunk.value, mtp_enabled=bool(mtp.value),
                     sampling_supported=bool(sampling.value))
+
+    def select(self, session):
+        """Which session (0 .. capacity; the last has no slot to count on) the
+        calls that follow address."""
+        self._check(self.lib.qvm_select_session(self.handle, session))
+
+    def end_session(self):
+        self._check(self.lib.qvm_end_session(self.handle))
 
     def begin_session(self, **parameters):
         names = (c_char_p * len(parameters))(*[n.encode() for n in parameters])
