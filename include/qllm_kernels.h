@@ -181,6 +181,31 @@ int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,
                                    float* partials, uint32_t k_splits,
                                    uint32_t batch, void* stream);
 
+/* Balanced forms of the two launches above and below whose tile count leaves a
+ * ragged last round over the CUs (the q/k/v launch: 320 tiles, the gate/up
+ * launch: 544 tile pairs, on 256 CUs): the tiles past the last full round are
+ * cut along K over as many small workgroups as give every CU one more, equal,
+ * share; the small workgroup that finishes a tile last adds the others' sums in
+ * a fixed order and runs the epilogue.  Values of the cut tiles differ from the
+ * plain launch in F32 summation order only.  `workspace`: device memory of
+ * qllm_fp4_gemm_balance_workspace_bytes() bytes, 16-byte aligned, zeroed once
+ * by the caller and then left alone (the kernel returns its counters to zero);
+ * launches that share a workspace must not overlap.  No counterpart in the
+ * reference, whose launches have one thread block per output row group
+ * (transformer_kernels.cu:7559-7593). */
+size_t qllm_fp4_gemm_balance_workspace_bytes(void);
+int32_t qllm_fp4_gemm_bf16_split_balanced(const qllm_fp4_matrix* matrix,
+                                          const void* input, size_t input_bytes,
+                                          const qllm_gemm_segment* segments,
+                                          uint32_t segment_count, uint32_t batch,
+                                          void* workspace, size_t workspace_bytes,
+                                          void* stream);
+int32_t qllm_fp4_swiglu_bf16_balanced(const qllm_fp4_matrix* gate,
+                                      const qllm_fp4_matrix* up, const void* input,
+                                      size_t input_bytes, void* output,
+                                      uint32_t batch, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
 /* Gate and up projections of one SwiGLU block in a single pass over a shared
  * BF16 input: out[m,n] = bf16(bf16(silu(gate[m,n])) * up[m,n]) stored as
  * bf16 [batch, rows].  Fuses two qllm_fp4_gemm_bf16 calls with silu_product

@@ -24,6 +24,7 @@
 //    for a K that is a multiple of 64.
 #include "common.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 
 namespace qllm {
@@ -88,6 +89,20 @@ struct GemmArgs {
   uint32_t segment_rows[3];
   uint32_t segment_kind[3];
   void* segment_output[3];
+  // Balanced tail: a launch whose tile count is not a multiple of the CU
+  // count leaves a few CUs with one workgroup more than the rest, and the
+  // launch lasts as long as they do.  With balance_splits > 1 the tiles from
+  // balance_first_tile on are cut along K over balance_splits small
+  // workgroups each (grid = balance_first_tile + extra tiles * splits), so
+  // that every CU gets the same share.  A small workgroup leaves its sums in
+  // balance_partials [extra tile][split][TILES][items] (write-through stores)
+  // and bumps the tile's counter; the one that finds it at splits - 1 adds the
+  // partials in split order, whichever workgroup it is, runs the epilogue and
+  // puts the counter back to zero.  Nobody waits for anybody.
+  uint32_t balance_first_tile;
+  uint32_t balance_splits;
+  float* balance_partials;
+  uint32_t* balance_counters;
 };
 
 // Epilogue store of one value.
@@ -103,6 +118,16 @@ __device__ __forceinline__ void store_output(void* output, uint32_t kind,
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Balanced tail (GemmArgs::balance_*): most small workgroups per cut tile, and
+// the layout of the workspace that serves it - one counter per cut tile, then
+// the partials.
+constexpr uint32_t kMaxBalanceSplits = 8;
+constexpr uint32_t kMaxBalanceTiles = 128;
+constexpr size_t kBalanceCounterBytes = 4096;
+constexpr size_t kBalanceWorkspaceBytes =
+    kBalanceCounterBytes +
+    size_t{kMaxBalanceTiles} * kMaxBalanceSplits * 2u * 256u * sizeof(float);
 
 // 4x4 transpose of dwords across the four 16-lane rows of a wave: on return
 // register d of row c holds what register c of row d held.
@@ -178,9 +203,17 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint32_t h = args.tile_rows;
   const uint32_t half_rows = h / 2u;
   const uint32_t tile_lane = n < half_rows ? n : half_rows - 1u;
-  const uint32_t splits = args.k_splits > 1u ? args.k_splits : 1u;
-  const uint32_t tile_index = blockIdx.x / splits;
-  const uint32_t split = blockIdx.x - tile_index * splits;
+  const bool balanced =
+      args.balance_splits > 1u && blockIdx.x >= args.balance_first_tile;
+  const uint32_t splits =
+      balanced ? args.balance_splits : (args.k_splits > 1u ? args.k_splits : 1u);
+  const uint32_t extra_index =
+      balanced ? (blockIdx.x - args.balance_first_tile) / splits : 0u;
+  const uint32_t tile_index =
+      balanced ? args.balance_first_tile + extra_index : blockIdx.x / splits;
+  const uint32_t split =
+      balanced ? blockIdx.x - args.balance_first_tile - extra_index * splits
+               : blockIdx.x - tile_index * splits;
   const uint32_t first_row = tile_index * h;
 
   // Weight and scale streams: wave-uniform start of the tile's stream plus a
@@ -411,16 +444,64 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       }
   __syncthreads();
 
-  if (!item_valid) return;
   float total = 0.0f;
+  float up = 0.0f;   // tile 1 is the up projection of the same rows
+  if (threadIdx.x < kItems) {
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) total += reduce[w][0][item_half][item_reg][item_lane];
+    for (int w = 0; w < WAVES; ++w) {
+      total += reduce[w][0][item_half][item_reg][item_lane];
+      if (TILES == 2) up += reduce[w][TILES - 1][item_half][item_reg][item_lane];
+    }
+  }
+  if (balanced) {
+    // hand the sums over; the last of the tile's workgroups finishes it
+    float* const slot = args.balance_partials +
+                        static_cast<size_t>(extra_index) * splits * TILES * kItems;
+    if (threadIdx.x < kItems) {
+      float* const mine = slot + static_cast<size_t>(split) * TILES * kItems;
+      __hip_atomic_store(mine + threadIdx.x, total, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      if (TILES == 2)
+        __hip_atomic_store(mine + kItems + threadIdx.x, up, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // the stores have reached memory before the counter moves
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    __shared__ uint32_t arrived;
+    if (threadIdx.x == 0u) {
+      arrived = __hip_atomic_fetch_add(args.balance_counters + extra_index, 1u,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (arrived == splits - 1u)
+        __hip_atomic_store(args.balance_counters + extra_index, 0u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (arrived != splits - 1u) return;
+    // every partial is requested before the first is used: one round trip
+    float part[kMaxBalanceSplits][TILES];
+    if (threadIdx.x < kItems) {
+#pragma unroll
+      for (uint32_t s = 0; s < kMaxBalanceSplits; ++s) {
+        const float* theirs = slot + static_cast<size_t>(s) * TILES * kItems;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+          part[s][t] = s < splits
+                           ? __hip_atomic_load(theirs + t * kItems + threadIdx.x,
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                           : 0.0f;
+      }
+      total = 0.0f;
+      up = 0.0f;
+#pragma unroll
+      for (uint32_t s = 0; s < kMaxBalanceSplits; ++s) {
+        total += part[s][0];
+        if (TILES == 2) up += part[s][TILES - 1];
+      }
+    }
+  }
+  if (!item_valid) return;
   if (TILES == 2) {
-    // tile 1 is the up projection of the same rows
-    float up = 0.0f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w)
-      up += reduce[w][TILES - 1][item_half][item_reg][item_lane];
     const float activated = bf16_round(total / (1.0f + __expf(-total)));
     static_cast<uint16_t*>(args.output)[item_index] =
         static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
@@ -434,7 +515,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     store_output(args.segment_output[segment], args.segment_kind[segment],
                  static_cast<size_t>(item_batch) * args.segment_rows[segment] + local,
                  total);
-  } else if (splits > 1u) {
+  } else if (splits > 1u && !balanced) {
     static_cast<float*>(args.output)[static_cast<size_t>(split) * BATCH * args.rows +
                                      item_index] = total;
   } else {
@@ -577,12 +658,43 @@ int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
 // One tile per workgroup (a gate tile and its up tile for the fused SwiGLU
 // pair), or k_splits workgroups per tile; four waves split K, eight when the
 // launch has too few workgroups to give every CU one.
+uint32_t compute_units() {
+  static const uint32_t count = [] {
+    int device = 0, units = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount,
+                              device) != hipSuccess ||
+        units <= 0)
+      return 256u;
+    return static_cast<uint32_t>(units);
+  }();
+  return count;
+}
+
 int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
-                    bool swiglu, hipStream_t stream) {
+                    bool swiglu, hipStream_t stream, void* balance_workspace = nullptr) {
   const uint32_t splits = args.k_splits > 1u ? args.k_splits : 1u;
-  const uint32_t tiles =
+  uint32_t tiles =
       (args.rows + args.tile_rows - 1u) / args.tile_rows * splits;
   const uint32_t waves = tiles <= 256u && !swiglu ? 8u : 4u;
+  if (balance_workspace && splits == 1u) {
+    // the tiles past the last full round over the CUs, cut so that their
+    // pieces make one more, equal, round
+    const uint32_t units = compute_units();
+    const uint32_t extra = tiles > units ? tiles % units : 0u;
+    const uint32_t cut =
+        extra ? std::min({units / extra, kMaxBalanceSplits,
+                          args.padded_columns / kChunk})
+              : 0u;
+    if (cut >= 2u && extra <= kMaxBalanceTiles) {
+      args.balance_first_tile = tiles - extra;
+      args.balance_splits = cut;
+      args.balance_counters = static_cast<uint32_t*>(balance_workspace);
+      args.balance_partials = reinterpret_cast<float*>(
+          static_cast<uint8_t*>(balance_workspace) + kBalanceCounterBytes);
+      tiles = args.balance_first_tile + extra * cut;
+    }
+  }
 #define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
   return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
                                                     stream)
@@ -843,10 +955,65 @@ extern "C" int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,
                      false, as_stream(stream));
 }
 
+namespace {
+bool balance_workspace_ok(const void* workspace, size_t bytes) {
+  return workspace && bytes >= kBalanceWorkspaceBytes &&
+         reinterpret_cast<uintptr_t>(workspace) % 16u == 0u;
+}
+
+int32_t gemm_bf16_split(const qllm_fp4_matrix* matrix, const void* input,
+                        size_t input_bytes, const qllm_gemm_segment* segments,
+                        uint32_t segment_count, uint32_t batch,
+                        void* balance_workspace, void* stream);
+int32_t swiglu_bf16(const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up,
+                    const void* input, size_t input_bytes, void* output,
+                    uint32_t batch, void* balance_workspace, void* stream);
+}  // namespace
+
+extern "C" size_t qllm_fp4_gemm_balance_workspace_bytes(void) {
+  return kBalanceWorkspaceBytes;
+}
+
 extern "C" int32_t qllm_fp4_gemm_bf16_split(
     const qllm_fp4_matrix* matrix, const void* input, size_t input_bytes,
     const qllm_gemm_segment* segments, uint32_t segment_count, uint32_t batch,
     void* stream) {
+  return gemm_bf16_split(matrix, input, input_bytes, segments, segment_count,
+                         batch, nullptr, stream);
+}
+
+extern "C" int32_t qllm_fp4_gemm_bf16_split_balanced(
+    const qllm_fp4_matrix* matrix, const void* input, size_t input_bytes,
+    const qllm_gemm_segment* segments, uint32_t segment_count, uint32_t batch,
+    void* workspace, size_t workspace_bytes, void* stream) {
+  if (!balance_workspace_ok(workspace, workspace_bytes))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid balanced GEMM workspace");
+  return gemm_bf16_split(matrix, input, input_bytes, segments, segment_count,
+                         batch, workspace, stream);
+}
+
+extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
+                                        const qllm_fp4_matrix* up,
+                                        const void* input, size_t input_bytes,
+                                        void* output, uint32_t batch,
+                                        void* stream) {
+  return swiglu_bf16(gate, up, input, input_bytes, output, batch, nullptr, stream);
+}
+
+extern "C" int32_t qllm_fp4_swiglu_bf16_balanced(
+    const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up, const void* input,
+    size_t input_bytes, void* output, uint32_t batch, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  if (!balance_workspace_ok(workspace, workspace_bytes))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid balanced GEMM workspace");
+  return swiglu_bf16(gate, up, input, input_bytes, output, batch, workspace, stream);
+}
+
+namespace {
+int32_t gemm_bf16_split(const qllm_fp4_matrix* matrix, const void* input,
+                        size_t input_bytes, const qllm_gemm_segment* segments,
+                        uint32_t segment_count, uint32_t batch,
+                        void* balance_workspace, void* stream) {
   if (!matrix_ok(matrix) || !input || !segments || !segment_count ||
       segment_count > 3u || !batch || batch > 8u ||
       input_bytes < static_cast<size_t>(batch) * matrix->padded_columns * 2u)
@@ -904,14 +1071,12 @@ extern "C" int32_t qllm_fp4_gemm_bf16_split(
   args.tile_rows = matrix_tile_rows(matrix);
   return launch_mfma(args, static_cast<int>(matrix->scale_scheme),
                      matrix->layout == QLLM_LAYOUT_TILED, batch, false,
-                     as_stream(stream));
+                     as_stream(stream), balance_workspace);
 }
 
-extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
-                                        const qllm_fp4_matrix* up,
-                                        const void* input, size_t input_bytes,
-                                        void* output, uint32_t batch,
-                                        void* stream) {
+int32_t swiglu_bf16(const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up,
+                    const void* input, size_t input_bytes, void* output,
+                    uint32_t batch, void* balance_workspace, void* stream) {
   if (!matrix_ok(gate) || !matrix_ok(up) || gate->rows != up->rows ||
       gate->padded_columns != up->padded_columns ||
       gate->scale_scheme != up->scale_scheme || gate->layout != up->layout ||
@@ -931,8 +1096,9 @@ extern "C" int32_t qllm_fp4_swiglu_bf16(const qllm_fp4_matrix* gate,
   args.tile_rows = matrix_tile_rows(gate);
   return launch_mfma(args, static_cast<int>(gate->scale_scheme),
                      gate->layout == QLLM_LAYOUT_TILED, batch, true,
-                     as_stream(stream));
+                     as_stream(stream), balance_workspace);
 }
+}  // namespace
 
 extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
                                           const int8_t* input,

@@ -334,6 +334,13 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
     projection_partials_ = static_cast<float*>(
         device_alloc(projection_splits_ * rows * g_.hidden * 4U));
 
+  // counters and partial sums of the balanced q/k/v and gate/up launches
+  // (zeroed once; the kernels leave the counters at zero)
+  gemm_workspace_bytes_ = qllm_fp4_gemm_balance_workspace_bytes();
+  gemm_workspace_ = device_alloc(gemm_workspace_bytes_);
+  hip_check(hipMemset(gemm_workspace_, 0, gemm_workspace_bytes_),
+            "clear GEMM balance workspace");
+
   if (const char* text = std::getenv("QLLM_PROVIDER_QKV_SPLITS"))
     qkv_splits_ =
         static_cast<std::uint32_t>(std::clamp(std::atoi(text), 0, 16));
@@ -1566,9 +1573,9 @@ void Mi355DenseFp4Provider::enqueue_attention_block(std::uint32_t index,
         {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
         {key_, kv_rows, QLLM_OUT_F32},
         {value_, kv_rows, QLLM_OUT_F32}};
-    status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
-                                          hidden_bytes, projections, 3U, rows,
-                                          stream_));
+    status_check(qllm_fp4_gemm_bf16_split_balanced(
+        &layer.qkv.descriptor, normalized_, hidden_bytes, projections, 3U, rows,
+        gemm_workspace_, gemm_workspace_bytes_, stream_));
     enqueue_attention(index, rows, first_position, deferred_positions, query_,
                       key_, value_, attention_);
   }
@@ -1582,10 +1589,10 @@ void Mi355DenseFp4Provider::enqueue_ffn_block(std::uint32_t index,
                                               bool leave_partials) {
   const auto& layer = layers_[index];
   enqueue_normalise(layer.post_attention_norm, rows);
-  status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor, &layer.up.descriptor,
-                                    normalized_,
-                                    std::size_t{rows} * g_.hidden * 2U,
-                                    activation_, rows, stream_));
+  status_check(qllm_fp4_swiglu_bf16_balanced(
+      &layer.gate.descriptor, &layer.up.descriptor, normalized_,
+      std::size_t{rows} * g_.hidden * 2U, activation_, rows, gemm_workspace_,
+      gemm_workspace_bytes_, stream_));
   enqueue_residual_projection(layer.down.descriptor, activation_,
                               std::size_t{rows} * g_.intermediate * 2U, rows,
                               leave_partials);
@@ -2154,10 +2161,9 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
     const auto launch_one = [&](std::uint32_t index) {
       const auto& layer = layers_[index % g_.layers];
       if (which == "ffn_gate_up") {
-        status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
-                                          &layer.up.descriptor, normalized_,
-                                          hidden_bytes, activation_, rows,
-                                          stream_));
+        status_check(qllm_fp4_swiglu_bf16_balanced(
+            &layer.gate.descriptor, &layer.up.descriptor, normalized_, hidden_bytes,
+            activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream_));
       } else if (which == "ffn_down") {
         // as the target pass launches it
         const auto& down = layer.down.descriptor;
@@ -2184,8 +2190,9 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
               {query_, qkv.rows - 2U * kv_rows, QLLM_OUT_F32},
               {key_, kv_rows, QLLM_OUT_F32},
               {value_, kv_rows, QLLM_OUT_F32}};
-          status_check(qllm_fp4_gemm_bf16_split(&qkv, normalized_, hidden_bytes,
-                                                projections, 3U, rows, stream_));
+          status_check(qllm_fp4_gemm_bf16_split_balanced(
+              &qkv, normalized_, hidden_bytes, projections, 3U, rows,
+              gemm_workspace_, gemm_workspace_bytes_, stream_));
         }
       } else if (which == "attention_output") {
         const auto& output = layer.output.descriptor;
@@ -2290,10 +2297,10 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
       const auto filler = [&](std::uint32_t round) {
         for (std::uint32_t index = 0; index < fillers; ++index) {
           const auto& layer = layers_[(round * fillers + index) % g_.layers];
-          status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor,
-                                            &layer.up.descriptor, normalized_,
-                                            hidden_bytes, activation_, rows,
-                                            stream_));
+          status_check(qllm_fp4_swiglu_bf16_balanced(
+              &layer.gate.descriptor, &layer.up.descriptor, normalized_,
+              hidden_bytes, activation_, rows, gemm_workspace_,
+              gemm_workspace_bytes_, stream_));
         }
       };
       filler(0U);
@@ -2509,9 +2516,9 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
       {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
       {key_, kv_rows, QLLM_OUT_F32},
       {value_, kv_rows, QLLM_OUT_F32}};
-  status_check(qllm_fp4_gemm_bf16_split(&layer.qkv.descriptor, normalized_,
-                                        hidden_bytes, projections, 3U, rows,
-                                        stream));
+  status_check(qllm_fp4_gemm_bf16_split_balanced(
+      &layer.qkv.descriptor, normalized_, hidden_bytes, projections, 3U, rows,
+      gemm_workspace_, gemm_workspace_bytes_, stream));
   const auto pages = const_cast<const void* const*>(device_page_table_);
   if (deferred_positions) {
     status_check(qllm_qkv_rope_batch_deferred(
@@ -2560,9 +2567,9 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                    nullptr, normalized_, g_.hidden, rows,
                                    g_.hidden, g_.norm_epsilon,
                                    g_.zero_centered_norm, stream));
-  status_check(qllm_fp4_swiglu_bf16(&layer.gate.descriptor, &layer.up.descriptor,
-                                    normalized_, hidden_bytes, activation_, rows,
-                                    stream));
+  status_check(qllm_fp4_swiglu_bf16_balanced(
+      &layer.gate.descriptor, &layer.up.descriptor, normalized_, hidden_bytes,
+      activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream));
   // a single-row pass leaves its hidden state where the next pass reads it
   const bool retain_in_place = rows == 1U && produce_logits;
   status_check(qllm_fp4_gemm_bf16(

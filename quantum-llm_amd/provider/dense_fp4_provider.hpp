@@ -460,6 +460,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   // measured 11.4-14.5 us against 11.7 us uncut.
   float* qkv_partials_ = nullptr;          // [splits][rows][q + k + v rows]
   std::uint32_t qkv_splits_ = 0U;
+  void* gemm_workspace_{};
+  std::size_t gemm_workspace_bytes_{};
   void* select_workspace_{};
   std::size_t select_workspace_bytes_{};
   std::uint32_t* argmax_tokens_{};

@@ -99,6 +99,9 @@ SIGNATURES = {
     "qllm_fp4_swiglu_bf16_tall": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
     "qllm_fp4_gemm_bf16_tall_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_fp4_swiglu_bf16": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_balance_workspace_bytes": (c_size_t, []),
+    "qllm_fp4_gemm_bf16_split_balanced": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p, c_size_t, c_void_p]),
+    "qllm_fp4_swiglu_bf16_balanced": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
     "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32, c_uint32]),
     "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),

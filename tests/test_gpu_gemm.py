@@ -311,3 +311,104 @@ def test_k_split_rejects_what_it_does_not_take(device):
         with pytest.raises(qh.QllmError):
             qh.call("qllm_fp4_gemm_bf16_partial", matrix, qh.ptr(d_act), d_act.numel() * 2,
                     qh.ptr(partials), splits, rows_in_batch, None)
+
+
+# ---- balanced tail: the tiles past the last full round over the CUs cut along K ----
+
+def _balance_workspace(device):
+    size = qh.call("qllm_fp4_gemm_balance_workspace_bytes")
+    return torch.zeros(size, dtype=torch.uint8, device=device), size
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_F16_BLOCK16, ol.SCALE_UE8M0_BLOCK32])
+@pytest.mark.parametrize("rows,padded,batch", [(17408, 5120, 5), (10240, 1024, 5),
+                                               (8224, 512, 8), (9000, 128, 1)])
+def test_balanced_swiglu_matches_oracle_and_the_plain_launch(device, scheme, rows, padded,
+                                                             batch):
+    """Gate/up with a ragged last round: cut tiles against the oracle, uncut
+    tiles bit-equal to the plain launch, the same bits on every run and the
+    workspace's counters back at zero."""
+    rng = np.random.default_rng(rows + padded + scheme)
+    gate = synth.fp4_matrix(rng, rows, padded, scheme)
+    up = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(0.02 * rng.standard_normal((batch, padded)).astype(np.float32))
+    tensors = [gu.device_tensor(x, device) for x in (*gate, *up)]
+    gate_m, keep_g = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded,
+                                              padded, scheme), device)
+    up_m, keep_u = qh.prepack(qh.fp4_matrix(tensors[2], tensors[3], rows, padded,
+                                            padded, scheme), device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    workspace, size = _balance_workspace(device)
+    plain = torch.zeros((batch, rows), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_fp4_swiglu_bf16", gate_m, up_m, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(plain), batch, None)
+    runs = []
+    for _ in range(3):
+        out = torch.zeros((batch, rows), dtype=torch.bfloat16, device=device)
+        qh.call("qllm_fp4_swiglu_bf16_balanced", gate_m, up_m, qh.ptr(d_act),
+                d_act.numel() * 2, qh.ptr(out), batch, qh.ptr(workspace), size, None)
+        torch.cuda.synchronize()
+        runs.append(out.view(torch.uint16).cpu().numpy())
+        assert int(workspace[:4096].view(torch.int32).abs().sum()) == 0
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    tiles = (rows + 31) // 32
+    uncut = (tiles - tiles % units) * 32 if tiles > units else rows
+    assert np.array_equal(runs[0][:, :uncut], plain.view(torch.uint16).cpu().numpy()[:, :uncut])
+    # a sample of rows against the oracle (all of the cut ones)
+    pick = np.unique(np.concatenate([rng.choice(rows, 256, replace=False),
+                                     np.arange(min(uncut, rows - 1), rows)]))
+    g = ol.fp4_linear_f64(gate[0][pick], gate[1][pick], scheme, len(pick), padded, act)
+    u = ol.fp4_linear_f64(up[0][pick], up[1][pick], scheme, len(pick), padded, act)
+    got = ol.bf16_from_bits(runs[0])[:, pick]
+    gu.assert_close(got, ol.silu_product(g, u, True), rtol=1e-2, atol=1e-3, what="balanced swiglu")
+    del keep_g, keep_u
+
+
+@pytest.mark.parametrize("scheme", [ol.SCALE_F16_BLOCK16, ol.SCALE_UE8M0_BLOCK32])
+def test_balanced_split_projection_matches_oracle(device, scheme):
+    """q/k/v of the 27B shape ([8192 + 1024 + 1024, 5120], 320 tiles): the 64
+    tiles past the first round are cut in four."""
+    rng = np.random.default_rng(41 + scheme)
+    rows, padded, batch = 10240, 5120, 5
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    tensors = [gu.device_tensor(x, device) for x in (codes, scales)]
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                                            scheme), device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    workspace, size = _balance_workspace(device)
+    parts = [8192, 1024, 1024]
+    outs = [torch.zeros((batch, part), device=device) for part in parts]
+    segments = (qh.GemmSegment * 3)(*[qh.GemmSegment(qh.ptr(o), part, qh.OUT_F32)
+                                      for o, part in zip(outs, parts)])
+    for _ in range(2):
+        qh.call("qllm_fp4_gemm_bf16_split_balanced", matrix, qh.ptr(d_act),
+                d_act.numel() * 2, segments, 3, batch, qh.ptr(workspace), size, None)
+    torch.cuda.synchronize()
+    got = np.concatenate([o.cpu().numpy() for o in outs], axis=1)
+    pick = np.unique(np.concatenate([rng.choice(rows, 384, replace=False),
+                                     np.arange(8192, rows, 7)]))
+    want = ol.fp4_linear_f64(codes[pick], scales[pick], scheme, len(pick), padded, act)
+    gu.assert_close(got[:, pick], want, what="balanced q/k/v")
+    plain = gu.gemm(device, codes, scales, scheme, rows, padded, act)
+    assert np.array_equal(got[:, :8192], plain[:, :8192])
+    np.testing.assert_allclose(got, plain, rtol=1e-4, atol=1e-3)
+    assert int(workspace[:4096].view(torch.int32).abs().sum()) == 0
+    del keep
+
+
+def test_balanced_launch_rejects_a_bad_workspace(device):
+    rng = np.random.default_rng(2)
+    codes, scales = synth.fp4_matrix(rng, 64, 128, ol.SCALE_F16_BLOCK16)
+    tensors = [gu.device_tensor(x, device) for x in (codes, scales)]
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], 64, 128, 128,
+                                            ol.SCALE_F16_BLOCK16), device)
+    buffer = torch.zeros(4096, device=device)
+    with pytest.raises(qh.QllmError):
+        qh.call("qllm_fp4_swiglu_bf16_balanced", matrix, matrix, qh.ptr(buffer), 5 * 256,
+                qh.ptr(buffer), 5, qh.ptr(buffer), 1024, None)
+    with pytest.raises(qh.QllmError):
+        qh.call("qllm_fp4_swiglu_bf16_balanced", matrix, matrix, qh.ptr(buffer), 5 * 256,
+                qh.ptr(buffer), 5, 0, 1 << 22, None)
+    del keep
