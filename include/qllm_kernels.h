@@ -133,7 +133,8 @@ int32_t qllm_convert_f32_to_bf16_batch(const float* input, void* output,
 
 /* FP4 weights x Q8 activations, batch <= 8; out[m*rows+n].
  * replaces fp4_gemv_q8_batch_weight_reuse (transformer_kernels.hpp:92-97).
- * Block-32 UE8M0 row-major matrices only. */
+ * Block-32 UE8M0 matrices; the streaming layout runs on the matrix cores
+ * (qllm_fp4_gemm_q8), the row-major one on a wave per output row. */
 int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
                                const int8_t* input,
                                const float* input_scales, float* output,
@@ -167,6 +168,35 @@ int32_t qllm_fp4_gemm_bf16_split(const qllm_fp4_matrix* matrix,
                                  const qllm_gemm_segment* segments,
                                  uint32_t segment_count, uint32_t batch,
                                  void* stream);
+
+/* The reference's default activation contract on the matrix cores: int8 rows
+ * with one F32 scale each (qllm_quantize_q8_batch) against block-32 UE8M0
+ * weights in the streaming layout, out = 0.5 * s_m * sum over blocks of
+ * 2^(e - 127) * (integer block sum) - the statement of
+ * fp4_gemv_q8_batch5_tensor_core_kernel (transformer_kernels.cu:1162-1275),
+ * called from project_quantized (dense_fp4_provider.cpp:6229-6267).  Block sums
+ * are exact, blocks are accumulated in F32.  K % 64 == 0; input 16-byte
+ * aligned, [batch, padded_columns] int8.  `residual` as in qllm_fp4_gemm_bf16.
+ * The split form serves q/k/v stored as one matrix, the SwiGLU form stores
+ * silu(gate) * up as F32 (silu_product_kernel without bf16 rounding,
+ * transformer_kernels.cu:2774-2783): the reference quantises that product to
+ * Q8 again before the down projection.  `workspace` of the split and SwiGLU
+ * forms: NULL, or the balanced-tail workspace described further down. */
+int32_t qllm_fp4_gemm_q8(const qllm_fp4_matrix* matrix, const int8_t* input,
+                         const float* input_scales, void* output,
+                         uint32_t output_kind, const float* residual,
+                         uint32_t batch, void* stream);
+int32_t qllm_fp4_gemm_q8_split(const qllm_fp4_matrix* matrix, const int8_t* input,
+                               const float* input_scales,
+                               const qllm_gemm_segment* segments,
+                               uint32_t segment_count, uint32_t batch,
+                               void* workspace, size_t workspace_bytes,
+                               void* stream);
+int32_t qllm_fp4_swiglu_q8(const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up,
+                           const int8_t* input, const float* input_scales,
+                           float* output, uint32_t batch, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
 
 /* The same product with K cut over k_splits workgroups per tile (tiled layout
  * only, 1 <= k_splits <= 16): partials f32 [k_splits][batch][rows], split s
@@ -268,6 +298,18 @@ int32_t qllm_rms_norm_batch(const float* input, const float* weight,
                             uint32_t bf16_padded_columns, uint32_t rows,
                             uint32_t elements, float epsilon,
                             int32_t zero_centered, void* stream);
+
+/* RMSNorm of every row followed by its per-row Q8 quantisation, in one launch:
+ * normalize_rows then quantize_rows of the reference
+ * (dense_fp4_provider.cpp:5740-5778, 5983-5992; kernels
+ * transformer_kernels.cu:2469-2503, 912-946) with the same operations on the
+ * same F32 values, so codes and scales equal qllm_rms_norm_batch followed by
+ * qllm_quantize_q8_batch.  elements % 4 == 0, at most 16384; pointers 16-byte
+ * aligned; output_q8 [rows, elements], scales [rows]. */
+int32_t qllm_rms_norm_q8_batch(const float* input, const float* weight,
+                               int8_t* output_q8, float* scales, uint32_t rows,
+                               uint32_t elements, float epsilon,
+                               int32_t zero_centered, void* stream);
 
 /* The residual add of a projection computed as K-split partials
  * (qllm_fp4_gemm_bf16_partial) folded into the RMSNorm that follows:

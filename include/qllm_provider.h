@@ -57,6 +57,12 @@ typedef struct qllm_dense_geometry {
    * (qllm_provider_prefill); 0 = 32768.  The reference's prompt path runs
    * prefill_chunk_tokens rows per program step (moe_vm_runner.cpp:682-745). */
   uint32_t prefill_chunk_rows;
+  /* 1 = per-row Q8 activations into every projection, the reference's default
+   * contract (an artifact without dense_activation_input_bf16,
+   * prepare_dense_activation dense_fp4_provider.cpp:5983-6003); 0 = bf16
+   * activations.  Q8 needs scale_scheme 0 (block-32 UE8M0) and projection
+   * widths that are multiples of 64. */
+  uint32_t activation_q8;
 } qllm_dense_geometry;
 
 const char* qllm_provider_last_error(void);

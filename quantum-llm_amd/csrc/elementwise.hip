@@ -191,12 +191,56 @@ __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
 // partials[1] + ... (added in that order; partial p of the row lies
 // `partial_stride` floats after partial p - 1) and that sum is also written
 // back to `sum_out`.
+// four values -> four Q8 codes: clamp(rn(value / scale), -127, 127)
+// (transformer_kernels.cu:912-946), packed low byte first
+__device__ __forceinline__ uint32_t q8_pack4(float4 value, float scale) {
+  const auto code = [scale](float x) {
+    const int rounded = __float2int_rn(__fdiv_rn(x, scale));
+    return static_cast<uint32_t>(max(-127, min(127, rounded))) & 0xffu;
+  };
+  return code(value.x) | (code(value.y) << 8) | (code(value.z) << 16) |
+         (code(value.w) << 24);
+}
+
+// Per-row Q8 of rows of up to 5 * 4096 values: the row is fetched once and
+// stays in registers between the maximum and the codes.  columns % 4 == 0.
+__global__ __launch_bounds__(1024) void quantize_q8_wide_kernel(
+    const float* input, int8_t* output, float* scales, uint32_t columns,
+    uint32_t padded_columns) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  const float4* x = reinterpret_cast<const float4*>(input + row * columns);
+  const uint32_t vectors = columns / 4u;
+  float4 values[5];
+  float maximum = 0.0f;
+#pragma unroll
+  for (int slot = 0; slot < 5; ++slot) {
+    const uint32_t index = slot * 1024u + threadIdx.x;
+    values[slot] = index < vectors ? x[index] : make_float4(0.f, 0.f, 0.f, 0.f);
+    maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(values[slot].x), fabsf(values[slot].y)),
+                                   fmaxf(fabsf(values[slot].z), fabsf(values[slot].w))));
+  }
+  maximum = block_max(maximum, scratch);
+  const float scale = maximum > 0.0f ? maximum / 127.0f : 1.0f;
+  if (threadIdx.x == 0) scales[row] = scale;
+  uint32_t* target = reinterpret_cast<uint32_t*>(output + row * padded_columns);
+#pragma unroll
+  for (int slot = 0; slot < 5; ++slot) {
+    const uint32_t index = slot * 1024u + threadIdx.x;
+    if (index < vectors) target[index] = q8_pack4(values[slot], scale);
+  }
+  for (uint32_t index = vectors + threadIdx.x; index < padded_columns / 4u;
+       index += 1024u)
+    target[index] = 0u;
+}
+
 __device__ __forceinline__ void rms_norm_row_wide(
     const float* input_row, const float* weight, float* out_f32,
     uint16_t* out_bf16, uint32_t bf16_columns, uint32_t elements,
     float epsilon, bool zero_centered, float* scratch,
     const float* partial_row = nullptr, uint32_t partial_count = 0u,
-    size_t partial_stride = 0u, float* sum_out = nullptr) {
+    size_t partial_stride = 0u, float* sum_out = nullptr,
+    int8_t* out_q8 = nullptr, float* out_q8_scale = nullptr) {
   const float4* x = reinterpret_cast<const float4*>(input_row);
   const uint32_t vectors = elements / 4u;
   // the row and its weights are fetched together, before the reduction
@@ -269,6 +313,27 @@ __device__ __forceinline__ void rms_norm_row_wide(
       packed.y = f32_to_bf16_bits(result.z) | (f32_to_bf16_bits(result.w) << 16);
       reinterpret_cast<uint2*>(out_bf16)[index] = packed;
     }
+    values[slot] = result;
+  }
+  if (out_q8) {
+    // the row quantised as quantize_q8_batch_kernel quantises the F32 norm
+    // output (same operations on the same values)
+    float maximum = 0.0f;
+#pragma unroll
+    for (int slot = 0; slot < 4; ++slot) {
+      if (slot * blockDim.x + threadIdx.x >= vectors) continue;
+      maximum = fmaxf(maximum, fmaxf(fmaxf(fabsf(values[slot].x), fabsf(values[slot].y)),
+                                     fmaxf(fabsf(values[slot].z), fabsf(values[slot].w))));
+    }
+    maximum = block_max(maximum, scratch);
+    const float scale = maximum > 0.0f ? maximum / 127.0f : 1.0f;
+    if (threadIdx.x == 0) *out_q8_scale = scale;
+#pragma unroll
+    for (int slot = 0; slot < 4; ++slot) {
+      const uint32_t index = slot * blockDim.x + threadIdx.x;
+      if (index >= vectors) continue;
+      reinterpret_cast<uint32_t*>(out_q8)[index] = q8_pack4(values[slot], scale);
+    }
   }
   if (out_bf16)
     for (uint32_t index = elements + threadIdx.x; index < bf16_columns;
@@ -287,6 +352,18 @@ __global__ __launch_bounds__(1024) void rms_norm_batch_wide_kernel(
       output_f32 ? output_f32 + row * elements : nullptr,
       output_bf16 ? output_bf16 + row * bf16_padded_columns : nullptr,
       bf16_padded_columns, elements, epsilon, zero_centered, scratch);
+}
+
+// RMSNorm of a row straight into its per-row Q8 form (normalize_rows followed
+// by quantize_rows, dense_fp4_provider.cpp:5740-5778, 5983-5992, in one launch).
+__global__ __launch_bounds__(1024) void rms_norm_q8_kernel(
+    const float* input, const float* weight, int8_t* output_q8, float* scales,
+    uint32_t elements, float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  rms_norm_row_wide(input + row * elements, weight, nullptr, nullptr, 0u, elements,
+                    epsilon, zero_centered, scratch, nullptr, 0u, 0u, nullptr,
+                    output_q8 + row * elements, scales + row);
 }
 
 // hidden[r] += partials[0][r] + ... + partials[count-1][r], then its RMSNorm in
@@ -404,9 +481,35 @@ extern "C" int32_t qllm_quantize_q8_batch(const float* input, int8_t* output,
   if (!input || !output || !scales || !rows || !columns ||
       padded_columns < columns)
     return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 batch quantization");
-  quantize_q8_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
-      input, output, scales, columns, padded_columns, bf16_input != 0);
+  const bool wide =
+      !bf16_input && columns % 4u == 0u && padded_columns % 4u == 0u &&
+      columns <= 5u * 4096u &&
+      ((reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output)) &
+       15u) == 0u;
+  if (wide)
+    quantize_q8_wide_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+        input, output, scales, columns, padded_columns);
+  else
+    quantize_q8_batch_kernel<<<rows, 256, 0, as_stream(stream)>>>(
+        input, output, scales, columns, padded_columns, bf16_input != 0);
   return launched("quantize Q8 batch");
+}
+
+extern "C" int32_t qllm_rms_norm_q8_batch(const float* input, const float* weight,
+                                          int8_t* output_q8, float* scales,
+                                          uint32_t rows, uint32_t elements,
+                                          float epsilon, int32_t zero_centered,
+                                          void* stream) {
+  const auto aligned = [](const void* pointer) {
+    return reinterpret_cast<uintptr_t>(pointer) % 16u == 0u;
+  };
+  if (!input || !output_q8 || !scales || !rows || rows > 65535u || !elements ||
+      elements % 4u != 0u || elements > 16384u || !(epsilon > 0.0f) ||
+      !aligned(input) || !aligned(output_q8) || (weight && !aligned(weight)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 RMSNorm");
+  rms_norm_q8_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+      input, weight, output_q8, scales, elements, epsilon, zero_centered != 0);
+  return launched("Q8 RMSNorm");
 }
 
 extern "C" int32_t qllm_convert_f32_to_bf16_batch(

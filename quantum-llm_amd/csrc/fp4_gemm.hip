@@ -35,6 +35,20 @@ constexpr int kSchemeF16 = QLLM_SCALE_F16_BLOCK16;
 
 constexpr uint32_t kChunk = 64;            // K elements per wave step
 
+// eight int8 codes -> the same integers as bf16 (exact: seven bits)
+__device__ __forceinline__ bf16x8 q8x8_to_bf16(uint2 bytes) {
+  const uint32_t word[2] = {bytes.x, bytes.y};
+  bf16x8 result;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int32_t code =
+        static_cast<int32_t>(word[k >> 2] << (24 - 8 * (k & 3))) >> 24;
+    const uint32_t bits = __builtin_bit_cast(uint32_t, static_cast<float>(code));
+    result[k] = __builtin_bit_cast(__bf16, static_cast<uint16_t>(bits >> 16));
+  }
+  return result;
+}
+
 __device__ __forceinline__ bf16x8 expand_fp4x8(uint32_t packed, float scale) {
   const bf16x2 p0 = fp4x2_to_bf16<0>(packed, scale);
   const bf16x2 p1 = fp4x2_to_bf16<1>(packed, scale);
@@ -70,7 +84,9 @@ struct GemmTile {
 
 struct GemmArgs {
   GemmTile tile[2];
-  const uint16_t* activations;  // bf16 [batch, padded_columns]
+  const uint16_t* activations;  // bf16 [batch, padded_columns]; Q8: int8
+  // Q8 kernels: the scale of every activation row, applied to its sums
+  const float* activation_scales;
   void* output;
   const float* residual;
   uint32_t rows;
@@ -123,11 +139,16 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // the layout of the workspace that serves it - one counter per cut tile, then
 // the partials.
 constexpr uint32_t kMaxBalanceSplits = 8;
-constexpr uint32_t kMaxBalanceTiles = 128;
+constexpr uint32_t kMaxBalanceTiles = 1024;   // one counter each
 constexpr size_t kBalanceCounterBytes = 4096;
-constexpr size_t kBalanceWorkspaceBytes =
-    kBalanceCounterBytes +
-    size_t{kMaxBalanceTiles} * kMaxBalanceSplits * 2u * 256u * sizeof(float);
+constexpr size_t kBalanceWorkspaceBytes = size_t{4} << 20;
+// floats of one small workgroup's hand-over: a slot per tile of the pair
+constexpr size_t balance_slot_floats(bool pair) { return (pair ? 2u : 1u) * 256u; }
+
+bool balance_workspace_ok(const void* workspace, size_t bytes) {
+  return workspace && bytes >= kBalanceWorkspaceBytes &&
+         reinterpret_cast<uintptr_t>(workspace) % 16u == 0u;
+}
 
 // 4x4 transpose of dwords across the four 16-lane rows of a wave: on return
 // register d of row c holds what register c of row d held.
@@ -175,11 +196,22 @@ __device__ __forceinline__ void transpose_rows4(uint32_t (&v)[4]) {
 // Batches of up to 6 rows sit in MFMA rows {0,1,2,4,5,6} of each half: those
 // are accumulator registers 0..2 of both row groups, one FMA fewer than rows
 // 0..5 would cost.
-template <int SCHEME, int BATCH, int TILES, int WAVES, bool TILED>
+//
+// Q8: the activations are the reference's per-row Q8 (int8 codes and one F32
+// scale per row, quantize_q8_batch_kernel, transformer_kernels.cu:912-946) and
+// the result is its integer statement (fp4_gemv_q8_batch5_tensor_core_kernel,
+// :1162-1275): out = 0.5 * s_m * sum over 32-blocks of 2^(e - 127) * (integer
+// block sum).  The codes enter the same matrix instruction as exact bf16
+// integers (|q| <= 127), the weights as exact bf16 (E2M1 value times a power of
+// two): every product and every block sum is exact in F32, the blocks are
+// accumulated in F32 as the reference accumulates them, the row scale is
+// applied in the epilogue.  A chunk's codes are 4 * batch sixteen-byte pieces
+// (16 columns each); a lane's fragment is eight consecutive bytes of a piece.
+template <int SCHEME, int BATCH, int TILES, int WAVES, bool TILED, bool Q8 = false>
 __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     const GemmArgs args) {
   constexpr int PF = 4;                // chunks in flight per lane
-  constexpr int PIECES = 8 * BATCH;    // activation pieces per chunk
+  constexpr int PIECES = (Q8 ? 4 : 8) * BATCH;   // activation pieces per chunk
   constexpr bool COMPACT = BATCH <= 6;
   constexpr int REGS = COMPACT ? 3 : 4;  // accumulator registers in use
   constexpr int kZeroPiece = 64;
@@ -250,7 +282,9 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   //   ->  act[m][chunk*64 + octet*8 .. +8]
   const uint32_t piece = lane < PIECES ? lane : PIECES - 1u;
   const uint32_t activation_lane =
-      ((piece % BATCH) * K + (piece / BATCH) * 8u) * 2u;
+      Q8 ? (piece % BATCH) * K + (piece / BATCH) * 16u
+         : ((piece % BATCH) * K + (piece / BATCH) * 8u) * 2u;
+  constexpr uint32_t kActivationChunkBytes = Q8 ? kChunk : kChunk * 2u;
   const uint8_t* activation_base =
       reinterpret_cast<const uint8_t*>(args.activations);
   // A fragment of span s: MFMA row n carries batch row m of block n/8; lane
@@ -262,8 +296,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     const uint32_t m = COMPACT ? (r >> 2) * 3u + (r & 3u) : r;
     const bool live =
         m < BATCH && (!COMPACT || (r & 3u) < 3u) && (g >> 1) == (n >> 3);
-    fragment_piece[0] = live ? g * BATCH + m : kZeroPiece;
-    fragment_piece[1] = live ? (4u + g) * BATCH + m : kZeroPiece;
+    if (Q8) {
+      // byte offsets into the ring slot: columns 32s + 8g .. + 8 of row m
+      fragment_piece[0] = live ? ((g >> 1) * BATCH + m) * 16u + (g & 1u) * 8u
+                               : kZeroPiece * 16u;
+      fragment_piece[1] = live ? ((2u + (g >> 1)) * BATCH + m) * 16u + (g & 1u) * 8u
+                               : kZeroPiece * 16u;
+    } else {
+      fragment_piece[0] = live ? g * BATCH + m : kZeroPiece;
+      fragment_piece[1] = live ? (4u + g) * BATCH + m : kZeroPiece;
+    }
   }
   if (lane < 2u) ring[wave][lane][kZeroPiece] = make_uint4(0u, 0u, 0u, 0u);
 
@@ -337,7 +379,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       }
     }
     activation[slot] = *reinterpret_cast<const uint4*>(
-        activation_base + chunk * (kChunk * 2u) + activation_lane);
+        activation_base + chunk * kActivationChunkBytes + activation_lane);
   };
 
   if (my_chunks) {
@@ -367,8 +409,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
         __builtin_amdgcn_wave_barrier();
         bf16x8 a[2];
 #pragma unroll
-        for (int span = 0; span < 2; ++span)
-          a[span] = __builtin_bit_cast(bf16x8, stage[fragment_piece[span]]);
+        for (int span = 0; span < 2; ++span) {
+          if constexpr (Q8) {
+            const uint2 bytes = *reinterpret_cast<const uint2*>(
+                reinterpret_cast<const uint8_t*>(stage) + fragment_piece[span]);
+            a[span] = q8x8_to_bf16(bytes);
+          } else {
+            a[span] = __builtin_bit_cast(bf16x8, stage[fragment_piece[span]]);
+          }
+        }
         __builtin_amdgcn_wave_barrier();
 
 #pragma unroll
@@ -456,13 +505,13 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   if (balanced) {
     // hand the sums over; the last of the tile's workgroups finishes it
     float* const slot = args.balance_partials +
-                        static_cast<size_t>(extra_index) * splits * TILES * kItems;
+                        static_cast<size_t>(extra_index) * splits * TILES * 256u;
     if (threadIdx.x < kItems) {
-      float* const mine = slot + static_cast<size_t>(split) * TILES * kItems;
+      float* const mine = slot + static_cast<size_t>(split) * TILES * 256u;
       __hip_atomic_store(mine + threadIdx.x, total, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
       if (TILES == 2)
-        __hip_atomic_store(mine + kItems + threadIdx.x, up, __ATOMIC_RELAXED,
+        __hip_atomic_store(mine + 256u + threadIdx.x, up, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
     }
     // the stores have reached memory before the counter moves
@@ -483,11 +532,11 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     if (threadIdx.x < kItems) {
 #pragma unroll
       for (uint32_t s = 0; s < kMaxBalanceSplits; ++s) {
-        const float* theirs = slot + static_cast<size_t>(s) * TILES * kItems;
+        const float* theirs = slot + static_cast<size_t>(s) * TILES * 256u;
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
           part[s][t] = s < splits
-                           ? __hip_atomic_load(theirs + t * kItems + threadIdx.x,
+                           ? __hip_atomic_load(theirs + t * 256u + threadIdx.x,
                                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                            : 0.0f;
       }
@@ -501,7 +550,19 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
     }
   }
   if (!item_valid) return;
+  if constexpr (Q8) {
+    const float row_scale = args.activation_scales[item_batch];
+    total *= row_scale;
+    up *= row_scale;
+  }
   if (TILES == 2) {
+    if (args.output_kind == QLLM_OUT_F32) {
+      // F32 activations (silu_product_kernel without bf16 rounding,
+      // transformer_kernels.cu:2774-2783)
+      static_cast<float*>(args.output)[item_index] =
+          total / (1.0f + __expf(-total)) * up;
+      return;
+    }
     const float activated = bf16_round(total / (1.0f + __expf(-total)));
     static_cast<uint16_t*>(args.output)[item_index] =
         static_cast<uint16_t>(f32_to_bf16_bits(activated * up));
@@ -628,30 +689,30 @@ bool matrix_ok(const qllm_fp4_matrix* m) {
            tile_rows_ok(m->tile_rows)));
 }
 
-template <int SCHEME, int BATCH, int TILES, bool TILED>
+template <int SCHEME, int BATCH, int TILES, bool TILED, bool Q8>
 int32_t launch_mfma_waves(const GemmArgs& args, uint32_t grid, uint32_t waves,
                           hipStream_t stream) {
   if (waves == 4u)
-    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4, TILED>
+    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 4, TILED, Q8>
         <<<grid, 256, 0, stream>>>(args);
   else
-    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8, TILED>
+    fp4_gemm_mfma_kernel<SCHEME, BATCH, TILES, 8, TILED, Q8>
         <<<grid, 512, 0, stream>>>(args);
-  return launched("FP4 MFMA GEMM");
+  return launched(Q8 ? "FP4 x Q8 MFMA GEMM" : "FP4 MFMA GEMM");
 }
 
-template <int SCHEME, int TILES, bool TILED>
+template <int SCHEME, int TILES, bool TILED, bool Q8 = false>
 int32_t launch_mfma_batch(const GemmArgs& args, uint32_t batch, uint32_t grid,
                           uint32_t waves, hipStream_t stream) {
   switch (batch) {
-    case 1: return launch_mfma_waves<SCHEME, 1, TILES, TILED>(args, grid, waves, stream);
-    case 2: return launch_mfma_waves<SCHEME, 2, TILES, TILED>(args, grid, waves, stream);
-    case 3: return launch_mfma_waves<SCHEME, 3, TILES, TILED>(args, grid, waves, stream);
-    case 4: return launch_mfma_waves<SCHEME, 4, TILES, TILED>(args, grid, waves, stream);
-    case 5: return launch_mfma_waves<SCHEME, 5, TILES, TILED>(args, grid, waves, stream);
-    case 6: return launch_mfma_waves<SCHEME, 6, TILES, TILED>(args, grid, waves, stream);
-    case 7: return launch_mfma_waves<SCHEME, 7, TILES, TILED>(args, grid, waves, stream);
-    default: return launch_mfma_waves<SCHEME, 8, TILES, TILED>(args, grid, waves, stream);
+    case 1: return launch_mfma_waves<SCHEME, 1, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 2: return launch_mfma_waves<SCHEME, 2, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 3: return launch_mfma_waves<SCHEME, 3, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 4: return launch_mfma_waves<SCHEME, 4, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 5: return launch_mfma_waves<SCHEME, 5, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 6: return launch_mfma_waves<SCHEME, 6, TILES, TILED, Q8>(args, grid, waves, stream);
+    case 7: return launch_mfma_waves<SCHEME, 7, TILES, TILED, Q8>(args, grid, waves, stream);
+    default: return launch_mfma_waves<SCHEME, 8, TILES, TILED, Q8>(args, grid, waves, stream);
   }
 }
 
@@ -676,7 +737,8 @@ int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
   const uint32_t splits = args.k_splits > 1u ? args.k_splits : 1u;
   uint32_t tiles =
       (args.rows + args.tile_rows - 1u) / args.tile_rows * splits;
-  const uint32_t waves = tiles <= 256u && !swiglu ? 8u : 4u;
+  const size_t partial_capacity =
+      (kBalanceWorkspaceBytes - kBalanceCounterBytes) / sizeof(float);
   if (balance_workspace && splits == 1u) {
     // the tiles past the last full round over the CUs, cut so that their
     // pieces make one more, equal, round
@@ -686,7 +748,8 @@ int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
         extra ? std::min({units / extra, kMaxBalanceSplits,
                           args.padded_columns / kChunk})
               : 0u;
-    if (cut >= 2u && extra <= kMaxBalanceTiles) {
+    if (cut >= 2u && extra <= kMaxBalanceTiles &&
+        size_t{extra} * cut * balance_slot_floats(swiglu) <= partial_capacity) {
       args.balance_first_tile = tiles - extra;
       args.balance_splits = cut;
       args.balance_counters = static_cast<uint32_t*>(balance_workspace);
@@ -695,9 +758,23 @@ int32_t launch_mfma(GemmArgs args, int scheme, bool tiled, uint32_t batch,
       tiles = args.balance_first_tile + extra * cut;
     }
   }
+  // four waves split K, eight when the launch has too few workgroups to give
+  // every CU one
+  const uint32_t waves = tiles <= 256u && !swiglu ? 8u : 4u;
 #define QLLM_LAUNCH(SCHEME_, TILES_, TILED_)                                  \
   return launch_mfma_batch<SCHEME_, TILES_, TILED_>(args, batch, tiles, waves, \
                                                     stream)
+  if (args.activation_scales) {
+    // Q8 activations: block-32 UE8M0 matrices in the streaming layout
+    if (scheme != kSchemeUe8m0 || !tiled)
+      return fail(QLLM_INVALID_ARGUMENT,
+                  "the Q8 matrix-core GEMM takes tiled block-32 UE8M0 matrices");
+    if (swiglu)
+      return launch_mfma_batch<kSchemeUe8m0, 2, true, true>(args, batch, tiles,
+                                                           waves, stream);
+    return launch_mfma_batch<kSchemeUe8m0, 1, true, true>(args, batch, tiles, waves,
+                                                         stream);
+  }
   if (scheme == kSchemeF16) {
     if (tiled) {
       if (swiglu) QLLM_LAUNCH(kSchemeF16, 2, true);
@@ -956,10 +1033,6 @@ extern "C" int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,
 }
 
 namespace {
-bool balance_workspace_ok(const void* workspace, size_t bytes) {
-  return workspace && bytes >= kBalanceWorkspaceBytes &&
-         reinterpret_cast<uintptr_t>(workspace) % 16u == 0u;
-}
 
 int32_t gemm_bf16_split(const qllm_fp4_matrix* matrix, const void* input,
                         size_t input_bytes, const qllm_gemm_segment* segments,
@@ -1100,11 +1173,108 @@ int32_t swiglu_bf16(const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up,
 }
 }  // namespace
 
+namespace {
+// the checks every Q8 matrix-core launch shares
+bool q8_gemm_ok(const qllm_fp4_matrix* matrix, const int8_t* input,
+                const float* input_scales, uint32_t batch) {
+  return matrix_ok(matrix) && matrix->scale_scheme == QLLM_SCALE_UE8M0_BLOCK32 &&
+         matrix->layout == QLLM_LAYOUT_TILED && input && input_scales && batch &&
+         batch <= 8u && reinterpret_cast<uintptr_t>(input) % 16u == 0u;
+}
+
+GemmArgs q8_gemm_args(const qllm_fp4_matrix* matrix, const int8_t* input,
+                      const float* input_scales) {
+  GemmArgs args{};
+  args.tile[0] = {matrix->weights, static_cast<const uint8_t*>(matrix->scales)};
+  args.tile[1] = args.tile[0];
+  args.activations = reinterpret_cast<const uint16_t*>(input);
+  args.activation_scales = input_scales;
+  args.rows = matrix->rows;
+  args.padded_columns = matrix->padded_columns;
+  args.tile_rows = matrix_tile_rows(matrix);
+  return args;
+}
+}  // namespace
+
+extern "C" int32_t qllm_fp4_gemm_q8(const qllm_fp4_matrix* matrix,
+                                    const int8_t* input, const float* input_scales,
+                                    void* output, uint32_t output_kind,
+                                    const float* residual, uint32_t batch,
+                                    void* stream) {
+  if (!q8_gemm_ok(matrix, input, input_scales, batch) || !output ||
+      output_kind > QLLM_OUT_BF16 ||
+      (residual && output_kind == QLLM_OUT_BF16 &&
+       static_cast<const void*>(residual) == output))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 x Q8 GEMM");
+  GemmArgs args = q8_gemm_args(matrix, input, input_scales);
+  args.output = output;
+  args.output_kind = output_kind;
+  args.residual = residual;
+  return launch_mfma(args, kSchemeUe8m0, true, batch, false, as_stream(stream));
+}
+
+extern "C" int32_t qllm_fp4_gemm_q8_split(const qllm_fp4_matrix* matrix,
+                                          const int8_t* input,
+                                          const float* input_scales,
+                                          const qllm_gemm_segment* segments,
+                                          uint32_t segment_count, uint32_t batch,
+                                          void* workspace, size_t workspace_bytes,
+                                          void* stream) {
+  if (!q8_gemm_ok(matrix, input, input_scales, batch) || !segments ||
+      !segment_count || segment_count > 3u ||
+      (workspace && !balance_workspace_ok(workspace, workspace_bytes)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid split FP4 x Q8 GEMM");
+  GemmArgs args = q8_gemm_args(matrix, input, input_scales);
+  uint64_t total_rows = 0;
+  for (uint32_t s = 0; s < segment_count; ++s) {
+    if (!segments[s].output || !segments[s].rows ||
+        segments[s].output_kind > QLLM_OUT_BF16)
+      return fail(QLLM_INVALID_ARGUMENT, "invalid split FP4 x Q8 GEMM segment");
+    args.segment_rows[s] = segments[s].rows;
+    args.segment_kind[s] = segments[s].output_kind;
+    args.segment_output[s] = segments[s].output;
+    total_rows += segments[s].rows;
+  }
+  if (total_rows != matrix->rows)
+    return fail(QLLM_INVALID_ARGUMENT,
+                "split FP4 x Q8 GEMM: segment rows do not add up to the matrix");
+  args.segments = segment_count;
+  args.output = segments[0].output;
+  args.output_kind = segments[0].output_kind;
+  return launch_mfma(args, kSchemeUe8m0, true, batch, false, as_stream(stream),
+                     workspace);
+}
+
+extern "C" int32_t qllm_fp4_swiglu_q8(const qllm_fp4_matrix* gate,
+                                      const qllm_fp4_matrix* up,
+                                      const int8_t* input,
+                                      const float* input_scales, float* output,
+                                      uint32_t batch, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+  if ((workspace && !balance_workspace_ok(workspace, workspace_bytes)) ||
+      !q8_gemm_ok(gate, input, input_scales, batch) || !matrix_ok(up) ||
+      gate->rows != up->rows || gate->padded_columns != up->padded_columns ||
+      up->scale_scheme != gate->scale_scheme || up->layout != gate->layout ||
+      matrix_tile_rows(gate) != matrix_tile_rows(up) || !output)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid fused FP4 x Q8 SwiGLU GEMM");
+  GemmArgs args = q8_gemm_args(gate, input, input_scales);
+  args.tile[1] = {up->weights, static_cast<const uint8_t*>(up->scales)};
+  args.output = output;
+  args.output_kind = QLLM_OUT_F32;
+  return launch_mfma(args, kSchemeUe8m0, true, batch, true, as_stream(stream),
+                     workspace);
+}
+
 extern "C" int32_t qllm_fp4_gemv_q8_batch(const qllm_fp4_matrix* matrix,
                                           const int8_t* input,
                                           const float* input_scales,
                                           float* output, uint32_t batch,
                                           int32_t bf16_output, void* stream) {
+  // the streaming layout goes to the matrix cores
+  if (matrix_ok(matrix) && matrix->layout == QLLM_LAYOUT_TILED)
+    return qllm_fp4_gemm_q8(matrix, input, input_scales, output,
+                            bf16_output ? QLLM_OUT_F32_BF16_ROUNDED : QLLM_OUT_F32,
+                            nullptr, batch, stream);
   if (!matrix_ok(matrix) || matrix->scale_scheme != QLLM_SCALE_UE8M0_BLOCK32 ||
       matrix->layout != QLLM_LAYOUT_ROW_MAJOR || !input || !input_scales ||
       !output || !batch || batch > 8u)

@@ -169,6 +169,12 @@ er::Status dense_geometry_from_artifact(const er::ModelDescriptor& model,
     if (!attention_seen || !ffn_seen)
       return invalid("program has no dense attention or FFN operation");
 
+    // The activation contract (compiler/expert_pack/compile.py:256-279): an
+    // artifact takes bf16 activation input only when it says so; the default
+    // is per-row Q8, which exists for block-32 UE8M0 weights.
+    g.activation_q8 = attribute(model, "dense_activation_input_bf16") != 1U &&
+                      g.scale_scheme == QLLM_SCALE_UE8M0_BLOCK32;
+
     g.mtp_layers = 0U;
     g.draft_depth = 4U;
     if (model.exact_decode_program) {

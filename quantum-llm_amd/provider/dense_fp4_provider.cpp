@@ -334,6 +334,24 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
     projection_partials_ = static_cast<float*>(
         device_alloc(projection_splits_ * rows * g_.hidden * 4U));
 
+  if (g_.activation_q8) {
+    if (g_.scale_scheme != QLLM_SCALE_UE8M0_BLOCK32 || g_.hidden % 64U != 0U ||
+        g_.intermediate % 64U != 0U ||
+        (std::size_t{g_.query_heads} * g_.head_dim) % 64U != 0U)
+      throw std::invalid_argument(
+          "Q8 activations need block-32 UE8M0 weights and projection widths "
+          "that are multiples of 64");
+    const std::size_t columns = std::max(widest, std::size_t{2U} * g_.hidden);
+    q8_ = static_cast<std::int8_t*>(device_alloc(rows * columns));
+    q8_scales_ = static_cast<float*>(device_alloc(rows * 4U));
+    activation_f32_ = static_cast<float*>(device_alloc(rows * columns * 4U));
+    if (g_.mtp_layers)
+      mtp_fusion_f32_ =
+          static_cast<float*>(device_alloc(rows * 2U * g_.hidden * 4U));
+    // every projection adds its residual itself: the norm reads one array
+    projection_splits_ = 0U;
+    qkv_splits_ = 0U;
+  }
   // counters and partial sums of the balanced q/k/v and gate/up launches
   // (zeroed once; the kernels leave the counters at zero)
   gemm_workspace_bytes_ = qllm_fp4_gemm_balance_workspace_bytes();
@@ -344,7 +362,8 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
   if (const char* text = std::getenv("QLLM_PROVIDER_QKV_SPLITS"))
     qkv_splits_ =
         static_cast<std::uint32_t>(std::clamp(std::atoi(text), 0, 16));
-  if (g_.kv_encoding != KvEncoding::q4_f16_per_head) qkv_splits_ = 0U;
+  if (g_.kv_encoding != KvEncoding::q4_f16_per_head || g_.activation_q8)
+    qkv_splits_ = 0U;
   if (qkv_splits_ > 1U)
     qkv_partials_ = static_cast<float*>(device_alloc(
         qkv_splits_ * rows * (query_width + 2U * kv_width) * 4U));
@@ -1427,7 +1446,7 @@ void Mi355DenseFp4Provider::enqueue_attention(
     launch.maximum_splits = maximum_splits_;
     launch.query_stride = query_stride;
     launch.output_gated = g_.output_gated;
-    launch.output_kind = QLLM_OUT_BF16;
+    launch.output_kind = g_.activation_q8 ? QLLM_OUT_F32 : QLLM_OUT_BF16;
     launch.stream = stream;
     launch.device_positions = deferred_positions ? positions_ : nullptr;
     if (fused) {
@@ -1472,7 +1491,7 @@ void Mi355DenseFp4Provider::enqueue_attention(
     launch.maximum_splits = maximum_splits_;
     launch.query_stride = query_stride;
     launch.output_gated = g_.output_gated;
-    launch.output_kind = QLLM_OUT_BF16;
+    launch.output_kind = g_.activation_q8 ? QLLM_OUT_F32 : QLLM_OUT_BF16;
     launch.stream = stream;
     status_check(qllm_attention_paged_f16(&launch));
   }
@@ -1515,8 +1534,39 @@ void Mi355DenseFp4Provider::enqueue_rope_table(std::uint32_t rows,
 
 // RMSNorm of hidden_ into normalized_ (bf16), first adding the partials a
 // K-split residual projection left behind.
+// Per-row Q8 of `rows` F32 rows (quantize_rows, dense_fp4_provider.cpp:5983-
+// 5992) into q8_ / q8_scales_, what the next projection reads.
+void Mi355DenseFp4Provider::enqueue_quantise(const float* input,
+                                             std::uint32_t rows,
+                                             std::uint32_t columns) {
+  status_check(qllm_quantize_q8_batch(input, q8_, q8_scales_, rows, columns,
+                                      columns, 0, stream_));
+}
+
+// RMSNorm of `rows` rows of `input` into q8_ / q8_scales_: one launch where the
+// fused kernel takes the row length, otherwise the norm and the quantisation.
+void Mi355DenseFp4Provider::enqueue_normalise_q8(const float* input,
+                                                 const float* weight,
+                                                 std::uint32_t rows) {
+  if (g_.hidden % 4U == 0U && g_.hidden <= 16384U) {
+    status_check(qllm_rms_norm_q8_batch(input, weight, q8_, q8_scales_, rows,
+                                        g_.hidden, g_.norm_epsilon,
+                                        g_.zero_centered_norm, stream_));
+    return;
+  }
+  status_check(qllm_rms_norm_batch(input, weight, activation_f32_, nullptr, 0U, rows,
+                                   g_.hidden, g_.norm_epsilon,
+                                   g_.zero_centered_norm, stream_));
+  enqueue_quantise(activation_f32_, rows, g_.hidden);
+}
+
 void Mi355DenseFp4Provider::enqueue_normalise(const float* weight,
                                               std::uint32_t rows) {
+  if (g_.activation_q8) {
+    // normalize_rows then quantize_rows (:5740-5778, :5983-5992)
+    enqueue_normalise_q8(hidden_, weight, rows);
+    return;
+  }
   if (pending_partials_)
     status_check(qllm_rms_norm_residual_batch(
         hidden_, projection_partials_, pending_partials_, weight, normalized_,
@@ -1533,6 +1583,12 @@ void Mi355DenseFp4Provider::enqueue_normalise(const float* weight,
 void Mi355DenseFp4Provider::enqueue_residual_projection(
     const qllm_fp4_matrix& matrix, const std::uint16_t* input,
     std::size_t input_bytes, std::uint32_t rows, bool leave_partials) {
+  if (g_.activation_q8) {
+    // the projection's input was quantised into q8_ by the caller
+    status_check(qllm_fp4_gemm_q8(&matrix, q8_, q8_scales_, hidden_, QLLM_OUT_F32,
+                                  hidden_, rows, stream_));
+    return;
+  }
   if (leave_partials && projection_splits_ > 1U &&
       matrix.layout == QLLM_LAYOUT_TILED &&
       matrix.padded_columns / 64U >= projection_splits_) {
@@ -1559,6 +1615,22 @@ void Mi355DenseFp4Provider::enqueue_attention_block(std::uint32_t index,
   enqueue_normalise(layer.input_norm, rows);
   // query, key and value projections (:7004-7011) in one launch
   const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+  if (g_.activation_q8) {
+    const qllm_gemm_segment projections[3] = {
+        {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+        {key_, kv_rows, QLLM_OUT_F32},
+        {value_, kv_rows, QLLM_OUT_F32}};
+    status_check(qllm_fp4_gemm_q8_split(&layer.qkv.descriptor, q8_, q8_scales_,
+                                        projections, 3U, rows, gemm_workspace_,
+                                        gemm_workspace_bytes_, stream_));
+    // F32 attention output, quantised for the output projection (:7996)
+    enqueue_attention(index, rows, first_position, deferred_positions, query_,
+                      key_, value_,
+                      reinterpret_cast<std::uint16_t*>(activation_f32_));
+    enqueue_quantise(activation_f32_, rows, g_.query_heads * g_.head_dim);
+    enqueue_residual_projection(layer.output.descriptor, nullptr, 0U, rows, false);
+    return;
+  }
   const bool cut_qkv = qkv_splits_ > 1U &&
                        layer.qkv.descriptor.layout == QLLM_LAYOUT_TILED &&
                        layer.qkv.descriptor.padded_columns / 64U >= qkv_splits_;
@@ -1589,6 +1661,17 @@ void Mi355DenseFp4Provider::enqueue_ffn_block(std::uint32_t index,
                                               bool leave_partials) {
   const auto& layer = layers_[index];
   enqueue_normalise(layer.post_attention_norm, rows);
+  if (g_.activation_q8) {
+    // one quantisation shared by gate and up, the F32 SiLU product quantised
+    // again for the down projection (run_ffn, :8258-8290)
+    status_check(qllm_fp4_swiglu_q8(&layer.gate.descriptor, &layer.up.descriptor,
+                                    q8_, q8_scales_, activation_f32_, rows,
+                                    gemm_workspace_, gemm_workspace_bytes_,
+                                    stream_));
+    enqueue_quantise(activation_f32_, rows, g_.intermediate);
+    enqueue_residual_projection(layer.down.descriptor, nullptr, 0U, rows, false);
+    return;
+  }
   status_check(qllm_fp4_swiglu_bf16_balanced(
       &layer.gate.descriptor, &layer.up.descriptor, normalized_,
       std::size_t{rows} * g_.hidden * 2U, activation_, rows, gemm_workspace_,
@@ -1606,6 +1689,16 @@ void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
                                          std::uint32_t rows) {
   if (pending_partials_ && first_row != 0U)
     throw std::runtime_error("head over a row range needs a complete hidden state");
+  if (g_.activation_q8) {
+    enqueue_normalise_q8(hidden_ + std::size_t{first_row} * g_.hidden, final_norm_,
+                         rows);
+    status_check(qllm_fp4_gemm_q8(&head_.descriptor, q8_, q8_scales_, logits_,
+                                  QLLM_OUT_F32, nullptr, rows, stream_));
+    status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
+                                   select_workspace_, select_workspace_bytes_,
+                                   stream_));
+    return;
+  }
   if (first_row == 0U) {
     enqueue_normalise(final_norm_, rows);
   } else {
@@ -1814,6 +1907,11 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
     if (!embedding_ready_ || !head_ready_ || attention_ops_ != g_.layers ||
         ffn_ops_ != g_.layers)
       return {{er::ErrorCode::invalid_argument, "target program is not prepared"},
+              0U};
+    if (g_.activation_q8)
+      return {{er::ErrorCode::invalid_argument,
+               "the tall prompt path takes bf16 activation input; with Q8 "
+               "activations a prompt goes through the program in row batches"},
               0U};
     for (const auto token : tokens)
       if (token >= g_.vocabulary)
@@ -2160,7 +2258,35 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
     }
     const auto launch_one = [&](std::uint32_t index) {
       const auto& layer = layers_[index % g_.layers];
-      if (which == "ffn_gate_up") {
+      if (g_.activation_q8 && which != "attention") {
+        // the Q8 forms of the same launches (inputs: whatever q8_ holds)
+        const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
+        if (which == "ffn_gate_up") {
+          status_check(qllm_fp4_swiglu_q8(&layer.gate.descriptor,
+                                          &layer.up.descriptor, q8_, q8_scales_,
+                                          activation_f32_, rows, gemm_workspace_,
+                                          gemm_workspace_bytes_, stream_));
+        } else if (which == "ffn_down") {
+          status_check(qllm_fp4_gemm_q8(&layer.down.descriptor, q8_, q8_scales_,
+                                        query_, QLLM_OUT_F32, nullptr, rows, stream_));
+        } else if (which == "qkv") {
+          const qllm_gemm_segment projections[3] = {
+              {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
+              {key_, kv_rows, QLLM_OUT_F32},
+              {value_, kv_rows, QLLM_OUT_F32}};
+          status_check(qllm_fp4_gemm_q8_split(&layer.qkv.descriptor, q8_, q8_scales_,
+                                              projections, 3U, rows, gemm_workspace_,
+                                              gemm_workspace_bytes_, stream_));
+        } else if (which == "attention_output") {
+          status_check(qllm_fp4_gemm_q8(&layer.output.descriptor, q8_, q8_scales_,
+                                        query_, QLLM_OUT_F32, nullptr, rows, stream_));
+        } else if (which == "lm_head") {
+          status_check(qllm_fp4_gemm_q8(&head_.descriptor, q8_, q8_scales_, logits_,
+                                        QLLM_OUT_F32, nullptr, rows, stream_));
+        } else {
+          throw std::runtime_error("unknown kernel name: " + which);
+        }
+      } else if (which == "ffn_gate_up") {
         status_check(qllm_fp4_swiglu_bf16_balanced(
             &layer.gate.descriptor, &layer.up.descriptor, normalized_, hidden_bytes,
             activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream_));
@@ -2478,7 +2604,50 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                         mtp_embedding_, rows, stream));
   // [RMSNorm(embedding) | RMSNorm(previous target hidden)] -> fusion projection
   const std::size_t half_bytes = std::size_t{g_.hidden} * 2U;
-  if (g_.hidden <= 16384U) {
+  const bool q8 = g_.activation_q8;
+  // RMSNorm of `count` rows as the input of the projection that follows: bf16
+  // rows in normalized_, or Q8 rows in q8_
+  const auto normalise = [&](const float* rows_in, const float* weight,
+                             std::uint32_t count) {
+    if (q8) {
+      enqueue_normalise_q8(rows_in, weight, count);
+    } else {
+      status_check(qllm_rms_norm_batch(rows_in, weight, nullptr, normalized_,
+                                       g_.hidden, count, g_.hidden, g_.norm_epsilon,
+                                       g_.zero_centered_norm, stream));
+    }
+  };
+  // a projection of the rows prepared above (or of bf16 rows elsewhere)
+  const auto project = [&](const qllm_fp4_matrix& matrix, const std::uint16_t* bf16,
+                           std::size_t bf16_bytes, float* out, const float* residual,
+                           std::uint32_t count) {
+    if (q8)
+      status_check(qllm_fp4_gemm_q8(&matrix, q8_, q8_scales_, out, QLLM_OUT_F32,
+                                    residual, count, stream));
+    else
+      status_check(qllm_fp4_gemm_bf16(&matrix, bf16, bf16_bytes, out, QLLM_OUT_F32,
+                                      residual, count, stream));
+  };
+  if (q8) {
+    // both norms in F32 side by side, one quantisation of the 2 * hidden row
+    // (the fusion projection's input is one activation row, :8716-8735)
+    const std::size_t half_f32 = std::size_t{g_.hidden} * 4U;
+    status_check(qllm_rms_norm_batch(mtp_embedding_, mtp_.embedding_norm,
+                                     activation_f32_, nullptr, 0U, rows, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm, stream));
+    hip_check(hipMemcpy2DAsync(mtp_fusion_f32_, 2U * half_f32, activation_f32_,
+                               half_f32, half_f32, rows, hipMemcpyDeviceToDevice,
+                               hip_stream),
+              "assemble MTP normalized embedding batch");
+    status_check(qllm_rms_norm_batch(previous_hidden, mtp_.hidden_norm,
+                                     activation_f32_, nullptr, 0U, rows, g_.hidden,
+                                     g_.norm_epsilon, g_.zero_centered_norm, stream));
+    hip_check(hipMemcpy2DAsync(mtp_fusion_f32_ + g_.hidden, 2U * half_f32,
+                               activation_f32_, half_f32, half_f32, rows,
+                               hipMemcpyDeviceToDevice, hip_stream),
+              "assemble MTP target hidden batch");
+    enqueue_quantise(mtp_fusion_f32_, rows, 2U * g_.hidden);
+  } else if (g_.hidden <= 16384U) {
     status_check(qllm_rms_norm_concat_batch(
         mtp_embedding_, mtp_.embedding_norm, previous_hidden, mtp_.hidden_norm,
         mtp_fusion_input_, rows, g_.hidden, g_.norm_epsilon,
@@ -2499,26 +2668,27 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                hipMemcpyDeviceToDevice, hip_stream),
               "assemble MTP target hidden batch");
   }
-  status_check(qllm_fp4_gemm_bf16(&mtp_.fusion.descriptor, mtp_fusion_input_,
-                                  std::size_t{rows} * 2U * half_bytes,
-                                  mtp_hidden_, QLLM_OUT_F32, nullptr, rows,
-                                  stream));
+  project(mtp_.fusion.descriptor, mtp_fusion_input_,
+          std::size_t{rows} * 2U * half_bytes, mtp_hidden_, nullptr, rows);
 
   // one transformer block over its own Q8 cache (run_full_attention + run_ffn)
   const auto& layer = mtp_.layer;
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
   const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
-  status_check(qllm_rms_norm_batch(mtp_hidden_, layer.input_norm, nullptr,
-                                   normalized_, g_.hidden, rows, g_.hidden,
-                                   g_.norm_epsilon, g_.zero_centered_norm, stream));
+  normalise(mtp_hidden_, layer.input_norm, rows);
   const qllm_gemm_segment projections[3] = {
       {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
       {key_, kv_rows, QLLM_OUT_F32},
       {value_, kv_rows, QLLM_OUT_F32}};
-  status_check(qllm_fp4_gemm_bf16_split_balanced(
-      &layer.qkv.descriptor, normalized_, hidden_bytes, projections, 3U, rows,
-      gemm_workspace_, gemm_workspace_bytes_, stream));
+  if (q8)
+    status_check(qllm_fp4_gemm_q8_split(&layer.qkv.descriptor, q8_, q8_scales_,
+                                        projections, 3U, rows, gemm_workspace_,
+                                        gemm_workspace_bytes_, stream));
+  else
+    status_check(qllm_fp4_gemm_bf16_split_balanced(
+        &layer.qkv.descriptor, normalized_, hidden_bytes, projections, 3U, rows,
+        gemm_workspace_, gemm_workspace_bytes_, stream));
   const auto pages = const_cast<const void* const*>(device_page_table_);
   if (deferred_positions) {
     status_check(qllm_qkv_rope_batch_deferred(
@@ -2540,7 +2710,7 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   qllm_q8_attention_launch launch{};
   launch.query = query_;
   launch.device_pages = pages;
-  launch.output = attention_;
+  launch.output = q8 ? static_cast<void*>(activation_f32_) : attention_;
   launch.partial_maxima = partial_maxima_;
   launch.partial_sums = partial_sums_;
   launch.partial_outputs = partial_outputs_;
@@ -2555,28 +2725,30 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   launch.maximum_splits = maximum_splits_;
   launch.query_stride = query_stride;
   launch.output_gated = g_.output_gated;
-  launch.output_kind = QLLM_OUT_BF16;
+  launch.output_kind = g_.activation_q8 ? QLLM_OUT_F32 : QLLM_OUT_BF16;
   launch.stream = stream;
   launch.device_positions = deferred_positions ? mtp_positions_ : nullptr;
   status_check(qllm_attention_paged_q8(&launch));
-  status_check(qllm_fp4_gemm_bf16(
-      &layer.output.descriptor, attention_,
-      std::size_t{rows} * g_.query_heads * g_.head_dim * 2U, mtp_hidden_,
-      QLLM_OUT_F32, mtp_hidden_, rows, stream));
-  status_check(qllm_rms_norm_batch(mtp_hidden_, layer.post_attention_norm,
-                                   nullptr, normalized_, g_.hidden, rows,
-                                   g_.hidden, g_.norm_epsilon,
-                                   g_.zero_centered_norm, stream));
-  status_check(qllm_fp4_swiglu_bf16_balanced(
-      &layer.gate.descriptor, &layer.up.descriptor, normalized_, hidden_bytes,
-      activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream));
+  if (q8) enqueue_quantise(activation_f32_, rows, g_.query_heads * g_.head_dim);
+  project(layer.output.descriptor, attention_,
+          std::size_t{rows} * g_.query_heads * g_.head_dim * 2U, mtp_hidden_,
+          mtp_hidden_, rows);
+  normalise(mtp_hidden_, layer.post_attention_norm, rows);
+  if (q8) {
+    status_check(qllm_fp4_swiglu_q8(&layer.gate.descriptor, &layer.up.descriptor,
+                                    q8_, q8_scales_, activation_f32_, rows,
+                                    gemm_workspace_, gemm_workspace_bytes_, stream));
+    enqueue_quantise(activation_f32_, rows, g_.intermediate);
+  } else {
+    status_check(qllm_fp4_swiglu_bf16_balanced(
+        &layer.gate.descriptor, &layer.up.descriptor, normalized_, hidden_bytes,
+        activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream));
+  }
   // a single-row pass leaves its hidden state where the next pass reads it
   const bool retain_in_place = rows == 1U && produce_logits;
-  status_check(qllm_fp4_gemm_bf16(
-      &layer.down.descriptor, activation_,
-      std::size_t{rows} * g_.intermediate * 2U,
-      retain_in_place ? mtp_last_hidden_ : mtp_hidden_, QLLM_OUT_F32,
-      mtp_hidden_, rows, stream));
+  project(layer.down.descriptor, activation_,
+          std::size_t{rows} * g_.intermediate * 2U,
+          retain_in_place ? mtp_last_hidden_ : mtp_hidden_, mtp_hidden_, rows);
   if (produce_logits) {
     // draft head: the last row, draft norm, the head's first draft_vocabulary
     // rows
@@ -2586,14 +2758,9 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                     mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
                     g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
                 "retain final MTP hidden state");
-    const float* final_hidden = mtp_last_hidden_;
-    status_check(qllm_rms_norm_batch(final_hidden, mtp_.draft_norm, nullptr,
-                                     normalized_, g_.hidden, 1U, g_.hidden,
-                                     g_.norm_epsilon, g_.zero_centered_norm,
-                                     stream));
-    status_check(qllm_fp4_gemm_bf16(&mtp_.head_prefix, normalized_,
-                                    std::size_t{g_.hidden} * 2U, mtp_logits_,
-                                    QLLM_OUT_F32, nullptr, 1U, stream));
+    normalise(mtp_last_hidden_, mtp_.draft_norm, 1U);
+    project(mtp_.head_prefix, normalized_, std::size_t{g_.hidden} * 2U, mtp_logits_,
+            nullptr, 1U);
     status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U,
                                    mtp_argmax_, select_workspace_,
                                    select_workspace_bytes_, stream));
@@ -3213,6 +3380,8 @@ Mi355DenseFp4Provider::telemetry() const {
   values["provider_mtp_kv_page_offset"] = mtp_page_offset_;
   values["provider_weight_bytes"] = weight_bytes_;
   values["provider_kv_page_bytes"] = kv_page_bytes_;
+  // dense_fp4_provider.cpp:3117-3119
+  values["provider_dense_activation_input_bf16"] = g_.activation_q8 ? 0U : 1U;
   // dense_fp4_provider.cpp:3170-3200
   if (g_.profile_gpu_phases) {
     const auto phase = [this](GpuPhase which) {

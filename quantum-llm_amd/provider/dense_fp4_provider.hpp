@@ -62,6 +62,12 @@ struct DenseGeometry final {
   // passes of 4096 rows, whose o and down projections load the CUs unevenly;
   // the workspace of a pass is about 200 KB per row).
   std::uint32_t prefill_chunk_rows{0};
+  // The artifact's activation contract (prepare_dense_activation,
+  // dense_fp4_provider.cpp:5983-6003): true = every projection takes per-row
+  // Q8 activations and runs the reference's integer statement (the default of
+  // an artifact that does not declare dense_activation_input_bf16), false =
+  // bf16 activations.  Q8 needs block-32 UE8M0 weights and K % 64 == 0.
+  bool activation_q8{};
   // Requests that may be open at once (request slots,
   // dense_fp4_provider.cpp:5514-5518, 6554-6588): each owns its KV pages, its
   // presence bytes and its proposer state.
@@ -229,6 +235,11 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   [[nodiscard]] const float* hidden() const noexcept { return hidden_; }
   [[nodiscard]] void* stream() const noexcept { return stream_; }
   [[nodiscard]] const DenseGeometry& geometry() const noexcept { return g_; }
+  // The tall prompt path takes bf16 activations; with Q8 activations a prompt
+  // goes through the program in row batches.
+  [[nodiscard]] bool supports_tall_prefill() const noexcept {
+    return !g_.activation_q8;
+  }
   [[nodiscard]] bool profiles_gpu_phases() const noexcept {
     return g_.profile_gpu_phases;
   }
@@ -460,6 +471,16 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   // measured 11.4-14.5 us against 11.7 us uncut.
   float* qkv_partials_ = nullptr;          // [splits][rows][q + k + v rows]
   std::uint32_t qkv_splits_ = 0U;
+  // Q8 activation contract: the quantised rows of the projection about to
+  // run, their scales, and the F32 values they were quantised from
+  std::int8_t* q8_{};
+  float* q8_scales_{};
+  float* activation_f32_{};
+  float* mtp_fusion_f32_{};   // [rows, 2 * hidden] both input norms of the proposer
+  void enqueue_quantise(const float* input, std::uint32_t rows,
+                        std::uint32_t columns);
+  void enqueue_normalise_q8(const float* input, const float* weight,
+                            std::uint32_t rows);
   void* gemm_workspace_{};
   std::size_t gemm_workspace_bytes_{};
   void* select_workspace_{};

@@ -84,6 +84,7 @@ extern "C" qllm_provider* qllm_provider_create(
     g.mtp_layers = geometry->mtp_layers;
     g.draft_vocabulary = geometry->draft_vocabulary;
     g.prefill_chunk_rows = geometry->prefill_chunk_rows;
+    g.activation_q8 = geometry->activation_q8 != 0U;
     auto handle = std::make_unique<qllm_provider>();
     handle->provider = std::make_shared<qllm::Mi355DenseFp4Provider>(g);
     return handle.release();

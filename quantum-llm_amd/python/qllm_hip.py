@@ -102,12 +102,16 @@ SIGNATURES = {
     "qllm_fp4_gemm_balance_workspace_bytes": (c_size_t, []),
     "qllm_fp4_gemm_bf16_split_balanced": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_uint32, c_void_p, c_size_t, c_void_p]),
     "qllm_fp4_swiglu_bf16_balanced": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
+    "qllm_fp4_gemm_q8": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_uint32, c_void_p]),
+    "qllm_fp4_gemm_q8_split": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_size_t, c_void_p]),
+    "qllm_fp4_swiglu_q8": (c_int32, [POINTER(Fp4Matrix), POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_size_t, c_void_p]),
     "qllm_fp4_packed_weight_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_fp4_packed_scale_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32, c_uint32]),
     "qllm_fp4_prepack": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_void_p, c_void_p, POINTER(Fp4Matrix), c_void_p]),
     "qllm_fp4_unpack_rows": (c_int32, [POINTER(Fp4Matrix), c_uint32, c_uint32, c_void_p, c_void_p, c_void_p]),
     "qllm_fp4_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_uint32, c_void_p]),
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_residual_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),

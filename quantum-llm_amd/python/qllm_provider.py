@@ -29,7 +29,7 @@ class DenseGeometry(Structure):
                 ("kv_encoding", c_uint32), ("kv_page_tokens", c_uint32),
                 ("max_context", c_uint32), ("draft_depth", c_uint32),
                 ("mtp_layers", c_uint32), ("draft_vocabulary", c_uint32),
-                ("prefill_chunk_rows", c_uint32)]
+                ("prefill_chunk_rows", c_uint32), ("activation_q8", c_uint32)]
 
 
 SIGNATURES = {

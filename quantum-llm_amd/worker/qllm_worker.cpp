@@ -272,7 +272,7 @@ class Request final {
   void ingest(std::span<const std::uint32_t> prompt, Counters& counters) {
     const Stopwatch watch;
     const std::size_t batch = engine_.chunk_tokens();
-    if (prompt.size() > batch) {
+    if (prompt.size() > batch && engine_.provider().supports_tall_prefill()) {
       const auto result = engine_.provider().prefill(session_->state(), prompt,
                                                      position_, session_->request());
       expect_ok(result.status);

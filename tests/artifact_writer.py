@@ -89,7 +89,7 @@ class PackWriter:
 
 
 def dense_program(model, tensor_names, mtp=True, draft_depth=4, draft_vocabulary=0,
-                  max_context=4096, architecture="tiny.dense.fp4"):
+                  max_context=4096, architecture="tiny.dense.fp4", activation_input=None):
     """runtime-model.tsv text for a TinyModel; `tensor_names` is filled with
     the tensor name -> (kind, payload) map the pack must hold."""
     m = model
@@ -102,6 +102,13 @@ def dense_program(model, tensor_names, mtp=True, draft_depth=4, draft_vocabulary
     exact = "decode.mtp.dense-full-attention.fp4-block32.exact.v2"
     if mtp:
         kernels.append((exact, 2))
+    # the activation contract as the compiler writes it
+    # (compiler/expert_pack/compile.py:256-279): bf16 input is an attribute plus
+    # a required kernel, Q8 - the default - is the absence of both
+    if activation_input is None:
+        activation_input = "q8" if getattr(m, "activation_q8", False) else "bf16"
+    if activation_input == "bf16":
+        kernels.append(("dense.activation-input.bfloat16.v1", 1))
     d, Q, KV, H, I, V = (m.head_dim, m.query_heads, m.kv_heads, m.hidden,
                          m.intermediate, m.vocabulary)
     q_rows = Q * d * (2 if gated else 1)
@@ -124,6 +131,8 @@ def dense_program(model, tensor_names, mtp=True, draft_depth=4, draft_vocabulary
         ("rotary_dimension", m.rotary_dim),
         ("zero_centered_norm", int(m.zero_centered)),
         ("mtp_layers", 1 if mtp else 0)]
+    if activation_input == "bf16":
+        attributes.append(("dense_activation_input_bf16", 1))
     lines += [f"attribute\t{key}\t{value}" for key, value in attributes]
     embedding = fp4("model.embed_tokens.weight", m.embedding, V, H)
     final_norm = f32("model.norm.weight", m.final_norm)
@@ -203,12 +212,13 @@ def dense_program(model, tensor_names, mtp=True, draft_depth=4, draft_vocabulary
 
 def write_artifact(root, model, mtp=True, draft_depth=4, draft_vocabulary=0,
                    max_context=4096, program_text=None, mutate_manifest=None,
-                   completed=True):
+                   completed=True, activation_input=None):
     """Writes the directory; returns the manifest dictionary."""
     os.makedirs(root, exist_ok=True)
     tensors = {}
     text = dense_program(model, tensors, mtp=mtp, draft_depth=draft_depth,
-                         draft_vocabulary=draft_vocabulary, max_context=max_context)
+                         draft_vocabulary=draft_vocabulary, max_context=max_context,
+                         activation_input=activation_input)
     if program_text is not None:
         text = program_text
     pack = PackWriter()

@@ -74,10 +74,24 @@ class TinyModel:
             self.mtp["query_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
             self.mtp["key_norm"] = (0.1 * rng.standard_normal(head_dim)).astype(np.float32)
 
-    def linear(self, m, x_bf16, rows):
+    # The artifact's activation contract (prepare_dense_activation,
+    # dense_fp4_provider.cpp:5983-6003): False = bf16 activations into every
+    # projection, True = per-row Q8 and the integer statement (block-32 UE8M0
+    # weights only); intermediate activations then stay F32.
+    activation_q8 = False
+
+    def linear(self, m, x, rows):
         codes, scales = m
-        return ol.fp4_linear_f64(codes, scales, self.scheme, rows, codes.shape[1] * 2,
-                                 x_bf16)
+        padded = codes.shape[1] * 2
+        if self.activation_q8:
+            q8, act_scales = ol.quantize_q8_rows(x, padded)
+            return ol.fp4_linear_block32_q8(codes, scales, rows, padded, q8, act_scales)
+        return ol.fp4_linear_f64(codes, scales, self.scheme, rows, padded, x)
+
+    def activations(self, x):
+        """A projection's input as the contract has it: bf16-rounded, or F32
+        (the Q8 quantisation is part of the projection)."""
+        return np.asarray(x, dtype=np.float32) if self.activation_q8 else ol.bf16_round(x)
 
 
 def _record_slices(model, layer, page_tokens, position, kv_head):
@@ -124,7 +138,8 @@ def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
     codes, scales = m.embedding
     hidden = ol.fp4_embedding(codes, scales, m.scheme, m.hidden, m.hidden, tokens)
     for layer, block in enumerate(m.blocks):
-        x = ol.rms_norm_rows(hidden, block["input_norm"], m.eps, m.zero_centered, True)
+        x = ol.rms_norm_rows(hidden, block["input_norm"], m.eps, m.zero_centered,
+                             not m.activation_q8)
         q = m.linear(block["query"], x, Q * stride).reshape(rows, Q, stride)
         k = m.linear(block["key"], x, KV * d).reshape(rows, KV, d)
         v = m.linear(block["value"], x, KV * d).reshape(rows, KV, d)
@@ -158,15 +173,16 @@ def run_target(model: TinyModel, tokens, first_position, kv_pages, page_tokens,
             attention = ol.attention_f16(shape, q, kv_pages, True)
         else:
             attention = ol.attention_q4h(shape, q, kv_pages, "f64")
-        attention = ol.bf16_round(attention.reshape(rows, Q * d))
+        attention = m.activations(attention.reshape(rows, Q * d))
         hidden = hidden + m.linear(block["output"], attention, m.hidden)
         x = ol.rms_norm_rows(hidden, block["post_attention_norm"], m.eps,
-                             m.zero_centered, True)
+                             m.zero_centered, not m.activation_q8)
         gate = m.linear(block["gate"], x, m.intermediate)
         up = m.linear(block["up"], x, m.intermediate)
-        activation = ol.silu_product(gate, up, True)
+        activation = ol.silu_product(gate, up, not m.activation_q8)
         hidden = hidden + m.linear(block["down"], activation, m.hidden)
-    x = ol.rms_norm_rows(hidden, m.final_norm, m.eps, m.zero_centered, True)
+    x = ol.rms_norm_rows(hidden, m.final_norm, m.eps, m.zero_centered,
+                         not m.activation_q8)
     logits = m.linear(m.head, x, m.vocabulary)
     return logits, hidden
 
@@ -187,12 +203,14 @@ def run_mtp(model: TinyModel, tokens, previous_hidden, mtp_length, q8_pages,
     stride = d * (2 if m.output_gated else 1)
     codes, scales = m.embedding
     embedding = ol.fp4_embedding(codes, scales, m.scheme, m.hidden, m.hidden, tokens)
+    rounded = not m.activation_q8
     fused = np.concatenate([
-        ol.rms_norm_rows(embedding, w["embedding_norm"], m.eps, m.zero_centered, True),
-        ol.rms_norm_rows(previous_hidden, w["hidden_norm"], m.eps, m.zero_centered, True)],
+        ol.rms_norm_rows(embedding, w["embedding_norm"], m.eps, m.zero_centered, rounded),
+        ol.rms_norm_rows(previous_hidden, w["hidden_norm"], m.eps, m.zero_centered,
+                         rounded)],
         axis=1)
     hidden = m.linear(w["fusion"], fused, m.hidden)
-    x = ol.rms_norm_rows(hidden, w["input_norm"], m.eps, m.zero_centered, True)
+    x = ol.rms_norm_rows(hidden, w["input_norm"], m.eps, m.zero_centered, rounded)
     q = m.linear(w["query"], x, Q * stride).reshape(rows, Q, stride)
     k = m.linear(w["key"], x, KV * d).reshape(rows, KV, d)
     v = m.linear(w["value"], x, KV * d).reshape(rows, KV, d)
@@ -231,16 +249,17 @@ def run_mtp(model: TinyModel, tokens, previous_hidden, mtp_length, q8_pages,
     shape = ol.AttentionShape(rows, Q, KV, d, mtp_length + 1, page_tokens, 0,
                               int(m.output_gated))
     attention = ol.attention_q8(shape, q, q8_pages, page_offset)
-    attention = ol.bf16_round(attention.reshape(rows, Q * d))
+    attention = m.activations(attention.reshape(rows, Q * d))
     hidden = hidden + m.linear(w["output"], attention, m.hidden)
-    x = ol.rms_norm_rows(hidden, w["post_attention_norm"], m.eps, m.zero_centered, True)
+    x = ol.rms_norm_rows(hidden, w["post_attention_norm"], m.eps, m.zero_centered,
+                         rounded)
     activation = ol.silu_product(m.linear(w["gate"], x, m.intermediate),
-                                 m.linear(w["up"], x, m.intermediate), True)
+                                 m.linear(w["up"], x, m.intermediate), rounded)
     hidden = hidden + m.linear(w["down"], activation, m.hidden)
-    x = ol.rms_norm_rows(hidden[-1:], w["draft_norm"], m.eps, m.zero_centered, True)
+    x = ol.rms_norm_rows(hidden[-1:], w["draft_norm"], m.eps, m.zero_centered, rounded)
     head_codes, head_scales = m.head
-    logits = ol.fp4_linear_f64(head_codes[:draft_vocabulary], head_scales[:draft_vocabulary],
-                               m.scheme, draft_vocabulary, m.hidden, x)[0]
+    logits = m.linear((head_codes[:draft_vocabulary], head_scales[:draft_vocabulary]), x,
+                      draft_vocabulary)[0]
     return logits, hidden
 
 
@@ -257,7 +276,7 @@ def build_provider(model: TinyModel, qp, page_tokens=64, max_context=256,
         zero_centered_norm=int(m.zero_centered), scale_scheme=m.scheme,
         kv_encoding=kv_encoding, kv_page_tokens=page_tokens, max_context=max_context,
         draft_depth=4, mtp_layers=int(mtp), draft_vocabulary=draft_vocabulary,
-        prefill_chunk_rows=prefill_chunk_rows)
+        prefill_chunk_rows=prefill_chunk_rows, activation_q8=int(m.activation_q8))
     abi = 16 if m.scheme == ol.SCALE_F16_BLOCK16 else 3
     tag = "fp4-f16-block16" if m.scheme == ol.SCALE_F16_BLOCK16 else "fp4-block32"
     d, Q, KV, H, I, V = m.head_dim, m.query_heads, m.kv_heads, m.hidden, m.intermediate, m.vocabulary

@@ -412,3 +412,151 @@ def test_balanced_launch_rejects_a_bad_workspace(device):
         qh.call("qllm_fp4_swiglu_bf16_balanced", matrix, matrix, qh.ptr(buffer), 5 * 256,
                 qh.ptr(buffer), 5, 0, 1 << 22, None)
     del keep
+
+
+# ---- the reference's default activation contract (Q8 rows) on the matrix cores ----
+
+def _q8_case(device, rng, rows, columns, batch, x=None):
+    padded = (columns + 63) // 64 * 64
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    if x is None:
+        x = rng.standard_normal((batch, columns)).astype(np.float32)
+    q8, act_scales = ol.quantize_q8_rows(x, padded)
+    tensors = [gu.device_tensor(t, device) for t in (codes, scales)]
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, columns, padded,
+                                            ol.SCALE_UE8M0_BLOCK32), device)
+    return (codes, scales, padded, q8, act_scales, matrix, (tensors, keep),
+            gu.device_tensor(q8, device), gu.device_tensor(act_scales, device))
+
+
+def test_q8_matrix_core_gemm_on_the_reference_fixture(device):
+    """dense_fp4_cuda_smoke.cpp:139-216 (67 x 100 padded to 128, five rows of
+    0.7 sin(0.071 i)), its own threshold 2e-4 (:4911), through the streaming
+    layout and the matrix cores."""
+    rows, columns, padded, batch = 67, 100, 128, 5
+    r = np.arange(rows)[:, None]
+    scales = (124 + (r + np.arange(padded // 32)[None, :]) % 7).astype(np.uint8)
+    pair = np.arange(padded // 2)[None, :]
+    codes = (((r + 3 * pair) % 16) | (((5 * r + pair + 1) % 16) << 4)).astype(np.uint8)
+    x = (np.sin(np.arange(batch * columns, dtype=np.float32) * np.float32(0.071)) *
+         np.float32(0.7)).astype(np.float32).reshape(batch, columns)
+    q8, act_scales = ol.quantize_q8_rows(x, padded)
+    want = ol.fp4_linear_block32_q8(codes, scales, rows, padded, q8, act_scales)
+    d_codes, d_scales = gu.device_tensor(codes, device), gu.device_tensor(scales, device)
+    matrix, keep = qh.prepack(qh.fp4_matrix(d_codes, d_scales, rows, columns, padded, 0), device)
+    d_q8, d_s = gu.device_tensor(q8, device), gu.device_tensor(act_scales, device)
+    out = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemv_q8_batch", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out), batch,
+            0, None)
+    torch.cuda.synchronize()
+    assert np.abs(out.cpu().numpy() - want).max() < 2e-4
+    del keep
+
+
+@pytest.mark.parametrize("rows,columns,batch", [
+    (17408, 5120, 5), (5120, 17408, 5), (10240, 5120, 5), (5120, 8192, 5), (320, 192, 1),
+    (1000, 1000, 8), (96, 64, 3)])
+def test_q8_matrix_core_gemm_matches_the_integer_statement(device, rows, columns, batch):
+    """Model shapes (gate/up, down, q/k/v, o) and ragged ones against
+    qo_fp4_linear_block32_q8 - integer block sums, one F32 FMA per block - at
+    the reference's own 2e-4; with a residual and the three output kinds."""
+    rng = np.random.default_rng(rows * 7 + columns)
+    codes, scales, padded, q8, act_scales, matrix, keep, d_q8, d_s = _q8_case(
+        device, rng, rows, columns, batch)
+    want = ol.fp4_linear_block32_q8(codes, scales, rows, padded, q8, act_scales)
+    bound = 2e-4 * max(1.0, np.abs(want).max())
+    out = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out), qh.OUT_F32,
+            None, batch, None)
+    torch.cuda.synchronize()
+    assert np.abs(out.cpu().numpy() - want).max() <= bound
+    residual = rng.standard_normal((batch, rows)).astype(np.float32)
+    d_residual = gu.device_tensor(residual, device)
+    qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(d_residual),
+            qh.OUT_F32, qh.ptr(d_residual), batch, None)
+    rounded = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(rounded),
+            qh.OUT_F32_BF16_ROUNDED, None, batch, None)
+    torch.cuda.synchronize()
+    assert np.abs(d_residual.cpu().numpy() - (want + residual)).max() <= bound + 1e-5
+    assert np.array_equal(rounded.cpu().numpy(), ol.bf16_round(out.cpu().numpy()))
+    del keep
+
+
+def test_q8_matrix_core_head_on_sampled_vocabulary_rows(device):
+    """lm_head [151936, 5120] x Q8 rows: the whole launch, 512 sampled rows
+    against the integer statement."""
+    rows, columns, batch = 151936, 5120, 5
+    codes = torch.randint(0, 256, (rows, columns // 2), dtype=torch.uint8, device=device)
+    scales = torch.randint(118, 124, (rows, columns // 32), dtype=torch.uint8, device=device)
+    matrix, keep = qh.prepack(qh.fp4_matrix(codes, scales, rows, columns, columns, 0), device)
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((batch, columns)).astype(np.float32)
+    q8, act_scales = ol.quantize_q8_rows(x, columns)
+    d_q8, d_s = gu.device_tensor(q8, device), gu.device_tensor(act_scales, device)
+    out = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out), qh.OUT_F32,
+            None, batch, None)
+    torch.cuda.synchronize()
+    pick = np.sort(rng.choice(rows, 512, replace=False))
+    index = torch.from_numpy(pick).to(device)
+    want = ol.fp4_linear_block32_q8(codes[index].cpu().numpy(), scales[index].cpu().numpy(),
+                                    len(pick), columns, q8, act_scales)
+    got = out.cpu().numpy()[:, pick]
+    assert np.abs(got - want).max() <= 2e-4 * max(1.0, np.abs(want).max())
+    del keep
+
+
+def test_q8_split_and_swiglu_forms(device):
+    """q/k/v as three segments equal the one-output launch bit for bit; the
+    fused gate/up launch stores silu(gate) * up in F32 from the same sums."""
+    rng = np.random.default_rng(77)
+    rows, columns, batch = 1536, 1024, 5
+    codes, scales, padded, q8, act_scales, matrix, keep, d_q8, d_s = _q8_case(
+        device, rng, rows, columns, batch)
+    whole = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(whole), qh.OUT_F32,
+            None, batch, None)
+    parts = [1024, 256, 256]
+    outs = [torch.zeros((batch, part), device=device) for part in parts]
+    segments = (qh.GemmSegment * 3)(*[qh.GemmSegment(qh.ptr(o), part, qh.OUT_F32)
+                                      for o, part in zip(outs, parts)])
+    qh.call("qllm_fp4_gemm_q8_split", matrix, qh.ptr(d_q8), qh.ptr(d_s), segments, 3, batch,
+            None, 0, None)
+    up_codes, up_scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    up_tensors = [gu.device_tensor(t, device) for t in (up_codes, up_scales)]
+    up_matrix, keep_up = qh.prepack(qh.fp4_matrix(up_tensors[0], up_tensors[1], rows, columns,
+                                                  padded, 0), device)
+    fused = torch.zeros((batch, rows), device=device)
+    qh.call("qllm_fp4_swiglu_q8", matrix, up_matrix, qh.ptr(d_q8), qh.ptr(d_s),
+            qh.ptr(fused), batch, None, 0, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(np.concatenate([o.cpu().numpy() for o in outs], axis=1),
+                          whole.cpu().numpy())
+    gate = ol.fp4_linear_block32_q8(codes, scales, rows, padded, q8, act_scales)
+    up = ol.fp4_linear_block32_q8(up_codes, up_scales, rows, padded, q8, act_scales)
+    want = ol.silu_product(gate, up, False)
+    got = fused.cpu().numpy()
+    assert np.abs(got - want).max() <= 2e-4 * max(1.0, np.abs(want).max())
+    del keep, keep_up
+
+
+def test_q8_matrix_core_gemm_rejects_what_it_does_not_take(device):
+    rng = np.random.default_rng(3)
+    codes, scales, padded, q8, act_scales, matrix, keep, d_q8, d_s = _q8_case(
+        device, rng, 64, 128, 2)
+    out = torch.zeros((2, 64), device=device)
+    f16_codes, f16_scales = synth.fp4_matrix(rng, 64, 128, ol.SCALE_F16_BLOCK16)
+    tensors = [gu.device_tensor(t, device) for t in (f16_codes, f16_scales)]
+    f16_matrix, keep2 = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], 64, 128, 128,
+                                                 ol.SCALE_F16_BLOCK16), device)
+    with pytest.raises(qh.QllmError):      # binary16 block-16 scales have no Q8 form
+        qh.call("qllm_fp4_gemm_q8", f16_matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out),
+                qh.OUT_F32, None, 2, None)
+    with pytest.raises(qh.QllmError):      # no scales
+        qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), None, qh.ptr(out), qh.OUT_F32,
+                None, 2, None)
+    with pytest.raises(qh.QllmError):      # batch > 8
+        qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out),
+                qh.OUT_F32, None, 9, None)
+    del keep, keep2

@@ -332,3 +332,55 @@ def test_batched_topk_rejects_what_it_does_not_take(device):
         with pytest.raises(qh.QllmError):
             qh.call("qllm_topk_logits_batch", qh.ptr(values), count, stride, k, rows,
                     qh.ptr(out_v), qh.ptr(out_i), qh.ptr(workspace), bytes_, None)
+
+
+@pytest.mark.parametrize("zero_centered", [False, True])
+@pytest.mark.parametrize("rows,elements", [(5, 5120), (1, 256), (8, 16384), (3, 1000)])
+def test_norm_into_q8_equals_norm_then_quantise(device, rows, elements, zero_centered):
+    """qllm_rms_norm_q8_batch against qllm_rms_norm_batch + qllm_quantize_q8_batch
+    (bit-equal: the same operations on the same values) and against the
+    oracle's Q8 of the oracle's norm (the reference's quantiser is byte-exact
+    on equal inputs; the norms agree to F32 rounding, so a code may differ by
+    one step where a value sits on a rounding boundary)."""
+    rng = np.random.default_rng(rows + elements)
+    x = (2.0 * rng.standard_normal((rows, elements))).astype(np.float32)
+    weight = (0.2 * rng.standard_normal(elements)).astype(np.float32)
+    d_x, d_w = gu.device_tensor(x, device), gu.device_tensor(weight, device)
+    fused_q8 = torch.zeros((rows, elements), dtype=torch.int8, device=device)
+    fused_scales = torch.zeros(rows, device=device)
+    qh.call("qllm_rms_norm_q8_batch", qh.ptr(d_x), qh.ptr(d_w), qh.ptr(fused_q8),
+            qh.ptr(fused_scales), rows, elements, 1e-6, int(zero_centered), None)
+    normed = torch.zeros((rows, elements), device=device)
+    qh.call("qllm_rms_norm_batch", qh.ptr(d_x), qh.ptr(d_w), qh.ptr(normed), None, 0, rows,
+            elements, 1e-6, int(zero_centered), None)
+    two_q8 = torch.zeros((rows, elements), dtype=torch.int8, device=device)
+    two_scales = torch.zeros(rows, device=device)
+    qh.call("qllm_quantize_q8_batch", qh.ptr(normed), qh.ptr(two_q8), qh.ptr(two_scales),
+            rows, elements, elements, 0, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(fused_q8.cpu().numpy(), two_q8.cpu().numpy())
+    assert np.array_equal(fused_scales.cpu().numpy(), two_scales.cpu().numpy())
+    # the quantiser itself, byte-exact against the oracle on the GPU's own norm
+    want_q8, want_scales = ol.quantize_q8_rows(normed.cpu().numpy(), elements)
+    assert np.array_equal(two_q8.cpu().numpy(), want_q8)
+    assert np.array_equal(two_scales.cpu().numpy(), want_scales)
+    reference = ol.rms_norm_rows(x, weight, 1e-6, zero_centered, False)
+    q8, _ = ol.quantize_q8_rows(reference, elements)
+    assert np.abs(q8.astype(np.int32) - want_q8.astype(np.int32)).max() <= 1
+
+
+@pytest.mark.parametrize("rows,columns,padded", [(5, 17408, 17408), (5, 8192, 8192),
+                                                 (2, 20480, 20480), (3, 100, 128)])
+def test_wide_rows_quantise_byte_exactly(device, rows, columns, padded):
+    rng = np.random.default_rng(columns)
+    x = (3.0 * rng.standard_normal((rows, columns))).astype(np.float32)
+    x[0, 7] = 0.0
+    d_x = gu.device_tensor(x, device)
+    d_q8 = torch.full((rows, padded), 5, dtype=torch.int8, device=device)
+    d_s = torch.zeros(rows, device=device)
+    qh.call("qllm_quantize_q8_batch", qh.ptr(d_x), qh.ptr(d_q8), qh.ptr(d_s), rows, columns,
+            padded, 0, None)
+    torch.cuda.synchronize()
+    want_q8, want_scales = ol.quantize_q8_rows(x, padded)
+    assert np.array_equal(d_q8.cpu().numpy(), want_q8)
+    assert np.array_equal(d_s.cpu().numpy(), want_scales)
