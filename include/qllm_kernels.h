@@ -340,6 +340,17 @@ int32_t qllm_rms_norm_concat_batch(const float* first,
                                    uint32_t elements, float epsilon,
                                    int32_t zero_centered, void* stream);
 
+/* The same with the first half's rows taken from an FP4 embedding matrix
+ * (row-major) at `tokens`: qllm_fp4_embedding_batch folded into the norm - the
+ * proposer's embedding lookup and its two input norms in one launch (run_mtp,
+ * dense_fp4_provider.cpp:8699-8735).  Same values as the lookup followed by
+ * qllm_rms_norm_concat_batch; elements = embedding->columns. */
+int32_t qllm_rms_norm_concat_embedding_batch(
+    const qllm_fp4_matrix* embedding, const uint32_t* tokens,
+    const float* first_weight, const float* second, const float* second_weight,
+    void* output_bf16, uint32_t rows, float epsilon, int32_t zero_centered,
+    void* stream);
+
 /* replaces add_in_place (transformer_kernels.hpp:310-312). */
 int32_t qllm_add_in_place(float* destination, const float* source,
                           uint32_t elements, int32_t bf16_output,
@@ -653,6 +664,22 @@ int32_t qllm_store_kv_paged_q8_batch_deferred(
     const uint32_t* device_positions, uint32_t rows, uint32_t kv_heads,
     uint32_t head_dim, void* stream);
 
+/* qllm_qkv_rope_batch and qllm_store_kv_paged_q8_batch in one launch: the
+ * rotary of a batch's queries and keys, then the rotated key and the value of
+ * every (row, kv head) as Q8 records - the proposer's
+ * gated_gqa_qkv_rope_paged_batch_kernel<q8> (transformer_kernels.cu:3550-3643,
+ * records :601-625).  Same values and bytes as the two launches.
+ * device_positions (NULL, or device words read when the kernel runs): word 0
+ * the first cache position, word 1 the first rotary position. */
+int32_t qllm_qkv_rope_store_q8_batch(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, size_t page_offset_bytes, uint32_t page_tokens,
+    uint32_t first_cache_position, uint32_t first_rotary_position,
+    const uint32_t* device_positions, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream);
+
 /* replaces gated_gqa_attention_microbatch_paged_q8_tensor_core and
  * gated_gqa_attention_decode_paged_q8_tensor_core (transformer_kernels.hpp:
  * 873, 944; launch struct PagedQ8GatedGqaPrefillLaunch): row r attends tokens
@@ -710,6 +737,29 @@ int32_t qllm_rollout_advance(const uint32_t* selected, uint32_t* next_token,
                              uint32_t* draft_tokens, uint32_t capacity,
                              uint32_t rows, uint32_t* device_positions,
                              void* stream);
+
+/* A head: logits [batch, rows] = matrix . input (qllm_fp4_gemm_bf16, F32
+ * output) and tokens[m] = arg-max of row m (qllm_argmax_batch's ordering:
+ * larger first, ties to the lower id, NaN never, 0xffffffff for a row without
+ * a selectable value), in two launches: the projection's epilogue leaves every
+ * tile's best (value, row) in `workspace`, one block per batch row picks the
+ * winner.  Replaces the projection followed by argmax_batch_kernel in run_head
+ * (dense_fp4_provider.cpp:8393-8432; kernel transformer_kernels.cu:7059-7092)
+ * without the second pass over the logits.  With `advance` (batch 1) the
+ * winner is also handed on as qllm_rollout_advance does.  K % 64 == 0. */
+typedef struct qllm_rollout_step {
+  uint32_t* next_token;        /* device: the next pass's input token */
+  uint32_t* draft_tokens;      /* device: draft list, entry positions[3] */
+  uint32_t capacity;           /* entries of draft_tokens */
+  uint32_t rows;               /* positions 0..2 advance by this */
+  uint32_t* device_positions;  /* device: cache, rotary, context, draft slot */
+} qllm_rollout_step;
+size_t qllm_fp4_head_workspace_bytes(const qllm_fp4_matrix* matrix, uint32_t batch);
+int32_t qllm_fp4_head_argmax(const qllm_fp4_matrix* matrix, const void* input,
+                             size_t input_bytes, float* logits, uint32_t batch,
+                             uint32_t* tokens, void* workspace,
+                             size_t workspace_bytes,
+                             const qllm_rollout_step* advance, void* stream);
 
 /* replaces argmax_batch (transformer_kernels.hpp:1266-1269): ties to the
  * lower index, NaN never wins.  workspace: at least

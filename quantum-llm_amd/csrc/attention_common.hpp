@@ -128,27 +128,67 @@ __device__ __forceinline__ uint32_t uniform_word(const uint32_t* words,
   return ((constant_words)words)[index];
 }
 
+// One wave writes the K (kind 0) or V (kind 1) vector of (cache slot, kv head)
+// into the proposer's Q8 layer at `layer_base` (page + the layer's offset):
+// codes [kind][slot][kv head][head_dim] int8, then scales [kind][kv head]
+// [page_tokens] binary16; scale = f16(max(absmax / 127, 2^-24)), code =
+// clamp(rn(x / scale), -127, 127) (transformer_kernels.cu:601-625).  `source`
+// may lie in LDS or in global memory.
+__device__ __forceinline__ void q8_encode_record(const float* source,
+                                                 uint32_t head_dim, uint8_t* layer_base,
+                                                 uint32_t kind, uint32_t slot,
+                                                 uint32_t kv_head, uint32_t kv_heads,
+                                                 uint32_t page_tokens, uint32_t lane) {
+  const size_t codes_bytes = static_cast<size_t>(page_tokens) * kv_heads * head_dim;
+  const size_t record = static_cast<size_t>(slot) * kv_heads + kv_head;
+  float maximum = 0.0f;
+  for (uint32_t index = lane; index < head_dim; index += 64u)
+    maximum = fmaxf(maximum, fabsf(source[index]));
+  maximum = wave_max(maximum);
+  const uint32_t scale_bits = f32_to_f16_bits(fmaxf(maximum / 127.0f, 0x1p-24f));
+  const float scale = f16_bits_to_f32(scale_bits);
+  int8_t* codes =
+      reinterpret_cast<int8_t*>(layer_base + kind * codes_bytes) + record * head_dim;
+  for (uint32_t index = lane; index < head_dim; index += 64u) {
+    const int code = max(-127, min(127, __float2int_rn(source[index] / scale)));
+    codes[index] = static_cast<int8_t>(code);
+  }
+  if (lane == 0u) {
+    uint16_t* scales = reinterpret_cast<uint16_t*>(layer_base + 2u * codes_bytes) +
+                       static_cast<size_t>(kind) * kv_heads * page_tokens;
+    scales[static_cast<size_t>(kv_head) * page_tokens + slot] =
+        static_cast<uint16_t>(scale_bits);
+  }
+}
+
 // Tiles [first, last) of the context that wave `wave` of split `split` walks.
 // split_tokens == 0: balanced - the context's tiles are dealt evenly over
 // every wave of the grid row, whatever the context length.  Otherwise split
 // s covers tokens [s*split_tokens, (s+1)*split_tokens) and its tiles are dealt
 // evenly over the workgroup's waves.
+// tail_work (balanced only): what the waves at the end of the context do
+// besides their tiles, in tiles' worth of time - the deal is over
+// context_tiles + tail_work tiles of which the last tail_work do not exist, so
+// those waves walk that many fewer.
 __device__ __forceinline__ void wave_tile_range(uint32_t context_tiles,
                                                 uint32_t tile_tokens,
                                                 uint32_t split_tokens,
                                                 uint32_t split, uint32_t splits,
                                                 uint32_t wave,
                                                 uint32_t& tile_first,
-                                                uint32_t& tile_last) {
+                                                uint32_t& tile_last,
+                                                uint32_t tail_work = 0u) {
   if (split_tokens == 0u) {
     // floor(slot * tiles / slots) in 32-bit arithmetic: with tiles = q * slots
     // + r it is slot * q + floor(slot * r / slots), and slot * r < slots^2
     const uint32_t slots = splits * kSplitWaves;
     const uint32_t slot = split * kSplitWaves + wave;
-    const uint32_t quotient = context_tiles / slots;
-    const uint32_t remainder = context_tiles - quotient * slots;
-    tile_first = slot * quotient + slot * remainder / slots;
-    tile_last = (slot + 1u) * quotient + (slot + 1u) * remainder / slots;
+    const uint32_t dealt = context_tiles + tail_work;
+    const uint32_t quotient = dealt / slots;
+    const uint32_t remainder = dealt - quotient * slots;
+    tile_first = min(slot * quotient + slot * remainder / slots, context_tiles);
+    tile_last = min((slot + 1u) * quotient + (slot + 1u) * remainder / slots,
+                    context_tiles);
   } else {
     const uint32_t split_tiles = split_tokens / tile_tokens;
     const uint32_t begin = min(split * split_tiles, context_tiles);

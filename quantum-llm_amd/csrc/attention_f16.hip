@@ -69,31 +69,11 @@ __global__ __launch_bounds__(64) void q8_store_kernel(
   uint8_t* page = static_cast<uint8_t*>(const_cast<void*>(
                       page_table[position / page_tokens])) + page_offset;
   const uint32_t slot = position % page_tokens;
-  const size_t codes_bytes = static_cast<size_t>(page_tokens) * kv_heads * head_dim;
-  const size_t record = static_cast<size_t>(slot) * kv_heads + kv_head;
 #pragma unroll
-  for (int kind = 0; kind < 2; ++kind) {
-    const float* source = (kind ? value : key) +
-                          (static_cast<size_t>(row) * kv_heads + kv_head) * head_dim;
-    float maximum = 0.0f;
-    for (uint32_t index = lane; index < head_dim; index += 64u)
-      maximum = fmaxf(maximum, fabsf(source[index]));
-    maximum = wave_max(maximum);
-    const uint32_t scale_bits = f32_to_f16_bits(fmaxf(maximum / 127.0f, 0x1p-24f));
-    const float scale = f16_bits_to_f32(scale_bits);
-    int8_t* codes = reinterpret_cast<int8_t*>(page + kind * codes_bytes) +
-                    record * head_dim;
-    for (uint32_t index = lane; index < head_dim; index += 64u) {
-      const int code = max(-127, min(127, __float2int_rn(source[index] / scale)));
-      codes[index] = static_cast<int8_t>(code);
-    }
-    if (lane == 0u) {
-      uint16_t* scales = reinterpret_cast<uint16_t*>(page + 2u * codes_bytes) +
-                         static_cast<size_t>(kind) * kv_heads * page_tokens;
-      scales[static_cast<size_t>(kv_head) * page_tokens + slot] =
-          static_cast<uint16_t>(scale_bits);
-    }
-  }
+  for (uint32_t kind = 0; kind < 2u; ++kind)
+    q8_encode_record((kind ? value : key) +
+                         (static_cast<size_t>(row) * kv_heads + kv_head) * head_dim,
+                     head_dim, page, kind, slot, kv_head, kv_heads, page_tokens, lane);
 }
 
 // 8 int8 codes -> 8 exact binary16 values: code + 128 becomes the low mantissa

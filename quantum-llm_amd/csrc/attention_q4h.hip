@@ -170,6 +170,41 @@ __device__ __forceinline__ void lds_wait(T (&values)[N]) {
                    "+v"(values[12]), "+v"(values[13]), "+v"(values[14]),
                    "+v"(values[15]) :: "memory");
 }
+// Global loads the compiler's wait insertion does not see, for values whose
+// arrival the kernel waits for itself (vmem_wait_units, then tie()): a wait the
+// compiler places counts only the loads it knows, so it would also wait for
+// every direct-to-LDS load issued after them.  `base` is wave-uniform.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+template <int OFFSET>
+__device__ __forceinline__ float load_f32_uncounted(const void* base,
+                                                    uint32_t byte_offset) {
+  float value;
+  asm volatile("global_load_dword %0, %1, %2 offset:%3"
+               : "=v"(value) : "v"(byte_offset), "s"(base), "n"(OFFSET) : "memory");
+  return value;
+}
+__device__ __forceinline__ f32x2 load_f32x2_uncounted(const void* base,
+                                                      uint32_t byte_offset) {
+  f32x2 value;
+  asm volatile("global_load_dwordx2 %0, %1, %2"
+               : "=v"(value) : "v"(byte_offset), "s"(base) : "memory");
+  return value;
+}
+// orders every use of `value` after the volatile statements before this one
+template <typename T>
+__device__ __forceinline__ void tie(T& value) {
+  asm volatile("" : "+v"(value));
+}
+// at most `units` * UNIT vmem loads still in flight; `units` is wave-uniform
+template <int UNIT>
+__device__ __forceinline__ void vmem_wait_units(uint32_t units) {
+  static_assert(4 * UNIT < 64, "vmcnt holds six bits");
+  if (units == 0u) vmem_wait<0>();
+  else if (units == 1u) vmem_wait<UNIT>();
+  else if (units == 2u) vmem_wait<2 * UNIT>();
+  else if (units == 3u) vmem_wait<3 * UNIT>();
+  else vmem_wait<4 * UNIT>();
+}
 // (value & mask) | (base & ~mask) in one instruction
 __device__ __forceinline__ uint32_t insert_bits(uint32_t mask, uint32_t value,
                                                 uint32_t base) {
@@ -439,7 +474,14 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   constexpr int PASSES = ROW / 16;    // direct loads per code plane and tile
   constexpr int KS_LOADS = PASSES + 1;       // K codes + K scales
   constexpr int V_LOADS = PASSES + 1;        // V codes + V scales
-  __shared__ __attribute__((aligned(16))) uint8_t stage[kSplitWaves * STAGE];
+  static_assert(KS_LOADS == V_LOADS, "the waits count loads in units of one half tile");
+  // Tiles of a wave in flight.  At head_dim 128 LDS holds two staging areas
+  // per wave: the wave's first two tiles set out together at the start (at
+  // 32K tokens a wave has two tiles in all), and a tile's half is refilled
+  // with the tile after the next.
+  constexpr int DEPTH = 1;
+  __shared__ __attribute__((aligned(16)))
+  uint8_t stage[kSplitWaves * STAGE * DEPTH];
   // query operands in MFMA order, then per matrix row its scale and the number
   // of tokens it may attend
   __shared__ __attribute__((aligned(16)))
@@ -461,12 +503,18 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
   // tiles [tile_first, tile_last) of this wave
   uint32_t tile_first, tile_last;
+  // (fused: the workgroup at the end of the context also encodes the batch's
+  // K/V records, lays them over its tiles and writes them to their pages -
+  // about two tiles' worth of time for each of its waves.  The plain kernel
+  // deals the same way, so that both add up a context in the same order.)
+  constexpr uint32_t kTailWork = 2u * kSplitWaves;
   wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y, wave,
-                  tile_first, tile_last);
+                  tile_first, tile_last, kTailWork);
 
-  uint8_t* stage_k = stage + wave * STAGE;
+  // the wave's staging areas: tile t of the wave uses area t % DEPTH
+  uint8_t* const stage_base = stage + wave * (STAGE * DEPTH);
   const uint32_t stage_k_lds =
-      __builtin_amdgcn_readfirstlane(lds_address(stage_k));
+      __builtin_amdgcn_readfirstlane(lds_address(stage_base));
   const uint32_t stage_s_lds = stage_k_lds + CODES;
   const uint32_t stage_v_lds = stage_s_lds + 256;
   const uint32_t stage_vs_lds = stage_v_lds + CODES;
@@ -484,7 +532,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // KS_LOADS direct loads: K codes and K scales of a tile.  Pass `pass` covers
   // the 1 KiB at pass*1024 of the tile's K rows; lanes 0..31 then fetch the
   // scales of tokens 2l, 2l+1 (lanes 32..63 repeat them).
-  auto stage_keys = [&](uint32_t tile) {
+  auto stage_keys = [&](uint32_t tile, uint32_t area) {
     const uint32_t lane_now = fresh_lane_index();
     const uint32_t tile_begin = tile * 64u;
     const void* page = uniform_page(args.page_table, tile_begin / args.page_tokens);
@@ -497,14 +545,14 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass)
       copy16_to_lds(key_rows + pass * 1024, lane_now * 16u,
-                    stage_k_lds + pass * 1024);
-    copy4_to_lds(key_scales, 4u * (lane_now & 31u), stage_s_lds);
+                    stage_k_lds + area + pass * 1024);
+    copy4_to_lds(key_scales, 4u * (lane_now & 31u), stage_s_lds + area);
   };
   // V_LOADS direct loads: V codes and V scales of a tile.  V row R holds token
   // 16*((R/4)%4) + 4*(R/16) + R%4, so the 16 tokens a lane group reads back
   // transposed sit in 16 consecutive rows; the lane's share of that map is
   // separable from the pass's share.
-  auto stage_values = [&](uint32_t tile) {
+  auto stage_values = [&](uint32_t tile, uint32_t area) {
     const uint32_t lane_now = fresh_lane_index();
     const uint32_t lane_row = lane_now / kParts;  // row inside a pass
     const uint32_t value_lane_offset =
@@ -526,9 +574,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       const uint32_t pass_token = 16u * ((first_row >> 2) & 3u) +
                                   4u * (first_row >> 4) + (first_row & 3u);
       copy16_to_lds(value_rows + pass_token * ROW, value_lane_offset,
-                    stage_v_lds + pass * 1024);
+                    stage_v_lds + area + pass * 1024);
     }
-    copy4_to_lds(value_scales, 4u * (lane_now & 31u), stage_vs_lds);
+    copy4_to_lds(value_scales, 4u * (lane_now & 31u), stage_vs_lds + area);
+  };
+  // The wave's first DEPTH tiles set out; returns how many half tiles (K or V
+  // of one tile) that put in flight.
+  auto stage_first_tiles = [&]() -> uint32_t {
+    uint32_t halves = 0u;
+#pragma unroll
+    for (int ahead = 0; ahead < DEPTH; ++ahead)
+      if (tile_first + ahead < tile_last) {
+        stage_keys(tile_first + ahead, ahead * STAGE);
+        stage_values(tile_first + ahead, ahead * STAGE);
+        halves += 2u;
+      }
+    return halves;
   };
 
   // ---- query operands (B side of S = K.Q), built once per workgroup ---------
@@ -540,7 +601,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   // fused mode: scratch of the per-wave rotary, then the batch's fresh K/V
   // records [K codes | V codes | K scale | V scale] of this KV head
   constexpr int RECORD = D + 16;
-  constexpr int FRESH_ROWS = FUSED ? RT * 16 : 1;
+  // (the fused launch takes at most 16 rows)
+  constexpr int FRESH_ROWS = FUSED ? 16 : 1;
   // at head_dim 256 the rotary scratch lies in the (still empty) staging area
   // and the first tile sets out after the query work: LDS has no room for both
   constexpr bool SCRATCH_IN_STAGE = D == 256;
@@ -551,7 +613,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   if constexpr (FUSED) {
     first_cache_position = args.device_positions ? uniform_word(args.device_positions, 0u)
                                                  : args.first_cache_position;
-    float* shared = SCRATCH_IN_STAGE ? reinterpret_cast<float*>(stage_k)
+    float* shared = SCRATCH_IN_STAGE ? reinterpret_cast<float*>(stage_base)
                                      : rope_scratch + wave * (2 * D);
     float* rotated = shared + D;
     const uint32_t half = args.rotary_dim / 2u;
@@ -559,19 +621,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     constexpr int ROWS_PER_WAVE = RT * 16 / kSplitWaves;
     // Everything the wave will need comes in one round trip: its query rows
     // (matrix rows wave, wave + 8, ...), the batch's K/V row it encodes, norm
-    // weights and the rows' (cos, sin).
+    // weights and the rows' (cos, sin).  The loads before the tiles are ones
+    // the kernel waits for itself, so that the tiles stay in flight behind
+    // them while the rows are rotated and quantised.
     float q_values[ROWS_PER_WAVE][N];
-    float2 q_entry[ROWS_PER_WAVE][N];
+    f32x2 q_entry_raw[ROWS_PER_WAVE][N];
     float weights[2][N];                            // query norm, key norm
     // (without norm weights the loads read the query buffer instead and their
     // values go unused: no branch, no wait of its own)
     const float* q_weight = args.q_weight ? args.q_weight : args.query;
     const float* k_weight = args.k_weight ? args.k_weight : args.query;
-#pragma unroll
-    for (int k = 0; k < N; ++k) {
-      weights[0][k] = q_weight[lane + 64u * k];
-      weights[1][k] = k_weight[lane + 64u * k];
-    }
+    [&]<int... K>(std::integer_sequence<int, K...>) {
+      ((weights[0][K] = load_f32_uncounted<256 * K>(uniform_pointer(
+            reinterpret_cast<const uint8_t*>(q_weight)), 4u * lane)), ...);
+      ((weights[1][K] = load_f32_uncounted<256 * K>(uniform_pointer(
+            reinterpret_cast<const uint8_t*>(k_weight)), 4u * lane)), ...);
+    }(std::make_integer_sequence<int, N>{});
     // (rows past the batch fetch the last row again; nothing uses the values.
     // Row and head of matrix row wave + 8 item follow from those of the row
     // before, all on the scalar unit)
@@ -597,11 +662,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
                               member) * args.query_stride)));
         const float2* entries = reinterpret_cast<const float2*>(uniform_pointer(
             reinterpret_cast<const uint8_t*>(args.rope_table + fetched_row * half)));
-#pragma unroll
-        for (int k = 0; k < N; ++k) {
-          q_values[item][k] = source[lane + 64u * k];
-          q_entry[item][k] = entries[pair_of_lane[k]];
-        }
+        [&]<int... K>(std::integer_sequence<int, K...>) {
+          ((q_values[item][K] = load_f32_uncounted<256 * K>(source, 4u * lane)), ...);
+          ((q_entry_raw[item][K] =
+                load_f32x2_uncounted(entries, 8u * pair_of_lane[K])), ...);
+        }(std::make_integer_sequence<int, N>{});
         member += member_step;
         row += row_step;
         if (member >= group) {
@@ -612,16 +677,14 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     }
     uint32_t workgroup_first, workgroup_last, unused;
     wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y, 0u,
-                    workgroup_first, unused);
+                    workgroup_first, unused, kTailWork);
     wave_tile_range(context_tiles, 64u, args.split_tokens, split, gridDim.y,
-                    kSplitWaves - 1u, unused, workgroup_last);
+                    kSplitWaves - 1u, unused, workgroup_last, kTailWork);
     reaches_batch = workgroup_first < workgroup_last &&
                     workgroup_last * 64u > first_cache_position;
-    // the wave's first tile sets out first: the work below hides behind it
-    if (!SCRATCH_IN_STAGE && tile_first < tile_last) {
-      stage_keys(tile_first);
-      stage_values(tile_first);
-    }
+    // the wave's first tiles set out first: the work below hides behind them
+    uint32_t halves_in_flight = 0u;
+    if (!SCRATCH_IN_STAGE) halves_in_flight = stage_first_tiles();
     // batch rows wave, wave + 8, ... are this wave's to encode (one for the
     // usual batches; the rest, if any, are fetched when their turn comes)
     const bool writes_pages = reaches_batch && workgroup_last == context_tiles;
@@ -637,7 +700,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
         k_entry[k] = args.rope_table[row * half + pair_of_lane[k]];
       }
     };
-    if (reaches_batch && wave < args.rows) fetch_record(wave);
+    if (reaches_batch && wave < args.rows) {
+      fetch_record(wave);
+      halves_in_flight = 0u;   // these loads came after the tiles: wait for all
+    }
     // where element lane + 64 k of a row goes inside the row's operand bytes:
     // k-step 2 (d / 128) + (d % 32) / 16, lane quad (d % 128) / 32, byte slot
     // (even elements of each half of 8 first, then the odd ones)
@@ -662,6 +728,23 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     // in 48 slots): it alone sits behind a branch, which leaves it out then.
     const bool last_item_live =
         wave + kSplitWaves * (ROWS_PER_WAVE - 1) < matrix_rows;
+    // loads complete in issue order: the rows, their (cos, sin) and the weights
+    // are here once nothing but the tiles issued after them is in flight
+    vmem_wait_units<KS_LOADS>(halves_in_flight);
+    float2 q_entry[ROWS_PER_WAVE][N];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+      tie(weights[0][k]);
+      tie(weights[1][k]);
+    }
+#pragma unroll
+    for (int item = 0; item < ROWS_PER_WAVE; ++item)
+#pragma unroll
+      for (int k = 0; k < N; ++k) {
+        tie(q_values[item][k]);
+        tie(q_entry_raw[item][k]);
+        q_entry[item][k] = make_float2(q_entry_raw[item][k][0], q_entry_raw[item][k][1]);
+      }
     const auto quantise_rows = [&](auto rotate) {
 #pragma unroll
       for (int item = 0; item < ROWS_PER_WAVE; ++item) {
@@ -798,10 +881,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       // every lane is done with the scratch before the tile lands on it
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       __builtin_amdgcn_wave_barrier();
-      stage_keys(tile_first);
-      stage_values(tile_first);
+      stage_first_tiles();
     }
-    vmem_wait<0>();
+    // a workgroup that fetched batch records or wrote them to their pages has
+    // loads and stores of other kinds in flight: the tile loop counts tiles only
+    if (reaches_batch) vmem_wait<0>();
   } else if (args.query_operands) {
     // prepared by the rotary kernel: the planes go straight to LDS, one KiB
     // per wave and load, the scales with them
@@ -829,13 +913,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
   }
   // the wave's first tile sets out before the query work below, which its
   // flight time covers
-  if (!FUSED && tile_first < tile_last) {
-    stage_keys(tile_first);
-    stage_values(tile_first);
-  }
+  uint32_t halves_after_operands = 0u;
+  if (!FUSED) halves_after_operands = stage_first_tiles();
   if (FUSED) {
   } else if (args.query_operands) {
-    vmem_wait<0>();
+    // the operands were asked for before the tiles
+    vmem_wait_units<KS_LOADS>(halves_after_operands);
   } else if (wave < static_cast<uint32_t>(RT * KSTEPS)) {
     // wave u builds k-step u % KSTEPS of row tile u / KSTEPS (the row's scale
     // needs the whole row, so every such wave reads all of it)
@@ -919,13 +1002,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
   // per-lane LDS addresses of the staged tile
   // K: lane (token = col, quad) takes 16 bytes of each sub-tile's K row
-  const uint32_t key_address = stage_k_lds + col * ROW + 16u * quad;
+  // (they start in staging area 0 and change areas with every tile)
+  uint32_t key_address = stage_k_lds + col * ROW + 16u * quad;
   // scales of tokens 16*st + 4*quad + i (i = 0..3)
-  const uint32_t scale_address = stage_s_lds + 8u * quad;
-  const uint32_t value_scale_address = stage_vs_lds + 8u * quad;
+  uint32_t scale_address = stage_s_lds + 8u * quad;
+  // (the V scales lie CODES + 256 bytes past the K scales)
   // V: lane (col, quad) supplies LDS row 16*quad + col, i.e. token
   // 16*(col/4) + 4*quad + col%4 of the tile
-  const uint32_t value_address = stage_v_lds + (16u * quad + col) * ROW;
+  uint32_t value_address = stage_v_lds + (16u * quad + col) * ROW;
+  uint32_t area = 0u;   // of the tile at hand: 0 or STAGE
 
   // ---- running state ---------------------------------------------------------
   float running_max[RT];   // in t units
@@ -947,9 +1032,14 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     const uint32_t tile_begin = tile * 64u;
     const bool needs_mask = tile_begin + 64u > first_context_tokens;
     const bool has_next = tile + 1u < tile_last;
+    // this tile's staging area, and whether the tile DEPTH ahead refills it
+    const bool refills = tile + DEPTH < tile_last;
+    const uint32_t ahead_units = DEPTH == 2 && has_next ? 2u : 0u;
+    uint8_t* const stage_k = stage_base + area;
 
     // ---- K codes and scales out of LDS ----------------------------------------
-    vmem_wait<V_LOADS>();
+    // in flight, oldest first: this tile's K, its V, the next tile's K and V
+    vmem_wait_units<KS_LOADS>(1u + ahead_units);
     if constexpr (FUSED) {
       // the batch's own tokens inside this tile, [batch_first, batch_last):
       // their fresh records go over whatever the pages held, once the whole
@@ -998,8 +1088,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
     }(std::make_integer_sequence<int, 4>{});
     lds_wait(key_raw);
     lds_wait(scale_raw);
-    // that half of the staging area is free: fetch the next tile's K
-    if (has_next) stage_keys(tile + 1u);
+    // that half of the staging area is free: fetch the K of the tile that
+    // uses it next
+    if (refills) stage_keys(tile + DEPTH, area);
 
     // K nibbles widened to int8 * 16 (sub-tile st, k-step h), scales of tokens
     // 16*st + 4*quad + i
@@ -1071,8 +1162,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       }
       if (needs_mask) {
         // only the tiles that reach past the first row's context get here
-        const uint32_t first_token = tile_begin + 4u * quad;
-        const uint32_t limit = exchange_limit[16 * rt + col];
+        const uint32_t lane_now = fresh_lane_index();
+        const uint32_t first_token = tile_begin + 4u * (lane_now >> 4);
+        const uint32_t limit = exchange_limit[16 * rt + (lane_now & 15u)];
 #pragma unroll
         for (int st = 0; st < 4; ++st)
 #pragma unroll
@@ -1082,14 +1174,12 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
 
       if (rt == 0) {
         // ---- V scales out of LDS ----------------------------------------------
-        // in flight, oldest first: this tile's V, the next tile's K
-        if (has_next)
-          vmem_wait<KS_LOADS>();
-        else
-          vmem_wait<0>();
+        // in flight, oldest first: this tile's V, the next tile's K and V,
+        // the K just asked for
+        vmem_wait_units<KS_LOADS>(ahead_units + (refills ? 1u : 0u));
         u32x2 value_scale_raw[4];
         [&]<int... I>(std::integer_sequence<int, I...>) {
-          ((value_scale_raw[I] = lds_read8<I * 32>(value_scale_address)), ...);
+          ((value_scale_raw[I] = lds_read8<I * 32 + CODES + 256>(scale_address)), ...);
         }(std::make_integer_sequence<int, 4>{});
         lds_wait(value_scale_raw);
 #pragma unroll
@@ -1103,8 +1193,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
             if (needs_mask) {
               // records no row can see may be uninitialised: keep their scale
               // (any bit pattern) away from the matrix core
-              if (tile_begin + 32u * u + 4u * quad + c >= last_context) lo = 0u;
-              if (tile_begin + 32u * u + 16u + 4u * quad + c >= last_context)
+              const uint32_t quad_now = fresh_lane_index() >> 4;
+              if (tile_begin + 32u * u + 4u * quad_now + c >= last_context) lo = 0u;
+              if (tile_begin + 32u * u + 16u + 4u * quad_now + c >= last_context)
                 hi = 0u;
             }
             v_scale[u][c] = __builtin_bit_cast(f16x2, lo | (hi << 16));
@@ -1162,7 +1253,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void q4h_attention_split_kernel(
       ((transposed[I] = lds_read8_transposed4<I * 8>(value_address)), ...);
     }(std::make_integer_sequence<int, DT>{});
     lds_wait(transposed);
-    if (has_next) stage_values(tile + 1u);
+    if (refills) stage_values(tile + DEPTH, area);
+    if constexpr (DEPTH == 2) {
+      // on to the other staging area
+      const uint32_t step = area ? static_cast<uint32_t>(-STAGE) : STAGE;
+      key_address += step;
+      scale_address += step;
+      value_address += step;
+      area = STAGE - area;
+    }
 
     // ---- O^T += V^T . P^T -------------------------------------------------------
 #pragma unroll
@@ -1871,7 +1970,8 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
     uint32_t rotary_dim, float epsilon, float theta, bool bf16_activations,
     const uint32_t* device_positions, const float* partials,
     uint32_t partial_count, uint32_t rows, uint8_t* operands,
-    float* operand_scales) {
+    float* operand_scales, const void* const* q8_page_table = nullptr,
+    size_t q8_page_offset = 0u) {
   __shared__ float shared[256];
   __shared__ float rotated[256];
   if (device_positions) {
@@ -1971,6 +2071,20 @@ __global__ __launch_bounds__(64) void qkv_rope_q4h_kernel(
   float* k = key + (static_cast<size_t>(row) * kv_heads + head) * head_dim;
   head_norm_rope(k, k_weight, head_dim, rotary_dim, rotary_position, epsilon,
                  theta, bf16_activations, shared, rotated, lane);
+  if (q8_page_table) {
+    // the proposer's Q8 cache: the rotated key and the value of this (row, kv
+    // head) as Q8 records, what a separate store launch would write
+    const uint32_t position = first_cache_position + row;
+    uint8_t* layer_base = static_cast<uint8_t*>(const_cast<void*>(
+                              q8_page_table[position / page_tokens])) + q8_page_offset;
+    __syncthreads();   // `rotated` is complete (one wave)
+    q8_encode_record(rotated, head_dim, layer_base, 0u, position % page_tokens, head,
+                     kv_heads, page_tokens, lane);
+    q8_encode_record(value + (static_cast<size_t>(row) * kv_heads + head) * head_dim,
+                     head_dim, layer_base, 1u, position % page_tokens, head, kv_heads,
+                     page_tokens, lane);
+    return;
+  }
   if (!page_table) return;  // rotary only; the caller stores K/V itself
   const uint32_t position = first_cache_position + row;
   uint8_t* page = static_cast<uint8_t*>(
@@ -2280,6 +2394,37 @@ extern "C" int32_t qllm_qkv_rope_batch_deferred(
   return launched("deferred QKV rope batch");
 }
 
+// Rotary (and per-head norm) of a batch's queries and keys plus the K/V store
+// into the proposer's Q8 cache, in one launch; device_positions (optional):
+// word 0 the first cache position, word 1 the first rotary position.
+extern "C" int32_t qllm_qkv_rope_store_q8_batch(
+    float* query, uint32_t query_stride, float* key, const float* value,
+    const float* q_norm_weight, const float* k_norm_weight,
+    const void* const* page_table, size_t page_offset_bytes, uint32_t page_tokens,
+    uint32_t first_cache_position, uint32_t first_rotary_position,
+    const uint32_t* device_positions, uint32_t rows, uint32_t query_heads,
+    uint32_t kv_heads, uint32_t head_dim, uint32_t rotary_dim, float epsilon,
+    float rope_theta, int32_t bf16_activations, void* stream) {
+  if (!query || !key || !value || !page_table || !page_tokens || !rows ||
+      !query_heads || !kv_heads || query_heads < kv_heads ||
+      query_heads % kv_heads || !head_dim || head_dim > 256u || head_dim % 2u ||
+      query_stride < head_dim || !rotary_dim || rotary_dim > head_dim ||
+      rotary_dim % 2u || !(epsilon > 0.0f) || !(rope_theta > 0.0f) ||
+      page_offset_bytes % 16u ||
+      (!device_positions &&
+       (first_cache_position > 0xffffffffu - (rows - 1u) ||
+        first_rotary_position > 0xffffffffu - (rows - 1u))))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid QKV rope + Q8 store batch");
+  qkv_rope_q4h_kernel<<<dim3(query_heads + kv_heads, rope_grid_rows(rows)), 64, 0,
+                        as_stream(stream)>>>(
+      query, query_stride, key, value, q_norm_weight, k_norm_weight, nullptr, 0u,
+      page_tokens, first_cache_position, first_rotary_position, query_heads,
+      kv_heads, head_dim, rotary_dim, epsilon, rope_theta, bf16_activations != 0,
+      device_positions, nullptr, 0u, rows, nullptr, nullptr, page_table,
+      page_offset_bytes);
+  return launched("QKV rope + Q8 store batch");
+}
+
 extern "C" int32_t qllm_quantize_gqa_queries_q8(
     const float* query, uint32_t query_stride, int8_t* q8, float* query_scales,
     uint32_t rows, uint32_t query_heads, uint32_t head_dim, void* stream) {
@@ -2479,6 +2624,7 @@ int32_t launch_q4h_attention(const qllm_q4h_attention_launch* launch,
   int32_t status;
   if (rope) {
     if (!rope->key || !rope->value || !rope->rope_table || !rope->rotary_dim ||
+        launch->rows > 16u ||
         rope->rotary_dim > launch->head_dim || rope->rotary_dim % 2u ||
         !(rope->epsilon > 0.0f) ||
         (!launch->device_positions &&

@@ -113,6 +113,25 @@ __device__ __forceinline__ float block_max(float value, float* scratch) {
   return total;
 }
 
+// What a captured proposer pass does with its arg-max token before the next
+// pass starts (qllm_rollout_advance): the token becomes the next pass's input
+// and the next entry of the draft list, the positions move on by `rows`.
+struct RolloutAdvance {
+  uint32_t* next_token;
+  uint32_t* draft_tokens;
+  uint32_t capacity;
+  uint32_t rows;
+  uint32_t* positions;
+};
+
+// Stage 2 of an arg-max whose stage-1 partials lie in [batch][blocks] arrays
+// (select.hip); with `advance` (batch 1) the same launch also advances the
+// rollout with the winner.
+int32_t launch_argmax_final(const float* partial_values,
+                            const uint32_t* partial_indices, uint32_t blocks,
+                            uint32_t batch, uint32_t* output,
+                            const RolloutAdvance* advance, hipStream_t stream);
+
 // splitmix64 counter generator shared with the host-side restatement.
 __host__ __device__ inline uint64_t mix64(uint64_t seed, uint64_t index) {
   uint64_t value = seed ^ (index * 0x9e3779b97f4a7c15ull + 0x632be59bd9b4e019ull);

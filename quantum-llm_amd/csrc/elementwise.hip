@@ -191,6 +191,34 @@ __global__ __launch_bounds__(256) void rms_norm_batch_kernel(
 // partials[1] + ... (added in that order; partial p of the row lies
 // `partial_stride` floats after partial p - 1) and that sum is also written
 // back to `sum_out`.
+// Columns 4 * vector .. + 3 of a row-major FP4 row as F32: the values
+// fp4_embedding_batch_kernel gives (twice(code) * 0.5 * scale, sign applied
+// last).
+__device__ __forceinline__ float4 fp4_row_vector(const uint8_t* codes_row,
+                                                 const uint8_t* scales_row,
+                                                 uint32_t scheme, uint32_t vector) {
+  const uint32_t column = vector * 4u;
+  const uint32_t codes =
+      *reinterpret_cast<const uint16_t*>(codes_row + column / 2u);
+  const float scale =
+      scheme == QLLM_SCALE_F16_BLOCK16
+          ? f16_bits_to_f32(reinterpret_cast<const uint16_t*>(scales_row)[column / 16u])
+          : ue8m0_to_f32(scales_row[column / 32u]);
+  float values[4];
+#pragma unroll
+  for (uint32_t i = 0; i < 4u; ++i) {
+    const uint32_t code = (codes >> (4u * i)) & 0x0fu;
+    const uint32_t index = code & 7u;
+    const float twice = index <= 4u ? static_cast<float>(index)
+                        : index == 5u ? 6.0f
+                        : index == 6u ? 8.0f
+                                      : 12.0f;
+    const float value = twice * 0.5f * scale;
+    values[i] = (code & 8u) ? -value : value;
+  }
+  return make_float4(values[0], values[1], values[2], values[3]);
+}
+
 // four values -> four Q8 codes: clamp(rn(value / scale), -127, 127)
 // (transformer_kernels.cu:912-946), packed low byte first
 __device__ __forceinline__ uint32_t q8_pack4(float4 value, float scale) {
@@ -240,7 +268,10 @@ __device__ __forceinline__ void rms_norm_row_wide(
     float epsilon, bool zero_centered, float* scratch,
     const float* partial_row = nullptr, uint32_t partial_count = 0u,
     size_t partial_stride = 0u, float* sum_out = nullptr,
-    int8_t* out_q8 = nullptr, float* out_q8_scale = nullptr) {
+    int8_t* out_q8 = nullptr, float* out_q8_scale = nullptr,
+    const uint8_t* fp4_codes_row = nullptr, const uint8_t* fp4_scales_row = nullptr,
+    uint32_t fp4_scheme = 0u) {
+  // with fp4_codes_row the row is an FP4 embedding row, decoded on the way in
   const float4* x = reinterpret_cast<const float4*>(input_row);
   const uint32_t vectors = elements / 4u;
   // the row and its weights are fetched together, before the reduction
@@ -250,7 +281,11 @@ __device__ __forceinline__ void rms_norm_row_wide(
 #pragma unroll
   for (int slot = 0; slot < 4; ++slot) {
     const uint32_t index = slot * blockDim.x + threadIdx.x;
-    values[slot] = index < vectors ? x[index] : make_float4(0.f, 0.f, 0.f, 0.f);
+    values[slot] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (index < vectors)
+      values[slot] = fp4_codes_row ? fp4_row_vector(fp4_codes_row, fp4_scales_row,
+                                                    fp4_scheme, index)
+                                   : x[index];
     factors[slot] = make_float4(1.f, 1.f, 1.f, 1.f);
     if (weight && index < vectors)
       factors[slot] = reinterpret_cast<const float4*>(weight)[index];
@@ -396,6 +431,39 @@ __global__ __launch_bounds__(1024) void rms_norm_concat_kernel(
       second_half ? second_weight : first_weight, nullptr,
       output_bf16 + row * 2u * elements + (second_half ? elements : 0u),
       elements, elements, epsilon, zero_centered, scratch);
+}
+
+// The proposer's input: row r of the output is [RMSNorm(embedding of
+// tokens[r]) | RMSNorm(second[r])] in bf16 - the embedding lookup
+// (fp4_embedding_batch_kernel) folded into the first half's norm.  A token
+// outside the vocabulary gives a row of zeros, as the lookup does.
+__global__ __launch_bounds__(1024) void rms_norm_concat_embedding_kernel(
+    const uint8_t* codes, const uint8_t* scales, uint32_t scheme,
+    uint32_t padded_columns, uint32_t vocabulary, const uint32_t* tokens,
+    const float* first_weight, const float* second, const float* second_weight,
+    uint16_t* output_bf16, uint32_t elements, float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  uint16_t* out = output_bf16 + row * 2u * elements;
+  if (blockIdx.y != 0u) {
+    rms_norm_row_wide(second + row * elements, second_weight, nullptr,
+                      out + elements, elements, elements, epsilon, zero_centered,
+                      scratch);
+    return;
+  }
+  const size_t token = tokens[row];
+  if (token >= vocabulary) {
+    for (uint32_t index = threadIdx.x; index < elements; index += blockDim.x)
+      out[index] = 0u;
+    return;
+  }
+  const size_t scale_row_bytes = scheme == QLLM_SCALE_F16_BLOCK16
+                                     ? padded_columns / 8u
+                                     : padded_columns / 32u;
+  rms_norm_row_wide(nullptr, first_weight, nullptr, out, elements, elements, epsilon,
+                    zero_centered, scratch, nullptr, 0u, 0u, nullptr, nullptr, nullptr,
+                    codes + token * (padded_columns / 2u),
+                    scales + token * scale_row_bytes, scheme);
 }
 
 // transformer_kernels.cu:2522-2528
@@ -615,6 +683,32 @@ extern "C" int32_t qllm_rms_norm_concat_batch(
       static_cast<uint16_t*>(output_bf16), elements, epsilon,
       zero_centered != 0);
   return launched("RMSNorm concat batch");
+}
+
+extern "C" int32_t qllm_rms_norm_concat_embedding_batch(
+    const qllm_fp4_matrix* embedding, const uint32_t* tokens,
+    const float* first_weight, const float* second, const float* second_weight,
+    void* output_bf16, uint32_t rows, float epsilon, int32_t zero_centered,
+    void* stream) {
+  if (!embedding || !embedding->weights || !embedding->scales || !embedding->rows ||
+      embedding->layout != QLLM_LAYOUT_ROW_MAJOR || embedding->scale_scheme > 1u ||
+      embedding->padded_columns < embedding->columns ||
+      embedding->padded_columns % 32u || !tokens || !second || !output_bf16 ||
+      !rows || !embedding->columns || embedding->columns % 4u ||
+      embedding->columns > 16384u || !(epsilon > 0.0f) ||
+      ((reinterpret_cast<uintptr_t>(first_weight) |
+        reinterpret_cast<uintptr_t>(second) |
+        reinterpret_cast<uintptr_t>(second_weight)) & 15u) ||
+      (reinterpret_cast<uintptr_t>(embedding->weights) & 1u) ||
+      (reinterpret_cast<uintptr_t>(embedding->scales) & 1u) ||
+      (reinterpret_cast<uintptr_t>(output_bf16) & 7u))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid RMSNorm concat of an embedding batch");
+  rms_norm_concat_embedding_kernel<<<dim3(rows, 2u), 1024, 0, as_stream(stream)>>>(
+      embedding->weights, static_cast<const uint8_t*>(embedding->scales),
+      embedding->scale_scheme, embedding->padded_columns, embedding->rows, tokens,
+      first_weight, second, second_weight, static_cast<uint16_t*>(output_bf16),
+      embedding->columns, epsilon, zero_centered != 0);
+  return launched("RMSNorm concat of an embedding batch");
 }
 
 extern "C" int32_t qllm_add_in_place(float* destination, const float* source,

@@ -119,6 +119,13 @@ struct GemmArgs {
   uint32_t balance_splits;
   float* balance_partials;
   uint32_t* balance_counters;
+  // Stage 1 of the arg-max over the output rows (a head's logits), taken from
+  // the epilogue: with argmax_values (TILES == 1, F32 output, one workgroup
+  // per tile) the tile's best (value, output row) of every batch row goes to
+  // argmax_values / argmax_indices [batch][tiles] - larger value first, equal
+  // values by lower row, NaN never - and a one-block launch picks the winner.
+  float* argmax_values;
+  uint32_t* argmax_indices;
 };
 
 // Epilogue store of one value.
@@ -549,12 +556,47 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
       }
     }
   }
-  if (!item_valid) return;
   if constexpr (Q8) {
-    const float row_scale = args.activation_scales[item_batch];
-    total *= row_scale;
-    up *= row_scale;
+    if (item_valid) {
+      const float row_scale = args.activation_scales[item_batch];
+      total *= row_scale;
+      up *= row_scale;
+    }
   }
+  if constexpr (TILES == 1) {
+    if (args.argmax_values != nullptr) {
+      // the tile's best logit per batch row, on the values that are stored
+      const float value = total + residual_value;
+      __syncthreads();   // every wave has read its sums out of `reduce`
+      float* const best_values = &reduce[0][0][0][0][0];
+      uint32_t* const best_rows = reinterpret_cast<uint32_t*>(best_values) + kItems;
+      if (threadIdx.x < kItems) {
+        best_values[threadIdx.x] = item_valid ? value : -INFINITY;
+        best_rows[threadIdx.x] = item_valid ? item_row : 0xffffffffu;
+      }
+      __syncthreads();
+      if (threadIdx.x < BATCH) {
+        const uint32_t m = threadIdx.x;
+        const uint32_t group = m / (COMPACT ? 3u : 4u);
+        const uint32_t reg = m % (COMPACT ? 3u : 4u);
+        float best = -INFINITY;
+        uint32_t best_row = 0xffffffffu;
+        for (uint32_t half = 0; half < 2u; ++half)
+          for (uint32_t k = 0; k < 16u; ++k) {
+            const uint32_t slot = (half * REGS + reg) * 32u + group * 16u + k;
+            const float candidate = best_values[slot];
+            const uint32_t candidate_row = best_rows[slot];
+            if (candidate > best || (candidate == best && candidate_row < best_row)) {
+              best = candidate;
+              best_row = candidate_row;
+            }
+          }
+        args.argmax_values[m * gridDim.x + blockIdx.x] = best;
+        args.argmax_indices[m * gridDim.x + blockIdx.x] = best_row;
+      }
+    }
+  }
+  if (!item_valid) return;
   if (TILES == 2) {
     if (args.output_kind == QLLM_OUT_F32) {
       // F32 activations (silu_product_kernel without bf16 rounding,
@@ -1005,6 +1047,54 @@ extern "C" int32_t qllm_fp4_gemm_bf16(const qllm_fp4_matrix* matrix,
             input, nullptr, output, residual, matrix->rows,
             matrix->padded_columns, batch, output_kind);
   return launched("FP4 BF16 GEMV");
+}
+
+extern "C" size_t qllm_fp4_head_workspace_bytes(const qllm_fp4_matrix* matrix,
+                                                uint32_t batch) {
+  if (!matrix_ok(matrix) || !batch) return 0;
+  const size_t tiles =
+      (matrix->rows + matrix_tile_rows(matrix) - 1u) / matrix_tile_rows(matrix);
+  return tiles * batch * (sizeof(float) + sizeof(uint32_t));
+}
+
+extern "C" int32_t qllm_fp4_head_argmax(const qllm_fp4_matrix* matrix,
+                                        const void* input, size_t input_bytes,
+                                        float* logits, uint32_t batch,
+                                        uint32_t* tokens, void* workspace,
+                                        size_t workspace_bytes,
+                                        const qllm_rollout_step* advance,
+                                        void* stream) {
+  if (!matrix_ok(matrix) || !input || !logits || !batch || batch > 8u || !tokens ||
+      !workspace || matrix->padded_columns % kChunk != 0u ||
+      workspace_bytes < qllm_fp4_head_workspace_bytes(matrix, batch) ||
+      input_bytes < static_cast<size_t>(batch) * matrix->padded_columns * 2u ||
+      (advance && (batch != 1u || !advance->next_token || !advance->draft_tokens ||
+                   !advance->rows || !advance->device_positions)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid FP4 head with arg-max");
+  GemmArgs args{};
+  args.tile[0] = {matrix->weights, static_cast<const uint8_t*>(matrix->scales)};
+  args.tile[1] = args.tile[0];
+  args.activations = static_cast<const uint16_t*>(input);
+  args.output = logits;
+  args.rows = matrix->rows;
+  args.padded_columns = matrix->padded_columns;
+  args.output_kind = QLLM_OUT_F32;
+  args.tile_rows = matrix_tile_rows(matrix);
+  const uint32_t tiles = (matrix->rows + args.tile_rows - 1u) / args.tile_rows;
+  args.argmax_values = static_cast<float*>(workspace);
+  args.argmax_indices =
+      reinterpret_cast<uint32_t*>(args.argmax_values + static_cast<size_t>(tiles) * batch);
+  if (const int32_t status =
+          launch_mfma(args, static_cast<int>(matrix->scale_scheme),
+                      matrix->layout == QLLM_LAYOUT_TILED, batch, false,
+                      as_stream(stream)))
+    return status;
+  RolloutAdvance step{};
+  if (advance)
+    step = {advance->next_token, advance->draft_tokens, advance->capacity,
+            advance->rows, advance->device_positions};
+  return launch_argmax_final(args.argmax_values, args.argmax_indices, tiles, batch,
+                             tokens, advance ? &step : nullptr, as_stream(stream));
 }
 
 extern "C" int32_t qllm_fp4_gemm_bf16_partial(const qllm_fp4_matrix* matrix,

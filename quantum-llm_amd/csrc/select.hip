@@ -103,9 +103,11 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(
   }
 }
 
+// `advance.positions` non-null (one row): thread 0 also does what
+// rollout_advance_kernel does with the winner.
 __global__ __launch_bounds__(256) void argmax_final_kernel(
     const float* partial_values, const uint32_t* partial_indices,
-    uint32_t blocks_per_row, uint32_t* output) {
+    uint32_t blocks_per_row, uint32_t* output, RolloutAdvance advance) {
   __shared__ float shared_values[4];
   __shared__ uint32_t shared_indices[4];
   const uint32_t request = blockIdx.x;
@@ -120,7 +122,17 @@ __global__ __launch_bounds__(256) void argmax_final_kernel(
     }
   }
   block_best(best, index, shared_values, shared_indices);
-  if (threadIdx.x == 0u) output[request] = index;
+  if (threadIdx.x != 0u) return;
+  output[request] = index;
+  if (advance.positions && request == 0u) {
+    const uint32_t slot = advance.positions[3];
+    advance.next_token[0] = index;
+    if (slot < advance.capacity) advance.draft_tokens[slot] = index;
+    advance.positions[0] += advance.rows;
+    advance.positions[1] += advance.rows;
+    advance.positions[2] += advance.rows;
+    advance.positions[3] = slot + 1u;
+  }
 }
 
 __global__ __launch_bounds__(64) void rollout_advance_kernel(
@@ -406,6 +418,17 @@ __global__ __launch_bounds__(64) void mark_presence_kernel(
 }
 
 }  // namespace
+
+int32_t launch_argmax_final(const float* partial_values,
+                            const uint32_t* partial_indices, uint32_t blocks,
+                            uint32_t batch, uint32_t* output,
+                            const RolloutAdvance* advance, hipStream_t stream) {
+  argmax_final_kernel<<<batch, 256, 0, stream>>>(
+      partial_values, partial_indices, blocks, output,
+      advance ? *advance : RolloutAdvance{});
+  return launched("argmax of the head's tile maxima");
+}
+
 }  // namespace qllm
 
 using namespace qllm;
@@ -429,7 +452,7 @@ extern "C" int32_t qllm_argmax_batch(const float* values, uint32_t count,
   argmax_partial_kernel<<<dim3(blocks, batch), 256, 0, as_stream(stream)>>>(
       values, count, partial_values, partial_indices, blocks);
   argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
-      partial_values, partial_indices, blocks, output);
+      partial_values, partial_indices, blocks, output, RolloutAdvance{});
   return launched("argmax batch");
 }
 
@@ -498,7 +521,7 @@ extern "C" int32_t qllm_argmax_batch_static(const float* values, uint32_t count,
   argmax_partial_kernel<<<dim3(blocks, batch), 256, 0, as_stream(stream)>>>(
       values, count, partial_values, partial_indices, blocks);
   argmax_final_kernel<<<batch, 256, 0, as_stream(stream)>>>(
-      partial_values, partial_indices, blocks, output);
+      partial_values, partial_indices, blocks, output, RolloutAdvance{});
   return launched("argmax batch static");
 }
 

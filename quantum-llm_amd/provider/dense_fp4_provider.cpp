@@ -399,8 +399,12 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
         device_alloc(std::size_t{max_rows_} * g_.rotary_dim * 4U));
   }
 
+  // the heads' tile maxima: 32 vocabulary rows per tile
+  const std::size_t head_maxima_bytes =
+      (std::size_t{g_.vocabulary} + 31U) / 32U * max_rows_ * 8U;
   select_workspace_bytes_ = std::max(
-      qllm_argmax_workspace_bytes(g_.vocabulary, max_rows_),
+      std::max(head_maxima_bytes,
+               qllm_argmax_workspace_bytes(g_.vocabulary, max_rows_)),
       std::max(qllm_topk_workspace_bytes(g_.vocabulary, kMaximumGpuSamplingTopK),
                qllm_topk_batch_workspace_bytes(g_.vocabulary,
                                                kMaximumGpuSamplingTopK, max_rows_)));
@@ -1707,12 +1711,33 @@ void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
         normalized_, g_.hidden, rows, g_.hidden, g_.norm_epsilon,
         g_.zero_centered_norm, stream_));
   }
-  status_check(qllm_fp4_gemm_bf16(&head_.descriptor, normalized_,
-                                  std::size_t{rows} * g_.hidden * 2U, logits_,
+  enqueue_head_projection(head_.descriptor, logits_, rows, argmax_tokens_, nullptr);
+}
+
+// logits = head . normalized_ and their arg-max tokens: the projection's
+// epilogue leaves the tiles' maxima for a one-block launch to finish (with
+// `advance`, which also hands the winner to the next proposer pass); matrices
+// the matrix-core kernel does not take go through the plain arg-max.
+void Mi355DenseFp4Provider::enqueue_head_projection(
+    const qllm_fp4_matrix& head, float* logits, std::uint32_t rows,
+    std::uint32_t* tokens, const qllm_rollout_step* advance) {
+  const std::size_t input_bytes = std::size_t{rows} * g_.hidden * 2U;
+  if (head.padded_columns % 64U == 0U &&
+      qllm_fp4_head_workspace_bytes(&head, rows) <= select_workspace_bytes_) {
+    status_check(qllm_fp4_head_argmax(&head, normalized_, input_bytes, logits, rows,
+                                      tokens, select_workspace_,
+                                      select_workspace_bytes_, advance, stream_));
+    return;
+  }
+  status_check(qllm_fp4_gemm_bf16(&head, normalized_, input_bytes, logits,
                                   QLLM_OUT_F32, nullptr, rows, stream_));
-  status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
-                                 select_workspace_, select_workspace_bytes_,
-                                 stream_));
+  status_check(qllm_argmax_batch(logits, head.rows, rows, tokens, select_workspace_,
+                                 select_workspace_bytes_, stream_));
+  if (advance)
+    status_check(qllm_rollout_advance(tokens, advance->next_token,
+                                      advance->draft_tokens, advance->capacity,
+                                      advance->rows, advance->device_positions,
+                                      stream_));
 }
 
 void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
@@ -1745,20 +1770,18 @@ void Mi355DenseFp4Provider::enqueue_target(const std::uint32_t* device_tokens,
 
 // The proposer's pass over a prompt chunk: row r pairs tokens[r] (the token
 // after prompt position `position` + r) with the target's hidden state of that
-// position, which prefill() left in prefill_hidden_.  Same operations as
-// enqueue_mtp without the draft head, on the tall-batch GEMM and the batched
-// Q8 attention; writes the proposer's cache records position .. position +
+// position, which prefill() left in prefill_hidden_.  The operations of
+// enqueue_mtp up to the key / value store, on the tall-batch GEMM and the
+// Q8 cache store; writes the proposer's cache records position .. position +
 // rows - 1 and reuses the prefill buffers (prefill_hidden_ becomes the
 // proposer's residual stream).
 void Mi355DenseFp4Provider::enqueue_mtp_prefill(
-    std::span<const std::uint32_t> tokens, std::uint32_t position,
-    std::uint32_t attention_batch) {
+    std::span<const std::uint32_t> tokens, std::uint32_t position) {
   void* const stream = stream_;
   const auto hip_stream = static_cast<hipStream_t>(stream_);
   const auto rows = static_cast<std::uint32_t>(tokens.size());
   const auto& layer = mtp_.layer;
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
-  const std::size_t attention_width = std::size_t{g_.query_heads} * g_.head_dim;
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   float* const embedding = prefill_embedding_;            // f32 [rows, hidden]
   std::uint16_t* const fusion_input = prefill_activation_;  // bf16 [rows, 2 hidden]
@@ -1796,58 +1819,33 @@ void Mi355DenseFp4Provider::enqueue_mtp_prefill(
   status_check(qllm_store_kv_paged_q8_batch(
       prefill_key_, prefill_value_, pages, mtp_page_offset_, g_.kv_page_tokens,
       position, rows, g_.kv_heads, g_.head_dim, stream));
-  qllm_q8_attention_launch launch{};
-  launch.query = prefill_query_;
-  launch.device_pages = pages;
-  launch.output = prefill_attention_;
-  launch.partial_maxima = prefill_partial_maxima_;
-  launch.partial_sums = prefill_partial_sums_;
-  launch.partial_outputs = prefill_partial_outputs_;
-  launch.page_offset_bytes = mtp_page_offset_;
-  launch.first_context_tokens = position + 1U;
-  launch.rows = rows;
-  launch.page_tokens = g_.kv_page_tokens;
-  launch.query_heads = g_.query_heads;
-  launch.kv_heads = g_.kv_heads;
-  launch.head_dim = g_.head_dim;
-  launch.split_tokens = 0U;
-  launch.maximum_splits = prefill_splits_for(rows, attention_batch);
-  launch.query_stride = query_stride;
-  launch.output_gated = g_.output_gated;
-  launch.output_kind = QLLM_OUT_BF16;
-  launch.stream = stream;
-  status_check(qllm_attention_paged_q8_batched(&launch, attention_batch));
-  status_check(qllm_fp4_gemm_bf16_tall(
-      &layer.output.descriptor, prefill_attention_,
-      std::size_t{rows} * attention_width * 2U, prefill_hidden_, QLLM_OUT_F32,
-      prefill_hidden_, rows, stream));
-  status_check(qllm_rms_norm_batch(prefill_hidden_, layer.post_attention_norm,
-                                   nullptr, prefill_normalized_, g_.hidden, rows,
-                                   g_.hidden, g_.norm_epsilon,
-                                   g_.zero_centered_norm, stream));
-  status_check(qllm_fp4_swiglu_bf16_tall(
-      &layer.gate.descriptor, &layer.up.descriptor, prefill_normalized_,
-      hidden_bytes, prefill_activation_, rows, stream));
-  status_check(qllm_fp4_gemm_bf16_tall(
-      &layer.down.descriptor, prefill_activation_,
-      std::size_t{rows} * g_.intermediate * 2U, prefill_hidden_, QLLM_OUT_F32,
-      prefill_hidden_, rows, stream));
+  // The pass ends with the cache records: the proposer has one layer and a
+  // prompt pass asks for no draft, so nothing reads what its attention and
+  // MLP would compute.
 }
 
 // The buffers of a prompt pass of up to `rows` rows.  A longer prompt than any
 // before replaces them by larger ones (the stream is idle between prefills).
 void Mi355DenseFp4Provider::ensure_prefill_workspace(std::uint32_t rows) {
   if (rows <= prefill_rows_) return;
-  if (prefill_rows_) {
-    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
-              "drain the stream before the prefill workspace grows");
+  const auto release = [this] {
     for (void* pointer : prefill_allocations_) (void)hipFree(pointer);
     prefill_allocations_.clear();
     prefill_rows_ = 0U;
+  };
+  if (prefill_rows_) {
+    hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)),
+              "drain the stream before the prefill workspace grows");
+    release();
   }
-  const auto allocate = [this](std::size_t bytes) {
+  // an allocation that fails part-way leaves no workspace at all rather than
+  // a mix of new and dangling buffers: the next prompt starts over
+  const auto allocate = [this, &release](std::size_t bytes) {
     void* pointer{};
-    hip_check(hipMalloc(&pointer, bytes), "allocate prefill workspace");
+    if (const auto error = hipMalloc(&pointer, bytes); error != hipSuccess) {
+      release();
+      hip_check(error, "allocate prefill workspace");
+    }
     prefill_allocations_.push_back(pointer);
     return pointer;
   };
@@ -2081,8 +2079,7 @@ Mi355DenseFp4Provider::PrefillResult Mi355DenseFp4Provider::prefill(
         const bool tall = g_.hidden <= 16384U &&
                           mtp_.fusion.descriptor.layout == QLLM_LAYOUT_TILED;
         if (pairs && tall) {
-          enqueue_mtp_prefill(tokens.subspan(done + 1U, pairs), position,
-                              attention_batch);
+          enqueue_mtp_prefill(tokens.subspan(done + 1U, pairs), position);
           state->mtp_length += pairs;
           ++mtp_passes_;
           mtp_rows_ += pairs;
@@ -2600,8 +2597,13 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   void* const stream = stream_;
   const auto hip_stream = static_cast<hipStream_t>(stream_);
   const std::uint32_t rotary_position = cache_position + 1U;  // row 0
-  status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, mtp_tokens_,
-                                        mtp_embedding_, rows, stream));
+  // the lookup is part of the input norms' launch where that kernel serves
+  const bool fused_lookup = !g_.activation_q8 && g_.hidden <= 16384U &&
+                            g_.hidden % 4U == 0U &&
+                            embedding_.descriptor.layout == QLLM_LAYOUT_ROW_MAJOR;
+  if (!fused_lookup)
+    status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, mtp_tokens_,
+                                          mtp_embedding_, rows, stream));
   // [RMSNorm(embedding) | RMSNorm(previous target hidden)] -> fusion projection
   const std::size_t half_bytes = std::size_t{g_.hidden} * 2U;
   const bool q8 = g_.activation_q8;
@@ -2647,6 +2649,11 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                hipMemcpyDeviceToDevice, hip_stream),
               "assemble MTP target hidden batch");
     enqueue_quantise(mtp_fusion_f32_, rows, 2U * g_.hidden);
+  } else if (fused_lookup) {
+    status_check(qllm_rms_norm_concat_embedding_batch(
+        &embedding_.descriptor, mtp_tokens_, mtp_.embedding_norm, previous_hidden,
+        mtp_.hidden_norm, mtp_fusion_input_, rows, g_.norm_epsilon,
+        g_.zero_centered_norm, stream));
   } else if (g_.hidden <= 16384U) {
     status_check(qllm_rms_norm_concat_batch(
         mtp_embedding_, mtp_.embedding_norm, previous_hidden, mtp_.hidden_norm,
@@ -2690,22 +2697,22 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
         &layer.qkv.descriptor, normalized_, hidden_bytes, projections, 3U, rows,
         gemm_workspace_, gemm_workspace_bytes_, stream));
   const auto pages = const_cast<const void* const*>(device_page_table_);
-  if (deferred_positions) {
-    status_check(qllm_qkv_rope_batch_deferred(
-        query_, query_stride, key_, layer.query_norm, layer.key_norm,
-        mtp_positions_, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
-        g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
-    status_check(qllm_store_kv_paged_q8_batch_deferred(
-        key_, value_, pages, mtp_page_offset_, g_.kv_page_tokens,
-        mtp_positions_, rows, g_.kv_heads, g_.head_dim, stream));
-  } else {
-    status_check(qllm_qkv_rope_batch(
-        query_, query_stride, key_, layer.query_norm, layer.key_norm,
-        rotary_position, rows, g_.query_heads, g_.kv_heads, g_.head_dim,
-        g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0, stream));
-    status_check(qllm_store_kv_paged_q8_batch(
-        key_, value_, pages, mtp_page_offset_, g_.kv_page_tokens,
-        cache_position, rows, g_.kv_heads, g_.head_dim, stream));
+  // rotary of q and k and the rows' Q8 K/V records in one launch
+  status_check(qllm_qkv_rope_store_q8_batch(
+      query_, query_stride, key_, value_, layer.query_norm, layer.key_norm, pages,
+      mtp_page_offset_, g_.kv_page_tokens, cache_position, rotary_position,
+      deferred_positions ? mtp_positions_ : nullptr, rows, g_.query_heads,
+      g_.kv_heads, g_.head_dim, g_.rotary_dim, g_.norm_epsilon, g_.rope_theta, 0,
+      stream));
+  if (!produce_logits) {
+    // A pass that only feeds the proposer's cache ends here: the layer has no
+    // successor, so nothing reads its attention or FFN output (the reference
+    // computes them all the same, run_mtp :8737-8766).
+    if (deferred_positions)
+      status_check(qllm_rollout_advance(mtp_argmax_, mtp_tokens_,
+                                        mtp_draft_tokens_, g_.draft_depth, rows,
+                                        mtp_positions_, stream));
+    return;
   }
   qllm_q8_attention_launch launch{};
   launch.query = query_;
@@ -2745,30 +2752,33 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
         activation_, rows, gemm_workspace_, gemm_workspace_bytes_, stream));
   }
   // a single-row pass leaves its hidden state where the next pass reads it
-  const bool retain_in_place = rows == 1U && produce_logits;
+  const bool retain_in_place = rows == 1U;
   project(layer.down.descriptor, activation_,
           std::size_t{rows} * g_.intermediate * 2U,
           retain_in_place ? mtp_last_hidden_ : mtp_hidden_, mtp_hidden_, rows);
-  if (produce_logits) {
-    // draft head: the last row, draft norm, the head's first draft_vocabulary
-    // rows
-    if (!retain_in_place)
-      hip_check(hipMemcpyAsync(
-                    mtp_last_hidden_,
-                    mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
-                    g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
-                "retain final MTP hidden state");
-    normalise(mtp_last_hidden_, mtp_.draft_norm, 1U);
+  // draft head: the last row, draft norm, the head's first draft_vocabulary rows
+  if (!retain_in_place)
+    hip_check(hipMemcpyAsync(mtp_last_hidden_,
+                             mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
+                             g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
+              "retain final MTP hidden state");
+  normalise(mtp_last_hidden_, mtp_.draft_norm, 1U);
+  if (q8) {
     project(mtp_.head_prefix, normalized_, std::size_t{g_.hidden} * 2U, mtp_logits_,
             nullptr, 1U);
-    status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U,
-                                   mtp_argmax_, select_workspace_,
-                                   select_workspace_bytes_, stream));
+    status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U, mtp_argmax_,
+                                   select_workspace_, select_workspace_bytes_,
+                                   stream));
+    if (deferred_positions)
+      status_check(qllm_rollout_advance(mtp_argmax_, mtp_tokens_, mtp_draft_tokens_,
+                                        g_.draft_depth, rows, mtp_positions_, stream));
+    return;
   }
-  if (deferred_positions)
-    status_check(qllm_rollout_advance(mtp_argmax_, mtp_tokens_,
-                                      mtp_draft_tokens_, g_.draft_depth, rows,
-                                      mtp_positions_, stream));
+  // the draft head, its arg-max and the hand-over to the next pass
+  const qllm_rollout_step advance{mtp_tokens_, mtp_draft_tokens_, g_.draft_depth, rows,
+                                  mtp_positions_};
+  enqueue_head_projection(mtp_.head_prefix, mtp_logits_, 1U, mtp_argmax_,
+                          deferred_positions ? &advance : nullptr);
 }
 
 // Replays the proposer pass captured for (rows, source of the previous hidden

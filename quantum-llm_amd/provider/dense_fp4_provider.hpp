@@ -312,6 +312,9 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void enqueue_ffn_block(std::uint32_t index, std::uint32_t rows,
                          bool leave_partials);
   void enqueue_head(std::uint32_t first_row, std::uint32_t rows);
+  void enqueue_head_projection(const qllm_fp4_matrix& head, float* logits,
+                               std::uint32_t rows, std::uint32_t* tokens,
+                               const qllm_rollout_step* advance);
   // run_head with a request (dense_fp4_provider.cpp:8433-8517): presence
   // penalty, arg-max or sampling of the single head row in logits_, the
   // emitted token marked
@@ -393,7 +396,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
                    bool produce_logits, std::uint32_t cache_position,
                    bool deferred_positions);
   void enqueue_mtp_prefill(std::span<const std::uint32_t> tokens,
-                           std::uint32_t position, std::uint32_t attention_batch);
+                           std::uint32_t position);
   void launch_mtp_graph(std::uint32_t rows, bool chained,
                         std::uint32_t drafts = 0U);
   // run_mtp + extend_mtp_rollout replayed from captured graphs

@@ -37,6 +37,12 @@ class Fp4Matrix(Structure):
                 ("layout", c_uint32), ("tile_rows", c_uint32)]
 
 
+class RolloutStep(Structure):
+    _fields_ = [("next_token", c_void_p), ("draft_tokens", c_void_p),
+                ("capacity", c_uint32), ("rows", c_uint32),
+                ("device_positions", c_void_p)]
+
+
 class Q4hAttentionLaunch(Structure):
     _fields_ = [("query", c_void_p), ("q8_queries", c_void_p),
                 ("query_scales", c_void_p), ("page_table", c_void_p),
@@ -114,6 +120,7 @@ SIGNATURES = {
     "qllm_rms_norm_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_residual_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_concat_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_silu_product": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_q4h_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
@@ -138,6 +145,9 @@ SIGNATURES = {
     "qllm_q8_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),
     "qllm_store_kv_paged_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_void_p]),
     "qllm_store_kv_paged_q8_batch_deferred": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_void_p]),
+    "qllm_qkv_rope_store_q8_batch": (c_int32, [c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32, c_uint32, c_uint32, c_void_p, c_uint32, c_uint32, c_uint32, c_uint32, c_uint32, c_float, c_float, c_int32, c_void_p]),
+    "qllm_fp4_head_workspace_bytes": (c_size_t, [POINTER(Fp4Matrix), c_uint32]),
+    "qllm_fp4_head_argmax": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_size_t, c_void_p, c_uint32, c_void_p, c_void_p, c_size_t, POINTER(RolloutStep), c_void_p]),
     "qllm_rollout_advance": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p, c_void_p]),
     "qllm_attention_paged_q8": (c_int32, [POINTER(Q8AttentionLaunch)]),
     "qllm_argmax_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),

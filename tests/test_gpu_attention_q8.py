@@ -184,3 +184,74 @@ def test_q8_batched_launch_equals_one_launch_per_batch(device, total, first, Q, 
     if total * (Q // KV) > (32 if d == 256 else 48):
         with pytest.raises(qh.QllmError):
             qh.call("qllm_attention_paged_q8_batched", launch, total)
+
+
+@pytest.mark.parametrize("deferred", [False, True])
+@pytest.mark.parametrize("rows,Q,KV,d,rotary,gated,qk_norm", [
+    (1, 24, 4, 256, 64, True, True),      # one rollout pass at the 27B geometry
+    (5, 8, 2, 128, 128, False, False),
+    (8, 16, 8, 128, 64, True, True)])
+def test_rotary_with_q8_store_equals_the_two_launches(device, rows, Q, KV, d, rotary,
+                                                      gated, qk_norm, deferred):
+    """qllm_qkv_rope_store_q8_batch against the oracle's rotary, and bit-equal -
+    queries, keys and cache bytes - to qllm_qkv_rope_batch followed by
+    qllm_store_kv_paged_q8_batch; cache position and rotary position differ by
+    one as in the proposer, given as arguments or as device words."""
+    rng = np.random.default_rng(rows * 31 + Q)
+    page_tokens, offset, cache_first = 64, 4096, 61       # the rows cross a page edge
+    rotary_first = cache_first + 1
+    stride = d * (2 if gated else 1)
+    q = rng.standard_normal((rows, Q, stride)).astype(np.float32)
+    k = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    v = rng.standard_normal((rows, KV, d)).astype(np.float32)
+    qw = (0.1 * rng.standard_normal(d)).astype(np.float32) if qk_norm else None
+    kw = (0.1 * rng.standard_normal(d)).astype(np.float32) if qk_norm else None
+    d_qw = None if qw is None else gu.device_tensor(qw, device)
+    d_kw = None if kw is None else gu.device_tensor(kw, device)
+    layer_bytes = ol.q8_layer_bytes(page_tokens, KV, d)
+
+    def pages():
+        held = [torch.zeros(offset + layer_bytes, dtype=torch.uint8, device=device)
+                for _ in range(2)]
+        return held, torch.tensor([p.data_ptr() for p in held], dtype=torch.int64,
+                                  device=device)
+
+    one_q, one_k, d_v = (gu.device_tensor(x, device) for x in (q, k, v))
+    one_pages, one_table = pages()
+    words = torch.tensor([cache_first, rotary_first, 0, 0], dtype=torch.int32,
+                         device=device)
+    qh.call("qllm_qkv_rope_store_q8_batch", qh.ptr(one_q), stride, qh.ptr(one_k),
+            qh.ptr(d_v), qh.ptr(d_qw), qh.ptr(d_kw), qh.ptr(one_table), offset,
+            page_tokens, 0 if deferred else cache_first, 0 if deferred else rotary_first,
+            qh.ptr(words) if deferred else None, rows, Q, KV, d, rotary, 1e-6, 1e6, 0,
+            None)
+    two_q, two_k = (gu.device_tensor(x, device) for x in (q, k))
+    two_pages, two_table = pages()
+    qh.call("qllm_qkv_rope_batch", qh.ptr(two_q), stride, qh.ptr(two_k), qh.ptr(d_qw),
+            qh.ptr(d_kw), rotary_first, rows, Q, KV, d, rotary, 1e-6, 1e6, 0, None)
+    qh.call("qllm_store_kv_paged_q8_batch", qh.ptr(two_k), qh.ptr(d_v),
+            qh.ptr(two_table), offset, page_tokens, cache_first, rows, KV, d, None)
+    torch.cuda.synchronize()
+    assert torch.equal(one_q, two_q) and torch.equal(one_k, two_k)
+    for one, two in zip(one_pages, two_pages):
+        assert torch.equal(one, two)
+    got_q, got_k = one_q.cpu().numpy(), one_k.cpu().numpy()
+    for r in range(rows):
+        for h in range(Q):
+            want = ol.head_norm_rope(q[r, h, :d], qw, rotary, rotary_first + r, 1e-6, 1e6)
+            assert np.abs(got_q[r, h, :d] - want).max() < 2e-5
+        for h in range(KV):
+            want = ol.head_norm_rope(k[r, h], kw, rotary, rotary_first + r, 1e-6, 1e6)
+            assert np.abs(got_k[r, h] - want).max() < 2e-5
+    if gated:
+        assert np.array_equal(got_q[..., d:], q[..., d:])
+    # the records are the oracle's encoding of the keys the kernel produced
+    want_pages = [np.zeros(offset + layer_bytes, dtype=np.uint8) for _ in range(2)]
+    for r in range(rows):
+        for h in range(KV):
+            ol.q8_store(want_pages[(cache_first + r) // page_tokens], offset, page_tokens,
+                        cache_first + r, h, KV, d, got_k[r, h], v[r, h])
+    for got, want in zip(one_pages, want_pages):
+        assert np.array_equal(
+            gu.q8_planes_to_records(got.cpu().numpy(), offset, page_tokens, KV, d),
+            want[offset:])

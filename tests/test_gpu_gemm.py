@@ -560,3 +560,153 @@ def test_q8_matrix_core_gemm_rejects_what_it_does_not_take(device):
         qh.call("qllm_fp4_gemm_q8", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(out),
                 qh.OUT_F32, None, 9, None)
     del keep, keep2
+
+
+def _head_argmax(device, matrix, act, batch, advance=None):
+    rows = matrix.rows
+    logits = torch.full((batch, rows), -7.0, device=device)
+    tokens = torch.full((batch,), 12345, dtype=torch.int32, device=device)
+    need = qh.call("qllm_fp4_head_workspace_bytes", matrix, batch)
+    workspace = torch.zeros(need, dtype=torch.uint8, device=device)
+    d_act = gu.device_tensor(ol.bf16_bits(act), device)
+    qh.call("qllm_fp4_head_argmax", matrix, qh.ptr(d_act), d_act.numel() * 2,
+            qh.ptr(logits), batch, qh.ptr(tokens), qh.ptr(workspace), need, advance, None)
+    torch.cuda.synchronize()
+    return logits, tokens.cpu().numpy().astype(np.uint32)
+
+
+def _two_pass_argmax(device, logits):
+    batch, rows = logits.shape
+    tokens = torch.zeros(batch, dtype=torch.int32, device=device)
+    need = qh.call("qllm_argmax_workspace_bytes", rows, batch)
+    workspace = torch.zeros(need, dtype=torch.uint8, device=device)
+    qh.call("qllm_argmax_batch", qh.ptr(logits), rows, batch, qh.ptr(tokens),
+            qh.ptr(workspace), need, None)
+    torch.cuda.synchronize()
+    return tokens.cpu().numpy().astype(np.uint32)
+
+
+@pytest.mark.parametrize("tiled", [True, False])
+@pytest.mark.parametrize("scheme", [ol.SCALE_UE8M0_BLOCK32, ol.SCALE_F16_BLOCK16])
+@pytest.mark.parametrize("rows,padded,batch", [(1000, 1024, 5), (4099, 512, 8), (31, 64, 1),
+                                               (20000, 256, 3)])
+def test_head_with_argmax_equals_projection_then_argmax(device, scheme, rows, padded, batch,
+                                                        tiled):
+    """The head's projection with the arg-max taken in its epilogue: logits bit
+    for bit those of the plain projection, tokens those of qllm_argmax_batch
+    on them and of numpy on the oracle's ordering; vocabulary sizes that end
+    inside a tile."""
+    rng = np.random.default_rng(rows + padded + batch + scheme)
+    codes, scales = synth.fp4_matrix(rng, rows, padded, scheme)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    tensors = [gu.device_tensor(t, device) for t in (codes, scales)]
+    matrix = qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded, scheme)
+    keep = None
+    if tiled:
+        matrix, keep = qh.prepack(matrix, device)
+    logits, tokens = _head_argmax(device, matrix, act, batch)
+    plain = gu.gemm(device, codes, scales, scheme, rows, padded, act, tiled=tiled)
+    got = logits.cpu().numpy()
+    assert np.array_equal(got, plain)
+    assert np.array_equal(tokens, _two_pass_argmax(device, logits))
+    assert np.array_equal(tokens, got.argmax(axis=1).astype(np.uint32))
+    del keep
+
+
+def test_head_with_argmax_ties_and_nan(device):
+    """Equal logits go to the lower row wherever the rows lie (same tile, other
+    tiles); a row whose scale is NaN never wins; a head of NaN rows only selects
+    nothing (0xffffffff), as qllm_argmax_batch does."""
+    rng = np.random.default_rng(5)
+    rows, padded, batch = 700, 256, 4
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    reference = ol.fp4_linear_f64(codes, scales, ol.SCALE_UE8M0_BLOCK32, rows, padded, act)
+    winner = int(reference[0].argmax())
+    for copy in (3, 40, 650):                  # the same row thrice more: exact ties
+        if copy != winner:
+            codes[copy], scales[copy] = codes[winner], scales[winner]
+    scales[1, 0] = 255                         # UE8M0 NaN: row 1 is NaN for every batch row
+    tensors = [gu.device_tensor(t, device) for t in (codes, scales)]
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                                            ol.SCALE_UE8M0_BLOCK32), device)
+    logits, tokens = _head_argmax(device, matrix, act, batch)
+    got = logits.cpu().numpy()
+    assert np.isnan(got[:, 1]).all()
+    assert tokens[0] == min(winner, 3)
+    assert np.array_equal(tokens, _two_pass_argmax(device, logits))
+    assert np.array_equal(tokens, np.nanargmax(got, axis=1).astype(np.uint32))
+    scales[:, 0] = 255
+    d_scales = gu.device_tensor(scales, device)
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], d_scales, rows, padded, padded,
+                                            ol.SCALE_UE8M0_BLOCK32), device)
+    logits, tokens = _head_argmax(device, matrix, act, batch)
+    assert np.isnan(logits.cpu().numpy()).all()
+    assert (tokens == 0xFFFFFFFF).all()
+    assert np.array_equal(tokens, _two_pass_argmax(device, logits))
+    del keep
+
+
+def test_head_with_argmax_hands_the_winner_to_the_next_pass(device):
+    """With a rollout step the selection kernel also does what
+    qllm_rollout_advance does: next token, draft list entry, positions."""
+    rng = np.random.default_rng(6)
+    rows, padded = 5000, 512
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    act = ol.bf16_round(rng.standard_normal((1, padded)).astype(np.float32))
+    tensors = [gu.device_tensor(t, device) for t in (codes, scales)]
+    matrix, keep = qh.prepack(qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                                            ol.SCALE_UE8M0_BLOCK32), device)
+    for slot, capacity in ((1, 4), (4, 4)):    # a free draft entry; a full list
+        state = []
+        for fused in (True, False):
+            next_token = torch.full((1,), 77, dtype=torch.int32, device=device)
+            drafts = torch.full((4,), 99, dtype=torch.int32, device=device)
+            positions = torch.tensor([10, 11, 12, slot], dtype=torch.int32, device=device)
+            step = qh.RolloutStep(qh.ptr(next_token), qh.ptr(drafts), capacity, 3,
+                                  qh.ptr(positions))
+            if fused:
+                logits, tokens = _head_argmax(device, matrix, act, 1, step)
+            else:
+                logits, tokens = _head_argmax(device, matrix, act, 1)
+                selected = torch.tensor(tokens.astype(np.int32), device=device)
+                qh.call("qllm_rollout_advance", qh.ptr(selected), qh.ptr(next_token),
+                        qh.ptr(drafts), capacity, 3, qh.ptr(positions), None)
+                torch.cuda.synchronize()
+            state.append((tokens.tolist(), next_token.tolist(), drafts.tolist(),
+                          positions.tolist()))
+        assert state[0] == state[1]
+        token = state[0][0][0]
+        assert token == int(logits.cpu().numpy()[0].argmax())
+        assert state[0][1] == [token]
+        assert state[0][2] == [token if entry == slot else 99 for entry in range(4)]
+        assert state[0][3] == [13, 14, 15, slot + 1]
+    del keep
+
+
+def test_head_with_argmax_rejects_what_it_does_not_take(device):
+    rng = np.random.default_rng(8)
+    rows, padded = 64, 128
+    codes, scales = synth.fp4_matrix(rng, rows, padded, ol.SCALE_UE8M0_BLOCK32)
+    tensors = [gu.device_tensor(t, device) for t in (codes, scales)]
+    matrix = qh.fp4_matrix(tensors[0], tensors[1], rows, padded, padded,
+                           ol.SCALE_UE8M0_BLOCK32)
+    act = torch.zeros((2, padded), dtype=torch.bfloat16, device=device)
+    logits = torch.zeros((2, rows), device=device)
+    tokens = torch.zeros(2, dtype=torch.int32, device=device)
+    need = qh.call("qllm_fp4_head_workspace_bytes", matrix, 2)
+    workspace = torch.zeros(need, dtype=torch.uint8, device=device)
+    step = qh.RolloutStep(qh.ptr(tokens), qh.ptr(tokens), 1, 1, qh.ptr(tokens))
+
+    def status(*arguments):
+        return qh.load().qllm_fp4_head_argmax(*arguments)
+
+    good = [matrix, qh.ptr(act), act.numel() * 2, qh.ptr(logits), 2, qh.ptr(tokens),
+            qh.ptr(workspace), need, None, None]
+    assert status(*good) == 0
+    torch.cuda.synchronize()
+    for index, value in ((7, need - 1), (4, 9), (4, 0), (2, act.numel() * 2 - 1),
+                         (5, None), (6, None), (8, step)):   # a rollout step takes one row
+        bad = list(good)
+        bad[index] = value
+        assert status(*bad) == 4, index        # QLLM_INVALID_ARGUMENT

@@ -384,3 +384,47 @@ def test_wide_rows_quantise_byte_exactly(device, rows, columns, padded):
     want_q8, want_scales = ol.quantize_q8_rows(x, padded)
     assert np.array_equal(d_q8.cpu().numpy(), want_q8)
     assert np.array_equal(d_s.cpu().numpy(), want_scales)
+
+
+@pytest.mark.parametrize("scheme", [0, 1])
+@pytest.mark.parametrize("rows,elements", [(1, 5120), (5, 256), (8, 1024)])
+def test_lookup_with_two_norms_equals_the_three_launches(device, scheme, rows, elements):
+    """[RMSNorm(embedding[token]) | RMSNorm(hidden)] straight from the FP4
+    table: bit-equal to qllm_fp4_embedding_batch followed by
+    qllm_rms_norm_concat_batch, and the first half within the reference's 2e-5
+    (plus the bf16 rounding) of the oracle's norm of the oracle's lookup."""
+    rng = np.random.default_rng(scheme * 7 + rows)
+    V = 300
+    codes, scales = synth.fp4_matrix(rng, V, elements, scheme)
+    tokens = rng.integers(0, V, rows).astype(np.uint32)
+    tokens[0] = V - 1
+    hidden = (rng.standard_normal((rows, elements)) * 2).astype(np.float32)
+    wa = (0.1 * rng.standard_normal(elements)).astype(np.float32)
+    wb = (0.1 * rng.standard_normal(elements)).astype(np.float32)
+    d = [gu.device_tensor(x, device) for x in (codes, scales, tokens, hidden, wa, wb)]
+    table = qh.fp4_matrix(d[0], d[1], V, elements, elements, scheme)
+    fused = torch.zeros((rows, 2 * elements), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_concat_embedding_batch", table, qh.ptr(d[2]), qh.ptr(d[4]),
+            qh.ptr(d[3]), qh.ptr(d[5]), qh.ptr(fused), rows, 1e-6, 1, None)
+    looked_up = torch.zeros((rows, elements), device=device)
+    qh.call("qllm_fp4_embedding_batch", table, qh.ptr(d[2]), qh.ptr(looked_up), rows, None)
+    apart = torch.zeros_like(fused)
+    qh.call("qllm_rms_norm_concat_batch", qh.ptr(looked_up), qh.ptr(d[4]), qh.ptr(d[3]),
+            qh.ptr(d[5]), qh.ptr(apart), rows, elements, 1e-6, 1, None)
+    torch.cuda.synchronize()
+    assert torch.equal(fused, apart)
+    embedding = ol.fp4_embedding(codes, scales, scheme, elements, elements, tokens)
+    want = ol.rms_norm_rows(embedding, wa, 1e-6, True)
+    got = fused.float().cpu().numpy()[:, :elements]
+    assert (np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 2e-5).all()
+    # a tiled table, an out-of-range width and missing operands are turned down
+    bad = qh.fp4_matrix(d[0], d[1], V, elements, elements, scheme)
+    bad.layout = 1
+    for arguments in ((bad, qh.ptr(d[2]), qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
+                       qh.ptr(fused), rows, 1e-6, 1, None),
+                      (table, None, qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
+                       qh.ptr(fused), rows, 1e-6, 1, None),
+                      (table, qh.ptr(d[2]), qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
+                       qh.ptr(fused), 0, 1e-6, 1, None)):
+        with pytest.raises(qh.QllmError):
+            qh.call("qllm_rms_norm_concat_embedding_batch", *arguments)
