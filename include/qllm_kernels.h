@@ -325,6 +325,19 @@ int32_t qllm_rms_norm_residual_batch(float* hidden, const float* partials,
                                      float epsilon, int32_t zero_centered,
                                      void* stream);
 
+/* The same with the sum written elsewhere: sum[r] = residual[r] + partials[0][r]
+ * + ... (from zero when residual is NULL), output_bf16[r] = RMSNorm(sum[r]).
+ * The proposer's projections use it: the fusion projection has no residual
+ * (run_mtp, dense_fp4_provider.cpp:8716-8735) and a single-row pass leaves its
+ * last sum where the next pass reads it (:8766-8783).  `sum` may be
+ * `residual`; same limits as above. */
+int32_t qllm_rms_norm_partials_batch(const float* residual, float* sum,
+                                     const float* partials, uint32_t partial_count,
+                                     const float* weight, void* output_bf16,
+                                     uint32_t rows, uint32_t elements,
+                                     float epsilon, int32_t zero_centered,
+                                     void* stream);
+
 /* Two normalisations into one bf16 batch: output row r, of 2 * elements
  * columns, is [RMSNorm(first[r]) | RMSNorm(second[r])], each half with its own
  * weight (either may be NULL) and the values of qllm_rms_norm_batch.  The
@@ -344,12 +357,15 @@ int32_t qllm_rms_norm_concat_batch(const float* first,
  * (row-major) at `tokens`: qllm_fp4_embedding_batch folded into the norm - the
  * proposer's embedding lookup and its two input norms in one launch (run_mtp,
  * dense_fp4_provider.cpp:8699-8735).  Same values as the lookup followed by
- * qllm_rms_norm_concat_batch; elements = embedding->columns. */
+ * qllm_rms_norm_concat_batch; elements = embedding->columns.  presence (NULL,
+ * or vocabulary bytes): the batch's tokens are marked as qllm_mark_presence
+ * marks them - the pass over the tokens a verify step emitted
+ * (:11261-11270). */
 int32_t qllm_rms_norm_concat_embedding_batch(
     const qllm_fp4_matrix* embedding, const uint32_t* tokens,
     const float* first_weight, const float* second, const float* second_weight,
     void* output_bf16, uint32_t rows, float epsilon, int32_t zero_centered,
-    void* stream);
+    uint8_t* presence, void* stream);
 
 /* replaces add_in_place (transformer_kernels.hpp:310-312). */
 int32_t qllm_add_in_place(float* destination, const float* source,

@@ -299,48 +299,14 @@ double qllm_sampling_counter_uniform(uint64_t seed, uint32_t position,
                                      uint32_t stream, uint32_t index);
 
 /* ---- artifact reader ----------------------------------------------------------
- * Host only; none of these calls touches a device.  Text results are written
- * NUL-terminated into `dump` (truncated to `capacity`), their full length
- * into `*dump_bytes`; on failure the status is the reference's ErrorCode and
- * the message is in qllm_provider_last_error(). */
+ * Host only; none of these calls touches a device.  On failure the status is
+ * the reference's ErrorCode and the message is in qllm_provider_last_error(). */
 
 /* sha256() of runtime/include/expert/runtime/sha256.hpp:26. */
 int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest32);
 /* The same digest computed without the CPU's SHA instructions, which
  * qllm_sha256 uses where the host has them. */
 int32_t qllm_sha256_portable(const void* data, size_t bytes, uint8_t* digest32);
-
-/* parse_model_descriptor_artifact (runtime/include/expert/runtime/
- * model_descriptor.hpp:276-281; runtime/src/model_descriptor.cpp:527-723):
- * parses and validates the text of runtime-model.tsv.  The result is the
- * descriptor in a canonical line form: the program's own records with maps in
- * key order, component namespaces resolved against namespace_base, and the
- * content hash. */
-int32_t qllm_model_descriptor_parse(const char* text, size_t text_bytes,
-                                    const uint8_t* content_sha256,
-                                    uint64_t namespace_base, char* dump,
-                                    size_t capacity, size_t* dump_bytes);
-/* Binds a model program against providers described in text ("provider
- * <name> <priority> <callable 0|1>" lines, each followed by its "capability
- * <name> <minimum_abi> <maximum_abi>" lines, tab separated) and writes a
- * canonical report: registration statuses, the bind status, the providers of
- * the plan and the compiled program (ExecutionProviderRegistry::add / bind,
- * runtime/src/execution_provider.cpp:10-131; compile_model_program,
- * runtime/src/model_descriptor.cpp:374-490).  executable != 0 binds callable
- * providers only. */
-int32_t qllm_model_program_bind(const char* text, size_t text_bytes,
-                                const uint8_t* content_sha256,
-                                uint64_t namespace_base, const char* providers,
-                                int32_t executable, char* dump, size_t capacity,
-                                size_t* dump_bytes);
-
-/* load_model_descriptor_artifact (model_descriptor.hpp:282-285): the file
- * must have expected_bytes bytes and the expected SHA-256. */
-int32_t qllm_model_descriptor_load(const char* path, uint64_t expected_bytes,
-                                   const uint8_t* expected_sha256,
-                                   const uint8_t* content_sha256,
-                                   uint64_t namespace_base, char* dump,
-                                   size_t capacity, size_t* dump_bytes);
 
 /* ModelArtifact::load (+ configure_mtp_draft_depth when mtp_draft_depth != 0)
  * and, with map_tensors, MappedModelTensorStore::create
@@ -350,9 +316,6 @@ typedef struct qllm_artifact qllm_artifact;
 int32_t qllm_artifact_open(const char* root, uint32_t mtp_draft_depth,
                            int32_t map_tensors, qllm_artifact** artifact);
 void qllm_artifact_close(qllm_artifact* artifact);
-/* "pack" and "tensor" lines of the index, then the model descriptor. */
-int32_t qllm_artifact_dump(const qllm_artifact* artifact, char* dump,
-                           size_t capacity, size_t* dump_bytes);
 /* IModelTensorStore::resolve (program_executor.hpp:57-62): the mapped record
  * of a dense tensor; with check_header the record's 256-byte header is
  * checked against the index entry first (compiler/expert_pack/validate.py:

@@ -1,11 +1,17 @@
-// C-callable shim over the reference's own artifact reader.  TEST
-// INFRASTRUCTURE ONLY.  Compiled together with the reference sources
-// runtime/src/{model_descriptor,execution_provider,model_artifact,
-// model_tensor_store,sha256,expert_catalog,expert_record}.cpp and
-// core/src/json.cpp, read where they lie
-// in the reference tree, into oracle/_ref/libqllm_ref_artifact.so.  The shim
-// adds no logic: it calls the reference's functions and prints their results
-// with the same writer (descriptor_dump.hpp) the product uses on its own types.
+// C-callable shim over an artifact reader and provider registry that follow
+// the declarations of namespace expert::runtime.  TEST INFRASTRUCTURE ONLY:
+// it exists so that tests can print what a reader made of its input and compare
+// two readers line by line.  Built twice by oracle/Makefile:
+//   - with the reference sources runtime/src/{model_descriptor,
+//     execution_provider,model_artifact,model_tensor_store,sha256,
+//     expert_catalog,expert_record}.cpp and core/src/json.cpp, read where they
+//     lie in the reference tree, into oracle/_ref/libqllm_ref_artifact.so
+//     (functions qref_*);
+//   - with -DQLLM_SHIM_OVER_PRODUCT against this repository's headers and
+//     libqllm_provider.so, into oracle/libqllm_provider_probe.so (functions
+//     qprobe_*).
+// The shim adds no logic: it calls the reader's functions and prints their
+// results with one writer (descriptor_dump.hpp, registry_probe.hpp).
 #include "expert/runtime/model_artifact.hpp"
 #include "expert/runtime/model_descriptor.hpp"
 #include "expert/runtime/model_tensor_store.hpp"
@@ -21,6 +27,12 @@
 #include <string>
 
 namespace er = expert::runtime;
+
+#ifdef QLLM_SHIM_OVER_PRODUCT
+#define SHIM(name) qprobe_##name
+#else
+#define SHIM(name) qref_##name
+#endif
 
 namespace {
 
@@ -56,12 +68,12 @@ struct Artifact {
 
 extern "C" {
 
-void qref_sha256(const void* data, std::size_t bytes, std::uint8_t* digest) {
+void SHIM(sha256)(const void* data, std::size_t bytes, std::uint8_t* digest) {
   const auto result = er::sha256({static_cast<const std::byte*>(data), bytes});
   std::memcpy(digest, result.data(), result.size());
 }
 
-int qref_model_descriptor_parse(const char* text, std::size_t text_bytes,
+int SHIM(model_descriptor_parse)(const char* text, std::size_t text_bytes,
                                 const std::uint8_t* content_sha256,
                                 std::uint64_t namespace_base, char* dump,
                                 std::size_t capacity, std::size_t* dump_bytes) {
@@ -73,7 +85,7 @@ int qref_model_descriptor_parse(const char* text, std::size_t text_bytes,
   return 0;
 }
 
-int qref_model_descriptor_load(const char* path, std::uint64_t expected_bytes,
+int SHIM(model_descriptor_load)(const char* path, std::uint64_t expected_bytes,
                                const std::uint8_t* expected_sha256,
                                const std::uint8_t* content_sha256,
                                std::uint64_t namespace_base, char* dump,
@@ -89,7 +101,7 @@ int qref_model_descriptor_load(const char* path, std::uint64_t expected_bytes,
 
 // the reference's ExecutionProviderRegistry and compile_model_program
 // (runtime/src/execution_provider.cpp, model_descriptor.cpp:374-490)
-void qref_model_program_bind(const char* text, std::size_t text_bytes,
+void SHIM(model_program_bind)(const char* text, std::size_t text_bytes,
                              const std::uint8_t* content_sha256,
                              std::uint64_t namespace_base, const char* providers,
                              int executable, char* dump, std::size_t capacity,
@@ -99,7 +111,7 @@ void qref_model_program_bind(const char* text, std::size_t text_bytes,
             dump, capacity, dump_bytes);
 }
 
-int qref_artifact_open(const char* root, std::uint32_t mtp_draft_depth,
+int SHIM(artifact_open)(const char* root, std::uint32_t mtp_draft_depth,
                        int map_tensors, void** out, char* message,
                        std::size_t capacity) {
   *out = nullptr;
@@ -114,15 +126,15 @@ int qref_artifact_open(const char* root, std::uint32_t mtp_draft_depth,
   return 0;
 }
 
-void qref_artifact_close(void* artifact) { delete static_cast<Artifact*>(artifact); }
+void SHIM(artifact_close)(void* artifact) { delete static_cast<Artifact*>(artifact); }
 
-void qref_artifact_dump(const void* artifact, char* dump, std::size_t capacity,
+void SHIM(artifact_dump)(const void* artifact, char* dump, std::size_t capacity,
                         std::size_t* dump_bytes) {
   copy_text(qllm::dump::model_artifact(static_cast<const Artifact*>(artifact)->artifact),
             dump, capacity, dump_bytes);
 }
 
-int qref_artifact_tensor(void* artifact, const char* name, const void** record,
+int SHIM(artifact_tensor)(void* artifact, const char* name, const void** record,
                          std::uint64_t* record_bytes, char* message,
                          std::size_t capacity) {
   const auto resolved = static_cast<Artifact*>(artifact)->store.resolve(name);

@@ -243,16 +243,24 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
       for (int i = 0; i < 4; ++i) out[dt][rt][i] = 0.0f;
   }
 
-  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+  // Q8 cache: a tile's codes and scales as the lanes fetch them - V granules
+  // (8 codes) pass * 64 + lane, the K operand rows, the scales of the lane's
+  // tokens.  The next tile's are asked for before the tile at hand is worked on,
+  // so a wave always has one tile in flight (the binary16 cache at head_dim 128
+  // has the kernel below for that) - where the registers hold a second tile.
+  constexpr bool AHEAD = Q8 && D == 128 && RT <= 2;
+  constexpr int V_PASSES = kF16Tile * GR / 64;
+  struct Q8Tile {
+    uint2 value[V_PASSES];
+    uint2 key[2][KSTEPS];
+    uint2 key_scale[2];
+    uint2 value_scale[2];
+  };
+  const auto fetch_q8_tile = [&](uint32_t tile, Q8Tile& loaded) {
     const uint32_t tile_begin = tile * kF16Tile;
-    const bool needs_mask = tile_begin + kF16Tile > first_context_tokens;
     const void* page_base = uniform_page(args.pages, tile_begin / args.page_tokens);
     const uint32_t tile_slot = tile_begin % args.page_tokens;
-    // binary16 cache
-    const uint16_t* keys = static_cast<const uint16_t*>(page_base) + layer_offset +
-                           static_cast<size_t>(tile_slot) * row_stride + kv_head * D;
-    const uint16_t* values = keys + page_values;
-    // Q8 cache: code planes, then scale planes [kv_heads][page_tokens]
+    // code planes, then scale planes [kv_heads][page_tokens]
     const uint8_t* keys8 = static_cast<const uint8_t*>(page_base) + args.page_offset +
                            static_cast<size_t>(tile_slot) * row_stride + kv_head * D;
     const uint8_t* values8 = keys8 + page_values;
@@ -262,6 +270,47 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
         static_cast<size_t>(kv_head) * args.page_tokens + tile_slot;
     const uint16_t* value_scales =
         key_scales + static_cast<size_t>(args.kv_heads) * args.page_tokens;
+#pragma unroll
+    for (int pass = 0; pass < V_PASSES; ++pass) {
+      const uint32_t piece = pass * 64u + lane;
+      loaded.value[pass] = *reinterpret_cast<const uint2*>(
+          values8 + static_cast<size_t>(piece / GR) * row_stride + (piece % GR) * 8u);
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        loaded.key[st][ks] = *reinterpret_cast<const uint2*>(
+            keys8 + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
+            8u * quad);
+      loaded.key_scale[st] =
+          *reinterpret_cast<const uint2*>(key_scales + 16u * st + 4u * quad);
+      loaded.value_scale[st] =
+          *reinterpret_cast<const uint2*>(value_scales + 16u * st + 4u * quad);
+    }
+  };
+  Q8Tile q8_tile{}, q8_next{};
+  if constexpr (AHEAD)
+    if (tile_first < tile_last) fetch_q8_tile(tile_first, q8_tile);
+
+  for (uint32_t tile = tile_first; tile < tile_last; ++tile) {
+    const uint32_t tile_begin = tile * kF16Tile;
+    const bool needs_mask = tile_begin + kF16Tile > first_context_tokens;
+    if constexpr (AHEAD) {
+      if (tile + 1u < tile_last) fetch_q8_tile(tile + 1u, q8_next);
+    } else if constexpr (Q8) {
+      fetch_q8_tile(tile, q8_tile);
+    }
+    // binary16 cache
+    const uint16_t* keys = nullptr;
+    const uint16_t* values = nullptr;
+    if constexpr (!Q8) {
+      const void* page_base = uniform_page(args.pages, tile_begin / args.page_tokens);
+      const uint32_t tile_slot = tile_begin % args.page_tokens;
+      keys = static_cast<const uint16_t*>(page_base) + layer_offset +
+             static_cast<size_t>(tile_slot) * row_stride + kv_head * D;
+      values = keys + page_values;
+    }
 
     // ---- V tile -> LDS (swizzled rows) ----------------------------------------
 #pragma unroll
@@ -271,9 +320,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
       const uint32_t part = piece % GR;
       uint4 value;
       if constexpr (Q8)
-        value = __builtin_bit_cast(
-            uint4, int8x8_to_f16(*reinterpret_cast<const uint2*>(
-                       values8 + static_cast<size_t>(token) * row_stride + part * 8u)));
+        value = __builtin_bit_cast(uint4, int8x8_to_f16(q8_tile.value[pass]));
       else
         value = *reinterpret_cast<const uint4*>(
             values + static_cast<size_t>(token) * row_stride + part * 8u);
@@ -293,9 +340,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         if constexpr (Q8)
-          key_operand[st][ks] = int8x8_to_f16(*reinterpret_cast<const uint2*>(
-              keys8 + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
-              8u * quad));
+          key_operand[st][ks] = int8x8_to_f16(q8_tile.key[st][ks]);
         else
           key_operand[st][ks] = *reinterpret_cast<const f16x8*>(
               keys + static_cast<size_t>(16u * st + col) * row_stride + 32u * ks +
@@ -309,8 +354,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
     if constexpr (Q8) {
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
-        const uint2 k = *reinterpret_cast<const uint2*>(key_scales + 16u * st + 4u * quad);
-        uint2 v = *reinterpret_cast<const uint2*>(value_scales + 16u * st + 4u * quad);
+        const uint2 k = q8_tile.key_scale[st];
+        uint2 v = q8_tile.value_scale[st];
         key_scale[st][0] = f16_bits_to_f32(k.x & 0xffffu) * score_unit;
         key_scale[st][1] = f16_bits_to_f32(k.x >> 16) * score_unit;
         key_scale[st][2] = f16_bits_to_f32(k.y & 0xffffu) * score_unit;
@@ -412,6 +457,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void f16_attention_split_kernel(
       }
     }
     __builtin_amdgcn_wave_barrier();
+    if constexpr (AHEAD) q8_tile = q8_next;
   }
 
 #pragma unroll

@@ -285,7 +285,8 @@ __device__ __forceinline__ void rms_norm_row_wide(
     if (index < vectors)
       values[slot] = fp4_codes_row ? fp4_row_vector(fp4_codes_row, fp4_scales_row,
                                                     fp4_scheme, index)
-                                   : x[index];
+                     : input_row   ? x[index]
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
     factors[slot] = make_float4(1.f, 1.f, 1.f, 1.f);
     if (weight && index < vectors)
       factors[slot] = reinterpret_cast<const float4*>(weight)[index];
@@ -401,20 +402,21 @@ __global__ __launch_bounds__(1024) void rms_norm_q8_kernel(
                     output_q8 + row * elements, scales + row);
 }
 
-// hidden[r] += partials[0][r] + ... + partials[count-1][r], then its RMSNorm in
-// bf16: the residual add of a projection whose K was cut over workgroups
-// (qllm_fp4_gemm_bf16_partial) folded into the norm that follows it.
+// sum[r] = residual[r] + partials[0][r] + ... + partials[count-1][r] (from zero
+// without a residual), then its RMSNorm in bf16: the residual add of a
+// projection whose K was cut over workgroups (qllm_fp4_gemm_bf16_partial)
+// folded into the norm that follows it.  `sum` may be `residual`.
 __global__ __launch_bounds__(1024) void rms_norm_residual_kernel(
-    float* hidden, const float* partials, uint32_t partial_count,
-    const float* weight, uint16_t* output_bf16, uint32_t elements,
-    float epsilon, bool zero_centered) {
+    const float* residual, float* sum, const float* partials,
+    uint32_t partial_count, const float* weight, uint16_t* output_bf16,
+    uint32_t elements, float epsilon, bool zero_centered) {
   __shared__ float scratch[16];
   const size_t row = blockIdx.x;
-  rms_norm_row_wide(hidden + row * elements, weight, nullptr,
+  rms_norm_row_wide(residual ? residual + row * elements : nullptr, weight, nullptr,
                     output_bf16 + row * elements, elements, elements, epsilon,
                     zero_centered, scratch, partials + row * elements,
                     partial_count, static_cast<size_t>(gridDim.x) * elements,
-                    hidden + row * elements);
+                    sum + row * elements);
 }
 
 // Row r of the output is [RMSNorm(first[r]) | RMSNorm(second[r])] in bf16:
@@ -441,7 +443,8 @@ __global__ __launch_bounds__(1024) void rms_norm_concat_embedding_kernel(
     const uint8_t* codes, const uint8_t* scales, uint32_t scheme,
     uint32_t padded_columns, uint32_t vocabulary, const uint32_t* tokens,
     const float* first_weight, const float* second, const float* second_weight,
-    uint16_t* output_bf16, uint32_t elements, float epsilon, bool zero_centered) {
+    uint16_t* output_bf16, uint32_t elements, float epsilon, bool zero_centered,
+    uint8_t* presence) {
   __shared__ float scratch[16];
   const size_t row = blockIdx.x;
   uint16_t* out = output_bf16 + row * 2u * elements;
@@ -452,6 +455,8 @@ __global__ __launch_bounds__(1024) void rms_norm_concat_embedding_kernel(
     return;
   }
   const size_t token = tokens[row];
+  // (mark_presence_kernel's store, for callers whose batch is emitted tokens)
+  if (presence && threadIdx.x == 0u && token < vocabulary) presence[token] = 1u;
   if (token >= vocabulary) {
     for (uint32_t index = threadIdx.x; index < elements; index += blockDim.x)
       out[index] = 0u;
@@ -661,9 +666,28 @@ extern "C" int32_t qllm_rms_norm_residual_batch(
   // (measured on rows of 5120: 320 threads, four float4 each, take 6.0 us
   // against 4.75 us with 1024: one CU's few waves wait longer for the row)
   rms_norm_residual_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
-      hidden, partials, partial_count, weight,
+      hidden, hidden, partials, partial_count, weight,
       static_cast<uint16_t*>(output_bf16), elements, epsilon, zero_centered != 0);
   return launched("residual RMSNorm");
+}
+
+extern "C" int32_t qllm_rms_norm_partials_batch(
+    const float* residual, float* sum, const float* partials,
+    uint32_t partial_count, const float* weight, void* output_bf16, uint32_t rows,
+    uint32_t elements, float epsilon, int32_t zero_centered, void* stream) {
+  const auto aligned = [](const void* pointer) {
+    return reinterpret_cast<uintptr_t>(pointer) % 16u == 0u;
+  };
+  if (!sum || !partials || !partial_count || partial_count > 16u ||
+      !output_bf16 || !rows || rows > 65535u || !elements ||
+      elements % 4u != 0u || elements > 16384u || !aligned(residual) ||
+      !aligned(sum) || !aligned(partials) || !aligned(output_bf16) ||
+      (weight && !aligned(weight)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid RMSNorm of partial sums");
+  rms_norm_residual_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+      residual, sum, partials, partial_count, weight,
+      static_cast<uint16_t*>(output_bf16), elements, epsilon, zero_centered != 0);
+  return launched("RMSNorm of partial sums");
 }
 
 extern "C" int32_t qllm_rms_norm_concat_batch(
@@ -689,7 +713,7 @@ extern "C" int32_t qllm_rms_norm_concat_embedding_batch(
     const qllm_fp4_matrix* embedding, const uint32_t* tokens,
     const float* first_weight, const float* second, const float* second_weight,
     void* output_bf16, uint32_t rows, float epsilon, int32_t zero_centered,
-    void* stream) {
+    uint8_t* presence, void* stream) {
   if (!embedding || !embedding->weights || !embedding->scales || !embedding->rows ||
       embedding->layout != QLLM_LAYOUT_ROW_MAJOR || embedding->scale_scheme > 1u ||
       embedding->padded_columns < embedding->columns ||
@@ -707,7 +731,7 @@ extern "C" int32_t qllm_rms_norm_concat_embedding_batch(
       embedding->weights, static_cast<const uint8_t*>(embedding->scales),
       embedding->scale_scheme, embedding->padded_columns, embedding->rows, tokens,
       first_weight, second, second_weight, static_cast<uint16_t*>(output_bf16),
-      embedding->columns, epsilon, zero_centered != 0);
+      embedding->columns, epsilon, zero_centered != 0, presence);
   return launched("RMSNorm concat of an embedding batch");
 }
 

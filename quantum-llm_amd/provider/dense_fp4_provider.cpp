@@ -1711,7 +1711,8 @@ void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
         normalized_, g_.hidden, rows, g_.hidden, g_.norm_epsilon,
         g_.zero_centered_norm, stream_));
   }
-  enqueue_head_projection(head_.descriptor, logits_, rows, argmax_tokens_, nullptr);
+  enqueue_head_projection(head_.descriptor, normalized_, logits_, rows,
+                          argmax_tokens_, nullptr);
 }
 
 // logits = head . normalized_ and their arg-max tokens: the projection's
@@ -1719,17 +1720,17 @@ void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
 // `advance`, which also hands the winner to the next proposer pass); matrices
 // the matrix-core kernel does not take go through the plain arg-max.
 void Mi355DenseFp4Provider::enqueue_head_projection(
-    const qllm_fp4_matrix& head, float* logits, std::uint32_t rows,
-    std::uint32_t* tokens, const qllm_rollout_step* advance) {
+    const qllm_fp4_matrix& head, const std::uint16_t* input, float* logits,
+    std::uint32_t rows, std::uint32_t* tokens, const qllm_rollout_step* advance) {
   const std::size_t input_bytes = std::size_t{rows} * g_.hidden * 2U;
   if (head.padded_columns % 64U == 0U &&
       qllm_fp4_head_workspace_bytes(&head, rows) <= select_workspace_bytes_) {
-    status_check(qllm_fp4_head_argmax(&head, normalized_, input_bytes, logits, rows,
+    status_check(qllm_fp4_head_argmax(&head, input, input_bytes, logits, rows,
                                       tokens, select_workspace_,
                                       select_workspace_bytes_, advance, stream_));
     return;
   }
-  status_check(qllm_fp4_gemm_bf16(&head, normalized_, input_bytes, logits,
+  status_check(qllm_fp4_gemm_bf16(&head, input, input_bytes, logits,
                                   QLLM_OUT_F32, nullptr, rows, stream_));
   status_check(qllm_argmax_batch(logits, head.rows, rows, tokens, select_workspace_,
                                  select_workspace_bytes_, stream_));
@@ -2593,7 +2594,8 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                         const float* previous_hidden,
                                         bool produce_logits,
                                         std::uint32_t cache_position,
-                                        bool deferred_positions) {
+                                        bool deferred_positions,
+                                        std::uint8_t* mark_emitted) {
   void* const stream = stream_;
   const auto hip_stream = static_cast<hipStream_t>(stream_);
   const std::uint32_t rotary_position = cache_position + 1U;  // row 0
@@ -2601,9 +2603,13 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   const bool fused_lookup = !g_.activation_q8 && g_.hidden <= 16384U &&
                             g_.hidden % 4U == 0U &&
                             embedding_.descriptor.layout == QLLM_LAYOUT_ROW_MAJOR;
-  if (!fused_lookup)
+  if (!fused_lookup) {
     status_check(qllm_fp4_embedding_batch(&embedding_.descriptor, mtp_tokens_,
                                           mtp_embedding_, rows, stream));
+    if (mark_emitted)
+      status_check(qllm_mark_presence(mark_emitted, mtp_tokens_, rows,
+                                      g_.vocabulary, stream));
+  }
   // [RMSNorm(embedding) | RMSNorm(previous target hidden)] -> fusion projection
   const std::size_t half_bytes = std::size_t{g_.hidden} * 2U;
   const bool q8 = g_.activation_q8;
@@ -2653,7 +2659,7 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
     status_check(qllm_rms_norm_concat_embedding_batch(
         &embedding_.descriptor, mtp_tokens_, mtp_.embedding_norm, previous_hidden,
         mtp_.hidden_norm, mtp_fusion_input_, rows, g_.norm_epsilon,
-        g_.zero_centered_norm, stream));
+        g_.zero_centered_norm, mark_emitted, stream));
   } else if (g_.hidden <= 16384U) {
     status_check(qllm_rms_norm_concat_batch(
         mtp_embedding_, mtp_.embedding_norm, previous_hidden, mtp_.hidden_norm,
@@ -2675,15 +2681,37 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                hipMemcpyDeviceToDevice, hip_stream),
               "assemble MTP target hidden batch");
   }
-  project(mtp_.fusion.descriptor, mtp_fusion_input_,
-          std::size_t{rows} * 2U * half_bytes, mtp_hidden_, nullptr, rows);
-
+  // The projections onto the hidden width have few rows for the GPU: with bf16
+  // activations their K is cut over workgroups and the norm that follows adds
+  // the partial sums to the residual stream (as in the target's layers).
+  // sum = residual + matrix * input, normalized_ = RMSNorm(sum) under `weight`.
+  const auto project_and_normalise =
+      [&](const qllm_fp4_matrix& matrix, const std::uint16_t* bf16,
+          std::size_t bf16_bytes, const float* residual, float* sum,
+          const float* weight) {
+        if (!q8 && projection_splits_ > 1U && matrix.layout == QLLM_LAYOUT_TILED &&
+            matrix.padded_columns / 64U >= projection_splits_ &&
+            g_.hidden <= 16384U && g_.hidden % 4U == 0U) {
+          status_check(qllm_fp4_gemm_bf16_partial(&matrix, bf16, bf16_bytes,
+                                                  projection_partials_,
+                                                  projection_splits_, rows, stream));
+          status_check(qllm_rms_norm_partials_batch(
+              residual, sum, projection_partials_, projection_splits_, weight,
+              normalized_, rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm,
+              stream));
+          return;
+        }
+        project(matrix, bf16, bf16_bytes, sum, residual, rows);
+        normalise(sum, weight, rows);
+      };
   // one transformer block over its own Q8 cache (run_full_attention + run_ffn)
   const auto& layer = mtp_.layer;
   const std::uint32_t query_stride = g_.head_dim * (g_.output_gated ? 2U : 1U);
   const std::size_t hidden_bytes = std::size_t{rows} * g_.hidden * 2U;
   const std::uint32_t kv_rows = g_.kv_heads * g_.head_dim;
-  normalise(mtp_hidden_, layer.input_norm, rows);
+  project_and_normalise(mtp_.fusion.descriptor, mtp_fusion_input_,
+                        std::size_t{rows} * 2U * half_bytes, nullptr, mtp_hidden_,
+                        layer.input_norm);
   const qllm_gemm_segment projections[3] = {
       {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
       {key_, kv_rows, QLLM_OUT_F32},
@@ -2737,10 +2765,9 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   launch.device_positions = deferred_positions ? mtp_positions_ : nullptr;
   status_check(qllm_attention_paged_q8(&launch));
   if (q8) enqueue_quantise(activation_f32_, rows, g_.query_heads * g_.head_dim);
-  project(layer.output.descriptor, attention_,
-          std::size_t{rows} * g_.query_heads * g_.head_dim * 2U, mtp_hidden_,
-          mtp_hidden_, rows);
-  normalise(mtp_hidden_, layer.post_attention_norm, rows);
+  project_and_normalise(layer.output.descriptor, attention_,
+                        std::size_t{rows} * g_.query_heads * g_.head_dim * 2U,
+                        mtp_hidden_, mtp_hidden_, layer.post_attention_norm);
   if (q8) {
     status_check(qllm_fp4_swiglu_q8(&layer.gate.descriptor, &layer.up.descriptor,
                                     q8_, q8_scales_, activation_f32_, rows,
@@ -2753,17 +2780,20 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
   }
   // a single-row pass leaves its hidden state where the next pass reads it
   const bool retain_in_place = rows == 1U;
-  project(layer.down.descriptor, activation_,
-          std::size_t{rows} * g_.intermediate * 2U,
-          retain_in_place ? mtp_last_hidden_ : mtp_hidden_, mtp_hidden_, rows);
+  float* const last_sum = retain_in_place ? mtp_last_hidden_ : mtp_hidden_;
+  const auto retain_last_row = [&] {
+    if (!retain_in_place)
+      hip_check(hipMemcpyAsync(mtp_last_hidden_,
+                               mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
+                               g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
+                "retain final MTP hidden state");
+  };
   // draft head: the last row, draft norm, the head's first draft_vocabulary rows
-  if (!retain_in_place)
-    hip_check(hipMemcpyAsync(mtp_last_hidden_,
-                             mtp_hidden_ + std::size_t{rows - 1U} * g_.hidden,
-                             g_.hidden * 4U, hipMemcpyDeviceToDevice, hip_stream),
-              "retain final MTP hidden state");
-  normalise(mtp_last_hidden_, mtp_.draft_norm, 1U);
   if (q8) {
+    project(layer.down.descriptor, activation_,
+            std::size_t{rows} * g_.intermediate * 2U, last_sum, mtp_hidden_, rows);
+    retain_last_row();
+    normalise(mtp_last_hidden_, mtp_.draft_norm, 1U);
     project(mtp_.head_prefix, normalized_, std::size_t{g_.hidden} * 2U, mtp_logits_,
             nullptr, 1U);
     status_check(qllm_argmax_batch(mtp_logits_, g_.draft_vocabulary, 1U, mtp_argmax_,
@@ -2774,10 +2804,18 @@ void Mi355DenseFp4Provider::enqueue_mtp(std::uint32_t rows,
                                         g_.draft_depth, rows, mtp_positions_, stream));
     return;
   }
+  // (every row goes through the norm that finishes the down projection; the
+  // head reads the last)
+  project_and_normalise(layer.down.descriptor, activation_,
+                        std::size_t{rows} * g_.intermediate * 2U, mtp_hidden_,
+                        last_sum, mtp_.draft_norm);
+  retain_last_row();
   // the draft head, its arg-max and the hand-over to the next pass
   const qllm_rollout_step advance{mtp_tokens_, mtp_draft_tokens_, g_.draft_depth, rows,
                                   mtp_positions_};
-  enqueue_head_projection(mtp_.head_prefix, mtp_logits_, 1U, mtp_argmax_,
+  enqueue_head_projection(mtp_.head_prefix,
+                          normalized_ + std::size_t{rows - 1U} * g_.hidden,
+                          mtp_logits_, 1U, mtp_argmax_,
                           deferred_positions ? &advance : nullptr);
 }
 
@@ -2800,7 +2838,10 @@ void Mi355DenseFp4Provider::launch_mtp_graph(std::uint32_t rows, bool chained,
     hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal),
               "begin proposer capture");
     try {
-      enqueue_mtp(rows, chained ? mtp_last_hidden_ : hidden_, true, 0U, true);
+      // the pass over the target's hidden rows takes the tokens the verify
+      // step emitted: it also marks them present
+      enqueue_mtp(rows, chained ? mtp_last_hidden_ : hidden_, true, 0U, true,
+                  chained ? nullptr : presence_);
       for (std::uint32_t pass = 1; pass < drafts; ++pass)
         enqueue_mtp(1U, mtp_last_hidden_, true, 0U, true);
     } catch (...) {
@@ -3095,9 +3136,15 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
               300U));
 
     const auto positions_advanced = static_cast<std::uint32_t>(accepted + 1U);
-    {
+    const bool future_exact =
+        invocation.position + positions_advanced + 1U < invocation.context_limit;
+    // The captured passes select their drafts on the device without the
+    // presence bytes; a request with a penalty takes the uncaptured ones.
+    const bool captured_proposal =
+        mtp_.ready && future_exact && use_graphs_ && penalty == 0.0;
+    if (!captured_proposal) {
       // accepted drafts and the next token are emitted tokens from here on
-      // (:11261-11270)
+      // (:11261-11270); the captured proposer pass marks them itself
       std::vector<std::uint32_t> emitted_now;
       for (std::size_t index = 0; index < accepted; ++index)
         emitted_now.push_back(state->draft_predictions[index].token);
@@ -3112,14 +3159,10 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
       for (std::size_t index = 0; index < accepted; ++index)
         mtp_tokens.push_back(state->draft_predictions[index].token);
       mtp_tokens.push_back(next_token);
-      const bool future_exact = invocation.position + positions_advanced + 1U <
-                                invocation.context_limit;
       state->mtp_length = invocation.position;
       state->draft_valid = false;
       state->draft_predictions.clear();
-      // The captured passes select their drafts on the device without the
-      // presence bytes; a request with a penalty takes the uncaptured ones.
-      if (future_exact && use_graphs_ && penalty == 0.0) {
+      if (captured_proposal) {
         propose_with_graphs(*state, mtp_tokens, invocation.request,
                             invocation.context_limit);
       } else {

@@ -312,7 +312,8 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void enqueue_ffn_block(std::uint32_t index, std::uint32_t rows,
                          bool leave_partials);
   void enqueue_head(std::uint32_t first_row, std::uint32_t rows);
-  void enqueue_head_projection(const qllm_fp4_matrix& head, float* logits,
+  void enqueue_head_projection(const qllm_fp4_matrix& head,
+                               const std::uint16_t* input, float* logits,
                                std::uint32_t rows, std::uint32_t* tokens,
                                const qllm_rollout_step* advance);
   // run_head with a request (dense_fp4_provider.cpp:8433-8517): presence
@@ -394,7 +395,7 @@ class Mi355DenseFp4Provider final : public er::IOperationProvider {
   void ensure_prefill_workspace(std::uint32_t rows);
   void enqueue_mtp(std::uint32_t rows, const float* previous_hidden,
                    bool produce_logits, std::uint32_t cache_position,
-                   bool deferred_positions);
+                   bool deferred_positions, std::uint8_t* mark_emitted = nullptr);
   void enqueue_mtp_prefill(std::span<const std::uint32_t> tokens,
                            std::uint32_t position);
   void launch_mtp_graph(std::uint32_t rows, bool chained,

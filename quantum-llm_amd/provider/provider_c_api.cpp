@@ -15,8 +15,6 @@
 #include "dense_fp4_provider.hpp"
 #include "dense_record.hpp"
 #include "expert/runtime/sha256.hpp"
-#include "descriptor_dump.hpp"
-#include "registry_probe.hpp"
 
 namespace er = expert::runtime;
 
@@ -758,27 +756,6 @@ struct qllm_artifact {
   er::MappedModelTensorStore store;
 };
 
-namespace {
-
-int32_t copy_text(const std::string& text, char* buffer, size_t capacity,
-                  size_t* bytes) {
-  if (bytes) *bytes = text.size();
-  if (buffer && capacity) {
-    const size_t count = std::min(text.size(), capacity - 1U);
-    std::memcpy(buffer, text.data(), count);
-    buffer[count] = '\0';
-  }
-  return QLLM_OK;
-}
-
-er::Sha256Digest digest_of(const uint8_t* bytes) {
-  er::Sha256Digest digest{};
-  if (bytes) std::memcpy(digest.data(), bytes, digest.size());
-  return digest;
-}
-
-}  // namespace
-
 extern "C" int32_t qllm_sha256(const void* data, size_t bytes, uint8_t* digest) {
   if ((!data && bytes) || !digest)
     return fail(QLLM_INVALID_ARGUMENT, "SHA-256 arguments are invalid");
@@ -796,47 +773,6 @@ extern "C" int32_t qllm_sha256_portable(const void* data, size_t bytes,
       er::sha256_portable({static_cast<const std::byte*>(data), bytes});
   std::memcpy(digest, result.data(), result.size());
   return QLLM_OK;
-}
-
-extern "C" int32_t qllm_model_descriptor_parse(
-    const char* text, size_t text_bytes, const uint8_t* content_sha256,
-    uint64_t namespace_base, char* dump, size_t capacity, size_t* dump_bytes) {
-  if (!text && text_bytes)
-    return fail(QLLM_INVALID_ARGUMENT, "model program text is null");
-  const auto parsed = er::parse_model_descriptor_artifact(
-      {text, text_bytes}, digest_of(content_sha256), namespace_base);
-  if (!parsed.status.ok()) return from_status(parsed.status);
-  return copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
-                   dump_bytes);
-}
-
-extern "C" int32_t qllm_model_program_bind(
-    const char* text, size_t text_bytes, const uint8_t* content_sha256,
-    uint64_t namespace_base, const char* providers, int32_t executable,
-    char* dump, size_t capacity, size_t* dump_bytes) {
-  if ((!text && text_bytes) || !providers)
-    return fail(QLLM_INVALID_ARGUMENT, "model program or providers are null");
-  try {
-    return copy_text(
-        qllm::dump::bind_report({text, text_bytes}, digest_of(content_sha256),
-                                namespace_base, providers, executable != 0),
-        dump, capacity, dump_bytes);
-  } catch (const std::exception& error) {
-    return fail(QLLM_INTERNAL, error.what());
-  }
-}
-
-extern "C" int32_t qllm_model_descriptor_load(
-    const char* path, uint64_t expected_bytes, const uint8_t* expected_sha256,
-    const uint8_t* content_sha256, uint64_t namespace_base, char* dump,
-    size_t capacity, size_t* dump_bytes) {
-  if (!path) return fail(QLLM_INVALID_ARGUMENT, "model program path is null");
-  const auto parsed = er::load_model_descriptor_artifact(
-      path, expected_bytes, digest_of(expected_sha256), digest_of(content_sha256),
-      namespace_base);
-  if (!parsed.status.ok()) return from_status(parsed.status);
-  return copy_text(qllm::dump::model_descriptor(parsed.descriptor), dump, capacity,
-                   dump_bytes);
 }
 
 extern "C" int32_t qllm_artifact_open(const char* root, uint32_t mtp_draft_depth,
@@ -864,17 +800,6 @@ extern "C" int32_t qllm_artifact_open(const char* root, uint32_t mtp_draft_depth
 }
 
 extern "C" void qllm_artifact_close(qllm_artifact* artifact) { delete artifact; }
-
-extern "C" int32_t qllm_artifact_dump(const qllm_artifact* artifact, char* dump,
-                                      size_t capacity, size_t* dump_bytes) {
-  if (!artifact) return fail(QLLM_INVALID_ARGUMENT, "artifact is null");
-  try {
-    return copy_text(qllm::dump::model_artifact(artifact->artifact), dump, capacity,
-                     dump_bytes);
-  } catch (const std::exception& error) {
-    return fail(QLLM_INTERNAL, error.what());
-  }
-}
 
 extern "C" int32_t qllm_artifact_tensor(qllm_artifact* artifact, const char* name,
                                         int32_t check_header, const void** record,

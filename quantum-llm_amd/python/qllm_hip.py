@@ -119,8 +119,9 @@ SIGNATURES = {
     "qllm_rms_norm_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_residual_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_partials_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
-    "qllm_rms_norm_concat_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_concat_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_float, c_int32, c_void_p, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_silu_product": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),
     "qllm_q4h_layer_bytes": (c_size_t, [c_uint32, c_uint32, c_uint32]),

@@ -75,12 +75,8 @@ SIGNATURES = {
     "qllm_provider_prefill": (c_int32, [c_void_p, c_void_p, c_uint32, c_uint32, POINTER(c_uint32)]),
     "qllm_sha256": (c_int32, [c_void_p, c_size_t, c_void_p]),
     "qllm_sha256_portable": (c_int32, [c_void_p, c_size_t, c_void_p]),
-    "qllm_model_descriptor_parse": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
-    "qllm_model_program_bind": (c_int32, [c_char_p, c_size_t, c_char_p, c_uint64, c_char_p, c_int32, c_char_p, c_size_t, POINTER(c_size_t)]),
-    "qllm_model_descriptor_load": (c_int32, [c_char_p, c_uint64, c_char_p, c_char_p, c_uint64, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_artifact_open": (c_int32, [c_char_p, c_uint32, c_int32, POINTER(c_void_p)]),
     "qllm_artifact_close": (None, [c_void_p]),
-    "qllm_artifact_dump": (c_int32, [c_void_p, c_char_p, c_size_t, POINTER(c_size_t)]),
     "qllm_artifact_tensor": (c_int32, [c_void_p, c_char_p, c_int32, POINTER(c_void_p), POINTER(c_uint64)]),
 }
 

@@ -404,8 +404,10 @@ def test_lookup_with_two_norms_equals_the_three_launches(device, scheme, rows, e
     d = [gu.device_tensor(x, device) for x in (codes, scales, tokens, hidden, wa, wb)]
     table = qh.fp4_matrix(d[0], d[1], V, elements, elements, scheme)
     fused = torch.zeros((rows, 2 * elements), dtype=torch.bfloat16, device=device)
+    presence = torch.zeros(V, dtype=torch.uint8, device=device)
     qh.call("qllm_rms_norm_concat_embedding_batch", table, qh.ptr(d[2]), qh.ptr(d[4]),
-            qh.ptr(d[3]), qh.ptr(d[5]), qh.ptr(fused), rows, 1e-6, 1, None)
+            qh.ptr(d[3]), qh.ptr(d[5]), qh.ptr(fused), rows, 1e-6, 1, qh.ptr(presence),
+            None)
     looked_up = torch.zeros((rows, elements), device=device)
     qh.call("qllm_fp4_embedding_batch", table, qh.ptr(d[2]), qh.ptr(looked_up), rows, None)
     apart = torch.zeros_like(fused)
@@ -413,6 +415,10 @@ def test_lookup_with_two_norms_equals_the_three_launches(device, scheme, rows, e
             qh.ptr(d[5]), qh.ptr(apart), rows, elements, 1e-6, 1, None)
     torch.cuda.synchronize()
     assert torch.equal(fused, apart)
+    # the batch's tokens, and only they, are marked present
+    marked = np.zeros(V, dtype=np.uint8)
+    marked[tokens] = 1
+    assert np.array_equal(presence.cpu().numpy(), marked)
     embedding = ol.fp4_embedding(codes, scales, scheme, elements, elements, tokens)
     want = ol.rms_norm_rows(embedding, wa, 1e-6, True)
     got = fused.float().cpu().numpy()[:, :elements]
@@ -421,10 +427,52 @@ def test_lookup_with_two_norms_equals_the_three_launches(device, scheme, rows, e
     bad = qh.fp4_matrix(d[0], d[1], V, elements, elements, scheme)
     bad.layout = 1
     for arguments in ((bad, qh.ptr(d[2]), qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
-                       qh.ptr(fused), rows, 1e-6, 1, None),
+                       qh.ptr(fused), rows, 1e-6, 1, None, None),
                       (table, None, qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
-                       qh.ptr(fused), rows, 1e-6, 1, None),
+                       qh.ptr(fused), rows, 1e-6, 1, None, None),
                       (table, qh.ptr(d[2]), qh.ptr(d[4]), qh.ptr(d[3]), qh.ptr(d[5]),
-                       qh.ptr(fused), 0, 1e-6, 1, None)):
+                       qh.ptr(fused), 0, 1e-6, 1, None, None)):
         with pytest.raises(qh.QllmError):
             qh.call("qllm_rms_norm_concat_embedding_batch", *arguments)
+
+
+def test_norm_of_partial_sums_with_and_without_a_residual(device):
+    """qllm_rms_norm_partials_batch: the sum goes where it is told (in place, or
+    elsewhere with the residual left alone, or from zero without a residual),
+    bit-equal to qllm_rms_norm_residual_batch on the same operands."""
+    rng = np.random.default_rng(12)
+    rows, elements, count = 5, 5120, 3
+    hidden = rng.standard_normal((rows, elements)).astype(np.float32)
+    partials = rng.standard_normal((count, rows, elements)).astype(np.float32)
+    weight = (0.1 * rng.standard_normal(elements)).astype(np.float32)
+    d_partials, d_weight = gu.device_tensor(partials, device), gu.device_tensor(weight, device)
+
+    def run(residual, separate_sum):
+        d_residual = None if residual is None else gu.device_tensor(residual, device)
+        d_sum = (torch.full((rows, elements), 7.0, device=device)
+                 if separate_sum or d_residual is None else d_residual)
+        out = torch.zeros((rows, elements), dtype=torch.bfloat16, device=device)
+        qh.call("qllm_rms_norm_partials_batch", qh.ptr(d_residual), qh.ptr(d_sum),
+                qh.ptr(d_partials), count, qh.ptr(d_weight), qh.ptr(out), rows, elements,
+                1e-6, 1, None)
+        torch.cuda.synchronize()
+        return d_residual, d_sum.cpu().numpy(), out.float().cpu().numpy()
+
+    reference = gu.device_tensor(hidden, device)
+    want_out = torch.zeros((rows, elements), dtype=torch.bfloat16, device=device)
+    qh.call("qllm_rms_norm_residual_batch", qh.ptr(reference), qh.ptr(d_partials), count,
+            qh.ptr(d_weight), qh.ptr(want_out), rows, elements, 1e-6, 1, None)
+    torch.cuda.synchronize()
+    want_sum = reference.cpu().numpy()
+    assert np.array_equal(want_sum, ((hidden + partials[0]) + partials[1]) + partials[2])
+    for separate in (False, True):
+        residual, got_sum, got_out = run(hidden, separate)
+        assert np.array_equal(got_sum, want_sum)
+        assert np.array_equal(got_out, want_out.float().cpu().numpy())
+        if separate:
+            assert np.array_equal(residual.cpu().numpy(), hidden)
+    _, got_sum, got_out = run(None, True)
+    want = (partials[0] + partials[1]) + partials[2]
+    assert np.array_equal(got_sum, want)
+    normed = ol.rms_norm_rows(want, weight, 1e-6, True)
+    assert (np.abs(got_out - normed) <= np.abs(normed) * 2.0 ** -8 + 2e-5).all()
