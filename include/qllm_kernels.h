@@ -793,7 +793,10 @@ int32_t qllm_argmax_batch(const float* values, uint32_t count,
  * <= 8192 (qllm_argmax_workspace_bytes(count, batch) <=
  * qllm_argmax_static_capacity_bytes()); larger requests fail with
  * QLLM_INVALID_ARGUMENT.  Every call on a GPU shares that GPU's array: calls
- * that overlap on one GPU (different streams or threads) race. */
+ * that overlap on one GPU (different streams, threads or provider instances)
+ * race, and nothing detects it.  The first call on a device looks the array's
+ * address up and must be made outside stream capture; later calls only launch
+ * kernels. */
 size_t qllm_argmax_static_capacity_bytes(void);
 int32_t qllm_argmax_batch_static(const float* values, uint32_t count,
                                  uint32_t batch, uint32_t* output,

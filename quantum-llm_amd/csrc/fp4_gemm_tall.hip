@@ -20,11 +20,16 @@
 //    weight times an 11-bit scale).  It is split into two binary16 values,
 //    hi = the product rounded to binary16 and lo = its rounding error, which
 //    a fused multiply-add returns exactly; they go through the matrix cores
-//    one after the other into the same F32 accumulator; the bf16 activations are converted to binary16 (exact
-//    between 6.1e-5 and 65504 in magnitude - the range of a decoder's
-//    normalised activations; beyond it they saturate or lose low bits).  The
-//    products are therefore the exact ones, as in the small-batch kernel, at
-//    twice the matrix instructions.
+//    one after the other into the same F32 accumulator; the bf16 activations
+//    are converted to binary16 (exact between 6.1e-5 and 65504 in magnitude -
+//    the range of a decoder's normalised activations; beyond it they saturate
+//    or lose low bits).  The products are the exact ones, as in the small-batch
+//    kernel, at twice the matrix instructions - for block scales between 2^-13
+//    (1.22e-4) and 10917 in magnitude: both halves are formed in binary16, so
+//    a weight of 6 under a larger scale overflows it (the small-batch kernel
+//    multiplies in F32 and stays finite), and under a smaller scale the low
+//    half has bits below 2^-24 and is cut short (a relative error of up to
+//    2^-11 in that weight).  Checkpoint scales lie well inside.
 #include "common.hpp"
 
 #include <type_traits>

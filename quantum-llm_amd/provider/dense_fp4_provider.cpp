@@ -1071,6 +1071,10 @@ std::uint32_t Mi355DenseFp4Provider::select_head_token(
                              hipMemcpyDeviceToHost, stream),
               "copy dense FP4 greedy token");
     hip_check(hipStreamSynchronize(stream), "copy dense FP4 greedy token");
+    // a row without a finite logit selects nothing (0xffffffff): reported
+    // before the presence bytes or the caller's state change
+    if (selected >= g_.vocabulary)
+      throw std::runtime_error("head logits have no finite maximum");
   } else {
     // the penalty, if any, has been applied: the distribution is taken from
     // the row as it stands
@@ -3096,6 +3100,11 @@ er::ExactDecodeExecutionHandle Mi355DenseFp4Provider::execute_exact_decode(
                                hipMemcpyDeviceToHost, stream),
                 "copy exact greedy tokens");
       hip_check(hipStreamSynchronize(stream), "copy exact greedy tokens");
+      // a row without a finite logit selects nothing (0xffffffff): reported
+      // here, before the proposer or the request state is touched
+      for (std::uint32_t row = 0; row < rows; ++row)
+        if (staging_->download[row] >= g_.vocabulary)
+          throw std::runtime_error("target logits have no finite maximum");
       for (std::uint32_t row = 0; row < rows; ++row)
         target_distributions.push_back({{{staging_->download[row], 1.0}}});
     } else if (request_parameter(invocation.request, "sampling_top_k") != 0U) {

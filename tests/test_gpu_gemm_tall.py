@@ -76,6 +76,30 @@ def test_tall_gemm_rows_equal_the_small_batch_kernel(device, scheme):
     gu.assert_close(big, small, rtol=2e-3, atol=2e-4, what="tall vs small-batch rows")
 
 
+def test_tall_gemm_binary16_scales_at_the_ends_of_their_exact_range(device):
+    """Block scales of 2^-13 and of 10912 (6 x 10912 = 65472 is the largest
+    product binary16 holds): inside that range weight x scale is carried
+    exactly by the two binary16 halves, so the tall kernel agrees with the
+    oracle as tightly as for ordinary scales.  Scales below the range (6e-5)
+    lose the low half's last bits: within 2^-11 of each product."""
+    rng = np.random.default_rng(21)
+    rows, padded, batch = 256, 1024, 130
+    codes, _ = synth.fp4_matrix(rng, rows, padded, ol.SCALE_F16_BLOCK16)
+    act = ol.bf16_round(rng.standard_normal((batch, padded)).astype(np.float32))
+    for low, high, tolerance in ((2.0 ** -13, 10912.0, 2e-6), (6e-5, 8192.0, 2.0 ** -11)):
+        values = np.where(rng.random((rows, padded // 16)) < 0.5, low, high)
+        scales = values.astype(np.float16).view(np.uint16)
+        want = ol.fp4_linear_f64(codes, scales, ol.SCALE_F16_BLOCK16, rows, padded, act)
+        got = tall(device, codes, scales, ol.SCALE_F16_BLOCK16, rows, padded, act)
+        assert np.isfinite(got).all()
+        # the error bound is relative to the sum of |products|, not to the result
+        magnitude = ol.fp4_linear_f64(codes & 0x77, scales, ol.SCALE_F16_BLOCK16, rows, padded,
+                                      np.abs(act))
+        assert (np.abs(got - want) <= tolerance * np.sqrt(padded) * magnitude + 1e-30).all()
+        small = gu.gemm(device, codes, scales, ol.SCALE_F16_BLOCK16, rows, padded, act[:5])
+        assert (np.abs(small - want[:5]) <= 2e-6 * np.sqrt(padded) * magnitude[:5] + 1e-30).all()
+
+
 def test_tall_split_outputs(device):
     rng = np.random.default_rng(9)
     scheme, padded, batch = ol.SCALE_F16_BLOCK16, 1024, 140

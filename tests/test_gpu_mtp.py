@@ -257,6 +257,39 @@ def test_draft_logits_without_a_finite_maximum_are_reported(device):
     provider.close()
 
 
+def test_target_logits_without_a_finite_maximum_leave_the_request_as_it_was(device):
+    """A final norm full of NaN makes every target logit NaN: the rows' arg-max
+    selects no token (0xffffffff).  The greedy verify step reports that before
+    it touches the proposer or the request - the drafts it was given are still
+    there and no proposer pass ran - and so does the head of a prompt."""
+    rng = np.random.default_rng(6)
+    c = CONFIGS["baseline"]
+    model = step_oracle.TinyModel(
+        rng, 256, 512, 2, 8, 2, c["head_dim"], 256, c["scheme"],
+        output_gated=c["output_gated"], qk_norm=c["qk_norm"],
+        zero_centered=c["zero_centered"], rotary_dim=c["rotary_dim"])
+    model.final_norm[:] = np.nan
+    provider = step_oracle.build_provider(model, qp, mtp=True,
+                                          draft_vocabulary=DRAFT_VOCABULARY)
+    provider.run_target(rng.integers(0, 256, 5).astype(np.uint32), 0)
+    provider.begin_request(temperature_ppm=0)
+    provider.synchronize(3, 5)        # the proposer has its own norms: drafts exist
+    drafts = provider.drafts()
+    assert len(drafts) == 4
+    passes = provider.telemetry("provider_mtp_passes")
+    for attempt in range(2):          # the same call fails the same way again
+        with pytest.raises(qp.ProviderError) as error:
+            provider.verify(3, 5, 256)
+        assert "target logits have no finite maximum" in str(error.value)
+        assert provider.drafts() == drafts
+        assert provider.telemetry("provider_mtp_passes") == passes
+        assert provider.telemetry("provider_exact_calls") == 0
+    with pytest.raises(qp.ProviderError) as error:
+        provider.prefill(rng.integers(0, 256, 7).astype(np.uint32), 0)
+    assert "head logits have no finite maximum" in str(error.value)
+    provider.close()
+
+
 def test_rollout_stops_at_the_context_limit(device):
     rng, model, provider = make("baseline", 37, max_context=64)
     V = model.vocabulary
