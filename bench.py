@@ -27,8 +27,8 @@ sys.path.insert(0, os.path.join(ROOT, "quantum-llm_amd", "python"))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the fused gate/up kernel moves, from the FETCH_SIZE and
 # WRITE_SIZE hardware counters scaled by a 256 MiB copy (summary and commands
-# in profiles/hot_kernels_hbm_traffic.md); 1.04x the algorithmic bytes.
-GATE_UP_TRAFFIC_BYTES = 116230823
+# in profiles/hot_kernels_hbm_traffic.md); 1.01x the algorithmic bytes.
+GATE_UP_TRAFFIC_BYTES = 112914399
 
 MODEL = dict(hidden=5120, intermediate=17408, layers=64, query_heads=64, kv_heads=8,
              head_dim=128, rotary_dim=128, vocabulary=151936, rope_theta=1.0e6,

@@ -348,33 +348,43 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
   const uint32_t chunks = (split + 1u) * all_chunks / splits - first_chunk_of_split;
   const uint32_t my_chunks =
       chunks > wave ? (chunks - wave + WAVES - 1u) / WAVES : 0u;
-  // Prefetch is unconditional: indices past the wave's last chunk are clamped
-  // to it (loaded again and ignored), which keeps the load/wait pattern of the
-  // unrolled ring static.
+  // Prefetch is unconditional, which keeps the load/wait pattern of the
+  // unrolled ring static: an index past the wave's last chunk fetches the
+  // first 16 bytes of the activations instead, in every lane (one line that
+  // every workgroup keeps in L2; the value is ignored).  Fetching the last
+  // chunk again would go back to HBM for it: streamed lines do not stay.
   const uint32_t last_index = my_chunks ? my_chunks - 1u : 0u;
 
   uint4 codes[PF][TILES];
   uint32_t scales[PF][TILES][SCALE_WORDS];
   uint4 activation[PF];
   auto issue = [&](int slot, uint32_t index) {
-    const uint32_t chunk = first_chunk_of_split + wave + index * WAVES;   // uniform
+    const bool past = index > last_index;                                 // uniform
+    const uint32_t chunk =
+        first_chunk_of_split + wave + min(index, last_index) * WAVES;     // uniform
+    const uint32_t weight_offset = past ? 0u : weight_lane;
+    const uint32_t scale_offset[2] = {past ? 0u : scale_lane[0],
+                                      past ? 0u : scale_lane[1]};
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-      codes[slot][t] = load_stream16(
-          weight_base[t] + static_cast<size_t>(chunk) * weight_step + weight_lane);
+      const uint8_t* weight_chunk =
+          past ? activation_base
+               : weight_base[t] + static_cast<size_t>(chunk) * weight_step;
+      codes[slot][t] = load_stream16(weight_chunk + weight_offset);
       const uint8_t* scale_chunk =
-          scale_base[t] + static_cast<size_t>(chunk) * scale_step;
+          past ? activation_base
+               : scale_base[t] + static_cast<size_t>(chunk) * scale_step;
       if constexpr (TILED && F16) {
-        const uint2 v = load_stream8(scale_chunk + scale_lane[0]);
+        const uint2 v = load_stream8(scale_chunk + scale_offset[0]);
         scales[slot][t][0] = v.x;
         scales[slot][t][1] = v.y;
       } else if constexpr (TILED) {
         scales[slot][t][0] =
-            *reinterpret_cast<const uint32_t*>(scale_chunk + scale_lane[0]);
+            *reinterpret_cast<const uint32_t*>(scale_chunk + scale_offset[0]);
       } else if constexpr (F16) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          const uint2 v = load_stream8(scale_chunk + scale_lane[j]);
+          const uint2 v = load_stream8(scale_chunk + scale_offset[j]);
           scales[slot][t][2 * j] = v.x;
           scales[slot][t][2 * j + 1] = v.y;
         }
@@ -382,7 +392,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           scales[slot][t][j] =
-              *reinterpret_cast<const uint16_t*>(scale_chunk + scale_lane[j]);
+              *reinterpret_cast<const uint16_t*>(scale_chunk + scale_offset[j]);
       }
     }
     activation[slot] = *reinterpret_cast<const uint4*>(
@@ -391,8 +401,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
 
   if (my_chunks) {
 #pragma unroll
-    for (int slot = 0; slot < PF; ++slot)
-      issue(slot, min(static_cast<uint32_t>(slot), last_index));
+    for (int slot = 0; slot < PF; ++slot) issue(slot, static_cast<uint32_t>(slot));
 
     for (uint32_t base = 0; base < my_chunks; base += PF) {
 #pragma unroll
@@ -407,7 +416,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp4_gemm_mfma_kernel(
           for (int w = 0; w < SCALE_WORDS; ++w) s[t][w] = scales[slot][t][w];
         }
         const uint4 x = activation[slot];
-        issue(slot, min(index + PF, last_index));
+        issue(slot, index + PF);
         if (index >= my_chunks) continue;
 
         // activation pieces -> wave-private ring -> A fragments
