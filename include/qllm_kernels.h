@@ -192,6 +192,14 @@ int32_t qllm_fp4_gemm_q8_split(const qllm_fp4_matrix* matrix, const int8_t* inpu
                                uint32_t segment_count, uint32_t batch,
                                void* workspace, size_t workspace_bytes,
                                void* stream);
+/* qllm_fp4_gemm_q8 with K cut over k_splits workgroups per tile, as
+ * qllm_fp4_gemm_bf16_partial cuts it: partials f32 [k_splits][batch][rows],
+ * each already times the row's activation scale; the consumer adds them in
+ * index order (qllm_rms_norm_partials_q8_batch does).  Against the one-sum
+ * form the F32 additions are regrouped, nothing else. */
+int32_t qllm_fp4_gemm_q8_partial(const qllm_fp4_matrix* matrix, const int8_t* input,
+                                 const float* input_scales, float* partials,
+                                 uint32_t k_splits, uint32_t batch, void* stream);
 int32_t qllm_fp4_swiglu_q8(const qllm_fp4_matrix* gate, const qllm_fp4_matrix* up,
                            const int8_t* input, const float* input_scales,
                            float* output, uint32_t batch, void* workspace,
@@ -337,6 +345,17 @@ int32_t qllm_rms_norm_partials_batch(const float* residual, float* sum,
                                      uint32_t rows, uint32_t elements,
                                      float epsilon, int32_t zero_centered,
                                      void* stream);
+
+/* qllm_rms_norm_partials_batch with the norm's output in per-row Q8 form, as
+ * qllm_rms_norm_q8_batch leaves it (normalize_rows + quantize_rows,
+ * dense_fp4_provider.cpp:5740-5778, 5983-5992). */
+int32_t qllm_rms_norm_partials_q8_batch(const float* residual, float* sum,
+                                        const float* partials,
+                                        uint32_t partial_count, const float* weight,
+                                        int8_t* output_q8, float* scales,
+                                        uint32_t rows, uint32_t elements,
+                                        float epsilon, int32_t zero_centered,
+                                        void* stream);
 
 /* Two normalisations into one bf16 batch: output row r, of 2 * elements
  * columns, is [RMSNorm(first[r]) | RMSNorm(second[r])], each half with its own

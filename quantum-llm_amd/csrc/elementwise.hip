@@ -402,6 +402,21 @@ __global__ __launch_bounds__(1024) void rms_norm_q8_kernel(
                     output_q8 + row * elements, scales + row);
 }
 
+// The same on a row that is first completed from K-split partial sums
+// (rms_norm_residual_kernel below, with the Q8 output of rms_norm_q8_kernel).
+__global__ __launch_bounds__(1024) void rms_norm_residual_q8_kernel(
+    const float* residual, float* sum, const float* partials,
+    uint32_t partial_count, const float* weight, int8_t* output_q8, float* scales,
+    uint32_t elements, float epsilon, bool zero_centered) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  rms_norm_row_wide(residual ? residual + row * elements : nullptr, weight, nullptr,
+                    nullptr, 0u, elements, epsilon, zero_centered, scratch,
+                    partials + row * elements, partial_count,
+                    static_cast<size_t>(gridDim.x) * elements, sum + row * elements,
+                    output_q8 + row * elements, scales + row);
+}
+
 // sum[r] = residual[r] + partials[0][r] + ... + partials[count-1][r] (from zero
 // without a residual), then its RMSNorm in bf16: the residual add of a
 // projection whose K was cut over workgroups (qllm_fp4_gemm_bf16_partial)
@@ -583,6 +598,25 @@ extern "C" int32_t qllm_rms_norm_q8_batch(const float* input, const float* weigh
   rms_norm_q8_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
       input, weight, output_q8, scales, elements, epsilon, zero_centered != 0);
   return launched("Q8 RMSNorm");
+}
+
+extern "C" int32_t qllm_rms_norm_partials_q8_batch(
+    const float* residual, float* sum, const float* partials,
+    uint32_t partial_count, const float* weight, int8_t* output_q8, float* scales,
+    uint32_t rows, uint32_t elements, float epsilon, int32_t zero_centered,
+    void* stream) {
+  const auto aligned = [](const void* pointer) {
+    return reinterpret_cast<uintptr_t>(pointer) % 16u == 0u;
+  };
+  if (!sum || !partials || !partial_count || partial_count > 16u || !output_q8 ||
+      !scales || !rows || rows > 65535u || !elements || elements % 4u != 0u ||
+      elements > 16384u || !(epsilon > 0.0f) || !aligned(residual) || !aligned(sum) ||
+      !aligned(partials) || !aligned(output_q8) || (weight && !aligned(weight)))
+    return fail(QLLM_INVALID_ARGUMENT, "invalid Q8 RMSNorm of partial sums");
+  rms_norm_residual_q8_kernel<<<rows, 1024, 0, as_stream(stream)>>>(
+      residual, sum, partials, partial_count, weight, output_q8, scales, elements,
+      epsilon, zero_centered != 0);
+  return launched("Q8 RMSNorm of partial sums");
 }
 
 extern "C" int32_t qllm_convert_f32_to_bf16_batch(

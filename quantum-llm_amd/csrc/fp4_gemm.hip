@@ -1312,6 +1312,21 @@ extern "C" int32_t qllm_fp4_gemm_q8(const qllm_fp4_matrix* matrix,
   return launch_mfma(args, kSchemeUe8m0, true, batch, false, as_stream(stream));
 }
 
+extern "C" int32_t qllm_fp4_gemm_q8_partial(const qllm_fp4_matrix* matrix,
+                                            const int8_t* input,
+                                            const float* input_scales,
+                                            float* partials, uint32_t k_splits,
+                                            uint32_t batch, void* stream) {
+  if (!q8_gemm_ok(matrix, input, input_scales, batch) || !partials || !k_splits ||
+      k_splits > matrix->padded_columns / kChunk || k_splits > 16u)
+    return fail(QLLM_INVALID_ARGUMENT, "invalid partial FP4 x Q8 GEMM");
+  GemmArgs args = q8_gemm_args(matrix, input, input_scales);
+  args.output = partials;
+  args.output_kind = QLLM_OUT_F32;
+  args.k_splits = k_splits;
+  return launch_mfma(args, kSchemeUe8m0, true, batch, false, as_stream(stream));
+}
+
 extern "C" int32_t qllm_fp4_gemm_q8_split(const qllm_fp4_matrix* matrix,
                                           const int8_t* input,
                                           const float* input_scales,

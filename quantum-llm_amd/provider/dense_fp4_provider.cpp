@@ -348,8 +348,7 @@ void Mi355DenseFp4Provider::allocate_workspaces() {
     if (g_.mtp_layers)
       mtp_fusion_f32_ =
           static_cast<float*>(device_alloc(rows * 2U * g_.hidden * 4U));
-    // every projection adds its residual itself: the norm reads one array
-    projection_splits_ = 0U;
+    // (q/k/v is never cut here: its rows go through the rotary as they are)
     qkv_splits_ = 0U;
   }
   // counters and partial sums of the balanced q/k/v and gate/up launches
@@ -1572,7 +1571,14 @@ void Mi355DenseFp4Provider::enqueue_normalise(const float* weight,
                                               std::uint32_t rows) {
   if (g_.activation_q8) {
     // normalize_rows then quantize_rows (:5740-5778, :5983-5992)
-    enqueue_normalise_q8(hidden_, weight, rows);
+    if (pending_partials_)
+      status_check(qllm_rms_norm_partials_q8_batch(
+          hidden_, hidden_, projection_partials_, pending_partials_, weight, q8_,
+          q8_scales_, rows, g_.hidden, g_.norm_epsilon, g_.zero_centered_norm,
+          stream_));
+    else
+      enqueue_normalise_q8(hidden_, weight, rows);
+    pending_partials_ = 0U;
     return;
   }
   if (pending_partials_)
@@ -1591,15 +1597,23 @@ void Mi355DenseFp4Provider::enqueue_normalise(const float* weight,
 void Mi355DenseFp4Provider::enqueue_residual_projection(
     const qllm_fp4_matrix& matrix, const std::uint16_t* input,
     std::size_t input_bytes, std::uint32_t rows, bool leave_partials) {
+  const bool cut = leave_partials && projection_splits_ > 1U &&
+                   matrix.layout == QLLM_LAYOUT_TILED &&
+                   matrix.padded_columns / 64U >= projection_splits_;
   if (g_.activation_q8) {
     // the projection's input was quantised into q8_ by the caller
-    status_check(qllm_fp4_gemm_q8(&matrix, q8_, q8_scales_, hidden_, QLLM_OUT_F32,
-                                  hidden_, rows, stream_));
+    if (cut && g_.hidden % 4U == 0U && g_.hidden <= 16384U) {
+      status_check(qllm_fp4_gemm_q8_partial(&matrix, q8_, q8_scales_,
+                                            projection_partials_, projection_splits_,
+                                            rows, stream_));
+      pending_partials_ = projection_splits_;
+    } else {
+      status_check(qllm_fp4_gemm_q8(&matrix, q8_, q8_scales_, hidden_, QLLM_OUT_F32,
+                                    hidden_, rows, stream_));
+    }
     return;
   }
-  if (leave_partials && projection_splits_ > 1U &&
-      matrix.layout == QLLM_LAYOUT_TILED &&
-      matrix.padded_columns / 64U >= projection_splits_) {
+  if (cut) {
     status_check(qllm_fp4_gemm_bf16_partial(&matrix, input, input_bytes,
                                             projection_partials_,
                                             projection_splits_, rows, stream_));
@@ -1636,7 +1650,8 @@ void Mi355DenseFp4Provider::enqueue_attention_block(std::uint32_t index,
                       key_, value_,
                       reinterpret_cast<std::uint16_t*>(activation_f32_));
     enqueue_quantise(activation_f32_, rows, g_.query_heads * g_.head_dim);
-    enqueue_residual_projection(layer.output.descriptor, nullptr, 0U, rows, false);
+    enqueue_residual_projection(layer.output.descriptor, nullptr, 0U, rows,
+                                leave_partials);
     return;
   }
   const bool cut_qkv = qkv_splits_ > 1U &&
@@ -1677,7 +1692,8 @@ void Mi355DenseFp4Provider::enqueue_ffn_block(std::uint32_t index,
                                     gemm_workspace_, gemm_workspace_bytes_,
                                     stream_));
     enqueue_quantise(activation_f32_, rows, g_.intermediate);
-    enqueue_residual_projection(layer.down.descriptor, nullptr, 0U, rows, false);
+    enqueue_residual_projection(layer.down.descriptor, nullptr, 0U, rows,
+                                leave_partials);
     return;
   }
   status_check(qllm_fp4_swiglu_bf16_balanced(
@@ -1698,8 +1714,11 @@ void Mi355DenseFp4Provider::enqueue_head(std::uint32_t first_row,
   if (pending_partials_ && first_row != 0U)
     throw std::runtime_error("head over a row range needs a complete hidden state");
   if (g_.activation_q8) {
-    enqueue_normalise_q8(hidden_ + std::size_t{first_row} * g_.hidden, final_norm_,
-                         rows);
+    if (first_row == 0U)
+      enqueue_normalise(final_norm_, rows);   // finishes a cut projection too
+    else
+      enqueue_normalise_q8(hidden_ + std::size_t{first_row} * g_.hidden, final_norm_,
+                           rows);
     status_check(qllm_fp4_gemm_q8(&head_.descriptor, q8_, q8_scales_, logits_,
                                   QLLM_OUT_F32, nullptr, rows, stream_));
     status_check(qllm_argmax_batch(logits_, g_.vocabulary, rows, argmax_tokens_,
@@ -2269,8 +2288,16 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
                                           activation_f32_, rows, gemm_workspace_,
                                           gemm_workspace_bytes_, stream_));
         } else if (which == "ffn_down") {
-          status_check(qllm_fp4_gemm_q8(&layer.down.descriptor, q8_, q8_scales_,
-                                        query_, QLLM_OUT_F32, nullptr, rows, stream_));
+          // as the target pass launches it
+          if (projection_splits_ > 1U &&
+              layer.down.descriptor.padded_columns / 64U >= projection_splits_)
+            status_check(qllm_fp4_gemm_q8_partial(
+                &layer.down.descriptor, q8_, q8_scales_, projection_partials_,
+                projection_splits_, rows, stream_));
+          else
+            status_check(qllm_fp4_gemm_q8(&layer.down.descriptor, q8_, q8_scales_,
+                                          query_, QLLM_OUT_F32, nullptr, rows,
+                                          stream_));
         } else if (which == "qkv") {
           const qllm_gemm_segment projections[3] = {
               {query_, layer.qkv.descriptor.rows - 2U * kv_rows, QLLM_OUT_F32},
@@ -2280,8 +2307,15 @@ er::Status Mi355DenseFp4Provider::time_kernel(const std::string& which,
                                               projections, 3U, rows, gemm_workspace_,
                                               gemm_workspace_bytes_, stream_));
         } else if (which == "attention_output") {
-          status_check(qllm_fp4_gemm_q8(&layer.output.descriptor, q8_, q8_scales_,
-                                        query_, QLLM_OUT_F32, nullptr, rows, stream_));
+          if (projection_splits_ > 1U &&
+              layer.output.descriptor.padded_columns / 64U >= projection_splits_)
+            status_check(qllm_fp4_gemm_q8_partial(
+                &layer.output.descriptor, q8_, q8_scales_, projection_partials_,
+                projection_splits_, rows, stream_));
+          else
+            status_check(qllm_fp4_gemm_q8(&layer.output.descriptor, q8_, q8_scales_,
+                                          query_, QLLM_OUT_F32, nullptr, rows,
+                                          stream_));
         } else if (which == "lm_head") {
           status_check(qllm_fp4_gemm_q8(&head_.descriptor, q8_, q8_scales_, logits_,
                                         QLLM_OUT_F32, nullptr, rows, stream_));

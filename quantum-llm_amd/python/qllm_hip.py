@@ -120,6 +120,8 @@ SIGNATURES = {
     "qllm_rms_norm_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_residual_batch": (c_int32, [c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_partials_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_rms_norm_partials_q8_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_uint32, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
+    "qllm_fp4_gemm_q8_partial": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_void_p]),
     "qllm_rms_norm_concat_batch": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_uint32, c_float, c_int32, c_void_p]),
     "qllm_rms_norm_concat_embedding_batch": (c_int32, [POINTER(Fp4Matrix), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_uint32, c_float, c_int32, c_void_p, c_void_p]),
     "qllm_add_in_place": (c_int32, [c_void_p, c_void_p, c_uint32, c_int32, c_void_p]),

@@ -541,6 +541,58 @@ def test_q8_split_and_swiglu_forms(device):
     del keep, keep_up
 
 
+@pytest.mark.parametrize("rows,columns,batch,splits", [(5120, 17408, 5, 3), (5120, 8192, 5, 3),
+                                                       (320, 1024, 8, 2), (64, 128, 1, 2)])
+def test_q8_k_split_partials_add_up_to_the_integer_statement(device, rows, columns, batch,
+                                                             splits):
+    """qllm_fp4_gemm_q8_partial: split s holds the blocks of its share of K times
+    the row scale; added in index order they are the reference's sum within its
+    2e-4 (the F32 additions are regrouped, nothing else), and
+    qllm_rms_norm_partials_q8_batch finishes residual + sum and leaves the
+    bytes qllm_rms_norm_q8_batch leaves for the same row."""
+    rng = np.random.default_rng(rows + columns)
+    codes, scales, padded, q8, act_scales, matrix, keep, d_q8, d_s = _q8_case(
+        device, rng, rows, columns, batch)
+    partials = torch.zeros((splits, batch, rows), device=device)
+    qh.call("qllm_fp4_gemm_q8_partial", matrix, qh.ptr(d_q8), qh.ptr(d_s), qh.ptr(partials),
+            splits, batch, None)
+    torch.cuda.synchronize()
+    want = ol.fp4_linear_block32_q8(codes, scales, rows, padded, q8, act_scales)
+    parts = partials.cpu().numpy()
+    total = parts[0].copy()
+    for index in range(1, splits):
+        total += parts[index]
+    assert np.abs(total - want).max() <= 2e-4 * max(1.0, np.abs(want).max())
+    assert all(np.abs(parts[index]).max() > 0 for index in range(splits))
+    if rows % 4 == 0 and rows <= 16384:
+        residual = rng.standard_normal((batch, rows)).astype(np.float32)
+        weight = (0.1 * rng.standard_normal(rows)).astype(np.float32)
+        d_residual, d_weight = gu.device_tensor(residual, device), gu.device_tensor(weight, device)
+        summed = torch.zeros((batch, rows), device=device)
+        out = torch.zeros((batch, rows), dtype=torch.int8, device=device)
+        out_scales = torch.zeros(batch, device=device)
+        qh.call("qllm_rms_norm_partials_q8_batch", qh.ptr(d_residual), qh.ptr(summed),
+                qh.ptr(partials), splits, qh.ptr(d_weight), qh.ptr(out), qh.ptr(out_scales),
+                batch, rows, 1e-6, 1, None)
+        torch.cuda.synchronize()
+        expected_sum = residual.copy()
+        for index in range(splits):
+            expected_sum += parts[index]
+        assert np.array_equal(summed.cpu().numpy(), expected_sum)
+        assert np.array_equal(d_residual.cpu().numpy(), residual)
+        d_sum = gu.device_tensor(expected_sum, device)
+        plain = torch.zeros_like(out)
+        plain_scales = torch.zeros_like(out_scales)
+        qh.call("qllm_rms_norm_q8_batch", qh.ptr(d_sum), qh.ptr(d_weight), qh.ptr(plain),
+                qh.ptr(plain_scales), batch, rows, 1e-6, 1, None)
+        torch.cuda.synchronize()
+        assert torch.equal(out, plain) and torch.equal(out_scales, plain_scales)
+    with pytest.raises(qh.QllmError):      # more splits than chunks of K
+        qh.call("qllm_fp4_gemm_q8_partial", matrix, qh.ptr(d_q8), qh.ptr(d_s),
+                qh.ptr(partials), padded // 64 + 1, batch, None)
+    del keep
+
+
 def test_q8_matrix_core_gemm_rejects_what_it_does_not_take(device):
     rng = np.random.default_rng(3)
     codes, scales, padded, q8, act_scales, matrix, keep, d_q8, d_s = _q8_case(
