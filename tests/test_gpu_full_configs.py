@@ -31,13 +31,20 @@ SEED = 20241125
 TAG = "decode.mtp.dense-full-attention.fp4-f16-block16.exact.v2"
 
 
-def provider_with(layers, context=CONTEXT, kv_seed=7):
+Q8_TAG = "decode.mtp.dense-full-attention.fp4-block32.exact.v2"
+
+
+def provider_with(layers, context=CONTEXT, kv_seed=7, activation_q8=False):
+    """The benchmark's model; with `activation_q8` the same shapes under the
+    artifact's default contract (block-32 UE8M0 scales, per-row Q8 activations)."""
     geometry = dict(MODEL, layers=layers, max_context=context + 256)
+    if activation_q8:
+        geometry.update(scale_scheme=0, activation_q8=1)
     provider = qp.Provider(**geometry)
     provider.load_synthetic_weights(SEED)
     if context:
         provider.prefill_synthetic_kv(context, kv_seed)
-    provider.prepare_exact_decode(TAG)
+    provider.prepare_exact_decode(Q8_TAG if activation_q8 else TAG)
     return provider
 
 
@@ -45,15 +52,18 @@ class HostLayerModel(step_oracle.TinyModel):
     """The first layer of the provider's random-init model as host tensors, a
     few rows of the embedding and a sample of the head's rows."""
 
-    def __init__(self, provider, tokens, head_rows):
+    def __init__(self, provider, tokens, head_rows, activation_q8=False):
         H, I, Q, KV, d = (MODEL["hidden"], MODEL["intermediate"], MODEL["query_heads"],
                           MODEL["kv_heads"], MODEL["head_dim"])
+        self.activation_q8 = activation_q8
+        scheme = 0 if activation_q8 else 1
         self.hidden, self.intermediate, self.layers = H, I, 1
         self.query_heads, self.kv_heads, self.head_dim = Q, KV, d
         self.rotary_dim, self.rope_theta, self.eps = d, MODEL["rope_theta"], MODEL["norm_epsilon"]
-        self.scheme, self.output_gated, self.qk_norm, self.zero_centered = 1, False, False, False
+        self.scheme, self.output_gated, self.qk_norm, self.zero_centered = (
+            scheme, False, False, False)
         rows = lambda name, first, count, columns: provider.matrix_rows(  # noqa: E731
-            name, first, count, columns, 1)
+            name, first, count, columns, scheme)
         embedded = [rows("token_embedding", int(t), 1, H) for t in tokens]
         self.embedding = (np.concatenate([e[0] for e in embedded]),
                           np.concatenate([e[1] for e in embedded]))
@@ -74,29 +84,40 @@ class HostLayerModel(step_oracle.TinyModel):
         self.vocabulary = len(head_rows)
 
 
-def test_one_layer_of_the_27b_model_at_32k_against_the_composed_oracle(device):
+@pytest.mark.parametrize("activation_q8", [False, True])
+def test_one_layer_of_the_27b_model_at_32k_against_the_composed_oracle(device, activation_q8):
     """Hidden 5120, 64Q/8KV heads of 128, FFN 17408, vocabulary 151936, 32768
     cached tokens: every operation of a layer at its benchmark shape, composed,
-    against the CPU oracle on the weights read back from the device."""
+    against the CPU oracle on the weights read back from the device - with bf16
+    activations (binary16 block scales, the benchmark's configuration) and
+    under the artifact's default contract (UE8M0 block scales, per-row Q8
+    activations: the integer statement of the reference's linears)."""
     rng = np.random.default_rng(3)
-    provider = provider_with(1)
+    provider = provider_with(1, activation_q8=activation_q8)
     tokens = rng.integers(0, MODEL["vocabulary"], 5).astype(np.uint32)
     head_rows = np.sort(rng.choice(MODEL["vocabulary"], 384, replace=False))
     pages_before = [provider.kv_page(index) for index in range(CONTEXT // 256 + 1)]
     provider.run_target(tokens, CONTEXT)
     logits, hidden = provider.logits(5), provider.hidden(5)
     observed = [provider.kv_page(index) for index in range(CONTEXT // 256 + 1)]
-    model = HostLayerModel(provider, tokens, head_rows)
+    model = HostLayerModel(provider, tokens, head_rows, activation_q8)
     report = {}
     want_logits, want_hidden = step_oracle.run_target(
         model, np.arange(5, dtype=np.uint32), CONTEXT, pages_before, 256, observed, report)
     assert report["record_byte_diffs"] <= 0.03 * report["record_bytes"]
     relative = np.linalg.norm(hidden - want_hidden) / np.linalg.norm(want_hidden)
-    assert relative < 1e-2, relative
+    # Under the Q8 contract both sides quantise their own activations five times
+    # in the layer: where they differ in the last place before a quantisation
+    # (the attention output, within its 1e-2) a code falls the other way and
+    # moves that element by a whole step of absmax / 127 - on the heavy-tailed
+    # rows of a random-init model most elements are small against that step.
+    # Measured 2.1e-2 (bf16 contract: 5.5e-3); each linear on identical codes is
+    # held to 2e-4 in test_gpu_gemm.py.
+    assert relative < (4e-2 if activation_q8 else 1e-2), relative
     assert np.abs(hidden - want_hidden).max() < 0.05 * np.abs(want_hidden).max()
     sampled = logits[:, head_rows]
     relative = np.linalg.norm(sampled - want_logits) / np.linalg.norm(want_logits)
-    assert relative < 2e-2, relative
+    assert relative < (5e-2 if activation_q8 else 2e-2), relative
     provider.close()
 
 
